@@ -1,0 +1,95 @@
+/* TEST INFRASTRUCTURE ONLY.
+ *
+ * CPU restatement of the reference's GGUF k-quant decode path (PromeTorch
+ * torch/io/gguf_dequant.h, torch/io/cpu_quant_gemv.h, torch/io/gguf_model.h
+ * forward_decode_cpu, aten/src/ATen/native/cpu/hot_loops.cpp RoPE,
+ * aten/src/ATen/native/cpu/VectorizedOps.h exp256_ps).  It is the checker the
+ * GPU kernels are compared against and the timed "port" CPU baseline; it is
+ * never linked into, loaded by, or called from the shipped library.
+ *
+ * Pinning status (what fixes each function independently of this file):
+ *   po_fp16_to_fp32        all 65536 inputs vs numpy float16->float32, and vs the compiled reference
+ *   po_get_scale_min_k4    exhaustive 6-bit pack/unpack round trip + compiled reference
+ *   po_dequantize_q4_k/q6_k golden blocks from the compiled reference (bit-exact) + closed form in numpy
+ *   po_quantize_x_q8       golden vectors from the compiled reference (bit-exact) + numpy rint invariants
+ *   po_q4k_gemv            golden y from the compiled reference (bit-exact) + exact int dots vs numpy
+ *   po_q6k_gemv            golden y from the compiled reference (bit-exact) + float64 dot of dequant
+ *   po_rmsnorm_*           compiled reference + float64 numpy
+ *   po_rope_*              compiled reference + float64 closed form (NeoX pairing)
+ *   po_exp256              compiled reference + float64 exp
+ *   po_attn_head, po_silu_mul, po_argmax, po_decode_step
+ *                          golden logits / token ids of the compiled reference's
+ *                          forward_decode_cpu on a tiny and the full-size model
+ */
+#ifndef PTM_ORACLE_H
+#define PTM_ORACLE_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { PO_Q4_K = 12, PO_Q6_K = 14 };
+
+float po_fp16_to_fp32(uint16_t h);
+uint16_t po_fp32_to_fp16(float f); /* round-to-nearest-even, IEEE */
+void po_get_scale_min_k4(int j, const uint8_t* q, uint8_t* sc, uint8_t* m);
+void po_dequantize_q4_k(const void* src, float* dst, int64_t n);
+void po_dequantize_q6_k(const void* src, float* dst, int64_t n);
+
+/* Q8 activation blocks, flat: d[K/32], sum[K/32], qs[K] */
+void po_quantize_x_q8(const float* x, int64_t K, float* d, float* sum, int8_t* qs);
+
+void po_q4k_gemv(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride);
+void po_q4k_gemv_f32(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride);
+void po_q6k_gemv(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride);
+void po_q6k_gemv_f32(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride);
+/* dispatcher: type 12 -> po_q4k_gemv, 14 -> po_q6k_gemv, anything else: silent no-op */
+void po_cpu_quant_gemv(uint32_t type, const void* W, const float* x, float* y,
+                       int64_t K, int64_t N, int64_t stride);
+/* Integer sub-block dots of one Q4_K row against Q8 x: isum[K/32] (exact int32). */
+void po_q4k_row_isums(const void* row, const int8_t* qs, int64_t K, int32_t* isum);
+
+void po_rmsnorm_seq(const float* x, const float* gamma, float eps, int add_one, int64_t H, float* out);
+void po_rmsnorm_vec(const float* x, const float* gamma, float eps, int add_one, int64_t H, float* out);
+void po_rope_precompute(float* c, float* s, int64_t pos, int64_t head_dim, float base);
+void po_rope_apply_neox(float* q, float* k, const float* c, const float* s,
+                        int64_t n_heads, int64_t n_kv_heads, int64_t head_dim);
+void po_exp256(const float* in, float* out, int64_t n8);
+/* one query head against T cached positions; k,v point at this kv-head's column
+ * block of row 0, row pitch kv_dim floats; scores is scratch[T] */
+void po_attn_head(const float* q, const float* k, const float* v, int64_t T, int64_t kv_dim,
+                  int64_t head_dim, float scale, float* scores, float* out);
+void po_silu_mul(float* gate, const float* up, int64_t n);
+int64_t po_argmax(const float* x, int64_t n);
+
+typedef struct {
+    const void* data; uint32_t type; int64_t rows, cols, stride;
+} po_qweight;
+
+typedef struct {
+    po_qweight q, k, v, o, gate, up, down;
+    const float *attn_norm, *ffn_norm, *q_norm, *k_norm;
+    float *k_cache, *v_cache; /* [max_seq][kv_dim] fp32 storage */
+} po_layer;
+
+typedef struct {
+    int64_t vocab, hidden, n_layers, n_heads, n_kv_heads, head_dim, inter, max_seq;
+    float rope_base, eps;
+    int kv_fp16;            /* 1: round appended K/V rows to fp16 (what an fp16 cache stores) */
+    const float* embedding; /* fp32 [vocab][hidden], or NULL to dequantize rows of lm_head (Q6_K, tied) */
+    po_layer* layers;
+    const float* out_norm;
+    po_qweight lm_head;
+    int64_t seq_len;
+} po_model;
+
+/* One decode step (forward_decode_cpu order, Q4_K_M fallbacks); writes logits[vocab],
+ * advances seq_len, returns greedy argmax. hidden_out (optional) gets the final-normed hidden. */
+int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_out);
+int po_num_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,160 @@
+"""Seeded synthetic GGUF k-quant data for the benchmark configurations.
+
+Everything is generated with numpy's PCG64 stream from an explicit seed, so the same
+call yields the same bytes wherever it runs.  Block layouts follow the GGUF super-block
+formats (reference: torch/io/gguf_dequant.h:158,160,289-297,301-319,392-408).
+"""
+from __future__ import annotations
+
+import numpy as np
+
+Q4_K, Q6_K = 12, 14
+BLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
+
+
+def rng_for(seed: int, *stream: int) -> np.random.Generator:
+    """Independent generator for (seed, stream ids...)."""
+    return np.random.Generator(np.random.PCG64(np.random.SeedSequence([seed, *stream])))
+
+
+def row_stride(qtype: int, cols: int) -> int:
+    assert cols % 256 == 0
+    return cols // 256 * BLOCK_BYTES[qtype]
+
+
+def pack_scales_k4(sc: np.ndarray, mn: np.ndarray) -> np.ndarray:
+    """Pack 8 six-bit scales and 8 six-bit mins ([..., 8] uint8 each) into [..., 12] bytes,
+    the inverse of get_scale_min_k4 (reference: gguf_dequant.h:289-297)."""
+    sc = sc.astype(np.uint8)
+    mn = mn.astype(np.uint8)
+    out = np.empty(sc.shape[:-1] + (12,), dtype=np.uint8)
+    out[..., 0:4] = (sc[..., 0:4] & 63) | ((sc[..., 4:8] >> 4) << 6)
+    out[..., 4:8] = (mn[..., 0:4] & 63) | ((mn[..., 4:8] >> 4) << 6)
+    out[..., 8:12] = (sc[..., 4:8] & 0x0F) | ((mn[..., 4:8] & 0x0F) << 4)
+    return out
+
+
+def make_q4k(rng: np.random.Generator, rows: int, cols: int, d_scale: float = 0.01) -> np.ndarray:
+    """[rows, cols/256*144] uint8 of Q4_K super-blocks: d, dmin = fp16(|N(0,1)|*d_scale),
+    6-bit scales/mins uniform 0..63, 4-bit quants uniform 0..15."""
+    nb = rows * (cols // 256)
+    blk = np.empty((nb, 144), dtype=np.uint8)
+    dd = (np.abs(rng.standard_normal((nb, 2), dtype=np.float32)) * np.float32(d_scale)).astype(np.float16)
+    blk[:, 0:4] = dd.view(np.uint8).reshape(nb, 4)
+    sm = rng.integers(0, 64, size=(nb, 16), dtype=np.uint8)
+    blk[:, 4:16] = pack_scales_k4(sm[:, :8], sm[:, 8:])
+    blk[:, 16:144] = rng.integers(0, 256, size=(nb, 128), dtype=np.uint8)
+    return blk.reshape(rows, cols // 256 * 144)
+
+
+def make_q6k(rng: np.random.Generator, rows: int, cols: int, d_scale: float = 0.005) -> np.ndarray:
+    """[rows, cols/256*210] uint8 of Q6_K super-blocks: ql/qh uniform bytes (quants 0..63),
+    16 int8 scales uniform -32..31, d = fp16(|N(0,1)|*d_scale)."""
+    nb = rows * (cols // 256)
+    blk = np.empty((nb, 210), dtype=np.uint8)
+    blk[:, 0:192] = rng.integers(0, 256, size=(nb, 192), dtype=np.uint8)
+    blk[:, 192:208] = rng.integers(-32, 32, size=(nb, 16), dtype=np.int8).view(np.uint8)
+    d = (np.abs(rng.standard_normal((nb, 1), dtype=np.float32)) * np.float32(d_scale)).astype(np.float16)
+    blk[:, 208:210] = d.view(np.uint8).reshape(nb, 2)
+    return blk.reshape(rows, cols // 256 * 210)
+
+
+def make_weight(rng, qtype: int, rows: int, cols: int) -> np.ndarray:
+    return make_q4k(rng, rows, cols) if qtype == Q4_K else make_q6k(rng, rows, cols)
+
+
+def make_x(rng: np.random.Generator, n: int) -> np.ndarray:
+    return rng.standard_normal(n, dtype=np.float32)
+
+
+# --------------------------------------------------------------------------------------
+# closed-form numpy dequantisers (independent of the C oracle; used to pin it)
+# --------------------------------------------------------------------------------------
+def unpack_scales_k4(q12: np.ndarray):
+    """[..., 12] bytes -> (sc[..., 8], mn[..., 8]) per get_scale_min_k4."""
+    q = q12.astype(np.uint8)
+    sc = np.empty(q.shape[:-1] + (8,), dtype=np.uint8)
+    mn = np.empty_like(sc)
+    sc[..., 0:4] = q[..., 0:4] & 63
+    mn[..., 0:4] = q[..., 4:8] & 63
+    sc[..., 4:8] = (q[..., 8:12] & 0x0F) | ((q[..., 0:4] >> 6) << 4)
+    mn[..., 4:8] = (q[..., 8:12] >> 4) | ((q[..., 4:8] >> 6) << 4)
+    return sc, mn
+
+
+def dequant_q4k_np(raw: np.ndarray) -> np.ndarray:
+    blk = raw.reshape(-1, 144)
+    d = blk[:, 0:2].copy().view(np.float16).astype(np.float32)   # [nb,1]
+    dmin = blk[:, 2:4].copy().view(np.float16).astype(np.float32)
+    sc, mn = unpack_scales_k4(blk[:, 4:16])
+    qs = blk[:, 16:144].reshape(-1, 4, 32)
+    q = np.stack([qs & 0x0F, qs >> 4], axis=2).reshape(-1, 8, 32).astype(np.float32)  # sub-block order
+    ds = (d * sc.astype(np.float32))[:, :, None]
+    ms = (dmin * mn.astype(np.float32))[:, :, None]
+    return (ds * q - ms).astype(np.float32).reshape(-1)
+
+
+def dequant_q6k_np(raw: np.ndarray) -> np.ndarray:
+    blk = raw.reshape(-1, 210)
+    nb = blk.shape[0]
+    ql = blk[:, 0:128].reshape(nb, 2, 2, 32)      # [half][which32][l]
+    qh = blk[:, 128:192].reshape(nb, 2, 32)
+    sc = blk[:, 192:208].copy().view(np.int8).astype(np.float32).reshape(nb, 2, 4, 2)  # [half][grp][l/16]
+    d = blk[:, 208:210].copy().view(np.float16).astype(np.float32).reshape(nb, 1, 1, 1)
+    out = np.empty((nb, 2, 4, 32), dtype=np.float32)
+    for grp in range(4):
+        lo = ql[:, :, grp & 1, :]
+        nib = (lo >> 4) if (grp & 2) else (lo & 0x0F)
+        q = (nib | (((qh >> (2 * grp)) & 3) << 4)).astype(np.int32) - 32
+        s = np.repeat(sc[:, :, grp, :], 16, axis=-1)          # [nb,2,32]
+        out[:, :, grp, :] = (d[:, :, 0, :] * s) * q.astype(np.float32)
+    return out.reshape(-1)
+
+
+# --------------------------------------------------------------------------------------
+# model-shaped bundles
+# --------------------------------------------------------------------------------------
+QWEN3_4B = dict(vocab=151936, hidden=2560, n_layers=36, n_heads=32, n_kv_heads=8, head_dim=128,
+                inter=9728, rope_base=1.0e6, eps=1.0e-6)
+TINY = dict(vocab=1024, hidden=256, n_layers=2, n_heads=4, n_kv_heads=2, head_dim=64,
+            inter=512, rope_base=1.0e6, eps=1.0e-6)
+
+# (name, quant type, rows-key, cols-key) for the Q4_K_M mix: v and down in Q6_K
+LAYER_MATS = (("q", Q4_K), ("k", Q4_K), ("v", Q6_K), ("o", Q4_K), ("gate", Q4_K), ("up", Q4_K), ("down", Q6_K))
+
+
+def layer_shapes(cfg: dict) -> dict:
+    H, qd, kvd, I = cfg["hidden"], cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"], cfg["inter"]
+    return {"q": (qd, H), "k": (kvd, H), "v": (kvd, H), "o": (H, qd), "gate": (I, H), "up": (I, H), "down": (H, I)}
+
+
+def make_layer(seed: int, layer: int, cfg: dict) -> dict:
+    """One decoder layer's seven weight matrices plus its four norm vectors
+    (gamma = 1 + 0.1*N(0,1))."""
+    shp = layer_shapes(cfg)
+    out = {}
+    for i, (name, qt) in enumerate(LAYER_MATS):
+        out[name] = (qt, make_weight(rng_for(seed, 1, layer, i), qt, *shp[name]))
+    g = rng_for(seed, 2, layer)
+    for name, n in (("attn_norm", cfg["hidden"]), ("ffn_norm", cfg["hidden"]),
+                    ("q_norm", cfg["head_dim"]), ("k_norm", cfg["head_dim"])):
+        out[name] = (np.float32(1.0) + np.float32(0.1) * g.standard_normal(n, dtype=np.float32)).astype(np.float32)
+    return out
+
+
+def make_head(seed: int, cfg: dict) -> dict:
+    """Tied Q6_K token-embedding / lm_head table and the output norm."""
+    g = rng_for(seed, 3)
+    return {
+        "lm_head": make_q6k(g, cfg["vocab"], cfg["hidden"]),
+        "out_norm": (np.float32(1.0) + np.float32(0.1) * g.standard_normal(cfg["hidden"], dtype=np.float32)).astype(np.float32),
+    }
+
+
+def make_kv_prefill(seed: int, layer: int, cfg: dict, n_pos: int):
+    """fp16 K/V cache contents for positions [0, n_pos): N(0,1) rounded to fp16."""
+    g = rng_for(seed, 4, layer)
+    kvd = cfg["n_kv_heads"] * cfg["head_dim"]
+    k = g.standard_normal((n_pos, kvd), dtype=np.float32).astype(np.float16)
+    v = g.standard_normal((n_pos, kvd), dtype=np.float32).astype(np.float16)
+    return k, v
