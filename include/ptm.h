@@ -1,0 +1,243 @@
+/*
+ * ptm.h — C ABI of libptm_hip.so: MI355X (gfx950) kernels for the GGUF Q4_K / Q6_K
+ * batch-1 decode path of PromeTorch.
+ *
+ * Every entry point is the flat-C counterpart of one operator the reference declares in
+ * aten/src/ATen/cuda/CUDAOps.h (C++ `at::cuda::launch_*`, cited per function below);
+ * include/ptm_at_cuda_shim.h re-exposes them under the reference's own names.
+ *
+ * Conventions (reference: CUDAOps.h, gguf_model.h:3117-3140):
+ *   - all pointers are DEVICE pointers unless a parameter says "host";
+ *   - weights are raw GGUF super-blocks exactly as stored in the file, row-major
+ *     [N][K/256] blocks, row_stride_bytes = K/256 * {144 (Q4_K), 210 (Q6_K)};
+ *   - activations and outputs are fp32; K % 256 == 0; x and y 16-byte aligned;
+ *   - launches are asynchronous on `stream` (a hipStream_t, NULL = default stream),
+ *     allocate nothing, and are legal inside hipStreamBeginCapture/EndCapture;
+ *   - unlike the reference's void launchers, each call returns PTM_OK or a negative
+ *     PTM_E_* after validating its arguments on the host; nothing throws.
+ */
+#ifndef PTM_H
+#define PTM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ptm_stream_t; /* hipStream_t */
+
+enum {
+    PTM_OK = 0,
+    PTM_E_NULL = -1,        /* required pointer is NULL */
+    PTM_E_SHAPE = -2,       /* K not a multiple of 256, non-positive size, stride too small ... */
+    PTM_E_ALIGN = -3,       /* pointer/stride alignment precondition violated */
+    PTM_E_UNSUPPORTED = -4, /* quant type / head_dim / size outside what the kernels implement */
+    PTM_E_HIP = -5,         /* a HIP runtime call failed (ptm_last_hip_error() has the code) */
+    PTM_E_RANGE = -6,       /* position / token beyond the allocated cache or table */
+    PTM_E_STATE = -7        /* object used before initialisation or after an error */
+};
+
+enum { PTM_TYPE_Q4_K = 12, PTM_TYPE_Q6_K = 14 }; /* ggml type ids, gguf_dequant.h:29-58 */
+
+const char* ptm_strerror(int code);
+int ptm_last_hip_error(void);
+int ptm_version(void);
+/* Number of compute units of the current device (used to size grids). */
+int ptm_device_cus(void);
+
+/* ---- dequantisation -------------------------------------------------------------- */
+/* Q4_K / Q6_K super-blocks -> fp32, bit-exact with dequantize_q4_k / dequantize_q6_k
+ * (gguf_dequant.h:304-341, :395-430). n_elems % 256 == 0. */
+int ptm_dequant_q4k(const void* blocks, float* out, int64_t n_elems, ptm_stream_t stream);
+int ptm_dequant_q6k(const void* blocks, float* out, int64_t n_elems, ptm_stream_t stream);
+/* Q4_K -> fp16, COLUMN-major out[k*N + n]; replaces launch_dequant_q4k_to_fp16 (CUDAOps.h:477-480). */
+int ptm_dequant_q4k_to_fp16(const void* W, void* out_fp16, int K, int N, int64_t row_stride_bytes,
+                            ptm_stream_t stream);
+
+/* ---- Q8 activation blocks -------------------------------------------------------- */
+/* Quantise x[K] the way the reference CPU GEMV does (cpu_quant_gemv.h:147-198): per 32
+ * values d = amax/127, q = clamp(rne(x/d), -127, 127), sum = d * sum(q).
+ * Device layout of q8: int8 qs[K], then float d[K/32], then float sum[K/32]
+ * (ptm_q8_bytes(K) = K + K/4 bytes, 16-byte aligned).  Plays the role of
+ * launch_quantize_q8_1 (CUDAOps.h:462-464) with the CPU path's block format. */
+int64_t ptm_q8_bytes(int K);
+int ptm_quantize_q8(const float* x, void* q8, int K, ptm_stream_t stream);
+
+/* ---- dequant-fused GEMV: y[N] (+)= W[N,K] . x[K] --------------------------------- */
+/* Q4_K with the reference CPU semantics (Q8 activations, exact int32 sub-block dots, fp32
+ * combine; cpu_quant_gemv.h:505-685).  Replaces launch_q4km_gemv / launch_q4km_persistent_gemv
+ * / _v2 (CUDAOps.h:427-448) and, with accumulate != 0, launch_q4km_persistent_gemv_accumulate
+ * (CUDAOps.h:613-616). x is quantised inside the kernel. */
+int ptm_q4k_gemv(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes,
+                 int accumulate, ptm_stream_t stream);
+/* Same with x already quantised by ptm_quantize_q8 (replaces launch_q4km_q8_gemv, CUDAOps.h:467-470). */
+int ptm_q4k_gemv_q8(const void* W, const void* x_q8, float* y, int K, int N, int64_t row_stride_bytes,
+                    int accumulate, ptm_stream_t stream);
+/* Q6_K with fp32 activations (cpu_quant_gemv.h:883-1020). Replaces launch_q6k_gemv (CUDAOps.h:498-501). */
+int ptm_q6k_gemv(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes,
+                 int accumulate, ptm_stream_t stream);
+/* Q6_K GEMV with a fused greedy argmax (strict '>', lowest index on ties):
+ * writes *out_index (int64, device) and, if logits != NULL, logits[N].
+ * workspace: ptm_argmax_workspace_bytes(N) bytes of device scratch.
+ * Fuses launch_q6k_gemv + launch_argmax (CUDAOps.h:498-501, :145). */
+int64_t ptm_argmax_workspace_bytes(int N);
+int ptm_q6k_gemv_argmax(const void* W, const float* x, float* logits, int K, int N,
+                        int64_t row_stride_bytes, int64_t* out_index, void* workspace,
+                        ptm_stream_t stream);
+/* Type dispatcher mirroring cpu_quant_gemv (cpu_quant_gemv.h:1635-1688) and gemv_scratch
+ * (gguf_model.h:3117-3140): 12 -> Q4_K, 14 -> Q6_K; anything else returns PTM_E_UNSUPPORTED
+ * and launches nothing (the reference silently no-ops). */
+int ptm_quant_gemv(uint32_t ggml_type, const void* W, const float* x, float* y, int K, int N,
+                   int64_t row_stride_bytes, int accumulate, ptm_stream_t stream);
+
+/* Two / three Q4_K projections of the same x in one launch.
+ * Replace launch_q4km_fused_gate_up_gemv (CUDAOps.h:453-458) and
+ * launch_q4km_fused_qkv_gemv (CUDAOps.h:578-583). */
+int ptm_q4k_fused_gate_up_gemv(const void* w_gate, const void* w_up, const float* x, float* y_gate,
+                               float* y_up, int K, int N_gate, int N_up, int64_t row_stride_bytes,
+                               ptm_stream_t stream);
+int ptm_q4k_fused_qkv_gemv(const void* w_q, const void* w_k, const void* w_v, const float* x,
+                           float* out_q, float* out_k, float* out_v, int K, int N_q, int N_k, int N_v,
+                           int64_t row_stride_bytes, ptm_stream_t stream);
+/* RMSNorm(x)*gamma computed in the kernel, then the projection(s).  Replace
+ * launch_q4km_fused_rmsnorm_gemv / _qkv_gemv / _gate_up_gemv (CUDAOps.h:589-628). */
+int ptm_q4k_fused_rmsnorm_gemv(const float* x, const float* norm_w, const void* W, float* y, int K,
+                               int N, int64_t row_stride_bytes, float eps, int add_one,
+                               ptm_stream_t stream);
+int ptm_q4k_fused_rmsnorm_qkv_gemv(const float* x, const float* norm_w, const void* w_q, const void* w_k,
+                                   const void* w_v, float* out_q, float* out_k, float* out_v, int K,
+                                   int N_q, int N_k, int N_v, int64_t row_stride_bytes, float eps,
+                                   int add_one, ptm_stream_t stream);
+int ptm_q4k_fused_rmsnorm_gate_up_gemv(const float* x, const float* norm_w, const void* w_gate,
+                                       const void* w_up, float* y_gate, float* y_up, int K, int N_gate,
+                                       int N_up, int64_t row_stride_bytes, float eps, int add_one,
+                                       ptm_stream_t stream);
+/* RMSNorm + gate/up projections + SiLU(gate)*up in one launch: act[N] (no counterpart launcher in
+ * the reference; it is launch_q4km_fused_rmsnorm_gate_up_gemv followed by launch_silu_mul,
+ * gguf_model.h:2954-2986). */
+int ptm_q4k_fused_rmsnorm_gate_up_silu(const float* x, const float* norm_w, const void* w_gate,
+                                       const void* w_up, float* act, int K, int N,
+                                       int64_t row_stride_bytes, float eps, int add_one,
+                                       ptm_stream_t stream);
+
+/* ---- decode-step glue ------------------------------------------------------------ */
+/* Row-wise RMSNorm: out = x * 1/sqrt(mean(x^2)+eps) * (gamma [+1]).  launch_rms_norm (CUDAOps.h:382-385).
+ * If q8_out != NULL (rows must be 1, hidden % 256 == 0) the Q8 blocks of the result are written too. */
+int ptm_rms_norm(const float* in, const float* weight, float* out, int rows, int hidden, float eps,
+                 int add_one, void* q8_out, ptm_stream_t stream);
+/* In-place per-head RMSNorm over [rows][n_heads][head_dim]. launch_per_head_rms_norm (CUDAOps.h:387-390). */
+int ptm_per_head_rms_norm(float* data, const float* weight, int rows, int n_heads, int head_dim,
+                          float eps, int add_one, ptm_stream_t stream);
+/* Fused per-head QK-norm + RoPE + K/V cache append for one token.
+ * Q [n_heads*head_dim] and K [n_kv_heads*head_dim] are updated in place; K and V rows are written
+ * to the caches at row *d_past_len.  q_norm_w/k_norm_w may be NULL (no QK-norm).
+ * neox != 0: pairs (d, d+head_dim/2) as the reference CPU path applies for qwen3
+ * (hot_loops.cpp:2035-2061); neox == 0: interleaved pairs (2d, 2d+1) as the reference CUDA
+ * kernel (FlashDecoding.cu:309-312).  kv_fp16 != 0: caches are fp16 [max_seq][kv_dim], else fp32.
+ * rope_table: optional [max_seq][head_dim] fp32 rows of (cos[0..hd/2), sin[0..hd/2)); if NULL the
+ * angles are computed on the device from rope_freq_base.
+ * Replaces launch_fused_qknorm_rope_kvwrite(_graph) (CUDAOps.h:563-570, :653-659). */
+int ptm_qknorm_rope_kvwrite(float* Q, float* K, const float* V, const float* q_norm_w,
+                            const float* k_norm_w, void* K_cache, void* V_cache, int n_heads,
+                            int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                            float rope_freq_base, const float* rope_table, float eps, int add_one,
+                            int neox, int kv_fp16, ptm_stream_t stream);
+/* Host-side helper: fill table[max_seq][head_dim] with the reference's fp32 cos/sin
+ * (hot_loops.cpp:1853-1876: freq = 1/powf(base, 2d/hd), theta = pos*freq). table is a HOST pointer. */
+int ptm_rope_table_host(float* table, int max_seq, int head_dim, float rope_freq_base);
+/* fp32 rows -> fp16 cache rows. launch_fp16_kv_cache_write (CUDAOps.h:635-638). */
+int ptm_fp16_kv_cache_write(const float* src, void* dst_cache_fp16, int64_t num_new_rows, int64_t cols,
+                            int64_t offset_row, ptm_stream_t stream);
+
+/* Split-KV single-token GQA attention.  Attends positions [0, *d_past_len] (inclusive: the row
+ * just appended).  Caches are [max_seq][n_kv_heads*head_dim] fp16 (kv_fp16 != 0) or fp32.
+ * Scratch (caller-owned): partial_O [S*n_heads*head_dim], partial_lse [S*n_heads] (sum of exp),
+ * partial_max [S*n_heads] with S = ptm_flash_decode_num_splits(max_seq).
+ * Replaces launch_flash_decode(_fp16)(_graph) + flash_decode_num_splits / _kv_chunk_size
+ * (CUDAOps.h:543-557, :641-673). head_dim must be 64 or 128. */
+int ptm_flash_decode_kv_chunk_size(void);
+int ptm_flash_decode_num_splits(int total_seq);
+int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, float* O,
+                     float* partial_O, float* partial_lse, float* partial_max, int n_heads,
+                     int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq, float scale,
+                     int kv_fp16, ptm_stream_t stream);
+
+/* out = silu(gate) * up. launch_silu_mul (CUDAOps.h:416-418). */
+int ptm_silu_mul(const float* gate, const float* up, float* out, int64_t n, ptm_stream_t stream);
+/* out[hidden] = emb_table[*d_token_id][:]. launch_embedding_lookup (CUDAOps.h:149-152). */
+int ptm_embedding_row(const float* emb_table, float* out, const int* d_token_id, int hidden,
+                      ptm_stream_t stream);
+/* Same, dequantising row *d_token_id of a Q6_K table (tied lm_head; gguf_model.h:6774 dequantises
+ * the whole table at load instead). */
+int ptm_embedding_row_q6k(const void* table_q6k, float* out, const int* d_token_id, int hidden,
+                          int64_t row_stride_bytes, ptm_stream_t stream);
+/* *out = index of the maximum (strict '>', lowest index on ties). launch_argmax (CUDAOps.h:145). */
+int ptm_argmax(const float* in, int64_t* out, int64_t n, ptm_stream_t stream);
+/* out = a + b; out = in. launch_add / launch_copy (CUDAOps.h:63, :83). */
+int ptm_add(const float* a, const float* b, float* out, int64_t n, ptm_stream_t stream);
+int ptm_copy(const float* in, float* out, int64_t n, ptm_stream_t stream);
+
+/* ---- prefill: quantised-weight GEMM, Y[M,N] = X[M,K] . W[N,K]^T ------------------ */
+/* The reference has no quantised GEMM: matmul_q loops M single-row GEMVs
+ * (gguf_model.h:7029-7036, :7056-7061).  These tile the weights through LDS once and use MFMA.
+ * X is bf16 row-major [M][K]; Y fp32 row-major [M][N].
+ * Q4_K: rows of X are quantised to Q8 blocks (same rule as ptm_quantize_q8, applied to the
+ * bf16->fp32 values) and int8 MFMA computes the exact sub-block integer dots.
+ * Q6_K: dequantised weights (exact in bf16x2 split) times bf16 X on bf16 MFMA, fp32 accumulate.
+ * workspace: ptm_qgemm_workspace_bytes(M, K) device bytes. */
+int64_t ptm_qgemm_workspace_bytes(int M, int K);
+int ptm_qgemm_q4k(const void* W, const void* X_bf16, float* Y, int M, int K, int N,
+                  int64_t row_stride_bytes, void* workspace, ptm_stream_t stream);
+int ptm_qgemm_q6k(const void* W, const void* X_bf16, float* Y, int M, int K, int N,
+                  int64_t row_stride_bytes, void* workspace, ptm_stream_t stream);
+
+/* ---- batch-1 decode runtime (GGUFModel::forward_decode, gguf_model.h:2575-3113) --- */
+typedef struct {
+    const void* data;         /* device, raw super-blocks */
+    uint32_t ggml_type;       /* PTM_TYPE_Q4_K or PTM_TYPE_Q6_K */
+    int32_t rows, cols;       /* N, K */
+    int64_t row_stride_bytes;
+} ptm_qweight; /* the device half of QuantizedWeight, gguf_model.h:336-385 */
+
+typedef struct {
+    ptm_qweight q, k, v, o, gate, up, down;
+    const float *attn_norm, *ffn_norm, *q_norm, *k_norm; /* device fp32 */
+    void *k_cache, *v_cache; /* device [max_seq][kv_dim], fp16 or fp32 per kv_fp16 */
+} ptm_layer;
+
+typedef struct {
+    int32_t vocab, hidden, n_layers, n_heads, n_kv_heads, head_dim, inter, max_seq;
+    float rope_freq_base, rms_eps;
+    int32_t kv_fp16;              /* 1: fp16 KV cache, 0: fp32 (as the reference's decode) */
+    int32_t use_graph;            /* 1: capture the token step in a hipGraph and replay it */
+    const float* embedding_f32;   /* device [vocab][hidden] fp32, or NULL to use lm_head rows (Q6_K, tied) */
+    const ptm_layer* layers;      /* HOST array of n_layers descriptors (copied) */
+    const float* out_norm;        /* device */
+    ptm_qweight lm_head;
+} ptm_decode_config;
+
+typedef struct ptm_decoder ptm_decoder;
+
+/* Allocates scratch, the RoPE table, the decode stream and device scalars once; nothing is
+ * allocated afterwards.  The KV caches and weights stay caller-owned. */
+int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out);
+void ptm_decode_destroy(ptm_decoder* d);
+/* Set the number of positions already present in the KV caches (after prefill). */
+int ptm_decode_set_past_len(ptm_decoder* d, int64_t past_len);
+/* One greedy step: feeds token_id at position past_len, returns the argmax token through
+ * *next_token (host), advances past_len.  Synchronous like forward_decode + GPU argmax
+ * (gguf_model.h:3107, :4850-4859). */
+int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token);
+/* n greedy steps feeding each output back in, without host round trips between tokens:
+ * tokens_out[n] (host). */
+int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_out);
+/* Device pointers to the last step's logits [vocab] and final-normed hidden [hidden]. */
+const float* ptm_decode_logits(ptm_decoder* d);
+const float* ptm_decode_hidden(ptm_decoder* d);
+void* ptm_decode_stream(ptm_decoder* d);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PTM_H */

@@ -344,8 +344,9 @@ static inline __m256 exp8(__m256 x) {
     x = _mm256_max_ps(_mm256_min_ps(x, _mm256_set1_ps(88.3762626647949f)), _mm256_set1_ps(-88.3762626647949f));
     const __m256 n = _mm256_round_ps(_mm256_mul_ps(x, _mm256_set1_ps(1.44269504088896341f)),
                                      _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC);
-    x = _mm256_sub_ps(x, _mm256_mul_ps(n, _mm256_set1_ps(0.693359375f)));
-    x = _mm256_sub_ps(x, _mm256_mul_ps(n, _mm256_set1_ps(-2.12194440e-4f)));
+    /* the reference build fuses both "x - n*c" steps of the range reduction */
+    x = _mm256_fnmadd_ps(n, _mm256_set1_ps(0.693359375f), x);
+    x = _mm256_fnmadd_ps(n, _mm256_set1_ps(-2.12194440e-4f), x);
     static const float coef[5] = {1.3981999507E-3f, 8.3334519073E-3f, 4.1665795894E-2f,
                                   1.6666665459E-1f, 5.0000001201E-1f};
     __m256 y = _mm256_set1_ps(1.9875691500E-4f);

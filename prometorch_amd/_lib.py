@@ -1,0 +1,109 @@
+"""ctypes binding of libptm_hip.so (the C ABI declared in include/ptm.h).
+
+There is no fallback: if the library has not been built, or an entry point is missing,
+loading raises.  Build it with `python -m prometorch_amd.build` (hipcc, gfx950)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libptm_hip.so")
+
+vp, i64, i32, u32, f32 = C.c_void_p, C.c_int64, C.c_int, C.c_uint32, C.c_float
+
+
+class PtmError(RuntimeError):
+    def __init__(self, code: int, what: str):
+        super().__init__(f"{what}: {code}")
+        self.code = code
+
+
+class QWeight(C.Structure):
+    _fields_ = [("data", vp), ("ggml_type", u32), ("rows", C.c_int32), ("cols", C.c_int32), ("row_stride_bytes", i64)]
+
+
+class Layer(C.Structure):
+    _fields_ = [(n, QWeight) for n in ("q", "k", "v", "o", "gate", "up", "down")] + \
+               [(n, vp) for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "k_cache", "v_cache")]
+
+
+class DecodeConfig(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")] + \
+               [("rope_freq_base", f32), ("rms_eps", f32), ("kv_fp16", C.c_int32), ("use_graph", C.c_int32),
+                ("embedding_f32", vp), ("layers", C.POINTER(Layer)), ("out_norm", vp), ("lm_head", QWeight)]
+
+
+# name -> (restype, argtypes); every function declared in include/ptm.h
+SIGNATURES = {
+    "ptm_strerror": (C.c_char_p, [i32]),
+    "ptm_last_hip_error": (i32, []),
+    "ptm_version": (i32, []),
+    "ptm_device_cus": (i32, []),
+    "ptm_dequant_q4k": (i32, [vp, vp, i64, vp]),
+    "ptm_dequant_q6k": (i32, [vp, vp, i64, vp]),
+    "ptm_dequant_q4k_to_fp16": (i32, [vp, vp, i32, i32, i64, vp]),
+    "ptm_q8_bytes": (i64, [i32]),
+    "ptm_quantize_q8": (i32, [vp, vp, i32, vp]),
+    "ptm_q4k_gemv": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
+    "ptm_q4k_gemv_q8": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
+    "ptm_q6k_gemv": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
+    "ptm_argmax_workspace_bytes": (i64, [i32]),
+    "ptm_q6k_gemv_argmax": (i32, [vp, vp, vp, i32, i32, i64, vp, vp, vp]),
+    "ptm_quant_gemv": (i32, [u32, vp, vp, vp, i32, i32, i64, i32, vp]),
+    "ptm_q4k_fused_gate_up_gemv": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i64, vp]),
+    "ptm_q4k_fused_qkv_gemv": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, vp]),
+    "ptm_q4k_fused_rmsnorm_gemv": (i32, [vp, vp, vp, vp, i32, i32, i64, f32, i32, vp]),
+    "ptm_q4k_fused_rmsnorm_qkv_gemv": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, f32, i32, vp]),
+    "ptm_q4k_fused_rmsnorm_gate_up_gemv": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, i64, f32, i32, vp]),
+    "ptm_q4k_fused_rmsnorm_gate_up_silu": (i32, [vp, vp, vp, vp, vp, i32, i32, i64, f32, i32, vp]),
+    "ptm_rms_norm": (i32, [vp, vp, vp, i32, i32, f32, i32, vp, vp]),
+    "ptm_per_head_rms_norm": (i32, [vp, vp, i32, i32, i32, f32, i32, vp]),
+    "ptm_qknorm_rope_kvwrite": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, vp, f32, i32, i32, i32, vp]),
+    "ptm_rope_table_host": (i32, [vp, i32, i32, f32]),
+    "ptm_fp16_kv_cache_write": (i32, [vp, vp, i64, i64, i64, vp]),
+    "ptm_flash_decode_kv_chunk_size": (i32, []),
+    "ptm_flash_decode_num_splits": (i32, [i32]),
+    "ptm_flash_decode": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, i32, vp]),
+    "ptm_silu_mul": (i32, [vp, vp, vp, i64, vp]),
+    "ptm_embedding_row": (i32, [vp, vp, vp, i32, vp]),
+    "ptm_embedding_row_q6k": (i32, [vp, vp, vp, i32, i64, vp]),
+    "ptm_argmax": (i32, [vp, vp, i64, vp]),
+    "ptm_add": (i32, [vp, vp, vp, i64, vp]),
+    "ptm_copy": (i32, [vp, vp, i64, vp]),
+    "ptm_qgemm_workspace_bytes": (i64, [i32, i32]),
+    "ptm_qgemm_q4k": (i32, [vp, vp, vp, i32, i32, i32, i64, vp, vp]),
+    "ptm_qgemm_q6k": (i32, [vp, vp, vp, i32, i32, i32, i64, vp, vp]),
+    "ptm_decode_create": (i32, [C.POINTER(DecodeConfig), C.POINTER(vp)]),
+    "ptm_decode_destroy": (None, [vp]),
+    "ptm_decode_set_past_len": (i32, [vp, i64]),
+    "ptm_decode_step": (i32, [vp, i32, C.POINTER(i64)]),
+    "ptm_decode_greedy": (i32, [vp, i32, i32, C.POINTER(i64)]),
+    "ptm_decode_logits": (vp, [vp]),
+    "ptm_decode_hidden": (vp, [vp]),
+    "ptm_decode_stream": (vp, [vp]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the library and bind every declared symbol; raises if anything is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(f"{LIB_PATH} is not built: run `python -m prometorch_amd.build` (hipcc --offload-arch=gfx950)")
+    L = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(L, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = L
+    return L
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = load().ptm_strerror(code).decode()
+        raise PtmError(code, f"{what}: {msg}")

@@ -1,0 +1,289 @@
+// Batch-1 greedy decode runtime: the MI355X counterpart of GGUFModel::forward_decode
+// (reference: torch/io/gguf_model.h:2575-3113) and of the greedy argmax that follows it
+// (:4850-4859).  One HIP stream, scratch allocated once, the whole token step captured in a
+// hipGraph; the position and the current token live in device memory, and the last kernel of a
+// step feeds the argmax back as the next token, so consecutive tokens need no host round trip.
+//
+// Per layer (Q4_K_M mix: q/k/o/gate/up Q4_K, v/down Q6_K):
+//   rms_norm (+Q8 of the result)            -> xn, xq8
+//   Q4_K {q,k} from xq8 ; Q6_K v from xn    (quant type is dispatched per tensor, as gemv_scratch does)
+//   qknorm + NeoX RoPE + K/V append
+//   split-KV attention + merge
+//   o-proj GEMV accumulating into the residual
+//   rmsnorm + gate + up + SiLU*up in one launch
+//   down-proj GEMV accumulating into the residual
+#include "ptm_common.h"
+
+#include <new>
+#include <vector>
+
+namespace ptm {
+int q4k_gemv_multi(int n_mat, const void* const* W, float* const* y, const int* N, const void* x, bool x_is_q8,
+                   const float* gamma, float eps, int add_one, int K, int64_t stride, bool accumulate, hipStream_t s);
+int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8, const float* gamma, float eps,
+                     int add_one, float* act, int K, int N, int64_t stride, hipStream_t s);
+int q6k_gemv_impl(const void* W, const float* x, float* y, int K, int N, int64_t stride, bool accumulate,
+                  hipStream_t s);
+
+__global__ void set_scalars_kernel(int* d_token, int token, int64_t* d_past, int64_t past, int* d_step) {
+    *d_token = token;
+    *d_past = past;
+    *d_step = 0;
+}
+// end of a step: publish the chosen token, feed it back, advance the position
+__global__ void advance_kernel(const int64_t* d_next, int* d_token, int64_t* d_past, int* d_step,
+                               int64_t* tokens_out, int cap) {
+    const int64_t nx = *d_next;
+    const int st = *d_step;
+    if (st < cap) tokens_out[st] = nx;
+    *d_token = (int)nx;
+    *d_past = *d_past + 1;
+    *d_step = st + 1;
+}
+}  // namespace ptm
+
+using namespace ptm;
+
+struct ptm_decoder {
+    ptm_decode_config cfg{};
+    std::vector<ptm_layer> layers;
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    bool captured = false;
+    void* slab = nullptr;
+    float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *act = nullptr,
+          *gate = nullptr, *up = nullptr, *logits = nullptr, *pO = nullptr, *pL = nullptr, *pM = nullptr,
+          *rope = nullptr;
+    uint8_t* xq8 = nullptr;
+    void* amax_ws = nullptr;
+    int* d_token = nullptr;
+    int* d_step = nullptr;
+    int64_t* d_past = nullptr;
+    int64_t* d_next = nullptr;
+    int64_t* d_tokens = nullptr;
+    int64_t* h_pinned = nullptr;  // [max_seq] pinned host staging for token ids
+    int64_t past_len = 0;
+    int status = PTM_OK;
+};
+
+static int qw_check(const ptm_qweight& w, int rows, int cols) {
+    if (!w.data) return PTM_E_NULL;
+    if (w.rows != rows || w.cols != cols) return PTM_E_SHAPE;
+    if (w.ggml_type != PTM_TYPE_Q4_K && w.ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
+    return PTM_OK;
+}
+
+static int gemv_any(const ptm_qweight& w, const float* x_f32, float* y, bool acc, hipStream_t s) {
+    if (w.ggml_type == PTM_TYPE_Q4_K) {
+        const void* W = w.data;
+        const int N = w.rows;
+        return q4k_gemv_multi(1, &W, &y, &N, x_f32, false, nullptr, 0.f, 0, w.cols, w.row_stride_bytes, acc, s);
+    }
+    return q6k_gemv_impl(w.data, x_f32, y, w.cols, w.rows, w.row_stride_bytes, acc, s);
+}
+
+// Enqueue one token step on d->stream. Everything it reads that changes per token is in device memory.
+static int enqueue_step(ptm_decoder* d) {
+    const ptm_decode_config& c = d->cfg;
+    hipStream_t s = d->stream;
+    const int H = c.hidden, hd = c.head_dim, qd = c.n_heads * hd, kvd = c.n_kv_heads * hd;
+    int rc;
+#define PTM_TRY(call) do { rc = (call); if (rc != PTM_OK) return rc; } while (0)
+    if (c.embedding_f32) PTM_TRY(ptm_embedding_row(c.embedding_f32, d->x, d->d_token, H, s));
+    else PTM_TRY(ptm_embedding_row_q6k(c.lm_head.data, d->x, d->d_token, H, c.lm_head.row_stride_bytes, s));
+
+    for (int li = 0; li < c.n_layers; ++li) {
+        const ptm_layer& L = d->layers[li];
+        // attention norm; Q8 copy for the Q4_K projections
+        PTM_TRY(ptm_rms_norm(d->x, L.attn_norm, d->xn, 1, H, c.rms_eps, 0, d->xq8, s));
+        {
+            // Q4_K projections share one launch and the Q8 activations; Q6_K ones read fp32 xn
+            const ptm_qweight* w[3] = {&L.q, &L.k, &L.v};
+            float* y[3] = {d->q, d->k, d->v};
+            const void* W4[3]; float* y4[3]; int N4[3]; int n4 = 0;
+            for (int i = 0; i < 3; ++i) {
+                if (w[i]->ggml_type == PTM_TYPE_Q4_K) {
+                    W4[n4] = w[i]->data; y4[n4] = y[i]; N4[n4] = w[i]->rows; ++n4;
+                } else {
+                    PTM_TRY(gemv_any(*w[i], d->xn, y[i], false, s));
+                }
+            }
+            if (n4 > 0)
+                PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->xq8, true, nullptr, 0.f, 0, H, (int64_t)(H / 256) * 144, false, s));
+        }
+        PTM_TRY(ptm_qknorm_rope_kvwrite(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, c.n_heads,
+                                        c.n_kv_heads, hd, d->d_past, c.max_seq, c.rope_freq_base, d->rope, c.rms_eps,
+                                        0, 1, c.kv_fp16, s));
+        PTM_TRY(ptm_flash_decode(d->q, L.k_cache, L.v_cache, d->attn, d->pO, d->pL, d->pM, c.n_heads, c.n_kv_heads,
+                                 hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd), c.kv_fp16, s));
+        PTM_TRY(gemv_any(L.o, d->attn, d->x, true, s));  // x += Wo . attn
+        if (L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
+            L.gate.row_stride_bytes == L.up.row_stride_bytes && L.gate.rows == L.up.rows) {
+            PTM_TRY(q4k_gate_up_silu(L.gate.data, L.up.data, d->x, false, L.ffn_norm, c.rms_eps, 0, d->act, H,
+                                     L.gate.rows, L.gate.row_stride_bytes, s));
+        } else {
+            PTM_TRY(ptm_rms_norm(d->x, L.ffn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+            PTM_TRY(gemv_any(L.gate, d->xn, d->gate, false, s));
+            PTM_TRY(gemv_any(L.up, d->xn, d->up, false, s));
+            PTM_TRY(ptm_silu_mul(d->gate, d->up, d->act, c.inter, s));
+        }
+        PTM_TRY(gemv_any(L.down, d->act, d->x, true, s));  // x += Wdown . act
+    }
+    PTM_TRY(ptm_rms_norm(d->x, c.out_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+    if (c.lm_head.ggml_type == PTM_TYPE_Q6_K) {
+        PTM_TRY(ptm_q6k_gemv_argmax(c.lm_head.data, d->xn, d->logits, H, c.vocab, c.lm_head.row_stride_bytes,
+                                    d->d_next, d->amax_ws, s));
+    } else {
+        PTM_TRY(gemv_any(c.lm_head, d->xn, d->logits, false, s));
+        PTM_TRY(ptm_argmax(d->logits, d->d_next, c.vocab, s));
+    }
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->d_next, d->d_token, d->d_past, d->d_step,
+                       d->d_tokens, c.max_seq);
+    return launch_status();
+#undef PTM_TRY
+}
+
+extern "C" {
+
+int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
+    if (!cfg || !out || !cfg->layers || !cfg->out_norm) return PTM_E_NULL;
+    *out = nullptr;
+    const ptm_decode_config& c = *cfg;
+    if (c.vocab <= 0 || c.hidden <= 0 || c.n_layers <= 0 || c.n_heads <= 0 || c.n_kv_heads <= 0 || c.inter <= 0 ||
+        c.max_seq <= 0 || (c.hidden % 256) || (c.inter % 256) || ((c.n_heads * c.head_dim) % 256) ||
+        (c.n_heads % c.n_kv_heads))
+        return PTM_E_SHAPE;
+    if (c.head_dim != 64 && c.head_dim != 128) return PTM_E_UNSUPPORTED;
+    const int H = c.hidden, qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim;
+    int rc = qw_check(c.lm_head, c.vocab, H);
+    if (rc != PTM_OK) return rc;
+    if (!c.embedding_f32 && c.lm_head.ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
+    for (int i = 0; i < c.n_layers; ++i) {
+        const ptm_layer& L = c.layers[i];
+        if (!L.attn_norm || !L.ffn_norm || !L.q_norm || !L.k_norm || !L.k_cache || !L.v_cache) return PTM_E_NULL;
+        if ((rc = qw_check(L.q, qd, H)) || (rc = qw_check(L.k, kvd, H)) || (rc = qw_check(L.v, kvd, H)) ||
+            (rc = qw_check(L.o, H, qd)) || (rc = qw_check(L.gate, c.inter, H)) || (rc = qw_check(L.up, c.inter, H)) ||
+            (rc = qw_check(L.down, H, c.inter)))
+            return rc;
+    }
+    ptm_decoder* d = new (std::nothrow) ptm_decoder();
+    if (!d) return PTM_E_STATE;
+    d->cfg = c;
+    d->layers.assign(c.layers, c.layers + c.n_layers);
+    d->cfg.layers = d->layers.data();
+
+    const int S = ptm_flash_decode_num_splits(c.max_seq);
+    auto up16 = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t o = off; off += up16(bytes); return o; };
+    const size_t o_x = take(4 * (size_t)H), o_xn = take(4 * (size_t)H), o_q = take(4 * (size_t)qd),
+                 o_k = take(4 * (size_t)kvd), o_v = take(4 * (size_t)kvd), o_attn = take(4 * (size_t)qd),
+                 o_act = take(4 * (size_t)c.inter), o_gate = take(4 * (size_t)c.inter),
+                 o_up = take(4 * (size_t)c.inter), o_logits = take(4 * (size_t)c.vocab),
+                 o_pO = take(4 * (size_t)S * c.n_heads * c.head_dim), o_pL = take(4 * (size_t)S * c.n_heads),
+                 o_pM = take(4 * (size_t)S * c.n_heads), o_rope = take(4 * (size_t)c.max_seq * c.head_dim),
+                 o_xq8 = take((size_t)ptm_q8_bytes(H > c.inter ? H : c.inter)),
+                 o_ws = take((size_t)ptm_argmax_workspace_bytes(c.vocab)), o_tok = take(256), o_past = take(256),
+                 o_next = take(256), o_step = take(256), o_tokens = take(8 * (size_t)c.max_seq);
+    if ((rc = hip_status(hipMalloc(&d->slab, off))) != PTM_OK) { delete d; return rc; }
+    uint8_t* base = static_cast<uint8_t*>(d->slab);
+    d->x = (float*)(base + o_x); d->xn = (float*)(base + o_xn); d->q = (float*)(base + o_q);
+    d->k = (float*)(base + o_k); d->v = (float*)(base + o_v); d->attn = (float*)(base + o_attn);
+    d->act = (float*)(base + o_act); d->gate = (float*)(base + o_gate); d->up = (float*)(base + o_up);
+    d->logits = (float*)(base + o_logits); d->pO = (float*)(base + o_pO); d->pL = (float*)(base + o_pL);
+    d->pM = (float*)(base + o_pM); d->rope = (float*)(base + o_rope); d->xq8 = base + o_xq8;
+    d->amax_ws = base + o_ws; d->d_token = (int*)(base + o_tok); d->d_past = (int64_t*)(base + o_past);
+    d->d_next = (int64_t*)(base + o_next); d->d_step = (int*)(base + o_step);
+    d->d_tokens = (int64_t*)(base + o_tokens);
+
+    if ((rc = hip_status(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
+    if ((rc = hip_status(hipHostMalloc((void**)&d->h_pinned, 8 * (size_t)c.max_seq, hipHostMallocDefault))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
+    {
+        std::vector<float> tab((size_t)c.max_seq * c.head_dim);
+        ptm_rope_table_host(tab.data(), c.max_seq, c.head_dim, c.rope_freq_base);
+        if ((rc = hip_status(hipMemcpy(d->rope, tab.data(), tab.size() * 4, hipMemcpyHostToDevice))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
+    }
+    hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, d->stream, d->d_token, 0, d->d_past, (int64_t)0, d->d_step);
+    if ((rc = hip_status(hipStreamSynchronize(d->stream))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
+    *out = d;
+    return PTM_OK;
+}
+
+void ptm_decode_destroy(ptm_decoder* d) {
+    if (!d) return;
+    if (d->stream) (void)hipStreamSynchronize(d->stream);
+    if (d->exec) (void)hipGraphExecDestroy(d->exec);
+    if (d->graph) (void)hipGraphDestroy(d->graph);
+    if (d->h_pinned) (void)hipHostFree(d->h_pinned);
+    if (d->slab) (void)hipFree(d->slab);
+    if (d->stream) (void)hipStreamDestroy(d->stream);
+    delete d;
+}
+
+int ptm_decode_set_past_len(ptm_decoder* d, int64_t past_len) {
+    if (!d) return PTM_E_NULL;
+    if (past_len < 0 || past_len >= d->cfg.max_seq) return PTM_E_RANGE;
+    d->past_len = past_len;
+    return PTM_OK;
+}
+
+// Run n chained steps starting from `token`; token ids land in d_tokens[0..n) and h_pinned[0..n).
+static int run_steps(ptm_decoder* d, int token, int n) {
+    if (d->status != PTM_OK) return PTM_E_STATE;
+    if (n <= 0) return PTM_E_SHAPE;
+    if (token < 0 || token >= d->cfg.vocab) return PTM_E_RANGE;
+    if (d->past_len + n > d->cfg.max_seq) return PTM_E_RANGE;  // KV cache would overflow
+    hipStream_t s = d->stream;
+    hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, s, d->d_token, token, d->d_past, d->past_len, d->d_step);
+    int rc = launch_status();
+    if (rc != PTM_OK) return rc;
+    int done = 0;
+    if (d->cfg.use_graph && !d->captured) {
+        // first step eagerly (sets one-time kernel attributes outside capture), then capture
+        if ((rc = enqueue_step(d)) != PTM_OK) return d->status = rc;
+        done = 1;
+        {
+            if ((rc = hip_status(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal))) != PTM_OK) return d->status = rc;
+            const int rc_enq = enqueue_step(d);
+            hipGraph_t g = nullptr;
+            rc = hip_status(hipStreamEndCapture(s, &g));
+            if (rc_enq != PTM_OK || rc != PTM_OK) {
+                if (g) (void)hipGraphDestroy(g);
+                return d->status = (rc_enq != PTM_OK ? rc_enq : rc);
+            }
+            d->graph = g;
+            if ((rc = hip_status(hipGraphInstantiate(&d->exec, g, nullptr, nullptr, 0))) != PTM_OK) return d->status = rc;
+            d->captured = true;
+        }
+    }
+    for (; done < n; ++done) {
+        if (d->captured) rc = hip_status(hipGraphLaunch(d->exec, s));
+        else rc = enqueue_step(d);
+        if (rc != PTM_OK) return d->status = rc;
+    }
+    if ((rc = hip_status(hipMemcpyAsync(d->h_pinned, d->d_tokens, 8 * (size_t)n, hipMemcpyDeviceToHost, s))) != PTM_OK) return d->status = rc;
+    if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return d->status = rc;
+    d->past_len += n;
+    return PTM_OK;
+}
+
+int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token) {
+    if (!d || !next_token) return PTM_E_NULL;
+    const int rc = run_steps(d, token_id, 1);
+    if (rc == PTM_OK) *next_token = d->h_pinned[0];
+    return rc;
+}
+
+int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_out) {
+    if (!d || !tokens_out) return PTM_E_NULL;
+    const int rc = run_steps(d, first_token, n);
+    if (rc == PTM_OK) for (int i = 0; i < n; ++i) tokens_out[i] = d->h_pinned[i];
+    return rc;
+}
+
+const float* ptm_decode_logits(ptm_decoder* d) { return d ? d->logits : nullptr; }
+const float* ptm_decode_hidden(ptm_decoder* d) { return d ? d->xn : nullptr; }
+void* ptm_decode_stream(ptm_decoder* d) { return d ? d->stream : nullptr; }
+
+}  // extern "C"

@@ -1,0 +1,327 @@
+// Q4_K dequant-fused GEMV for gfx950 (wave64).
+//
+// Arithmetic follows the reference CPU kernel (torch/io/cpu_quant_gemv.h:505-685): the
+// activation vector is quantised to Q8 blocks of 32 (cpu_quant_gemv.h:147-198), each 32-wide
+// sub-block contributes  fma(d*sc*dx, (float)isum, -(dmin*m*sx))  with isum the exact int32
+// dot of 4-bit weights and int8 activations; only the order in which the per-sub-block terms
+// are added differs (per-lane chains + an 8-lane tree instead of two scalar chains).
+//
+// Data movement: one row is swept by an aligned group of 8 lanes; per super-block (144 B) lane j
+// fetches the 16-byte header {d, dmin, scales[12]} and the j-th 16-byte slice of qs[128] with
+// 128-bit loads, so a wave reads 8 rows x 144 B per step and every fetched byte is used.  A slice
+// holds 16 low nibbles (sub-block 2*(j/2)) and 16 high nibbles (sub-block 2*(j/2)+1); lane pairs
+// swap halves through one DPP move so that lane j ends up owning the complete integer dot of
+// sub-block j.  Q8 activations live in LDS (K + K/4 bytes) and are shared by the 32 rows of a
+// workgroup.
+#include "ptm_common.h"
+
+namespace ptm {
+
+struct Q4KArgs {
+    const uint8_t* W[3];
+    float* y[3];
+    int row_end[3];  // cumulative row counts of the (up to 3) matrices
+    int n_mat;
+    int total_rows;
+    int K;
+    int64_t stride;
+    const void* x;       // fp32 x[K] (XQ8 == false) or Q8 blocks (XQ8 == true)
+    const float* gamma;  // RMSNorm weight (NORM)
+    float eps;
+    int add_one;
+};
+
+enum { Q4K_THREADS = 256, Q4K_ROWS_PER_WG = 32 };
+
+// ---- prologue: bring the Q8 activation into LDS -------------------------------------------
+template <bool XQ8, bool NORM>
+__device__ __forceinline__ void q4k_stage_x(const Q4KArgs& a, uint8_t* lds) {
+    const int K = a.K;
+    const int tid = threadIdx.x;
+    if constexpr (XQ8) {
+        const uint4* src = reinterpret_cast<const uint4*>(a.x);
+        uint4* dst = reinterpret_cast<uint4*>(lds);
+        const int n16 = (K + K / 4) / 16;
+        for (int i = tid; i < n16; i += Q4K_THREADS) dst[i] = src[i];
+    } else {
+        const float4* x4 = reinterpret_cast<const float4*>(a.x);
+        float rs = 1.0f;
+        if constexpr (NORM) {
+            __shared__ float red[4];
+            float ss = 0.0f;
+            for (int i = tid; i < K / 4; i += Q4K_THREADS) {
+                const float4 v = x4[i];
+                ss = fmaf(v.x, v.x, ss);
+                ss = fmaf(v.y, v.y, ss);
+                ss = fmaf(v.z, v.z, ss);
+                ss = fmaf(v.w, v.w, ss);
+            }
+            ss = block_sum256(ss, red);
+            rs = 1.0f / sqrtf(ss / (float)K + a.eps);
+        }
+        int8_t* qs = reinterpret_cast<int8_t*>(lds);
+        float* xd = reinterpret_cast<float*>(lds + K);
+        float* xs = xd + K / 32;
+        // K/4 float4 slots, 8 consecutive slots = one Q8 block; K % 256 == 0 keeps lane groups whole
+        for (int i = tid; i < K / 4; i += Q4K_THREADS) {
+            float4 v = x4[i];
+            if constexpr (NORM) {
+                const float4 g = reinterpret_cast<const float4*>(a.gamma)[i];
+                const float one = a.add_one ? 1.0f : 0.0f;
+                v.x = v.x * rs * (g.x + one);
+                v.y = v.y * rs * (g.y + one);
+                v.z = v.z * rs * (g.z + one);
+                v.w = v.w * rs * (g.w + one);
+            }
+            float d, s;
+            const uint32_t packed = q8_quantize4(v, d, s);
+            reinterpret_cast<uint32_t*>(qs)[i] = packed;
+            if ((tid & 7) == 0) {
+                xd[i >> 3] = d;
+                xs[i >> 3] = s;
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// ---- one row: lane j of the 8-lane group returns its partial (sum over blocks of sub-block j) ---
+template <int U>
+__device__ __forceinline__ float q4k_row_partial(const uint8_t* __restrict__ row, int nblk,
+                                                 const uint8_t* __restrict__ lds, int K, int j) {
+    const int8_t* xq = reinterpret_cast<const int8_t*>(lds);
+    const float* xd = reinterpret_cast<const float*>(lds + K);
+    const float* xs = xd + K / 32;
+    const int g = j >> 1, half = j & 1;
+    const int xoff = g * 64 + half * 16;  // low-nibble activations; high-nibble ones are +32
+    float acc = 0.0f;
+    for (int b0 = 0; b0 < nblk; b0 += U) {
+        uint4 hdr[U], qv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int b = min(b0 + u, nblk - 1);
+            const uint8_t* p = row + (int64_t)b * 144;
+            hdr[u] = *reinterpret_cast<const uint4*>(p);
+            qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int b = b0 + u;
+            if (b < nblk) {
+                const int4 xl = *reinterpret_cast<const int4*>(xq + b * 256 + xoff);
+                const int4 xh = *reinterpret_cast<const int4*>(xq + b * 256 + xoff + 32);
+                int lo = 0, hi = 0;
+                lo = __builtin_amdgcn_sdot4((int)(qv[u].x & 0x0f0f0f0fu), xl.x, lo, false);
+                lo = __builtin_amdgcn_sdot4((int)(qv[u].y & 0x0f0f0f0fu), xl.y, lo, false);
+                lo = __builtin_amdgcn_sdot4((int)(qv[u].z & 0x0f0f0f0fu), xl.z, lo, false);
+                lo = __builtin_amdgcn_sdot4((int)(qv[u].w & 0x0f0f0f0fu), xl.w, lo, false);
+                hi = __builtin_amdgcn_sdot4((int)((qv[u].x >> 4) & 0x0f0f0f0fu), xh.x, hi, false);
+                hi = __builtin_amdgcn_sdot4((int)((qv[u].y >> 4) & 0x0f0f0f0fu), xh.y, hi, false);
+                hi = __builtin_amdgcn_sdot4((int)((qv[u].z >> 4) & 0x0f0f0f0fu), xh.z, hi, false);
+                hi = __builtin_amdgcn_sdot4((int)((qv[u].w >> 4) & 0x0f0f0f0fu), xh.w, hi, false);
+                // even lane keeps the low-nibble half-dot and receives its partner's; odd lane the high one
+                const int keep = half ? hi : lo;
+                const int give = half ? lo : hi;
+                const int isum = keep + dpp_i<0xB1>(give);
+                int sc, mn;
+                q4k_scale_min(hdr[u].y, hdr[u].z, hdr[u].w, j, sc, mn);
+                const float d = h2f(hdr[u].x), dmin = h2f(hdr[u].x >> 16);
+                const float w = d * (float)sc * xd[b * 8 + j];
+                const float c = dmin * (float)mn * xs[b * 8 + j];
+                acc += fmaf(w, (float)isum, -c);
+            }
+        }
+    }
+    return acc;
+}
+
+__device__ __forceinline__ float silu_mul_ref(float g, float u) {
+    // reference: gguf_model.h:3741-3755 (clamp, libm exp, 1/(1+e), g*sig, *u)
+    float ng = 0.0f - g;
+    ng = fminf(fmaxf(ng, -88.0f), 88.0f);
+    const float sig = 1.0f / (1.0f + expf(ng));
+    return (g * sig) * u;
+}
+
+// MODE 0: plain (y = or += W.x for up to three matrices over a flattened row space)
+// MODE 1: gate/up pair with SiLU: y[0][r] = silu(Wg[r].x) * (Wu[r].x)
+template <bool XQ8, bool NORM, bool ACC, int MODE, int U>
+__global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_kernel(const Q4KArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    q4k_stage_x<XQ8, NORM>(a, lds);
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane & 7;
+    const int r = blockIdx.x * Q4K_ROWS_PER_WG + wave * 8 + (lane >> 3);
+    const bool live = r < a.total_rows;
+    const int rr = live ? r : a.total_rows - 1;
+    const int nblk = a.K / 256;
+
+    if constexpr (MODE == 1) {
+        float pg = q4k_row_partial<U>(a.W[0] + (int64_t)rr * a.stride, nblk, lds, a.K, j);
+        float pu = q4k_row_partial<U>(a.W[1] + (int64_t)rr * a.stride, nblk, lds, a.K, j);
+        pg = sum8(pg);
+        pu = sum8(pu);
+        if (live && j == 0) a.y[0][rr] = silu_mul_ref(pg, pu);
+    } else {
+        int mat = 0, local = rr;
+        if (a.n_mat > 1 && rr >= a.row_end[0]) { mat = 1; local = rr - a.row_end[0]; }
+        if (a.n_mat > 2 && rr >= a.row_end[1]) { mat = 2; local = rr - a.row_end[1]; }
+        const uint8_t* W = mat == 0 ? a.W[0] : (mat == 1 ? a.W[1] : a.W[2]);
+        float* y = mat == 0 ? a.y[0] : (mat == 1 ? a.y[1] : a.y[2]);
+        float p = q4k_row_partial<U>(W + (int64_t)local * a.stride, nblk, lds, a.K, j);
+        p = sum8(p);
+        if (live && j == 0) {
+            if constexpr (ACC) y[local] += p;
+            else y[local] = p;
+        }
+    }
+}
+
+template <bool XQ8, bool NORM, bool ACC, int MODE>
+static int q4k_launch(const Q4KArgs& a, hipStream_t s) {
+    const int grid = (a.total_rows + Q4K_ROWS_PER_WG - 1) / Q4K_ROWS_PER_WG;
+    const size_t lds = (size_t)q8_bytes(a.K);
+    const int nblk = a.K / 256;
+    // blocks in flight per row: whole row when short, otherwise 8..10 per pass
+    if (nblk <= 4) hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 4>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
+    else if (nblk % 10 == 0 || nblk == 38) hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 10>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
+    else hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 8>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
+    return launch_status();
+}
+
+static int q4k_check(const void* W, const void* x, const void* y, int K, int N, int64_t stride) {
+    if (!W || !x || !y) return PTM_E_NULL;
+    if (K <= 0 || N <= 0 || (K % 256) != 0) return PTM_E_SHAPE;
+    if (K > 32768) return PTM_E_UNSUPPORTED;  // Q8 activations must fit the 40 KB LDS budget used here
+    if (stride < (int64_t)(K / 256) * 144) return PTM_E_SHAPE;
+    if ((stride & 15) != 0 || !aligned16(W) || !aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 3u)) return PTM_E_ALIGN;
+    return PTM_OK;
+}
+
+// Shared by the C entry points and the decode runtime.
+int q4k_gemv_multi(int n_mat, const void* const* W, float* const* y, const int* N, const void* x, bool x_is_q8,
+                   const float* gamma, float eps, int add_one, int K, int64_t stride, bool accumulate,
+                   hipStream_t s) {
+    Q4KArgs a{};
+    int total = 0;
+    for (int i = 0; i < n_mat; ++i) {
+        const int rc = q4k_check(W[i], x, y[i], K, N[i], stride);
+        if (rc != PTM_OK) return rc;
+        a.W[i] = static_cast<const uint8_t*>(W[i]);
+        a.y[i] = y[i];
+        total += N[i];
+        a.row_end[i] = total;
+    }
+    a.n_mat = n_mat;
+    a.total_rows = total;
+    a.K = K;
+    a.stride = stride;
+    a.x = x;
+    a.gamma = gamma;
+    a.eps = eps;
+    a.add_one = add_one;
+    if (gamma) {
+        if (x_is_q8) return PTM_E_UNSUPPORTED;
+        if (!aligned16(gamma)) return PTM_E_ALIGN;
+        return accumulate ? q4k_launch<false, true, true, 0>(a, s) : q4k_launch<false, true, false, 0>(a, s);
+    }
+    if (x_is_q8) return accumulate ? q4k_launch<true, false, true, 0>(a, s) : q4k_launch<true, false, false, 0>(a, s);
+    return accumulate ? q4k_launch<false, false, true, 0>(a, s) : q4k_launch<false, false, false, 0>(a, s);
+}
+
+int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8, const float* gamma, float eps,
+                     int add_one, float* act, int K, int N, int64_t stride, hipStream_t s) {
+    int rc = q4k_check(wg, x, act, K, N, stride);
+    if (rc != PTM_OK) return rc;
+    rc = q4k_check(wu, x, act, K, N, stride);
+    if (rc != PTM_OK) return rc;
+    Q4KArgs a{};
+    a.W[0] = static_cast<const uint8_t*>(wg);
+    a.W[1] = static_cast<const uint8_t*>(wu);
+    a.y[0] = act;
+    a.n_mat = 2;
+    a.row_end[0] = N;
+    a.total_rows = N;
+    a.K = K;
+    a.stride = stride;
+    a.x = x;
+    a.gamma = gamma;
+    a.eps = eps;
+    a.add_one = add_one;
+    if (gamma) {
+        if (x_is_q8) return PTM_E_UNSUPPORTED;
+        if (!aligned16(gamma)) return PTM_E_ALIGN;
+        return q4k_launch<false, true, false, 1>(a, s);
+    }
+    return x_is_q8 ? q4k_launch<true, false, false, 1>(a, s) : q4k_launch<false, false, false, 1>(a, s);
+}
+
+}  // namespace ptm
+
+using namespace ptm;
+
+extern "C" {
+
+int ptm_q4k_gemv(const void* W, const float* x, float* y, int K, int N, int64_t stride, int accumulate,
+                 ptm_stream_t stream) {
+    return q4k_gemv_multi(1, &W, &y, &N, x, false, nullptr, 0.f, 0, K, stride, accumulate != 0, as_stream(stream));
+}
+
+int ptm_q4k_gemv_q8(const void* W, const void* x_q8, float* y, int K, int N, int64_t stride, int accumulate,
+                    ptm_stream_t stream) {
+    return q4k_gemv_multi(1, &W, &y, &N, x_q8, true, nullptr, 0.f, 0, K, stride, accumulate != 0, as_stream(stream));
+}
+
+int ptm_q4k_fused_gate_up_gemv(const void* w_gate, const void* w_up, const float* x, float* y_gate, float* y_up,
+                               int K, int N_gate, int N_up, int64_t stride, ptm_stream_t stream) {
+    const void* W[2] = {w_gate, w_up};
+    float* y[2] = {y_gate, y_up};
+    const int N[2] = {N_gate, N_up};
+    return q4k_gemv_multi(2, W, y, N, x, false, nullptr, 0.f, 0, K, stride, false, as_stream(stream));
+}
+
+int ptm_q4k_fused_qkv_gemv(const void* w_q, const void* w_k, const void* w_v, const float* x, float* out_q,
+                           float* out_k, float* out_v, int K, int N_q, int N_k, int N_v, int64_t stride,
+                           ptm_stream_t stream) {
+    const void* W[3] = {w_q, w_k, w_v};
+    float* y[3] = {out_q, out_k, out_v};
+    const int N[3] = {N_q, N_k, N_v};
+    return q4k_gemv_multi(3, W, y, N, x, false, nullptr, 0.f, 0, K, stride, false, as_stream(stream));
+}
+
+int ptm_q4k_fused_rmsnorm_gemv(const float* x, const float* norm_w, const void* W, float* y, int K, int N,
+                               int64_t stride, float eps, int add_one, ptm_stream_t stream) {
+    if (!norm_w) return PTM_E_NULL;
+    return q4k_gemv_multi(1, &W, &y, &N, x, false, norm_w, eps, add_one, K, stride, false, as_stream(stream));
+}
+
+int ptm_q4k_fused_rmsnorm_qkv_gemv(const float* x, const float* norm_w, const void* w_q, const void* w_k,
+                                   const void* w_v, float* out_q, float* out_k, float* out_v, int K, int N_q,
+                                   int N_k, int N_v, int64_t stride, float eps, int add_one,
+                                   ptm_stream_t stream) {
+    if (!norm_w) return PTM_E_NULL;
+    const void* W[3] = {w_q, w_k, w_v};
+    float* y[3] = {out_q, out_k, out_v};
+    const int N[3] = {N_q, N_k, N_v};
+    return q4k_gemv_multi(3, W, y, N, x, false, norm_w, eps, add_one, K, stride, false, as_stream(stream));
+}
+
+int ptm_q4k_fused_rmsnorm_gate_up_gemv(const float* x, const float* norm_w, const void* w_gate,
+                                       const void* w_up, float* y_gate, float* y_up, int K, int N_gate,
+                                       int N_up, int64_t stride, float eps, int add_one, ptm_stream_t stream) {
+    if (!norm_w) return PTM_E_NULL;
+    const void* W[2] = {w_gate, w_up};
+    float* y[2] = {y_gate, y_up};
+    const int N[2] = {N_gate, N_up};
+    return q4k_gemv_multi(2, W, y, N, x, false, norm_w, eps, add_one, K, stride, false, as_stream(stream));
+}
+
+int ptm_q4k_fused_rmsnorm_gate_up_silu(const float* x, const float* norm_w, const void* w_gate,
+                                       const void* w_up, float* act, int K, int N, int64_t stride, float eps,
+                                       int add_one, ptm_stream_t stream) {
+    if (!norm_w) return PTM_E_NULL;
+    return q4k_gate_up_silu(w_gate, w_up, x, false, norm_w, eps, add_one, act, K, N, stride, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,128 @@
+"""Host-side wrapper of the decode runtime (ptm_decode_*), the counterpart of
+GGUFModel::load_quantized_to_cuda + forward_decode + greedy generate
+(reference: torch/io/gguf_model.h:1177-1360, :2575-3113, :4737-4901).
+
+Weights are uploaded verbatim as raw super-blocks; torch is used only to own device memory."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import DecodeConfig, Layer, QWeight, check
+
+_NAMES = ("q", "k", "v", "o", "gate", "up", "down")
+
+
+def _upload_bytes(a: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.uint8)).cuda()
+
+
+class Decoder:
+    """Greedy batch-1 decoder over caller-provided quantised weights.
+
+    layers: list of dicts with (qtype, uint8[rows, stride]) per projection name and fp32 norm
+    vectors 'attn_norm', 'ffn_norm', 'q_norm', 'k_norm'; head: {'lm_head': uint8 Q6_K table,
+    'out_norm': fp32}.  The token-embedding is the tied Q6_K table unless embedding_f32 is given."""
+
+    def __init__(self, cfg: dict, layers: list, head: dict, max_seq: int, kv_fp16: bool = True,
+                 use_graph: bool = True, embedding_f32=None, device: str = "cuda:0"):
+        self.L = _lib.load()
+        self.cfg = dict(cfg)
+        self.max_seq = max_seq
+        self.kv_fp16 = kv_fp16
+        torch.cuda.set_device(device)
+        self._keep = []
+        kvd = cfg["n_kv_heads"] * cfg["head_dim"]
+        kv_dtype = torch.float16 if kv_fp16 else torch.float32
+        self.k_cache, self.v_cache = [], []
+        arr = (Layer * cfg["n_layers"])()
+        for i, Ld in enumerate(layers):
+            for name in _NAMES:
+                qt, W = Ld[name]
+                t = _upload_bytes(W)
+                self._keep.append(t)
+                bb = 144 if qt == 12 else 210
+                setattr(arr[i], name, QWeight(t.data_ptr(), qt, W.shape[0], W.shape[1] // bb * 256, W.shape[1]))
+            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+                t = torch.from_numpy(np.ascontiguousarray(Ld[name], np.float32)).cuda()
+                self._keep.append(t)
+                setattr(arr[i], name, t.data_ptr())
+            kc = torch.zeros(max_seq, kvd, dtype=kv_dtype, device="cuda")
+            vc = torch.zeros(max_seq, kvd, dtype=kv_dtype, device="cuda")
+            self.k_cache.append(kc)
+            self.v_cache.append(vc)
+            arr[i].k_cache = kc.data_ptr()
+            arr[i].v_cache = vc.data_ptr()
+        self._layers = arr
+        lm = _upload_bytes(head["lm_head"])
+        on = torch.from_numpy(np.ascontiguousarray(head["out_norm"], np.float32)).cuda()
+        self._keep += [lm, on]
+        c = DecodeConfig()
+        for k in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter"):
+            setattr(c, k, cfg[k])
+        c.max_seq = max_seq
+        c.rope_freq_base = cfg["rope_base"]
+        c.rms_eps = cfg["eps"]
+        c.kv_fp16 = int(kv_fp16)
+        c.use_graph = int(use_graph)
+        if embedding_f32 is not None:
+            e = embedding_f32 if isinstance(embedding_f32, torch.Tensor) else torch.from_numpy(embedding_f32)
+            e = e.to(device="cuda", dtype=torch.float32).contiguous()
+            self._keep.append(e)
+            c.embedding_f32 = e.data_ptr()
+        else:
+            c.embedding_f32 = None
+        c.layers = arr
+        c.out_norm = on.data_ptr()
+        c.lm_head = QWeight(lm.data_ptr(), 14, cfg["vocab"], cfg["hidden"], head["lm_head"].shape[1])
+        self._cfg = c
+        torch.cuda.synchronize()
+        h = C.c_void_p()
+        check(self.L.ptm_decode_create(C.byref(c), C.byref(h)), "decode_create")
+        self.h = h
+
+    def set_kv(self, layer: int, k16: np.ndarray, v16: np.ndarray) -> None:
+        """Prefill: write cache rows [0, n) (fp16 values; widened when the cache is fp32)."""
+        n = k16.shape[0]
+        self.k_cache[layer][:n].copy_(torch.from_numpy(k16).to(self.k_cache[layer].dtype))
+        self.v_cache[layer][:n].copy_(torch.from_numpy(v16).to(self.v_cache[layer].dtype))
+
+    def set_past_len(self, n: int) -> None:
+        torch.cuda.synchronize()
+        check(self.L.ptm_decode_set_past_len(self.h, n), "decode_set_past_len")
+
+    def step(self, token: int) -> int:
+        out = C.c_int64()
+        check(self.L.ptm_decode_step(self.h, token, C.byref(out)), "decode_step")
+        return out.value
+
+    def greedy(self, first_token: int, n: int) -> list:
+        buf = (C.c_int64 * n)()
+        check(self.L.ptm_decode_greedy(self.h, first_token, n, buf), "decode_greedy")
+        return list(buf)
+
+    def _view(self, ptr: int, n: int) -> np.ndarray:
+        out = torch.empty(n, dtype=torch.float32, device="cuda")
+        _lib.check(self.L.ptm_copy(ptr, out.data_ptr(), n, None), "copy")
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    def logits(self) -> np.ndarray:
+        return self._view(self.L.ptm_decode_logits(self.h), self.cfg["vocab"])
+
+    def hidden(self) -> np.ndarray:
+        return self._view(self.L.ptm_decode_hidden(self.h), self.cfg["hidden"])
+
+    def close(self) -> None:
+        if getattr(self, "h", None):
+            self.L.ptm_decode_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

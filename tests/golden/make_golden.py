@@ -1,0 +1,252 @@
+"""Writes the golden fixtures under tests/golden/ by running the REFERENCE's own CPU code
+(oracle/_ref/libptm_ref.so, compiled from the reference checkout by `make -C oracle ref`).
+
+Run from the repo root in a container that has the reference checkout:
+    make -C oracle ref && python tests/golden/make_golden.py [--full]
+
+Inputs are regenerated from seeds by prometorch_amd.synth, so the fixtures hold only the
+reference's OUTPUTS (plus a few hand-built edge-case input blocks).  --full also runs the
+Qwen3-4B-shaped model for 128 greedy steps (about 3 GB of synthetic weights, a few minutes)."""
+from __future__ import annotations
+
+import argparse
+import hashlib
+import json
+import os
+import platform
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle import pyoracle as po  # noqa: E402
+from prometorch_amd import synth  # noqa: E402
+
+OUT = os.path.dirname(os.path.abspath(__file__))
+SEEDS = {"blocks": 101, "cfg1": 1001, "cfg2": 1002, "cfg3": 1003, "tiny": 7, "cfg4": 4004, "ragged": 1005}
+
+
+def sha(a: np.ndarray) -> str:
+    return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+def edge_blocks_q4k() -> np.ndarray:
+    """Hand-built Q4_K blocks: zero d, subnormal fp16 d/dmin, max scales, all-0 / all-15 quants."""
+    rng = synth.rng_for(SEEDS["blocks"], 9)
+    b = synth.make_q4k(rng, 8, 256).reshape(8, 144).copy()
+    b[0, 0:4] = 0                                       # d = dmin = 0
+    b[1, 0:2] = np.array([0x0001], np.uint16).view(np.uint8)  # smallest subnormal d
+    b[1, 2:4] = np.array([0x03FF], np.uint16).view(np.uint8)  # largest subnormal dmin
+    b[2, 4:16] = 0xFF                                   # all scales/mins 63
+    b[3, 16:144] = 0x00
+    b[4, 16:144] = 0xFF
+    b[5, 0:2] = np.array([0x7BFF], np.uint16).view(np.uint8)  # max finite d
+    b[6, 4:16] = 0x00
+    return b
+
+
+def edge_blocks_q6k() -> np.ndarray:
+    rng = synth.rng_for(SEEDS["blocks"], 10)
+    b = synth.make_q6k(rng, 8, 256).reshape(8, 210).copy()
+    b[0, 208:210] = 0
+    b[1, 208:210] = np.array([0x0001], np.uint16).view(np.uint8)
+    b[2, 192:208] = np.array([-128], np.int8).view(np.uint8)   # most negative scale
+    b[3, 192:208] = 127
+    b[4, 0:192] = 0x00                                  # q = -32 everywhere
+    b[5, 0:192] = 0xFF                                  # q = 31 everywhere
+    b[6, 208:210] = np.array([0x83FF], np.uint16).view(np.uint8)  # negative subnormal d
+    return b
+
+
+def ref_dequant(qt, raw):
+    raw = np.ascontiguousarray(raw, np.uint8).reshape(-1)
+    n = raw.size // (144 if qt == 12 else 210) * 256
+    out = np.empty(n, np.float32)
+    (po.ref().ref_dequantize_q4_k if qt == 12 else po.ref().ref_dequantize_q6_k)(po._p(raw), po._p(out), n)
+    return out
+
+
+def ref_q8(x):
+    K = x.size
+    d = np.empty(K // 32, np.float32)
+    s = np.empty(K // 32, np.float32)
+    q = np.empty(K, np.int8)
+    po.ref().ref_quantize_x_q8(po._p(x), K, po._p(d), po._p(s), po._p(q))
+    return d, s, q
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--full", action="store_true")
+    args = ap.parse_args()
+    assert po.have_ref(), "build oracle/_ref first: make -C oracle ref"
+    R = po.ref()
+    meta = {"made_with": "oracle/_ref/libptm_ref.so (g++ -O2 -std=c++17 -mavx2 -mfma; see oracle/Makefile)",
+            "python": platform.python_version(), "numpy": np.__version__, "threads": R.ref_num_threads(), "seeds": SEEDS}
+    g = {}
+
+    # ---- fp16 table: all 65536 inputs -----------------------------------------------
+    g["fp16_table_sha"] = np.frombuffer(sha(np.array([R.ref_fp16_to_fp32(h) for h in range(65536)], np.float32)).encode(), np.uint8)
+
+    # ---- blocks: 64 random + 8 edge blocks per format, reference dequant ----------------
+    rng = synth.rng_for(SEEDS["blocks"])
+    q4 = np.concatenate([synth.make_q4k(rng, 64, 256).reshape(64, 144), edge_blocks_q4k()])
+    q6 = np.concatenate([synth.make_q6k(rng, 64, 256).reshape(64, 210), edge_blocks_q6k()])
+    g["q4k_blocks"] = q4
+    g["q4k_deq"] = ref_dequant(12, q4)
+    g["q6k_blocks"] = q6
+    g["q6k_deq"] = ref_dequant(14, q6)
+
+    # ---- Q8 activation quantiser ---------------------------------------------------------
+    x = synth.make_x(rng, 2560)
+    x[32:64] = 0.0                       # all-zero block: d = 0, id = 0
+    x[64] = 127.0; x[65] = 0.5; x[66] = 1.5; x[67] = 2.5; x[68] = -0.5; x[69] = -1.5  # exact .5 ties -> half-even
+    x[64:96][6:] = 0.25
+    g["q8_x"] = x
+    g["q8_d"], g["q8_sum"], g["q8_qs"] = ref_q8(x)
+
+    # ---- cfg1: Q4_K GEMV 9728 x 2560 ------------------------------------------------------
+    r1 = synth.rng_for(SEEDS["cfg1"])
+    W = synth.make_q4k(r1, 9728, 2560)
+    x1 = synth.make_x(r1, 2560)
+    y = po.ref_gemv(12, W, x1)
+    g["cfg1_y256"] = y[:256].copy()
+    g["cfg1_sha"] = np.frombuffer(sha(y).encode(), np.uint8)
+    meta["cfg1_rms"] = float(np.sqrt((y.astype(np.float64) ** 2).mean()))
+    t = time.time()
+    for _ in range(5):
+        po.ref_gemv(12, W, x1)
+    meta["cfg1_ref_ms_8core_container"] = (time.time() - t) / 5 * 1e3
+
+    # ---- ragged / odd shapes (odd N exercises the unpaired-row path) ----------------------
+    rr = synth.rng_for(SEEDS["ragged"])
+    for i, (qt, N, K) in enumerate([(12, 33, 512), (12, 1, 256), (12, 77, 2560), (14, 7, 256), (14, 45, 1024)]):
+        Wr = synth.make_weight(rr, qt, N, K)
+        xr = synth.make_x(rr, K)
+        g[f"ragged{i}_y"] = po.ref_gemv(qt, Wr, xr)
+
+    # ---- cfg2: Q6_K lm_head GEMV + argmax (full size) -------------------------------------
+    r2 = synth.rng_for(SEEDS["cfg2"])
+    W2 = synth.make_q6k(r2, 151936, 2560)
+    x2 = synth.make_x(r2, 2560)
+    y2 = po.ref_gemv(14, W2, x2)
+    top = np.argsort(-y2, kind="stable")[:8]
+    g["cfg2_top8_idx"] = top.astype(np.int64)
+    g["cfg2_top8_val"] = y2[top]
+    g["cfg2_y256"] = y2[:256].copy()
+    g["cfg2_sha"] = np.frombuffer(sha(y2).encode(), np.uint8)
+    g["cfg2_argmax"] = np.array([int(np.argmax(y2))], np.int64)
+    del W2
+
+    # ---- cfg3: one Qwen3-4B layer's seven GEMVs, independent N(0,1) inputs -----------------
+    L = synth.make_layer(SEEDS["cfg3"], 0, synth.QWEN3_4B)
+    for i, (name, qt) in enumerate(synth.LAYER_MATS):
+        _, Wm = L[name]
+        K = Wm.shape[1] // (144 if qt == 12 else 210) * 256
+        xm = synth.make_x(synth.rng_for(SEEDS["cfg3"], 5, i), K)
+        ym = po.ref_gemv(qt, Wm, xm)
+        g[f"cfg3_{name}_y64"] = ym[:: max(1, ym.size // 64)][:64].copy()
+        g[f"cfg3_{name}_sha"] = np.frombuffer(sha(ym).encode(), np.uint8)
+    # fused RMSNorm + gate/up as the reference's CPU fusion computes it
+    xg = (synth.make_x(synth.rng_for(SEEDS["cfg3"], 6), 2560) * 3.0).astype(np.float32)
+    yg = np.empty(9728, np.float32)
+    yu = np.empty(9728, np.float32)
+    Wg = np.ascontiguousarray(L["gate"][1])
+    Wu = np.ascontiguousarray(L["up"][1])
+    gam = np.ascontiguousarray(L["ffn_norm"])
+    R.ref_fused_rmsnorm_gate_up(po._p(xg), po._p(gam), 1e-6, 0, 12, po._p(Wg), 12, po._p(Wu), po._p(yg), po._p(yu),
+                                2560, 9728, 9728, Wg.shape[1], Wu.shape[1])
+    g["cfg3_fused_gate_y64"] = yg[::152][:64].copy()
+    g["cfg3_fused_up_y64"] = yu[::152][:64].copy()
+
+    # ---- glue: rmsnorm, rope, exp ------------------------------------------------------------
+    rg = synth.rng_for(SEEDS["blocks"], 11)
+    xn = synth.make_x(rg, 2560)
+    gm = (1.0 + 0.1 * synth.make_x(rg, 2560)).astype(np.float32)
+    o = xn.copy()
+    R.ref_rmsnorm_inplace(po._p(o), po._p(gm), 1e-6, 0, 2560)
+    g["rms_x"], g["rms_g"], g["rms_out"] = xn, gm, o
+    for pos in (0, 1, 2048, 2175):
+        c = np.empty(64, np.float32)
+        s = np.empty(64, np.float32)
+        R.ref_rope_precompute(po._p(c), po._p(s), pos, 128, 1e6)
+        g[f"rope_cos_{pos}"], g[f"rope_sin_{pos}"] = c, s
+    qv = synth.make_x(rg, 4096)
+    kv = synth.make_x(rg, 1024)
+    g["rope_q_in"], g["rope_k_in"] = qv.copy(), kv.copy()
+    R.ref_rope_apply_neox(po._p(qv), po._p(kv), po._p(g["rope_cos_2048"]), po._p(g["rope_sin_2048"]), 32, 8, 128)
+    g["rope_q_out"], g["rope_k_out"] = qv, kv
+    e = np.linspace(-90, 20, 1024, dtype=np.float32)
+    eo = np.empty_like(e)
+    R.ref_exp256(po._p(e), po._p(eo), e.size // 8)
+    g["exp_in"], g["exp_out"] = e, eo
+
+    # ---- tiny model: full logits of the reference's forward_decode_cpu over 12 steps ----------
+    cfg = dict(synth.TINY)
+    layers = [synth.make_layer(SEEDS["tiny"], i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(SEEDS["tiny"], cfg)
+    emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    rm = po.RefModel(cfg, layers, head, 64, emb)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(SEEDS["tiny"], i, cfg, 19)
+        rm.set_kv(i, k, v)
+    tok, toks, lg = 3, [], []
+    for _ in range(12):
+        tok = rm.step(tok)
+        toks.append(tok)
+        lg.append(rm.logits.copy())
+    g["tiny_tokens"] = np.array(toks, np.int64)
+    g["tiny_logits"] = np.stack(lg)
+    rm.close()
+
+    np.savez_compressed(os.path.join(OUT, "golden_small.npz"), **g)
+
+    if args.full:
+        make_full(meta)
+    with open(os.path.join(OUT, "golden_meta.json"), "w") as f:
+        json.dump(meta, f, indent=1, sort_keys=True)
+    print("wrote", OUT)
+
+
+def make_full(meta):
+    """cfg4: Qwen3-4B shape, 36 layers, KV prefilled to 2048, 128 greedy steps on the reference CPU path
+    (fp32 KV rows for new tokens, as forward_decode_cpu keeps them)."""
+    cfg = dict(synth.QWEN3_4B)
+    seed = SEEDS["cfg4"]
+    t0 = time.time()
+    layers = [synth.make_layer(seed, i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(seed, cfg)
+    print("generated model in %.1fs" % (time.time() - t0), flush=True)
+    emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    max_seq, npos, steps = 2304, 2048, 128
+    rm = po.RefModel(cfg, layers, head, max_seq, emb)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(seed, i, cfg, npos)
+        rm.set_kv(i, k, v)
+    g = {}
+    tok, toks, margins, tops = 1, [], [], []
+    t0 = time.time()
+    for st in range(steps):
+        tok = rm.step(tok)
+        toks.append(tok)
+        srt = np.sort(rm.logits)
+        margins.append(float(srt[-1] - srt[-2]))
+        tops.append(float(srt[-1]))
+        if st in (0, 1, 63, 127):
+            g[f"logits256_step{st}"] = rm.logits[:256].copy()
+            g[f"logits_sha_step{st}"] = np.frombuffer(sha(rm.logits).encode(), np.uint8)
+            g[f"logits_std_step{st}"] = np.array([rm.logits.std()], np.float32)
+        if st % 16 == 0:
+            print("step", st, "tok", tok, "margin", margins[-1], "%.1fs" % (time.time() - t0), flush=True)
+    meta["cfg4_ref_tok_per_s_8core_container"] = steps / (time.time() - t0)
+    g["tokens"] = np.array(toks, np.int64)
+    g["margins"] = np.array(margins, np.float32)
+    g["top1"] = np.array(tops, np.float32)
+    rm.close()
+    np.savez_compressed(os.path.join(OUT, "golden_cfg4.npz"), **g)
+
+
+if __name__ == "__main__":
+    main()

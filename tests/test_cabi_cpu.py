@@ -1,0 +1,79 @@
+"""CPU: the C-ABI library loads and exports every symbol include/ptm.h declares; host-side
+argument validation returns error codes without touching a GPU."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from conftest import ROOT
+from prometorch_amd import _lib
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ptm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ptm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_built_and_exports_every_declared_symbol():
+    assert os.path.exists(_lib.LIB_PATH), "libptm_hip.so is not built (python -m prometorch_amd.build)"
+    raw = C.CDLL(_lib.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 40
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in ptm.h but not exported"
+    assert set(names) == set(_lib.SIGNATURES), set(names) ^ set(_lib.SIGNATURES)
+
+
+def test_shim_header_names_exist_in_abi():
+    shim = open(os.path.join(ROOT, "include", "ptm_at_cuda_shim.h")).read()
+    used = set(re.findall(r"\b(ptm_[a-z0-9_]+)\s*\(", shim))
+    assert used and used <= set(declared_symbols()), used - set(declared_symbols())
+
+
+def test_host_side_validation_codes():
+    L = _lib.load()
+    E_NULL, E_SHAPE, E_ALIGN, E_UNSUP = -1, -2, -3, -4
+    assert L.ptm_q4k_gemv(None, None, None, 256, 4, 144, 0, None) == E_NULL
+    assert L.ptm_q4k_gemv(16, 16, 16, 250, 4, 144, 0, None) == E_SHAPE       # K not a multiple of 256
+    assert L.ptm_q4k_gemv(16, 16, 16, 256, 0, 144, 0, None) == E_SHAPE       # empty N
+    assert L.ptm_q4k_gemv(16, 16, 16, 256, 4, 100, 0, None) == E_SHAPE       # stride < row bytes
+    assert L.ptm_q4k_gemv(24, 16, 16, 256, 4, 144, 0, None) == E_ALIGN
+    assert L.ptm_q4k_gemv(16, 16, 16, 65536, 4, 144 * 256, 0, None) == E_UNSUP
+    assert L.ptm_q6k_gemv(16, 16, 16, 256, 4, 209, 0, None) == E_SHAPE
+    assert L.ptm_q6k_gemv(17, 16, 16, 256, 4, 210, 0, None) == E_ALIGN
+    assert L.ptm_quant_gemv(13, 16, 16, 16, 256, 4, 176, 0, None) == E_UNSUP  # Q5_K: not on this path
+    assert L.ptm_flash_decode(16, 16, 16, 16, 16, 16, 16, 32, 8, 96, 16, 128, 1.0, 1, None) == E_UNSUP
+    assert L.ptm_flash_decode(16, 16, 16, 16, 16, 16, 16, 30, 8, 128, 16, 128, 1.0, 1, None) == E_SHAPE
+    assert L.ptm_dequant_q4k(16, 16, 100, None) == E_SHAPE
+    assert L.ptm_dequant_q4k(16, 16, 0, None) == 0                            # empty input is fine
+    assert L.ptm_rms_norm(16, 16, 16, 2, 256, 1e-6, 0, 16, None) == E_SHAPE   # Q8 output only for one row
+    assert L.ptm_strerror(E_SHAPE).decode().startswith("bad shape")
+    assert L.ptm_q8_bytes(2560) == 2560 + 640
+    assert L.ptm_flash_decode_num_splits(2176) == 34 and L.ptm_flash_decode_kv_chunk_size() == 64
+    assert L.ptm_decode_create(None, None) == E_NULL
+
+
+def test_rope_table_host_matches_oracle(po):
+    from prometorch_amd import ops
+    t = ops.rope_table(40, 128, 1e6).numpy()
+    for pos in (0, 1, 39):
+        c, s = po.rope_tables(pos, 128, 1e6)
+        assert np.array_equal(t[pos, :64].view(np.uint32), c.view(np.uint32))
+        assert np.array_equal(t[pos, 64:].view(np.uint32), s.view(np.uint32))
+
+
+def test_synth_generators_are_deterministic_and_in_range():
+    from prometorch_amd import synth
+    a = synth.make_q4k(synth.rng_for(3), 4, 512)
+    b = synth.make_q4k(synth.rng_for(3), 4, 512)
+    assert np.array_equal(a, b) and a.shape == (4, 288)
+    sc, mn = synth.unpack_scales_k4(a.reshape(-1, 144)[:, 4:16])
+    assert sc.max() <= 63 and mn.max() <= 63
+    w6 = synth.make_q6k(synth.rng_for(3), 4, 512).reshape(-1, 210)
+    s8 = w6[:, 192:208].view(np.int8)
+    assert s8.min() >= -32 and s8.max() <= 31
+    d = w6[:, 208:210].copy().view(np.float16)
+    assert np.all(d >= 0) and np.all(np.isfinite(d))
