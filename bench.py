@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF k-quant decode path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps 128] [--warmup 8]
+
+A "step" is one greedy decode token of the Qwen3-4B-shaped Q4_K_M model (36 layers, hidden 2560,
+32 q / 8 kv heads, head_dim 128, ffn 9728, vocab 151936; random-init seeded super-blocks; fp16 KV
+cache prefilled with 2048 seeded positions), i.e. BASELINE.json configs[3].  Weights, KV cache and
+scratch are resident in HBM before the timed region starts.  One JSON line is printed on stdout.
+
+Besides the token rate the line carries
+  roofline      the dominant kernel (fused RMSNorm + Q4_K gate/up GEMV + SiLU, 2 x 9728 x 2560),
+                algorithmic bytes per launch / average launch duration measured with HIP events on
+                the launching stream, cycling over the 36 layers' distinct weights (1 GB footprint)
+  gemv          the same measurement for configs[0] (Q4_K 9728x2560) and configs[1] (Q6_K lm_head)
+  cpu_baseline  the reference's CPU path (oracle/_ref build if present, else this repo's C port)
+                timed on this host for a bounded number of tokens of the same workload
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+SEED = 4004
+N_PREFILL = 2048
+MAX_SEQ = 2304
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def event_time_ms(fn, iters, torch):
+    """Average duration of fn() over `iters` back-to-back launches, HIP events on the current stream."""
+    s = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(min(iters, 8)):
+        fn(i)
+    s.synchronize()
+    e0.record(s)
+    for i in range(iters):
+        fn(i)
+    e1.record(s)
+    s.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--layers", type=int, default=36, help=argparse.SUPPRESS)  # debugging only; 36 is the workload
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on ONE GPU (batch-1 decode); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    if args.steps + args.warmup + N_PREFILL + 1 > MAX_SEQ:
+        print("bench.py: steps + warmup must stay below %d" % (MAX_SEQ - N_PREFILL - 1), file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from prometorch_amd import _lib, ops, synth
+    from prometorch_amd.decode import Decoder
+
+    _lib.load()  # fails loudly when the HIP library is not built
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    baseline = json.load(open(os.path.join(ROOT, "BASELINE.json")))
+
+    cfg = dict(synth.QWEN3_4B)
+    cfg["n_layers"] = args.layers
+    t0 = time.time()
+    layers = [synth.make_layer(SEED, i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(SEED, cfg)
+    log("synthetic model generated in %.1fs" % (time.time() - t0))
+    dec = Decoder(cfg, layers, head, max_seq=MAX_SEQ, kv_fp16=True, use_graph=True)
+    kvs = []
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(SEED, i, cfg, N_PREFILL)
+        dec.set_kv(i, k, v)
+        kvs.append((k, v))
+    torch.cuda.synchronize()
+    log("uploaded in %.1fs" % (time.time() - t0))
+
+    # ---- timed region: W warm-up tokens, then exactly K tokens, host-synchronous per token ----
+    dec.set_past_len(N_PREFILL)
+    tok = 1
+    for _ in range(args.warmup):
+        tok = dec.step(tok)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    toks = []
+    for _ in range(args.steps):
+        tok = dec.step(tok)
+        toks.append(tok)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t1
+    tok_s = args.steps / dt
+    log("decode: %d tokens in %.4fs = %.1f tok/s (%.3f ms/token)" % (args.steps, dt, tok_s, dt / args.steps * 1e3))
+
+    # same tokens with device-side token feedback (no host round trip between tokens)
+    dec.set_past_len(N_PREFILL)
+    dec.greedy(1, args.warmup)
+    t1 = time.perf_counter()
+    dec.set_past_len(N_PREFILL)
+    chained = dec.greedy(1, args.warmup + args.steps)
+    dt_chain = time.perf_counter() - t1
+    chained_tok_s = (args.warmup + args.steps) / dt_chain
+    tokens_equal = chained[args.warmup:] == toks
+    log("chained: %.1f tok/s, tokens identical to stepwise: %s" % (chained_tok_s, tokens_equal))
+
+    # ---- roofline of the dominant kernel, live, HIP events on the launching stream --------------
+    H, I = cfg["hidden"], cfg["inter"]
+    L0 = dec._layers
+    nL = cfg["n_layers"]
+    x = torch.randn(H, device="cuda")
+    act = torch.empty(I, device="cuda")
+    stride4 = H // 256 * 144
+    gate_up_bytes = 2 * I * stride4 + 4 * H + 4 * H + 4 * I  # two matrices + x + gamma in, act out
+
+    def run_gate_up(i):
+        Ld = L0[i % nL]
+        ops.fused_rmsnorm_gate_up_silu(x, Ld.ffn_norm, Ld.gate.data, Ld.up.data, act, H, I, stride4, 1e-6, False)
+
+    ms = event_time_ms(run_gate_up, 360, torch)
+    roof = {"bound": "hbm", "kernel": "q4k_gemv_kernel<fused rmsnorm + gate/up + silu> 2x9728x2560",
+            "achieved": gate_up_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": gate_up_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+            "bytes_per_launch": gate_up_bytes, "us_per_launch": ms * 1e3}
+    log("gate/up fused: %.2f us/launch, %.0f GB/s" % (ms * 1e3, roof["achieved"]))
+
+    gemv = {}
+    # configs[0]: single Q4_K GEMV 9728x2560 (x quantised in the kernel), cold (36 distinct matrices) and warm
+    y = torch.empty(I, device="cuda")
+    b0 = I * stride4 + 4 * H + 4 * I
+    ms_cold = event_time_ms(lambda i: ops.launch_q4km_persistent_gemv(L0[i % nL].gate.data, x, y, H, I, stride4), 360, torch)
+    ms_warm = event_time_ms(lambda i: ops.launch_q4km_persistent_gemv(L0[0].gate.data, x, y, H, I, stride4), 360, torch)
+    gemv["cfg0_q4k_9728x2560"] = {"bytes": b0, "us_cold": ms_cold * 1e3, "GBs_cold": b0 / ms_cold / 1e6,
+                                  "frac_cold": b0 / ms_cold / 1e6 / HBM_PEAK_GBS, "us_warm_cache": ms_warm * 1e3,
+                                  "GBs_warm_cache": b0 / ms_warm / 1e6}
+    # configs[1]: Q6_K lm_head 151936x2560 + argmax
+    V = cfg["vocab"]
+    stride6 = H // 256 * 210
+    logits = torch.empty(V, device="cuda")
+    idx = torch.zeros(1, dtype=torch.int64, device="cuda")
+    ws = torch.empty(ops.argmax_workspace_bytes(V), dtype=torch.uint8, device="cuda")
+    b1 = V * stride6 + 4 * H + 4 * V
+    lm = dec._cfg.lm_head.data
+    ms1 = event_time_ms(lambda i: ops.q6k_gemv_argmax(lm, x, logits, H, V, stride6, idx, ws), 40, torch)
+    gemv["cfg1_q6k_lm_head_argmax"] = {"bytes": b1, "us": ms1 * 1e3, "GBs": b1 / ms1 / 1e6, "frac": b1 / ms1 / 1e6 / HBM_PEAK_GBS}
+    # down projection Q6_K 2560x9728
+    xa = torch.randn(I, device="cuda")
+    yd = torch.empty(H, device="cuda")
+    strided = I // 256 * 210
+    b2 = H * strided + 4 * I + 4 * H
+    ms2 = event_time_ms(lambda i: ops.launch_q6k_gemv(L0[i % nL].down.data, xa, yd, I, H, strided), 360, torch)
+    gemv["q6k_down_2560x9728"] = {"bytes": b2, "us": ms2 * 1e3, "GBs": b2 / ms2 / 1e6, "frac": b2 / ms2 / 1e6 / HBM_PEAK_GBS}
+    log(json.dumps(gemv))
+    per_token_bytes = nL * 63866880 + V * stride6 + nL * 2 * (N_PREFILL + args.warmup + args.steps / 2) * 1024 * 2
+    dec.close()
+    del dec
+    torch.cuda.empty_cache()
+
+    # ---- CPU baseline on this host: bounded sample of the same workload ---------------------------
+    cpu = None
+    if args.cpu_tokens > 0:
+        try:
+            cpu = cpu_baseline(cfg, layers, head, kvs, args.cpu_tokens, toks, args.warmup)
+        except Exception as e:  # the baseline is reported, never required
+            log("cpu baseline failed: %r" % (e,))
+    out = {
+        "metric": baseline["metric"], "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[3]: batch-1 greedy decode, Qwen3-4B-shaped Q4_K_M (36 layers, q/k/o/gate/up Q4_K, "
+                               "v/down/lm_head Q6_K), fp16 KV prefilled 2048, %d new tokens" % args.steps,
+                   "kv_cache": "fp16", "graph": "hipGraph per token", "host_sync": "per token"},
+        "roofline": roof, "cpu_baseline": cpu, "gemv": gemv,
+        "chained_tok_s": chained_tok_s, "chained_tokens_identical": bool(tokens_equal),
+        "a100_published_tok_s": 82.6, "x_a100_published": tok_s / 82.6,
+        "token_hbm_frac": per_token_bytes / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
+    }
+    print(json.dumps(out), flush=True)
+
+
+def cpu_baseline(cfg, layers, head, kvs, n_tokens, gpu_tokens, warmup):
+    """Time the reference CPU decode path on this host for n_tokens tokens of the same workload."""
+    from oracle import pyoracle as po
+    kind = "port"
+    model = None
+    if po.have_ref():
+        try:
+            emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+            model = po.RefModel(cfg, layers, head, MAX_SEQ, emb)
+            kind = "reference"
+            cores = po.ref().ref_num_threads()
+        except OSError as e:
+            log("oracle/_ref not loadable (%r): timing the C port" % (e,))
+    if model is None:
+        model = po.OracleModel(cfg, layers, head, MAX_SEQ, kv_fp16=False)
+        cores = po.lib().po_num_threads()
+    for i, (k, v) in enumerate(kvs):
+        model.set_kv(i, k, v)
+    tok = model.step(1)  # warm-up token (page-in)
+    t = time.perf_counter()
+    for _ in range(n_tokens):
+        tok = model.step(tok)
+    dt = time.perf_counter() - t
+    log("cpu baseline (%s, %d threads): %.2f tok/s" % (kind, cores, n_tokens / dt))
+    if hasattr(model, "close"):
+        model.close()
+    return {"value": n_tokens / dt, "unit": "tok/s", "cores": int(cores), "kind": kind,
+            "sample": "%d greedy tokens of the same 36-layer model after 1 warm-up token, KV prefilled to %d (fp32 KV on the CPU)" % (n_tokens, N_PREFILL)}
+
+
+if __name__ == "__main__":
+    main()
