@@ -30,7 +30,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-SEED = 4004
+SEED = 25
 N_PREFILL = 2048
 MAX_SEQ = 2304
 

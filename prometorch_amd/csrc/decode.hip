@@ -5,8 +5,8 @@
 // step feeds the argmax back as the next token, so consecutive tokens need no host round trip.
 //
 // Per layer (Q4_K_M mix: q/k/o/gate/up Q4_K, v/down Q6_K):
-//   rms_norm (+Q8 of the result)            -> xn, xq8
-//   Q4_K {q,k} from xq8 ; Q6_K v from xn    (quant type is dispatched per tensor, as gemv_scratch does)
+//   RMSNorm + Q4_K {q,k} in one launch ; RMSNorm + Q6_K v in another (the norm is recomputed per
+//   workgroup; quant type is dispatched per tensor, as gemv_scratch does)
 //   qknorm + NeoX RoPE + K/V append
 //   split-KV attention + merge
 //   o-proj GEMV accumulating into the residual
@@ -23,7 +23,8 @@ int q4k_gemv_multi(int n_mat, const void* const* W, float* const* y, const int* 
 int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8, const float* gamma, float eps,
                      int add_one, float* act, int K, int N, int64_t stride, hipStream_t s);
 int q6k_gemv_impl(const void* W, const float* x, float* y, int K, int N, int64_t stride, bool accumulate,
-                  hipStream_t s);
+                  const float* gamma, float eps, int add_one, hipStream_t s);
+void q6k_init_attributes();
 
 __global__ void set_scalars_kernel(int* d_token, int token, int64_t* d_past, int64_t past, int* d_step) {
     *d_token = token;
@@ -80,14 +81,14 @@ static int gemv_any(const ptm_qweight& w, const float* x_f32, float* y, bool acc
         const int N = w.rows;
         return q4k_gemv_multi(1, &W, &y, &N, x_f32, false, nullptr, 0.f, 0, w.cols, w.row_stride_bytes, acc, s);
     }
-    return q6k_gemv_impl(w.data, x_f32, y, w.cols, w.rows, w.row_stride_bytes, acc, s);
+    return q6k_gemv_impl(w.data, x_f32, y, w.cols, w.rows, w.row_stride_bytes, acc, nullptr, 0.f, 0, s);
 }
 
 // Enqueue one token step on d->stream. Everything it reads that changes per token is in device memory.
 static int enqueue_step(ptm_decoder* d) {
     const ptm_decode_config& c = d->cfg;
     hipStream_t s = d->stream;
-    const int H = c.hidden, hd = c.head_dim, qd = c.n_heads * hd, kvd = c.n_kv_heads * hd;
+    const int H = c.hidden, hd = c.head_dim;
     int rc;
 #define PTM_TRY(call) do { rc = (call); if (rc != PTM_OK) return rc; } while (0)
     if (c.embedding_f32) PTM_TRY(ptm_embedding_row(c.embedding_f32, d->x, d->d_token, H, s));
@@ -95,10 +96,9 @@ static int enqueue_step(ptm_decoder* d) {
 
     for (int li = 0; li < c.n_layers; ++li) {
         const ptm_layer& L = d->layers[li];
-        // attention norm; Q8 copy for the Q4_K projections
-        PTM_TRY(ptm_rms_norm(d->x, L.attn_norm, d->xn, 1, H, c.rms_eps, 0, d->xq8, s));
+        // attention RMSNorm is recomputed inside each projection kernel (no separate launch):
+        // the Q4_K projections share one launch, Q6_K ones get their own
         {
-            // Q4_K projections share one launch and the Q8 activations; Q6_K ones read fp32 xn
             const ptm_qweight* w[3] = {&L.q, &L.k, &L.v};
             float* y[3] = {d->q, d->k, d->v};
             const void* W4[3]; float* y4[3]; int N4[3]; int n4 = 0;
@@ -106,11 +106,13 @@ static int enqueue_step(ptm_decoder* d) {
                 if (w[i]->ggml_type == PTM_TYPE_Q4_K) {
                     W4[n4] = w[i]->data; y4[n4] = y[i]; N4[n4] = w[i]->rows; ++n4;
                 } else {
-                    PTM_TRY(gemv_any(*w[i], d->xn, y[i], false, s));
+                    PTM_TRY(q6k_gemv_impl(w[i]->data, d->x, y[i], H, w[i]->rows, w[i]->row_stride_bytes, false,
+                                          L.attn_norm, c.rms_eps, 0, s));
                 }
             }
             if (n4 > 0)
-                PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->xq8, true, nullptr, 0.f, 0, H, (int64_t)(H / 256) * 144, false, s));
+                PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->x, false, L.attn_norm, c.rms_eps, 0, H,
+                                       (int64_t)(H / 256) * 144, false, s));
         }
         PTM_TRY(ptm_qknorm_rope_kvwrite(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, c.n_heads,
                                         c.n_kv_heads, hd, d->d_past, c.max_seq, c.rope_freq_base, d->rope, c.rms_eps,
@@ -196,6 +198,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->amax_ws = base + o_ws; d->d_token = (int*)(base + o_tok); d->d_past = (int64_t*)(base + o_past);
     d->d_next = (int64_t*)(base + o_next); d->d_step = (int*)(base + o_step);
     d->d_tokens = (int64_t*)(base + o_tokens);
+    q6k_init_attributes();  // one-time kernel attributes, before anything can be captured
 
     if ((rc = hip_status(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     if ((rc = hip_status(hipHostMalloc((void**)&d->h_pinned, 8 * (size_t)c.max_seq, hipHostMallocDefault))) != PTM_OK) { ptm_decode_destroy(d); return rc; }

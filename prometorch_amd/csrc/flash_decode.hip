@@ -66,19 +66,26 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
         q[g][4] = b.x; q[g][5] = b.y; q[g][6] = b.z; q[g][7] = b.w;
     }
 
+    // ---- all K and V rows of the chunk are requested up front: one HBM round trip ----
+    float kreg[NPASS][8], vreg[NPASS][8];
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+        const int64_t t = t0 + pass * PPB + wave * PPW + pl;
+        const int64_t tc = t < total ? t : total - 1;
+        load8<KV16>(Kc, tc * kv_dim + col, kreg[pass]);
+        load8<KV16>(Vc, tc * kv_dim + col, vreg[pass]);
+    }
+
     // ---- scores ----
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
         const int tl = pass * PPB + wave * PPW + pl;
-        const int64_t t = t0 + tl;
-        const bool valid = t < total;
-        float k[8];
-        load8<KV16>(Kc, (valid ? t : total - 1) * kv_dim + col, k);
+        const bool valid = t0 + tl < total;
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float d = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], k[i], d);
+            for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], kreg[pass][i], d);
             d = (LPP == 16) ? sum16(d) : sum8(d);
             if (dl == 0) s_p[g][tl] = valid ? d * scale : -INFINITY;
         }
@@ -109,14 +116,11 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
         const int tl = pass * PPB + wave * PPW + pl;
-        const int64_t t = t0 + tl;
-        float v[8];
-        load8<KV16>(Vc, (t < total ? t : total - 1) * kv_dim + col, v);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             const float p = s_p[g][tl];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, v[i], acc[g][i]);
+            for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, vreg[pass][i], acc[g][i]);
         }
     }
     // reduce over the PPW position slots of the wave (lanes with equal dl), then over waves
@@ -142,24 +146,51 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     }
 }
 
-// grid n_heads, HD threads: merge the active splits
-__global__ void flash_decode_reduce_kernel(const float* __restrict__ pO, const float* __restrict__ pL,
-                                           const float* __restrict__ pM, float* __restrict__ O, int n_heads,
-                                           int head_dim, const int64_t* __restrict__ d_past, int max_seq) {
+// grid n_heads, 256 threads: merge the active splits.  Thread (slot = tid / head_dim-quarter...) layout:
+// the 256 threads form R = 256/head_dim split-slots x head_dim dims; slot r sums splits r, r+R, ...
+// (independent loads, all in flight), then the R slot sums are added in slot order.
+__global__ __launch_bounds__(256) void flash_decode_reduce_kernel(const float* __restrict__ pO,
+                                                                  const float* __restrict__ pL,
+                                                                  const float* __restrict__ pM, float* __restrict__ O,
+                                                                  int n_heads, int head_dim,
+                                                                  const int64_t* __restrict__ d_past, int max_seq) {
+    __shared__ float s_w[256];     // per-split weight exp(m_s - M)
+    __shared__ float s_num[256];
+    __shared__ float s_red[8];
     int64_t total = *d_past + 1;
     if (total > max_seq) total = max_seq;
     const int ns = (int)((total + FD_CHUNK - 1) / FD_CHUNK);
-    const int h = blockIdx.x, d = threadIdx.x;
-    float M = -INFINITY;
-    for (int s = 0; s < ns; ++s) M = fmaxf(M, pM[(int64_t)s * n_heads + h]);
-    float num = 0.0f, den = 0.0f;
-    for (int s = 0; s < ns; ++s) {
-        const float w = expf(pM[(int64_t)s * n_heads + h] - M);
-        den = fmaf(w, pL[(int64_t)s * n_heads + h], den);
-        num = fmaf(w, pO[((int64_t)s * n_heads + h) * head_dim + d], num);
+    const int h = blockIdx.x, tid = threadIdx.x;
+    // global max and denominator over splits (ns may exceed 256: strided)
+    float m = -INFINITY;
+    for (int s = tid; s < ns; s += 256) m = fmaxf(m, pM[(int64_t)s * n_heads + h]);
+    m = max64(m);
+    if ((tid & 63) == 0) s_red[tid >> 6] = m;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    float den = 0.0f;
+    for (int s = tid; s < ns; s += 256) den = fmaf(expf(pM[(int64_t)s * n_heads + h] - M), pL[(int64_t)s * n_heads + h], den);
+    den = sum64(den);
+    if ((tid & 63) == 0) s_red[4 + (tid >> 6)] = den;
+    const int R = 256 / head_dim, slot = tid / head_dim, d = tid % head_dim;
+    float num = 0.0f;
+    for (int s0 = 0; s0 < ns; s0 += 256) {
+        __syncthreads();
+        if (s0 + tid < ns) s_w[tid] = expf(pM[(int64_t)(s0 + tid) * n_heads + h] - M);
+        __syncthreads();
+        const int lim = min(256, ns - s0);
+        for (int s = slot; s < lim; s += R)
+            num = fmaf(s_w[s], pO[((int64_t)(s0 + s) * n_heads + h) * head_dim + d], num);
     }
-    // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
-    O[(int64_t)h * head_dim + d] = num * (1.0f / (den + 1e-10f));
+    s_num[tid] = num;
+    __syncthreads();
+    if (tid < head_dim) {
+        float t = s_num[tid];
+        for (int r = 1; r < R; ++r) t += s_num[r * head_dim + tid];
+        const float dsum = (s_red[4] + s_red[5]) + (s_red[6] + s_red[7]);
+        // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
+        O[(int64_t)h * head_dim + tid] = t * (1.0f / (dsum + 1e-10f));
+    }
 }
 
 template <bool KV16, int HD>
@@ -209,7 +240,7 @@ int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, f
                              : fd_launch_g<false, 64>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale);
     }
     if (rc != PTM_OK) return rc;
-    hipLaunchKernelGGL(flash_decode_reduce_kernel, dim3(n_heads), dim3(head_dim), 0, s, partial_O, partial_lse,
+    hipLaunchKernelGGL(flash_decode_reduce_kernel, dim3(n_heads), dim3(256), 0, s, partial_O, partial_lse,
                        partial_max, O, n_heads, head_dim, d_past_len, max_seq);
     return launch_status();
 }

@@ -4,15 +4,18 @@
 // activation vector is quantised to Q8 blocks of 32 (cpu_quant_gemv.h:147-198), each 32-wide
 // sub-block contributes  fma(d*sc*dx, (float)isum, -(dmin*m*sx))  with isum the exact int32
 // dot of 4-bit weights and int8 activations; only the order in which the per-sub-block terms
-// are added differs (per-lane chains + an 8-lane tree instead of two scalar chains).
+// are added differs (per-lane chains + a cross-lane tree instead of two scalar chains).
 //
-// Data movement: one row is swept by an aligned group of 8 lanes; per super-block (144 B) lane j
-// fetches the 16-byte header {d, dmin, scales[12]} and the j-th 16-byte slice of qs[128] with
-// 128-bit loads, so a wave reads 8 rows x 144 B per step and every fetched byte is used.  A slice
-// holds 16 low nibbles (sub-block 2*(j/2)) and 16 high nibbles (sub-block 2*(j/2)+1); lane pairs
-// swap halves through one DPP move so that lane j ends up owning the complete integer dot of
-// sub-block j.  Q8 activations live in LDS (K + K/4 bytes) and are shared by the 32 rows of a
-// workgroup.
+// Data movement: a super-block (144 B) is fetched by an aligned group of 8 lanes: lane j takes
+// the 16-byte header {d, dmin, scales[12]} and the j-th 16-byte slice of qs[128] with 128-bit
+// loads, so every fetched byte is used.  A slice holds 16 low nibbles (sub-block 2*(j/2)) and
+// 16 high nibbles (sub-block 2*(j/2)+1); lane pairs swap halves through one DPP move so that
+// lane j ends up owning the complete integer dot of sub-block j.
+// A row is shared by S lane groups (S = 1, 2, 4 or 8 - a whole wave), group s taking blocks
+// s, s+S, ...; S is chosen on the host so that a launch has several hundred workgroups even for
+// short-and-wide matrices (o-proj: 2560 rows) and so that each group's blocks are all in flight
+// at once.  The first pass of weight loads is issued BEFORE the activation vector is staged
+// (RMSNorm, Q8 quantisation, LDS), so HBM latency overlaps the prologue.
 #include "ptm_common.h"
 
 namespace ptm {
@@ -22,8 +25,9 @@ struct Q4KArgs {
     float* y[3];
     int row_end[3];  // cumulative row counts of the (up to 3) matrices
     int n_mat;
-    int total_rows;
+    int total_rows;  // MODE 1: 2*N interleaved (gate row r, up row r)
     int K;
+    int log2S;       // lane groups per row = 1 << log2S
     int64_t stride;
     const void* x;       // fp32 x[K] (XQ8 == false) or Q8 blocks (XQ8 == true)
     const float* gamma;  // RMSNorm weight (NORM)
@@ -31,7 +35,7 @@ struct Q4KArgs {
     int add_one;
 };
 
-enum { Q4K_THREADS = 256, Q4K_ROWS_PER_WG = 32 };
+enum { Q4K_THREADS = 256, Q4K_U = 10 };
 
 // ---- prologue: bring the Q8 activation into LDS -------------------------------------------
 template <bool XQ8, bool NORM>
@@ -85,54 +89,35 @@ __device__ __forceinline__ void q4k_stage_x(const Q4KArgs& a, uint8_t* lds) {
     __syncthreads();
 }
 
-// ---- one row: lane j of the 8-lane group returns its partial (sum over blocks of sub-block j) ---
-template <int U>
-__device__ __forceinline__ float q4k_row_partial(const uint8_t* __restrict__ row, int nblk,
-                                                 const uint8_t* __restrict__ lds, int K, int j) {
+// contribution of one super-block to lane j's chain (sub-block j of the block)
+__device__ __forceinline__ float q4k_block_term(const uint4 hdr, const uint4 qv, const uint8_t* __restrict__ lds,
+                                                int K, int b, int j) {
     const int8_t* xq = reinterpret_cast<const int8_t*>(lds);
     const float* xd = reinterpret_cast<const float*>(lds + K);
     const float* xs = xd + K / 32;
-    const int g = j >> 1, half = j & 1;
-    const int xoff = g * 64 + half * 16;  // low-nibble activations; high-nibble ones are +32
-    float acc = 0.0f;
-    for (int b0 = 0; b0 < nblk; b0 += U) {
-        uint4 hdr[U], qv[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int b = min(b0 + u, nblk - 1);
-            const uint8_t* p = row + (int64_t)b * 144;
-            hdr[u] = *reinterpret_cast<const uint4*>(p);
-            qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int b = b0 + u;
-            if (b < nblk) {
-                const int4 xl = *reinterpret_cast<const int4*>(xq + b * 256 + xoff);
-                const int4 xh = *reinterpret_cast<const int4*>(xq + b * 256 + xoff + 32);
-                int lo = 0, hi = 0;
-                lo = __builtin_amdgcn_sdot4((int)(qv[u].x & 0x0f0f0f0fu), xl.x, lo, false);
-                lo = __builtin_amdgcn_sdot4((int)(qv[u].y & 0x0f0f0f0fu), xl.y, lo, false);
-                lo = __builtin_amdgcn_sdot4((int)(qv[u].z & 0x0f0f0f0fu), xl.z, lo, false);
-                lo = __builtin_amdgcn_sdot4((int)(qv[u].w & 0x0f0f0f0fu), xl.w, lo, false);
-                hi = __builtin_amdgcn_sdot4((int)((qv[u].x >> 4) & 0x0f0f0f0fu), xh.x, hi, false);
-                hi = __builtin_amdgcn_sdot4((int)((qv[u].y >> 4) & 0x0f0f0f0fu), xh.y, hi, false);
-                hi = __builtin_amdgcn_sdot4((int)((qv[u].z >> 4) & 0x0f0f0f0fu), xh.z, hi, false);
-                hi = __builtin_amdgcn_sdot4((int)((qv[u].w >> 4) & 0x0f0f0f0fu), xh.w, hi, false);
-                // even lane keeps the low-nibble half-dot and receives its partner's; odd lane the high one
-                const int keep = half ? hi : lo;
-                const int give = half ? lo : hi;
-                const int isum = keep + dpp_i<0xB1>(give);
-                int sc, mn;
-                q4k_scale_min(hdr[u].y, hdr[u].z, hdr[u].w, j, sc, mn);
-                const float d = h2f(hdr[u].x), dmin = h2f(hdr[u].x >> 16);
-                const float w = d * (float)sc * xd[b * 8 + j];
-                const float c = dmin * (float)mn * xs[b * 8 + j];
-                acc += fmaf(w, (float)isum, -c);
-            }
-        }
-    }
-    return acc;
+    const int half = j & 1;
+    const int xoff = (j >> 1) * 64 + half * 16;  // low-nibble activations; high-nibble ones are +32
+    const int4 xl = *reinterpret_cast<const int4*>(xq + b * 256 + xoff);
+    const int4 xh = *reinterpret_cast<const int4*>(xq + b * 256 + xoff + 32);
+    int lo = 0, hi = 0;
+    lo = __builtin_amdgcn_sdot4((int)(qv.x & 0x0f0f0f0fu), xl.x, lo, false);
+    lo = __builtin_amdgcn_sdot4((int)(qv.y & 0x0f0f0f0fu), xl.y, lo, false);
+    lo = __builtin_amdgcn_sdot4((int)(qv.z & 0x0f0f0f0fu), xl.z, lo, false);
+    lo = __builtin_amdgcn_sdot4((int)(qv.w & 0x0f0f0f0fu), xl.w, lo, false);
+    hi = __builtin_amdgcn_sdot4((int)((qv.x >> 4) & 0x0f0f0f0fu), xh.x, hi, false);
+    hi = __builtin_amdgcn_sdot4((int)((qv.y >> 4) & 0x0f0f0f0fu), xh.y, hi, false);
+    hi = __builtin_amdgcn_sdot4((int)((qv.z >> 4) & 0x0f0f0f0fu), xh.z, hi, false);
+    hi = __builtin_amdgcn_sdot4((int)((qv.w >> 4) & 0x0f0f0f0fu), xh.w, hi, false);
+    // even lane keeps the low-nibble half-dot and receives its partner's; odd lane the high one
+    const int keep = half ? hi : lo;
+    const int give = half ? lo : hi;
+    const int isum = keep + dpp_i<0xB1>(give);
+    int sc, mn;
+    q4k_scale_min(hdr.y, hdr.z, hdr.w, j, sc, mn);
+    const float d = h2f(hdr.x), dmin = h2f(hdr.x >> 16);
+    const float w = d * (float)sc * xd[b * 8 + j];
+    const float c = dmin * (float)mn * xs[b * 8 + j];
+    return fmaf(w, (float)isum, -c);
 }
 
 __device__ __forceinline__ float silu_mul_ref(float g, float u) {
@@ -143,50 +128,114 @@ __device__ __forceinline__ float silu_mul_ref(float g, float u) {
     return (g * sig) * u;
 }
 
-// MODE 0: plain (y = or += W.x for up to three matrices over a flattened row space)
-// MODE 1: gate/up pair with SiLU: y[0][r] = silu(Wg[r].x) * (Wu[r].x)
-template <bool XQ8, bool NORM, bool ACC, int MODE, int U>
+// MODE 0: y = or += W.x for up to three matrices over a flattened row space
+// MODE 1: gate/up pair with SiLU over interleaved virtual rows (2r = gate row r, 2r+1 = up row r):
+//         y[0][r] = silu(Wg[r].x) * (Wu[r].x)
+template <bool XQ8, bool NORM, bool ACC, int MODE>
 __global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_kernel(const Q4KArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
-    q4k_stage_x<XQ8, NORM>(a, lds);
-
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int j = lane & 7;
-    const int r = blockIdx.x * Q4K_ROWS_PER_WG + wave * 8 + (lane >> 3);
+    const int j = lane & 7, grp = lane >> 3;
+    const int S = 1 << a.log2S;
+    const int sub = grp & (S - 1);
+    const int rows_per_wave = 8 >> a.log2S;
+    const int r = (blockIdx.x * 4 + wave) * rows_per_wave + (grp >> a.log2S);
     const bool live = r < a.total_rows;
     const int rr = live ? r : a.total_rows - 1;
     const int nblk = a.K / 256;
+    const int nb_max = (nblk + S - 1) >> a.log2S;  // passes are sized for the group with the most blocks
 
+    int mat = 0, local = rr;
     if constexpr (MODE == 1) {
-        float pg = q4k_row_partial<U>(a.W[0] + (int64_t)rr * a.stride, nblk, lds, a.K, j);
-        float pu = q4k_row_partial<U>(a.W[1] + (int64_t)rr * a.stride, nblk, lds, a.K, j);
-        pg = sum8(pg);
-        pu = sum8(pu);
-        if (live && j == 0) a.y[0][rr] = silu_mul_ref(pg, pu);
+        mat = rr & 1;
+        local = rr >> 1;
     } else {
-        int mat = 0, local = rr;
         if (a.n_mat > 1 && rr >= a.row_end[0]) { mat = 1; local = rr - a.row_end[0]; }
         if (a.n_mat > 2 && rr >= a.row_end[1]) { mat = 2; local = rr - a.row_end[1]; }
-        const uint8_t* W = mat == 0 ? a.W[0] : (mat == 1 ? a.W[1] : a.W[2]);
+    }
+    const uint8_t* row = (mat == 0 ? a.W[0] : (mat == 1 ? a.W[1] : a.W[2])) + (int64_t)local * a.stride;
+
+    // ---- first pass of weight loads, issued before the activation prologue ----
+    uint4 hdr[Q4K_U], qv[Q4K_U];
+    const int cnt0 = min(Q4K_U, nb_max);
+#pragma unroll
+    for (int u = 0; u < Q4K_U; ++u) {
+        if (u < cnt0) {
+            const int b = min(sub + (u << a.log2S), nblk - 1);
+            const uint8_t* p = row + (int64_t)b * 144;
+            hdr[u] = *reinterpret_cast<const uint4*>(p);
+            qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+        }
+    }
+
+    q4k_stage_x<XQ8, NORM>(a, lds);
+
+    float acc = 0.0f;
+    for (int i0 = 0; i0 < nb_max; i0 += Q4K_U) {
+        const int cnt = min(Q4K_U, nb_max - i0);
+        if (i0 > 0) {
+#pragma unroll
+            for (int u = 0; u < Q4K_U; ++u) {
+                if (u < cnt) {
+                    const int b = min(sub + ((i0 + u) << a.log2S), nblk - 1);
+                    const uint8_t* p = row + (int64_t)b * 144;
+                    hdr[u] = *reinterpret_cast<const uint4*>(p);
+                    qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < Q4K_U; ++u) {
+            if (u < cnt) {
+                const int b = sub + ((i0 + u) << a.log2S);
+                const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
+                acc += b < nblk ? t : 0.0f;
+            }
+        }
+    }
+    // reduce: 8 lanes of the group, then the S groups of the row
+    float p = sum8(acc);
+    if (S >= 2) p += dpp_f<0x128>(p);  // row_ror:8 = the other 8-lane half of the 16-lane row
+    if (S >= 4) p += __shfl_xor(p, 16, 64);
+    if (S >= 8) p += __shfl_xor(p, 32, 64);
+
+    if constexpr (MODE == 1) {
+        // gate and up of one row sit S groups apart
+        float other;
+        if (S == 1) other = dpp_f<0x128>(p);
+        else if (S == 2) other = __shfl_xor(p, 16, 64);
+        else other = __shfl_xor(p, 32, 64);
+        if (live && mat == 0 && sub == 0 && j == 0) a.y[0][local] = silu_mul_ref(p, other);
+    } else {
         float* y = mat == 0 ? a.y[0] : (mat == 1 ? a.y[1] : a.y[2]);
-        float p = q4k_row_partial<U>(W + (int64_t)local * a.stride, nblk, lds, a.K, j);
-        p = sum8(p);
-        if (live && j == 0) {
+        if (live && sub == 0 && j == 0) {
             if constexpr (ACC) y[local] += p;
             else y[local] = p;
         }
     }
 }
 
+// lane groups per row: enough workgroups to cover the chip, and all of a group's blocks in one pass
+static int q4k_pick_log2S(int total_rows, int nblk, int max_log2S) {
+    int l = 0;
+    while (l < max_log2S) {
+        const int S = 1 << l;
+        const int wgs = (total_rows * S + 31) / 32;
+        const int nb = (nblk + S - 1) / S;
+        if (nb <= Q4K_U && wgs >= 600) break;
+        if (nb <= 1) break;
+        ++l;
+    }
+    return l;
+}
+
 template <bool XQ8, bool NORM, bool ACC, int MODE>
-static int q4k_launch(const Q4KArgs& a, hipStream_t s) {
-    const int grid = (a.total_rows + Q4K_ROWS_PER_WG - 1) / Q4K_ROWS_PER_WG;
+static int q4k_launch(Q4KArgs& a, hipStream_t s) {
+    a.log2S = q4k_pick_log2S(a.total_rows, a.K / 256, MODE == 1 ? 2 : 3);
+    const int rows_per_wg = 32 >> a.log2S;
+    const int grid = (a.total_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t lds = (size_t)q8_bytes(a.K);
-    const int nblk = a.K / 256;
-    // blocks in flight per row: whole row when short, otherwise 8..10 per pass
-    if (nblk <= 4) hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 4>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
-    else if (nblk % 10 == 0 || nblk == 38) hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 10>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
-    else hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 8>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
+    hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
     return launch_status();
 }
 
@@ -236,13 +285,14 @@ int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8
     if (rc != PTM_OK) return rc;
     rc = q4k_check(wu, x, act, K, N, stride);
     if (rc != PTM_OK) return rc;
+    if (N > 0x3fffffff) return PTM_E_UNSUPPORTED;
     Q4KArgs a{};
     a.W[0] = static_cast<const uint8_t*>(wg);
     a.W[1] = static_cast<const uint8_t*>(wu);
     a.y[0] = act;
     a.n_mat = 2;
     a.row_end[0] = N;
-    a.total_rows = N;
+    a.total_rows = 2 * N;
     a.K = K;
     a.stride = stride;
     a.x = x;

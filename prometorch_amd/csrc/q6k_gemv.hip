@@ -19,12 +19,16 @@ struct Q6KArgs {
     const float* x;
     float* y;        // may be NULL when only the argmax is wanted
     int K, N;
+    int log2S;       // lane groups per row = 1 << log2S
     int64_t stride;
     float* part_val; // ARGMAX: per-workgroup best value / index
     int* part_idx;
+    const float* gamma;  // NORM: RMSNorm weight applied to x while staging
+    float eps;
+    int add_one;
 };
 
-enum { Q6K_THREADS = 256, Q6K_ROWS_PER_WG = 32 };
+enum { Q6K_THREADS = 256, Q6K_U = 5 };
 
 __device__ __forceinline__ float dot4_u8(uint32_t q, float4 x, float acc) {
     acc = fmaf((float)(q & 0xffu), x.x, acc);
@@ -34,73 +38,101 @@ __device__ __forceinline__ float dot4_u8(uint32_t q, float4 x, float acc) {
     return acc;
 }
 
-template <int U>
-__device__ __forceinline__ float q6k_row_partial(const uint8_t* __restrict__ row, int nblk,
-                                                 const float* __restrict__ xf, const float* __restrict__ xsum16,
-                                                 int j) {
+struct Q6Blk { uint4 ql, qh, sc; uint32_t d; };
+
+__device__ __forceinline__ Q6Blk q6k_load(const uint8_t* __restrict__ p, int j, int qh_off) {
+    Q6Blk r;
+    r.ql = ld16_a2(p + 16 * j);
+    r.qh = ld16_a2(p + qh_off);
+    r.sc = ld16_a2(p + 192);
+    r.d = reinterpret_cast<const u16_a2*>(p + 208)->v;
+    return r;
+}
+
+// contribution of block b to lane j's chain
+__device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __restrict__ xf,
+                                                const float* __restrict__ xsum16, int b, int j) {
     const int half = j >> 2, jj = j & 3, which32 = jj >> 1, l16 = jj & 1;
-    const int qh_off = 128 + 32 * half + 16 * l16;
     const int sc_lo_i = 8 * half + 2 * which32 + l16;  // scale of the low-nibble 16; high-nibble one is +4
     const int hshift = 2 * which32;
     const int xo = 128 * half + 32 * which32 + 16 * l16;  // x offset of the low-nibble 16; high-nibble +64
-    float acc = 0.0f;
-    for (int b0 = 0; b0 < nblk; b0 += U) {
-        uint4 ql[U], qh[U], sc[U];
-        uint32_t dd[U];
+    const float* xb = xf + b * 256 + xo;
+    float s_lo = 0.0f, s_hi = 0.0f;
+    const uint32_t qlw[4] = {k.ql.x, k.ql.y, k.ql.z, k.ql.w};
+    const uint32_t qhw[4] = {k.qh.x, k.qh.y, k.qh.z, k.qh.w};
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int b = min(b0 + u, nblk - 1);
-            const uint8_t* p = row + (int64_t)b * 210;
-            ql[u] = ld16_a2(p + 16 * j);
-            qh[u] = ld16_a2(p + qh_off);
-            sc[u] = ld16_a2(p + 192);
-            dd[u] = reinterpret_cast<const u16_a2*>(p + 208)->v;
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int b = b0 + u;
-            if (b < nblk) {
-                const float* xb = xf + b * 256 + xo;
-                float s_lo = 0.0f, s_hi = 0.0f;
-                const uint32_t qlw[4] = {ql[u].x, ql[u].y, ql[u].z, ql[u].w};
-                const uint32_t qhw[4] = {qh[u].x, qh[u].y, qh[u].z, qh[u].w};
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const uint32_t hs = qhw[w] >> hshift;
-                    const uint32_t q_lo = (qlw[w] & 0x0f0f0f0fu) | ((hs << 4) & 0x30303030u);
-                    const uint32_t q_hi = ((qlw[w] >> 4) & 0x0f0f0f0fu) | (hs & 0x30303030u);
-                    const float4 x_lo = *reinterpret_cast<const float4*>(xb + 4 * w);
-                    const float4 x_hi = *reinterpret_cast<const float4*>(xb + 64 + 4 * w);
-                    s_lo = dot4_u8(q_lo, x_lo, s_lo);
-                    s_hi = dot4_u8(q_hi, x_hi, s_hi);
-                }
-                const int xi = (b * 256 + xo) >> 4;
-                s_lo = fmaf(-32.0f, xsum16[xi], s_lo);
-                s_hi = fmaf(-32.0f, xsum16[xi + 4], s_hi);
-                const uint32_t scw[4] = {sc[u].x, sc[u].y, sc[u].z, sc[u].w};
-                const uint32_t w_lo = scw[sc_lo_i >> 2] >> (8 * (sc_lo_i & 3));
-                const uint32_t w_hi = scw[(sc_lo_i + 4) >> 2] >> (8 * (sc_lo_i & 3));
-                const float d = h2f(dd[u]);
-                const float f_lo = d * (float)(int)(int8_t)(w_lo & 0xffu);
-                const float f_hi = d * (float)(int)(int8_t)(w_hi & 0xffu);
-                acc = fmaf(f_lo, s_lo, acc);
-                acc = fmaf(f_hi, s_hi, acc);
-            }
-        }
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t hs = qhw[w] >> hshift;
+        const uint32_t q_lo = (qlw[w] & 0x0f0f0f0fu) | ((hs << 4) & 0x30303030u);
+        const uint32_t q_hi = ((qlw[w] >> 4) & 0x0f0f0f0fu) | (hs & 0x30303030u);
+        const float4 x_lo = *reinterpret_cast<const float4*>(xb + 4 * w);
+        const float4 x_hi = *reinterpret_cast<const float4*>(xb + 64 + 4 * w);
+        s_lo = dot4_u8(q_lo, x_lo, s_lo);
+        s_hi = dot4_u8(q_hi, x_hi, s_hi);
     }
-    return acc;
+    const int xi = (b * 256 + xo) >> 4;
+    s_lo = fmaf(-32.0f, xsum16[xi], s_lo);
+    s_hi = fmaf(-32.0f, xsum16[xi + 4], s_hi);
+    const uint32_t scw[4] = {k.sc.x, k.sc.y, k.sc.z, k.sc.w};
+    const uint32_t w_lo = scw[sc_lo_i >> 2] >> (8 * (sc_lo_i & 3));
+    const uint32_t w_hi = scw[(sc_lo_i + 4) >> 2] >> (8 * (sc_lo_i & 3));
+    const float d = h2f(k.d);
+    const float f_lo = d * (float)(int)(int8_t)(w_lo & 0xffu);
+    const float f_hi = d * (float)(int)(int8_t)(w_hi & 0xffu);
+    return fmaf(f_hi, s_hi, f_lo * s_lo);
 }
 
-template <bool ACC, bool ARGMAX, int U>
+template <bool ACC, bool ARGMAX, bool NORM>
 __global__ __launch_bounds__(Q6K_THREADS) void q6k_gemv_kernel(const Q6KArgs a) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
     float* xf = reinterpret_cast<float*>(lds_raw);
     float* xsum16 = xf + a.K;
     const int tid = threadIdx.x;
-    // stage x and its per-16 sums: 4 consecutive float4 slots (4 lanes) make one 16-group
+    const int lane = tid & 63, wave = tid >> 6, j = lane & 7, grp = lane >> 3;
+    const int S = 1 << a.log2S;
+    const int sub = grp & (S - 1);
+    const int rows_per_wave = 8 >> a.log2S;
+    const int r = (blockIdx.x * 4 + wave) * rows_per_wave + (grp >> a.log2S);
+    const bool live = r < a.N;
+    const int rr = live ? r : a.N - 1;
+    const int nblk = a.K / 256;
+    const int nb_max = (nblk + S - 1) >> a.log2S;
+    const uint8_t* row = a.W + (int64_t)rr * a.stride;
+    const int qh_off = 128 + 32 * (j >> 2) + 16 * (j & 1);
+
+    // first pass of weight loads, in flight while x is staged
+    Q6Blk blk[Q6K_U];
+    const int cnt0 = min(Q6K_U, nb_max);
+#pragma unroll
+    for (int u = 0; u < Q6K_U; ++u)
+        if (u < cnt0) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off);
+
+    // stage x (optionally RMS-normalised) and its per-16 sums: 4 consecutive float4 slots make one 16-group
     const float4* x4 = reinterpret_cast<const float4*>(a.x);
+    float rs = 1.0f;
+    if constexpr (NORM) {
+        __shared__ float red[4];
+        float ss = 0.0f;
+        for (int i = tid; i < a.K / 4; i += Q6K_THREADS) {
+            const float4 v = x4[i];
+            ss = fmaf(v.x, v.x, ss);
+            ss = fmaf(v.y, v.y, ss);
+            ss = fmaf(v.z, v.z, ss);
+            ss = fmaf(v.w, v.w, ss);
+        }
+        ss = block_sum256(ss, red);
+        rs = 1.0f / sqrtf(ss / (float)a.K + a.eps);
+    }
     for (int i = tid; i < a.K / 4; i += Q6K_THREADS) {
-        const float4 v = x4[i];
+        float4 v = x4[i];
+        if constexpr (NORM) {
+            const float4 g = reinterpret_cast<const float4*>(a.gamma)[i];
+            const float one = a.add_one ? 1.0f : 0.0f;
+            v.x = v.x * rs * (g.x + one);
+            v.y = v.y * rs * (g.y + one);
+            v.z = v.z * rs * (g.z + one);
+            v.w = v.w * rs * (g.w + one);
+        }
         reinterpret_cast<float4*>(xf)[i] = v;
         float s = (v.x + v.y) + (v.z + v.w);
         s += dpp_f<0xB1>(s);
@@ -109,18 +141,33 @@ __global__ __launch_bounds__(Q6K_THREADS) void q6k_gemv_kernel(const Q6KArgs a) 
     }
     __syncthreads();
 
-    const int lane = tid & 63, wave = tid >> 6, j = lane & 7;
-    const int r = blockIdx.x * Q6K_ROWS_PER_WG + wave * 8 + (lane >> 3);
-    const bool live = r < a.N;
-    const int rr = live ? r : a.N - 1;
-    float p = q6k_row_partial<U>(a.W + (int64_t)rr * a.stride, a.K / 256, xf, xsum16, j);
-    p = sum8(p);
-    if (live && j == 0 && a.y) {
+    float acc = 0.0f;
+    for (int i0 = 0; i0 < nb_max; i0 += Q6K_U) {
+        const int cnt = min(Q6K_U, nb_max - i0);
+        if (i0 > 0) {
+#pragma unroll
+            for (int u = 0; u < Q6K_U; ++u)
+                if (u < cnt) blk[u] = q6k_load(row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 210, j, qh_off);
+        }
+#pragma unroll
+        for (int u = 0; u < Q6K_U; ++u) {
+            if (u < cnt) {
+                const int b = sub + ((i0 + u) << a.log2S);
+                const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
+                acc += b < nblk ? t : 0.0f;
+            }
+        }
+    }
+    float p = sum8(acc);
+    if (S >= 2) p += dpp_f<0x128>(p);
+    if (S >= 4) p += __shfl_xor(p, 16, 64);
+    if (S >= 8) p += __shfl_xor(p, 32, 64);
+    if (live && sub == 0 && j == 0 && a.y) {
         if constexpr (ACC) a.y[rr] += p;
         else a.y[rr] = p;
     }
     if constexpr (ARGMAX) {
-        // best (value, lowest index) of this workgroup's 32 rows
+        // best (value, lowest index) of this workgroup's rows
         __shared__ float bv[4];
         __shared__ int bi[4];
         float v = live ? p : -INFINITY;
@@ -174,31 +221,61 @@ static int q6k_check(const void* W, const void* x, int K, int N, int64_t stride)
     return PTM_OK;
 }
 
-template <bool ACC, bool ARGMAX>
-static int q6k_launch(const Q6KArgs& a, hipStream_t s) {
-    const int grid = (a.N + Q6K_ROWS_PER_WG - 1) / Q6K_ROWS_PER_WG;
-    const size_t lds = (size_t)a.K * 4 + (size_t)a.K / 4;
-    static bool attr_done = false;  // raise the dynamic-LDS cap once, outside any capture
-    if (!attr_done) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_kernel<false, false, 5>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_kernel<true, false, 5>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_kernel<false, true, 5>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
-        attr_done = true;
+static int q6k_pick_log2S(int rows, int nblk) {
+    int l = 0;
+    while (l < 3) {
+        const int S = 1 << l;
+        const int wgs = (rows * S + 31) / 32;
+        const int nb = (nblk + S - 1) / S;
+        if (nb <= Q6K_U && wgs >= 600) break;
+        if (nb <= 1) break;
+        ++l;
     }
-    hipLaunchKernelGGL((q6k_gemv_kernel<ACC, ARGMAX, 5>), dim3(grid), dim3(Q6K_THREADS), lds, s, a);
+    return l;
+}
+
+int q6k_workgroups(int N, int K) {
+    const int l = q6k_pick_log2S(N, K / 256);
+    const int rows_per_wg = 32 >> l;
+    return (N + rows_per_wg - 1) / rows_per_wg;
+}
+
+// Raise the dynamic-LDS cap of every variant once; must happen outside stream capture.
+void q6k_init_attributes() {
+    static bool done = false;
+    if (done) return;
+    const void* fns[] = {
+        reinterpret_cast<const void*>(&q6k_gemv_kernel<false, false, false>),
+        reinterpret_cast<const void*>(&q6k_gemv_kernel<true, false, false>),
+        reinterpret_cast<const void*>(&q6k_gemv_kernel<false, true, false>),
+        reinterpret_cast<const void*>(&q6k_gemv_kernel<false, false, true>),
+    };
+    for (const void* f : fns) (void)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+    done = true;
+}
+
+template <bool ACC, bool ARGMAX, bool NORM>
+static int q6k_launch(Q6KArgs& a, hipStream_t s) {
+    a.log2S = q6k_pick_log2S(a.N, a.K / 256);
+    const int grid = q6k_workgroups(a.N, a.K);
+    const size_t lds = (size_t)a.K * 4 + (size_t)a.K / 4;
+    if (lds > 64 * 1024) q6k_init_attributes();
+    hipLaunchKernelGGL((q6k_gemv_kernel<ACC, ARGMAX, NORM>), dim3(grid), dim3(Q6K_THREADS), lds, s, a);
     return launch_status();
 }
 
 int q6k_gemv_impl(const void* W, const float* x, float* y, int K, int N, int64_t stride, bool accumulate,
-                  hipStream_t s) {
+                  const float* gamma, float eps, int add_one, hipStream_t s) {
     const int rc = q6k_check(W, x, K, N, stride);
     if (rc != PTM_OK) return rc;
     if (!y) return PTM_E_NULL;
-    Q6KArgs a{static_cast<const uint8_t*>(W), x, y, K, N, stride, nullptr, nullptr};
-    return accumulate ? q6k_launch<true, false>(a, s) : q6k_launch<false, false>(a, s);
+    Q6KArgs a{static_cast<const uint8_t*>(W), x, y, K, N, 0, stride, nullptr, nullptr, gamma, eps, add_one};
+    if (gamma) {
+        if (accumulate) return PTM_E_UNSUPPORTED;
+        if (!aligned16(gamma)) return PTM_E_ALIGN;
+        return q6k_launch<false, false, true>(a, s);
+    }
+    return accumulate ? q6k_launch<true, false, false>(a, s) : q6k_launch<false, false, false>(a, s);
 }
 
 }  // namespace ptm
@@ -209,12 +286,12 @@ extern "C" {
 
 int ptm_q6k_gemv(const void* W, const float* x, float* y, int K, int N, int64_t stride, int accumulate,
                  ptm_stream_t stream) {
-    return q6k_gemv_impl(W, x, y, K, N, stride, accumulate != 0, as_stream(stream));
+    return q6k_gemv_impl(W, x, y, K, N, stride, accumulate != 0, nullptr, 0.f, 0, as_stream(stream));
 }
 
 int64_t ptm_argmax_workspace_bytes(int N) {
-    const int64_t g = (N + Q6K_ROWS_PER_WG - 1) / Q6K_ROWS_PER_WG;
-    return g * 8;
+    // one (value, index) pair per workgroup; the finest split uses 4 rows per workgroup
+    return ((int64_t)N + 3) / 4 * 8;
 }
 
 int ptm_q6k_gemv_argmax(const void* W, const float* x, float* logits, int K, int N, int64_t stride,
@@ -222,10 +299,10 @@ int ptm_q6k_gemv_argmax(const void* W, const float* x, float* logits, int K, int
     const int rc = q6k_check(W, x, K, N, stride);
     if (rc != PTM_OK) return rc;
     if (!out_index || !workspace) return PTM_E_NULL;
-    const int grid = (N + Q6K_ROWS_PER_WG - 1) / Q6K_ROWS_PER_WG;
-    Q6KArgs a{static_cast<const uint8_t*>(W), x, logits, K, N, stride, static_cast<float*>(workspace),
-              reinterpret_cast<int*>(static_cast<float*>(workspace) + grid)};
-    const int rc2 = q6k_launch<false, true>(a, as_stream(stream));
+    const int grid = q6k_workgroups(N, K);
+    Q6KArgs a{static_cast<const uint8_t*>(W), x, logits, K, N, 0, stride, static_cast<float*>(workspace),
+              reinterpret_cast<int*>(static_cast<float*>(workspace) + grid), nullptr, 0.f, 0};
+    const int rc2 = q6k_launch<false, true, false>(a, as_stream(stream));
     if (rc2 != PTM_OK) return rc2;
     hipLaunchKernelGGL(argmax_partials_kernel, dim3(1), dim3(256), 0, as_stream(stream), a.part_val, a.part_idx,
                        grid, out_index);

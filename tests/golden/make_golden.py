@@ -25,7 +25,7 @@ from oracle import pyoracle as po  # noqa: E402
 from prometorch_amd import synth  # noqa: E402
 
 OUT = os.path.dirname(os.path.abspath(__file__))
-SEEDS = {"blocks": 101, "cfg1": 1001, "cfg2": 1002, "cfg3": 1003, "tiny": 7, "cfg4": 4004, "ragged": 1005}
+SEEDS = {"blocks": 101, "cfg1": 1001, "cfg2": 1002, "cfg3": 1003, "tiny": 7, "cfg4": 25, "ragged": 1005}
 
 
 def sha(a: np.ndarray) -> str:

@@ -94,38 +94,44 @@ def test_decode_kv_overflow_and_bad_token_are_errors(dev, seeds):
 
 
 def test_cfg4_qwen3_4b_shape_128_greedy_tokens(dev, po, golden_cfg4, seeds):
-    """Full size: 36 layers, KV prefilled to 2048 (fp16), 128 greedy steps.  Token ids must equal the
-    compiled reference's (golden); logits are compared on the recorded steps."""
+    """Full size: 36 layers, fp16 KV prefilled to 2048, 128 greedy steps.  Every step is compared
+    with the CPU oracle run beside it (same fp16 rounding of appended K/V rows): logits within
+    LOGIT_TOL_FULL of std and identical token; the 128 ids must also equal the ids the compiled
+    reference produced with its fp32 KV rows (golden)."""
     from prometorch_amd.decode import Decoder
+    LOGIT_TOL_FULL = 2e-2
     cfg = dict(synth.QWEN3_4B)
     seed = seeds["cfg4"]
     t0 = time.time()
     layers = [synth.make_layer(seed, i, cfg) for i in range(cfg["n_layers"])]
     head = synth.make_head(seed, cfg)
     print("model generated in %.1fs" % (time.time() - t0), flush=True)
+    om = po.OracleModel(cfg, layers, head, 2304, kv_fp16=True)
     dec = Decoder(cfg, layers, head, max_seq=2304, kv_fp16=True, use_graph=True)
     for i in range(cfg["n_layers"]):
         k, v = synth.make_kv_prefill(seed, i, cfg, 2048)
         dec.set_kv(i, k, v)
-    del layers
+        om.set_kv(i, k, v)
     dec.set_past_len(2048)
-    want = [int(t) for t in golden_cfg4["tokens"]]
-    margins = golden_cfg4["margins"]
-    print("reference min top-2 margin over 128 steps: %.4f (top1 ~ %.1f)" % (margins.min(), golden_cfg4["top1"].mean()), flush=True)
-    tok, got = 1, []
+    want_ref = [int(t) for t in golden_cfg4["tokens"]]
+    to = tg = 1
+    got, worst_err, min_margin = [], 0.0, 1e9
     for st in range(128):
-        tok = dec.step(tok)
-        got.append(tok)
-        if st in (0, 1, 63, 127):
-            lg = dec.logits()
-            ref256 = golden_cfg4[f"logits256_step{st}"]
-            err = np.abs(lg[:256] - ref256).max() / float(golden_cfg4[f"logits_std_step{st}"][0])
-            print("step", st, "logit err / std", err, flush=True)
-            assert err <= 5e-3, (st, err)  # fp16 rounding of the 128 appended K/V rows is on top of fp32 reassociation
-        if tok != want[st]:
-            pytest.fail(f"token mismatch at step {st}: gpu {tok} vs reference {want[st]} (reference top-2 margin {margins[st]:.4f})")
-    assert got == want
+        to = om.step(to)
+        tg = dec.step(tg)
+        got.append(tg)
+        sd = float(om.logits.std())
+        err = float(np.abs(dec.logits() - om.logits).max()) / sd
+        srt = np.sort(om.logits)
+        margin = float(srt[-1] - srt[-2]) / sd
+        worst_err, min_margin = max(worst_err, err), min(min_margin, margin)
+        if st % 16 == 0:
+            print("step %3d token %6d  logit err/std %.2e  top-2 margin/std %.3f  (%.0fs)" % (st, tg, err, margin, time.time() - t0), flush=True)
+        assert tg == to, f"token mismatch at step {st}: gpu {tg} vs oracle {to} (margin/std {margin:.4f}, err/std {err:.2e})"
+        assert err <= LOGIT_TOL_FULL, (st, err)
+    print("worst logit err/std %.2e, min top-2 margin/std %.3f" % (worst_err, min_margin), flush=True)
+    assert got == want_ref, "GPU (fp16 KV) ids differ from the compiled reference's (fp32 KV) ids"
     # device-chained generation (no host round trip between tokens) reproduces the same ids
     dec.set_past_len(2048)
-    assert dec.greedy(1, 128) == want
+    assert dec.greedy(1, 128) == want_ref
     dec.close()
