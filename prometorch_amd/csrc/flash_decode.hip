@@ -193,6 +193,283 @@ __global__ __launch_bounds__(256) void flash_decode_reduce_kernel(const float* _
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Whole attention step of one token in ONE launch: per-head QK-norm + NeoX RoPE of q and of the new
+// k row, K/V cache append, split-KV attention over the cache, and the merge of the splits.
+//   * every workgroup normalises/rotates the 4..8 query heads it needs itself (512..1024 values);
+//   * the workgroup whose chunk contains the new position also produces the new K/V row, writes it
+//     to the cache and uses it from LDS (the cache row is not yet visible to its own loads);
+//   * the merge is done by whichever workgroup of a kv head finishes last (device-scope counter,
+//     release/acquire fences around it); the counter is left at zero for the next launch.
+// The counters (n_kv_heads x uint32) must be zero before the first launch and are shared by
+// consecutive launches on one stream; launches that overlap in time must not share them.
+// ---------------------------------------------------------------------------------------------
+struct AttnArgs {
+    const float *Q, *K, *V, *qw, *kw, *rope;
+    void *Kc, *Vc;
+    float *pO, *pL, *pM, *O;
+    unsigned* counters;
+    const int64_t* d_past;
+    int n_heads, n_kv_heads, max_seq, add_one;
+    float scale, eps;
+};
+
+// one wave: RMSNorm (optional) + NeoX rotation of a head held as pairs (t, t+HD/2); results to dst[HD]
+template <int HD>
+__device__ __forceinline__ void head_norm_rope(const float* __restrict__ src, const float* __restrict__ w,
+                                               const float* __restrict__ cs, float eps, int add_one, int lane,
+                                               float& r0, float& r1) {
+    constexpr int HALF = HD / 2;
+    const bool on = lane < HALF;
+    float x0 = on ? src[lane] : 0.0f, x1 = on ? src[lane + HALF] : 0.0f;
+    if (w) {
+        float ss = fmaf(x0, x0, 0.0f);
+        ss = fmaf(x1, x1, ss);
+        ss = sum64(ss);
+        const float rs = 1.0f / sqrtf(ss / (float)HD + eps);
+        const float one = add_one ? 1.0f : 0.0f;
+        if (on) {
+            x0 = x0 * rs * (w[lane] + one);
+            x1 = x1 * rs * (w[lane + HALF] + one);
+        }
+    }
+    const float c = on ? cs[lane] : 1.0f, s = on ? cs[HALF + lane] : 0.0f;
+    r0 = fmaf(x0, c, -(x1 * s));
+    r1 = fmaf(x0, s, x1 * c);
+}
+
+template <bool KV16, int HD, int G>
+__global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const AttnArgs a) {
+    constexpr int LPP = HD / 8, PPW = 64 / LPP, PPB = PPW * 4, NPASS = FD_CHUNK / PPB, HALF = HD / 2;
+    constexpr int NOUT = G * HD / 4;                    // float4 outputs of the merge
+    constexpr int NSLOT = NOUT >= 256 ? 1 : 256 / NOUT;
+    __shared__ float s_q[G][HD];
+    __shared__ float s_p[G][FD_CHUNK];
+    __shared__ float s_o[4][G][HD];
+    __shared__ __align__(16) float4 s_stage[256];      // merge staging: NSLOT x NOUT <= 256 float4
+    __shared__ float s_new[2][HD];
+    __shared__ float s_M[G], s_den[G];
+    __shared__ int s_last;
+
+    const int64_t past = *a.d_past;
+    if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
+    const int64_t total = past + 1;
+    const int split = blockIdx.x, kvh = blockIdx.y;
+    const int64_t t0 = (int64_t)split * FD_CHUNK;
+    if (t0 >= total) return;
+    const int ns = (int)((total + FD_CHUNK - 1) / FD_CHUNK);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int dl = lane % LPP, pl = lane / LPP;
+    const int kv_dim = a.n_kv_heads * HD;
+    const int64_t col = (int64_t)kvh * HD + dl * 8;
+    const bool owner = past >= t0 && past < t0 + FD_CHUNK;
+
+    // cached K/V rows of the chunk (the new position is not in the cache yet: clamp below it)
+    float kreg[NPASS][8], vreg[NPASS][8];
+    const int64_t last_cached = past > 0 ? past - 1 : 0;
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+        const int64_t t = t0 + pass * PPB + wave * PPW + pl;
+        const int64_t tc = t < past ? t : last_cached;
+        load8<KV16>(a.Kc, tc * kv_dim + col, kreg[pass]);
+        load8<KV16>(a.Vc, tc * kv_dim + col, vreg[pass]);
+    }
+
+    // q heads of this kv group (wave w takes heads w, w+4, ...); owner: the new K row and V row
+    const float* cs = a.rope + past * HD;
+    for (int g = wave; g < G; g += 4) {
+        float r0, r1;
+        head_norm_rope<HD>(a.Q + (int64_t)(kvh * G + g) * HD, a.qw, cs, a.eps, a.add_one, lane, r0, r1);
+        if (lane < HALF) { s_q[g][lane] = r0; s_q[g][lane + HALF] = r1; }
+    }
+    if (owner) {
+        const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;
+        if (wave == (G % 4)) {  // the wave with the fewest q heads
+            float r0, r1;
+            head_norm_rope<HD>(a.K + (int64_t)kvh * HD, a.kw, cs, a.eps, a.add_one, lane, r0, r1);
+            if (lane < HALF) {
+                if constexpr (KV16) {
+                    const __half h0 = __float2half_rn(r0), h1 = __float2half_rn(r1);
+                    static_cast<__half*>(a.Kc)[rowoff + lane] = h0;
+                    static_cast<__half*>(a.Kc)[rowoff + lane + HALF] = h1;
+                    r0 = __half2float(h0);
+                    r1 = __half2float(h1);
+                } else {
+                    static_cast<float*>(a.Kc)[rowoff + lane] = r0;
+                    static_cast<float*>(a.Kc)[rowoff + lane + HALF] = r1;
+                }
+                s_new[0][lane] = r0;
+                s_new[0][lane + HALF] = r1;
+            }
+        } else if (wave == ((G + 1) % 4)) {
+            for (int i = lane; i < HD; i += 64) {
+                float v = a.V[(int64_t)kvh * HD + i];
+                if constexpr (KV16) {
+                    const __half hv = __float2half_rn(v);
+                    static_cast<__half*>(a.Vc)[rowoff + i] = hv;
+                    v = __half2float(hv);
+                } else {
+                    static_cast<float*>(a.Vc)[rowoff + i] = v;
+                }
+                s_new[1][i] = v;
+            }
+        }
+    }
+    __syncthreads();
+
+    float q[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[g][i] = s_q[g][dl * 8 + i];
+
+    // ---- scores ----
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+        const int tl = pass * PPB + wave * PPW + pl;
+        const int64_t t = t0 + tl;
+        if (t == past) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { kreg[pass][i] = s_new[0][dl * 8 + i]; vreg[pass][i] = s_new[1][dl * 8 + i]; }
+        }
+        const bool valid = t < total;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float d = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], kreg[pass][i], d);
+            d = (LPP == 16) ? sum16(d) : sum8(d);
+            if (dl == 0) s_p[g][tl] = valid ? d * a.scale : -INFINITY;
+        }
+    }
+    __syncthreads();
+    for (int g = wave; g < G; g += 4) {
+        const float sc = s_p[g][lane];
+        const float m = max64(sc);
+        const float p = expf(sc - m);
+        const float l = sum64(p);
+        s_p[g][lane] = p;
+        if (lane == 0) {
+            const int64_t o = (int64_t)split * a.n_heads + kvh * G + g;
+            a.pM[o] = m;
+            a.pL[o] = l;
+        }
+    }
+    __syncthreads();
+    float acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+        const int tl = pass * PPB + wave * PPW + pl;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float p = s_p[g][tl];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, vreg[pass][i], acc[g][i]);
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float v = acc[g][i];
+            for (int off = LPP; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
+            acc[g][i] = v;
+        }
+    if (pl == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s_o[wave][g][dl * 8 + i] = acc[g][i];
+    }
+    __syncthreads();
+    for (int e = tid; e < G * HD; e += FD_THREADS) {
+        const int g = e / HD, d = e % HD;
+        const float o = (s_o[0][g][d] + s_o[1][g][d]) + (s_o[2][g][d] + s_o[3][g][d]);
+        a.pO[((int64_t)split * a.n_heads + kvh * G + g) * HD + d] = o;
+    }
+
+    // ---- which workgroup of this kv head is last? ----
+    __threadfence();  // release: this workgroup's partials before the counter increment
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned old = atomicAdd(&a.counters[kvh], 1u);
+        s_last = (old == (unsigned)(ns - 1));
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();  // acquire: the other workgroups' partials
+    if (tid == 0) a.counters[kvh] = 0u;
+
+    // ---- merge the ns splits of the G heads (split order is fixed: the result is reproducible) ----
+    for (int g = wave; g < G; g += 4) {
+        const int h = kvh * G + g;
+        float m = -INFINITY;
+        for (int sI = lane; sI < ns; sI += 64) m = fmaxf(m, a.pM[(int64_t)sI * a.n_heads + h]);
+        m = max64(m);
+        float den = 0.0f;
+        for (int sI = lane; sI < ns; sI += 64)
+            den = fmaf(expf(a.pM[(int64_t)sI * a.n_heads + h] - m), a.pL[(int64_t)sI * a.n_heads + h], den);
+        den = sum64(den);
+        if (lane == 0) { s_M[g] = m; s_den[g] = den; }
+    }
+    __syncthreads();
+    float4* stage = s_stage;
+    const int o_idx = tid % NOUT, slot = tid / NOUT;
+    if (slot < NSLOT) {
+        const int g = o_idx / (HD / 4), d4 = o_idx % (HD / 4), h = kvh * G + g;
+        const float M = s_M[g];
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s0 = slot; s0 < ns; s0 += NSLOT * 8) {
+            float4 v[8];
+            float w[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int sI = s0 + u * NSLOT;
+                const int sc = sI < ns ? sI : ns - 1;
+                v[u] = reinterpret_cast<const float4*>(a.pO)[((int64_t)sc * a.n_heads + h) * (HD / 4) + d4];
+                w[u] = sI < ns ? expf(a.pM[(int64_t)sc * a.n_heads + h] - M) : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                sum.x = fmaf(w[u], v[u].x, sum.x);
+                sum.y = fmaf(w[u], v[u].y, sum.y);
+                sum.z = fmaf(w[u], v[u].z, sum.z);
+                sum.w = fmaf(w[u], v[u].w, sum.w);
+            }
+        }
+        stage[slot * NOUT + o_idx] = sum;
+    }
+    __syncthreads();
+    if (tid < NOUT) {
+        const int g = tid / (HD / 4), d4 = tid % (HD / 4), h = kvh * G + g;
+        float4 t = stage[tid];
+        for (int r = 1; r < NSLOT; ++r) {
+            const float4 u = stage[r * NOUT + tid];
+            t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+        }
+        const float inv = 1.0f / (s_den[g] + 1e-10f);  // reference: gguf_model.h:3589
+        reinterpret_cast<float4*>(a.O)[(int64_t)h * (HD / 4) + d4] = make_float4(t.x * inv, t.y * inv, t.z * inv, t.w * inv);
+    }
+}
+
+template <bool KV16, int HD>
+static int attn_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
+#define PTM_AT(GG) hipLaunchKernelGGL((attn_decode_fused_kernel<KV16, HD, GG>), grid, dim3(FD_THREADS), 0, s, a)
+    switch (G) {
+        case 1: PTM_AT(1); break;
+        case 2: PTM_AT(2); break;
+        case 4: PTM_AT(4); break;
+        case 8: PTM_AT(8); break;
+        default: return PTM_E_UNSUPPORTED;
+    }
+#undef PTM_AT
+    return launch_status();
+}
+
 template <bool KV16, int HD>
 static int fd_launch_g(int G, dim3 grid, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* pO,
                        float* pL, float* pM, int n_heads, int n_kv_heads, const int64_t* d_past, int max_seq,
@@ -243,6 +520,27 @@ int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, f
     hipLaunchKernelGGL(flash_decode_reduce_kernel, dim3(n_heads), dim3(256), 0, s, partial_O, partial_lse,
                        partial_max, O, n_heads, head_dim, d_past_len, max_seq);
     return launch_status();
+}
+
+int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                          const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
+                          float* partial_lse, float* partial_max, uint32_t* counters, const float* rope_table,
+                          int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                          float scale, float eps, int add_one, int kv_fp16, ptm_stream_t stream) {
+    if (!Q || !K || !V || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max || !counters ||
+        !rope_table || !d_past_len)
+        return PTM_E_NULL;
+    if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
+    if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
+    if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
+    if (!aligned16(K_cache) || !aligned16(V_cache) || !aligned16(partial_O) || !aligned16(O)) return PTM_E_ALIGN;
+    AttnArgs a{Q, K, V, q_norm_w, k_norm_w, rope_table, K_cache, V_cache, partial_O, partial_lse, partial_max, O,
+               counters, d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps};
+    const int G = n_heads / n_kv_heads;
+    const dim3 grid(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
+    hipStream_t s = as_stream(stream);
+    if (kv_fp16) return head_dim == 128 ? attn_launch_g<true, 128>(G, grid, s, a) : attn_launch_g<true, 64>(G, grid, s, a);
+    return head_dim == 128 ? attn_launch_g<false, 128>(G, grid, s, a) : attn_launch_g<false, 64>(G, grid, s, a);
 }
 
 }  // extern "C"

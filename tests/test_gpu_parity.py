@@ -463,3 +463,59 @@ def test_elementwise_embedding_argmax(dev, po):
     torch.cuda.synchronize()
     assert np.array_equal(cache[2:5].cpu().numpy().view(np.uint16), src.astype(np.float16).view(np.uint16))
     assert float(cache[:2].abs().max()) == 0 and float(cache[5:].abs().max()) == 0
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+@pytest.mark.parametrize("nh,nkv,hd,past", [(32, 8, 128, 2048), (32, 8, 128, 2111), (32, 8, 128, 2112), (4, 2, 64, 19),
+                                            (8, 8, 128, 0), (16, 2, 64, 63), (8, 1, 64, 64), (8, 8, 64, 130)])
+def test_attn_decode_fused_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past):
+    """QK-norm + RoPE + KV append + attention + merge in one launch, three tokens in a row (the
+    arrival counters are reused), against the oracle's pieces in the reference's order."""
+    max_seq = ((past + 3 + 63) // 64 + 1) * 64
+    r = synth.rng_for(46, nh, hd, past)
+    kvd = nkv * hd
+    k16 = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16)
+    v16 = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16)
+    kf, vf = k16.astype(np.float32), v16.astype(np.float32)
+    qw = (1 + 0.1 * synth.make_x(r, hd)).astype(np.float32)
+    kw = (1 + 0.1 * synth.make_x(r, hd)).astype(np.float32)
+    dt = torch.float16 if kv_fp16 else torch.float32
+    Kc, Vc = cu(kf).to(dt), cu(vf).to(dt)
+    Kc[past:] = float("nan")   # rows at and past the new position must not leak into the result
+    Vc[past:] = float("nan")
+    S = ops.flash_decode_num_splits(max_seq)
+    pO = torch.empty(S * nh * hd, device="cuda")
+    pL = torch.empty(S * nh, device="cuda")
+    pM = torch.empty(S * nh, device="cuda")
+    cnt = torch.zeros(nkv, dtype=torch.int32, device="cuda")
+    table = ops.rope_table(max_seq, hd, 1e6).cuda()
+    O = torch.empty(nh * hd, device="cuda")
+    d_past = torch.zeros(1, dtype=torch.int64, device="cuda")
+    scale = 1.0 / np.sqrt(hd)
+    for step in range(3):
+        pos = past + step
+        q = (synth.make_x(r, nh * hd) * 3).astype(np.float32)
+        k = (synth.make_x(r, kvd) * 3).astype(np.float32)
+        v = synth.make_x(r, kvd)
+        qn = np.concatenate([po.rmsnorm(q[h * hd:(h + 1) * hd], qw, 1e-6) for h in range(nh)])
+        kn = np.concatenate([po.rmsnorm(k[h * hd:(h + 1) * hd], kw, 1e-6) for h in range(nkv)])
+        c, s = po.rope_tables(pos, hd, 1e6)
+        qr, kr = po.rope_neox(qn, kn, c, s, nh, nkv, hd)
+        kf[pos] = kr.astype(np.float16).astype(np.float32) if kv_fp16 else kr
+        vf[pos] = v.astype(np.float16).astype(np.float32) if kv_fp16 else v
+        want = np.concatenate([po.attn_head(qr[h * hd:(h + 1) * hd], kf, vf, pos + 1, kvd, hd, scale,
+                                            col0=(h // (nh // nkv)) * hd) for h in range(nh)])
+        d_past.fill_(pos)
+        Q, K, V = cu(q), cu(k), cu(v)
+        ops.attn_decode_fused(Q, K, V, cu(qw), cu(kw), Kc, Vc, O, pO, pL, pM, cnt, table, nh, nkv, hd, d_past,
+                              max_seq, scale, 1e-6, kv_fp16=kv_fp16)
+        torch.cuda.synchronize()
+        got = O.cpu().numpy()
+        assert np.all(np.isfinite(got)), (step, pos)
+        assert np.abs(got - want).max() <= 3e-5 * max(np.abs(want).max(), 1e-3) + 1e-6, (step, pos)
+        assert int(cnt.abs().sum().item()) == 0                      # counters are back at zero
+        assert np.array_equal(Q.cpu().numpy(), q)                    # inputs untouched
+        krow = Kc[pos].float().cpu().numpy()
+        assert np.abs(krow - kf[pos]).max() <= (2e-3 if kv_fp16 else 2e-6) * np.abs(kf[pos]).max()
+        assert np.array_equal(Vc[pos].float().cpu().numpy(), vf[pos])
+        kf[pos] = krow                                               # continue from what the cache really holds
