@@ -163,17 +163,15 @@ int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, f
                      int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq, float scale,
                      int kv_fp16, ptm_stream_t stream);
 
-/* The two operators above in ONE launch: per-head QK-norm + NeoX RoPE of Q and of the new K row, K/V
- * append at row *d_past_len, split-KV attention over rows [0, *d_past_len], merge of the splits
- * (done by the last workgroup of each kv head).  Q, K, V are the raw projections and are NOT
- * modified.  rope_table: device [max_seq][head_dim] as filled by ptm_rope_table_host (required).
- * counters: n_kv_heads uint32 of device scratch that must be zero before the first call; every call
- * leaves them zero.  Calls sharing counters / partial buffers must not overlap in time.
+/* The two operators above fused: one launch does per-head QK-norm + NeoX RoPE of Q and of the new K
+ * row, the K/V append at row *d_past_len and the split-KV attention over rows [0, *d_past_len]; a
+ * second small launch merges the splits.  Q, K, V are the raw projections and are NOT modified.
+ * rope_table: device [max_seq][head_dim] as filled by ptm_rope_table_host (required).
  * Stands in for launch_fused_qknorm_rope_kvwrite_graph + launch_flash_decode(_fp16)_graph
  * (CUDAOps.h:653-673) as forward_decode issues them back to back (gguf_model.h:2785-2832). */
 int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const float* q_norm_w,
                           const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
-                          float* partial_lse, float* partial_max, uint32_t* counters, const float* rope_table,
+                          float* partial_lse, float* partial_max, const float* rope_table,
                           int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
                           float scale, float eps, int add_one, int kv_fp16, ptm_stream_t stream);
 

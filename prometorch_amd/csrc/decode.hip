@@ -7,7 +7,7 @@
 // Per layer (Q4_K_M mix: q/k/o/gate/up Q4_K, v/down Q6_K):
 //   RMSNorm + Q4_K {q,k} in one launch ; RMSNorm + Q6_K v in another (the norm is recomputed per
 //   workgroup; quant type is dispatched per tensor, as gemv_scratch does)
-//   QK-norm + NeoX RoPE + K/V append + split-KV attention + merge in one launch
+//   QK-norm + NeoX RoPE + K/V append + split-KV attention in one launch, then the split merge
 //   o-proj GEMV accumulating into the residual
 //   rmsnorm + gate + up + SiLU*up in one launch
 //   down-proj GEMV accumulating into the residual
@@ -62,7 +62,6 @@ struct ptm_decoder {
     int64_t* d_past = nullptr;
     int64_t* d_next = nullptr;
     int64_t* d_tokens = nullptr;
-    uint32_t* counters = nullptr;  // per-kv-head arrival counters of the fused attention (kept at zero)
     int64_t* h_pinned = nullptr;  // [max_seq] pinned host staging for token ids
     int64_t past_len = 0;
     int status = PTM_OK;
@@ -114,9 +113,9 @@ static int enqueue_step(ptm_decoder* d) {
                 PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->x, false, L.attn_norm, c.rms_eps, 0, H,
                                        (int64_t)(H / 256) * 144, false, s));
         }
-        // QK-norm + RoPE + K/V append + split-KV attention + merge: one launch
+        // QK-norm + RoPE + K/V append + split-KV attention in one launch, plus the small merge launch
         PTM_TRY(ptm_attn_decode_fused(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn, d->pO,
-                                      d->pL, d->pM, d->counters, d->rope, c.n_heads, c.n_kv_heads, hd, d->d_past,
+                                      d->pL, d->pM, d->rope, c.n_heads, c.n_kv_heads, hd, d->d_past,
                                       c.max_seq, 1.0f / sqrtf((float)hd), c.rms_eps, 0, c.kv_fp16, s));
         PTM_TRY(gemv_any(L.o, d->attn, d->x, true, s));  // x += Wo . attn
         if (L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
@@ -186,8 +185,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
                  o_pM = take(4 * (size_t)S * c.n_heads), o_rope = take(4 * (size_t)c.max_seq * c.head_dim),
                  o_xq8 = take((size_t)ptm_q8_bytes(H > c.inter ? H : c.inter)),
                  o_ws = take((size_t)ptm_argmax_workspace_bytes(c.vocab)), o_tok = take(256), o_past = take(256),
-                 o_next = take(256), o_step = take(256), o_tokens = take(8 * (size_t)c.max_seq),
-                 o_cnt = take(4 * (size_t)c.n_kv_heads);
+                 o_next = take(256), o_step = take(256), o_tokens = take(8 * (size_t)c.max_seq);
     if ((rc = hip_status(hipMalloc(&d->slab, off))) != PTM_OK) { delete d; return rc; }
     uint8_t* base = static_cast<uint8_t*>(d->slab);
     d->x = (float*)(base + o_x); d->xn = (float*)(base + o_xn); d->q = (float*)(base + o_q);
@@ -198,8 +196,6 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->amax_ws = base + o_ws; d->d_token = (int*)(base + o_tok); d->d_past = (int64_t*)(base + o_past);
     d->d_next = (int64_t*)(base + o_next); d->d_step = (int*)(base + o_step);
     d->d_tokens = (int64_t*)(base + o_tokens);
-    d->counters = (uint32_t*)(base + o_cnt);
-    if ((rc = hip_status(hipMemset(d->counters, 0, 4 * (size_t)c.n_kv_heads))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     q6k_init_attributes();  // one-time kernel attributes, before anything can be captured
 
     if ((rc = hip_status(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking))) != PTM_OK) { ptm_decode_destroy(d); return rc; }

@@ -146,69 +146,101 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     }
 }
 
-// grid n_heads, 256 threads: merge the active splits.  Thread (slot = tid / head_dim-quarter...) layout:
-// the 256 threads form R = 256/head_dim split-slots x head_dim dims; slot r sums splits r, r+R, ...
-// (independent loads, all in flight), then the R slot sums are added in slot order.
-__global__ __launch_bounds__(256) void flash_decode_reduce_kernel(const float* __restrict__ pO,
-                                                                  const float* __restrict__ pL,
-                                                                  const float* __restrict__ pM, float* __restrict__ O,
-                                                                  int n_heads, int head_dim,
-                                                                  const int64_t* __restrict__ d_past, int max_seq) {
-    __shared__ float s_w[256];     // per-split weight exp(m_s - M)
-    __shared__ float s_num[256];
+// Merge of the active splits: grid n_heads, 256 threads = NSLOT split-slots x HD/4 float4 outputs.
+// Slot r sums splits r, r+NSLOT, ... in batches of 8 independent loads (the first batch is issued
+// before the max/denominator reductions so its latency overlaps them); slot sums are then added in
+// slot order, so the result does not depend on timing.
+template <int HD>
+__global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __restrict__ pO,
+                                                                 const float* __restrict__ pL,
+                                                                 const float* __restrict__ pM, float* __restrict__ O,
+                                                                 int n_heads, const int64_t* __restrict__ d_past,
+                                                                 int max_seq) {
+    constexpr int NOUT = HD / 4, NSLOT = 256 / NOUT;
+    __shared__ __align__(16) float4 s_stage[256];
     __shared__ float s_red[8];
     int64_t total = *d_past + 1;
     if (total > max_seq) total = max_seq;
+    if (total <= 0) return;
     const int ns = (int)((total + FD_CHUNK - 1) / FD_CHUNK);
     const int h = blockIdx.x, tid = threadIdx.x;
-    // global max and denominator over splits (ns may exceed 256: strided)
+    const int o_idx = tid % NOUT, slot = tid / NOUT;
+    const float4* pO4 = reinterpret_cast<const float4*>(pO);
+    float4 v[8];
+    float mm[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int sc = min(slot + u * NSLOT, ns - 1);
+        v[u] = pO4[((int64_t)sc * n_heads + h) * NOUT + o_idx];
+        mm[u] = pM[(int64_t)sc * n_heads + h];
+    }
     float m = -INFINITY;
-    for (int s = tid; s < ns; s += 256) m = fmaxf(m, pM[(int64_t)s * n_heads + h]);
+    for (int sI = tid; sI < ns; sI += 256) m = fmaxf(m, pM[(int64_t)sI * n_heads + h]);
     m = max64(m);
     if ((tid & 63) == 0) s_red[tid >> 6] = m;
     __syncthreads();
     const float M = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
     float den = 0.0f;
-    for (int s = tid; s < ns; s += 256) den = fmaf(expf(pM[(int64_t)s * n_heads + h] - M), pL[(int64_t)s * n_heads + h], den);
+    for (int sI = tid; sI < ns; sI += 256)
+        den = fmaf(expf(pM[(int64_t)sI * n_heads + h] - M), pL[(int64_t)sI * n_heads + h], den);
     den = sum64(den);
     if ((tid & 63) == 0) s_red[4 + (tid >> 6)] = den;
-    const int R = 256 / head_dim, slot = tid / head_dim, d = tid % head_dim;
-    float num = 0.0f;
-    for (int s0 = 0; s0 < ns; s0 += 256) {
-        __syncthreads();
-        if (s0 + tid < ns) s_w[tid] = expf(pM[(int64_t)(s0 + tid) * n_heads + h] - M);
-        __syncthreads();
-        const int lim = min(256, ns - s0);
-        for (int s = slot; s < lim; s += R)
-            num = fmaf(s_w[s], pO[((int64_t)(s0 + s) * n_heads + h) * head_dim + d], num);
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s0 = slot; s0 < ns; s0 += NSLOT * 8) {
+        if (s0 != slot) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int sc = min(s0 + u * NSLOT, ns - 1);
+                v[u] = pO4[((int64_t)sc * n_heads + h) * NOUT + o_idx];
+                mm[u] = pM[(int64_t)sc * n_heads + h];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float w = (s0 + u * NSLOT) < ns ? expf(mm[u] - M) : 0.0f;
+            sum.x = fmaf(w, v[u].x, sum.x);
+            sum.y = fmaf(w, v[u].y, sum.y);
+            sum.z = fmaf(w, v[u].z, sum.z);
+            sum.w = fmaf(w, v[u].w, sum.w);
+        }
     }
-    s_num[tid] = num;
+    s_stage[slot * NOUT + o_idx] = sum;
     __syncthreads();
-    if (tid < head_dim) {
-        float t = s_num[tid];
-        for (int r = 1; r < R; ++r) t += s_num[r * head_dim + tid];
+    if (tid < NOUT) {
+        float4 t = s_stage[tid];
+        for (int r = 1; r < NSLOT; ++r) {
+            const float4 u = s_stage[r * NOUT + tid];
+            t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+        }
         const float dsum = (s_red[4] + s_red[5]) + (s_red[6] + s_red[7]);
-        // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
-        O[(int64_t)h * head_dim + tid] = t * (1.0f / (dsum + 1e-10f));
+        const float inv = 1.0f / (dsum + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
+        reinterpret_cast<float4*>(O)[(int64_t)h * NOUT + tid] = make_float4(t.x * inv, t.y * inv, t.z * inv, t.w * inv);
     }
 }
 
+static int fd_merge(int head_dim, int n_heads, hipStream_t s, const float* pO, const float* pL, const float* pM, float* O,
+                    const int64_t* d_past, int max_seq) {
+    if (head_dim == 128)
+        hipLaunchKernelGGL(flash_decode_merge_kernel<128>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq);
+    else
+        hipLaunchKernelGGL(flash_decode_merge_kernel<64>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq);
+    return launch_status();
+}
+
 // ---------------------------------------------------------------------------------------------
-// Whole attention step of one token in ONE launch: per-head QK-norm + NeoX RoPE of q and of the new
-// k row, K/V cache append, split-KV attention over the cache, and the merge of the splits.
+// Front half of the attention step of one token in ONE launch: per-head QK-norm + NeoX RoPE of q and
+// of the new k row, K/V cache append, and the split-KV partial attention over the cache.
 //   * every workgroup normalises/rotates the 4..8 query heads it needs itself (512..1024 values);
 //   * the workgroup whose chunk contains the new position also produces the new K/V row, writes it
-//     to the cache and uses it from LDS (the cache row is not yet visible to its own loads);
-//   * the merge is done by whichever workgroup of a kv head finishes last (device-scope counter,
-//     release/acquire fences around it); the counter is left at zero for the next launch.
-// The counters (n_kv_heads x uint32) must be zero before the first launch and are shared by
-// consecutive launches on one stream; launches that overlap in time must not share them.
+//     to the cache and uses it from LDS (the cache row is not yet visible to its own loads).
+// The split merge stays a second, small launch: doing it in the last-arriving workgroup needs
+// device-scope release/acquire fences in all ~270 workgroups, which measured slower on MI355X
+// (L2 write-back per fence across the 8 XCDs) than the extra launch.
 // ---------------------------------------------------------------------------------------------
 struct AttnArgs {
     const float *Q, *K, *V, *qw, *kw, *rope;
     void *Kc, *Vc;
-    float *pO, *pL, *pM, *O;
-    unsigned* counters;
+    float *pO, *pL, *pM;
     const int64_t* d_past;
     int n_heads, n_kv_heads, max_seq, add_one;
     float scale, eps;
@@ -241,15 +273,10 @@ __device__ __forceinline__ void head_norm_rope(const float* __restrict__ src, co
 template <bool KV16, int HD, int G>
 __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const AttnArgs a) {
     constexpr int LPP = HD / 8, PPW = 64 / LPP, PPB = PPW * 4, NPASS = FD_CHUNK / PPB, HALF = HD / 2;
-    constexpr int NOUT = G * HD / 4;                    // float4 outputs of the merge
-    constexpr int NSLOT = NOUT >= 256 ? 1 : 256 / NOUT;
     __shared__ float s_q[G][HD];
     __shared__ float s_p[G][FD_CHUNK];
     __shared__ float s_o[4][G][HD];
-    __shared__ __align__(16) float4 s_stage[256];      // merge staging: NSLOT x NOUT <= 256 float4
     __shared__ float s_new[2][HD];
-    __shared__ float s_M[G], s_den[G];
-    __shared__ int s_last;
 
     const int64_t past = *a.d_past;
     if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
@@ -257,7 +284,6 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     const int split = blockIdx.x, kvh = blockIdx.y;
     const int64_t t0 = (int64_t)split * FD_CHUNK;
     if (t0 >= total) return;
-    const int ns = (int)((total + FD_CHUNK - 1) / FD_CHUNK);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int dl = lane % LPP, pl = lane / LPP;
     const int kv_dim = a.n_kv_heads * HD;
@@ -333,6 +359,10 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
             for (int i = 0; i < 8; ++i) { kreg[pass][i] = s_new[0][dl * 8 + i]; vreg[pass][i] = s_new[1][dl * 8 + i]; }
         }
         const bool valid = t < total;
+        if (!valid) {  // rows past the end carry weight 0; keep 0 * garbage from producing NaN
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vreg[pass][i] = 0.0f;
+        }
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float d = 0.0f;
@@ -392,68 +422,6 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
         a.pO[((int64_t)split * a.n_heads + kvh * G + g) * HD + d] = o;
     }
 
-    // ---- which workgroup of this kv head is last? ----
-    __threadfence();  // release: this workgroup's partials before the counter increment
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned old = atomicAdd(&a.counters[kvh], 1u);
-        s_last = (old == (unsigned)(ns - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();  // acquire: the other workgroups' partials
-    if (tid == 0) a.counters[kvh] = 0u;
-
-    // ---- merge the ns splits of the G heads (split order is fixed: the result is reproducible) ----
-    for (int g = wave; g < G; g += 4) {
-        const int h = kvh * G + g;
-        float m = -INFINITY;
-        for (int sI = lane; sI < ns; sI += 64) m = fmaxf(m, a.pM[(int64_t)sI * a.n_heads + h]);
-        m = max64(m);
-        float den = 0.0f;
-        for (int sI = lane; sI < ns; sI += 64)
-            den = fmaf(expf(a.pM[(int64_t)sI * a.n_heads + h] - m), a.pL[(int64_t)sI * a.n_heads + h], den);
-        den = sum64(den);
-        if (lane == 0) { s_M[g] = m; s_den[g] = den; }
-    }
-    __syncthreads();
-    float4* stage = s_stage;
-    const int o_idx = tid % NOUT, slot = tid / NOUT;
-    if (slot < NSLOT) {
-        const int g = o_idx / (HD / 4), d4 = o_idx % (HD / 4), h = kvh * G + g;
-        const float M = s_M[g];
-        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int s0 = slot; s0 < ns; s0 += NSLOT * 8) {
-            float4 v[8];
-            float w[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int sI = s0 + u * NSLOT;
-                const int sc = sI < ns ? sI : ns - 1;
-                v[u] = reinterpret_cast<const float4*>(a.pO)[((int64_t)sc * a.n_heads + h) * (HD / 4) + d4];
-                w[u] = sI < ns ? expf(a.pM[(int64_t)sc * a.n_heads + h] - M) : 0.0f;
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                sum.x = fmaf(w[u], v[u].x, sum.x);
-                sum.y = fmaf(w[u], v[u].y, sum.y);
-                sum.z = fmaf(w[u], v[u].z, sum.z);
-                sum.w = fmaf(w[u], v[u].w, sum.w);
-            }
-        }
-        stage[slot * NOUT + o_idx] = sum;
-    }
-    __syncthreads();
-    if (tid < NOUT) {
-        const int g = tid / (HD / 4), d4 = tid % (HD / 4), h = kvh * G + g;
-        float4 t = stage[tid];
-        for (int r = 1; r < NSLOT; ++r) {
-            const float4 u = stage[r * NOUT + tid];
-            t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
-        }
-        const float inv = 1.0f / (s_den[g] + 1e-10f);  // reference: gguf_model.h:3589
-        reinterpret_cast<float4*>(a.O)[(int64_t)h * (HD / 4) + d4] = make_float4(t.x * inv, t.y * inv, t.z * inv, t.w * inv);
-    }
 }
 
 template <bool KV16, int HD>
@@ -517,30 +485,31 @@ int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, f
                              : fd_launch_g<false, 64>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale);
     }
     if (rc != PTM_OK) return rc;
-    hipLaunchKernelGGL(flash_decode_reduce_kernel, dim3(n_heads), dim3(256), 0, s, partial_O, partial_lse,
-                       partial_max, O, n_heads, head_dim, d_past_len, max_seq);
-    return launch_status();
+    return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq);
 }
 
 int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const float* q_norm_w,
                           const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
-                          float* partial_lse, float* partial_max, uint32_t* counters, const float* rope_table,
+                          float* partial_lse, float* partial_max, const float* rope_table,
                           int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
                           float scale, float eps, int add_one, int kv_fp16, ptm_stream_t stream) {
-    if (!Q || !K || !V || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max || !counters ||
+    if (!Q || !K || !V || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max ||
         !rope_table || !d_past_len)
         return PTM_E_NULL;
     if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
     if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
     if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
     if (!aligned16(K_cache) || !aligned16(V_cache) || !aligned16(partial_O) || !aligned16(O)) return PTM_E_ALIGN;
-    AttnArgs a{Q, K, V, q_norm_w, k_norm_w, rope_table, K_cache, V_cache, partial_O, partial_lse, partial_max, O,
-               counters, d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps};
+    AttnArgs a{Q, K, V, q_norm_w, k_norm_w, rope_table, K_cache, V_cache, partial_O, partial_lse, partial_max,
+               d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps};
     const int G = n_heads / n_kv_heads;
     const dim3 grid(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
     hipStream_t s = as_stream(stream);
-    if (kv_fp16) return head_dim == 128 ? attn_launch_g<true, 128>(G, grid, s, a) : attn_launch_g<true, 64>(G, grid, s, a);
-    return head_dim == 128 ? attn_launch_g<false, 128>(G, grid, s, a) : attn_launch_g<false, 64>(G, grid, s, a);
+    int rc;
+    if (kv_fp16) rc = head_dim == 128 ? attn_launch_g<true, 128>(G, grid, s, a) : attn_launch_g<true, 64>(G, grid, s, a);
+    else rc = head_dim == 128 ? attn_launch_g<false, 128>(G, grid, s, a) : attn_launch_g<false, 64>(G, grid, s, a);
+    if (rc != PTM_OK) return rc;
+    return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq);
 }
 
 }  // extern "C"

@@ -210,14 +210,14 @@ def launch_flash_decode_fp16_graph(Q, K_cache_fp16, V_cache_fp16, O, partial_O, 
                               n_kv_heads, head_dim, d_past_len, max_seq, scale, stream, kv_fp16=True)
 
 
-def attn_decode_fused(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, partial_O, partial_lse, partial_max, counters,
+def attn_decode_fused(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, partial_O, partial_lse, partial_max,
                       rope_table, n_heads, n_kv_heads, head_dim, d_past_len, max_seq, scale, eps, add_one=False,
                       kv_fp16=True, stream=None):
-    """launch_fused_qknorm_rope_kvwrite_graph + launch_flash_decode(_fp16)_graph in one launch
+    """launch_fused_qknorm_rope_kvwrite_graph + launch_flash_decode(_fp16)_graph fused (one launch + a small merge launch)
     (CUDAOps.h:653-673; issued back to back at gguf_model.h:2785-2832)."""
     check(_L().ptm_attn_decode_fused(_ptr(Q), _ptr(K), _ptr(V), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(K_cache),
                                     _ptr(V_cache), _ptr(O), _ptr(partial_O), _ptr(partial_lse), _ptr(partial_max),
-                                    _ptr(counters), _ptr(rope_table), n_heads, n_kv_heads, head_dim, _ptr(d_past_len),
+                                    _ptr(rope_table), n_heads, n_kv_heads, head_dim, _ptr(d_past_len),
                                     max_seq, scale, eps, int(add_one), int(kv_fp16), _stream(stream)),
           "attn_decode_fused")
 
