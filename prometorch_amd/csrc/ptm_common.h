@@ -129,4 +129,79 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
     return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
+// ---- activation staging --------------------------------------------------------------------------
+// A 256-thread workgroup walks x[K] as float4 slots i = tid + 256*u.  Loads are issued four slots
+// at a time BEFORE any of them is consumed, so a staging pass costs one memory round trip per 4096
+// values instead of one per 1024.  For K <= 4096 the slots stay in registers between the
+// sum-of-squares pass and the normalise pass.
+struct XChunk { float4 v[4]; };
+
+__device__ __forceinline__ XChunk load_chunk(const float4* __restrict__ p, int base, int n4) {
+    XChunk c;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = base + (int)threadIdx.x + 256 * u;
+        c.v[u] = i < n4 ? p[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    return c;
+}
+
+__device__ __forceinline__ float chunk_sumsq(const XChunk& c, float ss) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        ss = fmaf(c.v[u].x, c.v[u].x, ss);
+        ss = fmaf(c.v[u].y, c.v[u].y, ss);
+        ss = fmaf(c.v[u].z, c.v[u].z, ss);
+        ss = fmaf(c.v[u].w, c.v[u].w, ss);
+    }
+    return ss;
+}
+
+// x * rs * (gamma [+1]) in the reference's order (cpu_quant_gemv.h:2599)
+__device__ __forceinline__ float4 norm4(float4 v, float4 g, float rs, float one) {
+    v.x = v.x * rs * (g.x + one);
+    v.y = v.y * rs * (g.y + one);
+    v.z = v.z * rs * (g.z + one);
+    v.w = v.w * rs * (g.w + one);
+    return v;
+}
+
+// Calls emit(i, value) for every float4 slot i of x (RMS-normalised with gamma when NORM), all 256
+// threads taking part; emit may use cross-lane ops (slots are handed out wave-uniformly: K % 256 == 0).
+template <bool NORM, typename Emit>
+__device__ __forceinline__ void stage_x_slots(const float* __restrict__ x, const float* __restrict__ gamma, int K,
+                                              float eps, int add_one, float* red4, Emit emit) {
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const float4* g4 = reinterpret_cast<const float4*>(gamma);
+    const int n4 = K / 4;
+    const bool kept = n4 <= 1024;
+    const float one = add_one ? 1.0f : 0.0f;
+    XChunk keep = load_chunk(x4, 0, n4), gk;
+    if constexpr (NORM) gk = load_chunk(g4, 0, n4);
+    float rs = 1.0f;
+    if constexpr (NORM) {
+        float ss = chunk_sumsq(keep, 0.0f);
+        for (int base = 1024; base < n4; base += 1024) ss = chunk_sumsq(load_chunk(x4, base, n4), ss);
+        ss = block_sum256(ss, red4);
+        rs = 1.0f / sqrtf(ss / (float)K + eps);
+    }
+    for (int base = 0; base < n4; base += 1024) {
+        XChunk c = keep, g = gk;
+        if (base > 0) {
+            c = load_chunk(x4, base, n4);
+            if constexpr (NORM) g = load_chunk(g4, base, n4);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = base + (int)threadIdx.x + 256 * u;
+            if (i < n4) {
+                float4 v = c.v[u];
+                if constexpr (NORM) v = norm4(v, g.v[u], rs, one);
+                emit(i, v);
+            }
+        }
+    }
+    (void)kept;
+}
+
 }  // namespace ptm

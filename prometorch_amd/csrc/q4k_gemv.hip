@@ -48,43 +48,20 @@ __device__ __forceinline__ void q4k_stage_x(const Q4KArgs& a, uint8_t* lds) {
         const int n16 = (K + K / 4) / 16;
         for (int i = tid; i < n16; i += Q4K_THREADS) dst[i] = src[i];
     } else {
-        const float4* x4 = reinterpret_cast<const float4*>(a.x);
-        float rs = 1.0f;
-        if constexpr (NORM) {
-            __shared__ float red[4];
-            float ss = 0.0f;
-            for (int i = tid; i < K / 4; i += Q4K_THREADS) {
-                const float4 v = x4[i];
-                ss = fmaf(v.x, v.x, ss);
-                ss = fmaf(v.y, v.y, ss);
-                ss = fmaf(v.z, v.z, ss);
-                ss = fmaf(v.w, v.w, ss);
-            }
-            ss = block_sum256(ss, red);
-            rs = 1.0f / sqrtf(ss / (float)K + a.eps);
-        }
+        __shared__ float red[4];
         int8_t* qs = reinterpret_cast<int8_t*>(lds);
         float* xd = reinterpret_cast<float*>(lds + K);
         float* xs = xd + K / 32;
-        // K/4 float4 slots, 8 consecutive slots = one Q8 block; K % 256 == 0 keeps lane groups whole
-        for (int i = tid; i < K / 4; i += Q4K_THREADS) {
-            float4 v = x4[i];
-            if constexpr (NORM) {
-                const float4 g = reinterpret_cast<const float4*>(a.gamma)[i];
-                const float one = a.add_one ? 1.0f : 0.0f;
-                v.x = v.x * rs * (g.x + one);
-                v.y = v.y * rs * (g.y + one);
-                v.z = v.z * rs * (g.z + one);
-                v.w = v.w * rs * (g.w + one);
-            }
-            float d, s;
-            const uint32_t packed = q8_quantize4(v, d, s);
+        // 8 consecutive float4 slots (8 lanes) = one Q8 block
+        stage_x_slots<NORM>(static_cast<const float*>(a.x), a.gamma, K, a.eps, a.add_one, red, [&](int i, float4 v) {
+            float d, sm;
+            const uint32_t packed = q8_quantize4(v, d, sm);
             reinterpret_cast<uint32_t*>(qs)[i] = packed;
             if ((tid & 7) == 0) {
                 xd[i >> 3] = d;
-                xs[i >> 3] = s;
+                xs[i >> 3] = sm;
             }
-        }
+        });
     }
     __syncthreads();
 }

@@ -108,36 +108,15 @@ __global__ __launch_bounds__(Q6K_THREADS) void q6k_gemv_kernel(const Q6KArgs a) 
         if (u < cnt0) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off);
 
     // stage x (optionally RMS-normalised) and its per-16 sums: 4 consecutive float4 slots make one 16-group
-    const float4* x4 = reinterpret_cast<const float4*>(a.x);
-    float rs = 1.0f;
-    if constexpr (NORM) {
+    {
         __shared__ float red[4];
-        float ss = 0.0f;
-        for (int i = tid; i < a.K / 4; i += Q6K_THREADS) {
-            const float4 v = x4[i];
-            ss = fmaf(v.x, v.x, ss);
-            ss = fmaf(v.y, v.y, ss);
-            ss = fmaf(v.z, v.z, ss);
-            ss = fmaf(v.w, v.w, ss);
-        }
-        ss = block_sum256(ss, red);
-        rs = 1.0f / sqrtf(ss / (float)a.K + a.eps);
-    }
-    for (int i = tid; i < a.K / 4; i += Q6K_THREADS) {
-        float4 v = x4[i];
-        if constexpr (NORM) {
-            const float4 g = reinterpret_cast<const float4*>(a.gamma)[i];
-            const float one = a.add_one ? 1.0f : 0.0f;
-            v.x = v.x * rs * (g.x + one);
-            v.y = v.y * rs * (g.y + one);
-            v.z = v.z * rs * (g.z + one);
-            v.w = v.w * rs * (g.w + one);
-        }
-        reinterpret_cast<float4*>(xf)[i] = v;
-        float s = (v.x + v.y) + (v.z + v.w);
-        s += dpp_f<0xB1>(s);
-        s += dpp_f<0x4E>(s);
-        if ((tid & 3) == 0) xsum16[i >> 2] = s;
+        stage_x_slots<NORM>(a.x, a.gamma, a.K, a.eps, a.add_one, red, [&](int i, float4 v) {
+            reinterpret_cast<float4*>(xf)[i] = v;
+            float sm = (v.x + v.y) + (v.z + v.w);
+            sm += dpp_f<0xB1>(sm);
+            sm += dpp_f<0x4E>(sm);
+            if ((tid & 3) == 0) xsum16[i >> 2] = sm;
+        });
     }
     __syncthreads();
 
