@@ -40,17 +40,25 @@ def log(*a):
 
 
 def event_time_ms(fn, iters, torch):
-    """Average duration of fn() over `iters` back-to-back launches, HIP events on the current stream."""
-    s = torch.cuda.current_stream()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for i in range(min(iters, 8)):
-        fn(i)
-    s.synchronize()
-    e0.record(s)
-    for i in range(iters):
-        fn(i)
-    e1.record(s)
-    s.synchronize()
+    """Average GPU duration of fn(i) over `iters` launches: the launches are captured into one graph
+    (so the host's per-call cost does not throttle them) and one replay is bracketed by HIP events
+    recorded on the stream the kernels run on."""
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        for i in range(4):
+            fn(i)  # first calls outside capture (one-time kernel attributes)
+        st.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            for i in range(iters):
+                fn(i)
+        g.replay()
+        st.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        g.replay()
+        e1.record(st)
+        st.synchronize()
     return e0.elapsed_time(e1) / iters
 
 

@@ -5,8 +5,8 @@
 // step feeds the argmax back as the next token, so consecutive tokens need no host round trip.
 //
 // Per layer (Q4_K_M mix: q/k/o/gate/up Q4_K, v/down Q6_K):
-//   RMSNorm + Q4_K {q,k} in one launch ; RMSNorm + Q6_K v in another (the norm is recomputed per
-//   workgroup; quant type is dispatched per tensor, as gemv_scratch does)
+//   RMSNorm + {q,k (Q4_K), v (Q6_K)} in one mixed launch (the norm is recomputed per workgroup; quant
+//   type is dispatched per tensor, as gemv_scratch does; other mixes fall back to one launch per type)
 //   QK-norm + NeoX RoPE + K/V append + split-KV attention in one launch, then the split merge
 //   o-proj GEMV accumulating into the residual
 //   rmsnorm + gate + up + SiLU*up in one launch
@@ -24,6 +24,9 @@ int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8
 int q6k_gemv_impl(const void* W, const float* x, float* y, int K, int N, int64_t stride, bool accumulate,
                   const float* gamma, float eps, int add_one, hipStream_t s);
 void q6k_init_attributes();
+int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const int* N4, int64_t stride4,
+                       const void* W6, float* y6, int N6, int64_t stride6, const float* x, const float* gamma,
+                       float eps, int add_one, int K, hipStream_t s);
 
 __global__ void set_scalars_kernel(int* d_token, int token, int64_t* d_past, int64_t past, int* d_step) {
     *d_token = token;
@@ -101,17 +104,23 @@ static int enqueue_step(ptm_decoder* d) {
             const ptm_qweight* w[3] = {&L.q, &L.k, &L.v};
             float* y[3] = {d->q, d->k, d->v};
             const void* W4[3]; float* y4[3]; int N4[3]; int n4 = 0;
+            int i6 = -1, n6 = 0;
             for (int i = 0; i < 3; ++i) {
-                if (w[i]->ggml_type == PTM_TYPE_Q4_K) {
-                    W4[n4] = w[i]->data; y4[n4] = y[i]; N4[n4] = w[i]->rows; ++n4;
-                } else {
-                    PTM_TRY(q6k_gemv_impl(w[i]->data, d->x, y[i], H, w[i]->rows, w[i]->row_stride_bytes, false,
-                                          L.attn_norm, c.rms_eps, 0, s));
-                }
+                if (w[i]->ggml_type == PTM_TYPE_Q4_K) { W4[n4] = w[i]->data; y4[n4] = y[i]; N4[n4] = w[i]->rows; ++n4; }
+                else { i6 = i; ++n6; }
             }
-            if (n4 > 0)
-                PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->x, false, L.attn_norm, c.rms_eps, 0, H,
-                                       (int64_t)(H / 256) * 144, false, s));
+            const int64_t s4 = (int64_t)(H / 256) * 144;
+            if (n6 == 1 && n4 >= 1 && H <= 16384) {
+                // the Q4_K_M mix (q, k in Q4_K; v in Q6_K): all three projections in one launch
+                PTM_TRY(rmsnorm_mixed_gemv(n4, W4, y4, N4, s4, w[i6]->data, y[i6], w[i6]->rows, w[i6]->row_stride_bytes,
+                                           d->x, L.attn_norm, c.rms_eps, 0, H, s));
+            } else {
+                for (int i = 0; i < 3; ++i)
+                    if (w[i]->ggml_type != PTM_TYPE_Q4_K)
+                        PTM_TRY(q6k_gemv_impl(w[i]->data, d->x, y[i], H, w[i]->rows, w[i]->row_stride_bytes, false,
+                                              L.attn_norm, c.rms_eps, 0, s));
+                if (n4 > 0) PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->x, false, L.attn_norm, c.rms_eps, 0, H, s4, false, s));
+            }
         }
         // QK-norm + RoPE + K/V append + split-KV attention in one launch, plus the small merge launch
         PTM_TRY(ptm_attn_decode_fused(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn, d->pO,

@@ -1,0 +1,54 @@
+// One launch for projections of the same activation vector that come in different quant types:
+// in a Q4_K_M file attn_q / attn_k are Q4_K while attn_v is Q6_K, so the reference issues three
+// GEMVs after one RMSNorm (torch/io/gguf_model.h:2750-2764).  Here workgroups [0, n6) run the
+// Q6_K body on the Q6_K matrix and the rest run the Q4_K body on up to three Q4_K matrices; each
+// workgroup recomputes the RMSNorm of x in its prologue, so no separate norm launch is needed.
+#include "q4k_body.h"
+#include "q6k_body.h"
+
+namespace ptm {
+
+__global__ __launch_bounds__(256) void rmsnorm_mixed_gemv_kernel(const Q4KArgs a4, const Q6KArgs a6, int n6_wgs) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    if ((int)blockIdx.x < n6_wgs) q6k_gemv_body<false, false, true>(a6, lds, blockIdx.x);
+    else q4k_gemv_body<false, true, false, 0>(a4, lds, (int)blockIdx.x - n6_wgs);
+}
+
+// y4[i] = W4[i] . norm(x) for the n4 Q4_K matrices (same K and stride), y6 = W6 . norm(x) (Q6_K, same K).
+int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const int* N4, int64_t stride4,
+                       const void* W6, float* y6, int N6, int64_t stride6, const float* x, const float* gamma,
+                       float eps, int add_one, int K, hipStream_t s) {
+    if (!x || !gamma || !W6 || !y6) return PTM_E_NULL;
+    if (n4 < 1 || n4 > 3 || K <= 0 || (K % 256) != 0 || N6 <= 0) return PTM_E_SHAPE;
+    if (K > 16384) return PTM_E_UNSUPPORTED;  // 64 KB of dynamic LDS without raising the cap
+    if (!aligned16(x) || !aligned16(gamma) || (stride4 & 15) || (stride6 & 1)) return PTM_E_ALIGN;
+    if (stride4 < (int64_t)(K / 256) * 144 || stride6 < (int64_t)(K / 256) * 210) return PTM_E_SHAPE;
+    Q4KArgs a4{};
+    int total = 0;
+    for (int i = 0; i < n4; ++i) {
+        if (!W4[i] || !y4[i]) return PTM_E_NULL;
+        if (N4[i] <= 0) return PTM_E_SHAPE;
+        if (!aligned16(W4[i])) return PTM_E_ALIGN;
+        a4.W[i] = static_cast<const uint8_t*>(W4[i]);
+        a4.y[i] = y4[i];
+        total += N4[i];
+        a4.row_end[i] = total;
+    }
+    a4.n_mat = n4;
+    a4.total_rows = total;
+    a4.K = K;
+    a4.stride = stride4;
+    a4.x = x;
+    a4.gamma = gamma;
+    a4.eps = eps;
+    a4.add_one = add_one;
+    a4.log2S = q4k_pick_log2S(total, K / 256, 3);
+    Q6KArgs a6{static_cast<const uint8_t*>(W6), x, y6, K, N6, q6k_pick_log2S(N6, K / 256), stride6, nullptr, nullptr,
+               gamma, eps, add_one};
+    const int n6 = q6k_workgroups(N6, K), n4w = q4k_workgroups(total, a4.log2S);
+    const size_t lds = (size_t)K * 4 + (size_t)K / 4;  // the Q6_K body's fp32 x + per-16 sums; Q4_K needs less
+    hipLaunchKernelGGL(rmsnorm_mixed_gemv_kernel, dim3(n6 + n4w), dim3(256), lds, s, a4, a6, n6);
+    return launch_status();
+}
+
+}  // namespace ptm

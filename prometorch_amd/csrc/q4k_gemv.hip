@@ -16,201 +16,20 @@
 // short-and-wide matrices (o-proj: 2560 rows) and so that each group's blocks are all in flight
 // at once.  The first pass of weight loads is issued BEFORE the activation vector is staged
 // (RMSNorm, Q8 quantisation, LDS), so HBM latency overlaps the prologue.
-#include "ptm_common.h"
+#include "q4k_body.h"
 
 namespace ptm {
 
-struct Q4KArgs {
-    const uint8_t* W[3];
-    float* y[3];
-    int row_end[3];  // cumulative row counts of the (up to 3) matrices
-    int n_mat;
-    int total_rows;  // MODE 1: 2*N interleaved (gate row r, up row r)
-    int K;
-    int log2S;       // lane groups per row = 1 << log2S
-    int64_t stride;
-    const void* x;       // fp32 x[K] (XQ8 == false) or Q8 blocks (XQ8 == true)
-    const float* gamma;  // RMSNorm weight (NORM)
-    float eps;
-    int add_one;
-};
-
-enum { Q4K_THREADS = 256, Q4K_U = 10 };
-
-// ---- prologue: bring the Q8 activation into LDS -------------------------------------------
-template <bool XQ8, bool NORM>
-__device__ __forceinline__ void q4k_stage_x(const Q4KArgs& a, uint8_t* lds) {
-    const int K = a.K;
-    const int tid = threadIdx.x;
-    if constexpr (XQ8) {
-        const uint4* src = reinterpret_cast<const uint4*>(a.x);
-        uint4* dst = reinterpret_cast<uint4*>(lds);
-        const int n16 = (K + K / 4) / 16;
-        for (int i = tid; i < n16; i += Q4K_THREADS) dst[i] = src[i];
-    } else {
-        __shared__ float red[4];
-        int8_t* qs = reinterpret_cast<int8_t*>(lds);
-        float* xd = reinterpret_cast<float*>(lds + K);
-        float* xs = xd + K / 32;
-        // 8 consecutive float4 slots (8 lanes) = one Q8 block
-        stage_x_slots<NORM>(static_cast<const float*>(a.x), a.gamma, K, a.eps, a.add_one, red, [&](int i, float4 v) {
-            float d, sm;
-            const uint32_t packed = q8_quantize4(v, d, sm);
-            reinterpret_cast<uint32_t*>(qs)[i] = packed;
-            if ((tid & 7) == 0) {
-                xd[i >> 3] = d;
-                xs[i >> 3] = sm;
-            }
-        });
-    }
-    __syncthreads();
-}
-
-// contribution of one super-block to lane j's chain (sub-block j of the block)
-__device__ __forceinline__ float q4k_block_term(const uint4 hdr, const uint4 qv, const uint8_t* __restrict__ lds,
-                                                int K, int b, int j) {
-    const int8_t* xq = reinterpret_cast<const int8_t*>(lds);
-    const float* xd = reinterpret_cast<const float*>(lds + K);
-    const float* xs = xd + K / 32;
-    const int half = j & 1;
-    const int xoff = (j >> 1) * 64 + half * 16;  // low-nibble activations; high-nibble ones are +32
-    const int4 xl = *reinterpret_cast<const int4*>(xq + b * 256 + xoff);
-    const int4 xh = *reinterpret_cast<const int4*>(xq + b * 256 + xoff + 32);
-    int lo = 0, hi = 0;
-    lo = __builtin_amdgcn_sdot4((int)(qv.x & 0x0f0f0f0fu), xl.x, lo, false);
-    lo = __builtin_amdgcn_sdot4((int)(qv.y & 0x0f0f0f0fu), xl.y, lo, false);
-    lo = __builtin_amdgcn_sdot4((int)(qv.z & 0x0f0f0f0fu), xl.z, lo, false);
-    lo = __builtin_amdgcn_sdot4((int)(qv.w & 0x0f0f0f0fu), xl.w, lo, false);
-    hi = __builtin_amdgcn_sdot4((int)((qv.x >> 4) & 0x0f0f0f0fu), xh.x, hi, false);
-    hi = __builtin_amdgcn_sdot4((int)((qv.y >> 4) & 0x0f0f0f0fu), xh.y, hi, false);
-    hi = __builtin_amdgcn_sdot4((int)((qv.z >> 4) & 0x0f0f0f0fu), xh.z, hi, false);
-    hi = __builtin_amdgcn_sdot4((int)((qv.w >> 4) & 0x0f0f0f0fu), xh.w, hi, false);
-    // even lane keeps the low-nibble half-dot and receives its partner's; odd lane the high one
-    const int keep = half ? hi : lo;
-    const int give = half ? lo : hi;
-    const int isum = keep + dpp_i<0xB1>(give);
-    int sc, mn;
-    q4k_scale_min(hdr.y, hdr.z, hdr.w, j, sc, mn);
-    const float d = h2f(hdr.x), dmin = h2f(hdr.x >> 16);
-    const float w = d * (float)sc * xd[b * 8 + j];
-    const float c = dmin * (float)mn * xs[b * 8 + j];
-    return fmaf(w, (float)isum, -c);
-}
-
-__device__ __forceinline__ float silu_mul_ref(float g, float u) {
-    // reference: gguf_model.h:3741-3755 (clamp, libm exp, 1/(1+e), g*sig, *u)
-    float ng = 0.0f - g;
-    ng = fminf(fmaxf(ng, -88.0f), 88.0f);
-    const float sig = 1.0f / (1.0f + expf(ng));
-    return (g * sig) * u;
-}
-
-// MODE 0: y = or += W.x for up to three matrices over a flattened row space
-// MODE 1: gate/up pair with SiLU over interleaved virtual rows (2r = gate row r, 2r+1 = up row r):
-//         y[0][r] = silu(Wg[r].x) * (Wu[r].x)
 template <bool XQ8, bool NORM, bool ACC, int MODE>
 __global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_kernel(const Q4KArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int j = lane & 7, grp = lane >> 3;
-    const int S = 1 << a.log2S;
-    const int sub = grp & (S - 1);
-    const int rows_per_wave = 8 >> a.log2S;
-    const int r = (blockIdx.x * 4 + wave) * rows_per_wave + (grp >> a.log2S);
-    const bool live = r < a.total_rows;
-    const int rr = live ? r : a.total_rows - 1;
-    const int nblk = a.K / 256;
-    const int nb_max = (nblk + S - 1) >> a.log2S;  // passes are sized for the group with the most blocks
-
-    int mat = 0, local = rr;
-    if constexpr (MODE == 1) {
-        mat = rr & 1;
-        local = rr >> 1;
-    } else {
-        if (a.n_mat > 1 && rr >= a.row_end[0]) { mat = 1; local = rr - a.row_end[0]; }
-        if (a.n_mat > 2 && rr >= a.row_end[1]) { mat = 2; local = rr - a.row_end[1]; }
-    }
-    const uint8_t* row = (mat == 0 ? a.W[0] : (mat == 1 ? a.W[1] : a.W[2])) + (int64_t)local * a.stride;
-
-    // ---- first pass of weight loads, issued before the activation prologue ----
-    uint4 hdr[Q4K_U], qv[Q4K_U];
-    const int cnt0 = min(Q4K_U, nb_max);
-#pragma unroll
-    for (int u = 0; u < Q4K_U; ++u) {
-        if (u < cnt0) {
-            const int b = min(sub + (u << a.log2S), nblk - 1);
-            const uint8_t* p = row + (int64_t)b * 144;
-            hdr[u] = *reinterpret_cast<const uint4*>(p);
-            qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
-        }
-    }
-
-    q4k_stage_x<XQ8, NORM>(a, lds);
-
-    float acc = 0.0f;
-    for (int i0 = 0; i0 < nb_max; i0 += Q4K_U) {
-        const int cnt = min(Q4K_U, nb_max - i0);
-        if (i0 > 0) {
-#pragma unroll
-            for (int u = 0; u < Q4K_U; ++u) {
-                if (u < cnt) {
-                    const int b = min(sub + ((i0 + u) << a.log2S), nblk - 1);
-                    const uint8_t* p = row + (int64_t)b * 144;
-                    hdr[u] = *reinterpret_cast<const uint4*>(p);
-                    qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < Q4K_U; ++u) {
-            if (u < cnt) {
-                const int b = sub + ((i0 + u) << a.log2S);
-                const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
-                acc += b < nblk ? t : 0.0f;
-            }
-        }
-    }
-    // reduce: 8 lanes of the group, then the S groups of the row
-    float p = sum8(acc);
-    if (S >= 2) p += dpp_f<0x128>(p);  // row_ror:8 = the other 8-lane half of the 16-lane row
-    if (S >= 4) p += __shfl_xor(p, 16, 64);
-    if (S >= 8) p += __shfl_xor(p, 32, 64);
-
-    if constexpr (MODE == 1) {
-        // gate and up of one row sit S groups apart
-        float other;
-        if (S == 1) other = dpp_f<0x128>(p);
-        else if (S == 2) other = __shfl_xor(p, 16, 64);
-        else other = __shfl_xor(p, 32, 64);
-        if (live && mat == 0 && sub == 0 && j == 0) a.y[0][local] = silu_mul_ref(p, other);
-    } else {
-        float* y = mat == 0 ? a.y[0] : (mat == 1 ? a.y[1] : a.y[2]);
-        if (live && sub == 0 && j == 0) {
-            if constexpr (ACC) y[local] += p;
-            else y[local] = p;
-        }
-    }
-}
-
-// lane groups per row: enough workgroups to cover the chip, and all of a group's blocks in one pass
-static int q4k_pick_log2S(int total_rows, int nblk, int max_log2S) {
-    int l = 0;
-    while (l < max_log2S) {
-        const int S = 1 << l;
-        const int wgs = (total_rows * S + 31) / 32;
-        const int nb = (nblk + S - 1) / S;
-        if (nb <= Q4K_U && wgs >= 600) break;
-        if (nb <= 1) break;
-        ++l;
-    }
-    return l;
+    q4k_gemv_body<XQ8, NORM, ACC, MODE>(a, lds, blockIdx.x);
 }
 
 template <bool XQ8, bool NORM, bool ACC, int MODE>
 static int q4k_launch(Q4KArgs& a, hipStream_t s) {
     a.log2S = q4k_pick_log2S(a.total_rows, a.K / 256, MODE == 1 ? 2 : 3);
-    const int rows_per_wg = 32 >> a.log2S;
-    const int grid = (a.total_rows + rows_per_wg - 1) / rows_per_wg;
+    const int grid = q4k_workgroups(a.total_rows, a.log2S);
     const size_t lds = (size_t)q8_bytes(a.K);
     hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
     return launch_status();

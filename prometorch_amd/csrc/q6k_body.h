@@ -1,0 +1,178 @@
+// Device code of the Q6_K dequant-fused GEMV (see q6k_gemv.hip for the design notes); kept in a
+// header so that a launch mixing Q4_K and Q6_K projections can call it per workgroup.
+#pragma once
+#include "ptm_common.h"
+
+namespace ptm {
+
+struct Q6KArgs {
+    const uint8_t* W;
+    const float* x;
+    float* y;        // may be NULL when only the argmax is wanted
+    int K, N;
+    int log2S;       // lane groups per row = 1 << log2S
+    int64_t stride;
+    float* part_val; // ARGMAX: per-workgroup best value / index
+    int* part_idx;
+    const float* gamma;  // NORM: RMSNorm weight applied to x while staging
+    float eps;
+    int add_one;
+};
+
+enum { Q6K_THREADS = 256, Q6K_U = 5 };
+
+__device__ __forceinline__ float dot4_u8(uint32_t q, float4 x, float acc) {
+    acc = fmaf((float)(q & 0xffu), x.x, acc);
+    acc = fmaf((float)((q >> 8) & 0xffu), x.y, acc);
+    acc = fmaf((float)((q >> 16) & 0xffu), x.z, acc);
+    acc = fmaf((float)(q >> 24), x.w, acc);
+    return acc;
+}
+
+struct Q6Blk { uint4 ql, qh, sc; uint32_t d; };
+
+__device__ __forceinline__ Q6Blk q6k_load(const uint8_t* __restrict__ p, int j, int qh_off) {
+    Q6Blk r;
+    r.ql = ld16_a2(p + 16 * j);
+    r.qh = ld16_a2(p + qh_off);
+    r.sc = ld16_a2(p + 192);
+    r.d = reinterpret_cast<const u16_a2*>(p + 208)->v;
+    return r;
+}
+
+// contribution of block b to lane j's chain
+__device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __restrict__ xf,
+                                                const float* __restrict__ xsum16, int b, int j) {
+    const int half = j >> 2, jj = j & 3, which32 = jj >> 1, l16 = jj & 1;
+    const int sc_lo_i = 8 * half + 2 * which32 + l16;  // scale of the low-nibble 16; high-nibble one is +4
+    const int hshift = 2 * which32;
+    const int xo = 128 * half + 32 * which32 + 16 * l16;  // x offset of the low-nibble 16; high-nibble +64
+    const float* xb = xf + b * 256 + xo;
+    float s_lo = 0.0f, s_hi = 0.0f;
+    const uint32_t qlw[4] = {k.ql.x, k.ql.y, k.ql.z, k.ql.w};
+    const uint32_t qhw[4] = {k.qh.x, k.qh.y, k.qh.z, k.qh.w};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t hs = qhw[w] >> hshift;
+        const uint32_t q_lo = (qlw[w] & 0x0f0f0f0fu) | ((hs << 4) & 0x30303030u);
+        const uint32_t q_hi = ((qlw[w] >> 4) & 0x0f0f0f0fu) | (hs & 0x30303030u);
+        const float4 x_lo = *reinterpret_cast<const float4*>(xb + 4 * w);
+        const float4 x_hi = *reinterpret_cast<const float4*>(xb + 64 + 4 * w);
+        s_lo = dot4_u8(q_lo, x_lo, s_lo);
+        s_hi = dot4_u8(q_hi, x_hi, s_hi);
+    }
+    const int xi = (b * 256 + xo) >> 4;
+    s_lo = fmaf(-32.0f, xsum16[xi], s_lo);
+    s_hi = fmaf(-32.0f, xsum16[xi + 4], s_hi);
+    const uint32_t scw[4] = {k.sc.x, k.sc.y, k.sc.z, k.sc.w};
+    const uint32_t w_lo = scw[sc_lo_i >> 2] >> (8 * (sc_lo_i & 3));
+    const uint32_t w_hi = scw[(sc_lo_i + 4) >> 2] >> (8 * (sc_lo_i & 3));
+    const float d = h2f(k.d);
+    const float f_lo = d * (float)(int)(int8_t)(w_lo & 0xffu);
+    const float f_hi = d * (float)(int)(int8_t)(w_hi & 0xffu);
+    return fmaf(f_hi, s_hi, f_lo * s_lo);
+}
+
+template <bool ACC, bool ARGMAX, bool NORM>
+__device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw, int wg) {
+    float* xf = reinterpret_cast<float*>(lds_raw);
+    float* xsum16 = xf + a.K;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6, j = lane & 7, grp = lane >> 3;
+    const int S = 1 << a.log2S;
+    const int sub = grp & (S - 1);
+    const int rows_per_wave = 8 >> a.log2S;
+    const int r = (wg * 4 + wave) * rows_per_wave + (grp >> a.log2S);
+    const bool live = r < a.N;
+    const int rr = live ? r : a.N - 1;
+    const int nblk = a.K / 256;
+    const int nb_max = (nblk + S - 1) >> a.log2S;
+    const uint8_t* row = a.W + (int64_t)rr * a.stride;
+    const int qh_off = 128 + 32 * (j >> 2) + 16 * (j & 1);
+
+    // first pass of weight loads, in flight while x is staged
+    Q6Blk blk[Q6K_U];
+    const int cnt0 = min(Q6K_U, nb_max);
+#pragma unroll
+    for (int u = 0; u < Q6K_U; ++u)
+        if (u < cnt0) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off);
+
+    // stage x (optionally RMS-normalised) and its per-16 sums: 4 consecutive float4 slots make one 16-group
+    {
+        __shared__ float red[4];
+        stage_x_slots<NORM>(a.x, a.gamma, a.K, a.eps, a.add_one, red, [&](int i, float4 v) {
+            reinterpret_cast<float4*>(xf)[i] = v;
+            float sm = (v.x + v.y) + (v.z + v.w);
+            sm += dpp_f<0xB1>(sm);
+            sm += dpp_f<0x4E>(sm);
+            if ((tid & 3) == 0) xsum16[i >> 2] = sm;
+        });
+    }
+    __syncthreads();
+
+    float acc = 0.0f;
+    for (int i0 = 0; i0 < nb_max; i0 += Q6K_U) {
+        const int cnt = min(Q6K_U, nb_max - i0);
+        if (i0 > 0) {
+#pragma unroll
+            for (int u = 0; u < Q6K_U; ++u)
+                if (u < cnt) blk[u] = q6k_load(row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 210, j, qh_off);
+        }
+#pragma unroll
+        for (int u = 0; u < Q6K_U; ++u) {
+            if (u < cnt) {
+                const int b = sub + ((i0 + u) << a.log2S);
+                const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
+                acc += b < nblk ? t : 0.0f;
+            }
+        }
+    }
+    float p = sum8(acc);
+    if (S >= 2) p += dpp_f<0x128>(p);
+    if (S >= 4) p += __shfl_xor(p, 16, 64);
+    if (S >= 8) p += __shfl_xor(p, 32, 64);
+    if (live && sub == 0 && j == 0 && a.y) {
+        if constexpr (ACC) a.y[rr] += p;
+        else a.y[rr] = p;
+    }
+    if constexpr (ARGMAX) {
+        // best (value, lowest index) of this workgroup's rows
+        __shared__ float bv[4];
+        __shared__ int bi[4];
+        float v = live ? p : -INFINITY;
+        int idx = rr;
+        for (int off = 8; off < 64; off <<= 1) {
+            const float ov = __shfl_xor(v, off, 64);
+            const int oi = __shfl_xor(idx, off, 64);
+            if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+        }
+        if (lane == 0) { bv[wave] = v; bi[wave] = idx; }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < 4; ++w)
+                if (bv[w] > v || (bv[w] == v && bi[w] < idx)) { v = bv[w]; idx = bi[w]; }
+            a.part_val[wg] = v;
+            a.part_idx[wg] = idx;
+        }
+    }
+}
+
+inline int q6k_pick_log2S(int rows, int nblk) {
+    int l = 0;
+    while (l < 3) {
+        const int S = 1 << l;
+        const int wgs = (rows * S + 31) / 32;
+        const int nb = (nblk + S - 1) / S;
+        if (nb <= Q6K_U && wgs >= 600) break;
+        if (nb <= 1) break;
+        ++l;
+    }
+    return l;
+}
+inline int q6k_workgroups(int N, int K) {
+    const int l = q6k_pick_log2S(N, K / 256);
+    const int rows_per_wg = 32 >> l;
+    return (N + rows_per_wg - 1) / rows_per_wg;
+}
+
+}  // namespace ptm
