@@ -290,6 +290,21 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     const int64_t col = (int64_t)kvh * HD + dl * 8;
     const bool owner = past >= t0 && past < t0 + FD_CHUNK;
 
+    // loads complete in issue order: the few q / norm-weight / rope values this wave needs go first,
+    // the chunk's K/V rows after them
+    const float* cs = a.rope + past * HD;
+    float qx0[(G + 3) / 4], qx1[(G + 3) / 4];
+#pragma unroll
+    for (int gi = 0; gi < (G + 3) / 4; ++gi) {
+        const int g = wave + 4 * gi;
+        const float* src = a.Q + (int64_t)(kvh * G + (g < G ? g : 0)) * HD;
+        qx0[gi] = lane < HALF ? src[lane] : 0.0f;
+        qx1[gi] = lane < HALF ? src[lane + HALF] : 0.0f;
+    }
+    float nw0 = 1.0f, nw1 = 1.0f;
+    if (a.qw && lane < HALF) { nw0 = a.qw[lane]; nw1 = a.qw[lane + HALF]; }
+    const float rc = lane < HALF ? cs[lane] : 1.0f, rsn = lane < HALF ? cs[HALF + lane] : 0.0f;
+
     // cached K/V rows of the chunk (the new position is not in the cache yet: clamp below it)
     float kreg[NPASS][8], vreg[NPASS][8];
     const int64_t last_cached = past > 0 ? past - 1 : 0;
@@ -302,11 +317,25 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     }
 
     // q heads of this kv group (wave w takes heads w, w+4, ...); owner: the new K row and V row
-    const float* cs = a.rope + past * HD;
-    for (int g = wave; g < G; g += 4) {
-        float r0, r1;
-        head_norm_rope<HD>(a.Q + (int64_t)(kvh * G + g) * HD, a.qw, cs, a.eps, a.add_one, lane, r0, r1);
-        if (lane < HALF) { s_q[g][lane] = r0; s_q[g][lane + HALF] = r1; }
+    const float one = a.add_one ? 1.0f : 0.0f;
+#pragma unroll
+    for (int gi = 0; gi < (G + 3) / 4; ++gi) {
+        const int g = wave + 4 * gi;
+        if (g < G) {
+            float x0 = qx0[gi], x1 = qx1[gi];
+            if (a.qw) {
+                float ss = fmaf(x0, x0, 0.0f);
+                ss = fmaf(x1, x1, ss);
+                ss = sum64(ss);
+                const float rs = 1.0f / sqrtf(ss / (float)HD + a.eps);
+                x0 = x0 * rs * (nw0 + one);
+                x1 = x1 * rs * (nw1 + one);
+            }
+            if (lane < HALF) {
+                s_q[g][lane] = fmaf(x0, rc, -(x1 * rsn));
+                s_q[g][lane + HALF] = fmaf(x0, rsn, x1 * rc);
+            }
+        }
     }
     if (owner) {
         const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;

@@ -166,27 +166,41 @@ __device__ __forceinline__ float4 norm4(float4 v, float4 g, float rs, float one)
     return v;
 }
 
-// Calls emit(i, value) for every float4 slot i of x (RMS-normalised with gamma when NORM), all 256
+// Staging is split in two so that a kernel can put its (few) activation loads in front of its (many)
+// weight loads: vector loads complete in issue order, so activation loads issued behind the weight
+// prefetch could only be consumed after every weight had arrived.
+//   XStage st = stage_issue<NORM>(x, gamma, K);      // loads of the first 4096 values (+ gamma)
+//   ... issue weight loads ...
+//   stage_finish<NORM>(st, x, gamma, K, eps, add_one, red, emit);
+// emit(i, value) is called for every float4 slot i of x (RMS-normalised with gamma when NORM), all 256
 // threads taking part; emit may use cross-lane ops (slots are handed out wave-uniformly: K % 256 == 0).
+struct XStage { XChunk x0, g0; };
+
+template <bool NORM>
+__device__ __forceinline__ XStage stage_issue(const float* __restrict__ x, const float* __restrict__ gamma, int K) {
+    XStage st;
+    st.x0 = load_chunk(reinterpret_cast<const float4*>(x), 0, K / 4);
+    if constexpr (NORM) st.g0 = load_chunk(reinterpret_cast<const float4*>(gamma), 0, K / 4);
+    return st;
+}
+
 template <bool NORM, typename Emit>
-__device__ __forceinline__ void stage_x_slots(const float* __restrict__ x, const float* __restrict__ gamma, int K,
-                                              float eps, int add_one, float* red4, Emit emit) {
+__device__ __forceinline__ void stage_finish(const XStage& st, const float* __restrict__ x,
+                                             const float* __restrict__ gamma, int K, float eps, int add_one,
+                                             float* red4, Emit emit) {
     const float4* x4 = reinterpret_cast<const float4*>(x);
     const float4* g4 = reinterpret_cast<const float4*>(gamma);
     const int n4 = K / 4;
-    const bool kept = n4 <= 1024;
     const float one = add_one ? 1.0f : 0.0f;
-    XChunk keep = load_chunk(x4, 0, n4), gk;
-    if constexpr (NORM) gk = load_chunk(g4, 0, n4);
     float rs = 1.0f;
     if constexpr (NORM) {
-        float ss = chunk_sumsq(keep, 0.0f);
+        float ss = chunk_sumsq(st.x0, 0.0f);
         for (int base = 1024; base < n4; base += 1024) ss = chunk_sumsq(load_chunk(x4, base, n4), ss);
         ss = block_sum256(ss, red4);
         rs = 1.0f / sqrtf(ss / (float)K + eps);
     }
     for (int base = 0; base < n4; base += 1024) {
-        XChunk c = keep, g = gk;
+        XChunk c = st.x0, g = st.g0;
         if (base > 0) {
             c = load_chunk(x4, base, n4);
             if constexpr (NORM) g = load_chunk(g4, base, n4);
@@ -201,7 +215,6 @@ __device__ __forceinline__ void stage_x_slots(const float* __restrict__ x, const
             }
         }
     }
-    (void)kept;
 }
 
 }  // namespace ptm

@@ -3,6 +3,8 @@
 #pragma once
 #include "ptm_common.h"
 
+#include <cstdlib>
+
 namespace ptm {
 
 struct Q4KArgs {
@@ -22,23 +24,48 @@ struct Q4KArgs {
 
 enum { Q4K_THREADS = 256, Q4K_U = 10 };
 
-// ---- prologue: bring the Q8 activation into LDS -------------------------------------------
+// ---- prologue: bring the Q8 activation into LDS; loads first (q4k_stage_issue), the rest after the
+// weight prefetch has been issued (q4k_stage_finish) --------------------------------------------------
+struct Q4KStage { XStage f; uint4 q8[2]; };
+
 template <bool XQ8, bool NORM>
-__device__ __forceinline__ void q4k_stage_x(const Q4KArgs a, uint8_t* lds) {
+__device__ __forceinline__ Q4KStage q4k_stage_issue(const Q4KArgs a) {
+    Q4KStage st;
+    if constexpr (XQ8) {
+        const uint4* src = reinterpret_cast<const uint4*>(a.x);
+        const int n16 = (a.K + a.K / 4) / 16;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int i = (int)threadIdx.x + Q4K_THREADS * u;
+            st.q8[u] = i < n16 ? src[i] : make_uint4(0, 0, 0, 0);
+        }
+    } else {
+        st.f = stage_issue<NORM>(static_cast<const float*>(a.x), a.gamma, a.K);
+    }
+    return st;
+}
+
+template <bool XQ8, bool NORM>
+__device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KArgs a, uint8_t* lds) {
     const int K = a.K;
     const int tid = threadIdx.x;
     if constexpr (XQ8) {
         const uint4* src = reinterpret_cast<const uint4*>(a.x);
         uint4* dst = reinterpret_cast<uint4*>(lds);
         const int n16 = (K + K / 4) / 16;
-        for (int i = tid; i < n16; i += Q4K_THREADS) dst[i] = src[i];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int i = tid + Q4K_THREADS * u;
+            if (i < n16) dst[i] = st.q8[u];
+        }
+        for (int i = tid + 2 * Q4K_THREADS; i < n16; i += Q4K_THREADS) dst[i] = src[i];
     } else {
         __shared__ float red[4];
         int8_t* qs = reinterpret_cast<int8_t*>(lds);
         float* xd = reinterpret_cast<float*>(lds + K);
         float* xs = xd + K / 32;
         // 8 consecutive float4 slots (8 lanes) = one Q8 block
-        stage_x_slots<NORM>(static_cast<const float*>(a.x), a.gamma, K, a.eps, a.add_one, red, [&](int i, float4 v) {
+        stage_finish<NORM>(st.f, static_cast<const float*>(a.x), a.gamma, K, a.eps, a.add_one, red, [&](int i, float4 v) {
             float d, sm;
             const uint32_t packed = q8_quantize4(v, d, sm);
             reinterpret_cast<uint32_t*>(qs)[i] = packed;
@@ -116,7 +143,8 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
     }
     const uint8_t* row = (mat == 0 ? a.W[0] : (mat == 1 ? a.W[1] : a.W[2])) + (int64_t)local * a.stride;
 
-    // ---- first pass of weight loads, issued before the activation prologue ----
+    // ---- activation loads first, then the first pass of weight loads, then the activation prologue ----
+    const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a);
     uint4 hdr[Q4K_U], qv[Q4K_U];
     const int cnt0 = min(Q4K_U, nb_max);
 #pragma unroll
@@ -129,7 +157,7 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
         }
     }
 
-    q4k_stage_x<XQ8, NORM>(a, lds);
+    q4k_stage_finish<XQ8, NORM>(stg, a, lds);
 
     float acc = 0.0f;
     for (int i0 = 0; i0 < nb_max; i0 += Q4K_U) {
@@ -177,7 +205,14 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
 }
 
 // lane groups per row: enough workgroups to cover the chip, and all of a group's blocks in one pass
+// PTM_Q4K_LOG2S / PTM_Q6K_LOG2S (0..3) override the heuristic, for tuning runs.
+inline int tuning_env(const char* name) {
+    const char* e = getenv(name);
+    return (e && e[0] >= '0' && e[0] <= '3' && e[1] == 0) ? e[0] - '0' : -1;
+}
 inline int q4k_pick_log2S(int total_rows, int nblk, int max_log2S) {
+    static const int forced = tuning_env("PTM_Q4K_LOG2S");
+    if (forced >= 0) return forced < max_log2S ? forced : max_log2S;
     int l = 0;
     while (l < max_log2S) {
         const int S = 1 << l;

@@ -3,6 +3,8 @@
 #pragma once
 #include "ptm_common.h"
 
+#include <cstdlib>
+
 namespace ptm {
 
 struct Q6KArgs {
@@ -90,7 +92,8 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
     const uint8_t* row = a.W + (int64_t)rr * a.stride;
     const int qh_off = 128 + 32 * (j >> 2) + 16 * (j & 1);
 
-    // first pass of weight loads, in flight while x is staged
+    // activation loads first (loads complete in issue order), then the first pass of weight loads
+    const XStage stg = stage_issue<NORM>(a.x, a.gamma, a.K);
     Q6Blk blk[Q6K_U];
     const int cnt0 = min(Q6K_U, nb_max);
 #pragma unroll
@@ -100,7 +103,7 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
     // stage x (optionally RMS-normalised) and its per-16 sums: 4 consecutive float4 slots make one 16-group
     {
         __shared__ float red[4];
-        stage_x_slots<NORM>(a.x, a.gamma, a.K, a.eps, a.add_one, red, [&](int i, float4 v) {
+        stage_finish<NORM>(stg, a.x, a.gamma, a.K, a.eps, a.add_one, red, [&](int i, float4 v) {
             reinterpret_cast<float4*>(xf)[i] = v;
             float sm = (v.x + v.y) + (v.z + v.w);
             sm += dpp_f<0xB1>(sm);
@@ -158,6 +161,11 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
 }
 
 inline int q6k_pick_log2S(int rows, int nblk) {
+    static const int forced = [] {
+        const char* e = getenv("PTM_Q6K_LOG2S");
+        return (e && e[0] >= '0' && e[0] <= '3' && e[1] == 0) ? e[0] - '0' : -1;
+    }();
+    if (forced >= 0) return forced;
     int l = 0;
     while (l < 3) {
         const int S = 1 << l;
