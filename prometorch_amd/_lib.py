@@ -8,7 +8,7 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libptm_hip.so")
+LIB_PATH = os.environ.get("PTM_LIB_PATH") or os.path.join(HERE, "libptm_hip.so")  # PTM_LIB_PATH: load another build
 
 vp, i64, i32, u32, f32 = C.c_void_p, C.c_int64, C.c_int, C.c_uint32, C.c_float
 

@@ -81,6 +81,9 @@ __device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KAr
 // contribution of one super-block to lane j's chain (sub-block j of the block)
 __device__ __forceinline__ float q4k_block_term(const uint4 hdr, const uint4 qv, const uint8_t* __restrict__ lds,
                                                 int K, int b, int j) {
+#if defined(PTM_EXP) && PTM_EXP == 1
+    return __int_as_float((hdr.x ^ qv.x ^ qv.y ^ qv.z ^ qv.w ^ hdr.y) & 0x3fffffff);
+#endif
     const int8_t* xq = reinterpret_cast<const int8_t*>(lds);
     const float* xd = reinterpret_cast<const float*>(lds + K);
     const float* xs = xd + K / 32;
