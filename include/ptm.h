@@ -192,12 +192,15 @@ int ptm_copy(const float* in, float* out, int64_t n, ptm_stream_t stream);
 
 /* ---- prefill: quantised-weight GEMM, Y[M,N] = X[M,K] . W[N,K]^T ------------------ */
 /* The reference has no quantised GEMM: matmul_q loops M single-row GEMVs
- * (gguf_model.h:7029-7036, :7056-7061).  These tile the weights through LDS once and use MFMA.
- * X is bf16 row-major [M][K]; Y fp32 row-major [M][N].
+ * (gguf_model.h:7029-7036, :7056-7061).  These read each weight tile once per 64 rows of X and
+ * use MFMA.  X is bf16 row-major [M][K] (16-byte aligned); Y fp32 row-major [M][N]; K % 256 == 0.
  * Q4_K: rows of X are quantised to Q8 blocks (same rule as ptm_quantize_q8, applied to the
- * bf16->fp32 values) and int8 MFMA computes the exact sub-block integer dots.
- * Q6_K: dequantised weights (exact in bf16x2 split) times bf16 X on bf16 MFMA, fp32 accumulate.
- * workspace: ptm_qgemm_workspace_bytes(M, K) device bytes. */
+ * bf16->fp32 values); int8 MFMA (K = 32 = one sub-block) gives the exact integer dots, scaled and
+ * accumulated in the GEMV's order, so every row equals ptm_q4k_gemv of that row bit for bit.
+ * Q6_K: (q - 32) as bf16 times bf16 X on bf16 MFMA (K = 16 = one scale group; products exact),
+ * each group sum scaled by d * scale in fp32.  Rows agree with ptm_q6k_gemv to fp32 rounding.
+ * workspace: ptm_qgemm_workspace_bytes(M, K) device bytes, 16-byte aligned (Q4_K only; Q6_K
+ * ignores it and accepts NULL). */
 int64_t ptm_qgemm_workspace_bytes(int M, int K);
 int ptm_qgemm_q4k(const void* W, const void* X_bf16, float* Y, int M, int K, int N,
                   int64_t row_stride_bytes, void* workspace, ptm_stream_t stream);
