@@ -30,6 +30,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the fused gate/up kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
+# script (KiB per dispatch: 13859.8 read, 38.0 written), reads scaled by 1.9998 = what FETCH_SIZE reports for
+# the 256 MiB copy this script also launches (profiles/decode_qwen3_4b_hbm_traffic_pmc.md).
+GATE_UP_TRAFFIC_BYTES = int((13859.8 * 1.9998 + 38.0) * 1024)
 SEED = 25
 N_PREFILL = 2048
 MAX_SEQ = 2304
@@ -146,7 +150,8 @@ def main():
     ms = event_time_ms(run_gate_up, 360, torch)
     roof = {"bound": "hbm", "kernel": "q4k_gemv_kernel<fused rmsnorm + gate/up + silu> 2x9728x2560",
             "achieved": gate_up_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": gate_up_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+            "frac": gate_up_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "traffic": GATE_UP_TRAFFIC_BYTES if args.layers == 36 else None,
             "bytes_per_launch": gate_up_bytes, "us_per_launch": ms * 1e3}
     log("gate/up fused: %.2f us/launch, %.0f GB/s" % (ms * 1e3, roof["achieved"]))
 
@@ -176,6 +181,24 @@ def main():
     b2 = H * strided + 4 * I + 4 * H
     ms2 = event_time_ms(lambda i: ops.launch_q6k_gemv(L0[i % nL].down.data, xa, yd, I, H, strided), 360, torch)
     gemv["q6k_down_2560x9728"] = {"bytes": b2, "us": ms2 * 1e3, "GBs": b2 / ms2 / 1e6, "frac": b2 / ms2 / 1e6 / HBM_PEAK_GBS}
+    # configs[4] (prefill): Q4_K GEMM on int8 MFMA, Llama-3-8B gate projection 14336x4096, 512 bf16 rows
+    Mq, Kq, Nq = 512, 4096, 14336
+    Wq = torch.from_numpy(synth.make_q4k(synth.rng_for(SEED, 5), Nq, Kq)).cuda()
+    Xq = torch.randn(Mq, Kq, device="cuda").to(torch.bfloat16)
+    Yq = torch.empty(Mq, Nq, device="cuda")
+    wsq = torch.empty(ops.qgemm_workspace_bytes(Mq, Kq), dtype=torch.uint8, device="cuda")
+    msq = event_time_ms(lambda i: ops.matmul_q(12, Wq, Xq, Yq, Mq, Kq, Nq, Kq // 256 * 144, wsq), 20, torch)
+    gemv["cfg4_q4k_prefill_gemm_512x4096x14336"] = {
+        "ops": 2.0 * Mq * Kq * Nq, "us": msq * 1e3, "TOPs": 2.0 * Mq * Kq * Nq / msq / 1e9,
+        "frac_int8_mfma_peak": 2.0 * Mq * Kq * Nq / msq / 1e9 / 5000.0}
+    del Wq, Xq, Yq, wsq
+    # plain copy of known size: the kernel the HBM byte counters are scaled by
+    ca = torch.empty(64 << 20, device="cuda")
+    cb = torch.empty(64 << 20, device="cuda")
+    msc = event_time_ms(lambda i: ops.launch_copy(ca, cb, ca.numel()), 4, torch)
+    gemv["copy_256MiB"] = {"bytes_read": ca.numel() * 4, "bytes_written": ca.numel() * 4, "us": msc * 1e3,
+                           "GBs": 2 * ca.numel() * 4 / msc / 1e6}
+    del ca, cb
     log(json.dumps(gemv))
     per_token_bytes = nL * 63866880 + V * stride6 + nL * 2 * (N_PREFILL + args.warmup + args.steps / 2) * 1024 * 2
     dec.close()
