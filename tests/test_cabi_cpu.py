@@ -33,6 +33,27 @@ def test_shim_header_names_exist_in_abi():
     assert used and used <= set(declared_symbols()), used - set(declared_symbols())
 
 
+def test_shim_header_compiles_as_host_cxx(tmp_path):
+    """Reference host code includes the shim in place of ATen/cuda/CUDAOps.h: it must be plain host C++."""
+    import shutil
+    import subprocess
+    if not (shutil.which("g++") and os.path.isdir("/opt/rocm/include")):
+        pytest.skip("no g++ / ROCm headers")
+    src = tmp_path / "uses_shim.cpp"
+    src.write_text(
+        '#include "ptm_at_cuda_shim.h"\n'
+        "void step(const void* w, const float* x, float* y, cudaStream_t s) {\n"
+        "    at::cuda::launch_q4km_persistent_gemv(w, x, y, 2560, 9728, 1440, s);\n"
+        "    at::cuda::launch_q6k_gemv(w, x, y, 2560, 1024, 2100);\n"
+        "    at::cuda::launch_rms_norm(x, x, y, 1, 2560, 1e-6f, false, s);\n"
+        "    at::cuda::launch_silu_mul(x, x, y, 9728, s);\n"
+        "}\n")
+    r = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-Werror", "-D__HIP_PLATFORM_AMD__",
+                        "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"), str(src)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
 def test_host_side_validation_codes():
     L = _lib.load()
     E_NULL, E_SHAPE, E_ALIGN, E_UNSUP = -1, -2, -3, -4
