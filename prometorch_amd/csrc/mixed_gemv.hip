@@ -8,10 +8,20 @@
 
 namespace ptm {
 
+template <int NB4, int NB6>
 __global__ __launch_bounds__(256) void rmsnorm_mixed_gemv_kernel(const Q4KArgs a4, const Q6KArgs a6, int n6_wgs) {
     extern __shared__ __align__(16) uint8_t lds[];
-    if ((int)blockIdx.x < n6_wgs) q6k_gemv_body<false, false, true>(a6, lds, blockIdx.x);
-    else q4k_gemv_body<false, true, false, 0>(a4, lds, (int)blockIdx.x - n6_wgs);
+    if ((int)blockIdx.x < n6_wgs) q6k_gemv_body<false, false, true, 1, NB6>(a6, lds, blockIdx.x);
+    else q4k_gemv_body<false, true, false, 0, NB4>(a4, lds, (int)blockIdx.x - n6_wgs);
+}
+
+template <int NB4>
+static void mixed_launch6(int nb6, dim3 grid, size_t lds, hipStream_t s, const Q4KArgs& a4, const Q6KArgs& a6, int n6) {
+    switch (nb6) {
+        case 2: hipLaunchKernelGGL((rmsnorm_mixed_gemv_kernel<NB4, 2>), grid, dim3(256), lds, s, a4, a6, n6); break;
+        case 3: hipLaunchKernelGGL((rmsnorm_mixed_gemv_kernel<NB4, 3>), grid, dim3(256), lds, s, a4, a6, n6); break;
+        default: hipLaunchKernelGGL((rmsnorm_mixed_gemv_kernel<NB4, 5>), grid, dim3(256), lds, s, a4, a6, n6); break;
+    }
 }
 
 // y4[i] = W4[i] . norm(x) for the n4 Q4_K matrices (same K and stride), y6 = W6 . norm(x) (Q6_K, same K).
@@ -47,7 +57,14 @@ int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const in
                gamma, eps, add_one};
     const int n6 = q6k_workgroups(N6, K), n4w = q4k_workgroups(total, a4.log2S);
     const size_t lds = (size_t)K * 4 + (size_t)K / 4;  // the Q6_K body's fp32 x + per-16 sums; Q4_K needs less
-    hipLaunchKernelGGL(rmsnorm_mixed_gemv_kernel, dim3(n6 + n4w), dim3(256), lds, s, a4, a6, n6);
+    const int nb6 = q6k_blocks_per_pass(N6, K);
+    const dim3 grid(n6 + n4w);
+    switch (q4k_blocks_per_pass(K / 256, a4.log2S)) {
+        case 2: mixed_launch6<2>(nb6, grid, lds, s, a4, a6, n6); break;
+        case 3: mixed_launch6<3>(nb6, grid, lds, s, a4, a6, n6); break;
+        case 5: mixed_launch6<5>(nb6, grid, lds, s, a4, a6, n6); break;
+        default: mixed_launch6<10>(nb6, grid, lds, s, a4, a6, n6); break;
+    }
     return launch_status();
 }
 

@@ -136,12 +136,25 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
 // sum-of-squares pass and the normalise pass.
 struct XChunk { float4 v[4]; };
 
-__device__ __forceinline__ XChunk load_chunk(const float4* __restrict__ p, int base, int n4) {
+// Activations are fetched with buffer loads: the hardware range check returns zeros for slots past the end of
+// the vector, so the load needs no predicate.  (A predicated global load is compiled to a branch around the
+// load; the compiler can then no longer count the loads in flight and waits for ALL of them, the weight
+// prefetch included, before the first use of x.)
+// Compiler-only fence: memory operations are neither moved nor scheduled across it.  Used to pin the ISSUE
+// order of loads (activations, then weights), which decides the order in which their data can be consumed.
+__device__ __forceinline__ void issue_order_fence() { asm volatile("" ::: "memory"); }
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ XChunk load_chunk(__amdgpu_buffer_rsrc_t rs, int base) {
     XChunk c;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int i = base + (int)threadIdx.x + 256 * u;
-        c.v[u] = i < n4 ? p[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, i * 16, 0, 0);
+        c.v[u] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
     }
     return c;
 }
@@ -169,52 +182,92 @@ __device__ __forceinline__ float4 norm4(float4 v, float4 g, float rs, float one)
 // Staging is split in two so that a kernel can put its (few) activation loads in front of its (many)
 // weight loads: vector loads complete in issue order, so activation loads issued behind the weight
 // prefetch could only be consumed after every weight had arrived.
-//   XStage st = stage_issue<NORM>(x, gamma, K);      // loads of the first 4096 values (+ gamma)
+//   XStage<NCH> st = stage_issue<NORM, NCH>(x, gamma, K, eps, add_one, red, emit);   // loads of the first NCH*4096 values
 //   ... issue weight loads ...
-//   stage_finish<NORM>(st, x, gamma, K, eps, add_one, red, emit);
+//   stage_finish<NORM, NCH>(st, K, eps, add_one, red, emit);
 // emit(i, value) is called for every float4 slot i of x (RMS-normalised with gamma when NORM), all 256
 // threads taking part; emit may use cross-lane ops (slots are handed out wave-uniformly: K % 256 == 0).
-struct XStage { XChunk x0, g0; };
+// Between the two calls only unconditional loads may be issued, and stage_finish issues none: the compiler
+// can then count the loads in flight and wait for exactly the activation loads.  Vectors longer than
+// NCH*4096 values take a slow path that stages the part beyond the register window first, inside stage_issue.
+template <int NCH = 1>
+struct XStage { XChunk x[NCH], g[NCH]; float rs; };
 
-template <bool NORM>
-__device__ __forceinline__ XStage stage_issue(const float* __restrict__ x, const float* __restrict__ gamma, int K) {
-    XStage st;
-    st.x0 = load_chunk(reinterpret_cast<const float4*>(x), 0, K / 4);
-    if constexpr (NORM) st.g0 = load_chunk(reinterpret_cast<const float4*>(gamma), 0, K / 4);
+template <bool NORM, typename Emit>
+__device__ __forceinline__ void emit_chunk(const XChunk& c, const XChunk& g, int base, int n4, float rs, float one,
+                                           Emit& emit) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int i = base + (int)threadIdx.x + 256 * u;
+        if (i < n4) {
+            float4 v = c.v[u];
+            if constexpr (NORM) v = norm4(v, g.v[u], rs, one);
+            emit(i, v);
+        }
+    }
+}
+
+template <bool NORM, int NCH = 1, typename Emit>
+__device__ __forceinline__ XStage<NCH> stage_issue(const float* __restrict__ x, const float* __restrict__ gamma, int K,
+                                                   float eps, int add_one, float* red4, Emit emit) {
+    const __amdgpu_buffer_rsrc_t x4 = make_rsrc(x, K * 4);
+    const __amdgpu_buffer_rsrc_t g4 = make_rsrc(NORM ? gamma : x, K * 4);
+    const int n4 = K / 4;
+    XStage<NCH> st;
+    st.rs = 1.0f;
+    // Slow path first, while no other load is in flight: the compiler cannot count loads across this loop and
+    // waits for everything outstanding where the paths join, which costs nothing here.
+    if (n4 > 1024 * NCH) {
+        if constexpr (NORM) {
+            float ss = 0.0f;
+            for (int base = 0; base < n4; base += 1024) ss = chunk_sumsq(load_chunk(x4, base), ss);
+            ss = block_sum256(ss, red4);
+            st.rs = 1.0f / sqrtf(ss / (float)K + eps);
+        }
+        for (int base = 1024 * NCH; base < n4; base += 1024) {
+            const XChunk c = load_chunk(x4, base);
+            XChunk g = c;
+            if constexpr (NORM) g = load_chunk(g4, base);
+            emit_chunk<NORM>(c, g, base, n4, st.rs, add_one ? 1.0f : 0.0f, emit);
+        }
+    }
+    issue_order_fence();  // keep the loads below from being hoisted above the slow path
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        st.x[c] = load_chunk(x4, 1024 * c);
+        if constexpr (NORM) st.g[c] = load_chunk(g4, 1024 * c);
+    }
     return st;
 }
 
-template <bool NORM, typename Emit>
-__device__ __forceinline__ void stage_finish(const XStage& st, const float* __restrict__ x,
-                                             const float* __restrict__ gamma, int K, float eps, int add_one,
-                                             float* red4, Emit emit) {
-    const float4* x4 = reinterpret_cast<const float4*>(x);
-    const float4* g4 = reinterpret_cast<const float4*>(gamma);
+template <bool NORM, int NCH = 1, typename Emit>
+__device__ __forceinline__ void stage_finish(const XStage<NCH>& st, int K, float eps, int add_one, float* red4,
+                                             Emit emit) {
     const int n4 = K / 4;
-    const float one = add_one ? 1.0f : 0.0f;
-    float rs = 1.0f;
+    float rs = st.rs;
     if constexpr (NORM) {
-        float ss = chunk_sumsq(st.x0, 0.0f);
-        for (int base = 1024; base < n4; base += 1024) ss = chunk_sumsq(load_chunk(x4, base, n4), ss);
-        ss = block_sum256(ss, red4);
-        rs = 1.0f / sqrtf(ss / (float)K + eps);
-    }
-    for (int base = 0; base < n4; base += 1024) {
-        XChunk c = st.x0, g = st.g0;
-        if (base > 0) {
-            c = load_chunk(x4, base, n4);
-            if constexpr (NORM) g = load_chunk(g4, base, n4);
-        }
+        if (n4 <= 1024 * NCH) {
+            float ss = 0.0f;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int i = base + (int)threadIdx.x + 256 * u;
-            if (i < n4) {
-                float4 v = c.v[u];
-                if constexpr (NORM) v = norm4(v, g.v[u], rs, one);
-                emit(i, v);
-            }
+            for (int c = 0; c < NCH; ++c) ss = chunk_sumsq(st.x[c], ss);
+            ss = block_sum256(ss, red4);
+            rs = 1.0f / sqrtf(ss / (float)K + eps);
         }
     }
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+        if (1024 * c < n4) emit_chunk<NORM>(st.x[c], st.g[c], 1024 * c, n4, rs, add_one ? 1.0f : 0.0f, emit);
+}
+
+// Blocks per pass for a lane group that owns nb_max blocks: the candidate (from a small set, so that the
+// number of kernel instances stays small) that wastes the fewest padded block slots; ties go to the larger.
+inline int pick_blocks_per_pass(int nb_max, const int* cand, int n_cand) {
+    int best = cand[0], best_waste = 1 << 30;
+    for (int i = 0; i < n_cand; ++i) {
+        const int waste = (nb_max + cand[i] - 1) / cand[i] * cand[i] - nb_max;
+        if (waste < best_waste || (waste == best_waste && cand[i] > best)) { best = cand[i]; best_waste = waste; }
+    }
+    return best;
 }
 
 }  // namespace ptm

@@ -24,56 +24,59 @@ struct Q4KArgs {
 
 enum { Q4K_THREADS = 256, Q4K_U = 10 };
 
-// ---- prologue: bring the Q8 activation into LDS; loads first (q4k_stage_issue), the rest after the
+// ---- prologue: bring the Q8 activation into LDS; loads first (q4k_stage_issue), the arithmetic after the
 // weight prefetch has been issued (q4k_stage_finish) --------------------------------------------------
-struct Q4KStage { XStage f; uint4 q8[2]; };
+struct Q4KStage { XStage<1> f; uint4 q8[2]; };
+
+// Q8 blocks of x go to LDS: 8 consecutive float4 slots (8 lanes) = one block
+struct Q4KEmit {
+    uint8_t* lds;
+    int K;
+    __device__ __forceinline__ void operator()(int i, float4 v) const {
+        float d, sm;
+        const uint32_t packed = q8_quantize4(v, d, sm);
+        reinterpret_cast<uint32_t*>(lds)[i] = packed;
+        if ((threadIdx.x & 7) == 0) {
+            float* xd = reinterpret_cast<float*>(lds + K);
+            xd[i >> 3] = d;
+            xd[K / 32 + (i >> 3)] = sm;
+        }
+    }
+};
 
 template <bool XQ8, bool NORM>
-__device__ __forceinline__ Q4KStage q4k_stage_issue(const Q4KArgs a) {
+__device__ __forceinline__ Q4KStage q4k_stage_issue(const Q4KArgs a, uint8_t* lds, float* red) {
     Q4KStage st;
     if constexpr (XQ8) {
         const uint4* src = reinterpret_cast<const uint4*>(a.x);
+        uint4* dst = reinterpret_cast<uint4*>(lds);
         const int n16 = (a.K + a.K / 4) / 16;
+        // beyond the register window (K > 6553): copied first, while no other load is in flight
+        for (int i = (int)threadIdx.x + 2 * Q4K_THREADS; i < n16; i += Q4K_THREADS) dst[i] = src[i];
+        issue_order_fence();  // keep the loads below from being hoisted above that loop
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int i = (int)threadIdx.x + Q4K_THREADS * u;
-            st.q8[u] = i < n16 ? src[i] : make_uint4(0, 0, 0, 0);
+            st.q8[u] = src[min(i, n16 - 1)];  // unconditional (clamped): keeps the load count static
         }
     } else {
-        st.f = stage_issue<NORM>(static_cast<const float*>(a.x), a.gamma, a.K);
+        st.f = stage_issue<NORM, 1>(static_cast<const float*>(a.x), a.gamma, a.K, a.eps, a.add_one, red, Q4KEmit{lds, a.K});
     }
     return st;
 }
 
 template <bool XQ8, bool NORM>
-__device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KArgs a, uint8_t* lds) {
-    const int K = a.K;
-    const int tid = threadIdx.x;
+__device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KArgs a, uint8_t* lds, float* red) {
     if constexpr (XQ8) {
-        const uint4* src = reinterpret_cast<const uint4*>(a.x);
         uint4* dst = reinterpret_cast<uint4*>(lds);
-        const int n16 = (K + K / 4) / 16;
+        const int n16 = (a.K + a.K / 4) / 16;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int i = tid + Q4K_THREADS * u;
+            const int i = (int)threadIdx.x + Q4K_THREADS * u;
             if (i < n16) dst[i] = st.q8[u];
         }
-        for (int i = tid + 2 * Q4K_THREADS; i < n16; i += Q4K_THREADS) dst[i] = src[i];
     } else {
-        __shared__ float red[4];
-        int8_t* qs = reinterpret_cast<int8_t*>(lds);
-        float* xd = reinterpret_cast<float*>(lds + K);
-        float* xs = xd + K / 32;
-        // 8 consecutive float4 slots (8 lanes) = one Q8 block
-        stage_finish<NORM>(st.f, static_cast<const float*>(a.x), a.gamma, K, a.eps, a.add_one, red, [&](int i, float4 v) {
-            float d, sm;
-            const uint32_t packed = q8_quantize4(v, d, sm);
-            reinterpret_cast<uint32_t*>(qs)[i] = packed;
-            if ((tid & 7) == 0) {
-                xd[i >> 3] = d;
-                xs[i >> 3] = sm;
-            }
-        });
+        stage_finish<NORM, 1>(st.f, a.K, a.eps, a.add_one, red, Q4KEmit{lds, a.K});
     }
     __syncthreads();
 }
@@ -123,7 +126,10 @@ __device__ __forceinline__ float silu_mul_ref(float g, float u) {
 // MODE 0: y = or += W.x for up to three matrices over a flattened row space
 // MODE 1: gate/up pair with SiLU over interleaved virtual rows (2r = gate row r, 2r+1 = up row r):
 //         y[0][r] = silu(Wg[r].x) * (Wu[r].x)
-template <bool XQ8, bool NORM, bool ACC, int MODE>
+// NB: super-blocks per lane group and pass; every pass issues exactly NB block loads, unconditionally (indices
+//     past the row's end are clamped, their terms dropped), so the count of loads in flight is static and a
+//     block is consumed as soon as it has arrived instead of after the whole prefetch.
+template <bool XQ8, bool NORM, bool ACC, int MODE, int NB>
 __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int wg) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 7, grp = lane >> 3;
@@ -147,42 +153,39 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
     const uint8_t* row = (mat == 0 ? a.W[0] : (mat == 1 ? a.W[1] : a.W[2])) + (int64_t)local * a.stride;
 
     // ---- activation loads first, then the first pass of weight loads, then the activation prologue ----
-    const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a);
-    uint4 hdr[Q4K_U], qv[Q4K_U];
-    const int cnt0 = min(Q4K_U, nb_max);
+    __shared__ float red[4];
+    const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a, lds, red);
+    uint4 hdr[NB], qv[NB];
+    issue_order_fence();
 #pragma unroll
-    for (int u = 0; u < Q4K_U; ++u) {
-        if (u < cnt0) {
-            const int b = min(sub + (u << a.log2S), nblk - 1);
-            const uint8_t* p = row + (int64_t)b * 144;
+    for (int u = 0; u < NB; ++u) {
+        const uint8_t* p = row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 144;
+        hdr[u] = *reinterpret_cast<const uint4*>(p);
+        qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+    }
+    issue_order_fence();
+
+    q4k_stage_finish<XQ8, NORM>(stg, a, lds, red);
+
+    float acc = 0.0f;
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        const int b = sub + (u << a.log2S);
+        const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
+        acc += b < nblk ? t : 0.0f;
+    }
+    for (int i0 = NB; i0 < nb_max; i0 += NB) {
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const uint8_t* p = row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 144;
             hdr[u] = *reinterpret_cast<const uint4*>(p);
             qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
         }
-    }
-
-    q4k_stage_finish<XQ8, NORM>(stg, a, lds);
-
-    float acc = 0.0f;
-    for (int i0 = 0; i0 < nb_max; i0 += Q4K_U) {
-        const int cnt = min(Q4K_U, nb_max - i0);
-        if (i0 > 0) {
 #pragma unroll
-            for (int u = 0; u < Q4K_U; ++u) {
-                if (u < cnt) {
-                    const int b = min(sub + ((i0 + u) << a.log2S), nblk - 1);
-                    const uint8_t* p = row + (int64_t)b * 144;
-                    hdr[u] = *reinterpret_cast<const uint4*>(p);
-                    qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < Q4K_U; ++u) {
-            if (u < cnt) {
-                const int b = sub + ((i0 + u) << a.log2S);
-                const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
-                acc += b < nblk ? t : 0.0f;
-            }
+        for (int u = 0; u < NB; ++u) {
+            const int b = sub + ((i0 + u) << a.log2S);
+            const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
+            acc += b < nblk ? t : 0.0f;
         }
     }
     // reduce: 8 lanes of the group, then the S groups of the row
@@ -230,6 +233,10 @@ inline int q4k_pick_log2S(int total_rows, int nblk, int max_log2S) {
 inline int q4k_workgroups(int total_rows, int log2S) {
     const int rows_per_wg = 32 >> log2S;
     return (total_rows + rows_per_wg - 1) / rows_per_wg;
+}
+inline int q4k_blocks_per_pass(int nblk, int log2S) {
+    static const int cand[] = {2, 3, 5, 10};
+    return pick_blocks_per_pass((nblk + (1 << log2S) - 1) >> log2S, cand, 4);
 }
 
 }  // namespace ptm

@@ -20,18 +20,23 @@
 
 namespace ptm {
 
-template <bool XQ8, bool NORM, bool ACC, int MODE>
+template <bool XQ8, bool NORM, bool ACC, int MODE, int NB>
 __global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_kernel(const Q4KArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
-    q4k_gemv_body<XQ8, NORM, ACC, MODE>(a, lds, blockIdx.x);
+    q4k_gemv_body<XQ8, NORM, ACC, MODE, NB>(a, lds, blockIdx.x);
 }
 
 template <bool XQ8, bool NORM, bool ACC, int MODE>
 static int q4k_launch(Q4KArgs& a, hipStream_t s) {
     a.log2S = q4k_pick_log2S(a.total_rows, a.K / 256, MODE == 1 ? 2 : 3);
-    const int grid = q4k_workgroups(a.total_rows, a.log2S);
+    const dim3 grid(q4k_workgroups(a.total_rows, a.log2S)), block(Q4K_THREADS);
     const size_t lds = (size_t)q8_bytes(a.K);
-    hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE>), dim3(grid), dim3(Q4K_THREADS), lds, s, a);
+    switch (q4k_blocks_per_pass(a.K / 256, a.log2S)) {
+        case 2: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 2>), grid, block, lds, s, a); break;
+        case 3: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 3>), grid, block, lds, s, a); break;
+        case 5: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 5>), grid, block, lds, s, a); break;
+        default: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 10>), grid, block, lds, s, a); break;
+    }
     return launch_status();
 }
 

@@ -75,7 +75,11 @@ __device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __r
     return fmaf(f_hi, s_hi, f_lo * s_lo);
 }
 
-template <bool ACC, bool ARGMAX, bool NORM>
+// XCH: chunks of 4096 activations whose loads go out before the weight prefetch (the rest trail it).
+// NB:  super-blocks per lane group and pass.  Every pass issues exactly NB block loads, unconditionally
+//      (block indices past the row's end are clamped and their terms dropped), so that the number of loads
+//      in flight is known at compile time and each block is consumed as soon as IT has arrived.
+template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
 __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw, int wg) {
     float* xf = reinterpret_cast<float*>(lds_raw);
     float* xsum16 = xf + a.K;
@@ -92,42 +96,41 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
     const uint8_t* row = a.W + (int64_t)rr * a.stride;
     const int qh_off = 128 + 32 * (j >> 2) + 16 * (j & 1);
 
+    // x (optionally RMS-normalised) goes to LDS with its per-16 sums: 4 consecutive float4 slots make one 16-group
+    __shared__ float red[4];
+    auto emit = [&](int i, float4 v) {
+        reinterpret_cast<float4*>(xf)[i] = v;
+        float sm = (v.x + v.y) + (v.z + v.w);
+        sm += dpp_f<0xB1>(sm);
+        sm += dpp_f<0x4E>(sm);
+        if ((tid & 3) == 0) xsum16[i >> 2] = sm;
+    };
     // activation loads first (loads complete in issue order), then the first pass of weight loads
-    const XStage stg = stage_issue<NORM>(a.x, a.gamma, a.K);
-    Q6Blk blk[Q6K_U];
-    const int cnt0 = min(Q6K_U, nb_max);
+    const XStage<XCH> stg = stage_issue<NORM, XCH>(a.x, a.gamma, a.K, a.eps, a.add_one, red, emit);
+    Q6Blk blk[NB];
+    issue_order_fence();
 #pragma unroll
-    for (int u = 0; u < Q6K_U; ++u)
-        if (u < cnt0) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off);
-
-    // stage x (optionally RMS-normalised) and its per-16 sums: 4 consecutive float4 slots make one 16-group
-    {
-        __shared__ float red[4];
-        stage_finish<NORM>(stg, a.x, a.gamma, a.K, a.eps, a.add_one, red, [&](int i, float4 v) {
-            reinterpret_cast<float4*>(xf)[i] = v;
-            float sm = (v.x + v.y) + (v.z + v.w);
-            sm += dpp_f<0xB1>(sm);
-            sm += dpp_f<0x4E>(sm);
-            if ((tid & 3) == 0) xsum16[i >> 2] = sm;
-        });
-    }
+    for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off);
+    issue_order_fence();
+    stage_finish<NORM, XCH>(stg, a.K, a.eps, a.add_one, red, emit);
     __syncthreads();
 
     float acc = 0.0f;
-    for (int i0 = 0; i0 < nb_max; i0 += Q6K_U) {
-        const int cnt = min(Q6K_U, nb_max - i0);
-        if (i0 > 0) {
 #pragma unroll
-            for (int u = 0; u < Q6K_U; ++u)
-                if (u < cnt) blk[u] = q6k_load(row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 210, j, qh_off);
-        }
+    for (int u = 0; u < NB; ++u) {
+        const int b = sub + (u << a.log2S);
+        const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
+        acc += b < nblk ? t : 0.0f;
+    }
+    for (int i0 = NB; i0 < nb_max; i0 += NB) {
 #pragma unroll
-        for (int u = 0; u < Q6K_U; ++u) {
-            if (u < cnt) {
-                const int b = sub + ((i0 + u) << a.log2S);
-                const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
-                acc += b < nblk ? t : 0.0f;
-            }
+        for (int u = 0; u < NB; ++u)
+            blk[u] = q6k_load(row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 210, j, qh_off);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int b = sub + ((i0 + u) << a.log2S);
+            const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
+            acc += b < nblk ? t : 0.0f;
         }
     }
     float p = sum8(acc);
@@ -181,6 +184,12 @@ inline int q6k_workgroups(int N, int K) {
     const int l = q6k_pick_log2S(N, K / 256);
     const int rows_per_wg = 32 >> l;
     return (N + rows_per_wg - 1) / rows_per_wg;
+}
+
+inline int q6k_blocks_per_pass(int N, int K) {
+    static const int cand[] = {2, 3, 5};
+    const int l = q6k_pick_log2S(N, K / 256);
+    return pick_blocks_per_pass((K / 256 + (1 << l) - 1) >> l, cand, 3);
 }
 
 }  // namespace ptm

@@ -14,10 +14,10 @@
 
 namespace ptm {
 
-template <bool ACC, bool ARGMAX, bool NORM>
+template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
 __global__ __launch_bounds__(Q6K_THREADS) void q6k_gemv_kernel(const Q6KArgs a) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
-    q6k_gemv_body<ACC, ARGMAX, NORM>(a, lds_raw, blockIdx.x);
+    q6k_gemv_body<ACC, ARGMAX, NORM, XCH, NB>(a, lds_raw, blockIdx.x);
 }
 
 __global__ __launch_bounds__(256) void argmax_partials_kernel(const float* pv, const int* pi, int n, int64_t* out) {
@@ -53,18 +53,45 @@ static int q6k_check(const void* W, const void* x, int K, int N, int64_t stride)
     return PTM_OK;
 }
 
-// Raise the dynamic-LDS cap of every variant once; must happen outside stream capture.
+template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
+static void q6k_raise_lds_cap() {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_kernel<ACC, ARGMAX, NORM, XCH, NB>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+}
+template <bool ACC, bool ARGMAX, bool NORM, int XCH>
+static void q6k_raise_lds_cap_nb() {
+    q6k_raise_lds_cap<ACC, ARGMAX, NORM, XCH, 2>();
+    q6k_raise_lds_cap<ACC, ARGMAX, NORM, XCH, 3>();
+    q6k_raise_lds_cap<ACC, ARGMAX, NORM, XCH, 5>();
+}
+// Raise the dynamic-LDS cap of every variant once (rows longer than 15K values need more than the default
+// 64 KB); must happen outside stream capture, so the decoder calls it when it is created.
 void q6k_init_attributes() {
     static bool done = false;
     if (done) return;
-    const void* fns[] = {
-        reinterpret_cast<const void*>(&q6k_gemv_kernel<false, false, false>),
-        reinterpret_cast<const void*>(&q6k_gemv_kernel<true, false, false>),
-        reinterpret_cast<const void*>(&q6k_gemv_kernel<false, true, false>),
-        reinterpret_cast<const void*>(&q6k_gemv_kernel<false, false, true>),
-    };
-    for (const void* f : fns) (void)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+    q6k_raise_lds_cap_nb<false, false, false, 1>();
+    q6k_raise_lds_cap_nb<true, false, false, 1>();
+    q6k_raise_lds_cap_nb<false, false, false, 3>();
+    q6k_raise_lds_cap_nb<true, false, false, 3>();
+    q6k_raise_lds_cap_nb<false, true, false, 1>();
+    q6k_raise_lds_cap_nb<false, false, true, 1>();
     done = true;
+}
+
+template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
+static int q6k_launch_nb(const Q6KArgs& a, int grid, size_t lds, hipStream_t s) {
+    if (lds > 64 * 1024) q6k_init_attributes();
+    hipLaunchKernelGGL((q6k_gemv_kernel<ACC, ARGMAX, NORM, XCH, NB>), dim3(grid), dim3(Q6K_THREADS), lds, s, a);
+    return launch_status();
+}
+
+template <bool ACC, bool ARGMAX, bool NORM, int XCH>
+static int q6k_launch_xch(const Q6KArgs& a, int grid, size_t lds, hipStream_t s) {
+    switch (q6k_blocks_per_pass(a.N, a.K)) {
+        case 2: return q6k_launch_nb<ACC, ARGMAX, NORM, XCH, 2>(a, grid, lds, s);
+        case 3: return q6k_launch_nb<ACC, ARGMAX, NORM, XCH, 3>(a, grid, lds, s);
+        default: return q6k_launch_nb<ACC, ARGMAX, NORM, XCH, 5>(a, grid, lds, s);
+    }
 }
 
 template <bool ACC, bool ARGMAX, bool NORM>
@@ -72,9 +99,11 @@ static int q6k_launch(Q6KArgs& a, hipStream_t s) {
     a.log2S = q6k_pick_log2S(a.N, a.K / 256);
     const int grid = q6k_workgroups(a.N, a.K);
     const size_t lds = (size_t)a.K * 4 + (size_t)a.K / 4;
-    if (lds > 64 * 1024) q6k_init_attributes();
-    hipLaunchKernelGGL((q6k_gemv_kernel<ACC, ARGMAX, NORM>), dim3(grid), dim3(Q6K_THREADS), lds, s, a);
-    return launch_status();
+    if constexpr (!ARGMAX && !NORM) {
+        // long rows (down projection): all of x is requested before the weights
+        if (a.K > 4096 && a.K <= 3 * 4096) return q6k_launch_xch<ACC, false, false, 3>(a, grid, lds, s);
+    }
+    return q6k_launch_xch<ACC, ARGMAX, NORM, 1>(a, grid, lds, s);
 }
 
 int q6k_gemv_impl(const void* W, const float* x, float* y, int K, int N, int64_t stride, bool accumulate,
