@@ -26,57 +26,133 @@ enum { Q4K_THREADS = 256, Q4K_U = 10 };
 
 // ---- prologue: bring the Q8 activation into LDS; loads first (q4k_stage_issue), the arithmetic after the
 // weight prefetch has been issued (q4k_stage_finish) --------------------------------------------------
-struct Q4KStage { XStage<1> f; uint4 q8[2]; };
+// fp32 x: thread t owns the 16 consecutive values [16t, 16t+16), i.e. half a Q8 block (lanes t, t^1 share a
+// block), so the two exact divisions of the Q8 rule are paid once per 16 values.  Every workgroup quantises the
+// whole vector, so this prologue is kept short: its instructions are issued by every wave of the launch.
+struct Q4KStage { float4 x[4], g[4]; float rs; u32x4 q8[2]; };
 
-// Q8 blocks of x go to LDS: 8 consecutive float4 slots (8 lanes) = one block
-struct Q4KEmit {
-    uint8_t* lds;
-    int K;
-    __device__ __forceinline__ void operator()(int i, float4 v) const {
-        float d, sm;
-        const uint32_t packed = q8_quantize4(v, d, sm);
-        reinterpret_cast<uint32_t*>(lds)[i] = packed;
-        if ((threadIdx.x & 7) == 0) {
-            float* xd = reinterpret_cast<float*>(lds + K);
-            xd[i >> 3] = d;
-            xd[K / 32 + (i >> 3)] = sm;
-        }
+__device__ __forceinline__ void q4k_load16(__amdgpu_buffer_rsrc_t r, int first, float4 (&v)[4]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(r, (first + 4 * u) * 4, 0, 0);  // zeros past the end
+        v[u] = make_float4(__uint_as_float(w.x), __uint_as_float(w.y), __uint_as_float(w.z), __uint_as_float(w.w));
     }
-};
+}
+__device__ __forceinline__ float q4k_sumsq16(const float4 (&v)[4], float ss) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        ss = fmaf(v[u].x, v[u].x, ss);
+        ss = fmaf(v[u].y, v[u].y, ss);
+        ss = fmaf(v[u].z, v[u].z, ss);
+        ss = fmaf(v[u].w, v[u].w, ss);
+    }
+    return ss;
+}
+// Q8 rule of quantize_x_q8 (reference: torch/io/cpu_quant_gemv.h:147-198) on the half block `unit` (16 values).
+template <bool NORM>
+__device__ __forceinline__ void q4k_quantize16_store(const float4 (&xv)[4], const float4 (&gv)[4], float rs, float one,
+                                                     int unit, uint8_t* lds, int K) {
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        float4 t = xv[u];
+        if constexpr (NORM) t = norm4(t, gv[u], rs, one);
+        v[4 * u] = t.x; v[4 * u + 1] = t.y; v[4 * u + 2] = t.z; v[4 * u + 3] = t.w;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    amax = fmaxf(amax, dpp_f<0xB1>(amax));
+    const float d = amax / 127.0f;
+    const float id = d > 0.0f ? 1.0f / d : 0.0f;
+    int isum = 0;
+    uint32_t w[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        uint32_t pk = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int q = max(-127, min(127, (int)rintf(v[4 * u + i] * id)));
+            isum += q;
+            pk |= (uint32_t)(q & 0xff) << (8 * i);
+        }
+        w[u] = pk;
+    }
+    isum += dpp_i<0xB1>(isum);
+    *reinterpret_cast<uint4*>(lds + 16 * unit) = make_uint4(w[0], w[1], w[2], w[3]);
+    if ((unit & 1) == 0) {
+        float* xd = reinterpret_cast<float*>(lds + K);
+        xd[unit >> 1] = d;
+        xd[K / 32 + (unit >> 1)] = d * (float)isum;
+    }
+}
 
 template <bool XQ8, bool NORM>
 __device__ __forceinline__ Q4KStage q4k_stage_issue(const Q4KArgs a, uint8_t* lds, float* red) {
     Q4KStage st;
+    const int tid = threadIdx.x;
+    st.rs = 1.0f;
     if constexpr (XQ8) {
         const uint4* src = reinterpret_cast<const uint4*>(a.x);
         uint4* dst = reinterpret_cast<uint4*>(lds);
         const int n16 = (a.K + a.K / 4) / 16;
         // beyond the register window (K > 6553): copied first, while no other load is in flight
-        for (int i = (int)threadIdx.x + 2 * Q4K_THREADS; i < n16; i += Q4K_THREADS) dst[i] = src[i];
+        for (int i = tid + 2 * Q4K_THREADS; i < n16; i += Q4K_THREADS) dst[i] = src[i];
         issue_order_fence();  // keep the loads below from being hoisted above that loop
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(a.x, n16 * 16);
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int i = (int)threadIdx.x + Q4K_THREADS * u;
-            st.q8[u] = src[min(i, n16 - 1)];  // unconditional (clamped): keeps the load count static
-        }
+        for (int u = 0; u < 2; ++u) st.q8[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (tid + Q4K_THREADS * u) * 16, 0, 0);
     } else {
-        st.f = stage_issue<NORM, 1>(static_cast<const float*>(a.x), a.gamma, a.K, a.eps, a.add_one, red, Q4KEmit{lds, a.K});
+        const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, a.K * 4);
+        const __amdgpu_buffer_rsrc_t rg = make_rsrc(NORM ? static_cast<const void*>(a.gamma) : a.x, a.K * 4);
+        const float one = a.add_one ? 1.0f : 0.0f;
+        // Slow path (K > 4096, beyond the 16 values per thread kept in registers) first, while no other load is in
+        // flight: the compiler cannot count loads across these loops and waits for everything where the paths join.
+        if (a.K > 16 * Q4K_THREADS) {
+            if constexpr (NORM) {
+                float ss = 0.0f;
+                for (int base = 0; base < a.K; base += 16 * Q4K_THREADS) {
+                    float4 t[4];
+                    q4k_load16(rx, base + 16 * tid, t);
+                    ss = q4k_sumsq16(t, ss);
+                }
+                ss = block_sum256(ss, red);
+                st.rs = 1.0f / sqrtf(ss / (float)a.K + a.eps);
+            }
+            for (int base = 16 * Q4K_THREADS; base < a.K; base += 16 * Q4K_THREADS) {
+                float4 t[4], g[4];
+                q4k_load16(rx, base + 16 * tid, t);
+                if constexpr (NORM) q4k_load16(rg, base + 16 * tid, g);
+                if (base + 16 * tid < a.K) q4k_quantize16_store<NORM>(t, g, st.rs, one, base / 16 + tid, lds, a.K);
+            }
+        }
+        issue_order_fence();
+        q4k_load16(rx, 16 * tid, st.x);
+        if constexpr (NORM) q4k_load16(rg, 16 * tid, st.g);
     }
     return st;
 }
 
 template <bool XQ8, bool NORM>
 __device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KArgs a, uint8_t* lds, float* red) {
+    const int tid = threadIdx.x;
     if constexpr (XQ8) {
         uint4* dst = reinterpret_cast<uint4*>(lds);
         const int n16 = (a.K + a.K / 4) / 16;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int i = (int)threadIdx.x + Q4K_THREADS * u;
-            if (i < n16) dst[i] = st.q8[u];
+            const int i = tid + Q4K_THREADS * u;
+            if (i < n16) dst[i] = make_uint4(st.q8[u].x, st.q8[u].y, st.q8[u].z, st.q8[u].w);
         }
     } else {
-        stage_finish<NORM, 1>(st.f, a.K, a.eps, a.add_one, red, Q4KEmit{lds, a.K});
+        float rs = st.rs;
+        if constexpr (NORM) {
+            if (a.K <= 16 * Q4K_THREADS) {
+                const float ss = block_sum256(q4k_sumsq16(st.x, 0.0f), red);
+                rs = 1.0f / sqrtf(ss / (float)a.K + a.eps);
+            }
+        }
+        if (16 * tid < a.K) q4k_quantize16_store<NORM>(st.x, st.g, rs, a.add_one ? 1.0f : 0.0f, tid, lds, a.K);
     }
     __syncthreads();
 }
@@ -84,7 +160,7 @@ __device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KAr
 // contribution of one super-block to lane j's chain (sub-block j of the block)
 __device__ __forceinline__ float q4k_block_term(const uint4 hdr, const uint4 qv, const uint8_t* __restrict__ lds,
                                                 int K, int b, int j) {
-#if defined(PTM_EXP) && PTM_EXP == 1
+#if defined(PTM_EXP) && (PTM_EXP == 1 || PTM_EXP == 3)
     return __int_as_float((hdr.x ^ qv.x ^ qv.y ^ qv.z ^ qv.w ^ hdr.y) & 0x3fffffff);
 #endif
     const int8_t* xq = reinterpret_cast<const int8_t*>(lds);
@@ -154,7 +230,11 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
 
     // ---- activation loads first, then the first pass of weight loads, then the activation prologue ----
     __shared__ float red[4];
+#if defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3)
+    Q4KStage stg;
+#else
     const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a, lds, red);
+#endif
     uint4 hdr[NB], qv[NB];
     issue_order_fence();
 #pragma unroll
@@ -164,8 +244,9 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
         qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
     }
     issue_order_fence();
-
+#if !(defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3))
     q4k_stage_finish<XQ8, NORM>(stg, a, lds, red);
+#endif
 
     float acc = 0.0f;
 #pragma unroll
