@@ -31,28 +31,53 @@ __device__ __forceinline__ float dot4_u8(uint32_t q, float4 x, float acc) {
     return acc;
 }
 
-struct Q6Blk { uint4 ql, qh, sc; uint32_t d; };
+// What one lane fetches of a block.  Blocks are 210 bytes, so every other block of a row starts 2 bytes off a
+// dword boundary, and 16-byte loads from such addresses run at a fraction of the aligned rate.  The ql / qh
+// pieces are therefore fetched as the dword-aligned 16 bytes at (address - mis), mis = 0 or 2, plus the
+// piece's last two bytes, and shifted into place with v_alignbyte.  The lane's two scales are fetched as single
+// signed bytes (no extraction arithmetic), d as a half word.
+struct Q6Blk { uint4 ql, qh; uint32_t ql_t, qh_t; int sc_lo, sc_hi; uint32_t d; uint32_t mis; };
 
-__device__ __forceinline__ Q6Blk q6k_load(const uint8_t* __restrict__ p, int j, int qh_off) {
+struct __attribute__((packed, aligned(4))) u128_a4 { uint32_t v[4]; };
+
+__device__ __forceinline__ Q6Blk q6k_load(const uint8_t* __restrict__ p, int j, int qh_off, int sc_off) {
     Q6Blk r;
-    r.ql = ld16_a2(p + 16 * j);
-    r.qh = ld16_a2(p + qh_off);
-    r.sc = ld16_a2(p + 192);
+    r.mis = (uint32_t)reinterpret_cast<uintptr_t>(p) & 2u;
+    const uint8_t* pa = p - r.mis;  // same dword as p, hence same page: never faults even at the first byte of an allocation
+    const u128_a4 l = *reinterpret_cast<const u128_a4*>(pa + 16 * j);
+    const u128_a4 h = *reinterpret_cast<const u128_a4*>(pa + qh_off);
+    r.ql = make_uint4(l.v[0], l.v[1], l.v[2], l.v[3]);
+    r.qh = make_uint4(h.v[0], h.v[1], h.v[2], h.v[3]);
+    r.ql_t = reinterpret_cast<const u16_a2*>(p + 16 * j + 14)->v;
+    r.qh_t = reinterpret_cast<const u16_a2*>(p + qh_off + 14)->v;
+    r.sc_lo = reinterpret_cast<const int8_t*>(p)[sc_off];
+    r.sc_hi = reinterpret_cast<const int8_t*>(p)[sc_off + 4];
     r.d = reinterpret_cast<const u16_a2*>(p + 208)->v;
     return r;
+}
+
+// the 16 bytes that start `mis` bytes into {w, tail}
+__device__ __forceinline__ void realign16(const uint4 w, uint32_t tail, uint32_t mis, uint32_t (&out)[4]) {
+    out[0] = __builtin_amdgcn_alignbyte(w.y, w.x, mis);
+    out[1] = __builtin_amdgcn_alignbyte(w.z, w.y, mis);
+    out[2] = __builtin_amdgcn_alignbyte(w.w, w.z, mis);
+    out[3] = __builtin_amdgcn_alignbyte(tail, w.w, mis);
 }
 
 // contribution of block b to lane j's chain
 __device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __restrict__ xf,
                                                 const float* __restrict__ xsum16, int b, int j) {
+#if defined(PTM_EXP) && (PTM_EXP == 1 || PTM_EXP == 3)
+    return __uint_as_float((k.ql.x ^ k.ql.y ^ k.ql.z ^ k.ql.w ^ k.qh.x ^ k.qh.y ^ k.qh.z ^ k.qh.w ^ k.sc_lo ^ k.sc_hi ^ k.d ^ k.ql_t ^ k.qh_t) & 0x3fffffffu);
+#endif
     const int half = j >> 2, jj = j & 3, which32 = jj >> 1, l16 = jj & 1;
-    const int sc_lo_i = 8 * half + 2 * which32 + l16;  // scale of the low-nibble 16; high-nibble one is +4
     const int hshift = 2 * which32;
     const int xo = 128 * half + 32 * which32 + 16 * l16;  // x offset of the low-nibble 16; high-nibble +64
     const float* xb = xf + b * 256 + xo;
     float s_lo = 0.0f, s_hi = 0.0f;
-    const uint32_t qlw[4] = {k.ql.x, k.ql.y, k.ql.z, k.ql.w};
-    const uint32_t qhw[4] = {k.qh.x, k.qh.y, k.qh.z, k.qh.w};
+    uint32_t qlw[4], qhw[4];
+    realign16(k.ql, k.ql_t, k.mis, qlw);
+    realign16(k.qh, k.qh_t, k.mis, qhw);
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
         const uint32_t hs = qhw[w] >> hshift;
@@ -66,12 +91,9 @@ __device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __r
     const int xi = (b * 256 + xo) >> 4;
     s_lo = fmaf(-32.0f, xsum16[xi], s_lo);
     s_hi = fmaf(-32.0f, xsum16[xi + 4], s_hi);
-    const uint32_t scw[4] = {k.sc.x, k.sc.y, k.sc.z, k.sc.w};
-    const uint32_t w_lo = scw[sc_lo_i >> 2] >> (8 * (sc_lo_i & 3));
-    const uint32_t w_hi = scw[(sc_lo_i + 4) >> 2] >> (8 * (sc_lo_i & 3));
     const float d = h2f(k.d);
-    const float f_lo = d * (float)(int)(int8_t)(w_lo & 0xffu);
-    const float f_hi = d * (float)(int)(int8_t)(w_hi & 0xffu);
+    const float f_lo = d * (float)k.sc_lo;  // scale of the low-nibble 16; the high-nibble one is 4 further
+    const float f_hi = d * (float)k.sc_hi;
     return fmaf(f_hi, s_hi, f_lo * s_lo);
 }
 
@@ -95,6 +117,7 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
     const int nb_max = (nblk + S - 1) >> a.log2S;
     const uint8_t* row = a.W + (int64_t)rr * a.stride;
     const int qh_off = 128 + 32 * (j >> 2) + 16 * (j & 1);
+    const int sc_off = 192 + 8 * (j >> 2) + 2 * ((j & 3) >> 1) + (j & 1);  // the lane's low-nibble scale
 
     // x (optionally RMS-normalised) goes to LDS with its per-16 sums: 4 consecutive float4 slots make one 16-group
     __shared__ float red[4];
@@ -106,13 +129,19 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
         if ((tid & 3) == 0) xsum16[i >> 2] = sm;
     };
     // activation loads first (loads complete in issue order), then the first pass of weight loads
+#if defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3 || PTM_EXP == 4 || PTM_EXP == 5)
+    XStage<XCH> stg;
+#else
     const XStage<XCH> stg = stage_issue<NORM, XCH>(a.x, a.gamma, a.K, a.eps, a.add_one, red, emit);
+#endif
     Q6Blk blk[NB];
     issue_order_fence();
 #pragma unroll
-    for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off);
+    for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off, sc_off);
     issue_order_fence();
+#if !(defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3 || PTM_EXP == 4 || PTM_EXP == 5))
     stage_finish<NORM, XCH>(stg, a.K, a.eps, a.add_one, red, emit);
+#endif
     __syncthreads();
 
     float acc = 0.0f;
@@ -125,7 +154,7 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
     for (int i0 = NB; i0 < nb_max; i0 += NB) {
 #pragma unroll
         for (int u = 0; u < NB; ++u)
-            blk[u] = q6k_load(row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 210, j, qh_off);
+            blk[u] = q6k_load(row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 210, j, qh_off, sc_off);
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
             const int b = sub + ((i0 + u) << a.log2S);
