@@ -270,13 +270,42 @@ __device__ __forceinline__ void head_norm_rope(const float* __restrict__ src, co
     r1 = fmaf(x0, s, x1 * c);
 }
 
+// Sum of N accumulators over the position slots of a wave (lanes with equal dl = lane % LPP), without LDS
+// traffic.  v_permlane32_swap exchanges lanes 32..63 of one register with lanes 0..31 of another, so ONE swap
+// and ONE add reduce TWO accumulators over the two wave halves (the first then lives in lanes 0..31, the second
+// in lanes 32..63); v_permlane16_swap does the same for odd/even rows of 16 lanes.  After both steps register k
+// of the result holds, in row r of the wave, the total of accumulator 4k + {0, 2, 1, 3}[r].
+template <int N, int LPP>
+__device__ __forceinline__ void reduce_position_slots(float (&acc)[N], float (&out)[N / 4]) {
+    static_assert(N % 4 == 0, "accumulator count must be a multiple of 4");
+    if constexpr (LPP == 8) {
+#pragma unroll
+        for (int k = 0; k < N; ++k) acc[k] += dpp_f<0x128>(acc[k]);  // row_ror:8 adds the other 8-lane half of the row
+    }
+    float half[N / 2];
+#pragma unroll
+    for (int k = 0; k < N / 2; ++k) {
+        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[2 * k]), __float_as_uint(acc[2 * k + 1]), false, false);
+        half[k] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+#pragma unroll
+    for (int k = 0; k < N / 4; ++k) {
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(half[2 * k]), __float_as_uint(half[2 * k + 1]), false, false);
+        out[k] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+}
+
+// Every wave works on its own 16 (HD 128) or 32 (HD 64) positions of the chunk from the loads to a wave-local
+// softmax partial (max, sum, weighted V); the four partials are merged through LDS behind the kernel's only
+// workgroup barrier.  Each wave prepares the q heads (and the new K/V row) itself: redundant arithmetic, but no
+// barrier and no idle waves on the path from "loads issued" to "partial written".
 template <bool KV16, int HD, int G>
 __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const AttnArgs a) {
     constexpr int LPP = HD / 8, PPW = 64 / LPP, PPB = PPW * 4, NPASS = FD_CHUNK / PPB, HALF = HD / 2;
-    __shared__ float s_q[G][HD];
-    __shared__ float s_p[G][FD_CHUNK];
+    __shared__ float s_q[4][G][HD];
+    __shared__ float s_new[4][2][HD];
     __shared__ float s_o[4][G][HD];
-    __shared__ float s_new[2][HD];
+    __shared__ float s_m[4][G], s_l[4][G];
 
     const int64_t past = *a.d_past;
     if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
@@ -289,23 +318,27 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     const int kv_dim = a.n_kv_heads * HD;
     const int64_t col = (int64_t)kvh * HD + dl * 8;
     const bool owner = past >= t0 && past < t0 + FD_CHUNK;
+    const bool on = lane < HALF;
+    const int lh = lane & (HALF - 1);
+    const bool has_norm = a.qw != nullptr;
 
-    // loads complete in issue order: the few q / norm-weight / rope values this wave needs go first,
-    // the chunk's K/V rows after them
+    // ---- loads, all unconditional so that their count is static: first the few values of the prologue ... ----
     const float* cs = a.rope + past * HD;
-    float qx0[(G + 3) / 4], qx1[(G + 3) / 4];
+    const float* qwp = has_norm ? a.qw : a.Q;  // a valid address either way; unused without norm weights
+    const float* kwp = has_norm ? a.kw : a.Q;
+    float qx0[G], qx1[G];
 #pragma unroll
-    for (int gi = 0; gi < (G + 3) / 4; ++gi) {
-        const int g = wave + 4 * gi;
-        const float* src = a.Q + (int64_t)(kvh * G + (g < G ? g : 0)) * HD;
-        qx0[gi] = lane < HALF ? src[lane] : 0.0f;
-        qx1[gi] = lane < HALF ? src[lane + HALF] : 0.0f;
+    for (int g = 0; g < G; ++g) {
+        const float* src = a.Q + (int64_t)(kvh * G + g) * HD;
+        qx0[g] = src[lh];
+        qx1[g] = src[lh + HALF];
     }
-    float nw0 = 1.0f, nw1 = 1.0f;
-    if (a.qw && lane < HALF) { nw0 = a.qw[lane]; nw1 = a.qw[lane + HALF]; }
-    const float rc = lane < HALF ? cs[lane] : 1.0f, rsn = lane < HALF ? cs[HALF + lane] : 0.0f;
-
-    // cached K/V rows of the chunk (the new position is not in the cache yet: clamp below it)
+    const float qn0 = qwp[lh], qn1 = qwp[lh + HALF], kn0 = kwp[lh], kn1 = kwp[lh + HALF];
+    const float rc = cs[lh], rsn = cs[HALF + lh];
+    float kx0 = a.K[(int64_t)kvh * HD + lh], kx1 = a.K[(int64_t)kvh * HD + lh + HALF];
+    float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
+    issue_order_fence();
+    // ---- ... then the cached K/V rows of this wave's positions (the new position is not cached: clamp below it) ----
     float kreg[NPASS][8], vreg[NPASS][8];
     const int64_t last_cached = past > 0 ? past - 1 : 0;
 #pragma unroll
@@ -315,77 +348,81 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
         load8<KV16>(a.Kc, tc * kv_dim + col, kreg[pass]);
         load8<KV16>(a.Vc, tc * kv_dim + col, vreg[pass]);
     }
+    issue_order_fence();
 
-    // q heads of this kv group (wave w takes heads w, w+4, ...); owner: the new K row and V row
+    // ---- per-head RMSNorm + NeoX rotation of the G query heads and of the new K row; V row as is ----
     const float one = a.add_one ? 1.0f : 0.0f;
 #pragma unroll
-    for (int gi = 0; gi < (G + 3) / 4; ++gi) {
-        const int g = wave + 4 * gi;
-        if (g < G) {
-            float x0 = qx0[gi], x1 = qx1[gi];
-            if (a.qw) {
-                float ss = fmaf(x0, x0, 0.0f);
-                ss = fmaf(x1, x1, ss);
-                ss = sum64(ss);
-                const float rs = 1.0f / sqrtf(ss / (float)HD + a.eps);
-                x0 = x0 * rs * (nw0 + one);
-                x1 = x1 * rs * (nw1 + one);
-            }
-            if (lane < HALF) {
-                s_q[g][lane] = fmaf(x0, rc, -(x1 * rsn));
-                s_q[g][lane + HALF] = fmaf(x0, rsn, x1 * rc);
-            }
+    for (int g = 0; g < G; ++g) {
+        float x0 = on ? qx0[g] : 0.0f, x1 = on ? qx1[g] : 0.0f;
+        if (has_norm) {
+            float ss = fmaf(x0, x0, 0.0f);
+            ss = fmaf(x1, x1, ss);
+            ss = sum64(ss);
+            const float rs = 1.0f / sqrtf(ss / (float)HD + a.eps);
+            x0 = x0 * rs * (qn0 + one);
+            x1 = x1 * rs * (qn1 + one);
+        }
+        if (on) {
+            s_q[wave][g][lane] = fmaf(x0, rc, -(x1 * rsn));
+            s_q[wave][g][lane + HALF] = fmaf(x0, rsn, x1 * rc);
         }
     }
-    if (owner) {
+    if (owner) {  // workgroup-uniform
+        float x0 = on ? kx0 : 0.0f, x1 = on ? kx1 : 0.0f;
+        if (has_norm) {
+            float ss = fmaf(x0, x0, 0.0f);
+            ss = fmaf(x1, x1, ss);
+            ss = sum64(ss);
+            const float rs = 1.0f / sqrtf(ss / (float)HD + a.eps);
+            x0 = x0 * rs * (kn0 + one);
+            x1 = x1 * rs * (kn1 + one);
+        }
+        float r0 = fmaf(x0, rc, -(x1 * rsn)), r1 = fmaf(x0, rsn, x1 * rc);
         const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;
-        if (wave == (G % 4)) {  // the wave with the fewest q heads
-            float r0, r1;
-            head_norm_rope<HD>(a.K + (int64_t)kvh * HD, a.kw, cs, a.eps, a.add_one, lane, r0, r1);
-            if (lane < HALF) {
-                if constexpr (KV16) {
-                    const __half h0 = __float2half_rn(r0), h1 = __float2half_rn(r1);
-                    static_cast<__half*>(a.Kc)[rowoff + lane] = h0;
-                    static_cast<__half*>(a.Kc)[rowoff + lane + HALF] = h1;
-                    r0 = __half2float(h0);
-                    r1 = __half2float(h1);
-                } else {
-                    static_cast<float*>(a.Kc)[rowoff + lane] = r0;
-                    static_cast<float*>(a.Kc)[rowoff + lane + HALF] = r1;
-                }
-                s_new[0][lane] = r0;
-                s_new[0][lane + HALF] = r1;
+        if constexpr (KV16) {
+            const __half h0 = __float2half_rn(r0), h1 = __float2half_rn(r1), g0 = __float2half_rn(vx0), g1 = __float2half_rn(vx1);
+            if (on && wave == 0) {
+                static_cast<__half*>(a.Kc)[rowoff + lane] = h0;
+                static_cast<__half*>(a.Kc)[rowoff + lane + HALF] = h1;
+                static_cast<__half*>(a.Vc)[rowoff + lane] = g0;
+                static_cast<__half*>(a.Vc)[rowoff + lane + HALF] = g1;
             }
-        } else if (wave == ((G + 1) % 4)) {
-            for (int i = lane; i < HD; i += 64) {
-                float v = a.V[(int64_t)kvh * HD + i];
-                if constexpr (KV16) {
-                    const __half hv = __float2half_rn(v);
-                    static_cast<__half*>(a.Vc)[rowoff + i] = hv;
-                    v = __half2float(hv);
-                } else {
-                    static_cast<float*>(a.Vc)[rowoff + i] = v;
-                }
-                s_new[1][i] = v;
+            r0 = __half2float(h0); r1 = __half2float(h1); vx0 = __half2float(g0); vx1 = __half2float(g1);
+        } else {
+            if (on && wave == 0) {
+                static_cast<float*>(a.Kc)[rowoff + lane] = r0;
+                static_cast<float*>(a.Kc)[rowoff + lane + HALF] = r1;
+                static_cast<float*>(a.Vc)[rowoff + lane] = vx0;
+                static_cast<float*>(a.Vc)[rowoff + lane + HALF] = vx1;
             }
         }
+        if (on) {
+            s_new[wave][0][lane] = r0;
+            s_new[wave][0][lane + HALF] = r1;
+            s_new[wave][1][lane] = vx0;
+            s_new[wave][1][lane + HALF] = vx1;
+        }
     }
-    __syncthreads();
+    // the values above are read back by other lanes of the SAME wave only
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
     float q[G][8];
 #pragma unroll
     for (int g = 0; g < G; ++g)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[g][i] = s_q[g][dl * 8 + i];
+        for (int i = 0; i < 8; ++i) q[g][i] = s_q[wave][g][dl * 8 + i];
 
-    // ---- scores ----
+    // ---- scores of this wave's positions; every lane of a position's lane group ends up with the score ----
+    float sc[G][NPASS];
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
-        const int tl = pass * PPB + wave * PPW + pl;
-        const int64_t t = t0 + tl;
+        const int64_t t = t0 + pass * PPB + wave * PPW + pl;
         if (t == past) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) { kreg[pass][i] = s_new[0][dl * 8 + i]; vreg[pass][i] = s_new[1][dl * 8 + i]; }
+            for (int i = 0; i < 8; ++i) { kreg[pass][i] = s_new[wave][0][dl * 8 + i]; vreg[pass][i] = s_new[wave][1][dl * 8 + i]; }
         }
         const bool valid = t < total;
         if (!valid) {  // rows past the end carry weight 0; keep 0 * garbage from producing NaN
@@ -398,59 +435,69 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
 #pragma unroll
             for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], kreg[pass][i], d);
             d = (LPP == 16) ? sum16(d) : sum8(d);
-            if (dl == 0) s_p[g][tl] = valid ? d * a.scale : -INFINITY;
+            sc[g][pass] = valid ? d * a.scale : -INFINITY;
         }
     }
-    __syncthreads();
-    for (int g = wave; g < G; g += 4) {
-        const float sc = s_p[g][lane];
-        const float m = max64(sc);
-        const float p = expf(sc - m);
-        const float l = sum64(p);
-        s_p[g][lane] = p;
+    // ---- wave-local softmax statistics and weighted V ----
+    float acc[G * 8];
+    float wm[G], wl[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float m = sc[g][0];
+#pragma unroll
+        for (int pass = 1; pass < NPASS; ++pass) m = fmaxf(m, sc[g][pass]);
+        for (int off = LPP; off < 64; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+        const float ms = m == -INFINITY ? 0.0f : m;  // a wave without valid positions contributes nothing
+        float l = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g * 8 + i] = 0.0f;
+#pragma unroll
+        for (int pass = 0; pass < NPASS; ++pass) {
+            const float p = expf(sc[g][pass] - ms);  // -inf -> 0
+            l += p;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g * 8 + i] = fmaf(p, vreg[pass][i], acc[g * 8 + i]);
+        }
+        for (int off = LPP; off < 64; off <<= 1) l += __shfl_xor(l, off, 64);
+        wm[g] = m;
+        wl[g] = l;
+    }
+    float red[G * 2];
+    reduce_position_slots<G * 8, LPP>(acc, red);
+    {
+        const int row = lane >> 4;                       // 16-lane row of the wave
+        const int sel = ((row & 1) << 1) | (row >> 1);   // {0, 2, 1, 3}[row]
+        if (LPP == 16 || (lane & 8) == 0) {
+#pragma unroll
+            for (int k = 0; k < G * 2; ++k) {
+                const int idx = 4 * k + sel;             // accumulator g*8 + i
+                s_o[wave][idx >> 3][dl * 8 + (idx & 7)] = red[k];
+            }
+        }
         if (lane == 0) {
-            const int64_t o = (int64_t)split * a.n_heads + kvh * G + g;
-            a.pM[o] = m;
-            a.pL[o] = l;
+#pragma unroll
+            for (int g = 0; g < G; ++g) { s_m[wave][g] = wm[g]; s_l[wave][g] = wl[g]; }
         }
     }
     __syncthreads();
-    float acc[G][8];
-#pragma unroll
-    for (int g = 0; g < G; ++g)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
-#pragma unroll
-    for (int pass = 0; pass < NPASS; ++pass) {
-        const int tl = pass * PPB + wave * PPW + pl;
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const float p = s_p[g][tl];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(p, vreg[pass][i], acc[g][i]);
-        }
-    }
-#pragma unroll
-    for (int g = 0; g < G; ++g)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float v = acc[g][i];
-            for (int off = LPP; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
-            acc[g][i] = v;
-        }
-    if (pl == 0) {
-#pragma unroll
-        for (int g = 0; g < G; ++g)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s_o[wave][g][dl * 8 + i] = acc[g][i];
-    }
-    __syncthreads();
+    // ---- merge the four wave partials into the chunk's partial ----
     for (int e = tid; e < G * HD; e += FD_THREADS) {
         const int g = e / HD, d = e % HD;
-        const float o = (s_o[0][g][d] + s_o[1][g][d]) + (s_o[2][g][d] + s_o[3][g][d]);
-        a.pO[((int64_t)split * a.n_heads + kvh * G + g) * HD + d] = o;
+        const float m0 = s_m[0][g], m1 = s_m[1][g], m2 = s_m[2][g], m3 = s_m[3][g];
+        const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));  // finite: the chunk holds at least one valid position
+        const float w0 = expf(m0 - M), w1 = expf(m1 - M), w2 = expf(m2 - M), w3 = expf(m3 - M);
+#if defined(PTM_EXP) && PTM_EXP == 7
+        const float o = ((w0 * s_o[0][g][d] + w1 * s_o[1][g][d]) + w2 * s_o[2][g][d]) + w3 * s_o[3][g][d];
+#else
+        const float o = (w0 * s_o[0][g][d] + w1 * s_o[1][g][d]) + (w2 * s_o[2][g][d] + w3 * s_o[3][g][d]);
+#endif
+        const int64_t oi = (int64_t)split * a.n_heads + kvh * G + g;
+        a.pO[oi * HD + d] = o;
+        if (d == 0) {
+            a.pM[oi] = M;
+            a.pL[oi] = (w0 * s_l[0][g] + w1 * s_l[1][g]) + (w2 * s_l[2][g] + w3 * s_l[3][g]);
+        }
     }
-
 }
 
 template <bool KV16, int HD>
