@@ -16,6 +16,12 @@ namespace ptm {
 
 enum { FD_CHUNK = 64, FD_THREADS = 256 };
 
+// e^x through the hardware base-2 exponential (v_exp_f32, 1 ulp): softmax weights need no more, and the libm
+// expf expands to a dozen instructions on a path whose cost is instruction count.  -inf gives 0.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+// 1/sqrt(x) through v_rsq_f32 (1 ulp) for the per-head RMS scale.
+__device__ __forceinline__ float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
+
 template <bool KV16>
 __device__ __forceinline__ void load8(const void* base, int64_t elem_off, float (&o)[8]) {
     if constexpr (KV16) {
@@ -345,8 +351,16 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     for (int pass = 0; pass < NPASS; ++pass) {
         const int64_t t = t0 + pass * PPB + wave * PPW + pl;
         const int64_t tc = t < past ? t : last_cached;
+#if defined(PTM_EXP) && PTM_EXP == 8
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { kreg[pass][i] = 0.01f * i; vreg[pass][i] = 0.02f * i; }
+#elif defined(PTM_EXP) && PTM_EXP == 9
+        load8<KV16>(a.Kc, ((int64_t)kvh * a.max_seq + tc) * HD + dl * 8, kreg[pass]);
+        load8<KV16>(a.Vc, ((int64_t)kvh * a.max_seq + tc) * HD + dl * 8, vreg[pass]);
+#else
         load8<KV16>(a.Kc, tc * kv_dim + col, kreg[pass]);
         load8<KV16>(a.Vc, tc * kv_dim + col, vreg[pass]);
+#endif
     }
     issue_order_fence();
 
@@ -359,7 +373,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
             float ss = fmaf(x0, x0, 0.0f);
             ss = fmaf(x1, x1, ss);
             ss = sum64(ss);
-            const float rs = 1.0f / sqrtf(ss / (float)HD + a.eps);
+            const float rs = fast_rsqrt(ss * (1.0f / (float)HD) + a.eps);
             x0 = x0 * rs * (qn0 + one);
             x1 = x1 * rs * (qn1 + one);
         }
@@ -374,7 +388,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
             float ss = fmaf(x0, x0, 0.0f);
             ss = fmaf(x1, x1, ss);
             ss = sum64(ss);
-            const float rs = 1.0f / sqrtf(ss / (float)HD + a.eps);
+            const float rs = fast_rsqrt(ss * (1.0f / (float)HD) + a.eps);
             x0 = x0 * rs * (kn0 + one);
             x1 = x1 * rs * (kn1 + one);
         }
@@ -453,7 +467,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
         for (int i = 0; i < 8; ++i) acc[g * 8 + i] = 0.0f;
 #pragma unroll
         for (int pass = 0; pass < NPASS; ++pass) {
-            const float p = expf(sc[g][pass] - ms);  // -inf -> 0
+            const float p = fast_exp(sc[g][pass] - ms);  // -inf -> 0
             l += p;
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[g * 8 + i] = fmaf(p, vreg[pass][i], acc[g * 8 + i]);
@@ -485,7 +499,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
         const int g = e / HD, d = e % HD;
         const float m0 = s_m[0][g], m1 = s_m[1][g], m2 = s_m[2][g], m3 = s_m[3][g];
         const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));  // finite: the chunk holds at least one valid position
-        const float w0 = expf(m0 - M), w1 = expf(m1 - M), w2 = expf(m2 - M), w3 = expf(m3 - M);
+        const float w0 = fast_exp(m0 - M), w1 = fast_exp(m1 - M), w2 = fast_exp(m2 - M), w3 = fast_exp(m3 - M);
 #if defined(PTM_EXP) && PTM_EXP == 7
         const float o = ((w0 * s_o[0][g][d] + w1 * s_o[1][g][d]) + w2 * s_o[2][g][d]) + w3 * s_o[3][g][d];
 #else
