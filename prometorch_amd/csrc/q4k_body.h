@@ -305,7 +305,7 @@ inline int q4k_pick_log2S(int total_rows, int nblk, int max_log2S) {
         const int S = 1 << l;
         const int wgs = (total_rows * S + 31) / 32;
         const int nb = (nblk + S - 1) / S;
-        if (nb <= Q4K_U && wgs >= 600) break;
+        if (nb <= 5 && wgs >= 600) break;  // 5 blocks in flight per group: measured better than 10 (registers -> occupancy)
         if (nb <= 1) break;
         ++l;
     }
