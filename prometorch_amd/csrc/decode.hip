@@ -24,6 +24,9 @@ int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8
 int q6k_gemv_impl(const void* W, const float* x, float* y, int K, int N, int64_t stride, bool accumulate,
                   const float* gamma, float eps, int add_one, hipStream_t s);
 void q6k_init_attributes();
+int q6k_gemv_argmax_impl(const void* W, const float* x, const float* gamma, float eps, int add_one, float* xn_out,
+                         float* logits, int K, int N, int64_t stride, int64_t* out_index, void* workspace,
+                         const ArgmaxAdvance adv, hipStream_t s);
 int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const int* N4, int64_t stride4,
                        const void* W6, float* y6, int N6, int64_t stride6, const float* x, const float* gamma,
                        float eps, int add_one, int K, hipStream_t s);
@@ -139,14 +142,15 @@ static int enqueue_step(ptm_decoder* d) {
         }
         PTM_TRY(gemv_any(L.down, d->act, d->x, true, s));  // x += Wdown . act
     }
-    PTM_TRY(ptm_rms_norm(d->x, c.out_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
     if (c.lm_head.ggml_type == PTM_TYPE_Q6_K) {
-        PTM_TRY(ptm_q6k_gemv_argmax(c.lm_head.data, d->xn, d->logits, H, c.vocab, c.lm_head.row_stride_bytes,
-                                    d->d_next, d->amax_ws, s));
-    } else {
-        PTM_TRY(gemv_any(c.lm_head, d->xn, d->logits, false, s));
-        PTM_TRY(ptm_argmax(d->logits, d->d_next, c.vocab, s));
+        // final RMSNorm in the lm_head prologue, step bookkeeping in the argmax tail: two launches for the whole tail
+        return q6k_gemv_argmax_impl(c.lm_head.data, d->x, c.out_norm, c.rms_eps, 0, d->xn, d->logits, H, c.vocab,
+                                    c.lm_head.row_stride_bytes, d->d_next, d->amax_ws,
+                                    ArgmaxAdvance{d->d_token, d->d_past, d->d_step, d->d_tokens, c.max_seq}, s);
     }
+    PTM_TRY(ptm_rms_norm(d->x, c.out_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+    PTM_TRY(gemv_any(c.lm_head, d->xn, d->logits, false, s));
+    PTM_TRY(ptm_argmax(d->logits, d->d_next, c.vocab, s));
     hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->d_next, d->d_token, d->d_past, d->d_step,
                        d->d_tokens, c.max_seq);
     return launch_status();

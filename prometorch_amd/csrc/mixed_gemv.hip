@@ -54,7 +54,7 @@ int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const in
     a4.add_one = add_one;
     a4.log2S = q4k_pick_log2S(total, K / 256, 3);
     Q6KArgs a6{static_cast<const uint8_t*>(W6), x, y6, K, N6, q6k_pick_log2S(N6, K / 256), stride6, nullptr, nullptr,
-               gamma, eps, add_one};
+               gamma, eps, add_one, nullptr};
     const int n6 = q6k_workgroups(N6, K), n4w = q4k_workgroups(total, a4.log2S);
     const size_t lds = (size_t)K * 4 + (size_t)K / 4;  // the Q6_K body's fp32 x + per-16 sums; Q4_K needs less
     const int nb6 = q6k_blocks_per_pass(N6, K);

@@ -21,6 +21,16 @@ inline int launch_status() { return hip_status(hipGetLastError()); }
 inline hipStream_t as_stream(ptm_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Bookkeeping of a decode step done by the thread that finishes the argmax (all NULL: plain argmax):
+// publish the token, feed it back as the next input, advance the position.
+struct ArgmaxAdvance {
+    int* d_token;
+    int64_t* d_past;
+    int* d_step;
+    int64_t* tokens_out;
+    int cap;
+};
+
 // ---- DPP lane exchanges (row = 16 lanes) ------------------------------------------------
 // quad_perm encodings: [1,0,3,2] = 0xB1 (xor 1), [2,3,0,1] = 0x4E (xor 2);
 // 0x141 = row_half_mirror (lane i <-> 7-i inside each 8), 0x140 = row_mirror (i <-> 15-i).

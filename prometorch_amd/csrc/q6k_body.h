@@ -19,6 +19,7 @@ struct Q6KArgs {
     const float* gamma;  // NORM: RMSNorm weight applied to x while staging
     float eps;
     int add_one;
+    float* xn_out;       // NORM: if not NULL, workgroup 0 also stores the normalised x[K] here
 };
 
 enum { Q6K_THREADS = 256, Q6K_U = 5 };
@@ -123,6 +124,9 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
     __shared__ float red[4];
     auto emit = [&](int i, float4 v) {
         reinterpret_cast<float4*>(xf)[i] = v;
+        if constexpr (NORM) {
+            if (wg == 0 && a.xn_out) reinterpret_cast<float4*>(a.xn_out)[i] = v;
+        }
         float sm = (v.x + v.y) + (v.z + v.w);
         sm += dpp_f<0xB1>(sm);
         sm += dpp_f<0x4E>(sm);

@@ -20,15 +20,32 @@ __global__ __launch_bounds__(Q6K_THREADS) void q6k_gemv_kernel(const Q6KArgs a) 
     q6k_gemv_body<ACC, ARGMAX, NORM, XCH, NB>(a, lds_raw, blockIdx.x);
 }
 
-__global__ __launch_bounds__(256) void argmax_partials_kernel(const float* pv, const int* pi, int n, int64_t* out) {
-    __shared__ float bv[4];
-    __shared__ int bi[4];
+// Final argmax over the per-workgroup (value, index) pairs: one workgroup of 1024 threads; every thread issues its
+// (up to 8 per round) loads before it compares, so a round costs one memory round trip.
+__global__ __launch_bounds__(1024) void argmax_partials_kernel(const float* pv, const int* pi, int n, int64_t* out,
+                                                               const ArgmaxAdvance adv) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    int step = 0;
+    int64_t past = 0;
+    if (threadIdx.x == 0 && adv.d_token) {  // fetched now so that the tail below does not wait on them
+        step = *adv.d_step;
+        past = *adv.d_past;
+    }
     float v = -INFINITY;
     int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += 256) {
-        const float ov = pv[i];
-        const int oi = pi[i];
-        if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    for (int base = 0; base < n; base += 8 * 1024) {
+        float tv[8];
+        int ti[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = min(base + (int)threadIdx.x + 1024 * u, n - 1);  // clamped: a repeated pair changes nothing
+            tv[u] = pv[i];
+            ti[u] = pi[i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (tv[u] > v || (tv[u] == v && ti[u] < idx)) { v = tv[u]; idx = ti[u]; }
     }
     for (int off = 1; off < 64; off <<= 1) {
         const float ov = __shfl_xor(v, off, 64);
@@ -38,9 +55,15 @@ __global__ __launch_bounds__(256) void argmax_partials_kernel(const float* pv, c
     if ((threadIdx.x & 63) == 0) { bv[threadIdx.x >> 6] = v; bi[threadIdx.x >> 6] = idx; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w)
+        for (int w = 1; w < 16; ++w)
             if (bv[w] > v || (bv[w] == v && bi[w] < idx)) { v = bv[w]; idx = bi[w]; }
         *out = (int64_t)idx;
+        if (adv.d_token) {
+            if (step < adv.cap) adv.tokens_out[step] = (int64_t)idx;
+            *adv.d_token = idx;
+            *adv.d_past = past + 1;
+            *adv.d_step = step + 1;
+        }
     }
 }
 
@@ -74,6 +97,7 @@ void q6k_init_attributes() {
     q6k_raise_lds_cap_nb<false, false, false, 3>();
     q6k_raise_lds_cap_nb<true, false, false, 3>();
     q6k_raise_lds_cap_nb<false, true, false, 1>();
+    q6k_raise_lds_cap_nb<false, true, true, 1>();
     q6k_raise_lds_cap_nb<false, false, true, 1>();
     done = true;
 }
@@ -111,13 +135,32 @@ int q6k_gemv_impl(const void* W, const float* x, float* y, int K, int N, int64_t
     const int rc = q6k_check(W, x, K, N, stride);
     if (rc != PTM_OK) return rc;
     if (!y) return PTM_E_NULL;
-    Q6KArgs a{static_cast<const uint8_t*>(W), x, y, K, N, 0, stride, nullptr, nullptr, gamma, eps, add_one};
+    Q6KArgs a{static_cast<const uint8_t*>(W), x, y, K, N, 0, stride, nullptr, nullptr, gamma, eps, add_one, nullptr};
     if (gamma) {
         if (accumulate) return PTM_E_UNSUPPORTED;
         if (!aligned16(gamma)) return PTM_E_ALIGN;
         return q6k_launch<false, false, true>(a, s);
     }
     return accumulate ? q6k_launch<true, false, false>(a, s) : q6k_launch<false, false, false>(a, s);
+}
+
+// lm_head of a decode step: optional RMSNorm of x in the prologue (gamma != NULL; the normalised vector is also
+// stored to xn_out by one workgroup), logits, their argmax, and optionally the step bookkeeping.
+int q6k_gemv_argmax_impl(const void* W, const float* x, const float* gamma, float eps, int add_one, float* xn_out,
+                         float* logits, int K, int N, int64_t stride, int64_t* out_index, void* workspace,
+                         const ArgmaxAdvance adv, hipStream_t s) {
+    const int rc = q6k_check(W, x, K, N, stride);
+    if (rc != PTM_OK) return rc;
+    if (!out_index || !workspace) return PTM_E_NULL;
+    if (gamma && !aligned16(gamma)) return PTM_E_ALIGN;
+    if (xn_out && !aligned16(xn_out)) return PTM_E_ALIGN;
+    const int grid = q6k_workgroups(N, K);
+    Q6KArgs a{static_cast<const uint8_t*>(W), x, logits, K, N, 0, stride, static_cast<float*>(workspace),
+              reinterpret_cast<int*>(static_cast<float*>(workspace) + grid), gamma, eps, add_one, xn_out};
+    const int rc2 = gamma ? q6k_launch<false, true, true>(a, s) : q6k_launch<false, true, false>(a, s);
+    if (rc2 != PTM_OK) return rc2;
+    hipLaunchKernelGGL(argmax_partials_kernel, dim3(1), dim3(1024), 0, s, a.part_val, a.part_idx, grid, out_index, adv);
+    return launch_status();
 }
 
 }  // namespace ptm
@@ -138,17 +181,8 @@ int64_t ptm_argmax_workspace_bytes(int N) {
 
 int ptm_q6k_gemv_argmax(const void* W, const float* x, float* logits, int K, int N, int64_t stride,
                         int64_t* out_index, void* workspace, ptm_stream_t stream) {
-    const int rc = q6k_check(W, x, K, N, stride);
-    if (rc != PTM_OK) return rc;
-    if (!out_index || !workspace) return PTM_E_NULL;
-    const int grid = q6k_workgroups(N, K);
-    Q6KArgs a{static_cast<const uint8_t*>(W), x, logits, K, N, 0, stride, static_cast<float*>(workspace),
-              reinterpret_cast<int*>(static_cast<float*>(workspace) + grid), nullptr, 0.f, 0};
-    const int rc2 = q6k_launch<false, true, false>(a, as_stream(stream));
-    if (rc2 != PTM_OK) return rc2;
-    hipLaunchKernelGGL(argmax_partials_kernel, dim3(1), dim3(256), 0, as_stream(stream), a.part_val, a.part_idx,
-                       grid, out_index);
-    return launch_status();
+    return q6k_gemv_argmax_impl(W, x, nullptr, 0.f, 0, nullptr, logits, K, N, stride, out_index, workspace,
+                                ArgmaxAdvance{nullptr, nullptr, nullptr, nullptr, 0}, as_stream(stream));
 }
 
 }  // extern "C"
