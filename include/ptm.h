@@ -206,6 +206,15 @@ int ptm_qgemm_q4k(const void* W, const void* X_bf16, float* Y, int M, int K, int
                   int64_t row_stride_bytes, void* workspace, ptm_stream_t stream);
 int ptm_qgemm_q6k(const void* W, const void* X_bf16, float* Y, int M, int K, int N,
                   int64_t row_stride_bytes, void* workspace, ptm_stream_t stream);
+/* Fast variant of the same product (Q4_K or Q6_K by ggml type id): rows of X are rounded to the
+ * reference's Q8 values (d*q per block of 32) and stored as fp16, weights are dequantised in
+ * registers and rounded to fp16, v_mfma_f32_32x32x16_f16 accumulates in fp32 over all of K.  Rows
+ * equal the reference GEMV up to the fp16 rounding of the operands (~1e-3 of rms(y) at most),
+ * inside the 1e-2 bar of the prefill path; use ptm_qgemm_q4k for bit-identical rows.
+ * workspace: ptm_qgemm_f16_workspace_bytes(M, K) device bytes, 16-byte aligned. */
+int64_t ptm_qgemm_f16_workspace_bytes(int M, int K);
+int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* Y, int M, int K, int N,
+                  int64_t row_stride_bytes, void* workspace, ptm_stream_t stream);
 
 /* ---- batch-1 decode runtime (GGUFModel::forward_decode, gguf_model.h:2575-3113) --- */
 typedef struct {

@@ -75,6 +75,8 @@ SIGNATURES = {
     "ptm_qgemm_workspace_bytes": (i64, [i32, i32]),
     "ptm_qgemm_q4k": (i32, [vp, vp, vp, i32, i32, i32, i64, vp, vp]),
     "ptm_qgemm_q6k": (i32, [vp, vp, vp, i32, i32, i32, i64, vp, vp]),
+    "ptm_qgemm_f16_workspace_bytes": (i64, [i32, i32]),
+    "ptm_qgemm_f16": (i32, [u32, vp, vp, vp, i32, i32, i32, i64, vp, vp]),
     "ptm_decode_create": (i32, [C.POINTER(DecodeConfig), C.POINTER(vp)]),
     "ptm_decode_destroy": (None, [vp]),
     "ptm_decode_set_past_len": (i32, [vp, i64]),

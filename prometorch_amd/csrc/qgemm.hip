@@ -259,6 +259,303 @@ __global__ __launch_bounds__(256) void qgemm_q6k_kernel(const uint8_t* __restric
             }
 }
 
+// =================================================================================================
+// Fast path: fp16 MFMA on dequantised weights.
+//   Activations: each row of X is rounded to the reference's Q8 values (d * q per block of 32, the rounding the
+//   CPU GEMV applies) and stored as fp16, scaled by a power of two per row so that it cannot overflow.
+//   Weights: dequantised in registers to their exact fp32 value, then rounded to fp16 (round toward zero, one
+//   instruction per pair).  v_mfma_f32_32x32x16_f16 accumulates in fp32 over the whole K, so there is NO per-sub-
+//   block epilogue: VALU work is the dequantisation only, and it is amortised over the 128 rows of X a workgroup
+//   owns.  Result = reference GEMV up to fp16 rounding of the operands (relative 2^-12 per element).
+//   Workgroup: 128 rows of X x 256 columns (wave w: columns 64w..64w+63 = two 32-wide MFMA tiles, all 128 rows =
+//   four 32-high tiles; 8 accumulator tiles = 128 VGPRs).  A 128 x 32 fp16 tile of X per sub-block step is shared
+//   through LDS (double-buffered); each wave dequantises only its own columns.
+//   The summation index of the MFMA is free to permute: lane half kh takes the 16 CONSECUTIVE elements
+//   [16 kh, 16 kh + 16) of a 32-wide sub-block (first 8 in k-step 0, next 8 in k-step 1), for A and B alike, so a
+//   lane's weights of one sub-block come from one 16-byte load.
+// =================================================================================================
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// LDS holds the fp16 X tile of a whole super-block step: 128 rows x 256 k, row pitch 528 B (16 consecutive lanes
+// x 16 B then hit all 64 banks once), double-buffered: 2 x 66 KB of the CU's 160 KB.
+enum { QF_TM = 128, QF_TN = 256, QF_PITCH = 528 };
+
+__host__ __device__ inline int qf_mpad(int M) { return (M + QF_TM - 1) / QF_TM * QF_TM; }
+
+// rows of X (bf16) -> fp16 rows Xh[Mpad][K] (Q8ROUND: first rounded to the reference's Q8 values d*q per block of
+// 32, the rounding its Q4_K GEMV applies; otherwise the bf16 value itself, as its Q6_K GEMV uses), divided by a
+// power of two per row (returned in rowscale) so that fp16 cannot overflow
+template <bool Q8ROUND>
+__global__ __launch_bounds__(256) void qgemm_prepare_rows_f16_kernel(const uint16_t* __restrict__ X, _Float16* __restrict__ Xh,
+                                                                     float* __restrict__ rowscale, int M, int K) {
+    __shared__ float red[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const int n4 = K / 4;
+    _Float16* dst = Xh + (int64_t)m * K;
+    if (m >= M) {  // padding rows: zeros
+        for (int i = tid; i < n4; i += 256) reinterpret_cast<uint2*>(dst)[i] = make_uint2(0, 0);
+        return;
+    }
+    const uint2* src = reinterpret_cast<const uint2*>(X + (int64_t)m * K);
+    float amax = 0.0f;
+    for (int i = tid; i < n4; i += 256) {
+        const uint2 raw = src[i];
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(bf16_to_f32(raw.x & 0xffffu)), fabsf(bf16_to_f32(raw.x >> 16))),
+                                 fmaxf(fabsf(bf16_to_f32(raw.y & 0xffffu)), fabsf(bf16_to_f32(raw.y >> 16)))));
+    }
+    amax = max64(amax);
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    // power of two that brings the row below 2^14 (fp16 tops out at 65504); 1 for ordinary activations
+    int e = 0;
+    if (amax > 16384.0f) { (void)frexpf(amax, &e); e -= 14; }
+    const float down = ldexpf(1.0f, -e);
+    if (tid == 0) rowscale[m] = ldexpf(1.0f, e);
+    for (int i = tid; i < n4; i += 256) {  // K % 256 == 0: whole waves, aligned groups of 8 lanes = one Q8 block
+        const uint2 raw = src[i];
+        float4 v;
+        v.x = bf16_to_f32(raw.x & 0xffffu);
+        v.y = bf16_to_f32(raw.x >> 16);
+        v.z = bf16_to_f32(raw.y & 0xffffu);
+        v.w = bf16_to_f32(raw.y >> 16);
+        if constexpr (Q8ROUND) {
+            float d, sm;
+            const uint32_t pk = q8_quantize4(v, d, sm);
+            v.x = d * (float)(int)(int8_t)(pk & 0xff);
+            v.y = d * (float)(int)(int8_t)((pk >> 8) & 0xff);
+            v.z = d * (float)(int)(int8_t)((pk >> 16) & 0xff);
+            v.w = d * (float)(int)(int8_t)(pk >> 24);
+        }
+        union { _Float16 h[4]; uint2 u; } o;
+        o.h[0] = (_Float16)(v.x * down);  // power-of-two scaling: exact
+        o.h[1] = (_Float16)(v.y * down);
+        o.h[2] = (_Float16)(v.z * down);
+        o.h[3] = (_Float16)(v.w * down);
+        reinterpret_cast<uint2*>(dst)[i] = o.u;
+    }
+}
+
+// 16 small integers (4 dwords of bytes, each < 1024) -> two fragments of 8 fp16 holding (byte - bias) * scale + offset.
+// A byte b becomes the fp16 number 1024 + b by writing it under the exponent byte 0x64 (one v_perm per pair); the
+// subtraction of 1024 + bias is exact, and one packed fp16 FMA applies scale and offset: 2.5 instructions per pair.
+__device__ __forceinline__ void bytes_to_frags(const uint32_t (&b)[4], float bias, float scale, float offset, h8& f0, h8& f1) {
+    const h2 sub = {(_Float16)(1024.0f + bias), (_Float16)(1024.0f + bias)};
+    const h2 sc = {(_Float16)scale, (_Float16)scale};
+    const h2 of = {(_Float16)offset, (_Float16)offset};
+    uint32_t o[8];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const uint32_t hq = __builtin_amdgcn_perm(0x64646464u, b[w], p ? 0x04030402u : 0x04010400u);
+            h2 q;
+            __builtin_memcpy(&q, &hq, 4);
+            const h2 v = __builtin_elementwise_fma(q - sub, sc, of);
+            __builtin_memcpy(&o[2 * w + p], &v, 4);
+        }
+    }
+    __builtin_memcpy(&f0, &o[0], 16);
+    __builtin_memcpy(&f1, &o[4], 16);
+}
+
+// ---- per-type weight access: what a lane (column n, element half kh) fetches of a 256-wide super-block ----
+struct Q4Tile {  // Q4_K: header + the lane's 16 bytes of each of the 4 groups of 64
+    uint4 hdr;
+    uint4 qs[4];
+    __device__ __forceinline__ void load(const uint8_t* blk, int kh) {
+        hdr = *reinterpret_cast<const uint4*>(blk);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) qs[g] = *reinterpret_cast<const uint4*>(blk + 16 + 32 * g + 16 * kh);
+    }
+    // sub-block s (0..7) of the block -> two fragments
+    __device__ __forceinline__ void frags(int s, int /*kh*/, h8& f0, h8& f1) const {
+        int sc, mn;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, s, sc, mn);
+        const float dsc = h2f(hdr.x) * (float)sc, dmn = h2f(hdr.x >> 16) * (float)mn;
+        const uint4 r = qs[s >> 1];
+        const int sh = 4 * (s & 1);
+        const uint32_t b[4] = {(r.x >> sh) & 0x0f0f0f0fu, (r.y >> sh) & 0x0f0f0f0fu, (r.z >> sh) & 0x0f0f0f0fu,
+                               (r.w >> sh) & 0x0f0f0f0fu};
+        bytes_to_frags(b, 0.0f, dsc, -dmn, f0, f1);  // (d*sc)*q - dmin*m, the dequantised value (gguf_dequant.h:304-341)
+    }
+    static constexpr int kBlockBytes = 144;
+    static constexpr bool kQ8Round = true;
+};
+struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh for each half, scales, d
+    uint4 ql[4], qh[2], sc;
+    uint32_t d;
+    __device__ __forceinline__ void load(const uint8_t* blk, int kh) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) ql[c] = ld16_a2(blk + 64 * (c >> 1) + 32 * (c & 1) + 16 * kh);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) qh[h] = ld16_a2(blk + 128 + 32 * h + 16 * kh);
+        sc = ld16_a2(blk + 192);
+        d = reinterpret_cast<const u16_a2*>(blk + 208)->v;
+    }
+    // step s (0..7): elements 32 s + 16 kh + (0..15) = half s/4, group gq = s%4, one scale (index 2 s + kh)
+    __device__ __forceinline__ void frags(int s, int kh, h8& f0, h8& f1) const {
+        const int half = s >> 2, gq = s & 3;
+        const uint4 l = ql[2 * half + (gq & 1)], hq = qh[half];
+        const int lsh = 4 * (gq >> 1), hsh = 2 * gq;
+        const uint32_t lw[4] = {l.x, l.y, l.z, l.w}, hw[4] = {hq.x, hq.y, hq.z, hq.w};
+        uint32_t b[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) b[w] = ((lw[w] >> lsh) & 0x0f0f0f0fu) | ((((hw[w] >> hsh) & 0x03030303u)) << 4);
+        const uint32_t scw[4] = {sc.x, sc.y, sc.z, sc.w};
+        const uint32_t pair = scw[s >> 1] >> (16 * (s & 1));            // scales 2s and 2s+1
+        const int sv = (int)(int8_t)((kh ? pair >> 8 : pair) & 0xffu);
+        bytes_to_frags(b, 32.0f, h2f(d) * (float)sv, 0.0f, f0, f1);     // d*scale*(q-32) (gguf_dequant.h:395-430)
+    }
+    static constexpr int kBlockBytes = 210;
+    static constexpr bool kQ8Round = false;
+};
+
+// X tile of a super-block step in LDS: thread t owns row t/2, byte half t%2 (256 B = 16 pieces of 16 B).  The
+// pieces of the NEXT block are fetched three per sub-block step during steps 0..5 of the current block and written
+// to the other LDS buffer two steps later, so a fetch has two step times to arrive and the block ends with the
+// next tile complete behind the only workgroup barrier of the block.  (After the last block the same code
+// re-fetches the last tile into the idle buffer: no conditionals in the steady-state loop.)
+template <typename Tile>
+__global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
+                                                        const float* __restrict__ rowscale, float* Y, int M, int K, int N) {
+    // W and Xh are deliberately not __restrict__: loads through a restrict pointer may be moved across the
+    // compiler fences below, and the prefetch distance of this loop depends on those fences
+    extern __shared__ __align__(16) uint8_t s_a[];  // [2][QF_TM * QF_PITCH]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, kh = lane >> 5;
+    const int m0 = blockIdx.y * QF_TM;
+    const int n_base = blockIdx.x * QF_TN + wave * 64;
+    const int nblk = K / 256;
+    const uint8_t* wrow[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) wrow[t] = W + (int64_t)min(n_base + 32 * t + j, N - 1) * stride;
+
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mt][t][r] = 0.0f;
+
+    // X tile of a block = 128 rows x 512 B = 4096 pieces of 16 B; piece q = 256 i + tid (i = 0..15) is row q / 32, bytes
+    // 16 (q % 32): a wave fetches two whole rows per instruction and writes LDS without bank conflicts
+    const int64_t x_row_bytes = (int64_t)K * 2;
+    const uint8_t* x_src = reinterpret_cast<const uint8_t*>(Xh) + (int64_t)(m0 + (tid >> 5)) * x_row_bytes + 16 * (tid & 31);
+    uint8_t* x_dst = s_a + (tid >> 5) * QF_PITCH + 16 * (tid & 31);
+    uint4 re0, re1, re2, ro0, ro1, ro2;  // pieces in flight: fetched at an even / odd step (scalars, not an array: they must stay in registers)
+    re0 = re1 = re2 = ro0 = ro1 = ro2 = make_uint4(0, 0, 0, 0);
+    // prologue: tile of block 0 -> LDS buffer 0, weights of block 0, fragments of step 0
+#pragma unroll
+    for (int p = 0; p < 16; ++p)
+        *reinterpret_cast<uint4*>(x_dst + 8 * p * QF_PITCH) = *reinterpret_cast<const uint4*>(x_src + 8 * p * x_row_bytes);
+    Tile cur[2], nxt[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) cur[t].load(wrow[t], kh);
+    h8 bf[2][2], bn[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) cur[t].frags(0, kh, bf[t][0], bf[t][1]);
+    __syncthreads();
+
+    for (int blk = 0; blk < nblk; ++blk) {
+        const int nb = min(blk + 1, nblk - 1);  // block whose tile and weights are fetched during this one
+        const uint8_t* a_cur = s_a + (blk & 1) * (QF_TM * QF_PITCH);
+        uint8_t* x_nxt = x_dst + ((blk & 1) ^ 1) * (QF_TM * QF_PITCH);
+        const uint8_t* x_from = x_src + (int64_t)nb * 512;
+        h8 af[2][4];  // X fragments of step 0 of this block (the tile became visible at the barrier)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+                af[ks][mt] = *reinterpret_cast<const h8*>(a_cur + (mt * 32 + j) * QF_PITCH + 32 * kh + 16 * ks);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {  // unrolled: the sub-block index selects registers
+            if (s >= 2) {  // pieces fetched two steps ago -> LDS
+                const int p = 3 * (s - 2);
+                *reinterpret_cast<uint4*>(x_nxt + 8 * p * QF_PITCH) = (s & 1) ? ro0 : re0;
+                if (p + 1 < 16) *reinterpret_cast<uint4*>(x_nxt + 8 * (p + 1) * QF_PITCH) = (s & 1) ? ro1 : re1;
+                if (p + 2 < 16) *reinterpret_cast<uint4*>(x_nxt + 8 * (p + 2) * QF_PITCH) = (s & 1) ? ro2 : re2;
+            }
+            if (s < 6) {
+                const int p = 3 * s;
+                const uint4 v0 = *reinterpret_cast<const uint4*>(x_from + 8 * p * x_row_bytes);
+                const uint4 v1 = *reinterpret_cast<const uint4*>(x_from + 8 * min(p + 1, 15) * x_row_bytes);
+                const uint4 v2 = *reinterpret_cast<const uint4*>(x_from + 8 * min(p + 2, 15) * x_row_bytes);
+                if (s & 1) { ro0 = v0; ro1 = v1; ro2 = v2; } else { re0 = v0; re1 = v1; re2 = v2; }
+            }
+            if (s == 0) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) nxt[t].load(wrow[t] + (int64_t)nb * Tile::kBlockBytes, kh);
+            }
+            issue_order_fence();  // the fetches stay HERE, two steps ahead of their use (the compiler would sink them to it)
+            // X fragments of the NEXT step are read from LDS now and weight fragments of the next step are prepared
+            // while this step's 16 MFMAs (all operands already in registers) run
+            h8 an[2][4];
+            if (s < 7) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt)
+                        an[ks][mt] = *reinterpret_cast<const h8*>(a_cur + (mt * 32 + j) * QF_PITCH + 64 * (s + 1) + 32 * kh + 16 * ks);
+            }
+#if defined(PTM_EXP) && PTM_EXP == 11
+#pragma unroll
+            for (int t = 0; t < 2; ++t) { bn[t][0] = bf[t][1]; bn[t][1] = bf[t][0]; }
+#else
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (s < 7) cur[t].frags(s + 1, kh, bn[t][0], bn[t][1]);
+                else nxt[t].frags(0, kh, bn[t][0], bn[t][1]);
+            }
+#endif
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                        acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks][mt], bf[t][ks], acc[mt][t], 0, 0, 0);
+            // issue order: one MFMA, then the vector work that fits under it (a 32x32x16 MFMA occupies the matrix pipe
+            // for 32 cycles = 8 vector instructions), so that neither pipe waits for the other
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);   // VALU
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) { bf[t][0] = bn[t][0]; bf[t][1] = bn[t][1]; }
+            if (s < 7) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt) af[ks][mt] = an[ks][mt];
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) cur[t] = nxt[t];
+        __syncthreads();  // next tile complete, this tile no longer read
+    }
+    // C layout of the 32x32 tile: column j = lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+            if (m < M) {
+                const float rs = rowscale[m];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int n = n_base + 32 * t + j;
+                    if (n < N) Y[(int64_t)m * N + n] = acc[mt][t][r] * rs;
+                }
+            }
+        }
+}
+
 static int qgemm_check(const void* W, const void* X, const void* Y, int M, int K, int N, int64_t stride, int blk_bytes) {
     if (!W || !X || !Y) return PTM_E_NULL;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 256) != 0) return PTM_E_SHAPE;
@@ -310,6 +607,49 @@ int ptm_qgemm_q6k(const void* W, const void* X_bf16, float* Y, int M, int K, int
     const dim3 grid((N + QG_NBLOCK - 1) / QG_NBLOCK, mp / QG_MCHUNK);
     hipLaunchKernelGGL(qgemm_q6k_kernel, grid, dim3(256), 0, as_stream(stream), static_cast<const uint8_t*>(W), stride,
                        static_cast<const uint16_t*>(X_bf16), Y, M, K, N);
+    return launch_status();
+}
+
+int64_t ptm_qgemm_f16_workspace_bytes(int M, int K) {
+    if (M <= 0 || K <= 0) return 0;
+    const int64_t mp = qf_mpad(M);
+    return mp * K * 2 + mp * 4;
+}
+
+int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* Y, int M, int K, int N, int64_t stride,
+                  void* workspace, ptm_stream_t stream) {
+    if (ggml_type != PTM_TYPE_Q4_K && ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
+    const int blk = ggml_type == PTM_TYPE_Q4_K ? 144 : 210;
+    const int rc = qgemm_check(W, X_bf16, Y, M, K, N, stride, blk);
+    if (rc != PTM_OK) return rc;
+    if (!workspace) return PTM_E_NULL;
+    if (!aligned16(workspace)) return PTM_E_ALIGN;
+    if (ggml_type == PTM_TYPE_Q4_K ? (!aligned16(W) || (stride & 15)) : ((stride & 1) || (reinterpret_cast<uintptr_t>(W) & 1u)))
+        return PTM_E_ALIGN;
+    const int mp = qf_mpad(M);
+    if (mp / QF_TM > 65535) return PTM_E_UNSUPPORTED;
+    _Float16* Xh = static_cast<_Float16*>(workspace);
+    float* rowscale = reinterpret_cast<float*>(Xh + (int64_t)mp * K);
+    hipStream_t s = as_stream(stream);
+    const size_t lds = 2 * (size_t)QF_TM * QF_PITCH;  // 132 KB: above the default 64 KB cap of dynamic LDS
+    static bool raised = false;
+    if (!raised) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        raised = true;
+    }
+    const dim3 grid((N + QF_TN - 1) / QF_TN, mp / QF_TM);
+    if (ggml_type == PTM_TYPE_Q4_K) {
+        hipLaunchKernelGGL(qgemm_prepare_rows_f16_kernel<true>, dim3(mp), dim3(256), 0, s, static_cast<const uint16_t*>(X_bf16),
+                           Xh, rowscale, M, K);
+        hipLaunchKernelGGL(qgemm_f16_kernel<Q4Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
+                           rowscale, Y, M, K, N);
+    } else {
+        hipLaunchKernelGGL(qgemm_prepare_rows_f16_kernel<false>, dim3(mp), dim3(256), 0, s, static_cast<const uint16_t*>(X_bf16),
+                           Xh, rowscale, M, K);
+        hipLaunchKernelGGL(qgemm_f16_kernel<Q6Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
+                           rowscale, Y, M, K, N);
+    }
     return launch_status();
 }
 

@@ -258,9 +258,20 @@ def qgemm_workspace_bytes(M, K):
     return _L().ptm_qgemm_workspace_bytes(M, K)
 
 
+def qgemm_f16_workspace_bytes(M, K):
+    return _L().ptm_qgemm_f16_workspace_bytes(M, K)
+
+
+def matmul_q_f16(quant_type, weights, x_bf16, y, M, K, N, row_stride_bytes, workspace, stream=None):
+    """Fast quantised-weight GEMM for M > 1 rows (fp16 MFMA on dequantised weights, Q8-rounded activations);
+    stands in for the M-GEMV loop of matmul_q (gguf_model.h:7029-7036) within the 1e-2 bar of the prefill path."""
+    check(_L().ptm_qgemm_f16(quant_type, _ptr(weights), _ptr(x_bf16), _ptr(y), M, K, N, row_stride_bytes,
+                             _ptr(workspace), _stream(stream)), "matmul_q_f16")
+
+
 def matmul_q(quant_type, weights, x_bf16, y, M, K, N, row_stride_bytes, workspace, stream=None):
-    """Quantised-weight GEMM for M > 1 rows; stands in for the M-GEMV loop of matmul_q
-    (gguf_model.h:7029-7036)."""
+    """Quantised-weight GEMM for M > 1 rows with the GEMV's arithmetic per row (Q4_K: bit-identical rows);
+    stands in for the M-GEMV loop of matmul_q (gguf_model.h:7029-7036)."""
     fn = _L().ptm_qgemm_q4k if quant_type == Q4_K else _L().ptm_qgemm_q6k
     if quant_type not in (Q4_K, Q6_K):
         raise PtmError(-4, "matmul_q: unsupported quant type")

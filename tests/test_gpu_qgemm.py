@@ -35,6 +35,16 @@ def gpu_qgemm(qt, W, xb, M, K, N):
     return Y.cpu().numpy()
 
 
+def gpu_qgemm_f16(qt, W, xb, M, K, N):
+    Wd = torch.from_numpy(W).cuda()
+    Xd = torch.from_numpy(xb.view(np.int16)).cuda()
+    Y = torch.full((M, N), 77.0, device="cuda")
+    ws = torch.empty(ops.qgemm_f16_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+    ops.matmul_q_f16(qt, Wd, Xd, Y, M, K, N, W.shape[1], ws)
+    torch.cuda.synchronize()
+    return Y.cpu().numpy()
+
+
 def oracle_rows(po, qt, W, xf):
     return np.stack([po.gemv(qt, W, xf[m]) for m in range(xf.shape[0])])
 
@@ -114,3 +124,64 @@ def test_qgemm_argument_errors(dev):
         ops.matmul_q(12, W, X, Y, 0, 256, 16, 144, ws)      # empty M
     with pytest.raises(PtmError):
         ops.matmul_q(13, W, X, Y, 4, 256, 16, 144, ws)      # not a K-quant this path handles
+
+
+# ---- fast path: fp16 MFMA on dequantised weights -------------------------------------------------------------
+QGEMM_F16_TOL = 1e-2   # the prefill path's stated bar: max |y - y_cpu| / rms(y_cpu) against the reference GEMV per row
+QGEMM_F16_EXPECT = 5e-3  # what fp16 rounding of both operands should stay under (measured ~1e-3)
+
+
+def oracle_rows_q8x(po, qt, W, xf):
+    """Reference rows.  Q6_K: the reference uses fp32 activations; the fast path rounds them to Q8 values first, so
+    its error against the reference's Q6_K GEMV includes that rounding (it is what the reference's Q4_K path does)."""
+    return np.stack([po.gemv(qt, W, xf[m]) for m in range(xf.shape[0])])
+
+
+@pytest.mark.parametrize("qt", [12, 14])
+@pytest.mark.parametrize("M,K,N", [(1, 256, 16), (5, 512, 48), (128, 512, 256), (130, 1024, 300), (257, 2560, 334),
+                                   (33, 256, 7)])
+def test_qgemm_f16_rows_vs_gemv(dev, po, qt, M, K, N):
+    r = synth.rng_for(44, qt, M, K, N)
+    W = synth.make_weight(r, qt, N, K)
+    xb, xf = bf16_round(r.standard_normal((M, K), dtype=np.float32))
+    Y = gpu_qgemm_f16(qt, W, xb, M, K, N)
+    ref = oracle_rows(po, qt, W, xf)
+    e = rel_err(Y, ref)
+    print(qt, M, K, N, "rel err", e, flush=True)
+    assert np.all(np.isfinite(Y))
+    assert e <= (QGEMM_F16_EXPECT if qt == 12 else QGEMM_F16_TOL)
+
+
+def test_qgemm_f16_large_and_zero_rows(dev, po):
+    M, K, N = 20, 512, 64
+    r = synth.rng_for(45)
+    x = r.standard_normal((M, K), dtype=np.float32)
+    x[3] = 0.0
+    x[4] *= 1e20      # far beyond fp16: exercised by the per-row power-of-two scale
+    x[5] *= 1e-3
+    xb, xf = bf16_round(x)
+    W = synth.make_weight(r, 12, N, K)
+    Y = gpu_qgemm_f16(12, W, xb, M, K, N)
+    ref = oracle_rows(po, 12, W, xf)
+    assert np.all(np.isfinite(Y)) and np.all(Y[3] == 0.0)
+    for m in range(M):
+        assert rel_err(Y[m], ref[m]) <= QGEMM_F16_EXPECT, m
+
+
+@pytest.mark.parametrize("qt,N,K", [(12, 4096, 4096), (12, 1024, 4096), (12, 14336, 4096), (14, 4096, 14336)])
+def test_qgemm_f16_llama3_8b_layer_shapes_m512(dev, po, qt, N, K):
+    M = 512
+    r = synth.rng_for(43, qt, N, K)
+    W = synth.make_weight(r, qt, N, K)
+    xb, xf = bf16_round(r.standard_normal((M, K), dtype=np.float32))
+    Y = gpu_qgemm_f16(qt, W, xb, M, K, N)
+    rows = np.unique(np.concatenate([np.arange(0, M, 61), [127, 128, 511]]))
+    ref = oracle_rows(po, qt, W, xf[rows])
+    e = rel_err(Y[rows], ref)
+    fro = float(np.linalg.norm(Y[rows] - ref) / np.linalg.norm(ref))
+    print(qt, N, K, "max/rms", e, "frobenius", fro, flush=True)
+    assert e <= QGEMM_F16_TOL and fro <= 3e-3
+    # against the bit-exact kernel on ALL rows (Q4_K): same bar
+    if qt == 12:
+        Yx = gpu_qgemm(qt, W, xb, M, K, N)
+        assert rel_err(Y, Yx) <= QGEMM_F16_EXPECT
