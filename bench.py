@@ -174,6 +174,14 @@ def main():
     lm = dec._cfg.lm_head.data
     ms1 = event_time_ms(lambda i: ops.q6k_gemv_argmax(lm, x, logits, H, V, stride6, idx, ws), 40, torch)
     gemv["cfg1_q6k_lm_head_argmax"] = {"bytes": b1, "us": ms1 * 1e3, "GBs": b1 / ms1 / 1e6, "frac": b1 / ms1 / 1e6 / HBM_PEAK_GBS}
+    # the Q4_K kernel on a launch large enough to amortise the launch floor (vocabulary-sized, 219 MB): shows what
+    # the kernel sustains once the ~1.6 us launch + ramp no longer dominates, as it does for a 14 MB matrix
+    Wbig = [torch.from_numpy(synth.make_q4k(synth.rng_for(SEED, 6 + i), V, H)).cuda() for i in range(3)]  # 657 MB > caches
+    ybig = torch.empty(V, device="cuda")
+    b3 = V * stride4 + 4 * H + 4 * V
+    ms3 = event_time_ms(lambda i: ops.launch_q4km_persistent_gemv(Wbig[i % 3], x, ybig, H, V, stride4), 42, torch)
+    gemv["q4k_large_151936x2560"] = {"bytes": b3, "us": ms3 * 1e3, "GBs": b3 / ms3 / 1e6, "frac": b3 / ms3 / 1e6 / HBM_PEAK_GBS}
+    del Wbig, ybig
     # down projection Q6_K 2560x9728
     xa = torch.randn(I, device="cuda")
     yd = torch.empty(H, device="cuda")

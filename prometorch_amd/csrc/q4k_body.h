@@ -16,6 +16,7 @@ struct Q4KArgs {
     int K;
     int log2S;       // lane groups per row = 1 << log2S
     int64_t stride;
+    int tiles_per_wg;    // row tiles (of 32 >> log2S rows) a workgroup walks with ONE staging of x (0 or 1: one tile)
     const void* x;       // fp32 x[K] (XQ8 == false) or Q8 blocks (XQ8 == true)
     const float* gamma;  // RMSNorm weight (NORM)
     float eps;
@@ -212,82 +213,94 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
     const int S = 1 << a.log2S;
     const int sub = grp & (S - 1);
     const int rows_per_wave = 8 >> a.log2S;
-    const int r = (wg * 4 + wave) * rows_per_wave + (grp >> a.log2S);
-    const bool live = r < a.total_rows;
-    const int rr = live ? r : a.total_rows - 1;
     const int nblk = a.K / 256;
     const int nb_max = (nblk + S - 1) >> a.log2S;  // passes are sized for the group with the most blocks
+    const int tpw = a.tiles_per_wg > 1 ? a.tiles_per_wg : 1;
+    const int n_tiles = (a.total_rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave);
 
-    int mat = 0, local = rr;
-    if constexpr (MODE == 1) {
-        mat = rr & 1;
-        local = rr >> 1;
-    } else {
-        if (a.n_mat > 1 && rr >= a.row_end[0]) { mat = 1; local = rr - a.row_end[0]; }
-        if (a.n_mat > 2 && rr >= a.row_end[1]) { mat = 2; local = rr - a.row_end[1]; }
-    }
-    const uint8_t* row = (mat == 0 ? a.W[0] : (mat == 1 ? a.W[1] : a.W[2])) + (int64_t)local * a.stride;
-
-    // ---- activation loads first, then the first pass of weight loads, then the activation prologue ----
-    __shared__ float red[4];
-#if defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3)
-    Q4KStage stg;
-#else
-    const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a, lds, red);
-#endif
-    uint4 hdr[NB], qv[NB];
-    issue_order_fence();
-#pragma unroll
-    for (int u = 0; u < NB; ++u) {
-        const uint8_t* p = row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 144;
-        hdr[u] = *reinterpret_cast<const uint4*>(p);
-        qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
-    }
-    issue_order_fence();
-#if !(defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3))
-    q4k_stage_finish<XQ8, NORM>(stg, a, lds, red);
-#endif
-
-    float acc = 0.0f;
-#pragma unroll
-    for (int u = 0; u < NB; ++u) {
-        const int b = sub + (u << a.log2S);
-        const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
-        acc += b < nblk ? t : 0.0f;
-    }
-    for (int i0 = NB; i0 < nb_max; i0 += NB) {
+    // One row tile: first pass of weight loads, `between` (the activation prologue on the first tile, nothing on the
+    // others), block terms, reduction, store.
+    auto run_tile = [&](int tile, auto&& between) {
+        const int r = (tile * 4 + wave) * rows_per_wave + (grp >> a.log2S);
+        const bool live = r < a.total_rows;
+        const int rr = live ? r : a.total_rows - 1;
+        int mat = 0, local = rr;
+        if constexpr (MODE == 1) {
+            mat = rr & 1;
+            local = rr >> 1;
+        } else {
+            if (a.n_mat > 1 && rr >= a.row_end[0]) { mat = 1; local = rr - a.row_end[0]; }
+            if (a.n_mat > 2 && rr >= a.row_end[1]) { mat = 2; local = rr - a.row_end[1]; }
+        }
+        const uint8_t* row = (mat == 0 ? a.W[0] : (mat == 1 ? a.W[1] : a.W[2])) + (int64_t)local * a.stride;
+        uint4 hdr[NB], qv[NB];
+        issue_order_fence();
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
-            const uint8_t* p = row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 144;
+            const uint8_t* p = row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 144;
             hdr[u] = *reinterpret_cast<const uint4*>(p);
             qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
         }
+        issue_order_fence();
+        between();
+
+        float acc = 0.0f;
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
-            const int b = sub + ((i0 + u) << a.log2S);
+            const int b = sub + (u << a.log2S);
             const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
             acc += b < nblk ? t : 0.0f;
         }
-    }
-    // reduce: 8 lanes of the group, then the S groups of the row
-    float p = sum8(acc);
-    if (S >= 2) p += dpp_f<0x128>(p);  // row_ror:8 = the other 8-lane half of the 16-lane row
-    if (S >= 4) p += __shfl_xor(p, 16, 64);
-    if (S >= 8) p += __shfl_xor(p, 32, 64);
-
-    if constexpr (MODE == 1) {
-        // gate and up of one row sit S groups apart
-        float other;
-        if (S == 1) other = dpp_f<0x128>(p);
-        else if (S == 2) other = __shfl_xor(p, 16, 64);
-        else other = __shfl_xor(p, 32, 64);
-        if (live && mat == 0 && sub == 0 && j == 0) a.y[0][local] = silu_mul_ref(p, other);
-    } else {
-        float* y = mat == 0 ? a.y[0] : (mat == 1 ? a.y[1] : a.y[2]);
-        if (live && sub == 0 && j == 0) {
-            if constexpr (ACC) y[local] += p;
-            else y[local] = p;
+        for (int i0 = NB; i0 < nb_max; i0 += NB) {
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                const uint8_t* p = row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 144;
+                hdr[u] = *reinterpret_cast<const uint4*>(p);
+                qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+            }
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                const int b = sub + ((i0 + u) << a.log2S);
+                const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
+                acc += b < nblk ? t : 0.0f;
+            }
         }
+        // reduce: 8 lanes of the group, then the S groups of the row
+        float p = sum8(acc);
+        if (S >= 2) p += dpp_f<0x128>(p);  // row_ror:8 = the other 8-lane half of the 16-lane row
+        if (S >= 4) p += __shfl_xor(p, 16, 64);
+        if (S >= 8) p += __shfl_xor(p, 32, 64);
+
+        if constexpr (MODE == 1) {
+            // gate and up of one row sit S groups apart
+            float other;
+            if (S == 1) other = dpp_f<0x128>(p);
+            else if (S == 2) other = __shfl_xor(p, 16, 64);
+            else other = __shfl_xor(p, 32, 64);
+            if (live && mat == 0 && sub == 0 && j == 0) a.y[0][local] = silu_mul_ref(p, other);
+        } else {
+            float* y = mat == 0 ? a.y[0] : (mat == 1 ? a.y[1] : a.y[2]);
+            if (live && sub == 0 && j == 0) {
+                if constexpr (ACC) y[local] += p;
+                else y[local] = p;
+            }
+        }
+    };
+
+    // ---- activation loads first, then the first tile's weight loads, then the activation prologue ----
+    __shared__ float red[4];
+#if defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3)
+    Q4KStage stg;
+    run_tile(wg * tpw, [] {});
+#else
+    const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a, lds, red);
+    run_tile(wg * tpw, [&] { q4k_stage_finish<XQ8, NORM>(stg, a, lds, red); });
+#endif
+    // further tiles reuse the staged activations: the quantisation of x is paid once per workgroup
+    for (int k = 1; k < tpw; ++k) {
+        const int tile = wg * tpw + k;
+        if (tile >= n_tiles) break;
+        run_tile(tile, [] {});
     }
 }
 
@@ -314,6 +327,18 @@ inline int q4k_pick_log2S(int total_rows, int nblk, int max_log2S) {
 inline int q4k_workgroups(int total_rows, int log2S) {
     const int rows_per_wg = 32 >> log2S;
     return (total_rows + rows_per_wg - 1) / rows_per_wg;
+}
+// Row tiles per workgroup: beyond ~1200 tiles a workgroup walks several, so that the activation prologue (every
+// workgroup quantises the whole vector) is amortised.  PTM_Q4K_TPW (1..9) overrides, for tuning runs.
+inline int q4k_tiles_per_wg(int n_tiles) {
+    static const int forced = [] {
+        const char* e = getenv("PTM_Q4K_TPW");
+        return (e && e[0] >= '1' && e[0] <= '9' && e[1] == 0) ? e[0] - '0' : 0;
+    }();
+    if (forced > 0) return forced;
+    int t = 1;
+    while (t < 8 && (n_tiles + t - 1) / t > 1280) ++t;
+    return t;
 }
 inline int q4k_blocks_per_pass(int nblk, int log2S) {
     static const int cand[] = {2, 3, 5, 10};

@@ -29,7 +29,9 @@ __global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_kernel(const Q4KArgs a) 
 template <bool XQ8, bool NORM, bool ACC, int MODE>
 static int q4k_launch(Q4KArgs& a, hipStream_t s) {
     a.log2S = q4k_pick_log2S(a.total_rows, a.K / 256, MODE == 1 ? 2 : 3);
-    const dim3 grid(q4k_workgroups(a.total_rows, a.log2S)), block(Q4K_THREADS);
+    const int n_tiles = q4k_workgroups(a.total_rows, a.log2S);
+    a.tiles_per_wg = q4k_tiles_per_wg(n_tiles);
+    const dim3 grid((n_tiles + a.tiles_per_wg - 1) / a.tiles_per_wg), block(Q4K_THREADS);
     const size_t lds = (size_t)q8_bytes(a.K);
     switch (q4k_blocks_per_pass(a.K / 256, a.log2S)) {
         case 2: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 2>), grid, block, lds, s, a); break;
