@@ -242,6 +242,8 @@ static int fd_merge(int head_dim, int n_heads, hipStream_t s, const float* pO, c
 // The split merge stays a second, small launch: doing it in the last-arriving workgroup needs
 // device-scope release/acquire fences in all ~270 workgroups, which measured slower on MI355X
 // (L2 write-back per fence across the 8 XCDs) than the extra launch.
+// The kernel's cost is instruction latency (about one wave per SIMD, each with a long dependent chain), not the
+// 8.6 MB of KV it reads, so the arithmetic is kept short: hardware exp2 / rsq, no barrier before the final merge.
 // ---------------------------------------------------------------------------------------------
 struct AttnArgs {
     const float *Q, *K, *V, *qw, *kw, *rope;

@@ -14,8 +14,12 @@
 // A row is shared by S lane groups (S = 1, 2, 4 or 8 - a whole wave), group s taking blocks
 // s, s+S, ...; S is chosen on the host so that a launch has several hundred workgroups even for
 // short-and-wide matrices (o-proj: 2560 rows) and so that each group's blocks are all in flight
-// at once.  The first pass of weight loads is issued BEFORE the activation vector is staged
-// (RMSNorm, Q8 quantisation, LDS), so HBM latency overlaps the prologue.
+// at once (five per group measured best: fewer registers, more waves per SIMD).  The first pass of
+// weight loads is issued BEFORE the activation vector is staged (RMSNorm, Q8 quantisation, LDS), so HBM
+// latency overlaps the prologue; every pass issues a fixed number of loads (template NB) and activations
+// come through range-checked buffer loads, so no load sits under a branch and the compiler can wait for
+// exactly the block it is about to use.  Very tall matrices let a workgroup walk several row tiles with
+// one staging of x.
 #include "q4k_body.h"
 
 namespace ptm {

@@ -5,11 +5,15 @@
 //   ql[16j .. 16j+16)            16 low nibbles  -> group (j%4)/2   of half j/4
 //                                16 high nibbles -> group (j%4)/2+2 of half j/4
 //   qh[32*(j/4) + 16*(j%2) ..+16) the 2-bit planes of those 32 weights
-//   scales[16] and d             (same for the 8 lanes)
-// with 128-bit loads (blocks are only 2-byte aligned; gfx950 global loads take that).
+//   its two scales (single signed bytes) and d
+// with dword-aligned 128-bit loads: blocks are 210 bytes, so every other block starts 2 bytes off a dword, and
+// 16-byte loads from such addresses run at a fraction of the aligned rate; the lane loads the aligned 16 bytes
+// just below plus the piece's last two bytes and shifts them into place with v_alignbyte.
 // Weights are assembled four at a time in a dword (q = nibble | twobits<<4, 0..63), converted
 // with v_cvt_f32_ubyteN and multiplied with x from LDS; the "-32" offset is applied once per
 // 16 weights through the per-16 sums of x kept in LDS:  sum (q-32) x = sum q x - 32 sum x.
+// Every pass issues a fixed number of block loads (template NB) behind the activation loads, so the compiler can
+// count the loads in flight and each block is consumed as soon as it has arrived.
 #include "q6k_body.h"
 
 namespace ptm {

@@ -1,8 +1,9 @@
 // Prefill: quantised-weight GEMM  Y[M,N] = X[M,K] . W[N,K]^T  on the matrix cores (gfx950 MFMA).
 //
 // The reference has no such kernel: for M > 1 rows matmul_q runs M independent GEMVs
-// (torch/io/gguf_model.h:7029-7036, :7056-7061), re-reading the weights M times.  These kernels keep the
-// GEMV's arithmetic per output row and read each weight tile once per 64 rows of X.
+// (torch/io/gguf_model.h:7029-7036, :7056-7061), re-reading the weights M times.  Two families:
+//   * exact kernels (below): the GEMV's arithmetic per output row, each weight tile read once per 64 rows of X;
+//   * a fast kernel (second half of this file): fp16 MFMA on weights dequantised in registers.
 //
 // Q4_K (reference row semantics: torch/io/cpu_quant_gemv.h:505-685)
 //   rows of X are quantised to Q8 blocks of 32 (same rule as the GEMV), and for every 32-wide sub-block
