@@ -35,7 +35,10 @@ enum {
     PTM_E_UNSUPPORTED = -4, /* quant type / head_dim / size outside what the kernels implement */
     PTM_E_HIP = -5,         /* a HIP runtime call failed (ptm_last_hip_error() has the code) */
     PTM_E_RANGE = -6,       /* position / token beyond the allocated cache or table */
-    PTM_E_STATE = -7        /* object used before initialisation or after an error */
+    PTM_E_STATE = -7,       /* object used before initialisation or after an error */
+    PTM_E_IO = -8,          /* file cannot be opened / mapped */
+    PTM_E_FORMAT = -9,      /* file is not well-formed GGUF, or a required key is missing or of the wrong kind */
+    PTM_E_NOT_FOUND = -10   /* no tensor / metadata key of that name */
 };
 
 enum { PTM_TYPE_Q4_K = 12, PTM_TYPE_Q6_K = 14 }; /* ggml type ids, gguf_dequant.h:29-58 */
@@ -260,6 +263,47 @@ int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_ou
 const float* ptm_decode_logits(ptm_decoder* d);
 const float* ptm_decode_hidden(ptm_decoder* d);
 void* ptm_decode_stream(ptm_decoder* d);
+
+/* ---- GGUF files: container reader and model loader --------------------------------------- */
+/* Reader for GGUF v2/v3 (the reference's GGUFReader, torch/io/gguf_loader.h:386-630): the file is
+ * memory-mapped; tensor data pointers are HOST pointers into the mapping, valid until close.
+ * dims[0] is the contiguous dimension (K), dims[1] the rows (N); nbytes is -1 for a ggml type this
+ * library does not size (anything but F32, F16, Q4_K, Q6_K). */
+typedef struct ptm_gguf ptm_gguf;
+typedef struct {
+    const char* name;
+    uint32_t ggml_type;
+    int32_t n_dims;
+    int64_t dims[4];
+    int64_t nbytes;
+    const void* data;
+} ptm_gguf_tensor;
+int ptm_gguf_open(const char* path, ptm_gguf** out);
+void ptm_gguf_close(ptm_gguf* g);
+int ptm_gguf_version(const ptm_gguf* g);
+int64_t ptm_gguf_alignment(const ptm_gguf* g);
+int64_t ptm_gguf_n_tensors(const ptm_gguf* g);
+int ptm_gguf_tensor_at(const ptm_gguf* g, int64_t i, ptm_gguf_tensor* out);
+int ptm_gguf_find_tensor(const ptm_gguf* g, const char* name, ptm_gguf_tensor* out);
+/* Metadata: integers and bools widened to int64, floats to double (an integer key also reads as
+ * float); strings by pointer (NULL if absent or not a string); arrays are not exposed. */
+int ptm_gguf_get_int(const ptm_gguf* g, const char* key, int64_t* out);
+int ptm_gguf_get_float(const ptm_gguf* g, const char* key, double* out);
+const char* ptm_gguf_get_string(const ptm_gguf* g, const char* key);
+
+/* From a .gguf file to a ready decoder: reads the `qwen3` hyper-parameters
+ * (<arch>.block_count, embedding_length, feed_forward_length, attention.head_count(_kv),
+ * attention.key_length, rope.freq_base, attention.layer_norm_rms_epsilon; gguf_model.h:126-181),
+ * uploads every blk.N.{attn_q,attn_k,attn_v,attn_output,ffn_gate,ffn_up,ffn_down}.weight and
+ * output.weight (or the tied token_embd.weight) verbatim (gguf_model.h:1177-1360), norm vectors as
+ * fp32, allocates zeroed KV caches for max_seq positions and creates the decode runtime.
+ * Matrices must be Q4_K or Q6_K; other architectures, biases and other types: PTM_E_UNSUPPORTED. */
+typedef struct ptm_model ptm_model;
+int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_graph, ptm_model** out);
+ptm_decoder* ptm_model_decoder(ptm_model* m); /* owned by the model */
+int ptm_model_config(const ptm_model* m, ptm_decode_config* out);
+int ptm_model_layer(const ptm_model* m, int i, ptm_layer* out);
+void ptm_model_free(ptm_model* m);
 
 #ifdef __cplusplus
 }

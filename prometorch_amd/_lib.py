@@ -34,6 +34,11 @@ class DecodeConfig(C.Structure):
                 ("embedding_f32", vp), ("layers", C.POINTER(Layer)), ("out_norm", vp), ("lm_head", QWeight)]
 
 
+class GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("ggml_type", u32), ("n_dims", C.c_int32), ("dims", i64 * 4), ("nbytes", i64),
+                ("data", vp)]
+
+
 # name -> (restype, argtypes); every function declared in include/ptm.h
 SIGNATURES = {
     "ptm_strerror": (C.c_char_p, [i32]),
@@ -85,6 +90,21 @@ SIGNATURES = {
     "ptm_decode_logits": (vp, [vp]),
     "ptm_decode_hidden": (vp, [vp]),
     "ptm_decode_stream": (vp, [vp]),
+    "ptm_gguf_open": (i32, [C.c_char_p, C.POINTER(vp)]),
+    "ptm_gguf_close": (None, [vp]),
+    "ptm_gguf_version": (i32, [vp]),
+    "ptm_gguf_alignment": (i64, [vp]),
+    "ptm_gguf_n_tensors": (i64, [vp]),
+    "ptm_gguf_tensor_at": (i32, [vp, i64, C.POINTER(GgufTensor)]),
+    "ptm_gguf_find_tensor": (i32, [vp, C.c_char_p, C.POINTER(GgufTensor)]),
+    "ptm_gguf_get_int": (i32, [vp, C.c_char_p, C.POINTER(i64)]),
+    "ptm_gguf_get_float": (i32, [vp, C.c_char_p, C.POINTER(C.c_double)]),
+    "ptm_gguf_get_string": (C.c_char_p, [vp, C.c_char_p]),
+    "ptm_model_load_gguf": (i32, [C.c_char_p, i32, i32, i32, C.POINTER(vp)]),
+    "ptm_model_decoder": (vp, [vp]),
+    "ptm_model_config": (i32, [vp, C.POINTER(DecodeConfig)]),
+    "ptm_model_layer": (i32, [vp, i32, C.POINTER(Layer)]),
+    "ptm_model_free": (None, [vp]),
 }
 
 _lib = None

@@ -296,6 +296,9 @@ const char* ptm_strerror(int code) {
         case PTM_E_HIP: return "HIP runtime error";
         case PTM_E_RANGE: return "index out of range";
         case PTM_E_STATE: return "invalid object state";
+        case PTM_E_IO: return "file cannot be opened or mapped";
+        case PTM_E_FORMAT: return "malformed GGUF file or missing / mistyped key";
+        case PTM_E_NOT_FOUND: return "no tensor or key of that name";
         default: return "unknown error";
     }
 }

@@ -1,0 +1,234 @@
+"""GGUF files: reader (ctypes over ptm_gguf_*), a writer for tests and tools, and the model loader
+(ptm_model_load_gguf), the counterpart of GGUFReader + GGUFModel::load (reference:
+torch/io/gguf_loader.h:386-630, torch/io/gguf_model.h:1177-1360)."""
+from __future__ import annotations
+
+import ctypes as C
+import struct
+
+import numpy as np
+
+from . import _lib
+from ._lib import DecodeConfig, GgufTensor, Layer, check
+
+F32, F16, Q4_K, Q6_K = 0, 1, 12, 14
+_T_U32, _T_I32, _T_F32, _T_BOOL, _T_STR, _T_ARR, _T_U64 = 4, 5, 6, 7, 8, 9, 10
+
+
+# ---------------------------------------------------------------------------------------------
+# writer (GGUF v3, little endian)
+# ---------------------------------------------------------------------------------------------
+def _s(x: str) -> bytes:
+    b = x.encode("utf-8")
+    return struct.pack("<Q", len(b)) + b
+
+
+def _kv(key: str, value) -> bytes:
+    out = _s(key)
+    if isinstance(value, bool):
+        return out + struct.pack("<IB", _T_BOOL, int(value))
+    if isinstance(value, int):
+        return out + (struct.pack("<II", _T_U32, value) if 0 <= value < 2 ** 32 else struct.pack("<IQ", _T_U64, value))
+    if isinstance(value, float):
+        return out + struct.pack("<If", _T_F32, value)
+    if isinstance(value, str):
+        return out + struct.pack("<I", _T_STR) + _s(value)
+    if isinstance(value, (list, tuple)):
+        if all(isinstance(v, str) for v in value):
+            return out + struct.pack("<IIQ", _T_ARR, _T_STR, len(value)) + b"".join(_s(v) for v in value)
+        if all(isinstance(v, int) for v in value):
+            return out + struct.pack("<IIQ", _T_ARR, _T_I32, len(value)) + struct.pack("<%di" % len(value), *value)
+        return out + struct.pack("<IIQ", _T_ARR, _T_F32, len(value)) + struct.pack("<%df" % len(value), *value)
+    raise TypeError(f"unsupported metadata value for {key}: {type(value)}")
+
+
+def write_gguf(path: str, metadata: dict, tensors: list, alignment: int = 32, version: int = 3) -> None:
+    """tensors: list of (name, ggml_type, dims, bytes-like) with dims[0] the contiguous dimension.
+    Quantised matrices are passed as their raw super-blocks."""
+    md = dict(metadata)
+    if alignment != 32:
+        md["general.alignment"] = alignment
+    head = struct.pack("<IIQQ", 0x46554747, version, len(tensors), len(md))
+    head += b"".join(_kv(k, v) for k, v in md.items())
+    infos, blobs, off = b"", [], 0
+    for name, gtype, dims, data in tensors:
+        raw = np.ascontiguousarray(data).tobytes() if isinstance(data, np.ndarray) else bytes(data)
+        infos += _s(name) + struct.pack("<I", len(dims)) + struct.pack("<%dQ" % len(dims), *dims) + struct.pack("<IQ", gtype, off)
+        pad = (-len(raw)) % alignment
+        blobs.append(raw + b"\0" * pad)
+        off += len(raw) + pad
+    pre = head + infos
+    pre += b"\0" * ((-len(pre)) % alignment)
+    with open(path, "wb") as f:
+        f.write(pre)
+        for b in blobs:
+            f.write(b)
+
+
+def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "qwen3", tied: bool = True,
+                  alignment: int = 32) -> None:
+    """Write a decoder (the dict form prometorch_amd.decode.Decoder takes) as a GGUF file with the
+    tensor names and metadata keys a qwen3 GGUF carries."""
+    md = {
+        "general.architecture": arch, "general.name": "synthetic",
+        f"{arch}.block_count": cfg["n_layers"], f"{arch}.embedding_length": cfg["hidden"],
+        f"{arch}.feed_forward_length": cfg["inter"], f"{arch}.attention.head_count": cfg["n_heads"],
+        f"{arch}.attention.head_count_kv": cfg["n_kv_heads"], f"{arch}.attention.key_length": cfg["head_dim"],
+        f"{arch}.attention.value_length": cfg["head_dim"], f"{arch}.rope.freq_base": float(cfg["rope_base"]),
+        f"{arch}.attention.layer_norm_rms_epsilon": float(cfg["eps"]), f"{arch}.context_length": 4096,
+        "tokenizer.ggml.model": "gpt2", "tokenizer.ggml.tokens": ["a", "b", "c"], "tokenizer.ggml.token_type": [1, 1, 1],
+    }
+    H = cfg["hidden"]
+    ts = [("token_embd.weight", Q6_K, [H, cfg["vocab"]], head["lm_head"])]
+    if not tied:
+        ts.append(("output.weight", Q6_K, [H, cfg["vocab"]], head["lm_head"]))
+    ts.append(("output_norm.weight", F32, [H], np.asarray(head["out_norm"], np.float32)))
+    names = {"q": "attn_q", "k": "attn_k", "v": "attn_v", "o": "attn_output", "gate": "ffn_gate", "up": "ffn_up", "down": "ffn_down"}
+    for i, L in enumerate(layers):
+        p = f"blk.{i}."
+        ts.append((p + "attn_norm.weight", F32, [H], np.asarray(L["attn_norm"], np.float32)))
+        for k, gname in names.items():
+            qt, W = L[k]
+            cols = W.shape[1] // (144 if qt == Q4_K else 210) * 256
+            ts.append((p + gname + ".weight", qt, [cols, W.shape[0]], W))
+        ts.append((p + "attn_q_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["q_norm"], np.float32)))
+        ts.append((p + "attn_k_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["k_norm"], np.float32)))
+        ts.append((p + "ffn_norm.weight", F32, [H], np.asarray(L["ffn_norm"], np.float32)))
+    write_gguf(path, md, ts, alignment=alignment)
+
+
+# ---------------------------------------------------------------------------------------------
+# reader
+# ---------------------------------------------------------------------------------------------
+class GGUFFile:
+    """Memory-mapped GGUF file; tensor data is exposed as numpy views of the mapping (valid until close)."""
+
+    def __init__(self, path: str):
+        self.L = _lib.load()
+        h = C.c_void_p()
+        check(self.L.ptm_gguf_open(path.encode(), C.byref(h)), f"gguf_open({path})")
+        self.h = h
+
+    @property
+    def version(self) -> int:
+        return self.L.ptm_gguf_version(self.h)
+
+    @property
+    def alignment(self) -> int:
+        return self.L.ptm_gguf_alignment(self.h)
+
+    def __len__(self) -> int:
+        return self.L.ptm_gguf_n_tensors(self.h)
+
+    def _wrap(self, t: GgufTensor) -> dict:
+        data = None
+        if t.nbytes >= 0:
+            data = np.ctypeslib.as_array((C.c_uint8 * t.nbytes).from_address(t.data)) if t.nbytes else np.zeros(0, np.uint8)
+        return {"name": t.name.decode(), "type": t.ggml_type, "dims": [t.dims[i] for i in range(t.n_dims)],
+                "nbytes": t.nbytes, "data": data}
+
+    def tensor(self, key) -> dict:
+        t = GgufTensor()
+        if isinstance(key, int):
+            check(self.L.ptm_gguf_tensor_at(self.h, key, C.byref(t)), "gguf_tensor_at")
+        else:
+            check(self.L.ptm_gguf_find_tensor(self.h, key.encode(), C.byref(t)), f"gguf_find_tensor({key})")
+        return self._wrap(t)
+
+    def get_int(self, key: str) -> int:
+        v = C.c_int64()
+        check(self.L.ptm_gguf_get_int(self.h, key.encode(), C.byref(v)), f"gguf_get_int({key})")
+        return v.value
+
+    def get_float(self, key: str) -> float:
+        v = C.c_double()
+        check(self.L.ptm_gguf_get_float(self.h, key.encode(), C.byref(v)), f"gguf_get_float({key})")
+        return v.value
+
+    def get_string(self, key: str):
+        s = self.L.ptm_gguf_get_string(self.h, key.encode())
+        return None if s is None else s.decode()
+
+    def close(self) -> None:
+        if getattr(self, "h", None):
+            self.L.ptm_gguf_close(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+# ---------------------------------------------------------------------------------------------
+# model loader
+# ---------------------------------------------------------------------------------------------
+class GGUFModel:
+    """A decoder created straight from a .gguf file; same stepping interface as decode.Decoder."""
+
+    def __init__(self, path: str, max_seq: int, kv_fp16: bool = True, use_graph: bool = True):
+        self.L = _lib.load()
+        m = C.c_void_p()
+        check(self.L.ptm_model_load_gguf(path.encode(), max_seq, int(kv_fp16), int(use_graph), C.byref(m)),
+              f"model_load_gguf({path})")
+        self.m = m
+        self.h = self.L.ptm_model_decoder(m)
+        c = DecodeConfig()
+        check(self.L.ptm_model_config(m, C.byref(c)), "model_config")
+        self.cfg = {k: getattr(c, k) for k in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")}
+        self.cfg.update(rope_base=c.rope_freq_base, eps=c.rms_eps, kv_fp16=bool(c.kv_fp16), tied=not bool(c.embedding_f32))
+
+    def layer(self, i: int) -> Layer:
+        out = Layer()
+        check(self.L.ptm_model_layer(self.m, i, C.byref(out)), "model_layer")
+        return out
+
+    def set_kv(self, layer: int, k16: np.ndarray, v16: np.ndarray) -> None:
+        import torch
+        Ld = self.layer(layer)
+        dt = torch.float16 if self.cfg["kv_fp16"] else torch.float32
+        for ptr, src in ((Ld.k_cache, k16), (Ld.v_cache, v16)):
+            t = torch.from_numpy(np.ascontiguousarray(src)).to(device="cuda", dtype=dt).contiguous()
+            nbytes = t.numel() * t.element_size()
+            n4 = nbytes // 4  # rows are multiples of 4 bytes: reuse the fp32 copy kernel for the raw bytes
+            check(self.L.ptm_copy(t.data_ptr(), ptr, n4, None), "copy")
+        torch.cuda.synchronize()
+
+    def set_past_len(self, n: int) -> None:
+        check(self.L.ptm_decode_set_past_len(self.h, n), "decode_set_past_len")
+
+    def step(self, token: int) -> int:
+        out = C.c_int64()
+        check(self.L.ptm_decode_step(self.h, token, C.byref(out)), "decode_step")
+        return out.value
+
+    def greedy(self, first_token: int, n: int) -> list:
+        buf = (C.c_int64 * n)()
+        check(self.L.ptm_decode_greedy(self.h, first_token, n, buf), "decode_greedy")
+        return list(buf)
+
+    def logits(self) -> np.ndarray:
+        import torch
+        out = torch.empty(self.cfg["vocab"], dtype=torch.float32, device="cuda")
+        check(self.L.ptm_copy(self.L.ptm_decode_logits(self.h), out.data_ptr(), self.cfg["vocab"], None), "copy")
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    def close(self) -> None:
+        if getattr(self, "m", None):
+            self.L.ptm_model_free(self.m)
+            self.m = None
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,75 @@
+"""GPU: a model loaded from a .gguf file (ptm_model_load_gguf) decodes exactly like the same weights handed to
+the decoder directly, and like the compiled reference's golden run."""
+import numpy as np
+import pytest
+
+from conftest import bits
+from prometorch_amd import gguf, synth
+from prometorch_amd._lib import PtmError
+
+pytestmark = pytest.mark.gpu
+
+
+def build_tiny(seeds):
+    cfg = dict(synth.TINY)
+    layers = [synth.make_layer(seeds["tiny"], i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(seeds["tiny"], cfg)
+    kv = [synth.make_kv_prefill(seeds["tiny"], i, cfg, 19) for i in range(cfg["n_layers"])]
+    return cfg, layers, head, kv
+
+
+@pytest.mark.parametrize("tied", [True, False])
+def test_gguf_model_decodes_like_direct_decoder(dev, seeds, golden, tmp_path, tied):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = build_tiny(seeds)
+    path = str(tmp_path / "tiny.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head, tied=tied, alignment=64)
+    m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
+    for k in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter"):
+        assert m.cfg[k] == cfg[k], k
+    assert m.cfg["tied"] == tied and abs(m.cfg["rope_base"] - cfg["rope_base"]) < 1 and abs(m.cfg["eps"] - cfg["eps"]) < 1e-12
+    emb = None
+    if not tied:  # an untied file gets an fp32 embedding table dequantised from token_embd
+        from oracle import pyoracle as po
+        emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False, embedding_f32=emb)
+    for i, (k, v) in enumerate(kv):
+        m.set_kv(i, k, v)
+        d.set_kv(i, k, v)
+    m.set_past_len(19)
+    d.set_past_len(19)
+    tm = td = 3
+    for st in range(12):
+        tm = m.step(tm)
+        td = d.step(td)
+        assert tm == td == int(golden["tiny_tokens"][st]), st
+        assert np.array_equal(bits(m.logits()), bits(d.logits())), st
+    assert m.greedy(tm, 8) == d.greedy(td, 8)
+    m.close()
+    d.close()
+
+
+def test_gguf_model_refuses_what_it_cannot_run(dev, seeds, tmp_path):
+    cfg, layers, head, _ = build_tiny(seeds)
+    p = str(tmp_path / "llama.gguf")
+    gguf.model_to_gguf(p, cfg, layers, head, arch="llama")
+    with pytest.raises(PtmError) as e:
+        gguf.GGUFModel(p, max_seq=64)
+    assert e.value.code == -4
+    # a tensor of the wrong shape
+    bad = [dict(L) for L in layers]
+    qt, W = bad[1]["down"]
+    bad[1]["down"] = (qt, W[:-1])
+    p2 = str(tmp_path / "short.gguf")
+    gguf.model_to_gguf(p2, cfg, bad, head)
+    with pytest.raises(PtmError) as e:
+        gguf.GGUFModel(p2, max_seq=64)
+    assert e.value.code == -2
+    # a missing tensor
+    p3 = str(tmp_path / "missing.gguf")
+    cfg3 = dict(cfg)
+    cfg3["n_layers"] = 3
+    gguf.model_to_gguf(p3, cfg3, layers, head)
+    with pytest.raises(PtmError) as e:
+        gguf.GGUFModel(p3, max_seq=64)
+    assert e.value.code == -10
