@@ -217,6 +217,18 @@ def main():
     gemv["copy_256MiB"] = {"bytes_read": ca.numel() * 4, "bytes_written": ca.numel() * 4, "us": msc * 1e3,
                            "GBs": 2 * ca.numel() * 4 / msc / 1e6}
     del ca, cb
+    # prompt prefill through all layers: 512 tokens from an empty context (row-batched GEMMs + causal attention)
+    prompt = [int(t) for t in synth.rng_for(SEED, 9).integers(0, V, 512)]
+    layer_params = H * (2 * cfg["n_heads"] * cfg["head_dim"] + 2 * cfg["n_kv_heads"] * cfg["head_dim"] + 3 * I)
+    dec.set_past_len(0)
+    dec.prefill(prompt)  # allocates the row scratch
+    t1 = time.perf_counter()
+    for _ in range(3):
+        dec.set_past_len(0)
+        dec.prefill(prompt)
+    dtp = (time.perf_counter() - t1) / 3
+    gemv["prefill_512_tokens"] = {"ms": dtp * 1e3, "tok_s": 512 / dtp,
+                                  "gemm_TFLOPs": 2.0 * 512 * nL * layer_params / dtp / 1e12}
     log(json.dumps(gemv))
     per_token_bytes = nL * 63866880 + V * stride6 + nL * 2 * (N_PREFILL + args.warmup + args.steps / 2) * 1024 * 2
     dec.close()

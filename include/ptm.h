@@ -218,6 +218,27 @@ int ptm_qgemm_q6k(const void* W, const void* X_bf16, float* Y, int M, int K, int
 int64_t ptm_qgemm_f16_workspace_bytes(int M, int K);
 int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* Y, int M, int K, int N,
                   int64_t row_stride_bytes, void* workspace, ptm_stream_t stream);
+/* The same with fp32 rows of X (what the reference's prefill holds) and an optional Y += result. */
+int ptm_qgemm_f16_f32(uint32_t ggml_type, const void* W, const float* X_f32, float* Y, int M, int K, int N,
+                      int64_t row_stride_bytes, void* workspace, int accumulate, ptm_stream_t stream);
+
+/* ---- prefill glue: the decode-step pieces batched over prompt rows ----------------------- */
+/* out[r][:] = embedding of d_tokens[r] from an fp32 table [vocab][hidden], or (table_f32 NULL) from Q6_K rows
+ * dequantised on the fly.  embedding_lookup, gguf_model.h:2513. */
+int ptm_embedding_rows(const float* table_f32, const void* table_q6k, int64_t q6k_row_stride_bytes, const int* d_tokens,
+                       int rows, int hidden, int vocab, float* out, ptm_stream_t stream);
+/* Row r (position pos0 + r): per-head RMSNorm (norm weights may both be NULL) + NeoX RoPE in place on
+ * Q [rows][n_heads*head_dim] and K [rows][kv_dim], K and V rows appended to the caches.  The row-batched form of
+ * ptm_qknorm_rope_kvwrite (launch_fused_qknorm_rope_kvwrite, CUDAOps.h:563-570). */
+int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
+                                 void* K_cache, void* V_cache, const float* rope_table, int rows, int n_heads,
+                                 int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float eps, int add_one,
+                                 int kv_fp16, ptm_stream_t stream);
+/* Causal GQA attention of prompt row r over cache positions [0, pos0 + r] (the rows' own K/V already appended);
+ * O [rows][n_heads*head_dim].  launch_causal_attention (gguf_model.h:7400; CUDAInference.cu:202-315). */
+int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cache, float* O, int rows, int n_heads,
+                          int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float scale, int kv_fp16,
+                          ptm_stream_t stream);
 
 /* ---- batch-1 decode runtime (GGUFModel::forward_decode, gguf_model.h:2575-3113) --- */
 typedef struct {
@@ -258,6 +279,13 @@ int ptm_decode_set_past_len(ptm_decoder* d, int64_t past_len);
 int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token);
 /* n greedy steps feeding each output back in, without host round trips between tokens:
  * tokens_out[n] (host). */
+/* Prefill: run n prompt tokens (host array) through the model at once, append their K/V rows at positions
+ * past_len .. past_len + n - 1 and return the greedy token that follows the prompt; logits of the last
+ * prompt token are left for ptm_decode_logits.  Rows go through the layers in chunks of chunk_rows
+ * (<= 0: 512) with the fast quantised GEMM, row-batched QK-norm + RoPE + KV append and causal attention.
+ * The counterpart of GGUFModel::forward(tokens, use_cache = true) (gguf_model.h:2510-2571); row m equals
+ * a decode step of token m up to the fp16 rounding of the GEMM operands.  Allocates its scratch on first use. */
+int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_rows, int64_t* next_token);
 int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_out);
 /* Device pointers to the last step's logits [vocab] and final-normed hidden [hidden]. */
 const float* ptm_decode_logits(ptm_decoder* d);

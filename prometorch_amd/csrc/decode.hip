@@ -27,6 +27,8 @@ void q6k_init_attributes();
 int q6k_gemv_argmax_impl(const void* W, const float* x, const float* gamma, float eps, int add_one, float* xn_out,
                          float* logits, int K, int N, int64_t stride, int64_t* out_index, void* workspace,
                          const ArgmaxAdvance adv, hipStream_t s);
+int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
+                   int64_t stride, void* workspace, bool accumulate, hipStream_t s);
 int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const int* N4, int64_t stride4,
                        const void* W6, float* y6, int N6, int64_t stride6, const float* x, const float* gamma,
                        float eps, int add_one, int K, hipStream_t s);
@@ -71,6 +73,13 @@ struct ptm_decoder {
     int64_t* h_pinned = nullptr;  // [max_seq] pinned host staging for token ids
     int64_t past_len = 0;
     int status = PTM_OK;
+    // prefill scratch for up to pf_rows prompt rows at a time (allocated on the first prefill)
+    void* pf_slab = nullptr;
+    int pf_rows = 0;
+    float *pf_x = nullptr, *pf_xn = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_attn = nullptr,
+          *pf_gate = nullptr, *pf_up = nullptr;
+    void* pf_ws = nullptr;
+    int* pf_tokens = nullptr;
 };
 
 static int qw_check(const ptm_qweight& w, int rows, int cols) {
@@ -157,6 +166,66 @@ static int enqueue_step(ptm_decoder* d) {
 #undef PTM_TRY
 }
 
+// ---- prefill: M prompt rows through the layers at once (reference: GGUFModel::forward with use_cache,
+// torch/io/gguf_model.h:2510-2571 and transformer_layer :7300-7460) -------------------------------------------
+static int prefill_alloc(ptm_decoder* d, int rows) {
+    if (d->pf_rows >= rows) return PTM_OK;
+    if (d->pf_slab) { (void)hipFree(d->pf_slab); d->pf_slab = nullptr; d->pf_rows = 0; }
+    const ptm_decode_config& c = d->cfg;
+    const size_t H = c.hidden, qd = (size_t)c.n_heads * c.head_dim, kvd = (size_t)c.n_kv_heads * c.head_dim, I = c.inter;
+    const size_t kmax = H > I ? (H > qd ? H : qd) : (I > qd ? I : qd);
+    auto up = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
+    const size_t R = (size_t)rows;
+    const size_t o_x = take(4 * R * H), o_xn = take(4 * R * H), o_q = take(4 * R * qd), o_k = take(4 * R * kvd),
+                 o_v = take(4 * R * kvd), o_attn = take(4 * R * qd), o_gate = take(4 * R * I), o_up = take(4 * R * I),
+                 o_ws = take((size_t)ptm_qgemm_f16_workspace_bytes(rows, (int)kmax)), o_tok = take(4 * R);
+    const int rc = hip_status(hipMalloc(&d->pf_slab, off));
+    if (rc != PTM_OK) return rc;
+    uint8_t* b = static_cast<uint8_t*>(d->pf_slab);
+    d->pf_x = (float*)(b + o_x); d->pf_xn = (float*)(b + o_xn); d->pf_q = (float*)(b + o_q); d->pf_k = (float*)(b + o_k);
+    d->pf_v = (float*)(b + o_v); d->pf_attn = (float*)(b + o_attn); d->pf_gate = (float*)(b + o_gate);
+    d->pf_up = (float*)(b + o_up); d->pf_ws = b + o_ws; d->pf_tokens = (int*)(b + o_tok);
+    d->pf_rows = rows;
+    return PTM_OK;
+}
+
+// rows [0, M) of one chunk at positions pos0 .. pos0 + M - 1; leaves the residual rows in pf_x
+static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t pos0) {
+    const ptm_decode_config& c = d->cfg;
+    hipStream_t s = d->stream;
+    const int H = c.hidden, hd = c.head_dim, qd = c.n_heads * hd, kvd = c.n_kv_heads * hd, I = c.inter;
+    int rc;
+#define PTM_TRY(call) do { rc = (call); if (rc != PTM_OK) return rc; } while (0)
+    PTM_TRY(hip_status(hipMemcpyAsync(d->pf_tokens, tokens_host, 4 * (size_t)M, hipMemcpyHostToDevice, s)));
+    PTM_TRY(ptm_embedding_rows(c.embedding_f32, c.embedding_f32 ? nullptr : c.lm_head.data, c.lm_head.row_stride_bytes,
+                               d->pf_tokens, M, H, c.vocab, d->pf_x, s));
+    auto gemm = [&](const ptm_qweight& w, const float* X, float* Y, bool acc) {
+        return qgemm_f16_impl(w.ggml_type, w.data, X, true, Y, M, w.cols, w.rows, w.row_stride_bytes, d->pf_ws, acc, s);
+    };
+    for (int li = 0; li < c.n_layers; ++li) {
+        const ptm_layer& L = d->layers[li];
+        PTM_TRY(ptm_rms_norm(d->pf_x, L.attn_norm, d->pf_xn, M, H, c.rms_eps, 0, nullptr, s));
+        PTM_TRY(gemm(L.q, d->pf_xn, d->pf_q, false));
+        PTM_TRY(gemm(L.k, d->pf_xn, d->pf_k, false));
+        PTM_TRY(gemm(L.v, d->pf_xn, d->pf_v, false));
+        PTM_TRY(ptm_qknorm_rope_kvwrite_rows(d->pf_q, d->pf_k, d->pf_v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->rope, M,
+                                             c.n_heads, c.n_kv_heads, hd, pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, s));
+        PTM_TRY(ptm_prefill_attention(d->pf_q, L.k_cache, L.v_cache, d->pf_attn, M, c.n_heads, c.n_kv_heads, hd, pos0,
+                                      c.max_seq, 1.0f / sqrtf((float)hd), c.kv_fp16, s));
+        PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true));  // x += attn . Wo^T
+        PTM_TRY(ptm_rms_norm(d->pf_x, L.ffn_norm, d->pf_xn, M, H, c.rms_eps, 0, nullptr, s));
+        PTM_TRY(gemm(L.gate, d->pf_xn, d->pf_gate, false));
+        PTM_TRY(gemm(L.up, d->pf_xn, d->pf_up, false));
+        PTM_TRY(ptm_silu_mul(d->pf_gate, d->pf_up, d->pf_gate, (int64_t)M * I, s));
+        PTM_TRY(gemm(L.down, d->pf_gate, d->pf_x, true));  // x += act . Wdown^T
+    }
+    (void)qd; (void)kvd;
+    return PTM_OK;
+#undef PTM_TRY
+}
+
 extern "C" {
 
 int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
@@ -230,6 +299,7 @@ void ptm_decode_destroy(ptm_decoder* d) {
     if (d->exec) (void)hipGraphExecDestroy(d->exec);
     if (d->graph) (void)hipGraphDestroy(d->graph);
     if (d->h_pinned) (void)hipHostFree(d->h_pinned);
+    if (d->pf_slab) (void)hipFree(d->pf_slab);
     if (d->slab) (void)hipFree(d->slab);
     if (d->stream) (void)hipStreamDestroy(d->stream);
     delete d;
@@ -279,6 +349,53 @@ static int run_steps(ptm_decoder* d, int token, int n) {
     if ((rc = hip_status(hipMemcpyAsync(d->h_pinned, d->d_tokens, 8 * (size_t)n, hipMemcpyDeviceToHost, s))) != PTM_OK) return d->status = rc;
     if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return d->status = rc;
     d->past_len += n;
+    return PTM_OK;
+}
+
+int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_rows, int64_t* next_token) {
+    if (!d || !tokens || !next_token) return PTM_E_NULL;
+    if (d->status != PTM_OK) return PTM_E_STATE;
+    if (n <= 0) return PTM_E_SHAPE;
+    if (d->past_len + n > d->cfg.max_seq) return PTM_E_RANGE;  // KV cache would overflow
+    for (int i = 0; i < n; ++i)
+        if (tokens[i] < 0 || tokens[i] >= d->cfg.vocab) return PTM_E_RANGE;
+    const ptm_decode_config& c = d->cfg;
+    if (chunk_rows <= 0) chunk_rows = 512;
+    if (chunk_rows > n) chunk_rows = n;
+    int rc = prefill_alloc(d, chunk_rows);
+    if (rc != PTM_OK) return rc;
+    hipStream_t s = d->stream;
+    int last_rows = 0;
+    for (int done = 0; done < n; done += last_rows) {
+        last_rows = n - done < chunk_rows ? n - done : chunk_rows;
+        if ((rc = prefill_chunk(d, tokens + done, last_rows, d->past_len + done)) != PTM_OK) return d->status = rc;
+    }
+    // only the last row is projected to logits (gguf_model.h:2551-2559): hand it to the decode tail, with the device-side
+    // position set so that the tail's bookkeeping leaves it at past_len + n
+    if ((rc = hip_status(hipMemcpyAsync(d->x, d->pf_x + (size_t)(last_rows - 1) * c.hidden, 4 * (size_t)c.hidden,
+                                        hipMemcpyDeviceToDevice, s))) != PTM_OK) return d->status = rc;
+    hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, s, d->d_token, (int)tokens[n - 1], d->d_past,
+                       d->past_len + n - 1, d->d_step);
+    if ((rc = launch_status()) != PTM_OK) return d->status = rc;
+    if (c.lm_head.ggml_type == PTM_TYPE_Q6_K) {
+        rc = q6k_gemv_argmax_impl(c.lm_head.data, d->x, c.out_norm, c.rms_eps, 0, d->xn, d->logits, c.hidden, c.vocab,
+                                  c.lm_head.row_stride_bytes, d->d_next, d->amax_ws,
+                                  ArgmaxAdvance{d->d_token, d->d_past, d->d_step, d->d_tokens, c.max_seq}, s);
+    } else {
+        rc = ptm_rms_norm(d->x, c.out_norm, d->xn, 1, c.hidden, c.rms_eps, 0, nullptr, s);
+        if (rc == PTM_OK) rc = gemv_any(c.lm_head, d->xn, d->logits, false, s);
+        if (rc == PTM_OK) rc = ptm_argmax(d->logits, d->d_next, c.vocab, s);
+        if (rc == PTM_OK) {
+            hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->d_next, d->d_token, d->d_past, d->d_step,
+                               d->d_tokens, c.max_seq);
+            rc = launch_status();
+        }
+    }
+    if (rc != PTM_OK) return d->status = rc;
+    if ((rc = hip_status(hipMemcpyAsync(d->h_pinned, d->d_tokens, 8, hipMemcpyDeviceToHost, s))) != PTM_OK) return d->status = rc;
+    if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return d->status = rc;
+    d->past_len += n;
+    *next_token = d->h_pinned[0];
     return PTM_OK;
 }
 

@@ -1,0 +1,280 @@
+// Prefill of M prompt tokens at once: the row-batched counterparts of the decode-step glue.
+//
+// The reference's prefill (GGUFModel::forward(tokens, use_cache), torch/io/gguf_model.h:2510-2571, layer body
+// transformer_layer :7300-7460) runs the layer
+// over all prompt rows: RMSNorm per row, matmul_q per projection, per-head QK-norm + RoPE at each row's position,
+// KV append, causal attention, residual adds.  Row m of the result is what M single-token decode steps give for
+// token m (same formulas as the decode kernels; positions past + m), so parity is checked against the CPU oracle
+// stepping the prompt token by token.
+//   embedding_rows        one embedding row per prompt token (fp32 table, or Q6_K rows dequantised on the fly)
+//   qknorm_rope_kv_rows   per (row, head): RMSNorm over the head, NeoX rotation at position pos0 + row; K and V rows
+//                         are appended to the cache (fp16 or fp32)
+//   prefill_attn          causal GQA attention of row m over cache positions [0, pos0 + m]: one wave per (row, kv
+//                         head) serves the G query heads; every lane group keeps its own online-softmax state over
+//                         the positions it visits (no cross-lane traffic inside the loop), merged once at the end
+#include "ptm_common.h"
+
+namespace ptm {
+
+__device__ __forceinline__ float pf_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
+// Q6_K element e (0..255) of a block (reference: dequantize_q6_k, torch/io/gguf_dequant.h:395-430)
+__device__ __forceinline__ float pf_q6k_elem(const uint8_t* blk, int e) {
+    const int half = e >> 7, r = e & 127, grp = r >> 5, l = r & 31;
+    const uint32_t ql = blk[64 * half + 32 * (grp & 1) + l], qh = blk[128 + 32 * half + l];
+    const int q = (int)(((ql >> (4 * (grp >> 1))) & 0xfu) | (((qh >> (2 * grp)) & 3u) << 4)) - 32;
+    const float d = h2f(reinterpret_cast<const u16_a2*>(blk + 208)->v);
+    const int sc = (int)(int8_t)blk[192 + 8 * half + 2 * grp + (l >> 4)];
+    return d * (float)sc * (float)q;
+}
+
+__global__ __launch_bounds__(256) void embedding_rows_kernel(const float* __restrict__ table_f32,
+                                                             const uint8_t* __restrict__ table_q6k, int64_t stride,
+                                                             const int* __restrict__ tokens, int hidden, int vocab,
+                                                             float* __restrict__ out) {
+    const int m = blockIdx.y;
+    int tok = tokens[m];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);  // ids are validated on the host; never read outside the table
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= hidden) return;
+    float v;
+    if (table_f32) v = table_f32[(int64_t)tok * hidden + i];
+    else v = pf_q6k_elem(table_q6k + (int64_t)tok * stride + (int64_t)(i >> 8) * 210, i & 255);
+    out[(int64_t)m * hidden + i] = v;
+}
+
+// grid (rows, n_heads + n_kv_heads), one wave; lane t owns the rotation pair (t, t + head_dim/2)
+template <bool KV16>
+__global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restrict__ Q, float* __restrict__ K,
+                                                                 const float* __restrict__ V, const float* __restrict__ qw,
+                                                                 const float* __restrict__ kw, void* __restrict__ Kc,
+                                                                 void* __restrict__ Vc, const float* __restrict__ rope,
+                                                                 int n_heads, int n_kv_heads, int head_dim, int64_t pos0,
+                                                                 float eps, int add_one) {
+    const int m = blockIdx.x, hb = blockIdx.y;
+    const bool is_k = hb >= n_heads;
+    const int h = is_k ? hb - n_heads : hb;
+    const int64_t pos = pos0 + m;
+    const int kv_dim = n_kv_heads * head_dim;
+    float* vec = is_k ? K + (int64_t)m * kv_dim + (int64_t)h * head_dim
+                      : Q + ((int64_t)m * n_heads + h) * head_dim;
+    const float* nw = is_k ? kw : qw;
+    const int half = head_dim / 2, t = threadIdx.x;
+    const bool on = t < half;
+    float x0 = on ? vec[t] : 0.0f, x1 = on ? vec[t + half] : 0.0f;
+    if (nw) {
+        float ss = fmaf(x0, x0, 0.0f);
+        ss = fmaf(x1, x1, ss);
+        ss = sum64(ss);
+        const float rs = 1.0f / sqrtf(ss / (float)head_dim + eps);
+        const float one = add_one ? 1.0f : 0.0f;
+        if (on) {
+            x0 = x0 * rs * (nw[t] + one);
+            x1 = x1 * rs * (nw[t + half] + one);
+        }
+    }
+    if (!on) return;
+    const float* cs = rope + pos * head_dim;
+    const float c = cs[t], s = cs[half + t];
+    const float r0 = fmaf(x0, c, -(x1 * s)), r1 = fmaf(x0, s, x1 * c);  // hot_loops.cpp:2035-2061
+    vec[t] = r0;
+    vec[t + half] = r1;
+    if (is_k) {
+        const int64_t off = pos * kv_dim + (int64_t)h * head_dim;
+        const float v0 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t], v1 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t + half];
+        if constexpr (KV16) {
+            __half* kc = static_cast<__half*>(Kc) + off;
+            __half* vc = static_cast<__half*>(Vc) + off;
+            kc[t] = __float2half_rn(r0);
+            kc[t + half] = __float2half_rn(r1);
+            vc[t] = __float2half_rn(v0);
+            vc[t + half] = __float2half_rn(v1);
+        } else {
+            float* kc = static_cast<float*>(Kc) + off;
+            float* vc = static_cast<float*>(Vc) + off;
+            kc[t] = r0;
+            kc[t + half] = r1;
+            vc[t] = v0;
+            vc[t + half] = v1;
+        }
+    }
+}
+
+template <bool KV16>
+__device__ __forceinline__ void pf_load8(const void* base, int64_t elem_off, float (&o)[8]) {
+    if constexpr (KV16) {
+        const uint4 r = *reinterpret_cast<const uint4*>(static_cast<const __half*>(base) + elem_off);
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[2 * i] = h2f(w[i]);
+            o[2 * i + 1] = h2f(w[i] >> 16);
+        }
+    } else {
+        const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(base) + elem_off);
+        const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(base) + elem_off + 4);
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+        o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    }
+}
+
+// grid (ceil(rows / 4), n_kv_heads), 4 waves = 4 consecutive rows of one kv head
+template <bool KV16, int HD, int G>
+__global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restrict__ Q, const void* __restrict__ Kc,
+                                                           const void* __restrict__ Vc, float* __restrict__ O, int rows,
+                                                           int n_heads, int n_kv_heads, int64_t pos0, float scale) {
+    constexpr int LPP = HD / 8, PPW = 64 / LPP;  // lanes per position, positions per wave and pass
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = blockIdx.x * 4 + wave, kvh = blockIdx.y;
+    if (m >= rows) return;  // wave-uniform; no barriers below
+    const int dl = lane % LPP, pl = lane / LPP;
+    const int kv_dim = n_kv_heads * HD;
+    const int64_t col = (int64_t)kvh * HD + dl * 8;
+    const int64_t limit = pos0 + m;  // last position this row may attend to (itself)
+
+    float q[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const float* src = Q + ((int64_t)m * n_heads + kvh * G + g) * HD + dl * 8;
+        const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
+        q[g][0] = a.x; q[g][1] = a.y; q[g][2] = a.z; q[g][3] = a.w;
+        q[g][4] = b.x; q[g][5] = b.y; q[g][6] = b.z; q[g][7] = b.w;
+    }
+    float mrun[G], lsum[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        mrun[g] = -INFINITY;
+        lsum[g] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
+    }
+    const int64_t n_pass = limit / PPW + 1;
+    float kn[8], vn[8];
+    {
+        const int64_t tc = pl <= limit ? pl : limit;
+        pf_load8<KV16>(Kc, tc * kv_dim + col, kn);
+        pf_load8<KV16>(Vc, tc * kv_dim + col, vn);
+    }
+    for (int64_t pass = 0; pass < n_pass; ++pass) {
+        float k[8], v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { k[i] = kn[i]; v[i] = vn[i]; }
+        const int64_t t = pass * PPW + pl;
+        if (pass + 1 < n_pass) {  // next pass's rows are requested before this pass's arithmetic
+            const int64_t tn = t + PPW;
+            const int64_t tc = tn <= limit ? tn : limit;
+            pf_load8<KV16>(Kc, tc * kv_dim + col, kn);
+            pf_load8<KV16>(Vc, tc * kv_dim + col, vn);
+        }
+        const bool valid = t <= limit;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float d = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], k[i], d);
+            d = (LPP == 16) ? sum16(d) : sum8(d);
+            const float s = valid ? d * scale : -INFINITY;
+            const float mnew = fmaxf(mrun[g], s);
+            const float muse = mnew == -INFINITY ? 0.0f : mnew;
+            const float corr = pf_exp(mrun[g] - muse);  // -inf -> 0 on the first valid position
+            const float p = pf_exp(s - muse);
+            lsum[g] = fmaf(lsum[g], corr, p);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(acc[g][i], corr, p * v[i]);
+            mrun[g] = mnew;
+        }
+    }
+    // merge the PPW position slots of the wave (lanes with equal dl)
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float M = mrun[g];
+        for (int off = LPP; off < 64; off <<= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+        const float w = pf_exp(mrun[g] - M);  // M is finite: position 0 is always valid for slot 0
+        float l = lsum[g] * w;
+        for (int off = LPP; off < 64; off <<= 1) l += __shfl_xor(l, off, 64);
+        const float inv = 1.0f / (l + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float a = acc[g][i] * w;
+            for (int off = LPP; off < 64; off <<= 1) a += __shfl_xor(a, off, 64);
+            acc[g][i] = a * inv;
+        }
+        if (pl == 0) {
+            float* dst = O + ((int64_t)m * n_heads + kvh * G + g) * HD + dl * 8;
+            *reinterpret_cast<float4*>(dst) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+            *reinterpret_cast<float4*>(dst + 4) = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
+        }
+    }
+}
+
+template <bool KV16, int HD>
+static int prefill_attn_launch(int G, dim3 grid, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* O,
+                               int rows, int n_heads, int n_kv_heads, int64_t pos0, float scale) {
+#define PTM_PA(GG) hipLaunchKernelGGL((prefill_attn_kernel<KV16, HD, GG>), grid, dim3(256), 0, s, Q, Kc, Vc, O, rows, n_heads, n_kv_heads, pos0, scale)
+    switch (G) {
+        case 1: PTM_PA(1); break;
+        case 2: PTM_PA(2); break;
+        case 4: PTM_PA(4); break;
+        case 8: PTM_PA(8); break;
+        default: return PTM_E_UNSUPPORTED;
+    }
+#undef PTM_PA
+    return launch_status();
+}
+
+}  // namespace ptm
+
+using namespace ptm;
+
+extern "C" {
+
+int ptm_embedding_rows(const float* table_f32, const void* table_q6k, int64_t q6k_row_stride_bytes, const int* d_tokens,
+                       int rows, int hidden, int vocab, float* out, ptm_stream_t stream) {
+    if ((!table_f32 && !table_q6k) || !d_tokens || !out) return PTM_E_NULL;
+    if (rows <= 0 || hidden <= 0 || vocab <= 0 || rows > 65535) return PTM_E_SHAPE;
+    if (!table_f32 && ((hidden % 256) != 0 || q6k_row_stride_bytes < (int64_t)(hidden / 256) * 210)) return PTM_E_SHAPE;
+    hipLaunchKernelGGL(embedding_rows_kernel, dim3((hidden + 255) / 256, rows), dim3(256), 0, as_stream(stream), table_f32,
+                       static_cast<const uint8_t*>(table_q6k), q6k_row_stride_bytes, d_tokens, hidden, vocab, out);
+    return launch_status();
+}
+
+int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
+                                 void* K_cache, void* V_cache, const float* rope_table, int rows, int n_heads,
+                                 int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float eps, int add_one,
+                                 int kv_fp16, ptm_stream_t stream) {
+    if (!Q || !K || !V || !K_cache || !V_cache || !rope_table) return PTM_E_NULL;
+    if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
+    if (rows <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || head_dim <= 0 || (head_dim & 1) || head_dim > 128)
+        return PTM_E_SHAPE;
+    if (pos0 < 0 || pos0 + rows > max_seq) return PTM_E_RANGE;  // never write outside the cache
+    if (n_heads + n_kv_heads > 65535) return PTM_E_UNSUPPORTED;
+    const dim3 grid(rows, n_heads + n_kv_heads);
+    if (kv_fp16)
+        hipLaunchKernelGGL(qknorm_rope_kv_rows_kernel<true>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
+                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one);
+    else
+        hipLaunchKernelGGL(qknorm_rope_kv_rows_kernel<false>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
+                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one);
+    return launch_status();
+}
+
+int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cache, float* O, int rows, int n_heads,
+                          int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float scale, int kv_fp16,
+                          ptm_stream_t stream) {
+    if (!Q || !K_cache || !V_cache || !O) return PTM_E_NULL;
+    if (rows <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
+    if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
+    if (pos0 < 0 || pos0 + rows > max_seq) return PTM_E_RANGE;
+    if (!aligned16(Q) || !aligned16(K_cache) || !aligned16(V_cache) || !aligned16(O)) return PTM_E_ALIGN;
+    if (n_kv_heads > 65535) return PTM_E_UNSUPPORTED;
+    const int G = n_heads / n_kv_heads;
+    const dim3 grid((rows + 3) / 4, n_kv_heads);
+    hipStream_t s = as_stream(stream);
+    if (kv_fp16)
+        return head_dim == 128 ? prefill_attn_launch<true, 128>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
+                               : prefill_attn_launch<true, 64>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
+    return head_dim == 128 ? prefill_attn_launch<false, 128>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
+                           : prefill_attn_launch<false, 64>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
+}
+
+}  // extern "C"

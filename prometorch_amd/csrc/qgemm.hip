@@ -285,11 +285,22 @@ enum { QF_TM = 128, QF_TN = 256, QF_PITCH = 528 };
 
 __host__ __device__ inline int qf_mpad(int M) { return (M + QF_TM - 1) / QF_TM * QF_TM; }
 
-// rows of X (bf16) -> fp16 rows Xh[Mpad][K] (Q8ROUND: first rounded to the reference's Q8 values d*q per block of
+// rows of X (bf16, or fp32 when XF32) -> fp16 rows Xh[Mpad][K] (Q8ROUND: first rounded to the reference's Q8 values d*q per block of
 // 32, the rounding its Q4_K GEMV applies; otherwise the bf16 value itself, as its Q6_K GEMV uses), divided by a
 // power of two per row (returned in rowscale) so that fp16 cannot overflow
-template <bool Q8ROUND>
-__global__ __launch_bounds__(256) void qgemm_prepare_rows_f16_kernel(const uint16_t* __restrict__ X, _Float16* __restrict__ Xh,
+template <bool XF32>
+__device__ __forceinline__ float4 load_x4(const void* row, int i) {
+    if constexpr (XF32) {
+        return reinterpret_cast<const float4*>(row)[i];
+    } else {
+        const uint2 raw = reinterpret_cast<const uint2*>(row)[i];
+        return make_float4(bf16_to_f32(raw.x & 0xffffu), bf16_to_f32(raw.x >> 16), bf16_to_f32(raw.y & 0xffffu),
+                           bf16_to_f32(raw.y >> 16));
+    }
+}
+
+template <bool Q8ROUND, bool XF32>
+__global__ __launch_bounds__(256) void qgemm_prepare_rows_f16_kernel(const void* __restrict__ X, _Float16* __restrict__ Xh,
                                                                      float* __restrict__ rowscale, int M, int K) {
     __shared__ float red[4];
     const int m = blockIdx.x, tid = threadIdx.x;
@@ -299,12 +310,11 @@ __global__ __launch_bounds__(256) void qgemm_prepare_rows_f16_kernel(const uint1
         for (int i = tid; i < n4; i += 256) reinterpret_cast<uint2*>(dst)[i] = make_uint2(0, 0);
         return;
     }
-    const uint2* src = reinterpret_cast<const uint2*>(X + (int64_t)m * K);
+    const void* src = static_cast<const uint8_t*>(X) + (int64_t)m * K * (XF32 ? 4 : 2);
     float amax = 0.0f;
     for (int i = tid; i < n4; i += 256) {
-        const uint2 raw = src[i];
-        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(bf16_to_f32(raw.x & 0xffffu)), fabsf(bf16_to_f32(raw.x >> 16))),
-                                 fmaxf(fabsf(bf16_to_f32(raw.y & 0xffffu)), fabsf(bf16_to_f32(raw.y >> 16)))));
+        const float4 v = load_x4<XF32>(src, i);
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
     }
     amax = max64(amax);
     if ((tid & 63) == 0) red[tid >> 6] = amax;
@@ -316,12 +326,7 @@ __global__ __launch_bounds__(256) void qgemm_prepare_rows_f16_kernel(const uint1
     const float down = ldexpf(1.0f, -e);
     if (tid == 0) rowscale[m] = ldexpf(1.0f, e);
     for (int i = tid; i < n4; i += 256) {  // K % 256 == 0: whole waves, aligned groups of 8 lanes = one Q8 block
-        const uint2 raw = src[i];
-        float4 v;
-        v.x = bf16_to_f32(raw.x & 0xffffu);
-        v.y = bf16_to_f32(raw.x >> 16);
-        v.z = bf16_to_f32(raw.y & 0xffffu);
-        v.w = bf16_to_f32(raw.y >> 16);
+        float4 v = load_x4<XF32>(src, i);
         if constexpr (Q8ROUND) {
             float d, sm;
             const uint32_t pk = q8_quantize4(v, d, sm);
@@ -421,7 +426,8 @@ struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh
 // re-fetches the last tile into the idle buffer: no conditionals in the steady-state loop.)
 template <typename Tile>
 __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
-                                                        const float* __restrict__ rowscale, float* Y, int M, int K, int N) {
+                                                        const float* __restrict__ rowscale, float* Y, int M, int K, int N,
+                                                        int accumulate) {
     // W and Xh are deliberately not __restrict__: loads through a restrict pointer may be moved across the
     // compiler fences below, and the prefetch distance of this loop depends on those fences
     extern __shared__ __align__(16) uint8_t s_a[];  // [2][QF_TM * QF_PITCH]
@@ -551,7 +557,11 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
                     const int n = n_base + 32 * t + j;
-                    if (n < N) Y[(int64_t)m * N + n] = acc[mt][t][r] * rs;
+                    if (n < N) {
+                        float* y = Y + (int64_t)m * N + n;
+                        const float v = acc[mt][t][r] * rs;
+                        *y = accumulate ? *y + v : v;
+                    }
                 }
             }
         }
@@ -564,6 +574,44 @@ static int qgemm_check(const void* W, const void* X, const void* Y, int M, int K
     if (!aligned16(X) || (reinterpret_cast<uintptr_t>(Y) & 3u)) return PTM_E_ALIGN;
     if ((int64_t)qg_mpad(M) / QG_MCHUNK > 65535) return PTM_E_UNSUPPORTED;
     return PTM_OK;
+}
+
+// Y (+)= X . W^T with X bf16 or fp32 rows; shared by the C entry points and the prefill runtime.
+int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
+                   int64_t stride, void* workspace, bool accumulate, hipStream_t s) {
+    if (ggml_type != PTM_TYPE_Q4_K && ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
+    const int blk = ggml_type == PTM_TYPE_Q4_K ? 144 : 210;
+    const int rc = qgemm_check(W, X, Y, M, K, N, stride, blk);
+    if (rc != PTM_OK) return rc;
+    if (!workspace) return PTM_E_NULL;
+    if (!aligned16(workspace)) return PTM_E_ALIGN;
+    if (ggml_type == PTM_TYPE_Q4_K ? (!aligned16(W) || (stride & 15)) : ((stride & 1) || (reinterpret_cast<uintptr_t>(W) & 1u)))
+        return PTM_E_ALIGN;
+    const int mp = qf_mpad(M);
+    if (mp / QF_TM > 65535) return PTM_E_UNSUPPORTED;
+    _Float16* Xh = static_cast<_Float16*>(workspace);
+    float* rowscale = reinterpret_cast<float*>(Xh + (int64_t)mp * K);
+    const size_t lds = 2 * (size_t)QF_TM * QF_PITCH;  // 132 KB: above the default 64 KB cap of dynamic LDS
+    static bool raised = false;
+    if (!raised) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        raised = true;
+    }
+    const dim3 grid((N + QF_TN - 1) / QF_TN, mp / QF_TM);
+    const int acc = accumulate ? 1 : 0;
+    if (ggml_type == PTM_TYPE_Q4_K) {
+        if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
+        else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
+        hipLaunchKernelGGL(qgemm_f16_kernel<Q4Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
+                           rowscale, Y, M, K, N, acc);
+    } else {
+        if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
+        else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
+        hipLaunchKernelGGL(qgemm_f16_kernel<Q6Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
+                           rowscale, Y, M, K, N, acc);
+    }
+    return launch_status();
 }
 
 }  // namespace ptm
@@ -619,39 +667,12 @@ int64_t ptm_qgemm_f16_workspace_bytes(int M, int K) {
 
 int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* Y, int M, int K, int N, int64_t stride,
                   void* workspace, ptm_stream_t stream) {
-    if (ggml_type != PTM_TYPE_Q4_K && ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
-    const int blk = ggml_type == PTM_TYPE_Q4_K ? 144 : 210;
-    const int rc = qgemm_check(W, X_bf16, Y, M, K, N, stride, blk);
-    if (rc != PTM_OK) return rc;
-    if (!workspace) return PTM_E_NULL;
-    if (!aligned16(workspace)) return PTM_E_ALIGN;
-    if (ggml_type == PTM_TYPE_Q4_K ? (!aligned16(W) || (stride & 15)) : ((stride & 1) || (reinterpret_cast<uintptr_t>(W) & 1u)))
-        return PTM_E_ALIGN;
-    const int mp = qf_mpad(M);
-    if (mp / QF_TM > 65535) return PTM_E_UNSUPPORTED;
-    _Float16* Xh = static_cast<_Float16*>(workspace);
-    float* rowscale = reinterpret_cast<float*>(Xh + (int64_t)mp * K);
-    hipStream_t s = as_stream(stream);
-    const size_t lds = 2 * (size_t)QF_TM * QF_PITCH;  // 132 KB: above the default 64 KB cap of dynamic LDS
-    static bool raised = false;
-    if (!raised) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        raised = true;
-    }
-    const dim3 grid((N + QF_TN - 1) / QF_TN, mp / QF_TM);
-    if (ggml_type == PTM_TYPE_Q4_K) {
-        hipLaunchKernelGGL(qgemm_prepare_rows_f16_kernel<true>, dim3(mp), dim3(256), 0, s, static_cast<const uint16_t*>(X_bf16),
-                           Xh, rowscale, M, K);
-        hipLaunchKernelGGL(qgemm_f16_kernel<Q4Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
-                           rowscale, Y, M, K, N);
-    } else {
-        hipLaunchKernelGGL(qgemm_prepare_rows_f16_kernel<false>, dim3(mp), dim3(256), 0, s, static_cast<const uint16_t*>(X_bf16),
-                           Xh, rowscale, M, K);
-        hipLaunchKernelGGL(qgemm_f16_kernel<Q6Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
-                           rowscale, Y, M, K, N);
-    }
-    return launch_status();
+    return qgemm_f16_impl(ggml_type, W, X_bf16, false, Y, M, K, N, stride, workspace, false, as_stream(stream));
+}
+
+int ptm_qgemm_f16_f32(uint32_t ggml_type, const void* W, const float* X_f32, float* Y, int M, int K, int N, int64_t stride,
+                      void* workspace, int accumulate, ptm_stream_t stream) {
+    return qgemm_f16_impl(ggml_type, W, X_f32, true, Y, M, K, N, stride, workspace, accumulate != 0, as_stream(stream));
 }
 
 }  // extern "C"

@@ -99,6 +99,15 @@ class Decoder:
         check(self.L.ptm_decode_step(self.h, token, C.byref(out)), "decode_step")
         return out.value
 
+    def prefill(self, tokens, chunk_rows: int = 0) -> int:
+        """Run the prompt through the model in row batches, appending its K/V rows; returns the greedy next token
+        (GGUFModel::forward with use_cache, gguf_model.h:2510-2571)."""
+        n = len(tokens)
+        buf = (C.c_int32 * n)(*[int(t) for t in tokens])
+        out = C.c_int64()
+        check(self.L.ptm_decode_prefill(self.h, buf, n, chunk_rows, C.byref(out)), "decode_prefill")
+        return out.value
+
     def greedy(self, first_token: int, n: int) -> list:
         buf = (C.c_int64 * n)()
         check(self.L.ptm_decode_greedy(self.h, first_token, n, buf), "decode_greedy")

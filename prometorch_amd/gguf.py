@@ -209,6 +209,13 @@ class GGUFModel:
         check(self.L.ptm_decode_step(self.h, token, C.byref(out)), "decode_step")
         return out.value
 
+    def prefill(self, tokens, chunk_rows: int = 0) -> int:
+        n = len(tokens)
+        buf = (C.c_int32 * n)(*[int(t) for t in tokens])
+        out = C.c_int64()
+        check(self.L.ptm_decode_prefill(self.h, buf, n, chunk_rows, C.byref(out)), "decode_prefill")
+        return out.value
+
     def greedy(self, first_token: int, n: int) -> list:
         buf = (C.c_int64 * n)()
         check(self.L.ptm_decode_greedy(self.h, first_token, n, buf), "decode_greedy")

@@ -269,6 +269,33 @@ def matmul_q_f16(quant_type, weights, x_bf16, y, M, K, N, row_stride_bytes, work
                              _ptr(workspace), _stream(stream)), "matmul_q_f16")
 
 
+def matmul_q_f16_f32(quant_type, weights, x_f32, y, M, K, N, row_stride_bytes, workspace, accumulate=False, stream=None):
+    """matmul_q_f16 on fp32 rows of X, optionally Y += result (the prefill's o-proj / down-proj residual adds)."""
+    check(_L().ptm_qgemm_f16_f32(quant_type, _ptr(weights), _ptr(x_f32), _ptr(y), M, K, N, row_stride_bytes,
+                                 _ptr(workspace), int(accumulate), _stream(stream)), "matmul_q_f16_f32")
+
+
+def embedding_rows(table_f32, table_q6k, q6k_row_stride_bytes, d_tokens, rows, hidden, vocab, out, stream=None):
+    """Rows of the token embedding for a batch of token ids (embedding_lookup, gguf_model.h:2513)."""
+    check(_L().ptm_embedding_rows(_ptr(table_f32), _ptr(table_q6k), q6k_row_stride_bytes, _ptr(d_tokens), rows, hidden,
+                                  vocab, _ptr(out), _stream(stream)), "embedding_rows")
+
+
+def qknorm_rope_kvwrite_rows(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, rope, rows, n_heads, n_kv_heads, head_dim,
+                             pos0, max_seq, eps, add_one, kv_fp16, stream=None):
+    """launch_fused_qknorm_rope_kvwrite (CUDAOps.h:563-570) over `rows` prompt rows at positions pos0 + r."""
+    check(_L().ptm_qknorm_rope_kvwrite_rows(_ptr(Q), _ptr(K), _ptr(V), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(K_cache),
+                                            _ptr(V_cache), _ptr(rope), rows, n_heads, n_kv_heads, head_dim, pos0, max_seq,
+                                            eps, int(add_one), int(kv_fp16), _stream(stream)), "qknorm_rope_kvwrite_rows")
+
+
+def prefill_attention(Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, head_dim, pos0, max_seq, scale, kv_fp16,
+                      stream=None):
+    """Causal GQA attention of prompt rows over the cache (launch_causal_attention, gguf_model.h:7400)."""
+    check(_L().ptm_prefill_attention(_ptr(Q), _ptr(K_cache), _ptr(V_cache), _ptr(O), rows, n_heads, n_kv_heads, head_dim,
+                                     pos0, max_seq, scale, int(kv_fp16), _stream(stream)), "prefill_attention")
+
+
 def matmul_q(quant_type, weights, x_bf16, y, M, K, N, row_stride_bytes, workspace, stream=None):
     """Quantised-weight GEMM for M > 1 rows with the GEMV's arithmetic per row (Q4_K: bit-identical rows);
     stands in for the M-GEMV loop of matmul_q (gguf_model.h:7029-7036)."""
