@@ -88,6 +88,7 @@ SIGNATURES = {
     "ptm_decode_step": (i32, [vp, i32, C.POINTER(i64)]),
     "ptm_decode_greedy": (i32, [vp, i32, i32, C.POINTER(i64)]),
     "ptm_decode_prefill": (i32, [vp, C.POINTER(C.c_int32), i32, i32, C.POINTER(i64)]),
+    "ptm_qgemm_f16_f32_workspace_bytes": (i64, [i32, i32, i32]),
     "ptm_qgemm_f16_f32": (i32, [u32, vp, vp, vp, i32, i32, i32, i64, vp, i32, vp]),
     "ptm_embedding_rows": (i32, [vp, vp, i64, vp, i32, i32, i32, vp, vp]),
     "ptm_qknorm_rope_kvwrite_rows": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, i32, vp]),

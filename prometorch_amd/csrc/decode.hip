@@ -28,7 +28,8 @@ int q6k_gemv_argmax_impl(const void* W, const float* x, const float* gamma, floa
                          float* logits, int K, int N, int64_t stride, int64_t* out_index, void* workspace,
                          const ArgmaxAdvance adv, hipStream_t s);
 int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
-                   int64_t stride, void* workspace, bool accumulate, hipStream_t s);
+                   int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, hipStream_t s);
+int qgemm_f16_splits(int N, int K);
 int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const int* N4, int64_t stride4,
                        const void* W6, float* y6, int N6, int64_t stride6, const float* x, const float* gamma,
                        float eps, int add_one, int K, hipStream_t s);
@@ -79,6 +80,8 @@ struct ptm_decoder {
     float *pf_x = nullptr, *pf_xn = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_attn = nullptr,
           *pf_gate = nullptr, *pf_up = nullptr;
     void* pf_ws = nullptr;
+    float* pf_split = nullptr;  // K-split partial sums of the GEMMs
+    size_t pf_split_bytes = 0;
     int* pf_tokens = nullptr;
 };
 
@@ -181,12 +184,21 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
     const size_t o_x = take(4 * R * H), o_xn = take(4 * R * H), o_q = take(4 * R * qd), o_k = take(4 * R * kvd),
                  o_v = take(4 * R * kvd), o_attn = take(4 * R * qd), o_gate = take(4 * R * I), o_up = take(4 * R * I),
                  o_ws = take((size_t)ptm_qgemm_f16_workspace_bytes(rows, (int)kmax)), o_tok = take(4 * R);
+    size_t split_elems = 0;  // widest splits x N over the layer's matrices (all layers have the same shapes)
+    for (const ptm_qweight* w : {&d->layers[0].q, &d->layers[0].k, &d->layers[0].v, &d->layers[0].o, &d->layers[0].gate,
+                                 &d->layers[0].up, &d->layers[0].down}) {
+        const size_t e = (size_t)qgemm_f16_splits(w->rows, w->cols) * w->rows;
+        split_elems = e > split_elems ? e : split_elems;
+    }
+    d->pf_split_bytes = 4 * R * split_elems;
+    const size_t o_split = take(d->pf_split_bytes);
     const int rc = hip_status(hipMalloc(&d->pf_slab, off));
     if (rc != PTM_OK) return rc;
     uint8_t* b = static_cast<uint8_t*>(d->pf_slab);
     d->pf_x = (float*)(b + o_x); d->pf_xn = (float*)(b + o_xn); d->pf_q = (float*)(b + o_q); d->pf_k = (float*)(b + o_k);
     d->pf_v = (float*)(b + o_v); d->pf_attn = (float*)(b + o_attn); d->pf_gate = (float*)(b + o_gate);
     d->pf_up = (float*)(b + o_up); d->pf_ws = b + o_ws; d->pf_tokens = (int*)(b + o_tok);
+    d->pf_split = (float*)(b + o_split);
     d->pf_rows = rows;
     return PTM_OK;
 }
@@ -202,7 +214,8 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
     PTM_TRY(ptm_embedding_rows(c.embedding_f32, c.embedding_f32 ? nullptr : c.lm_head.data, c.lm_head.row_stride_bytes,
                                d->pf_tokens, M, H, c.vocab, d->pf_x, s));
     auto gemm = [&](const ptm_qweight& w, const float* X, float* Y, bool acc) {
-        return qgemm_f16_impl(w.ggml_type, w.data, X, true, Y, M, w.cols, w.rows, w.row_stride_bytes, d->pf_ws, acc, s);
+        return qgemm_f16_impl(w.ggml_type, w.data, X, true, Y, M, w.cols, w.rows, w.row_stride_bytes, d->pf_ws, acc,
+                              d->pf_split, d->pf_split_bytes, s);
     };
     for (int li = 0; li < c.n_layers; ++li) {
         const ptm_layer& L = d->layers[li];

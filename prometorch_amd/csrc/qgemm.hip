@@ -427,7 +427,7 @@ struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh
 template <typename Tile>
 __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
                                                         const float* __restrict__ rowscale, float* Y, int M, int K, int N,
-                                                        int accumulate) {
+                                                        int accumulate, int blocks_per_split, float* partials) {
     // W and Xh are deliberately not __restrict__: loads through a restrict pointer may be moved across the
     // compiler fences below, and the prefetch distance of this loop depends on those fences
     extern __shared__ __align__(16) uint8_t s_a[];  // [2][QF_TM * QF_PITCH]
@@ -435,10 +435,13 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
     const int j = lane & 31, kh = lane >> 5;
     const int m0 = blockIdx.y * QF_TM;
     const int n_base = blockIdx.x * QF_TN + wave * 64;
-    const int nblk = K / 256;
+    // split K: workgroup z of the grid sums super-blocks [blk0, blk0 + nblk) into its own M x N partial
+    const int blk0 = blockIdx.z * blocks_per_split;
+    const int nblk = min(K / 256 - blk0, blocks_per_split);
     const uint8_t* wrow[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) wrow[t] = W + (int64_t)min(n_base + 32 * t + j, N - 1) * stride;
+    for (int t = 0; t < 2; ++t)
+        wrow[t] = W + (int64_t)min(n_base + 32 * t + j, N - 1) * stride + (int64_t)blk0 * Tile::kBlockBytes;
 
     f32x16 acc[4][2];
 #pragma unroll
@@ -451,7 +454,8 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
     // X tile of a block = 128 rows x 512 B = 4096 pieces of 16 B; piece q = 256 i + tid (i = 0..15) is row q / 32, bytes
     // 16 (q % 32): a wave fetches two whole rows per instruction and writes LDS without bank conflicts
     const int64_t x_row_bytes = (int64_t)K * 2;
-    const uint8_t* x_src = reinterpret_cast<const uint8_t*>(Xh) + (int64_t)(m0 + (tid >> 5)) * x_row_bytes + 16 * (tid & 31);
+    const uint8_t* x_src = reinterpret_cast<const uint8_t*>(Xh) + (int64_t)(m0 + (tid >> 5)) * x_row_bytes + 16 * (tid & 31) +
+                           (int64_t)blk0 * 512;
     uint8_t* x_dst = s_a + (tid >> 5) * QF_PITCH + 16 * (tid & 31);
     uint4 re0, re1, re2, ro0, ro1, ro2;  // pieces in flight: fetched at an even / odd step (scalars, not an array: they must stay in registers)
     re0 = re1 = re2 = ro0 = ro1 = ro2 = make_uint4(0, 0, 0, 0);
@@ -558,13 +562,51 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
                 for (int t = 0; t < 2; ++t) {
                     const int n = n_base + 32 * t + j;
                     if (n < N) {
-                        float* y = Y + (int64_t)m * N + n;
                         const float v = acc[mt][t][r] * rs;
-                        *y = accumulate ? *y + v : v;
+                        if (partials) {
+                            partials[((int64_t)blockIdx.z * M + m) * N + n] = v;
+                        } else {
+                            float* y = Y + (int64_t)m * N + n;
+                            *y = accumulate ? *y + v : v;
+                        }
                     }
                 }
             }
         }
+}
+
+// Y (+)= partials[0] + partials[1] + ... in that fixed order (deterministic, unlike atomics)
+__global__ __launch_bounds__(256) void qgemm_split_reduce_kernel(const float* __restrict__ P, int splits, float* __restrict__ Y,
+                                                                 int64_t total, int accumulate) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= total) return;
+    if (i + 4 <= total && (total & 3) == 0) {
+        float4 a = *reinterpret_cast<const float4*>(P + i);
+        for (int z = 1; z < splits; ++z) {
+            const float4 b = *reinterpret_cast<const float4*>(P + z * total + i);
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        }
+        float4* y = reinterpret_cast<float4*>(Y + i);
+        if (accumulate) { const float4 o = *y; a.x += o.x; a.y += o.y; a.z += o.z; a.w += o.w; }
+        *y = a;
+    } else {
+        for (int64_t e = i; e < total && e < i + 4; ++e) {
+            float a = P[e];
+            for (int z = 1; z < splits; ++z) a += P[z * total + e];
+            Y[e] = accumulate ? Y[e] + a : a;
+        }
+    }
+}
+
+// K splits for an N x K weight matrix: enough workgroups to fill the chip when N alone gives few column tiles
+// (a 2560-wide projection is 10 tiles).  Depends on N and K only -- not on M -- so that the summation order of a
+// row does not change with how many rows share the launch.
+int qgemm_f16_splits(int N, int K) {
+    const int ntiles = (N + QF_TN - 1) / QF_TN, nblk = K / 256;
+    int s = 64 / ntiles;  // 4 row tiles (512 rows) x ntiles x s ~ 256 workgroups
+    s = s > 8 ? 8 : s;
+    s = s > nblk / 2 ? nblk / 2 : s;
+    return s < 1 ? 1 : s;
 }
 
 static int qgemm_check(const void* W, const void* X, const void* Y, int M, int K, int N, int64_t stride, int blk_bytes) {
@@ -578,7 +620,7 @@ static int qgemm_check(const void* W, const void* X, const void* Y, int M, int K
 
 // Y (+)= X . W^T with X bf16 or fp32 rows; shared by the C entry points and the prefill runtime.
 int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
-                   int64_t stride, void* workspace, bool accumulate, hipStream_t s) {
+                   int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, hipStream_t s) {
     if (ggml_type != PTM_TYPE_Q4_K && ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
     const int blk = ggml_type == PTM_TYPE_Q4_K ? 144 : 210;
     const int rc = qgemm_check(W, X, Y, M, K, N, stride, blk);
@@ -598,18 +640,29 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         raised = true;
     }
-    const dim3 grid((N + QF_TN - 1) / QF_TN, mp / QF_TM);
+    const int nblk = K / 256;
+    int splits = split_ws ? qgemm_f16_splits(N, K) : 1;
+    while (splits > 1 && (size_t)splits * M * N * sizeof(float) > split_ws_bytes) --splits;
+    const int bps = (nblk + splits - 1) / splits;
+    splits = (nblk + bps - 1) / bps;  // no empty split
+    float* partials = splits > 1 ? split_ws : nullptr;
+    const dim3 grid((N + QF_TN - 1) / QF_TN, mp / QF_TM, splits);
     const int acc = accumulate ? 1 : 0;
     if (ggml_type == PTM_TYPE_Q4_K) {
         if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         hipLaunchKernelGGL(qgemm_f16_kernel<Q4Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
-                           rowscale, Y, M, K, N, acc);
+                           rowscale, Y, M, K, N, acc, bps, partials);
     } else {
         if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         hipLaunchKernelGGL(qgemm_f16_kernel<Q6Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
-                           rowscale, Y, M, K, N, acc);
+                           rowscale, Y, M, K, N, acc, bps, partials);
+    }
+    if (partials) {
+        const int64_t total = (int64_t)M * N;
+        hipLaunchKernelGGL(qgemm_split_reduce_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, partials, splits,
+                           Y, total, acc);
     }
     return launch_status();
 }
@@ -667,12 +720,25 @@ int64_t ptm_qgemm_f16_workspace_bytes(int M, int K) {
 
 int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* Y, int M, int K, int N, int64_t stride,
                   void* workspace, ptm_stream_t stream) {
-    return qgemm_f16_impl(ggml_type, W, X_bf16, false, Y, M, K, N, stride, workspace, false, as_stream(stream));
+    return qgemm_f16_impl(ggml_type, W, X_bf16, false, Y, M, K, N, stride, workspace, false, nullptr, 0, as_stream(stream));
+}
+
+int64_t ptm_qgemm_f16_f32_workspace_bytes(int M, int K, int N) {
+    if (M <= 0 || K <= 0 || N <= 0) return 0;
+    const int64_t base = (ptm_qgemm_f16_workspace_bytes(M, K) + 255) & ~(int64_t)255;
+    const int splits = qgemm_f16_splits(N, K);
+    return base + (splits > 1 ? (int64_t)splits * M * N * 4 : 0);
 }
 
 int ptm_qgemm_f16_f32(uint32_t ggml_type, const void* W, const float* X_f32, float* Y, int M, int K, int N, int64_t stride,
                       void* workspace, int accumulate, ptm_stream_t stream) {
-    return qgemm_f16_impl(ggml_type, W, X_f32, true, Y, M, K, N, stride, workspace, accumulate != 0, as_stream(stream));
+    if (M <= 0 || K <= 0 || N <= 0) return PTM_E_SHAPE;
+    if (!workspace) return PTM_E_NULL;
+    const int64_t base = (ptm_qgemm_f16_workspace_bytes(M, K) + 255) & ~(int64_t)255;
+    const int splits = qgemm_f16_splits(N, K);
+    return qgemm_f16_impl(ggml_type, W, X_f32, true, Y, M, K, N, stride, workspace, accumulate != 0,
+                          splits > 1 ? reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + base) : nullptr,
+                          splits > 1 ? (size_t)splits * M * N * 4 : 0, as_stream(stream));
 }
 
 }  // extern "C"

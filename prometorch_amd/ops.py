@@ -269,6 +269,10 @@ def matmul_q_f16(quant_type, weights, x_bf16, y, M, K, N, row_stride_bytes, work
                              _ptr(workspace), _stream(stream)), "matmul_q_f16")
 
 
+def qgemm_f16_f32_workspace_bytes(M, K, N):
+    return int(_L().ptm_qgemm_f16_f32_workspace_bytes(M, K, N))
+
+
 def matmul_q_f16_f32(quant_type, weights, x_f32, y, M, K, N, row_stride_bytes, workspace, accumulate=False, stream=None):
     """matmul_q_f16 on fp32 rows of X, optionally Y += result (the prefill's o-proj / down-proj residual adds)."""
     check(_L().ptm_qgemm_f16_f32(quant_type, _ptr(weights), _ptr(x_f32), _ptr(y), M, K, N, row_stride_bytes,

@@ -166,14 +166,18 @@ def test_prefill_attention_rejects_bad_shapes(dev):
 
 # ---- matmul on fp32 rows with accumulate -----------------------------------------------------------------------
 @pytest.mark.parametrize("qt", [12, 14])
-def test_qgemm_f16_f32_rows_and_accumulate(dev, po, qt):
-    M, K, N = 70, 1024, 300
-    r = synth.rng_for(65, qt)
+@pytest.mark.parametrize("M,K,N", [(70, 1024, 300),      # 2 column tiles, 4 super-blocks: K split in 2
+                                   (33, 2560, 1024),     # k/v projection of Qwen3-4B: K split in 5
+                                   (130, 4864, 2560),    # down-projection-like: 19 super-blocks in 6 uneven splits
+                                   (5, 256, 48),         # one super-block: no split
+                                   (64, 512, 9728)])     # wide: no split
+def test_qgemm_f16_f32_rows_and_accumulate(dev, po, qt, M, K, N):
+    r = synth.rng_for(65, qt, M, K, N)
     W = synth.make_weight(r, qt, N, K)
     x = r.standard_normal((M, K), dtype=np.float32)
     y0 = r.standard_normal((M, N), dtype=np.float32)
     ref = np.stack([po.gemv(qt, W, x[m]) for m in range(M)])
-    ws = torch.empty(ops.qgemm_f16_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(ops.qgemm_f16_f32_workspace_bytes(M, K, N), dtype=torch.uint8, device="cuda")
     Wd, Xd = cu(W), cu(x)
     Y = torch.full((M, N), 5.0, device="cuda")
     ops.matmul_q_f16_f32(qt, Wd, Xd, Y, M, K, N, W.shape[1], ws)
@@ -183,6 +187,12 @@ def test_qgemm_f16_f32_rows_and_accumulate(dev, po, qt):
     rms = np.sqrt((ref.astype(np.float64) ** 2).mean())
     assert np.abs(Y.cpu().numpy() - ref).max() / rms <= PREFILL_TOL
     assert np.array_equal(bits(Ya.cpu().numpy()), bits(y0 + Y.cpu().numpy()))   # Y += is one fp32 add of the same product
+    # a row's result does not depend on how many rows share the launch (the K split is a function of N and K only)
+    m3 = min(3, M)
+    Y3 = torch.empty((m3, N), device="cuda")
+    ops.matmul_q_f16_f32(qt, Wd, Xd[:m3].contiguous(), Y3, m3, K, N, W.shape[1], ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(Y3.cpu().numpy()), bits(Y[:m3].cpu().numpy()))
 
 
 # ---- whole prefill -------------------------------------------------------------------------------------------------
@@ -279,7 +289,8 @@ def test_prefill_layer_stage_by_stage_on_identical_inputs(dev, po, seeds):
     Kc = torch.zeros(max_seq, kvd, dtype=torch.float16, device="cuda")
     Vc = torch.zeros(max_seq, kvd, dtype=torch.float16, device="cuda")
     Kc[:pos0], Vc[:pos0] = cu(k0), cu(v0)
-    ws = torch.empty(ops.qgemm_f16_workspace_bytes(M, max(H, I, qd)), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(max(ops.qgemm_f16_f32_workspace_bytes(M, k_, n_) for k_, n_ in ((H, qd), (H, kvd), (qd, H), (H, I), (I, H))),
+                     dtype=torch.uint8, device="cuda")
     Wd = {n: cu(Ld[n][1]) for n in ("q", "k", "v", "o", "gate", "up", "down")}
 
     def gemm(name, X, Y, acc=False):
