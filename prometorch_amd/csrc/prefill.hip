@@ -12,9 +12,16 @@
 //   prefill_attn          causal GQA attention of row m over cache positions [0, pos0 + m]: one wave per (row, kv
 //                         head) serves the G query heads; every lane group keeps its own online-softmax state over
 //                         the positions it visits (no cross-lane traffic inside the loop), merged once at the end
+//   prefill_attn_mfma     the same attention on the matrix cores for an fp16 cache and 16 or more rows: a workgroup
+//                         owns one kv head and 128 query vectors (128 / G rows x G heads), walks the cache in tiles
+//                         of 32 positions staged through LDS, S^T = K . Q^T and O^T += V^T . P^T with
+//                         v_mfma_f32_32x32x16_f16, online softmax in the accumulator layout (a lane owns one query
+//                         vector's column).  Q and P are rounded to fp16: ~1e-3 of the output's scale.
 #include "ptm_common.h"
 
 namespace ptm {
+
+enum { PTM_PREFILL_MFMA_MIN_ROWS = 16 };  // fewer rows: the exact fp32 kernel (too few workgroups for the tiled one to pay)
 
 __device__ __forceinline__ float pf_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 
@@ -207,6 +214,178 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restri
     }
 }
 
+// ---- matrix-core version (fp16 cache) ----------------------------------------------------------------------------
+typedef _Float16 pf_h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 pf_h4 __attribute__((ext_vector_type(4)));
+typedef float pf_f16v __attribute__((ext_vector_type(16)));
+
+// v_mfma_f32_32x32x16_f16 operand layout used below: A (32 x 16): lane l holds row l % 32, summation indices
+// 8 (l / 32) + 0..7; B (16 x 32): lane l holds column l % 32, the same indices; C (32 x 32): lane l holds column
+// l % 32, rows 8 (r / 4) + 4 (l / 32) + r % 4 for r = 0..15.  The summation index may be permuted freely as long as A
+// and B agree, which is used twice: the 16 head-dim elements of a step are [16 ks + 8 kh, +8) for lane half kh,
+// and the 16 positions of a P.V step are the ones the lane already holds in its S^T accumulator.
+template <int HD, int G>
+__global__ __launch_bounds__(256) void prefill_attn_mfma_kernel(const float* __restrict__ Q, const __half* __restrict__ Kc,
+                                                                const __half* __restrict__ Vc, float* __restrict__ O, int rows,
+                                                                int n_heads, int n_kv_heads, int64_t pos0, float scale) {
+    constexpr int RPW = 32 / G;        // rows per wave (each with its G heads: 32 query vectors)
+    constexpr int BM = 4 * RPW;        // rows per workgroup
+    constexpr int KS = HD / 16;        // MFMA steps over the head dimension
+    constexpr int DT = HD / 32;        // 32-wide tiles of the output's head dimension
+    constexpr int KP = HD * 2 + 16;    // LDS pitch of a K row (bytes)
+    constexpr int VP = 64 + 8;         // LDS pitch of a V^T row: 32 positions of fp16 + padding
+    constexpr int PCS = 32 * HD / 8 / 256;  // 16-byte pieces of a 32-position tile per thread (1 or 2)
+    static_assert(PCS == 1 || PCS == 2, "tile smaller than the workgroup");
+    __shared__ __align__(16) uint8_t s_k[32 * KP];
+    __shared__ __align__(16) uint8_t s_vt[HD * VP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, kh = lane >> 5;
+    const int kvh = blockIdx.y;
+    const int m_base = (gridDim.x - 1 - blockIdx.x) * BM;  // longest row blocks are scheduled first
+    const int kv_dim = n_kv_heads * HD;
+
+    const int row = m_base + wave * RPW + j / G, head = kvh * G + j % G;
+    const int row_c = row < rows ? row : rows - 1;
+    const int64_t limit = pos0 + row_c;  // last position this query attends to
+    // scores are kept in base 2: q is scaled by scale * log2(e) before its rounding to fp16
+    const float qs = scale * 1.44269504088896340736f;
+    pf_h8 qf[KS];
+    {
+        const float* src = Q + ((int64_t)row_c * n_heads + head) * HD + 8 * kh;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const float4 a = *reinterpret_cast<const float4*>(src + 16 * ks), b = *reinterpret_cast<const float4*>(src + 16 * ks + 4);
+            qf[ks] = pf_h8{(_Float16)(a.x * qs), (_Float16)(a.y * qs), (_Float16)(a.z * qs), (_Float16)(a.w * qs),
+                           (_Float16)(b.x * qs), (_Float16)(b.y * qs), (_Float16)(b.z * qs), (_Float16)(b.w * qs)};
+        }
+    }
+    pf_f16v acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    const int last_row = (m_base + BM < rows ? m_base + BM : rows) - 1;
+    const int64_t t_end = pos0 + last_row;  // last position any query of this workgroup attends to
+    const int ntiles = (int)(t_end / 32) + 1;
+    // staging: piece q = tid + 256 i of a tile is position q / (HD / 8), elements 8 (q % (HD / 8)) .. +8
+    uint4 kreg0, kreg1, vreg0, vreg1;  // scalars, not arrays: they must stay in registers across the loop
+    kreg1 = vreg1 = make_uint4(0, 0, 0, 0);
+    auto piece_off = [&](int tile, int i) {
+        const int q = tid + 256 * i, p = q / (HD / 8), c = q % (HD / 8);
+        int64_t t = (int64_t)tile * 32 + p;
+        t = t <= t_end ? t : t_end;  // rows past the end are masked below; never read past the appended rows
+        return t * kv_dim + (int64_t)kvh * HD + 8 * c;
+    };
+    auto fetch = [&](int tile) {
+        const int64_t o0 = piece_off(tile, 0);
+        kreg0 = *reinterpret_cast<const uint4*>(Kc + o0);
+        vreg0 = *reinterpret_cast<const uint4*>(Vc + o0);
+        if constexpr (PCS > 1) {
+            const int64_t o1 = piece_off(tile, 1);
+            kreg1 = *reinterpret_cast<const uint4*>(Kc + o1);
+            vreg1 = *reinterpret_cast<const uint4*>(Vc + o1);
+        }
+    };
+    auto stage = [&](int i, const uint4& kr, const uint4& vr) {
+        const int q = tid + 256 * i, p = q / (HD / 8), c = q % (HD / 8);
+        *reinterpret_cast<uint4*>(s_k + p * KP + 16 * c) = kr;
+        uint8_t* vt = s_vt + (8 * c) * VP + 2 * p;  // transposed: V^T[d][position]
+        *reinterpret_cast<uint16_t*>(vt + 0 * VP) = (uint16_t)vr.x;
+        *reinterpret_cast<uint16_t*>(vt + 1 * VP) = (uint16_t)(vr.x >> 16);
+        *reinterpret_cast<uint16_t*>(vt + 2 * VP) = (uint16_t)vr.y;
+        *reinterpret_cast<uint16_t*>(vt + 3 * VP) = (uint16_t)(vr.y >> 16);
+        *reinterpret_cast<uint16_t*>(vt + 4 * VP) = (uint16_t)vr.z;
+        *reinterpret_cast<uint16_t*>(vt + 5 * VP) = (uint16_t)(vr.z >> 16);
+        *reinterpret_cast<uint16_t*>(vt + 6 * VP) = (uint16_t)vr.w;
+        *reinterpret_cast<uint16_t*>(vt + 7 * VP) = (uint16_t)(vr.w >> 16);
+    };
+    fetch(0);
+    for (int tile = 0; tile < ntiles; ++tile) {
+        __syncthreads();  // every wave has finished reading the previous tile
+        stage(0, kreg0, vreg0);
+        if constexpr (PCS > 1) stage(1, kreg1, vreg1);
+        __syncthreads();
+        if (tile + 1 < ntiles) fetch(tile + 1);  // in flight during this tile's arithmetic
+
+        // S^T tile: rows = the tile's 32 positions, column = this lane's query vector
+        pf_f16v sc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const pf_h8 a = *reinterpret_cast<const pf_h8*>(s_k + j * KP + (16 * ks + 8 * kh) * 2);
+            sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], sc, 0, 0, 0);
+        }
+        const int64_t t0 = (int64_t)tile * 32 + 4 * kh;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int64_t t = t0 + 8 * (r >> 2) + (r & 3);
+            sc[r] = t <= limit ? sc[r] : -INFINITY;
+            mx = fmaxf(mx, sc[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // the column's other 16 positions
+        const float m_new = fmaxf(m_run, mx);    // finite from the first tile on: position 0 is visible to every query
+        const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            sc[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
+            psum += sc[r];
+        }
+        const pf_h8 pb0 = {(_Float16)sc[0], (_Float16)sc[1], (_Float16)sc[2], (_Float16)sc[3],
+                           (_Float16)sc[4], (_Float16)sc[5], (_Float16)sc[6], (_Float16)sc[7]};
+        const pf_h8 pb1 = {(_Float16)sc[8], (_Float16)sc[9], (_Float16)sc[10], (_Float16)sc[11],
+                           (_Float16)sc[12], (_Float16)sc[13], (_Float16)sc[14], (_Float16)sc[15]};
+        l_run = fmaf(l_run, corr, psum);  // this lane's 16 positions of each tile; the two halves are added at the end
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+        // O^T += V^T . P^T: step ks sums the positions of accumulator registers 8 ks .. 8 ks + 7
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const uint8_t* vrow = s_vt + (32 * dt + j) * VP + (16 * ks + 4 * kh) * 2;
+                const pf_h4 lo = *reinterpret_cast<const pf_h4*>(vrow), hi = *reinterpret_cast<const pf_h4*>(vrow + 16);
+                const pf_h8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ks ? pb1 : pb0, acc[dt], 0, 0, 0);
+            }
+    }
+    const float l = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / (l + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
+    if (row < rows) {
+        float* dst = O + ((int64_t)row * n_heads + head) * HD + 4 * kh;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int rq = 0; rq < 4; ++rq)
+                *reinterpret_cast<float4*>(dst + 32 * dt + 8 * rq) =
+                    make_float4(acc[dt][4 * rq] * inv, acc[dt][4 * rq + 1] * inv, acc[dt][4 * rq + 2] * inv, acc[dt][4 * rq + 3] * inv);
+    }
+}
+
+template <int HD>
+static int prefill_attn_mfma_launch(int G, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* O, int rows,
+                                    int n_heads, int n_kv_heads, int64_t pos0, float scale) {
+    const int bm = 128 / G;
+    const dim3 grid((rows + bm - 1) / bm, n_kv_heads);
+#define PTM_PA(GG) hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG>), grid, dim3(256), 0, s, Q, static_cast<const __half*>(Kc), static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale)
+    switch (G) {
+        case 1: PTM_PA(1); break;
+        case 2: PTM_PA(2); break;
+        case 4: PTM_PA(4); break;
+        case 8: PTM_PA(8); break;
+        default: return PTM_E_UNSUPPORTED;
+    }
+#undef PTM_PA
+    return launch_status();
+}
+
 template <bool KV16, int HD>
 static int prefill_attn_launch(int G, dim3 grid, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* O,
                                int rows, int n_heads, int n_kv_heads, int64_t pos0, float scale) {
@@ -270,6 +449,9 @@ int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cac
     const int G = n_heads / n_kv_heads;
     const dim3 grid((rows + 3) / 4, n_kv_heads);
     hipStream_t s = as_stream(stream);
+    if (kv_fp16 && rows >= PTM_PREFILL_MFMA_MIN_ROWS && (G == 1 || G == 2 || G == 4 || G == 8))
+        return head_dim == 128 ? prefill_attn_mfma_launch<128>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
+                               : prefill_attn_mfma_launch<64>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
     if (kv_fp16)
         return head_dim == 128 ? prefill_attn_launch<true, 128>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
                                : prefill_attn_launch<true, 64>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);

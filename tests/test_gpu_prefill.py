@@ -128,9 +128,13 @@ def test_qknorm_rope_kvwrite_rows_without_norm_weights(dev, po):
 
 @pytest.mark.parametrize("kv_fp16", [True, False])
 @pytest.mark.parametrize("nh,nkv,hd,pos0,rows", [(32, 8, 128, 0, 70), (32, 8, 128, 300, 17), (4, 2, 64, 0, 33),
-                                                 (4, 4, 64, 19, 5), (16, 2, 128, 1, 1)])
+                                                 (4, 4, 64, 19, 5), (16, 2, 128, 1, 1), (16, 2, 128, 3, 40),
+                                                 (4, 4, 128, 0, 130), (8, 4, 64, 31, 97), (8, 1, 64, 0, 16),
+                                                 (32, 8, 128, 1000, 64)])
 def test_prefill_attention_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, pos0, rows):
-    """Row r attends to cache positions [0, pos0 + r]: later rows of the same batch must not leak in."""
+    """Row r attends to cache positions [0, pos0 + r]: later rows of the same batch must not leak in.  With an
+    fp16 cache and 16 or more rows the matrix-core kernel runs (Q and the softmax weights rounded to fp16: bar
+    1e-3 of the output's maximum, measured 1.5e-4..2.8e-4); otherwise the fp32 kernel (bar 1e-4)."""
     T = pos0 + rows
     max_seq = T + 2
     kvd = nkv * hd
@@ -151,7 +155,9 @@ def test_prefill_attention_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, pos0, rows):
     torch.cuda.synchronize()
     got = O.cpu().numpy()
     assert np.all(np.isfinite(got))
-    assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    e = np.abs(got - want).max() / np.abs(want).max()
+    print("attention nh %d nkv %d hd %d pos0 %d rows %d fp16 %s: max err / max %.2e" % (nh, nkv, hd, pos0, rows, kv_fp16, e), flush=True)
+    assert e <= (1e-3 if kv_fp16 and rows >= 16 else 1e-4)
 
 
 def test_prefill_attention_rejects_bad_shapes(dev):
@@ -340,7 +346,7 @@ def test_prefill_layer_stage_by_stage_on_identical_inputs(dev, po, seeds):
     a = A.cpu().numpy()
     rows_close(a, np.stack([np.concatenate([po.attn_head(qr[m, h * hd:(h + 1) * hd], kf, vf, pos0 + m + 1, kvd, hd, scale,
                                                          col0=(h // (nh // nkv)) * hd) for h in range(nh)]) for m in range(M)]),
-               "attention", 1e-4)
+               "attention", STAGE_TOL)
     gemm("o", A, X, acc=True)
     x1 = X.cpu().numpy()
     rows_close(x1 - x, cpu_gemm("o", a), "o proj (+=)")
@@ -380,19 +386,24 @@ def test_q8_rounding_noise_floor_of_the_oracle(po, seeds):
 
 
 def test_prefill_chunking_does_not_change_the_result(dev, seeds):
-    """Chunks only bound the scratch: rows are independent in every GEMM and attention reads the cache, so any
-    chunk size gives bit-identical logits."""
+    """Chunks only bound the scratch: rows are independent in every GEMM (the K split depends on N and K only) and
+    attention reads the cache in the same tiles, so any chunk size that stays on the same attention kernel gives
+    bit-identical logits; chunks under 16 rows use the fp32 attention kernel and agree within the end-to-end bars."""
     from prometorch_amd.decode import Decoder
     cfg, layers, head = build_tiny(seeds)
-    prompt = [int(t) for t in synth.rng_for(67).integers(0, cfg["vocab"], 40)]
+    prompt = [int(t) for t in synth.rng_for(67).integers(0, cfg["vocab"], 48)]
     outs = []
-    for chunk in (0, 16, 3):
+    for chunk in (0, 16, 24, 3):
         dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=False)
         tok = dec.prefill(prompt, chunk_rows=chunk)
         outs.append((tok, dec.logits()))
         dec.close()
-    for tok, lg in outs[1:]:
+    for tok, lg in outs[1:3]:
         assert tok == outs[0][0] and np.array_equal(bits(lg), bits(outs[0][1]))
+    err, rms, margin = logit_errors(outs[3][1], outs[0][1])
+    assert rms <= E2E_RMS_TOL and err <= E2E_MAX_TOL
+    if margin > 2 * err:
+        assert outs[3][0] == outs[0][0]
 
 
 def test_prefill_then_prefill_continues_the_context(dev, po, seeds):
