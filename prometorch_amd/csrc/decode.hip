@@ -28,7 +28,8 @@ int q6k_gemv_argmax_impl(const void* W, const float* x, const float* gamma, floa
                          float* logits, int K, int N, int64_t stride, int64_t* out_index, void* workspace,
                          const ArgmaxAdvance adv, hipStream_t s);
 int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
-                   int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, hipStream_t s);
+                   int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, bool reuse_rows,
+                   hipStream_t s);
 int qgemm_f16_splits(int N, int K);
 int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const int* N4, int64_t stride4,
                        const void* W6, float* y6, int N6, int64_t stride6, const float* x, const float* gamma,
@@ -213,13 +214,22 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
     PTM_TRY(hip_status(hipMemcpyAsync(d->pf_tokens, tokens_host, 4 * (size_t)M, hipMemcpyHostToDevice, s)));
     PTM_TRY(ptm_embedding_rows(c.embedding_f32, c.embedding_f32 ? nullptr : c.lm_head.data, c.lm_head.row_stride_bytes,
                                d->pf_tokens, M, H, c.vocab, d->pf_x, s));
+    // the workspace keeps the fp16 form of the last X it was given: consecutive products of the same rows with
+    // matrices of the same type (q and k, gate and up) convert them once
+    const float* ws_x = nullptr;
+    uint32_t ws_type = 0;
     auto gemm = [&](const ptm_qweight& w, const float* X, float* Y, bool acc) {
+        const bool reuse = X == ws_x && w.ggml_type == ws_type;
+        ws_x = (Y == X) ? nullptr : X;
+        ws_type = w.ggml_type;
         return qgemm_f16_impl(w.ggml_type, w.data, X, true, Y, M, w.cols, w.rows, w.row_stride_bytes, d->pf_ws, acc,
-                              d->pf_split, d->pf_split_bytes, s);
+                              d->pf_split, d->pf_split_bytes, reuse, s);
     };
+    auto touched = [&](const float* X) { if (ws_x == X) ws_x = nullptr; };  // X rewritten by a non-GEMM kernel
     for (int li = 0; li < c.n_layers; ++li) {
         const ptm_layer& L = d->layers[li];
         PTM_TRY(ptm_rms_norm(d->pf_x, L.attn_norm, d->pf_xn, M, H, c.rms_eps, 0, nullptr, s));
+        touched(d->pf_xn);
         PTM_TRY(gemm(L.q, d->pf_xn, d->pf_q, false));
         PTM_TRY(gemm(L.k, d->pf_xn, d->pf_k, false));
         PTM_TRY(gemm(L.v, d->pf_xn, d->pf_v, false));
@@ -227,11 +237,14 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
                                              c.n_heads, c.n_kv_heads, hd, pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, s));
         PTM_TRY(ptm_prefill_attention(d->pf_q, L.k_cache, L.v_cache, d->pf_attn, M, c.n_heads, c.n_kv_heads, hd, pos0,
                                       c.max_seq, 1.0f / sqrtf((float)hd), c.kv_fp16, s));
+        touched(d->pf_attn);
         PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true));  // x += attn . Wo^T
         PTM_TRY(ptm_rms_norm(d->pf_x, L.ffn_norm, d->pf_xn, M, H, c.rms_eps, 0, nullptr, s));
+        touched(d->pf_xn);
         PTM_TRY(gemm(L.gate, d->pf_xn, d->pf_gate, false));
         PTM_TRY(gemm(L.up, d->pf_xn, d->pf_up, false));
         PTM_TRY(ptm_silu_mul(d->pf_gate, d->pf_up, d->pf_gate, (int64_t)M * I, s));
+        touched(d->pf_gate);
         PTM_TRY(gemm(L.down, d->pf_gate, d->pf_x, true));  // x += act . Wdown^T
     }
     (void)qd; (void)kvd;

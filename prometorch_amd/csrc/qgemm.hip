@@ -620,7 +620,10 @@ static int qgemm_check(const void* W, const void* X, const void* Y, int M, int K
 
 // Y (+)= X . W^T with X bf16 or fp32 rows; shared by the C entry points and the prefill runtime.
 int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
-                   int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, hipStream_t s) {
+                   int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, bool reuse_rows,
+                   hipStream_t s) {
+    // reuse_rows: the workspace already holds these rows of X prepared by the previous call for a matrix of the
+    // same type (same rounding rule), so the conversion pass is skipped
     if (ggml_type != PTM_TYPE_Q4_K && ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
     const int blk = ggml_type == PTM_TYPE_Q4_K ? 144 : 210;
     const int rc = qgemm_check(W, X, Y, M, K, N, stride, blk);
@@ -649,12 +652,14 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     const dim3 grid((N + QF_TN - 1) / QF_TN, mp / QF_TM, splits);
     const int acc = accumulate ? 1 : 0;
     if (ggml_type == PTM_TYPE_Q4_K) {
-        if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
+        if (reuse_rows) {}
+        else if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         hipLaunchKernelGGL(qgemm_f16_kernel<Q4Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
                            rowscale, Y, M, K, N, acc, bps, partials);
     } else {
-        if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
+        if (reuse_rows) {}
+        else if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         hipLaunchKernelGGL(qgemm_f16_kernel<Q6Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
                            rowscale, Y, M, K, N, acc, bps, partials);
@@ -720,7 +725,7 @@ int64_t ptm_qgemm_f16_workspace_bytes(int M, int K) {
 
 int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* Y, int M, int K, int N, int64_t stride,
                   void* workspace, ptm_stream_t stream) {
-    return qgemm_f16_impl(ggml_type, W, X_bf16, false, Y, M, K, N, stride, workspace, false, nullptr, 0, as_stream(stream));
+    return qgemm_f16_impl(ggml_type, W, X_bf16, false, Y, M, K, N, stride, workspace, false, nullptr, 0, false, as_stream(stream));
 }
 
 int64_t ptm_qgemm_f16_f32_workspace_bytes(int M, int K, int N) {
@@ -738,7 +743,7 @@ int ptm_qgemm_f16_f32(uint32_t ggml_type, const void* W, const float* X_f32, flo
     const int splits = qgemm_f16_splits(N, K);
     return qgemm_f16_impl(ggml_type, W, X_f32, true, Y, M, K, N, stride, workspace, accumulate != 0,
                           splits > 1 ? reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + base) : nullptr,
-                          splits > 1 ? (size_t)splits * M * N * 4 : 0, as_stream(stream));
+                          splits > 1 ? (size_t)splits * M * N * 4 : 0, false, as_stream(stream));
 }
 
 }  // extern "C"
