@@ -487,3 +487,127 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
     free(buf);
     return best;
 }
+
+/* ================================================================================================
+ * Sampling
+ * ================================================================================================ */
+/* mt19937 (Matsumoto & Nishimura), the engine behind std::mt19937; the reference's sampler owns a
+ * function-local `static std::mt19937 rng(42)` (gguf_model.h:7740) */
+void po_mt19937_seed(po_mt19937* g, uint32_t seed) {
+    g->mt[0] = seed;
+    for (int i = 1; i < 624; ++i) g->mt[i] = 1812433253u * (g->mt[i - 1] ^ (g->mt[i - 1] >> 30)) + (uint32_t)i;
+    g->idx = 624;
+}
+uint32_t po_mt19937_next(po_mt19937* g) {
+    if (g->idx >= 624) {
+        for (int i = 0; i < 624; ++i) {
+            const uint32_t y = (g->mt[i] & 0x80000000u) | (g->mt[(i + 1) % 624] & 0x7fffffffu);
+            g->mt[i] = g->mt[(i + 397) % 624] ^ (y >> 1) ^ ((y & 1u) ? 0x9908b0dfu : 0u);
+        }
+        g->idx = 0;
+    }
+    uint32_t y = g->mt[g->idx++];
+    y ^= y >> 11;
+    y ^= (y << 7) & 0x9d2c5680u;
+    y ^= (y << 15) & 0xefc60000u;
+    y ^= y >> 18;
+    return y;
+}
+/* libstdc++ generate_canonical<float, 24> over a 32-bit engine: one draw, float(draw) / float(2^32), and a
+ * quotient that rounds up to 1 is replaced by the largest float below 1 (bits/random.tcc) */
+float po_uniform01(po_mt19937* g) {
+    const float sum = (float)po_mt19937_next(g);
+    float r = sum / 4294967296.0f;
+    if (r >= 1.0f) r = nextafterf(1.0f, 0.0f);
+    return r;
+}
+
+/* gguf_model.h:4926-4938: once per generated token, duplicates included */
+void po_repetition_penalty(float* logits, int64_t vocab, const int32_t* generated, int64_t n, float penalty) {
+    if (!(penalty > 1.0f)) return;
+    for (int64_t i = 0; i < n; ++i) {
+        const int32_t t = generated[i];
+        if (t >= 0 && t < vocab) {
+            if (logits[t] > 0) logits[t] /= penalty;
+            else logits[t] *= penalty;
+        }
+    }
+}
+
+typedef struct { float p; int32_t idx; } po_pi;
+static int po_pi_desc(const void* a, const void* b) {
+    const po_pi* x = (const po_pi*)a; const po_pi* y = (const po_pi*)b;
+    if (x->p > y->p) return -1;
+    if (x->p < y->p) return 1;
+    return x->idx < y->idx ? -1 : (x->idx > y->idx ? 1 : 0); /* the reference's std::sort leaves ties unordered */
+}
+static int po_float_desc(const void* a, const void* b) {
+    const float x = *(const float*)a, y = *(const float*)b;
+    return x > y ? -1 : (x < y ? 1 : 0);
+}
+
+/* gguf_model.h:7658-7751 */
+int32_t po_sample_token(const float* logits, int64_t vocab, float temperature, int top_k, float top_p, float r,
+                        float* probs_out, float* gap_out) {
+    if (gap_out) *gap_out = 1.0f;
+    if (temperature < 1e-6f) { /* :7662-7673 greedy */
+        const int32_t best = (int32_t)po_argmax(logits, vocab);
+        if (probs_out) { memset(probs_out, 0, sizeof(float) * (size_t)vocab); probs_out[best] = 1.0f; }
+        return best;
+    }
+    float* probs = (float*)malloc(sizeof(float) * (size_t)vocab);
+    for (int64_t i = 0; i < vocab; ++i) probs[i] = logits[i] / temperature; /* :7677-7679 */
+    if (top_k > 0 && top_k < vocab) { /* :7682-7691: below the k-th largest value -> -1e9 (ties at it stay) */
+        float* sorted = (float*)malloc(sizeof(float) * (size_t)vocab);
+        memcpy(sorted, probs, sizeof(float) * (size_t)vocab);
+        qsort(sorted, (size_t)vocab, sizeof(float), po_float_desc);
+        const float threshold = sorted[top_k - 1];
+        free(sorted);
+        for (int64_t i = 0; i < vocab; ++i)
+            if (probs[i] < threshold) probs[i] = -1e9f;
+    }
+    float max_val = probs[0]; /* :7694-7703 softmax, sums in index order */
+    for (int64_t i = 1; i < vocab; ++i) if (probs[i] > max_val) max_val = probs[i];
+    float sum_exp = 0.0f;
+    for (int64_t i = 0; i < vocab; ++i) { probs[i] = expf(probs[i] - max_val); sum_exp += probs[i]; }
+    float inv_sum = 1.0f / sum_exp;
+    for (int64_t i = 0; i < vocab; ++i) probs[i] *= inv_sum;
+    if (top_p < 1.0f) { /* :7706-7736 nucleus: descending until the running sum reaches top_p, then renormalise */
+        po_pi* sorted = (po_pi*)malloc(sizeof(po_pi) * (size_t)vocab);
+        int64_t m = 0;
+        for (int64_t i = 0; i < vocab; ++i)
+            if (probs[i] > 1e-10f) { sorted[m].p = probs[i]; sorted[m].idx = (int32_t)i; ++m; }
+        qsort(sorted, (size_t)m, sizeof(po_pi), po_pi_desc);
+        uint8_t* keep = (uint8_t*)calloc((size_t)vocab, 1);
+        float cumsum = 0.0f;
+        for (int64_t j = 0; j < m; ++j) {
+            keep[sorted[j].idx] = 1;
+            cumsum += sorted[j].p;
+            if (cumsum >= top_p) break;
+        }
+        for (int64_t i = 0; i < vocab; ++i) if (!keep[i]) probs[i] = 0.0f;
+        sum_exp = 0.0f;
+        for (int64_t i = 0; i < vocab; ++i) sum_exp += probs[i];
+        if (sum_exp > 0) {
+            inv_sum = 1.0f / sum_exp;
+            for (int64_t i = 0; i < vocab; ++i) probs[i] *= inv_sum;
+        }
+        free(keep);
+        free(sorted);
+    }
+    if (probs_out) memcpy(probs_out, probs, sizeof(float) * (size_t)vocab);
+    int32_t chosen = (int32_t)(vocab - 1); /* :7739-7750 inverse CDF in index order */
+    float cumsum = 0.0f, lo = 0.0f, gap = 1.0f;
+    for (int64_t i = 0; i < vocab; ++i) {
+        lo = cumsum;
+        cumsum += probs[i];
+        if (cumsum >= r) {
+            chosen = (int32_t)i;
+            gap = fminf(cumsum - r, r - lo);
+            break;
+        }
+    }
+    if (gap_out) *gap_out = gap;
+    free(probs);
+    return chosen;
+}

@@ -20,6 +20,14 @@
  *   po_attn_head, po_silu_mul, po_argmax, po_decode_step
  *                          golden logits / token ids of the compiled reference's
  *                          forward_decode_cpu on a tiny and the full-size model
+ *   po_mt19937_*, po_uniform01   the 10000th output of the default-seeded generator (4123659995, ISO C++
+ *                          [rand.predef]) + the tokens the compiled reference's sample_token draws with its
+ *                          mt19937(42) (golden_sampling.npz)
+ *   po_sample_token        golden tokens of the compiled reference's sample_token over seeded logits and
+ *                          parameter sets + numpy float64 restatement (top-k by partition, softmax,
+ *                          nucleus cut, inverse CDF)
+ *   po_repetition_penalty  numpy restatement with repeated ids (the reference applies the penalty once per
+ *                          occurrence); the reference holds it inline in generate(), so no compiled check
  */
 #ifndef PTM_ORACLE_H
 #define PTM_ORACLE_H
@@ -88,6 +96,18 @@ typedef struct {
  * advances seq_len, returns greedy argmax. hidden_out (optional) gets the final-normed hidden. */
 int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_out);
 int po_num_threads(void);
+
+/* ---- sampling (reference: GGUFModel::sample_token, gguf_model.h:7658-7751; penalty loop :4926-4938) ---- */
+typedef struct { uint32_t mt[624]; int idx; } po_mt19937;
+void po_mt19937_seed(po_mt19937* g, uint32_t seed);
+uint32_t po_mt19937_next(po_mt19937* g);
+/* std::uniform_real_distribution<float>(0, 1)(std::mt19937) as libstdc++ evaluates it */
+float po_uniform01(po_mt19937* g);
+void po_repetition_penalty(float* logits, int64_t vocab, const int32_t* generated, int64_t n, float penalty);
+/* r is the uniform draw.  probs_out (optional, [vocab]) receives the final distribution; gap_out (optional)
+ * the distance from r to the nearest edge of the chosen token's CDF interval (how robust the choice is). */
+int32_t po_sample_token(const float* logits, int64_t vocab, float temperature, int top_k, float top_p, float r,
+                        float* probs_out, float* gap_out);
 
 #ifdef __cplusplus
 }

@@ -76,6 +76,14 @@ def lib():
         L.po_silu_mul.argtypes = [_vp, _vp, _i64]
         L.po_argmax.argtypes = [_vp, _i64]
         L.po_get_scale_min_k4.argtypes = [_i32, _vp, _vp, _vp]
+        L.po_mt19937_seed.argtypes = [_vp, _u32]
+        L.po_mt19937_next.restype = _u32
+        L.po_mt19937_next.argtypes = [_vp]
+        L.po_uniform01.restype = _f32
+        L.po_uniform01.argtypes = [_vp]
+        L.po_repetition_penalty.argtypes = [_vp, _i64, _vp, _i64, _f32]
+        L.po_sample_token.restype = _i32
+        L.po_sample_token.argtypes = [_vp, _i64, _f32, _i32, _f32, _f32, _vp, _vp]
         _lib = L
     return _lib
 
@@ -186,6 +194,37 @@ def _qw(qtype, W):
     return QW(W.ctypes.data, qtype, N, stride // (144 if qtype == 12 else 210) * 256, stride), W
 
 
+class MT19937:
+    """std::mt19937 and the uniform float draw the reference's sampler makes from it."""
+
+    def __init__(self, seed: int = 42):
+        self.state = (C.c_uint32 * 625)()
+        lib().po_mt19937_seed(self.state, seed)
+
+    def next_u32(self) -> int:
+        return int(lib().po_mt19937_next(self.state))
+
+    def uniform01(self) -> float:
+        return float(lib().po_uniform01(self.state))
+
+
+def repetition_penalty(logits, generated, penalty):
+    out = np.array(logits, np.float32, copy=True)
+    g = np.ascontiguousarray(generated, np.int32)
+    lib().po_repetition_penalty(_p(out), out.size, _p(g), g.size, penalty)
+    return out
+
+
+def sample_token(logits, temperature, top_k, top_p, r, want_probs=False):
+    """-> (token, gap[, probs]); gap = distance from r to the nearest edge of the token's CDF interval."""
+    x = np.ascontiguousarray(logits, np.float32)
+    gap = C.c_float()
+    probs = np.empty(x.size, np.float32) if want_probs else None
+    tok = int(lib().po_sample_token(_p(x), x.size, temperature, top_k, top_p, r, _p(probs) if want_probs else None,
+                                    C.byref(gap)))
+    return (tok, gap.value, probs) if want_probs else (tok, gap.value)
+
+
 class OracleModel:
     """Host-side model for po_decode_step; keeps every numpy buffer alive."""
 
@@ -286,6 +325,8 @@ def ref():
         R.ref_model_seq_len.argtypes = [_vp]
         R.ref_model_decode.restype = _i64
         R.ref_model_decode.argtypes = [_vp, _i64, _vp]
+        R.ref_sample_token.restype = _i32
+        R.ref_sample_token.argtypes = [_vp, _vp, _i64, _f32, _i32, _f32]
         _ref = R
     return _ref
 

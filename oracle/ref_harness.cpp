@@ -185,4 +185,10 @@ int64_t ref_model_decode(void* h, int64_t token, float* logits_out) {
     for (int64_t j = 1; j < V; ++j) if (p[j] > bv) { bv = p[j]; best = j; }
     return best;
 }
+// GGUFModel::sample_token (torch/io/gguf_model.h:7658-7751).  Its generator is a function-local
+// `static std::mt19937 rng(42)`: the n-th sampling call of a process (temperature >= 1e-6) uses the n-th draw.
+int32_t ref_sample_token(void* h, const float* logits, int64_t vocab, float temperature, int top_k, float top_p) {
+    return static_cast<RefModel*>(h)->m.sample_token(vec_tensor(logits, vocab), temperature, top_k, top_p);
+}
+
 }  // extern "C"

@@ -169,3 +169,30 @@ def make_kv_prefill(seed: int, layer: int, cfg: dict, n_pos: int):
     k = g.standard_normal((n_pos, kvd), dtype=np.float32).astype(np.float16)
     v = g.standard_normal((n_pos, kvd), dtype=np.float32).astype(np.float16)
     return k, v
+
+
+# ---- sampling cases: (vocab, logit kind, temperature, top_k, top_p), in the order the golden run draws them ----
+SAMPLING_CASES = (
+    [(1000, "normal", 0.8, 40, 0.9), (1000, "normal", 1.0, 0, 1.0), (1000, "normal", 0.7, 1, 1.0),
+     (1000, "ties", 1.0, 40, 0.9), (1000, "ties", 1.5, 100, 0.5), (1000, "normal", 0.0, 40, 0.9),
+     (1000, "normal", 0.8, 0, 0.9), (1000, "peaked", 2.0, 5, 0.3), (1000, "normal", 1.0, 40, 1.0),
+     (1000, "normal", 0.8, 1000, 0.95), (1000, "negative", 0.8, 40, 0.9), (37, "normal", 0.8, 40, 0.9)]
+    + [(151936, "normal", 0.8, 40, 0.9)] * 6 + [(151936, "ties", 0.8, 40, 0.9), (151936, "peaked", 1.2, 64, 0.8),
+                                                  (151936, "normal", 0.6, 0, 0.9), (151936, "normal", 1.0, 1024, 1.0)]
+    + [(1000, "normal", 0.9, 50, 0.85)] * 24
+)
+
+
+def sampling_logits(case_index: int) -> np.ndarray:
+    """Logits of sampling case i.  normal: 3 N(0,1); ties: the same rounded to 0.25 (equal values around the
+    k-th largest); peaked: one token far ahead; negative: all below zero."""
+    vocab, kind = SAMPLING_CASES[case_index][:2]
+    g = rng_for(4242, case_index)
+    x = np.float32(3.0) * g.standard_normal(vocab, dtype=np.float32)
+    if kind == "ties":
+        x = (np.round(x * 4) / 4).astype(np.float32)
+    elif kind == "peaked":
+        x[int(g.integers(0, vocab))] += np.float32(12.0)
+    elif kind == "negative":
+        x = (-np.abs(x) - np.float32(1.0)).astype(np.float32)
+    return x

@@ -80,8 +80,13 @@ def ref_q8(x):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--full", action="store_true")
+    ap.add_argument("--sampling-only", action="store_true", help="write golden_sampling.npz and nothing else")
     args = ap.parse_args()
     assert po.have_ref(), "build oracle/_ref first: make -C oracle ref"
+    if args.sampling_only:
+        make_sampling()
+        print("wrote golden_sampling.npz")
+        return
     R = po.ref()
     meta = {"made_with": "oracle/_ref/libptm_ref.so (g++ -O2 -std=c++17 -mavx2 -mfma; see oracle/Makefile)",
             "python": platform.python_version(), "numpy": np.__version__, "threads": R.ref_num_threads(), "seeds": SEEDS}
@@ -202,12 +207,29 @@ def main():
     rm.close()
 
     np.savez_compressed(os.path.join(OUT, "golden_small.npz"), **g)
+    make_sampling()
 
     if args.full:
         make_full(meta)
     with open(os.path.join(OUT, "golden_meta.json"), "w") as f:
         json.dump(meta, f, indent=1, sort_keys=True)
     print("wrote", OUT)
+
+
+def make_sampling():
+    """The reference's sample_token over synth.SAMPLING_CASES, called in order in this (fresh) process: its
+    generator is a function-local static std::mt19937(42), so call n with temperature >= 1e-6 uses draw n.
+    (Nothing else in this script samples, so the draws start at the first.)"""
+    R = po.ref()
+    t = synth.TINY
+    h = R.ref_model_create(t["vocab"], t["hidden"], t["n_layers"], t["n_heads"], t["n_kv_heads"], t["head_dim"], t["inter"],
+                           t["rope_base"], t["eps"], 8)  # sample_token reads no model state
+    toks = []
+    for i, (vocab, kind, temperature, top_k, top_p) in enumerate(synth.SAMPLING_CASES):
+        x = np.ascontiguousarray(synth.sampling_logits(i))
+        toks.append(int(R.ref_sample_token(h, x.ctypes.data, vocab, temperature, top_k, top_p)))
+    R.ref_model_destroy(h)
+    np.savez_compressed(os.path.join(OUT, "golden_sampling.npz"), tokens=np.array(toks, np.int32))
 
 
 def make_full(meta):
