@@ -139,6 +139,25 @@ def main():
     tokens_equal = chained[args.warmup:] == toks
     log("chained: %.1f tok/s, tokens identical to stepwise: %s" % (chained_tok_s, tokens_equal))
 
+    # sampled generation with the sampler on the device (temperature 0.8, top-k 40, top-p 0.9, repetition penalty 1.1:
+    # PromeServe's defaults), host-synchronous per token like the timed greedy loop, and chained
+    us = ops.mt19937_uniforms(42, 0, args.warmup + args.steps)
+    dec.set_past_len(N_PREFILL)
+    dec.sampling_begin(0.8, 40, 0.9, 1.1)
+    tok_s_ = 1
+    for i in range(args.warmup):
+        tok_s_ = dec.sample(tok_s_, us[i:i + 1])[0]
+    t1 = time.perf_counter()
+    for i in range(args.steps):
+        tok_s_ = dec.sample(tok_s_, us[args.warmup + i:args.warmup + i + 1])[0]
+    sampled_tok_s = args.steps / (time.perf_counter() - t1)
+    dec.set_past_len(N_PREFILL)
+    dec.sampling_begin(0.8, 40, 0.9, 1.1)
+    t1 = time.perf_counter()
+    dec.sample(1, us)
+    sampled_chained_tok_s = (args.warmup + args.steps) / (time.perf_counter() - t1)
+    log("sampled (device top-k/top-p): %.1f tok/s per-token sync, %.1f tok/s chained" % (sampled_tok_s, sampled_chained_tok_s))
+
     # ---- roofline of the dominant kernel, live, HIP events on the launching stream --------------
     H, I = cfg["hidden"], cfg["inter"]
     L0 = dec._layers
@@ -251,6 +270,7 @@ def main():
                    "kv_cache": "fp16", "graph": "hipGraph per token", "host_sync": "per token"},
         "roofline": roof, "cpu_baseline": cpu, "gemv": gemv,
         "chained_tok_s": chained_tok_s, "chained_tokens_identical": bool(tokens_equal),
+        "sampled_tok_s": sampled_tok_s, "sampled_chained_tok_s": sampled_chained_tok_s,
         "a100_published_tok_s": 82.6, "x_a100_published": tok_s / 82.6,
         "token_hbm_frac": per_token_bytes / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
     }

@@ -189,6 +189,28 @@ int ptm_embedding_row_q6k(const void* table_q6k, float* out, const int* d_token_
                           int64_t row_stride_bytes, ptm_stream_t stream);
 /* *out = index of the maximum (strict '>', lowest index on ties). launch_argmax (CUDAOps.h:145). */
 int ptm_argmax(const float* in, int64_t* out, int64_t n, ptm_stream_t stream);
+/* ---- sampling on the device ------------------------------------------------------------------
+ * GGUFModel::sample_token (gguf_model.h:7658-7751) with the repetition penalty of generate() (:4926-4938)
+ * applied first: penalty once per earlier occurrence (counts[i]; NULL = none), temperature, top-k (ties at the
+ * k-th value kept), softmax, top-p, inverse CDF in index order against the uniform draw *d_uniform (device
+ * memory; the reference draws it from a static std::mt19937(42) through uniform_real_distribution<float>).
+ * temperature < 1e-6: argmax of the penalised logits, no draw.  Implemented for 1 <= top_k <= 1024 and
+ * top_k < vocab (PTM_E_UNSUPPORTED otherwise: sample on the host from ptm_decode_logits).  *out_token (device)
+ * is -1 when more than 2048 logits tie at the top-k threshold.  workspace: ptm_sampler_workspace_bytes() device
+ * bytes, 8-byte aligned, contents irrelevant.  Replaces the 608 KB logits copy + CPU sampling per token. */
+typedef struct ptm_sampling {
+    float temperature;
+    int32_t top_k;
+    float top_p;
+    float repeat_penalty;
+} ptm_sampling;
+int64_t ptm_sampler_workspace_bytes(void);
+int ptm_sample_token(const float* logits, int vocab, const int32_t* counts, const ptm_sampling* params,
+                     const float* d_uniform, void* workspace, int64_t* out_token, ptm_stream_t stream);
+/* n draws of std::uniform_real_distribution<float>(0, 1) over std::mt19937(seed) after skipping `skip` draws:
+ * the sequence the reference's sampler consumes (seed 42; one draw per sampled token).  Host memory. */
+int ptm_mt19937_uniforms(uint32_t seed, int64_t skip, int64_t n, float* out_host);
+
 /* out = a + b; out = in. launch_add / launch_copy (CUDAOps.h:63, :83). */
 int ptm_add(const float* a, const float* b, float* out, int64_t n, ptm_stream_t stream);
 int ptm_copy(const float* in, float* out, int64_t n, ptm_stream_t stream);
@@ -290,6 +312,13 @@ int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token);
  * The counterpart of GGUFModel::forward(tokens, use_cache = true) (gguf_model.h:2510-2571); row m equals
  * a decode step of token m up to the fp16 rounding of the GEMM operands.  Allocates its scratch on first use. */
 int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_rows, int64_t* next_token);
+/* Sampled generation (the decode loop of promeserve/api_handlers.h:848-923 with the sampling kept on the GPU).
+ * ptm_decode_sampling_begin starts a generation: stores the parameters and forgets the tokens generated so far
+ * (the repetition penalty only sees tokens generated since).  ptm_decode_sample then runs n chained steps from
+ * `token`, drawing with uniforms_host[0..n) (ptm_mt19937_uniforms gives the reference's sequence); ids land in
+ * out_tokens.  Stop tokens are the caller's business: generate in short runs and cut at the first one. */
+int ptm_decode_sampling_begin(ptm_decoder* d, const ptm_sampling* params);
+int ptm_decode_sample(ptm_decoder* d, int token_id, int n, const float* uniforms_host, int64_t* out_tokens);
 int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_out);
 /* Device pointers to the last step's logits [vocab] and final-normed hidden [hidden]. */
 const float* ptm_decode_logits(ptm_decoder* d);

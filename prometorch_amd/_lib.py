@@ -34,6 +34,10 @@ class DecodeConfig(C.Structure):
                 ("embedding_f32", vp), ("layers", C.POINTER(Layer)), ("out_norm", vp), ("lm_head", QWeight)]
 
 
+class Sampling(C.Structure):
+    _fields_ = [("temperature", f32), ("top_k", C.c_int32), ("top_p", f32), ("repeat_penalty", f32)]
+
+
 class GgufTensor(C.Structure):
     _fields_ = [("name", C.c_char_p), ("ggml_type", u32), ("n_dims", C.c_int32), ("dims", i64 * 4), ("nbytes", i64),
                 ("data", vp)]
@@ -93,6 +97,11 @@ SIGNATURES = {
     "ptm_embedding_rows": (i32, [vp, vp, i64, vp, i32, i32, i32, vp, vp]),
     "ptm_qknorm_rope_kvwrite_rows": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, i32, vp]),
     "ptm_prefill_attention": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, vp]),
+    "ptm_decode_sampling_begin": (i32, [vp, C.POINTER(Sampling)]),
+    "ptm_decode_sample": (i32, [vp, i32, i32, C.POINTER(f32), C.POINTER(i64)]),
+    "ptm_sampler_workspace_bytes": (i64, []),
+    "ptm_sample_token": (i32, [vp, i32, vp, C.POINTER(Sampling), vp, vp, vp, vp]),
+    "ptm_mt19937_uniforms": (i32, [u32, i64, i64, C.POINTER(f32)]),
     "ptm_decode_logits": (vp, [vp]),
     "ptm_decode_hidden": (vp, [vp]),
     "ptm_decode_stream": (vp, [vp]),

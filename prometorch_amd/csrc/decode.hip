@@ -31,6 +31,12 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
                    int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, bool reuse_rows,
                    hipStream_t s);
 int qgemm_f16_splits(int N, int K);
+int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
+                    const ptm_sampling* d_params, const float* d_uniforms, const int* d_step, void* workspace,
+                    int64_t* out_token, int32_t* counts_rw, ArgmaxAdvance adv, hipStream_t s);
+__global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
+}
 int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const int* N4, int64_t stride4,
                        const void* W6, float* y6, int N6, int64_t stride6, const float* x, const float* gamma,
                        float eps, int add_one, int K, hipStream_t s);
@@ -58,9 +64,19 @@ struct ptm_decoder {
     ptm_decode_config cfg{};
     std::vector<ptm_layer> layers;
     hipStream_t stream = nullptr;
-    hipGraph_t graph = nullptr;
+    hipGraph_t graph = nullptr;       // one greedy step
     hipGraphExec_t exec = nullptr;
     bool captured = false;
+    hipGraph_t graph_s = nullptr;     // one sampled step
+    hipGraphExec_t exec_s = nullptr;
+    bool captured_s = false;
+    // sampling state: parameters (host + device copy), occurrence counts of generated tokens, uniform draws
+    ptm_sampling sampling{0.0f, 1, 1.0f, 1.0f};
+    bool sampling_set = false;
+    ptm_sampling* d_sampling = nullptr;
+    int32_t* d_counts = nullptr;
+    float* d_uniforms = nullptr;
+    void* sampler_ws = nullptr;
     void* slab = nullptr;
     float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *act = nullptr,
           *gate = nullptr, *up = nullptr, *logits = nullptr, *pO = nullptr, *pL = nullptr, *pM = nullptr,
@@ -103,7 +119,7 @@ static int gemv_any(const ptm_qweight& w, const float* x_f32, float* y, bool acc
 }
 
 // Enqueue one token step on d->stream. Everything it reads that changes per token is in device memory.
-static int enqueue_step(ptm_decoder* d) {
+static int enqueue_step(ptm_decoder* d, bool sample = false) {
     const ptm_decode_config& c = d->cfg;
     hipStream_t s = d->stream;
     const int H = c.hidden, hd = c.head_dim;
@@ -154,6 +170,19 @@ static int enqueue_step(ptm_decoder* d) {
             PTM_TRY(ptm_silu_mul(d->gate, d->up, d->act, c.inter, s));
         }
         PTM_TRY(gemv_any(L.down, d->act, d->x, true, s));  // x += Wdown . act
+    }
+    if (sample) {
+        // logits (final RMSNorm in the lm_head prologue), then the sampler, whose last kernel does the step bookkeeping
+        if (c.lm_head.ggml_type == PTM_TYPE_Q6_K) {
+            PTM_TRY(q6k_gemv_impl(c.lm_head.data, d->x, d->logits, H, c.vocab, c.lm_head.row_stride_bytes, false, c.out_norm,
+                                  c.rms_eps, 0, s));
+        } else {
+            PTM_TRY(ptm_rms_norm(d->x, c.out_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+            PTM_TRY(gemv_any(c.lm_head, d->xn, d->logits, false, s));
+        }
+        return sampler_enqueue(d->logits, c.vocab, d->d_counts, d->sampling, d->d_sampling, d->d_uniforms, d->d_step,
+                               d->sampler_ws, d->d_next, d->d_counts,
+                               ArgmaxAdvance{d->d_token, d->d_past, d->d_step, d->d_tokens, c.max_seq}, s);
     }
     if (c.lm_head.ggml_type == PTM_TYPE_Q6_K) {
         // final RMSNorm in the lm_head prologue, step bookkeeping in the argmax tail: two launches for the whole tail
@@ -293,7 +322,9 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
                  o_pM = take(4 * (size_t)S * c.n_heads), o_rope = take(4 * (size_t)c.max_seq * c.head_dim),
                  o_xq8 = take((size_t)ptm_q8_bytes(H > c.inter ? H : c.inter)),
                  o_ws = take((size_t)ptm_argmax_workspace_bytes(c.vocab)), o_tok = take(256), o_past = take(256),
-                 o_next = take(256), o_step = take(256), o_tokens = take(8 * (size_t)c.max_seq);
+                 o_next = take(256), o_step = take(256), o_tokens = take(8 * (size_t)c.max_seq),
+                 o_samp = take(256), o_counts = take(4 * (size_t)c.vocab), o_unif = take(4 * (size_t)c.max_seq),
+                 o_sws = take((size_t)ptm_sampler_workspace_bytes());
     if ((rc = hip_status(hipMalloc(&d->slab, off))) != PTM_OK) { delete d; return rc; }
     uint8_t* base = static_cast<uint8_t*>(d->slab);
     d->x = (float*)(base + o_x); d->xn = (float*)(base + o_xn); d->q = (float*)(base + o_q);
@@ -304,6 +335,8 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->amax_ws = base + o_ws; d->d_token = (int*)(base + o_tok); d->d_past = (int64_t*)(base + o_past);
     d->d_next = (int64_t*)(base + o_next); d->d_step = (int*)(base + o_step);
     d->d_tokens = (int64_t*)(base + o_tokens);
+    d->d_sampling = (ptm_sampling*)(base + o_samp); d->d_counts = (int32_t*)(base + o_counts);
+    d->d_uniforms = (float*)(base + o_unif); d->sampler_ws = base + o_sws;
     q6k_init_attributes();  // one-time kernel attributes, before anything can be captured
 
     if ((rc = hip_status(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
@@ -324,6 +357,8 @@ void ptm_decode_destroy(ptm_decoder* d) {
     if (d->stream) (void)hipStreamSynchronize(d->stream);
     if (d->exec) (void)hipGraphExecDestroy(d->exec);
     if (d->graph) (void)hipGraphDestroy(d->graph);
+    if (d->exec_s) (void)hipGraphExecDestroy(d->exec_s);
+    if (d->graph_s) (void)hipGraphDestroy(d->graph_s);
     if (d->h_pinned) (void)hipHostFree(d->h_pinned);
     if (d->pf_slab) (void)hipFree(d->pf_slab);
     if (d->slab) (void)hipFree(d->slab);
@@ -338,8 +373,9 @@ int ptm_decode_set_past_len(ptm_decoder* d, int64_t past_len) {
     return PTM_OK;
 }
 
-// Run n chained steps starting from `token`; token ids land in d_tokens[0..n) and h_pinned[0..n).
-static int run_steps(ptm_decoder* d, int token, int n) {
+// Run n chained steps starting from `token` (greedy, or sampled with the stored parameters and the uniforms already
+// on the device); token ids land in d_tokens[0..n) and h_pinned[0..n).
+static int run_steps(ptm_decoder* d, int token, int n, bool sample = false) {
     if (d->status != PTM_OK) return PTM_E_STATE;
     if (n <= 0) return PTM_E_SHAPE;
     if (token < 0 || token >= d->cfg.vocab) return PTM_E_RANGE;
@@ -348,33 +384,69 @@ static int run_steps(ptm_decoder* d, int token, int n) {
     hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, s, d->d_token, token, d->d_past, d->past_len, d->d_step);
     int rc = launch_status();
     if (rc != PTM_OK) return rc;
+    bool& captured = sample ? d->captured_s : d->captured;
+    hipGraph_t& graph = sample ? d->graph_s : d->graph;
+    hipGraphExec_t& exec = sample ? d->exec_s : d->exec;
     int done = 0;
-    if (d->cfg.use_graph && !d->captured) {
+    if (d->cfg.use_graph && !captured) {
         // first step eagerly (sets one-time kernel attributes outside capture), then capture
-        if ((rc = enqueue_step(d)) != PTM_OK) return d->status = rc;
+        if ((rc = enqueue_step(d, sample)) != PTM_OK) return d->status = rc;
         done = 1;
         {
             if ((rc = hip_status(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal))) != PTM_OK) return d->status = rc;
-            const int rc_enq = enqueue_step(d);
+            const int rc_enq = enqueue_step(d, sample);
             hipGraph_t g = nullptr;
             rc = hip_status(hipStreamEndCapture(s, &g));
             if (rc_enq != PTM_OK || rc != PTM_OK) {
                 if (g) (void)hipGraphDestroy(g);
                 return d->status = (rc_enq != PTM_OK ? rc_enq : rc);
             }
-            d->graph = g;
-            if ((rc = hip_status(hipGraphInstantiate(&d->exec, g, nullptr, nullptr, 0))) != PTM_OK) return d->status = rc;
-            d->captured = true;
+            graph = g;
+            if ((rc = hip_status(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0))) != PTM_OK) return d->status = rc;
+            captured = true;
         }
     }
     for (; done < n; ++done) {
-        if (d->captured) rc = hip_status(hipGraphLaunch(d->exec, s));
-        else rc = enqueue_step(d);
+        if (captured) rc = hip_status(hipGraphLaunch(exec, s));
+        else rc = enqueue_step(d, sample);
         if (rc != PTM_OK) return d->status = rc;
     }
     if ((rc = hip_status(hipMemcpyAsync(d->h_pinned, d->d_tokens, 8 * (size_t)n, hipMemcpyDeviceToHost, s))) != PTM_OK) return d->status = rc;
     if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return d->status = rc;
     d->past_len += n;
+    return PTM_OK;
+}
+
+int ptm_decode_sampling_begin(ptm_decoder* d, const ptm_sampling* params) {
+    if (!d || !params) return PTM_E_NULL;
+    if (d->status != PTM_OK) return PTM_E_STATE;
+    const bool greedy = !(params->temperature >= 1e-6f);
+    if (!greedy) {
+        if (params->top_k <= 0 || params->top_k >= d->cfg.vocab || params->top_k > 1024) return PTM_E_UNSUPPORTED;
+        if (!(params->top_p > 0.0f)) return PTM_E_SHAPE;
+    }
+    hipStream_t s = d->stream;
+    int rc = hip_status(hipMemcpyAsync(d->d_sampling, params, sizeof(ptm_sampling), hipMemcpyHostToDevice, s));
+    if (rc != PTM_OK) return rc;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(64), dim3(256), 0, s, d->d_counts, (int64_t)d->cfg.vocab, 0);
+    if ((rc = launch_status()) != PTM_OK) return rc;
+    if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return rc;  // params may be a temporary of the caller
+    d->sampling = *params;
+    d->sampling_set = true;
+    return PTM_OK;
+}
+
+int ptm_decode_sample(ptm_decoder* d, int token_id, int n, const float* uniforms_host, int64_t* out_tokens) {
+    if (!d || !uniforms_host || !out_tokens) return PTM_E_NULL;
+    if (!d->sampling_set) return PTM_E_STATE;
+    if (n <= 0 || n > d->cfg.max_seq) return PTM_E_SHAPE;
+    int rc = hip_status(hipMemcpyAsync(d->d_uniforms, uniforms_host, 4 * (size_t)n, hipMemcpyHostToDevice, d->stream));
+    if (rc != PTM_OK) return rc;
+    if ((rc = run_steps(d, token_id, n, true)) != PTM_OK) return rc;
+    for (int i = 0; i < n; ++i) {
+        out_tokens[i] = d->h_pinned[i];
+        if (out_tokens[i] < 0) return PTM_E_UNSUPPORTED;  // more logits tie at the top-k threshold than the sampler holds
+    }
     return PTM_OK;
 }
 

@@ -1,0 +1,339 @@
+// Token sampling on the device: repetition penalty, temperature, top-k, softmax, top-p, inverse-CDF draw.
+//
+// The reference samples on the host (GGUFModel::sample_token, torch/io/gguf_model.h:7658-7751; the penalty loop
+// of generate(), :4926-4938; PromeServe's decode loop, promeserve/api_handlers.h:861-876) and so copies the whole
+// logit row (608 KB for a 151 936-token vocabulary) to the host every token.  Here only the chosen id leaves the GPU.
+//
+// Semantics kept from the reference, in its order:
+//   x_i = logit_i, divided (x > 0) or multiplied (x <= 0) by the penalty once per earlier occurrence of token i;
+//   x_i /= temperature; everything below the k-th largest x (duplicates counted, ties at it kept) is dropped;
+//   p = softmax(x) with sums taken in index order; top-p: tokens in descending p until the running sum reaches
+//   top_p, renormalised; the token is the first index whose running sum of p (index order) reaches the uniform
+//   draw r (index 0 when r <= 0, the last index when the sum never gets there).
+//   temperature < 1e-6: argmax (strict '>', lowest index) of the penalised logits.
+// Exact selection of the k-th largest x: a three-level radix select over the order-preserving integer image of x
+// (11 + 11 + 10 bits: one histogram pass over the vocabulary per level), then a gather of everything at or above
+// the threshold (<= SAMPLER_MAX_CAND, normally exactly k) and ONE workgroup that finishes on that short list,
+// doing the reference's sequential fp32 sums in the reference's order (so results differ from the CPU's only
+// through expf's last bit).
+#include "ptm_common.h"
+
+#include <random>
+
+namespace ptm {
+
+enum { SAMPLER_MAX_CAND = 2048, SAMPLER_MAX_TOPK = 1024, SAMPLER_ELEMS_PER_WG = 2048 };
+
+// workspace layout (uint32 words)
+enum {
+    SW_HIST0 = 0,                 // 2048 bins: key >> 21
+    SW_HIST1 = 2048,              // 2048 bins: (key >> 10) & 0x7ff among keys of the level-0 bin
+    SW_HIST2 = 4096,              // 1024 bins: key & 0x3ff among keys of the level-1 bin
+    SW_COUNT = 5120,              // number of gathered candidates
+    SW_CAND_KEY = 5128,           // [SAMPLER_MAX_CAND]
+    SW_CAND_IDX = SW_CAND_KEY + SAMPLER_MAX_CAND,
+    SW_WORDS = SW_CAND_IDX + SAMPLER_MAX_CAND,
+    SW_CLEAR_WORDS = SW_COUNT + 8
+};
+
+struct SamplerArgs {
+    const float* logits;
+    const int32_t* counts;          // occurrences of each token so far, or NULL
+    int vocab;
+    const ptm_sampling* d_params;   // device copy, or NULL: use `params`
+    ptm_sampling params;
+    uint32_t* ws;
+};
+
+__device__ __forceinline__ ptm_sampling sampler_params(const SamplerArgs& a) { return a.d_params ? *a.d_params : a.params; }
+
+// float -> uint32 whose unsigned order is the float order
+__device__ __forceinline__ uint32_t order_key(float x) {
+    const uint32_t u = __float_as_uint(x);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// the value the selection runs on: penalised logit, over temperature unless greedy
+__device__ __forceinline__ float sampler_value(const SamplerArgs& a, const ptm_sampling& p, int i) {
+    float x = a.logits[i];
+    if (a.counts && p.repeat_penalty > 1.0f) {
+        const int c = a.counts[i];
+        for (int n = 0; n < c; ++n) x = x > 0.0f ? x / p.repeat_penalty : x * p.repeat_penalty;
+    }
+    if (p.temperature >= 1e-6f) x = x / p.temperature;
+    return x + 0.0f;  // -0 -> +0: the reference compares values, the radix select compares bit patterns
+}
+__device__ __forceinline__ int sampler_k(const ptm_sampling& p) { return p.temperature >= 1e-6f ? p.top_k : 1; }
+
+// Which bin, counting from the top, holds the k-th largest key?  All 256 threads call it; returns the bin and how
+// many keys are still wanted inside it.  s_scan: 258 words of LDS.
+__device__ void select_bin(const uint32_t* hist, int nbins, int k, int& bin, int& k_in_bin, uint32_t* s_scan) {
+    const int tid = threadIdx.x, per = nbins / 256;
+    uint32_t mine = 0;
+    for (int j = 0; j < per; ++j) mine += hist[nbins - 1 - (tid * per + j)];
+    __syncthreads();
+    s_scan[tid] = mine;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {  // inclusive scan
+        const uint32_t add = tid >= off ? s_scan[tid - off] : 0;
+        __syncthreads();
+        s_scan[tid] += add;
+        __syncthreads();
+    }
+    const uint32_t incl = s_scan[tid], excl = incl - mine;
+    if (excl < (uint32_t)k && (uint32_t)k <= incl) {
+        uint32_t above = excl;
+        for (int j = 0; j < per; ++j) {
+            const int b = nbins - 1 - (tid * per + j);
+            const uint32_t h = hist[b];
+            if (above + h >= (uint32_t)k) {
+                s_scan[256] = (uint32_t)b;
+                s_scan[257] = (uint32_t)k - above;
+                break;
+            }
+            above += h;
+        }
+    }
+    __syncthreads();
+    bin = (int)s_scan[256];
+    k_in_bin = (int)s_scan[257];
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(256) void sampler_clear_kernel(uint32_t* ws) {
+    for (int i = threadIdx.x + blockIdx.x * 256; i < SW_CLEAR_WORDS; i += 256 * gridDim.x) ws[i] = 0;
+}
+
+// LEVEL 0/1/2: histogram of the level's bits among the keys that share the prefix chosen by the levels above
+template <int LEVEL>
+__global__ __launch_bounds__(256) void sampler_hist_kernel(SamplerArgs a) {
+    constexpr int NB = LEVEL == 2 ? 1024 : 2048;
+    __shared__ uint32_t s_hist[NB];
+    __shared__ uint32_t s_scan[258];
+    const int tid = threadIdx.x;
+    const ptm_sampling p = sampler_params(a);
+    int b0 = 0, b1 = 0, k = sampler_k(p);
+    if (LEVEL >= 1) select_bin(a.ws + SW_HIST0, 2048, k, b0, k, s_scan);
+    if (LEVEL >= 2) select_bin(a.ws + SW_HIST1, 2048, k, b1, k, s_scan);
+    for (int i = tid; i < NB; i += 256) s_hist[i] = 0;
+    __syncthreads();
+    const int base = blockIdx.x * SAMPLER_ELEMS_PER_WG;
+#pragma unroll
+    for (int u = 0; u < SAMPLER_ELEMS_PER_WG / 256; ++u) {
+        const int i = base + tid + 256 * u;
+        if (i < a.vocab) {
+            const uint32_t key = order_key(sampler_value(a, p, i));
+            if (LEVEL == 0) atomicAdd(&s_hist[key >> 21], 1u);
+            else if (LEVEL == 1) { if ((int)(key >> 21) == b0) atomicAdd(&s_hist[(key >> 10) & 0x7ffu], 1u); }
+            else { if ((key >> 10) == (((uint32_t)b0 << 11) | (uint32_t)b1)) atomicAdd(&s_hist[key & 0x3ffu], 1u); }
+        }
+    }
+    __syncthreads();
+    uint32_t* g = a.ws + (LEVEL == 0 ? SW_HIST0 : LEVEL == 1 ? SW_HIST1 : SW_HIST2);
+    for (int i = tid; i < NB; i += 256)
+        if (s_hist[i]) atomicAdd(&g[i], s_hist[i]);
+}
+
+// every key at or above the k-th largest goes to the candidate list (order of arrival; the finish kernel sorts)
+__global__ __launch_bounds__(256) void sampler_gather_kernel(SamplerArgs a) {
+    __shared__ uint32_t s_scan[258];
+    const int tid = threadIdx.x;
+    const ptm_sampling p = sampler_params(a);
+    int b0, b1, b2, k = sampler_k(p);
+    select_bin(a.ws + SW_HIST0, 2048, k, b0, k, s_scan);
+    select_bin(a.ws + SW_HIST1, 2048, k, b1, k, s_scan);
+    select_bin(a.ws + SW_HIST2, 1024, k, b2, k, s_scan);
+    const uint32_t threshold = ((uint32_t)b0 << 21) | ((uint32_t)b1 << 10) | (uint32_t)b2;
+    const int base = blockIdx.x * SAMPLER_ELEMS_PER_WG;
+#pragma unroll
+    for (int u = 0; u < SAMPLER_ELEMS_PER_WG / 256; ++u) {
+        const int i = base + tid + 256 * u;
+        if (i < a.vocab) {
+            const uint32_t key = order_key(sampler_value(a, p, i));
+            if (key >= threshold) {
+                const uint32_t slot = atomicAdd(&a.ws[SW_COUNT], 1u);
+                if (slot < SAMPLER_MAX_CAND) {
+                    a.ws[SW_CAND_KEY + slot] = key;
+                    a.ws[SW_CAND_IDX + slot] = (uint32_t)i;
+                }
+            }
+        }
+    }
+}
+
+// in-LDS bitonic sort of n (power of two) 64-bit keys, ascending, by 1024 threads
+__device__ void bitonic_sort_u64(unsigned long long* v, int n) {
+    for (int size = 2; size <= n; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int t = threadIdx.x; t < n / 2; t += 1024) {
+                const int lo = (t / stride) * 2 * stride + (t % stride), hi = lo + stride;
+                const bool up = ((lo & size) == 0);
+                const unsigned long long x = v[lo], y = v[hi];
+                if ((x > y) == up) { v[lo] = y; v[hi] = x; }
+            }
+        }
+    __syncthreads();
+}
+
+struct SamplerOut {
+    int64_t* out_token;       // chosen id (or -1: more than SAMPLER_MAX_CAND logits tie at the threshold)
+    const float* uniforms;    // r of step s is uniforms[s]
+    const int* d_step;        // NULL: s = 0
+    int32_t* counts_rw;       // NULL, or the occurrence counts to bump for the chosen token
+    ArgmaxAdvance adv;        // step bookkeeping of the decode loop (all NULL outside it)
+};
+
+__global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, SamplerOut o) {
+    __shared__ unsigned long long s_sort[SAMPLER_MAX_CAND];   // 16 KB
+    __shared__ float s_p[SAMPLER_MAX_CAND];                   // x, then p, in index order
+    __shared__ uint32_t s_idx[SAMPLER_MAX_CAND];
+    __shared__ uint8_t s_keep[SAMPLER_MAX_CAND];
+    __shared__ int s_token;
+    const int tid = threadIdx.x;
+    const ptm_sampling p = sampler_params(a);
+    const uint32_t total = a.ws[SW_COUNT];
+    const bool overflow = total > SAMPLER_MAX_CAND;
+    const int m = overflow ? SAMPLER_MAX_CAND : (int)total;
+    int n = 1;
+    while (n < m) n <<= 1;
+    // ---- candidates in index order ----
+    for (int i = tid; i < n; i += 1024)
+        s_sort[i] = i < m ? (((unsigned long long)a.ws[SW_CAND_IDX + i] << 32) | a.ws[SW_CAND_KEY + i]) : ~0ull;
+    bitonic_sort_u64(s_sort, n);
+    for (int i = tid; i < m; i += 1024) {
+        s_idx[i] = (uint32_t)(s_sort[i] >> 32);
+        s_p[i] = key_value((uint32_t)s_sort[i]);
+        s_keep[i] = 1;
+    }
+    __syncthreads();
+    const bool greedy = !(p.temperature >= 1e-6f);
+    if (!greedy) {
+        // ---- softmax over the kept values; sums in index order, as the reference's loops over the vocabulary do
+        // (dropped entries are exp(-1e9 - max) = 0 there and add nothing) ----
+        if (tid == 0) {
+            float mx = s_p[0];
+            for (int i = 1; i < m; ++i) mx = s_p[i] > mx ? s_p[i] : mx;
+            float sum = 0.0f;
+            for (int i = 0; i < m; ++i) { const float e = expf(s_p[i] - mx); s_p[i] = e; sum += e; }
+            const float inv = 1.0f / sum;
+            for (int i = 0; i < m; ++i) s_p[i] *= inv;
+        }
+        __syncthreads();
+        if (p.top_p < 1.0f) {
+            // descending p (ties: lower index first; the reference's std::sort leaves ties unordered); payload = position
+            for (int i = tid; i < n; i += 1024)
+                s_sort[i] = (i < m && s_p[i] > 1e-10f) ? (((unsigned long long)(~__float_as_uint(s_p[i])) << 32) | (uint32_t)i) : ~0ull;
+            bitonic_sort_u64(s_sort, n);
+            for (int i = tid; i < m; i += 1024) s_keep[i] = 0;
+            __syncthreads();
+            if (tid == 0) {
+                float cum = 0.0f;
+                for (int j = 0; j < m; ++j) {
+                    if (s_sort[j] == ~0ull) break;
+                    const int pos = (int)(uint32_t)s_sort[j];
+                    s_keep[pos] = 1;
+                    cum += s_p[pos];
+                    if (cum >= p.top_p) break;
+                }
+                float sum = 0.0f;
+                for (int i = 0; i < m; ++i) { if (!s_keep[i]) s_p[i] = 0.0f; sum += s_p[i]; }
+                if (sum > 0.0f) {
+                    const float inv = 1.0f / sum;
+                    for (int i = 0; i < m; ++i) s_p[i] *= inv;
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (tid == 0) {
+        int token;
+        if (overflow) {
+            token = -1;
+        } else if (greedy) {
+            token = (int)s_idx[0];  // every candidate equals the maximum; index order -> the lowest index
+        } else {
+            const float r = o.uniforms[o.d_step ? *o.d_step : 0];
+            token = a.vocab - 1;
+            if (r <= 0.0f) {
+                token = 0;  // the running sum reaches r at the very first index
+            } else {
+                float cum = 0.0f;
+                for (int i = 0; i < m; ++i) {
+                    cum += s_p[i];
+                    if (cum >= r) { token = (int)s_idx[i]; break; }
+                }
+            }
+        }
+        s_token = token;
+        if (o.out_token) *o.out_token = token;
+        if (o.counts_rw && token >= 0) o.counts_rw[token] += 1;
+        if (o.adv.d_step) {
+            const int st = *o.adv.d_step;
+            if (st < o.adv.cap) o.adv.tokens_out[st] = token;
+            *o.adv.d_token = token < 0 ? 0 : token;
+            *o.adv.d_past = *o.adv.d_past + 1;
+            *o.adv.d_step = st + 1;
+        }
+    }
+}
+
+static int sampler_check(const ptm_sampling& p, int vocab) {
+    if (vocab <= 0) return PTM_E_SHAPE;
+    if (!(p.temperature >= 1e-6f)) return PTM_OK;  // greedy: the other fields are not used
+    if (p.top_k <= 0 || p.top_k >= vocab || p.top_k > SAMPLER_MAX_TOPK) return PTM_E_UNSUPPORTED;
+    if (!(p.top_p > 0.0f)) return PTM_E_SHAPE;
+    return PTM_OK;
+}
+
+// host_params are validated here; when d_params is given the kernels read the device copy (which must hold the same values)
+int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
+                    const ptm_sampling* d_params, const float* d_uniforms, const int* d_step, void* workspace,
+                    int64_t* out_token, int32_t* counts_rw, ArgmaxAdvance adv, hipStream_t s) {
+    if (!logits || !workspace || !d_uniforms) return PTM_E_NULL;
+    const int rc = sampler_check(host_params, vocab);
+    if (rc != PTM_OK) return rc;
+    if (reinterpret_cast<uintptr_t>(workspace) & 7u) return PTM_E_ALIGN;
+    SamplerArgs a{logits, counts, vocab, d_params, host_params, static_cast<uint32_t*>(workspace)};
+    SamplerOut o{out_token, d_uniforms, d_step, counts_rw, adv};
+    const dim3 grid((vocab + SAMPLER_ELEMS_PER_WG - 1) / SAMPLER_ELEMS_PER_WG);
+    hipLaunchKernelGGL(sampler_clear_kernel, dim3(4), dim3(256), 0, s, a.ws);
+    hipLaunchKernelGGL(sampler_hist_kernel<0>, grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL(sampler_hist_kernel<1>, grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL(sampler_hist_kernel<2>, grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL(sampler_gather_kernel, grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL(sampler_finish_kernel, dim3(1), dim3(1024), 0, s, a, o);
+    return launch_status();
+}
+
+}  // namespace ptm
+
+using namespace ptm;
+
+extern "C" {
+
+int64_t ptm_sampler_workspace_bytes(void) { return (int64_t)SW_WORDS * 4; }
+
+int ptm_sample_token(const float* logits, int vocab, const int32_t* counts, const ptm_sampling* params, const float* d_uniform,
+                     void* workspace, int64_t* out_token, ptm_stream_t stream) {
+    if (!params || !out_token) return PTM_E_NULL;
+    return sampler_enqueue(logits, vocab, counts, *params, nullptr, d_uniform, nullptr, workspace, out_token, nullptr,
+                           ArgmaxAdvance{nullptr, nullptr, nullptr, nullptr, 0}, as_stream(stream));
+}
+
+// The reference's draws: `static std::mt19937 rng(42); std::uniform_real_distribution<float> dist(0.0f, 1.0f)`
+// (gguf_model.h:7740-7742): the standard library itself is the definition, one 32-bit output per draw.
+int ptm_mt19937_uniforms(uint32_t seed, int64_t skip, int64_t n, float* out_host) {
+    if (!out_host) return PTM_E_NULL;
+    if (skip < 0 || n < 0) return PTM_E_SHAPE;
+    std::mt19937 rng(seed);
+    rng.discard((unsigned long long)skip);
+    std::uniform_real_distribution<float> dist(0.0f, 1.0f);
+    for (int64_t i = 0; i < n; ++i) out_host[i] = dist(rng);
+    return PTM_OK;
+}
+
+}  // extern "C"

@@ -216,6 +216,20 @@ class GGUFModel:
         check(self.L.ptm_decode_prefill(self.h, buf, n, chunk_rows, C.byref(out)), "decode_prefill")
         return out.value
 
+    def sampling_begin(self, temperature: float, top_k: int, top_p: float, repeat_penalty: float = 1.0) -> None:
+        """Start a sampled generation: store the parameters, forget previously generated tokens."""
+        from ._lib import Sampling
+        check(self.L.ptm_decode_sampling_begin(self.h, Sampling(temperature, top_k, top_p, repeat_penalty)),
+              "decode_sampling_begin")
+
+    def sample(self, token: int, uniforms) -> list:
+        """len(uniforms) chained sampled steps from `token`, one uniform draw per step."""
+        n = len(uniforms)
+        u = (C.c_float * n)(*[float(x) for x in uniforms])
+        buf = (C.c_int64 * n)()
+        check(self.L.ptm_decode_sample(self.h, token, n, u, buf), "decode_sample")
+        return list(buf)
+
     def greedy(self, first_token: int, n: int) -> list:
         buf = (C.c_int64 * n)()
         check(self.L.ptm_decode_greedy(self.h, first_token, n, buf), "decode_greedy")

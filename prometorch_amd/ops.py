@@ -243,6 +243,28 @@ def launch_argmax(input, output, n, stream=None):
     check(_L().ptm_argmax(_ptr(input), _ptr(output), n, _stream(stream)), "argmax")
 
 
+def sampler_workspace_bytes():
+    return int(_L().ptm_sampler_workspace_bytes())
+
+
+def sample_token(logits, vocab, counts, temperature, top_k, top_p, repeat_penalty, d_uniform, workspace, out_token,
+                 stream=None):
+    """GGUFModel::sample_token (gguf_model.h:7658-7751) after the repetition penalty of generate() (:4926-4938), on
+    the device; d_uniform holds the uniform draw, out_token (int64, device) receives the id."""
+    from ._lib import Sampling
+    p = Sampling(temperature, top_k, top_p, repeat_penalty)
+    check(_L().ptm_sample_token(_ptr(logits), vocab, _ptr(counts), p, _ptr(d_uniform), _ptr(workspace), _ptr(out_token),
+                                _stream(stream)), "sample_token")
+
+
+def mt19937_uniforms(seed, skip, n):
+    """The reference sampler's uniform draws: std::uniform_real_distribution<float>(0, 1) over std::mt19937(seed)."""
+    import ctypes as C
+    buf = (C.c_float * n)()
+    check(_L().ptm_mt19937_uniforms(seed, skip, n, buf), "mt19937_uniforms")
+    return list(buf)
+
+
 def launch_add(a, b, out, n, stream=None):
     """CUDAOps.h:63"""
     check(_L().ptm_add(_ptr(a), _ptr(b), _ptr(out), n, _stream(stream)), "add")

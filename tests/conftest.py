@@ -29,6 +29,12 @@ def golden_cfg4():
 
 
 @pytest.fixture(scope="session")
+def golden_sampling():
+    """Tokens the compiled reference's sample_token drew for synth.SAMPLING_CASES, in order."""
+    return np.load(os.path.join(GOLDEN_DIR, "golden_sampling.npz"), allow_pickle=False)["tokens"]
+
+
+@pytest.fixture(scope="session")
 def seeds():
     import json
     with open(os.path.join(GOLDEN_DIR, "golden_meta.json")) as f:

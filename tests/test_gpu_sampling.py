@@ -1,0 +1,183 @@
+"""GPU parity of the device sampler (ptm_sample_token, ptm_decode_sample) against the CPU oracle's restatement of
+GGUFModel::sample_token (torch/io/gguf_model.h:7658-7751) and of the repetition penalty (:4926-4938).
+
+Bar: the same token as the oracle for the same uniform draw r whenever r is further than GAP_TOL from the edges of
+that token's interval of the cumulative distribution (device expf and glibc expf may differ in the last bit, which
+moves the edges by ~1e-7)."""
+import numpy as np
+import pytest
+import torch
+
+from prometorch_amd import ops, synth
+from prometorch_amd._lib import PtmError
+
+pytestmark = pytest.mark.gpu
+
+GAP_TOL = 1e-5
+
+
+def cu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def gpu_sample(x, temperature, top_k, top_p, r, counts=None, penalty=1.0):
+    ws = torch.empty(ops.sampler_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    ws.fill_(0xAB)  # contents must not matter
+    out = torch.full((1,), -7, dtype=torch.int64, device="cuda")
+    ops.sample_token(cu(x), x.size, None if counts is None else cu(counts.astype(np.int32)), temperature, top_k, top_p,
+                     penalty, cu(np.array([r], np.float32)), ws, out)
+    torch.cuda.synchronize()
+    return int(out.item())
+
+
+def supported(vocab, temperature, top_k):
+    return temperature < 1e-6 or (1 <= top_k <= 1024 and top_k < vocab)
+
+
+def test_mt19937_uniforms_are_the_reference_sequence(po):
+    g = po.MT19937(42)
+    want = [g.uniform01() for _ in range(300)]
+    assert ops.mt19937_uniforms(42, 0, 300) == want
+    assert ops.mt19937_uniforms(42, 100, 50) == want[100:150]
+    assert abs(want[0] - 0.3745401) < 1e-7
+
+
+def test_sample_token_cases_vs_oracle_and_reference_golden(dev, po, golden_sampling):
+    rng = po.MT19937(42)
+    checked = 0
+    for i, (vocab, kind, temperature, top_k, top_p) in enumerate(synth.SAMPLING_CASES):
+        x = synth.sampling_logits(i)
+        r = rng.uniform01() if temperature >= 1e-6 else 0.0
+        if not supported(vocab, temperature, top_k):
+            with pytest.raises(PtmError) as e:
+                gpu_sample(x, temperature, top_k, top_p, r)
+            assert e.value.code == -4
+            continue
+        tok_o, gap = po.sample_token(x, temperature, top_k, top_p, r)
+        assert tok_o == int(golden_sampling[i])        # the oracle is the compiled reference here
+        tok_g = gpu_sample(x, temperature, top_k, top_p, r)
+        print(i, vocab, kind, temperature, top_k, top_p, "r %.6f gap %.2e" % (r, gap), tok_g, tok_o, flush=True)
+        if gap > GAP_TOL:
+            assert tok_g == tok_o, i
+            checked += 1
+    assert checked >= 30
+
+
+@pytest.mark.parametrize("vocab,kind_case,temperature,top_k,top_p", [(1000, 0, 0.8, 40, 0.9), (151936, 12, 0.8, 40, 0.9),
+                                                                      (151936, 18, 1.0, 1024, 0.95), (1000, 3, 1.3, 7, 1.0),
+                                                                      (151936, 19, 0.5, 2, 0.5)])
+def test_sample_token_many_draws(dev, po, vocab, kind_case, temperature, top_k, top_p):
+    """The whole inverse CDF: 64 draws spread over (0, 1) plus the edges."""
+    x = synth.sampling_logits(kind_case)
+    assert x.size == vocab
+    rs = list(np.random.default_rng(kind_case).random(60).astype(np.float32)) + [0.0, 1e-30, 0.99999994, 0.5]
+    checked = 0
+    for r in rs:
+        tok_o, gap = po.sample_token(x, temperature, top_k, top_p, float(r))
+        tok_g = gpu_sample(x, temperature, top_k, top_p, float(r))
+        if gap > GAP_TOL or r == 0.0:
+            assert tok_g == tok_o, (float(r), gap)
+            checked += 1
+    assert checked >= 55
+
+
+def test_sample_token_with_repetition_penalty(dev, po):
+    vocab = 5000
+    g = synth.rng_for(81)
+    x = (3 * g.standard_normal(vocab, dtype=np.float32)).astype(np.float32)
+    top = np.argsort(x)[::-1]
+    generated = [int(top[0])] * 3 + [int(top[1]), int(top[5]), int(top[5]), int(np.argmin(x)), 17, 17, 17, 17]
+    counts = np.bincount(generated, minlength=vocab)
+    for penalty in (1.1, 1.5, 1.0):
+        xp = po.repetition_penalty(x, generated, penalty)
+        for r in (0.05, 0.31, 0.77, 0.93):
+            tok_o, gap = po.sample_token(xp, 0.8, 40, 0.9, r)
+            tok_g = gpu_sample(x, 0.8, 40, 0.9, r, counts=counts, penalty=penalty)
+            if gap > GAP_TOL:
+                assert tok_g == tok_o, (penalty, r)
+        # greedy over the penalised logits
+        assert gpu_sample(x, 0.0, 40, 0.9, 0.5, counts=counts, penalty=penalty) == int(np.argmax(xp))
+    # penalty 1.5 three times on the best token must dethrone it
+    assert int(np.argmax(po.repetition_penalty(x, generated, 1.5))) != int(top[0])
+
+
+def test_sample_token_greedy_ties_and_edges(dev, po):
+    x = np.zeros(3000, np.float32)
+    x[[5, 77, 2999]] = 4.0
+    assert gpu_sample(x, 0.0, 1, 1.0, 0.9) == 5                       # argmax: lowest index of the tied maxima
+    assert gpu_sample(x, 1.0, 2, 1.0, 0.99) == 2999                   # top-2 keeps all three ties; last interval
+    assert gpu_sample(x, 1.0, 2, 1.0, 0.5) == 77
+    assert gpu_sample(x, 1.0, 3, 1.0, 0.0) == 0                       # r = 0: index 0, whatever its probability
+    x = np.array([-0.0, 0.0, -1.0, 0.0], np.float32)                  # -0 and +0 are the same value to the reference
+    tok_o, _ = po.sample_token(x, 1.0, 2, 1.0, 0.5)
+    assert gpu_sample(x, 1.0, 2, 1.0, 0.5) == tok_o
+    flat = np.zeros(5000, np.float32)                                 # 5000 logits tie at the threshold: more than the list holds
+    assert gpu_sample(flat, 1.0, 4, 1.0, 0.5) == -1
+    flat2 = np.zeros(2048, np.float32)                                # exactly as many as it holds
+    tok_o, _ = po.sample_token(flat2, 1.0, 4, 1.0, 0.5)
+    assert gpu_sample(flat2, 1.0, 4, 1.0, 0.5) == tok_o
+
+
+def test_sample_token_argument_errors(dev):
+    x = np.zeros(100, np.float32)
+    for temperature, top_k, top_p in ((0.8, 0, 0.9), (0.8, 100, 0.9), (0.8, 2000, 0.9), (0.8, 40, 0.0)):
+        with pytest.raises(PtmError):
+            gpu_sample(x, temperature, top_k, top_p, 0.5)
+
+
+def build_tiny(seeds):
+    cfg = dict(synth.TINY)
+    layers = [synth.make_layer(seeds["tiny"], i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(seeds["tiny"], cfg)
+    return cfg, layers, head
+
+
+@pytest.mark.parametrize("use_graph", [True, False])
+@pytest.mark.parametrize("temperature,top_k,top_p,penalty", [(0.8, 40, 0.9, 1.1), (1.2, 8, 1.0, 1.0), (0.0, 40, 0.9, 1.3)])
+def test_decoder_sampled_generation_vs_oracle_loop(dev, po, seeds, use_graph, temperature, top_k, top_p, penalty):
+    """The reference's decode loop (api_handlers.h:848-923): penalise with the generated tokens, sample, feed back."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = build_tiny(seeds)
+    om = po.OracleModel(cfg, layers, head, 96, kv_fp16=True)
+    dec = Decoder(cfg, layers, head, max_seq=96, kv_fp16=True, use_graph=use_graph)
+    prompt = [int(t) for t in synth.rng_for(82).integers(0, cfg["vocab"], 9)]
+    for t in prompt[:-1]:
+        om.step(t)
+        dec.step(t)
+    n = 40
+    us = ops.mt19937_uniforms(42, 0, n)
+    dec.sampling_begin(temperature, top_k, top_p, penalty)
+    got = dec.sample(prompt[-1], us[:25]) 
+    got += dec.sample(got[-1], us[25:])            # a second run continues the same generation (counts are kept)
+    tok, generated, min_gap = prompt[-1], [], 1.0
+    for st in range(n):
+        om.step(tok)
+        lg = po.repetition_penalty(om.logits, generated, penalty) if generated else om.logits
+        tok, gap = po.sample_token(lg, temperature, top_k, top_p, us[st])
+        if gap <= 1e-4:
+            break                                  # a draw on an interval edge: both answers are legitimate, stop comparing
+        min_gap = min(min_gap, gap)
+        assert got[st] == tok, (st, gap)
+        generated.append(tok)
+    print("compared %d sampled steps, smallest gap %.2e" % (len(generated), min_gap), flush=True)
+    assert len(generated) >= 20
+    # sampling_begin forgets the history: the same draws from the same state reproduce the same tokens
+    dec.set_past_len(len(prompt) - 1)
+    dec.sampling_begin(temperature, top_k, top_p, penalty)
+    assert dec.sample(prompt[-1], us) == got
+    dec.close()
+
+
+def test_decoder_sampling_errors(dev, seeds):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = build_tiny(seeds)
+    dec = Decoder(cfg, layers, head, max_seq=32, kv_fp16=True, use_graph=False)
+    with pytest.raises(PtmError):
+        dec.sample(1, [0.5])                       # no sampling_begin yet
+    with pytest.raises(PtmError):
+        dec.sampling_begin(0.8, 0, 0.9)            # top-k off: not on the device
+    dec.sampling_begin(0.8, 40, 0.9)
+    with pytest.raises(PtmError):
+        dec.sample(1, [0.5] * 33)                  # would overflow the cache
+    assert len(dec.sample(1, [0.5] * 4)) == 4
+    dec.close()
