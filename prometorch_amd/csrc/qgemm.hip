@@ -419,21 +419,21 @@ struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh
     static constexpr bool kQ8Round = false;
 };
 
-// X tile of a super-block step in LDS: thread t owns row t/2, byte half t%2 (256 B = 16 pieces of 16 B).  The
-// pieces of the NEXT block are fetched three per sub-block step during steps 0..5 of the current block and written
-// to the other LDS buffer two steps later, so a fetch has two step times to arrive and the block ends with the
-// next tile complete behind the only workgroup barrier of the block.  (After the last block the same code
-// re-fetches the last tile into the idle buffer: no conditionals in the steady-state loop.)
-template <typename Tile>
-__global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
+// X tile of a super-block step in LDS.  The 16 pieces a thread owns of the NEXT block's tile are fetched at step 0
+// of the current block, followed by the next block's weights, and written to the other LDS buffer during steps
+// 3..6, so the block ends with the next tile complete behind the only workgroup barrier of the block.  (After the
+// last block the same code re-fetches the last tile into the idle buffer: no conditionals in the steady-state loop.)
+template <typename Tile, int MT>
+__global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
                                                         const float* __restrict__ rowscale, float* Y, int M, int K, int N,
                                                         int accumulate, int blocks_per_split, float* partials) {
     // W and Xh are deliberately not __restrict__: loads through a restrict pointer may be moved across the
     // compiler fences below, and the prefetch distance of this loop depends on those fences
-    extern __shared__ __align__(16) uint8_t s_a[];  // [2][QF_TM * QF_PITCH]
+    constexpr int TM = 32 * MT;                     // rows of X per workgroup (MT tiles of 32)
+    extern __shared__ __align__(16) uint8_t s_a[];  // [2][TM * QF_PITCH]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, kh = lane >> 5;
-    const int m0 = blockIdx.y * QF_TM;
+    const int m0 = blockIdx.y * TM;
     const int n_base = blockIdx.x * QF_TN + wave * 64;
     // split K: workgroup z of the grid sums super-blocks [blk0, blk0 + nblk) into its own M x N partial
     const int blk0 = blockIdx.z * blocks_per_split;
@@ -443,9 +443,9 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
     for (int t = 0; t < 2; ++t)
         wrow[t] = W + (int64_t)min(n_base + 32 * t + j, N - 1) * stride + (int64_t)blk0 * Tile::kBlockBytes;
 
-    f32x16 acc[4][2];
+    f32x16 acc[MT][2];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -457,11 +457,12 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
     const uint8_t* x_src = reinterpret_cast<const uint8_t*>(Xh) + (int64_t)(m0 + (tid >> 5)) * x_row_bytes + 16 * (tid & 31) +
                            (int64_t)blk0 * 512;
     uint8_t* x_dst = s_a + (tid >> 5) * QF_PITCH + 16 * (tid & 31);
-    uint4 re0, re1, re2, ro0, ro1, ro2;  // pieces in flight: fetched at an even / odd step (scalars, not an array: they must stay in registers)
-    re0 = re1 = re2 = ro0 = ro1 = ro2 = make_uint4(0, 0, 0, 0);
+    // the 16 pieces of the next tile in flight (scalars, not an array: they must stay in registers)
+    static_assert(MT == 1 || MT == 2 || MT == 4, "row tiles per workgroup");
+    uint4 x0, x1, x2, x3, x4, x5, x6, x7, x8, x9, x10, x11, x12, x13, x14, x15;
     // prologue: tile of block 0 -> LDS buffer 0, weights of block 0, fragments of step 0
 #pragma unroll
-    for (int p = 0; p < 16; ++p)
+    for (int p = 0; p < 4 * MT; ++p)
         *reinterpret_cast<uint4*>(x_dst + 8 * p * QF_PITCH) = *reinterpret_cast<const uint4*>(x_src + 8 * p * x_row_bytes);
     Tile cur[2], nxt[2];
 #pragma unroll
@@ -473,43 +474,50 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
 
     for (int blk = 0; blk < nblk; ++blk) {
         const int nb = min(blk + 1, nblk - 1);  // block whose tile and weights are fetched during this one
-        const uint8_t* a_cur = s_a + (blk & 1) * (QF_TM * QF_PITCH);
-        uint8_t* x_nxt = x_dst + ((blk & 1) ^ 1) * (QF_TM * QF_PITCH);
+        const uint8_t* a_cur = s_a + (blk & 1) * (TM * QF_PITCH);
+        uint8_t* x_nxt = x_dst + ((blk & 1) ^ 1) * (TM * QF_PITCH);
         const uint8_t* x_from = x_src + (int64_t)nb * 512;
-        h8 af[2][4];  // X fragments of step 0 of this block (the tile became visible at the barrier)
+        h8 af[2][MT];  // X fragments of step 0 of this block (the tile became visible at the barrier)
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
+            for (int mt = 0; mt < MT; ++mt)
                 af[ks][mt] = *reinterpret_cast<const h8*>(a_cur + (mt * 32 + j) * QF_PITCH + 32 * kh + 16 * ks);
 #pragma unroll
         for (int s = 0; s < 8; ++s) {  // unrolled: the sub-block index selects registers
-            if (s >= 2) {  // pieces fetched two steps ago -> LDS
-                const int p = 3 * (s - 2);
-                *reinterpret_cast<uint4*>(x_nxt + 8 * p * QF_PITCH) = (s & 1) ? ro0 : re0;
-                if (p + 1 < 16) *reinterpret_cast<uint4*>(x_nxt + 8 * (p + 1) * QF_PITCH) = (s & 1) ? ro1 : re1;
-                if (p + 2 < 16) *reinterpret_cast<uint4*>(x_nxt + 8 * (p + 2) * QF_PITCH) = (s & 1) ? ro2 : re2;
-            }
-            if (s < 6) {
-                const int p = 3 * s;
-                const uint4 v0 = *reinterpret_cast<const uint4*>(x_from + 8 * p * x_row_bytes);
-                const uint4 v1 = *reinterpret_cast<const uint4*>(x_from + 8 * min(p + 1, 15) * x_row_bytes);
-                const uint4 v2 = *reinterpret_cast<const uint4*>(x_from + 8 * min(p + 2, 15) * x_row_bytes);
-                if (s & 1) { ro0 = v0; ro1 = v1; ro2 = v2; } else { re0 = v0; re1 = v1; re2 = v2; }
-            }
+#define QF_LD(p) (*reinterpret_cast<const uint4*>(x_from + 8 * (p) * x_row_bytes))
+#define QF_ST(p, v) (*reinterpret_cast<uint4*>(x_nxt + 8 * (p) * QF_PITCH) = (v))
             if (s == 0) {
+                // All fetches of the block are issued here, tile pieces FIRST: loads return in order, so a wait for a
+                // piece must not have the weight loads (HBM latency, one cache line per lane) in front of it.  The
+                // pieces are written to LDS in steps 3..6 with the weights still in flight; the weights are first
+                // needed at step 7.
+                x0 = QF_LD(0); x1 = QF_LD(1); x2 = QF_LD(2); x3 = QF_LD(3);
+                if constexpr (MT >= 2) { x4 = QF_LD(4); x5 = QF_LD(5); x6 = QF_LD(6); x7 = QF_LD(7); }
+                if constexpr (MT >= 4) {
+                    x8 = QF_LD(8); x9 = QF_LD(9); x10 = QF_LD(10); x11 = QF_LD(11); x12 = QF_LD(12);
+                    x13 = QF_LD(13); x14 = QF_LD(14); x15 = QF_LD(15);
+                }
 #pragma unroll
                 for (int t = 0; t < 2; ++t) nxt[t].load(wrow[t] + (int64_t)nb * Tile::kBlockBytes, kh);
             }
+            if (s == 3) { QF_ST(0, x0); QF_ST(1, x1); QF_ST(2, x2); QF_ST(3, x3); }
+            if constexpr (MT >= 2) { if (s == 4) { QF_ST(4, x4); QF_ST(5, x5); QF_ST(6, x6); QF_ST(7, x7); } }
+            if constexpr (MT >= 4) {
+                if (s == 5) { QF_ST(8, x8); QF_ST(9, x9); QF_ST(10, x10); QF_ST(11, x11); }
+                if (s == 6) { QF_ST(12, x12); QF_ST(13, x13); QF_ST(14, x14); QF_ST(15, x15); }
+            }
+#undef QF_LD
+#undef QF_ST
             issue_order_fence();  // the fetches stay HERE, two steps ahead of their use (the compiler would sink them to it)
             // X fragments of the NEXT step are read from LDS now and weight fragments of the next step are prepared
             // while this step's 16 MFMAs (all operands already in registers) run
-            h8 an[2][4];
+            h8 an[2][MT];
             if (s < 7) {
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                    for (int mt = 0; mt < 4; ++mt)
+                    for (int mt = 0; mt < MT; ++mt)
                         an[ks][mt] = *reinterpret_cast<const h8*>(a_cur + (mt * 32 + j) * QF_PITCH + 64 * (s + 1) + 32 * kh + 16 * ks);
             }
 #if defined(PTM_EXP) && PTM_EXP == 11
@@ -525,17 +533,21 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt)
+                for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                     for (int t = 0; t < 2; ++t)
+#if defined(PTM_EXP) && PTM_EXP == 12
+                        acc[mt][t][0] += (float)af[ks][mt][0] * (float)bf[t][ks][0];
+#else
                         acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks][mt], bf[t][ks], acc[mt][t], 0, 0, 0);
+#endif
             // issue order: one MFMA, then the vector work that fits under it (a 32x32x16 MFMA occupies the matrix pipe
             // for 32 cycles = 8 vector instructions), so that neither pipe waits for the other
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < 4 * MT; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
-                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);   // VALU
+                __builtin_amdgcn_sched_group_barrier(0x002, 24 / MT, 0);   // VALU
             }
 #pragma unroll
             for (int t = 0; t < 2; ++t) { bf[t][0] = bn[t][0]; bf[t][1] = bn[t][1]; }
@@ -543,7 +555,7 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                    for (int mt = 0; mt < 4; ++mt) af[ks][mt] = an[ks][mt];
+                    for (int mt = 0; mt < MT; ++mt) af[ks][mt] = an[ks][mt];
             }
         }
 #pragma unroll
@@ -552,7 +564,7 @@ __global__ __launch_bounds__(256) void qgemm_f16_kernel(const uint8_t* W, int64_
     }
     // C layout of the 32x32 tile: column j = lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
@@ -609,6 +621,16 @@ int qgemm_f16_splits(int N, int K) {
     return s < 1 ? 1 : s;
 }
 
+// Rows per workgroup in tiles of 32: 4 (128 rows: each dequantised weight serves twice as many products) unless that
+// leaves most of the chip idle; then 2 (64 rows, two workgroups per CU).  The Q6_K variant of the small tile does
+// not fit its registers, so it is used only where the big tile would be half empty anyway.  A row's sum does not
+// depend on the choice (same K order).
+static int qgemm_f16_row_tiles(bool q4, int M, int N, int splits) {
+    if (M <= 64) return 2;
+    const int wgs = ((N + QF_TN - 1) / QF_TN) * ((M + 127) / 128) * splits;
+    return (q4 && wgs < 200) ? 2 : 4;
+}
+
 static int qgemm_check(const void* W, const void* X, const void* Y, int M, int K, int N, int64_t stride, int blk_bytes) {
     if (!W || !X || !Y) return PTM_E_NULL;
     if (M <= 0 || N <= 0 || K <= 0 || (K % 256) != 0) return PTM_E_SHAPE;
@@ -633,37 +655,44 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     if (ggml_type == PTM_TYPE_Q4_K ? (!aligned16(W) || (stride & 15)) : ((stride & 1) || (reinterpret_cast<uintptr_t>(W) & 1u)))
         return PTM_E_ALIGN;
     const int mp = qf_mpad(M);
-    if (mp / QF_TM > 65535) return PTM_E_UNSUPPORTED;
+    if (mp / 32 > 65535) return PTM_E_UNSUPPORTED;
     _Float16* Xh = static_cast<_Float16*>(workspace);
     float* rowscale = reinterpret_cast<float*>(Xh + (int64_t)mp * K);
-    const size_t lds = 2 * (size_t)QF_TM * QF_PITCH;  // 132 KB: above the default 64 KB cap of dynamic LDS
-    static bool raised = false;
-    if (!raised) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        raised = true;
-    }
     const int nblk = K / 256;
     int splits = split_ws ? qgemm_f16_splits(N, K) : 1;
     while (splits > 1 && (size_t)splits * M * N * sizeof(float) > split_ws_bytes) --splits;
     const int bps = (nblk + splits - 1) / splits;
     splits = (nblk + bps - 1) / bps;  // no empty split
     float* partials = splits > 1 ? split_ws : nullptr;
-    const dim3 grid((N + QF_TN - 1) / QF_TN, mp / QF_TM, splits);
     const int acc = accumulate ? 1 : 0;
-    if (ggml_type == PTM_TYPE_Q4_K) {
-        if (reuse_rows) {}
-        else if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
-        else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
-        hipLaunchKernelGGL(qgemm_f16_kernel<Q4Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
-                           rowscale, Y, M, K, N, acc, bps, partials);
-    } else {
-        if (reuse_rows) {}
+    const bool q4 = ggml_type == PTM_TYPE_Q4_K;
+    if (!reuse_rows) {
+        if (q4 && x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
+        else if (q4) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<true, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         else if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
-        hipLaunchKernelGGL(qgemm_f16_kernel<Q6Tile>, grid, dim3(256), lds, s, static_cast<const uint8_t*>(W), stride, Xh,
-                           rowscale, Y, M, K, N, acc, bps, partials);
     }
+    // rows per workgroup: 64 (two workgroups share a CU, so one's memory waits hide behind the other's arithmetic) or
+    // 128 (half the dequantisation work per product)
+    static const int mt_env = [] { const char* e = getenv("PTM_QGEMM_MT"); return e ? atoi(e) : 0; }();
+    const int MT = (mt_env == 2 || mt_env == 4) ? mt_env : qgemm_f16_row_tiles(q4, M, N, splits);
+    const int tm = 32 * MT;
+    const size_t lds = 2 * (size_t)tm * QF_PITCH;  // 132 KB / 66 KB: above the default 64 KB cap of dynamic LDS
+    static bool raised = false;
+    if (!raised) {
+        const int big = 2 * 128 * QF_PITCH, small = 2 * 64 * QF_PITCH;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
+        raised = true;
+    }
+    const dim3 grid((N + QF_TN - 1) / QF_TN, (M + tm - 1) / tm, splits);
+    const uint8_t* Wb = static_cast<const uint8_t*>(W);
+    if (q4 && MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    else if (q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    else if (MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    else hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     if (partials) {
         const int64_t total = (int64_t)M * N;
         hipLaunchKernelGGL(qgemm_split_reduce_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, partials, splits,
