@@ -165,29 +165,36 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
     constexpr int NOUT = HD / 4, NSLOT = 256 / NOUT;
     __shared__ __align__(16) float4 s_stage[256];
     __shared__ float s_red[8];
-    int64_t total = *d_past + 1;
-    if (total > max_seq) total = max_seq;
-    if (total <= 0) return;
-    const int ns = (int)((total + FD_CHUNK - 1) / FD_CHUNK);
     const int h = blockIdx.x, tid = threadIdx.x;
     const int o_idx = tid % NOUT, slot = tid / NOUT;
     const float4* pO4 = reinterpret_cast<const float4*>(pO);
+    // Every load of the common case goes out before the position is known: chunk slots past the last active one
+    // are clamped into the allocation (ns_max chunks) and dropped by selects below, so the kernel makes one
+    // memory round trip, not one for the position and a second for the data.
+    const int ns_max = (max_seq + FD_CHUNK - 1) / FD_CHUNK;
+    const int64_t past = *d_past;
     float4 v[8];
     float mm[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-        const int sc = min(slot + u * NSLOT, ns - 1);
+        const int sc = min(slot + u * NSLOT, ns_max - 1);
         v[u] = pO4[((int64_t)sc * n_heads + h) * NOUT + o_idx];
         mm[u] = pM[(int64_t)sc * n_heads + h];
     }
-    float m = -INFINITY;
-    for (int sI = tid; sI < ns; sI += 256) m = fmaxf(m, pM[(int64_t)sI * n_heads + h]);
+    const int s_first = min(tid, ns_max - 1);
+    const float pm_first = pM[(int64_t)s_first * n_heads + h], pl_first = pL[(int64_t)s_first * n_heads + h];
+    int64_t total = past + 1;
+    if (total > max_seq) total = max_seq;
+    if (total <= 0) return;
+    const int ns = (int)((total + FD_CHUNK - 1) / FD_CHUNK);
+    float m = tid < ns ? pm_first : -INFINITY;
+    for (int sI = tid + 256; sI < ns; sI += 256) m = fmaxf(m, pM[(int64_t)sI * n_heads + h]);
     m = max64(m);
     if ((tid & 63) == 0) s_red[tid >> 6] = m;
     __syncthreads();
     const float M = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    float den = 0.0f;
-    for (int sI = tid; sI < ns; sI += 256)
+    float den = tid < ns ? expf(pm_first - M) * pl_first : 0.0f;
+    for (int sI = tid + 256; sI < ns; sI += 256)
         den = fmaf(expf(pM[(int64_t)sI * n_heads + h] - M), pL[(int64_t)sI * n_heads + h], den);
     den = sum64(den);
     if ((tid & 63) == 0) s_red[4 + (tid >> 6)] = den;
@@ -203,11 +210,12 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const float w = (s0 + u * NSLOT) < ns ? expf(mm[u] - M) : 0.0f;
-            sum.x = fmaf(w, v[u].x, sum.x);
-            sum.y = fmaf(w, v[u].y, sum.y);
-            sum.z = fmaf(w, v[u].z, sum.z);
-            sum.w = fmaf(w, v[u].w, sum.w);
+            const bool on = (s0 + u * NSLOT) < ns;  // a select, not a zero weight: inactive slots may hold anything
+            const float w = expf(mm[u] - M);
+            sum.x = on ? fmaf(w, v[u].x, sum.x) : sum.x;
+            sum.y = on ? fmaf(w, v[u].y, sum.y) : sum.y;
+            sum.z = on ? fmaf(w, v[u].z, sum.z) : sum.z;
+            sum.w = on ? fmaf(w, v[u].w, sum.w) : sum.w;
         }
     }
     s_stage[slot * NOUT + o_idx] = sum;
