@@ -351,6 +351,12 @@ int ptm_gguf_find_tensor(const ptm_gguf* g, const char* name, ptm_gguf_tensor* o
 int ptm_gguf_get_int(const ptm_gguf* g, const char* key, int64_t* out);
 int ptm_gguf_get_float(const ptm_gguf* g, const char* key, double* out);
 const char* ptm_gguf_get_string(const ptm_gguf* g, const char* key);
+/* Array-valued metadata: element type (GGUF code: 0 u8, 1 i8, 2 u16, 3 i16, 4 u32, 5 i32, 6 f32, 7 bool, 8 string,
+ * 10 u64, 11 i64, 12 f64) and count; element i of a string array as (pointer into the mapping, length), not
+ * NUL-terminated; the packed little-endian elements of a numeric array.  GGUFValue::as_array (gguf_loader.h:69-89). */
+int ptm_gguf_get_array(const ptm_gguf* g, const char* key, uint32_t* elem_type, int64_t* count);
+int ptm_gguf_array_string(const ptm_gguf* g, const char* key, int64_t i, const char** data, int64_t* len);
+const void* ptm_gguf_array_data(const ptm_gguf* g, const char* key);
 
 /* From a .gguf file to a ready decoder: reads the `qwen3` hyper-parameters
  * (<arch>.block_count, embedding_length, feed_forward_length, attention.head_count(_kv),
@@ -365,6 +371,34 @@ ptm_decoder* ptm_model_decoder(ptm_model* m); /* owned by the model */
 int ptm_model_config(const ptm_model* m, ptm_decode_config* out);
 int ptm_model_layer(const ptm_model* m, int i, ptm_layer* out);
 void ptm_model_free(ptm_model* m);
+
+/* ---- tokenizer and chat template (host only) ----------------------------------------------------
+ * GGUFTokenizer (torch/io/tokenizer.h:24-643): byte-level BPE ("gpt2": Qwen, Llama-3) or word-marker BPE /
+ * greedy longest match (any other tokenizer.ggml.model), special tokens matched first, <0xNN> byte fallback.
+ * Same ids and same decoded bytes as the reference.  One difference: on a UTF-8 continuation byte that does not
+ * follow a letter the reference's "gpt2" splitter never returns; here the byte becomes a word of its own.
+ * Buffers are the caller's: a result that does not fit returns PTM_E_RANGE with the needed size in *n_ids / *len. */
+typedef struct ptm_tokenizer ptm_tokenizer;
+int ptm_tokenizer_create(const char* const* tokens, const int32_t* token_lens, int32_t n_tokens, const char* const* merges,
+                         const int32_t* merge_lens, int32_t n_merges, const char* model_type, int32_t bos_id,
+                         int32_t eos_id, int32_t pad_id, int32_t unk_id, int add_bos, ptm_tokenizer** out);
+/* GGUFTokenizer::load (tokenizer.h:42-121): tokenizer.ggml.{model,tokens,merges,*_token_id,add_bos_token}. */
+int ptm_tokenizer_from_gguf(const ptm_gguf* g, ptm_tokenizer** out);
+void ptm_tokenizer_free(ptm_tokenizer* t);
+int32_t ptm_tokenizer_vocab_size(const ptm_tokenizer* t);
+int ptm_tokenizer_special_ids(const ptm_tokenizer* t, int32_t* bos, int32_t* eos, int32_t* pad, int32_t* unk);
+/* encode (tokenizer.h:127-155), decode (:161-175), decode_token (:177-182). */
+int ptm_tokenizer_encode(const ptm_tokenizer* t, const char* text, int64_t text_len, int use_bos, int32_t* ids,
+                         int64_t cap, int64_t* n_ids);
+int ptm_tokenizer_decode(const ptm_tokenizer* t, const int32_t* ids, int64_t n_ids, int skip_special, char* out,
+                         int64_t cap, int64_t* len);
+int ptm_tokenizer_token(const ptm_tokenizer* t, int32_t id, char* out, int64_t cap, int64_t* len);
+/* GGUFModel::apply_chat_template (gguf_model.h:4178-4236): ChatML for qwen2/qwen3 (no_think adds "/no_think" to the
+ * system turn of qwen3), Phi-3, Gemma, Llama-3, Mistral (architecture "llama" with "mistral" in the model name), the
+ * bare prompt otherwise.  system: NULL = "You are a helpful assistant.", "" = no system turn (the reference reads
+ * PT_SYSTEM_PROMPT / PT_NO_THINK from the environment instead). */
+int ptm_chat_template(const char* architecture, const char* model_name, const char* system, int no_think,
+                      const char* prompt, char* out, int64_t cap, int64_t* len);
 
 #ifdef __cplusplus
 }

@@ -26,6 +26,8 @@
  *   po_sample_token        golden tokens of the compiled reference's sample_token over seeded logits and
  *                          parameter sets + numpy float64 restatement (top-k by partition, softmax,
  *                          nucleus cut, inverse CDF)
+ *   (tokenizer, chat template: no restatement here; the library's host code is compared directly with
+ *                          the compiled reference's outputs in tests/golden/golden_tokenizer.json)
  *   po_repetition_penalty  numpy restatement with repeated ids (the reference applies the penalty once per
  *                          occurrence); the reference holds it inline in generate(), so no compiled check
  */

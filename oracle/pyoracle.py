@@ -327,6 +327,19 @@ def ref():
         R.ref_model_decode.argtypes = [_vp, _i64, _vp]
         R.ref_sample_token.restype = _i32
         R.ref_sample_token.argtypes = [_vp, _vp, _i64, _f32, _i32, _f32]
+        R.ref_tokenizer_load.restype = _vp
+        R.ref_tokenizer_load.argtypes = [C.c_char_p]
+        R.ref_tokenizer_free.argtypes = [_vp]
+        R.ref_tokenizer_encode.restype = _i64
+        R.ref_tokenizer_encode.argtypes = [_vp, C.c_char_p, _i64, _i32, _vp, _i64]
+        R.ref_tokenizer_decode.restype = _i64
+        R.ref_tokenizer_decode.argtypes = [_vp, _vp, _i64, _i32, C.c_char_p, _i64]
+        R.ref_tokenizer_token.restype = _i64
+        R.ref_tokenizer_token.argtypes = [_vp, _i32, C.c_char_p, _i64]
+        R.ref_chat_template.restype = _i64
+        R.ref_chat_template.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p, _i64]
+        R.ref_gguf_n_tensors.restype = _i64
+        R.ref_gguf_n_tensors.argtypes = [C.c_char_p]
         _ref = R
     return _ref
 

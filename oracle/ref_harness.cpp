@@ -191,4 +191,48 @@ int32_t ref_sample_token(void* h, const float* logits, int64_t vocab, float temp
     return static_cast<RefModel*>(h)->m.sample_token(vec_tensor(logits, vocab), temperature, top_k, top_p);
 }
 
+// ---------------------------------------------------------------------------------
+// GGUFTokenizer (torch/io/tokenizer.h) loaded by the reference's own GGUFReader (torch/io/gguf_loader.h) from a
+// .gguf file, and GGUFModel::apply_chat_template (torch/io/gguf_model.h:4178-4236).
+// ---------------------------------------------------------------------------------
+void* ref_tokenizer_load(const char* gguf_path) {
+    g::GGUFReader reader;
+    reader.open(gguf_path);
+    auto* t = new torch::io::GGUFTokenizer();
+    t->load(reader);
+    return t;
+}
+void ref_tokenizer_free(void* h) { delete static_cast<torch::io::GGUFTokenizer*>(h); }
+int64_t ref_tokenizer_encode(void* h, const char* text, int64_t len, int use_bos, int32_t* out, int64_t cap) {
+    const auto ids = static_cast<torch::io::GGUFTokenizer*>(h)->encode(std::string(text, (size_t)len), use_bos != 0);
+    for (size_t i = 0; i < ids.size() && (int64_t)i < cap; ++i) out[i] = ids[i];
+    return (int64_t)ids.size();
+}
+int64_t ref_tokenizer_decode(void* h, const int32_t* ids, int64_t n, int skip_special, char* out, int64_t cap) {
+    const std::string s = static_cast<torch::io::GGUFTokenizer*>(h)->decode(std::vector<int32_t>(ids, ids + n), skip_special != 0);
+    memcpy(out, s.data(), (size_t)std::min<int64_t>(cap, (int64_t)s.size()));
+    return (int64_t)s.size();
+}
+int64_t ref_tokenizer_token(void* h, int32_t id, char* out, int64_t cap) {
+    const std::string s = static_cast<torch::io::GGUFTokenizer*>(h)->decode_token(id);
+    memcpy(out, s.data(), (size_t)std::min<int64_t>(cap, (int64_t)s.size()));
+    return (int64_t)s.size();
+}
+// architecture / model name as the reference keeps them in its config; the system prompt and the no-think switch
+// are read from the environment by the reference itself (PT_SYSTEM_PROMPT, PT_NO_THINK)
+int64_t ref_chat_template(const char* architecture, const char* model_name, const char* prompt, char* out, int64_t cap) {
+    GGUFModel m;
+    m.config.architecture = architecture;
+    m.config.model_name = model_name;
+    const std::string s = m.apply_chat_template(prompt);
+    memcpy(out, s.data(), (size_t)std::min<int64_t>(cap, (int64_t)s.size()));
+    return (int64_t)s.size();
+}
+// what the reference's reader sees of a file: tensor count, and name / type / dims / first bytes of tensor i
+int64_t ref_gguf_n_tensors(const char* gguf_path) {
+    g::GGUFReader reader;
+    reader.open(gguf_path);
+    return (int64_t)reader.tensors.size();
+}
+
 }  // extern "C"

@@ -115,6 +115,20 @@ SIGNATURES = {
     "ptm_gguf_get_int": (i32, [vp, C.c_char_p, C.POINTER(i64)]),
     "ptm_gguf_get_float": (i32, [vp, C.c_char_p, C.POINTER(C.c_double)]),
     "ptm_gguf_get_string": (C.c_char_p, [vp, C.c_char_p]),
+    "ptm_gguf_get_array": (i32, [vp, C.c_char_p, C.POINTER(u32), C.POINTER(i64)]),
+    "ptm_gguf_array_string": (i32, [vp, C.c_char_p, i64, C.POINTER(vp), C.POINTER(i64)]),
+    "ptm_gguf_array_data": (vp, [vp, C.c_char_p]),
+    "ptm_tokenizer_create": (i32, [C.POINTER(C.c_char_p), C.POINTER(C.c_int32), C.c_int32, C.POINTER(C.c_char_p),
+                                   C.POINTER(C.c_int32), C.c_int32, C.c_char_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                   i32, C.POINTER(vp)]),
+    "ptm_tokenizer_from_gguf": (i32, [vp, C.POINTER(vp)]),
+    "ptm_tokenizer_free": (None, [vp]),
+    "ptm_tokenizer_vocab_size": (C.c_int32, [vp]),
+    "ptm_tokenizer_special_ids": (i32, [vp] + [C.POINTER(C.c_int32)] * 4),
+    "ptm_tokenizer_encode": (i32, [vp, C.c_char_p, i64, i32, C.POINTER(C.c_int32), i64, C.POINTER(i64)]),
+    "ptm_tokenizer_decode": (i32, [vp, C.POINTER(C.c_int32), i64, i32, C.c_char_p, i64, C.POINTER(i64)]),
+    "ptm_tokenizer_token": (i32, [vp, C.c_int32, C.c_char_p, i64, C.POINTER(i64)]),
+    "ptm_chat_template": (i32, [C.c_char_p, C.c_char_p, C.c_char_p, i32, C.c_char_p, C.c_char_p, i64, C.POINTER(i64)]),
     "ptm_model_load_gguf": (i32, [C.c_char_p, i32, i32, i32, C.POINTER(vp)]),
     "ptm_model_decoder": (vp, [vp]),
     "ptm_model_config": (i32, [vp, C.POINTER(DecodeConfig)]),

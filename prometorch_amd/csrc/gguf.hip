@@ -33,7 +33,9 @@ struct GgufValue {
     double f = 0.0;      // floats, widened
     std::string s;       // strings
     uint32_t arr_type = 0;
-    uint64_t arr_n = 0;  // arrays are skipped; only their shape is kept
+    uint64_t arr_n = 0;
+    const uint8_t* arr_data = nullptr;      // first element of a numeric or string array, inside the mapping
+    std::vector<const uint8_t*> arr_items;  // string arrays: start of each element's u64 length (arrays of arrays: kept as shape only)
 };
 
 struct Cursor {
@@ -94,9 +96,14 @@ static bool read_value(Cursor& c, uint32_t type, GgufValue& v, int depth) {
             const int sz = scalar_size(v.arr_type);
             if (sz) {
                 if (v.arr_n > (uint64_t)(c.end - c.p) / sz) return false;
+                v.arr_data = c.p;
                 c.skip(v.arr_n * sz);
             } else if (v.arr_type == G_STR) {
+                if (v.arr_n > (uint64_t)(c.end - c.p) / 8) return false;  // every element has at least its length field
+                v.arr_data = c.p;
+                if (depth == 0) v.arr_items.reserve((size_t)v.arr_n);
                 for (uint64_t i = 0; i < v.arr_n && c.ok; ++i) {
+                    if (depth == 0) v.arr_items.push_back(c.p);
                     const uint64_t n = c.get<uint64_t>();
                     c.skip(n);
                 }
@@ -268,6 +275,37 @@ const char* ptm_gguf_get_string(const ptm_gguf* g, const char* key) {
     if (!g || !key) return nullptr;
     auto it = g->kv.find(key);
     return (it == g->kv.end() || it->second.type != G_STR) ? nullptr : it->second.s.c_str();
+}
+
+int ptm_gguf_get_array(const ptm_gguf* g, const char* key, uint32_t* elem_type, int64_t* count) {
+    if (!g || !key) return PTM_E_NULL;
+    auto it = g->kv.find(key);
+    if (it == g->kv.end()) return PTM_E_NOT_FOUND;
+    if (it->second.type != G_ARR) return PTM_E_FORMAT;
+    if (elem_type) *elem_type = it->second.arr_type;
+    if (count) *count = (int64_t)it->second.arr_n;
+    return PTM_OK;
+}
+
+int ptm_gguf_array_string(const ptm_gguf* g, const char* key, int64_t i, const char** data, int64_t* len) {
+    if (!g || !key || !data || !len) return PTM_E_NULL;
+    auto it = g->kv.find(key);
+    if (it == g->kv.end()) return PTM_E_NOT_FOUND;
+    const GgufValue& v = it->second;
+    if (v.type != G_ARR || v.arr_type != G_STR) return PTM_E_FORMAT;
+    if (i < 0 || (uint64_t)i >= v.arr_items.size()) return PTM_E_RANGE;
+    uint64_t n;
+    memcpy(&n, v.arr_items[(size_t)i], 8);  // bounds were checked when the file was parsed
+    *data = reinterpret_cast<const char*>(v.arr_items[(size_t)i] + 8);
+    *len = (int64_t)n;
+    return PTM_OK;
+}
+
+const void* ptm_gguf_array_data(const ptm_gguf* g, const char* key) {
+    if (!g || !key) return nullptr;
+    auto it = g->kv.find(key);
+    if (it == g->kv.end() || it->second.type != G_ARR || !scalar_size(it->second.arr_type)) return nullptr;
+    return it->second.arr_data;
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -18,8 +18,8 @@ _T_U32, _T_I32, _T_F32, _T_BOOL, _T_STR, _T_ARR, _T_U64 = 4, 5, 6, 7, 8, 9, 10
 # ---------------------------------------------------------------------------------------------
 # writer (GGUF v3, little endian)
 # ---------------------------------------------------------------------------------------------
-def _s(x: str) -> bytes:
-    b = x.encode("utf-8")
+def _s(x) -> bytes:
+    b = x if isinstance(x, bytes) else x.encode("utf-8")
     return struct.pack("<Q", len(b)) + b
 
 
@@ -34,7 +34,7 @@ def _kv(key: str, value) -> bytes:
     if isinstance(value, str):
         return out + struct.pack("<I", _T_STR) + _s(value)
     if isinstance(value, (list, tuple)):
-        if all(isinstance(v, str) for v in value):
+        if all(isinstance(v, (str, bytes)) for v in value):
             return out + struct.pack("<IIQ", _T_ARR, _T_STR, len(value)) + b"".join(_s(v) for v in value)
         if all(isinstance(v, int) for v in value):
             return out + struct.pack("<IIQ", _T_ARR, _T_I32, len(value)) + struct.pack("<%di" % len(value), *value)
@@ -148,6 +148,25 @@ class GGUFFile:
     def get_string(self, key: str):
         s = self.L.ptm_gguf_get_string(self.h, key.encode())
         return None if s is None else s.decode()
+
+    def get_array(self, key: str):
+        """Array-valued metadata: a list of bytes for string arrays, a numpy array for numeric ones."""
+        et, n = C.c_uint32(), C.c_int64()
+        check(self.L.ptm_gguf_get_array(self.h, key.encode(), C.byref(et), C.byref(n)), f"gguf_get_array({key})")
+        if et.value == _T_STR:
+            out = []
+            p, ln = C.c_void_p(), C.c_int64()
+            for i in range(n.value):
+                check(self.L.ptm_gguf_array_string(self.h, key.encode(), i, C.byref(p), C.byref(ln)), "gguf_array_string")
+                out.append(C.string_at(p.value, ln.value) if ln.value else b"")
+            return out
+        dt = {0: np.uint8, 1: np.int8, 2: np.uint16, 3: np.int16, 4: np.uint32, 5: np.int32, 6: np.float32, 7: np.uint8,
+              10: np.uint64, 11: np.int64, 12: np.float64}[et.value]
+        ptr = self.L.ptm_gguf_array_data(self.h, key.encode())
+        if not n.value:
+            return np.zeros(0, dt)
+        raw = C.string_at(ptr, n.value * np.dtype(dt).itemsize)
+        return np.frombuffer(raw, dt).copy()
 
     def close(self) -> None:
         if getattr(self, "h", None):

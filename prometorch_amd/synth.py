@@ -196,3 +196,115 @@ def sampling_logits(case_index: int) -> np.ndarray:
     elif kind == "negative":
         x = (-np.abs(x) - np.float32(1.0)).astype(np.float32)
     return x
+
+
+# ---- synthetic tokenizers: a small trained BPE per kind, and the texts the golden run encodes ----
+_CORPUS = (
+    "The quick brown fox jumps over the lazy dog. It's 2024, isn't it? They're here; we'll see what you've done.\n"
+    "I'd say she's right: 3.14159 is close to pi, and 1000000 is a million!  Tabs\tand  double  spaces   matter.\n"
+    "def encode(text):\n    return [ord(c) for c in text]  # comment\n\nfor i in range(10): print(i, i * i)\n"
+    "Привет, мир! Как дела? Это тест токенизатора: числа 12345 и знаки препинания...\n"
+    "你好，世界！这是一个分词器的测试。日本語のテキストも少し。\n"
+    "Emoji \U0001F600 and symbols éèüß € 100 — done. <tag> not special </tag>\n"
+    "the the the and and of of to to in in that that is is was was he he for for it it with with as as his his\n"
+)
+
+_SPECIALS = ["<|endoftext|>", "<|im_start|>", "<|im_end|>", "<think>", "</think>"]
+
+
+def _byte_char(b: int) -> str:
+    """GPT-2 bytes_to_unicode."""
+    if (33 <= b <= 126) or (161 <= b <= 172) or (174 <= b <= 255):
+        return chr(b)
+    if b <= 32:
+        return chr(0x100 + b)
+    if 127 <= b <= 160:
+        return chr(0x121 + b - 127)
+    return chr(0x143)
+
+
+def _train_bpe(words: dict, n_merges: int) -> list:
+    """words: tuple of symbols -> count.  Classic BPE training: merge the most frequent adjacent pair, repeatedly."""
+    merges = []
+    words = dict(words)
+    for _ in range(n_merges):
+        pairs = {}
+        for w, c in words.items():
+            for a, b in zip(w, w[1:]):
+                pairs[(a, b)] = pairs.get((a, b), 0) + c
+        if not pairs:
+            break
+        (a, b), _ = max(pairs.items(), key=lambda kv: (kv[1], kv[0]))
+        merges.append((a, b))
+        nw = {}
+        for w, c in words.items():
+            out, i = [], 0
+            while i < len(w):
+                if i + 1 < len(w) and w[i] == a and w[i + 1] == b:
+                    out.append(a + b)
+                    i += 2
+                else:
+                    out.append(w[i])
+                    i += 1
+            nw[tuple(out)] = nw.get(tuple(out), 0) + c
+        words = nw
+    return merges
+
+
+def make_tokenizer(kind: str, n_merges: int = 300) -> dict:
+    """kind 'gpt2': byte-level BPE (256 byte symbols, merges over space-prefixed words, ChatML-style specials);
+    'llama': word-marker BPE over UTF-8 characters with <0xNN> byte tokens; 'greedy': the llama vocabulary without
+    merges (longest-match mode).  Returns the tokenizer.ggml.* metadata."""
+    import re
+    if kind == "gpt2":
+        words = {}
+        for m in re.finditer(r" ?[^\W\d_]+| ?\d+| ?[^\s\w]+|\s+", _CORPUS):
+            w = tuple(_byte_char(b) for b in m.group(0).encode("utf-8"))
+            words[w] = words.get(w, 0) + 1
+        merges = _train_bpe(words, n_merges)
+        vocab = [_byte_char(b) for b in range(256)] + [a + b for a, b in merges] + _SPECIALS
+        eos = vocab.index("<|endoftext|>")
+        return {"tokenizer.ggml.model": "gpt2", "tokenizer.ggml.tokens": vocab,
+                "tokenizer.ggml.merges": [a + " " + b for a, b in merges], "tokenizer.ggml.bos_token_id": eos,
+                "tokenizer.ggml.eos_token_id": eos, "tokenizer.ggml.padding_token_id": eos,
+                "tokenizer.ggml.add_bos_token": False}
+    words = {}
+    for w in _CORPUS.replace("\n", " ").replace("\t", " ").split(" "):
+        if w:
+            t = tuple("▁" + w)
+            words[t] = words.get(t, 0) + 1
+    merges = _train_bpe(words, n_merges)
+    chars = sorted({c for w in words for c in w} - {"д"})          # one Cyrillic letter left out: byte fallback
+    vocab = ["<unk>", "<s>", "</s>"] + ["<0x%02X>" % b for b in range(256)] + chars + [a + b for a, b in merges] + ["\n"]
+    md = {"tokenizer.ggml.model": "llama", "tokenizer.ggml.tokens": vocab,
+          "tokenizer.ggml.scores": [0.0] * len(vocab), "tokenizer.ggml.bos_token_id": 1,
+          "tokenizer.ggml.eos_token_id": 2, "tokenizer.ggml.unknown_token_id": 0, "tokenizer.ggml.add_bos_token": True}
+    if kind == "llama":
+        md["tokenizer.ggml.merges"] = [a + " " + b for a, b in merges]
+    return md
+
+
+def tokenizer_texts(kind: str) -> list:
+    """Byte strings the golden run encodes.  For 'gpt2' none has a UTF-8 continuation byte that does not follow a
+    letter byte: the reference's splitter does not terminate on those."""
+    fixed = [
+        "", " ", "  ", "a", "Hello, world!", "hello world", " leading and trailing ", "two  spaces   three", "tabs\tand\nnewlines\r\n\n",
+        "It's what they're saying: I'd, we'll, you've, he's, I'm, don't 'quoted' 'tis", "'s", "'", "x'", "x'r", "x're",
+        "1234567890 3.14 2024-05-06 1,000", "snake_case CamelCase kebab-case path/to/file.py", "!!! ... ??? --- (()) [[ ]] {{}}",
+        "Привет, мир! Как дела?", "Сегодня 5 мая, погода хорошая.", "你好，世界！", "日本語のテキスト", "emoji \U0001F600\U0001F680 end",
+        "café naïve über straße €5", "<|im_start|>user\nHi<|im_end|>\n<|im_start|>assistant\n",
+        "<think>hmm</think>ok<|endoftext|>", "<|im_start|><|im_end|><|im_start|>", "a<b>c <0x41> <tag> <|unknown|> <>", "<s>x</s><unk>",
+        "the the the and of to in that is was", "def f(x):\n    return x * 2  # twice\n", "line1\n\nline3\n   indented\n\ttabbed",
+        "trailing spaces   ", "\n", "\n\n\n", " \n \n", "a\nb", "MiXeD 123abc456 abc123", "▁marker▁inside", "ĠG-dot Ċ",
+        "д д дд один два", "x" * 70, "ab" * 40 + " " + "the" * 30,
+    ]
+    out = [t.encode("utf-8") for t in fixed]
+    out += [b"\xffabc", b"a\x80\x81b", b"ok \xe4\xbd", b"\xc3(", b"\xc0\xc1 odd", b"abc\xf0\x9f\x98"]   # malformed UTF-8 that is safe for both splitters
+    g = rng_for(5151, 1 if kind == "gpt2" else 2)
+    alphabet = list("abcdefghijklmnopqrstuvwxyzTHE    \n\t.,!?'0123456789") + ["the", " and", "'s", "'re", "д", "ы", "你", "\U0001F600", "<|im_end|>", "<s>", "é"]
+    for _ in range(40):
+        n = int(g.integers(1, 60))
+        out.append("".join(alphabet[int(i)] for i in g.integers(0, len(alphabet), n)).encode("utf-8"))
+    if kind != "gpt2":
+        out += [bytes(g.integers(0, 256, int(g.integers(1, 40)), dtype=np.uint8)) for _ in range(20)]        # arbitrary bytes
+    return out

@@ -81,11 +81,16 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--full", action="store_true")
     ap.add_argument("--sampling-only", action="store_true", help="write golden_sampling.npz and nothing else")
+    ap.add_argument("--tokenizer-only", action="store_true", help="write golden_tokenizer.json and nothing else")
     args = ap.parse_args()
     assert po.have_ref(), "build oracle/_ref first: make -C oracle ref"
     if args.sampling_only:
         make_sampling()
         print("wrote golden_sampling.npz")
+        return
+    if args.tokenizer_only:
+        make_tokenizer_golden()
+        print("wrote golden_tokenizer.json")
         return
     R = po.ref()
     meta = {"made_with": "oracle/_ref/libptm_ref.so (g++ -O2 -std=c++17 -mavx2 -mfma; see oracle/Makefile)",
@@ -208,6 +213,7 @@ def main():
 
     np.savez_compressed(os.path.join(OUT, "golden_small.npz"), **g)
     make_sampling()
+    make_tokenizer_golden()
 
     if args.full:
         make_full(meta)
@@ -230,6 +236,68 @@ def make_sampling():
         toks.append(int(R.ref_sample_token(h, x.ctypes.data, vocab, temperature, top_k, top_p)))
     R.ref_model_destroy(h)
     np.savez_compressed(os.path.join(OUT, "golden_sampling.npz"), tokens=np.array(toks, np.int32))
+
+
+CHAT_CASES = [  # (architecture, model name, PT_SYSTEM_PROMPT or None = unset, PT_NO_THINK, prompt)
+    ("qwen3", "Qwen3-4B", None, False, "Hello!"), ("qwen3", "Qwen3-4B", None, True, "2+2?"), ("qwen3", "q", "", True, "x"),
+    ("qwen3", "q", "", False, "no system"), ("qwen2", "q2", "Be brief.", True, "hi"), ("phi3", "Phi-3", None, False, "p"),
+    ("phi3", "Phi-3", "", False, "p"), ("gemma3", "g", None, False, "hello"), ("gemma2", "g", "", False, "hello"),
+    ("llama", "Meta-Llama-3-8B", None, False, "hey"), ("llama", "Meta-Llama-3-8B", "", False, "hey"),
+    ("llama", "Mistral-7B-Instruct", None, False, "m"), ("llama", "MISTRAL", "", False, "m"), ("deepseek2", "x", None, False, "raw prompt"),
+]
+
+
+def make_tokenizer_golden():
+    """The reference's GGUFTokenizer over the synthetic tokenizers of prometorch_amd.synth (written as GGUF files by
+    this repository's writer and read back by the REFERENCE's GGUFReader) and its apply_chat_template."""
+    import base64
+    import tempfile
+    import ctypes as C
+    from prometorch_amd import gguf
+    R = po.ref()
+    b64 = lambda b: base64.b64encode(b).decode()
+    out = {"tokenizers": {}, "chat": []}
+    buf = C.create_string_buffer(1 << 16)
+    ids = (C.c_int32 * 4096)()
+
+    def text_of(fn, *args):  # the call first, the buffer after it
+        n = fn(*args, buf, 1 << 16)
+        assert n <= 1 << 16
+        return buf.raw[:n]
+
+    for kind in ("gpt2", "llama", "greedy"):
+        md = synth.make_tokenizer(kind)
+        md["general.architecture"] = "qwen3"
+        with tempfile.TemporaryDirectory() as d:
+            path = os.path.join(d, "tok.gguf")
+            gguf.write_gguf(path, md, [("dummy", 0, [4], np.zeros(4, np.float32))])
+            assert R.ref_gguf_n_tensors(path.encode()) == 1
+            h = R.ref_tokenizer_load(path.encode())
+        cases = []
+        for text in synth.tokenizer_texts(kind):
+            for use_bos in (True, False):
+                n = R.ref_tokenizer_encode(h, text, len(text), int(use_bos), ids, 4096)
+                assert n <= 4096
+                got = [int(ids[i]) for i in range(n)]
+                a = (C.c_int32 * max(1, n))(*got)
+                dec = [text_of(R.ref_tokenizer_decode, h, a, n, int(sk)) for sk in (True, False)]
+                cases.append({"text": b64(text), "use_bos": use_bos, "ids": got, "decoded_skip": b64(dec[0]), "decoded_all": b64(dec[1])})
+        n_vocab = len(md["tokenizer.ggml.tokens"])
+        toks = [b64(text_of(R.ref_tokenizer_token, h, i)) for i in range(-1, n_vocab + 1)]
+        out["tokenizers"][kind] = {"cases": cases, "token_bytes_from_minus1": toks}
+        R.ref_tokenizer_free(h)
+    for arch, name, sys_prompt, no_think, prompt in CHAT_CASES:
+        for k, v in (("PT_SYSTEM_PROMPT", sys_prompt), ("PT_NO_THINK", "1" if no_think else None)):
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+        out["chat"].append({"arch": arch, "name": name, "system": sys_prompt, "no_think": no_think, "prompt": prompt,
+                            "text": text_of(R.ref_chat_template, arch.encode(), name.encode(), prompt.encode()).decode()})
+    os.environ.pop("PT_SYSTEM_PROMPT", None)
+    os.environ.pop("PT_NO_THINK", None)
+    with open(os.path.join(OUT, "golden_tokenizer.json"), "w") as f:
+        json.dump(out, f, indent=0, sort_keys=True)
 
 
 def make_full(meta):
