@@ -66,9 +66,10 @@ def write_gguf(path: str, metadata: dict, tensors: list, alignment: int = 32, ve
 
 
 def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "qwen3", tied: bool = True,
-                  alignment: int = 32) -> None:
+                  alignment: int = 32, tokenizer: dict | None = None) -> None:
     """Write a decoder (the dict form prometorch_amd.decode.Decoder takes) as a GGUF file with the
-    tensor names and metadata keys a qwen3 GGUF carries."""
+    tensor names and metadata keys a qwen3 GGUF carries.  tokenizer: tokenizer.ggml.* metadata to store
+    (default: a three-token placeholder)."""
     md = {
         "general.architecture": arch, "general.name": "synthetic",
         f"{arch}.block_count": cfg["n_layers"], f"{arch}.embedding_length": cfg["hidden"],
@@ -78,6 +79,9 @@ def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "q
         f"{arch}.attention.layer_norm_rms_epsilon": float(cfg["eps"]), f"{arch}.context_length": 4096,
         "tokenizer.ggml.model": "gpt2", "tokenizer.ggml.tokens": ["a", "b", "c"], "tokenizer.ggml.token_type": [1, 1, 1],
     }
+    if tokenizer:
+        md = {k: v for k, v in md.items() if not k.startswith("tokenizer.")}
+        md.update(tokenizer)
     H = cfg["hidden"]
     ts = [("token_embd.weight", Q6_K, [H, cfg["vocab"]], head["lm_head"])]
     if not tied:

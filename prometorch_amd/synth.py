@@ -251,7 +251,7 @@ def _train_bpe(words: dict, n_merges: int) -> list:
     return merges
 
 
-def make_tokenizer(kind: str, n_merges: int = 300) -> dict:
+def make_tokenizer(kind: str, n_merges: int = 300, vocab_size: int | None = None) -> dict:
     """kind 'gpt2': byte-level BPE (256 byte symbols, merges over space-prefixed words, ChatML-style specials);
     'llama': word-marker BPE over UTF-8 characters with <0xNN> byte tokens; 'greedy': the llama vocabulary without
     merges (longest-match mode).  Returns the tokenizer.ggml.* metadata."""
@@ -263,6 +263,8 @@ def make_tokenizer(kind: str, n_merges: int = 300) -> dict:
             words[w] = words.get(w, 0) + 1
         merges = _train_bpe(words, n_merges)
         vocab = [_byte_char(b) for b in range(256)] + [a + b for a, b in merges] + _SPECIALS
+        if vocab_size:  # padded to a model's vocabulary with reserved specials
+            vocab += ["<|reserved_%d|>" % i for i in range(vocab_size - len(vocab))]
         eos = vocab.index("<|endoftext|>")
         return {"tokenizer.ggml.model": "gpt2", "tokenizer.ggml.tokens": vocab,
                 "tokenizer.ggml.merges": [a + " " + b for a, b in merges], "tokenizer.ggml.bos_token_id": eos,

@@ -73,3 +73,45 @@ def test_gguf_model_refuses_what_it_cannot_run(dev, seeds, tmp_path):
     with pytest.raises(PtmError) as e:
         gguf.GGUFModel(p3, max_seq=64)
     assert e.value.code == -10
+
+
+def test_text_to_text_through_one_file(dev, po, seeds, tmp_path):
+    """The whole path behind the C ABI from one .gguf file: chat template -> tokenizer -> prompt prefill -> sampled
+    decode on the device -> text; the token stream is checked against the oracle's loop (step the prompt token by
+    token, then penalise / sample / feed back with the same uniform draws)."""
+    from prometorch_amd import ops
+    from prometorch_amd.tokenizer import Tokenizer, chat_template
+    cfg, layers, head, _ = build_tiny(seeds)
+    tok_md = synth.make_tokenizer("gpt2", vocab_size=cfg["vocab"])
+    assert len(tok_md["tokenizer.ggml.tokens"]) == cfg["vocab"]
+    path = str(tmp_path / "chat.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head, tokenizer=tok_md)
+    f = gguf.GGUFFile(path)
+    tk = Tokenizer.from_gguf(f)
+    m = gguf.GGUFModel(path, max_seq=160, kv_fp16=True)
+    text = chat_template(f.get_string("general.architecture"), "Hello there, what's 2+2?", system="Be brief.")
+    ids = tk.encode(text)
+    assert 20 < len(ids) < 100 and ids[0] == tok_md["tokenizer.ggml.tokens"].index("<|im_start|>")
+    assert tk.decode(ids, skip_special=False) == text
+    n_new, params = 24, (0.8, 40, 0.9, 1.1)
+    us = ops.mt19937_uniforms(42, 0, n_new)
+    first = m.prefill(ids[:-1])                 # everything but the last prompt token; its successor is resampled below
+    m.sampling_begin(*params)
+    got = m.sample(ids[-1], us)
+    # oracle loop
+    om = po.OracleModel(cfg, layers, head, 160, kv_fp16=True)
+    for t in ids[:-1]:
+        om.step(t)
+    tok, generated = ids[-1], []
+    for st in range(n_new):
+        om.step(tok)
+        lg = po.repetition_penalty(om.logits, generated, params[3]) if generated else om.logits
+        tok, gap = po.sample_token(lg, params[0], params[1], params[2], us[st])
+        if gap <= 1e-3:
+            break   # the prefilled cache differs from the stepped one at the Q8-rounding-noise level: compare clear draws only
+        assert got[st] == tok, (st, gap)
+        generated.append(tok)
+    assert len(generated) >= 8 and first >= 0
+    reply = tk.decode(got)
+    assert isinstance(reply, bytes) and len(reply) > 0
+    m.close(); tk.close(); f.close()
