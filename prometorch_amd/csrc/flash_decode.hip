@@ -14,7 +14,10 @@
 
 namespace ptm {
 
-enum { FD_CHUNK = 64, FD_THREADS = 256 };
+#ifndef PTM_FD_CHUNK
+#define PTM_FD_CHUNK 64
+#endif
+enum { FD_CHUNK = PTM_FD_CHUNK, FD_THREADS = 256 };
 
 // e^x through the hardware base-2 exponential (v_exp_f32, 1 ulp): softmax weights need no more, and the libm
 // expf expands to a dozen instructions on a path whose cost is instruction count.  -inf gives 0.

@@ -468,7 +468,8 @@ def test_elementwise_embedding_argmax(dev, po):
 @pytest.mark.parametrize("kv_fp16", [True, False])
 @pytest.mark.parametrize("nh,nkv,hd,past", [(32, 8, 128, 2048), (32, 8, 128, 2111), (32, 8, 128, 2112), (4, 2, 64, 19),
                                             (8, 8, 128, 0), (16, 2, 64, 63), (8, 1, 64, 64), (8, 8, 64, 130), (4, 2, 64, 29),
-                                            (4, 2, 64, 31), (16, 2, 64, 61), (32, 8, 128, 14), (32, 8, 128, 62), (4, 4, 128, 5)])
+                                            (4, 2, 64, 31), (16, 2, 64, 61), (32, 8, 128, 14), (32, 8, 128, 62), (4, 4, 128, 5),
+                                            (32, 8, 128, 20000)])   # past the ~12 k positions where the reference's kernel stops
 def test_attn_decode_fused_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past):
     """QK-norm + RoPE + KV append + attention + merge in one launch, three tokens in a row, against the oracle's pieces in the reference's order."""
     max_seq = ((past + 3 + 63) // 64 + 1) * 64
