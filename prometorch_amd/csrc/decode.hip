@@ -33,7 +33,7 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
 int qgemm_f16_splits(int N, int K);
 int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
                     const ptm_sampling* d_params, const float* d_uniforms, const int* d_step, void* workspace,
-                    int64_t* out_token, int32_t* counts_rw, ArgmaxAdvance adv, hipStream_t s);
+                    int64_t* out_token, int32_t* counts_rw, ArgmaxAdvance adv, bool ws_kept_clean, hipStream_t s);
 __global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
     for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
 }
@@ -182,7 +182,7 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
         }
         return sampler_enqueue(d->logits, c.vocab, d->d_counts, d->sampling, d->d_sampling, d->d_uniforms, d->d_step,
                                d->sampler_ws, d->d_next, d->d_counts,
-                               ArgmaxAdvance{d->d_token, d->d_past, d->d_step, d->d_tokens, c.max_seq}, s);
+                               ArgmaxAdvance{d->d_token, d->d_past, d->d_step, d->d_tokens, c.max_seq}, true, s);
     }
     if (c.lm_head.ggml_type == PTM_TYPE_Q6_K) {
         // final RMSNorm in the lm_head prologue, step bookkeeping in the argmax tail: two launches for the whole tail
@@ -337,6 +337,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->d_tokens = (int64_t*)(base + o_tokens);
     d->d_sampling = (ptm_sampling*)(base + o_samp); d->d_counts = (int32_t*)(base + o_counts);
     d->d_uniforms = (float*)(base + o_unif); d->sampler_ws = base + o_sws;
+    if ((rc = hip_status(hipMemset(d->sampler_ws, 0, (size_t)ptm_sampler_workspace_bytes()))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     q6k_init_attributes();  // one-time kernel attributes, before anything can be captured
 
     if ((rc = hip_status(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking))) != PTM_OK) { ptm_decode_destroy(d); return rc; }

@@ -22,7 +22,7 @@
 
 namespace ptm {
 
-enum { SAMPLER_MAX_CAND = 2048, SAMPLER_MAX_TOPK = 1024, SAMPLER_ELEMS_PER_WG = 2048 };
+enum { SAMPLER_MAX_CAND = 2048, SAMPLER_MAX_TOPK = 1024, SAMPLER_ELEMS_PER_WG = 512 };
 
 // workspace layout (uint32 words)
 enum {
@@ -66,41 +66,45 @@ __device__ __forceinline__ float sampler_value(const SamplerArgs& a, const ptm_s
     if (p.temperature >= 1e-6f) x = x / p.temperature;
     return x + 0.0f;  // -0 -> +0: the reference compares values, the radix select compares bit patterns
 }
+// value of lane i (i uniform over the wave): v_readlane, no LDS round trip
+__device__ __forceinline__ float lane_f(float v, int i) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i)); }
+__device__ __forceinline__ uint32_t lane_u(uint32_t v, int i) { return (uint32_t)__builtin_amdgcn_readlane((int)v, i); }
+
 __device__ __forceinline__ int sampler_k(const ptm_sampling& p) { return p.temperature >= 1e-6f ? p.top_k : 1; }
 
 // Which bin, counting from the top, holds the k-th largest key?  All 256 threads call it; returns the bin and how
-// many keys are still wanted inside it.  s_scan: 258 words of LDS.
+// many keys are still wanted inside it.  s_scan: 8 words of LDS.  (Wave-level prefix sums: two barriers per call.)
 __device__ void select_bin(const uint32_t* hist, int nbins, int k, int& bin, int& k_in_bin, uint32_t* s_scan) {
-    const int tid = threadIdx.x, per = nbins / 256;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, per = nbins / 256;
     uint32_t mine = 0;
     for (int j = 0; j < per; ++j) mine += hist[nbins - 1 - (tid * per + j)];
-    __syncthreads();
-    s_scan[tid] = mine;
-    __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {  // inclusive scan
-        const uint32_t add = tid >= off ? s_scan[tid - off] : 0;
-        __syncthreads();
-        s_scan[tid] += add;
-        __syncthreads();
+    uint32_t incl = mine;  // inclusive prefix sum over the wave
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t up = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += up;
     }
-    const uint32_t incl = s_scan[tid], excl = incl - mine;
-    if (excl < (uint32_t)k && (uint32_t)k <= incl) {
+    __syncthreads();  // s_scan may still be read by the previous call
+    if (lane == 63) s_scan[wave] = incl;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) incl += s_scan[w];
+    const uint32_t excl = incl - mine;
+    if (excl < (uint32_t)k && (uint32_t)k <= incl) {  // exactly one thread: the counts sum to at least k
         uint32_t above = excl;
         for (int j = 0; j < per; ++j) {
             const int b = nbins - 1 - (tid * per + j);
             const uint32_t h = hist[b];
             if (above + h >= (uint32_t)k) {
-                s_scan[256] = (uint32_t)b;
-                s_scan[257] = (uint32_t)k - above;
+                s_scan[4] = (uint32_t)b;
+                s_scan[5] = (uint32_t)k - above;
                 break;
             }
             above += h;
         }
     }
     __syncthreads();
-    bin = (int)s_scan[256];
-    k_in_bin = (int)s_scan[257];
-    __syncthreads();
+    bin = (int)s_scan[4];
+    k_in_bin = (int)s_scan[5];
 }
 
 __global__ __launch_bounds__(256) void sampler_clear_kernel(uint32_t* ws) {
@@ -112,7 +116,7 @@ template <int LEVEL>
 __global__ __launch_bounds__(256) void sampler_hist_kernel(SamplerArgs a) {
     constexpr int NB = LEVEL == 2 ? 1024 : 2048;
     __shared__ uint32_t s_hist[NB];
-    __shared__ uint32_t s_scan[258];
+    __shared__ uint32_t s_scan[8];
     const int tid = threadIdx.x;
     const ptm_sampling p = sampler_params(a);
     int b0 = 0, b1 = 0, k = sampler_k(p);
@@ -124,10 +128,12 @@ __global__ __launch_bounds__(256) void sampler_hist_kernel(SamplerArgs a) {
 #pragma unroll
     for (int u = 0; u < SAMPLER_ELEMS_PER_WG / 256; ++u) {
         const int i = base + tid + 256 * u;
-        if (i < a.vocab) {
-            const uint32_t key = order_key(sampler_value(a, p, i));
-            if (LEVEL == 0) atomicAdd(&s_hist[key >> 21], 1u);
-            else if (LEVEL == 1) { if ((int)(key >> 21) == b0) atomicAdd(&s_hist[(key >> 10) & 0x7ffu], 1u); }
+        const bool in = i < a.vocab;
+        const uint32_t key = in ? order_key(sampler_value(a, p, i)) : 0u;
+        if (LEVEL == 0) {
+            if (in) atomicAdd(&s_hist[key >> 21], 1u);
+        } else if (in) {
+            if (LEVEL == 1) { if ((int)(key >> 21) == b0) atomicAdd(&s_hist[(key >> 10) & 0x7ffu], 1u); }
             else { if ((key >> 10) == (((uint32_t)b0 << 11) | (uint32_t)b1)) atomicAdd(&s_hist[key & 0x3ffu], 1u); }
         }
     }
@@ -139,7 +145,7 @@ __global__ __launch_bounds__(256) void sampler_hist_kernel(SamplerArgs a) {
 
 // every key at or above the k-th largest goes to the candidate list (order of arrival; the finish kernel sorts)
 __global__ __launch_bounds__(256) void sampler_gather_kernel(SamplerArgs a) {
-    __shared__ uint32_t s_scan[258];
+    __shared__ uint32_t s_scan[8];
     const int tid = threadIdx.x;
     const ptm_sampling p = sampler_params(a);
     int b0, b1, b2, k = sampler_k(p);
@@ -185,6 +191,7 @@ struct SamplerOut {
     const int* d_step;        // NULL: s = 0
     int32_t* counts_rw;       // NULL, or the occurrence counts to bump for the chosen token
     ArgmaxAdvance adv;        // step bookkeeping of the decode loop (all NULL outside it)
+    int leave_clean;          // zero the histograms and the candidate count for the next call (it then skips its clear launch)
 };
 
 __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, SamplerOut o) {
@@ -194,10 +201,93 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
     __shared__ uint8_t s_keep[SAMPLER_MAX_CAND];
     __shared__ int s_token;
     const int tid = threadIdx.x;
+    // every load whose address is known goes out first, in one round trip; the draw follows as soon as the step is known
     const ptm_sampling p = sampler_params(a);
     const uint32_t total = a.ws[SW_COUNT];
+    const uint32_t key0 = a.ws[SW_CAND_KEY + (tid & 63)], idx0 = a.ws[SW_CAND_IDX + (tid & 63)];
+    const int step = o.d_step ? *o.d_step : 0;
+    const int64_t past_now = o.adv.d_past ? *o.adv.d_past : 0;
+    const float r_draw = o.uniforms[step];
     const bool overflow = total > SAMPLER_MAX_CAND;
     const int m = overflow ? SAMPLER_MAX_CAND : (int)total;
+    if (m <= 64) {
+        // The usual case (k candidates, k <= 64): one wave, one candidate per lane, no workgroup barrier.  Order by
+        // counting, sequential sums by reading lane after lane -- the same additions in the same order as below.
+        if (tid >= 64) {
+            if (o.leave_clean) for (int i = tid - 64; i < SW_CLEAR_WORDS; i += 1024 - 64) if (i != SW_COUNT) a.ws[i] = 0;
+            return;
+        }
+        const int lane = tid;
+        const bool valid = lane < m;
+        const uint32_t key = valid ? key0 : 0u, idx = valid ? idx0 : 0xffffffffu;
+        int rank = 0;
+        for (int j = 0; j < m; ++j) rank += lane_u(idx, j) < idx;
+        if (valid) { s_idx[rank] = idx; s_p[rank] = key_value(key); }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint32_t id = valid ? s_idx[lane] : 0u;   // index order from here on
+        const float x = valid ? s_p[lane] : -INFINITY;
+        const bool greedy = !(p.temperature >= 1e-6f);
+        int token = a.vocab - 1;
+        if (greedy) {
+            token = (int)lane_u(id, 0);
+        } else {
+            const float mx = max64(x);
+            const float e = valid ? expf(x - mx) : 0.0f;
+            float sum = 0.0f;
+            for (int i = 0; i < m; ++i) sum += lane_f(e, i);
+            float pr = e * (1.0f / sum);
+            if (p.top_p < 1.0f) {
+                const bool elig = valid && pr > 1e-10f;
+                int r2 = 0, n_elig = 0;
+                for (int j = 0; j < m; ++j) {
+                    const float pj = lane_f(pr, j);
+                    const bool ej = pj > 1e-10f;
+                    n_elig += ej;
+                    r2 += ej && (pj > pr || (pj == pr && j < lane));
+                }
+                float* s_q = reinterpret_cast<float*>(s_sort);
+                if (elig) s_q[r2] = pr;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const float q = lane < n_elig ? s_q[lane] : 0.0f;
+                float cum = 0.0f;
+                int n_keep = n_elig;
+                for (int k = 0; k < n_elig; ++k) {
+                    cum += lane_f(q, k);
+                    if (cum >= p.top_p) { n_keep = k + 1; break; }
+                }
+                pr = (elig && r2 < n_keep) ? pr : 0.0f;
+                float s2 = 0.0f;
+                for (int i = 0; i < m; ++i) s2 += lane_f(pr, i);
+                if (s2 > 0.0f) pr *= 1.0f / s2;
+            }
+            const float r = r_draw;
+            if (r <= 0.0f) {
+                token = 0;
+            } else {
+                float cum = 0.0f;
+                for (int i = 0; i < m; ++i) {
+                    cum += lane_f(pr, i);
+                    if (cum >= r) { token = (int)lane_u(id, i); break; }
+                }
+            }
+        }
+        if (lane == 0) {
+            if (o.out_token) *o.out_token = token;
+            if (o.counts_rw) atomicAdd(&o.counts_rw[token], 1);  // no value needed back: nothing waits for it
+            if (o.adv.d_step) {
+                if (step < o.adv.cap) o.adv.tokens_out[step] = token;
+                *o.adv.d_token = token;
+                *o.adv.d_past = past_now + 1;
+                *o.adv.d_step = step + 1;
+            }
+            if (o.leave_clean) a.ws[SW_COUNT] = 0;
+        }
+        return;
+    }
     int n = 1;
     while (n < m) n <<= 1;
     // ---- candidates in index order ----
@@ -256,7 +346,7 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
         } else if (greedy) {
             token = (int)s_idx[0];  // every candidate equals the maximum; index order -> the lowest index
         } else {
-            const float r = o.uniforms[o.d_step ? *o.d_step : 0];
+            const float r = r_draw;
             token = a.vocab - 1;
             if (r <= 0.0f) {
                 token = 0;  // the running sum reaches r at the very first index
@@ -272,12 +362,14 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
         if (o.out_token) *o.out_token = token;
         if (o.counts_rw && token >= 0) o.counts_rw[token] += 1;
         if (o.adv.d_step) {
-            const int st = *o.adv.d_step;
-            if (st < o.adv.cap) o.adv.tokens_out[st] = token;
+            if (step < o.adv.cap) o.adv.tokens_out[step] = token;
             *o.adv.d_token = token < 0 ? 0 : token;
-            *o.adv.d_past = *o.adv.d_past + 1;
-            *o.adv.d_step = st + 1;
+            *o.adv.d_past = past_now + 1;
+            *o.adv.d_step = step + 1;
         }
+    }
+    if (o.leave_clean) {  // every thread read the candidate count long before (barriers above)
+        for (int i = tid; i < SW_CLEAR_WORDS; i += 1024) a.ws[i] = 0;
     }
 }
 
@@ -292,15 +384,17 @@ static int sampler_check(const ptm_sampling& p, int vocab) {
 // host_params are validated here; when d_params is given the kernels read the device copy (which must hold the same values)
 int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
                     const ptm_sampling* d_params, const float* d_uniforms, const int* d_step, void* workspace,
-                    int64_t* out_token, int32_t* counts_rw, ArgmaxAdvance adv, hipStream_t s) {
+                    int64_t* out_token, int32_t* counts_rw, ArgmaxAdvance adv, bool ws_kept_clean, hipStream_t s) {
+    // ws_kept_clean: the workspace was zeroed once by the caller and is only ever used through this function, whose last
+    // kernel then leaves it zeroed again: the clear launch is skipped
     if (!logits || !workspace || !d_uniforms) return PTM_E_NULL;
     const int rc = sampler_check(host_params, vocab);
     if (rc != PTM_OK) return rc;
     if (reinterpret_cast<uintptr_t>(workspace) & 7u) return PTM_E_ALIGN;
     SamplerArgs a{logits, counts, vocab, d_params, host_params, static_cast<uint32_t*>(workspace)};
-    SamplerOut o{out_token, d_uniforms, d_step, counts_rw, adv};
+    SamplerOut o{out_token, d_uniforms, d_step, counts_rw, adv, ws_kept_clean ? 1 : 0};
     const dim3 grid((vocab + SAMPLER_ELEMS_PER_WG - 1) / SAMPLER_ELEMS_PER_WG);
-    hipLaunchKernelGGL(sampler_clear_kernel, dim3(4), dim3(256), 0, s, a.ws);
+    if (!ws_kept_clean) hipLaunchKernelGGL(sampler_clear_kernel, dim3(4), dim3(256), 0, s, a.ws);
     hipLaunchKernelGGL(sampler_hist_kernel<0>, grid, dim3(256), 0, s, a);
     hipLaunchKernelGGL(sampler_hist_kernel<1>, grid, dim3(256), 0, s, a);
     hipLaunchKernelGGL(sampler_hist_kernel<2>, grid, dim3(256), 0, s, a);
@@ -321,7 +415,7 @@ int ptm_sample_token(const float* logits, int vocab, const int32_t* counts, cons
                      void* workspace, int64_t* out_token, ptm_stream_t stream) {
     if (!params || !out_token) return PTM_E_NULL;
     return sampler_enqueue(logits, vocab, counts, *params, nullptr, d_uniform, nullptr, workspace, out_token, nullptr,
-                           ArgmaxAdvance{nullptr, nullptr, nullptr, nullptr, 0}, as_stream(stream));
+                           ArgmaxAdvance{nullptr, nullptr, nullptr, nullptr, 0}, false, as_stream(stream));
 }
 
 // The reference's draws: `static std::mt19937 rng(42); std::uniform_real_distribution<float> dist(0.0f, 1.0f)`
