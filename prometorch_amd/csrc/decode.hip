@@ -31,6 +31,8 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
                    int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, bool reuse_rows,
                    hipStream_t s);
 int qgemm_f16_splits(int N, int K);
+int qgemm_f16_prepare_fused(int pre, const float* X, const float* X2, float eps, int add_one, void* ws_round, void* ws_plain,
+                            int M, int K, hipStream_t s);
 int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
                     const ptm_sampling* d_params, const float* d_uniforms, const int* d_step, void* workspace,
                     int64_t* out_token, int32_t* counts_rw, ArgmaxAdvance adv, bool ws_kept_clean, hipStream_t s);
@@ -94,9 +96,10 @@ struct ptm_decoder {
     // prefill scratch for up to pf_rows prompt rows at a time (allocated on the first prefill)
     void* pf_slab = nullptr;
     int pf_rows = 0;
-    float *pf_x = nullptr, *pf_xn = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_attn = nullptr,
+    float *pf_x = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_attn = nullptr,
           *pf_gate = nullptr, *pf_up = nullptr;
-    void* pf_ws = nullptr;
+    void* pf_ws = nullptr;   // fp16 rows for Q4_K matrices (Q8-rounded)
+    void* pf_ws2 = nullptr;  // fp16 rows for Q6_K matrices (plain)
     float* pf_split = nullptr;  // K-split partial sums of the GEMMs
     size_t pf_split_bytes = 0;
     int* pf_tokens = nullptr;
@@ -211,9 +214,10 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
     size_t off = 0;
     auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
     const size_t R = (size_t)rows;
-    const size_t o_x = take(4 * R * H), o_xn = take(4 * R * H), o_q = take(4 * R * qd), o_k = take(4 * R * kvd),
+    const size_t o_x = take(4 * R * H), o_q = take(4 * R * qd), o_k = take(4 * R * kvd),
                  o_v = take(4 * R * kvd), o_attn = take(4 * R * qd), o_gate = take(4 * R * I), o_up = take(4 * R * I),
-                 o_ws = take((size_t)ptm_qgemm_f16_workspace_bytes(rows, (int)kmax)), o_tok = take(4 * R);
+                 o_ws = take((size_t)ptm_qgemm_f16_workspace_bytes(rows, (int)kmax)),
+                 o_ws2 = take((size_t)ptm_qgemm_f16_workspace_bytes(rows, (int)kmax)), o_tok = take(4 * R);
     size_t split_elems = 0;  // widest splits x N over the layer's matrices (all layers have the same shapes)
     for (const ptm_qweight* w : {&d->layers[0].q, &d->layers[0].k, &d->layers[0].v, &d->layers[0].o, &d->layers[0].gate,
                                  &d->layers[0].up, &d->layers[0].down}) {
@@ -225,9 +229,9 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
     const int rc = hip_status(hipMalloc(&d->pf_slab, off));
     if (rc != PTM_OK) return rc;
     uint8_t* b = static_cast<uint8_t*>(d->pf_slab);
-    d->pf_x = (float*)(b + o_x); d->pf_xn = (float*)(b + o_xn); d->pf_q = (float*)(b + o_q); d->pf_k = (float*)(b + o_k);
+    d->pf_x = (float*)(b + o_x); d->pf_q = (float*)(b + o_q); d->pf_k = (float*)(b + o_k);
     d->pf_v = (float*)(b + o_v); d->pf_attn = (float*)(b + o_attn); d->pf_gate = (float*)(b + o_gate);
-    d->pf_up = (float*)(b + o_up); d->pf_ws = b + o_ws; d->pf_tokens = (int*)(b + o_tok);
+    d->pf_up = (float*)(b + o_up); d->pf_ws = b + o_ws; d->pf_ws2 = b + o_ws2; d->pf_tokens = (int*)(b + o_tok);
     d->pf_split = (float*)(b + o_split);
     d->pf_rows = rows;
     return PTM_OK;
@@ -243,38 +247,39 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
     PTM_TRY(hip_status(hipMemcpyAsync(d->pf_tokens, tokens_host, 4 * (size_t)M, hipMemcpyHostToDevice, s)));
     PTM_TRY(ptm_embedding_rows(c.embedding_f32, c.embedding_f32 ? nullptr : c.lm_head.data, c.lm_head.row_stride_bytes,
                                d->pf_tokens, M, H, c.vocab, d->pf_x, s));
-    // the workspace keeps the fp16 form of the last X it was given: consecutive products of the same rows with
-    // matrices of the same type (q and k, gate and up) convert them once
-    const float* ws_x = nullptr;
-    uint32_t ws_type = 0;
-    auto gemm = [&](const ptm_qweight& w, const float* X, float* Y, bool acc) {
-        const bool reuse = X == ws_x && w.ggml_type == ws_type;
-        ws_x = (Y == X) ? nullptr : X;
-        ws_type = w.ggml_type;
-        return qgemm_f16_impl(w.ggml_type, w.data, X, true, Y, M, w.cols, w.rows, w.row_stride_bytes, d->pf_ws, acc,
-                              d->pf_split, d->pf_split_bytes, reuse, s);
+    // Q4_K matrices take their rows from pf_ws (Q8-rounded fp16), Q6_K ones from pf_ws2 (plain fp16).  RMSNorm and
+    // SiLU.up are fused into the conversion (one launch fills both forms); a product whose rows are already in its
+    // workspace skips the conversion.
+    auto ws_of = [&](const ptm_qweight& w) { return w.ggml_type == PTM_TYPE_Q4_K ? d->pf_ws : d->pf_ws2; };
+    auto gemm = [&](const ptm_qweight& w, const float* X, float* Y, bool acc, bool rows_ready) {
+        return qgemm_f16_impl(w.ggml_type, w.data, X, true, Y, M, w.cols, w.rows, w.row_stride_bytes, ws_of(w), acc,
+                              d->pf_split, d->pf_split_bytes, rows_ready, s);
     };
-    auto touched = [&](const float* X) { if (ws_x == X) ws_x = nullptr; };  // X rewritten by a non-GEMM kernel
+    auto uses = [](uint32_t type, std::initializer_list<const ptm_qweight*> ws) {
+        for (const ptm_qweight* w : ws) if (w->ggml_type == type) return true;
+        return false;
+    };
     for (int li = 0; li < c.n_layers; ++li) {
         const ptm_layer& L = d->layers[li];
-        PTM_TRY(ptm_rms_norm(d->pf_x, L.attn_norm, d->pf_xn, M, H, c.rms_eps, 0, nullptr, s));
-        touched(d->pf_xn);
-        PTM_TRY(gemm(L.q, d->pf_xn, d->pf_q, false));
-        PTM_TRY(gemm(L.k, d->pf_xn, d->pf_k, false));
-        PTM_TRY(gemm(L.v, d->pf_xn, d->pf_v, false));
+        PTM_TRY(qgemm_f16_prepare_fused(1, d->pf_x, L.attn_norm, c.rms_eps, 0,
+                                        uses(PTM_TYPE_Q4_K, {&L.q, &L.k, &L.v}) ? d->pf_ws : nullptr,
+                                        uses(PTM_TYPE_Q6_K, {&L.q, &L.k, &L.v}) ? d->pf_ws2 : nullptr, M, H, s));
+        PTM_TRY(gemm(L.q, d->pf_x, d->pf_q, false, true));
+        PTM_TRY(gemm(L.k, d->pf_x, d->pf_k, false, true));
+        PTM_TRY(gemm(L.v, d->pf_x, d->pf_v, false, true));
         PTM_TRY(ptm_qknorm_rope_kvwrite_rows(d->pf_q, d->pf_k, d->pf_v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->rope, M,
                                              c.n_heads, c.n_kv_heads, hd, pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, s));
         PTM_TRY(ptm_prefill_attention(d->pf_q, L.k_cache, L.v_cache, d->pf_attn, M, c.n_heads, c.n_kv_heads, hd, pos0,
                                       c.max_seq, 1.0f / sqrtf((float)hd), c.kv_fp16, s));
-        touched(d->pf_attn);
-        PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true));  // x += attn . Wo^T
-        PTM_TRY(ptm_rms_norm(d->pf_x, L.ffn_norm, d->pf_xn, M, H, c.rms_eps, 0, nullptr, s));
-        touched(d->pf_xn);
-        PTM_TRY(gemm(L.gate, d->pf_xn, d->pf_gate, false));
-        PTM_TRY(gemm(L.up, d->pf_xn, d->pf_up, false));
-        PTM_TRY(ptm_silu_mul(d->pf_gate, d->pf_up, d->pf_gate, (int64_t)M * I, s));
-        touched(d->pf_gate);
-        PTM_TRY(gemm(L.down, d->pf_gate, d->pf_x, true));  // x += act . Wdown^T
+        PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true, false));  // x += attn . Wo^T
+        PTM_TRY(qgemm_f16_prepare_fused(1, d->pf_x, L.ffn_norm, c.rms_eps, 0,
+                                        uses(PTM_TYPE_Q4_K, {&L.gate, &L.up}) ? d->pf_ws : nullptr,
+                                        uses(PTM_TYPE_Q6_K, {&L.gate, &L.up}) ? d->pf_ws2 : nullptr, M, H, s));
+        PTM_TRY(gemm(L.gate, d->pf_x, d->pf_gate, false, true));
+        PTM_TRY(gemm(L.up, d->pf_x, d->pf_up, false, true));
+        PTM_TRY(qgemm_f16_prepare_fused(2, d->pf_gate, d->pf_up, 0.0f, 0, L.down.ggml_type == PTM_TYPE_Q4_K ? d->pf_ws : nullptr,
+                                        L.down.ggml_type == PTM_TYPE_Q6_K ? d->pf_ws2 : nullptr, M, I, s));
+        PTM_TRY(gemm(L.down, d->pf_gate, d->pf_x, true, true));  // x += act . Wdown^T
     }
     (void)qd; (void)kvd;
     return PTM_OK;

@@ -344,6 +344,91 @@ __global__ __launch_bounds__(256) void qgemm_prepare_rows_f16_kernel(const void*
     }
 }
 
+// The same conversion fused with what precedes a projection in the prompt pass, so that the fp32 intermediate is never
+// written: PRE 1 = RMSNorm of the row (x * rs * (gamma + add_one), the arithmetic and reduction order of
+// rms_norm_kernel), PRE 2 = SiLU(gate) * up (the arithmetic of silu_mul_kernel).  Writes the Q8-rounded form (for Q4_K
+// matrices) and / or the plain form (for Q6_K matrices) in one pass; either output may be NULL.
+template <int PRE>
+__global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* __restrict__ X, const float* __restrict__ X2,
+                                                                  float eps, int add_one, _Float16* __restrict__ Xh_round,
+                                                                  float* __restrict__ rs_round, _Float16* __restrict__ Xh_plain,
+                                                                  float* __restrict__ rs_plain, int M, int K) {
+    __shared__ float red[4];
+    __shared__ float red2[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const int n4 = K / 4;
+    if (m >= M) {  // padding rows: zeros
+        for (int i = tid; i < n4; i += 256) {
+            if (Xh_round) reinterpret_cast<uint2*>(Xh_round + (int64_t)m * K)[i] = make_uint2(0, 0);
+            if (Xh_plain) reinterpret_cast<uint2*>(Xh_plain + (int64_t)m * K)[i] = make_uint2(0, 0);
+        }
+        return;
+    }
+    const float* x = X + (int64_t)m * K;
+    const float* x2 = PRE == 2 ? X2 + (int64_t)m * K : X2;
+    float rs = 1.0f;
+    const float one = add_one ? 1.0f : 0.0f;
+    if constexpr (PRE == 1) {
+        float ss = 0.0f;
+        for (int i = tid; i < K; i += 256) ss = fmaf(x[i], x[i], ss);
+        ss = block_sum256(ss, red);
+        rs = 1.0f / sqrtf(ss / (float)K + eps);
+    }
+    auto value4 = [&](int i) {
+        const float4 a = reinterpret_cast<const float4*>(x)[i], b = reinterpret_cast<const float4*>(x2)[i];
+        float4 r;
+        if constexpr (PRE == 1) {
+            r.x = a.x * rs * (b.x + one); r.y = a.y * rs * (b.y + one); r.z = a.z * rs * (b.z + one); r.w = a.w * rs * (b.w + one);
+        } else {
+            auto silu_mul = [](float g, float u) {
+                float ng = 0.0f - g;
+                ng = fminf(fmaxf(ng, -88.0f), 88.0f);
+                return (g * (1.0f / (1.0f + expf(ng)))) * u;
+            };
+            r.x = silu_mul(a.x, b.x); r.y = silu_mul(a.y, b.y); r.z = silu_mul(a.z, b.z); r.w = silu_mul(a.w, b.w);
+        }
+        return r;
+    };
+    float amax = 0.0f;
+    for (int i = tid; i < n4; i += 256) {
+        const float4 v = value4(i);
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    }
+    amax = max64(amax);
+    if ((tid & 63) == 0) red2[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red2[0], red2[1]), fmaxf(red2[2], red2[3]));
+    int e = 0;
+    if (amax > 16384.0f) { (void)frexpf(amax, &e); e -= 14; }
+    const float down = ldexpf(1.0f, -e);
+    if (tid == 0) {
+        if (rs_round) rs_round[m] = ldexpf(1.0f, e);
+        if (rs_plain) rs_plain[m] = ldexpf(1.0f, e);
+    }
+    auto store4 = [&](_Float16* dst, int i, float4 v) {
+        union { _Float16 h[4]; uint2 u; } o;
+        o.h[0] = (_Float16)(v.x * down);
+        o.h[1] = (_Float16)(v.y * down);
+        o.h[2] = (_Float16)(v.z * down);
+        o.h[3] = (_Float16)(v.w * down);
+        reinterpret_cast<uint2*>(dst)[i] = o.u;
+    };
+    for (int i = tid; i < n4; i += 256) {  // K % 256 == 0: whole waves, aligned groups of 8 lanes = one Q8 block
+        const float4 v = value4(i);
+        if (Xh_plain) store4(Xh_plain + (int64_t)m * K, i, v);
+        if (Xh_round) {
+            float d, sm;
+            const uint32_t pk = q8_quantize4(v, d, sm);
+            float4 q;
+            q.x = d * (float)(int)(int8_t)(pk & 0xff);
+            q.y = d * (float)(int)(int8_t)((pk >> 8) & 0xff);
+            q.z = d * (float)(int)(int8_t)((pk >> 16) & 0xff);
+            q.w = d * (float)(int)(int8_t)(pk >> 24);
+            store4(Xh_round + (int64_t)m * K, i, q);
+        }
+    }
+}
+
 // 16 small integers (4 dwords of bytes, each < 1024) -> two fragments of 8 fp16 holding (byte - bias) * scale + offset.
 // A byte b becomes the fp16 number 1024 + b by writing it under the exponent byte 0x64 (one v_perm per pair); the
 // subtraction of 1024 + bias is exact, and one packed fp16 FMA applies scale and offset: 2.5 instructions per pair.
@@ -698,6 +783,24 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
         hipLaunchKernelGGL(qgemm_split_reduce_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, partials, splits,
                            Y, total, acc);
     }
+    return launch_status();
+}
+
+// Fills the row workspaces of qgemm_f16_impl (call it with reuse_rows afterwards): pre 1 = RMSNorm(X; gamma = X2), pre 2 =
+// SiLU(X) * X2.  ws_round serves Q4_K matrices, ws_plain Q6_K ones; either may be NULL.
+int qgemm_f16_prepare_fused(int pre, const float* X, const float* X2, float eps, int add_one, void* ws_round, void* ws_plain,
+                            int M, int K, hipStream_t s) {
+    if (!X || !X2 || (!ws_round && !ws_plain)) return PTM_E_NULL;
+    if (M <= 0 || K <= 0 || (K % 256) != 0) return PTM_E_SHAPE;
+    if (!aligned16(X) || !aligned16(X2) || !aligned16(ws_round) || !aligned16(ws_plain)) return PTM_E_ALIGN;
+    const int mp = qf_mpad(M);
+    _Float16* hr = static_cast<_Float16*>(ws_round);
+    _Float16* hp = static_cast<_Float16*>(ws_plain);
+    float* rr = hr ? reinterpret_cast<float*>(hr + (int64_t)mp * K) : nullptr;
+    float* rp = hp ? reinterpret_cast<float*>(hp + (int64_t)mp * K) : nullptr;
+    if (pre == 1) hipLaunchKernelGGL(qgemm_prepare_fused_kernel<1>, dim3(mp), dim3(256), 0, s, X, X2, eps, add_one, hr, rr, hp, rp, M, K);
+    else if (pre == 2) hipLaunchKernelGGL(qgemm_prepare_fused_kernel<2>, dim3(mp), dim3(256), 0, s, X, X2, eps, add_one, hr, rr, hp, rp, M, K);
+    else return PTM_E_UNSUPPORTED;
     return launch_status();
 }
 
