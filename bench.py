@@ -248,6 +248,16 @@ def main():
     dtp = (time.perf_counter() - t1) / 3
     gemv["prefill_512_tokens"] = {"ms": dtp * 1e3, "tok_s": 512 / dtp,
                                   "gemm_TFLOPs": 2.0 * 512 * nL * layer_params / dtp / 1e12}
+    prompt2k = [int(t) for t in synth.rng_for(SEED, 10).integers(0, V, 2048)]
+    dec.set_past_len(0)
+    dec.prefill(prompt2k)  # grows the row scratch to 2048 rows
+    t1 = time.perf_counter()
+    for _ in range(2):
+        dec.set_past_len(0)
+        dec.prefill(prompt2k)
+    dtp = (time.perf_counter() - t1) / 2
+    gemv["prefill_2048_tokens"] = {"ms": dtp * 1e3, "tok_s": 2048 / dtp,
+                                   "gemm_TFLOPs": 2.0 * 2048 * nL * layer_params / dtp / 1e12}
     log(json.dumps(gemv))
     per_token_bytes = nL * 63866880 + V * stride6 + nL * 2 * (N_PREFILL + args.warmup + args.steps / 2) * 1024 * 2
     dec.close()

@@ -308,7 +308,7 @@ int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token);
 /* Prefill: run n prompt tokens (host array) through the model at once, append their K/V rows at positions
  * past_len .. past_len + n - 1 and return the greedy token that follows the prompt; logits of the last
  * prompt token are left for ptm_decode_logits.  Rows go through the layers in chunks of chunk_rows
- * (<= 0: 512; at most 2048) with the fast quantised GEMM, row-batched QK-norm + RoPE + KV append and causal attention.
+ * (<= 0 or above 2048: 2048) with the fast quantised GEMM, row-batched QK-norm + RoPE + KV append and causal attention.
  * The counterpart of GGUFModel::forward(tokens, use_cache = true) (gguf_model.h:2510-2571); row m equals
  * a decode step of token m up to the fp16 rounding of the GEMM operands.  Allocates its scratch on first use. */
 int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_rows, int64_t* next_token);

@@ -336,8 +336,9 @@ inline int q4k_tiles_per_wg(int n_tiles) {
         return (e && e[0] >= '1' && e[0] <= '9' && e[1] == 0) ? e[0] - '0' : 0;
     }();
     if (forced > 0) return forced;
+    static const int max_wgs = [] { const char* e = getenv("PTM_Q4K_MAXWG"); return e ? atoi(e) : 1280; }();
     int t = 1;
-    while (t < 8 && (n_tiles + t - 1) / t > 1280) ++t;
+    while (t < 8 && (n_tiles + t - 1) / t > max_wgs) ++t;
     return t;
 }
 inline int q4k_blocks_per_pass(int nblk, int log2S) {
