@@ -242,7 +242,8 @@ int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* 
                   int64_t row_stride_bytes, void* workspace, ptm_stream_t stream);
 /* The same with fp32 rows of X (what the reference's prefill holds) and an optional Y += result.  When N gives
  * too few column tiles to fill the chip, K is split over several workgroups whose partial sums (held in the
- * workspace) are added in a fixed order, so results are reproducible; the split depends on N and K only.
+ * workspace) are added in a fixed order, so results are reproducible; the split depends on N, K and the class of M (<= 128,
+ * <= 256, more).
  * workspace: ptm_qgemm_f16_f32_workspace_bytes(M, K, N) bytes, 16-byte aligned. */
 int64_t ptm_qgemm_f16_f32_workspace_bytes(int M, int K, int N);
 int ptm_qgemm_f16_f32(uint32_t ggml_type, const void* W, const float* X_f32, float* Y, int M, int K, int N,

@@ -30,7 +30,7 @@ int q6k_gemv_argmax_impl(const void* W, const float* x, const float* gamma, floa
 int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
                    int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, bool reuse_rows,
                    hipStream_t s);
-int qgemm_f16_splits(int N, int K);
+int qgemm_f16_splits(int N, int K, int M);
 int qgemm_f16_prepare_fused(int pre, const float* X, const float* X2, float eps, int add_one, void* ws_round, void* ws_plain,
                             int M, int K, hipStream_t s);
 int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
@@ -221,10 +221,13 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
     size_t split_elems = 0;  // widest splits x N over the layer's matrices (all layers have the same shapes)
     for (const ptm_qweight* w : {&d->layers[0].q, &d->layers[0].k, &d->layers[0].v, &d->layers[0].o, &d->layers[0].gate,
                                  &d->layers[0].up, &d->layers[0].down}) {
-        const size_t e = (size_t)qgemm_f16_splits(w->rows, w->cols) * w->rows;
-        split_elems = e > split_elems ? e : split_elems;
+        for (const int m : {128, 256, rows}) {  // the split count depends on the row class: size for the widest use
+            const int mm = m < rows ? m : rows;
+            const size_t e = (size_t)qgemm_f16_splits(w->rows, w->cols, mm) * w->rows * (size_t)mm;
+            split_elems = e > split_elems ? e : split_elems;
+        }
     }
-    d->pf_split_bytes = 4 * R * split_elems;
+    d->pf_split_bytes = 4 * split_elems;
     const size_t o_split = take(d->pf_split_bytes);
     const int rc = hip_status(hipMalloc(&d->pf_slab, off));
     if (rc != PTM_OK) return rc;

@@ -695,13 +695,16 @@ __global__ __launch_bounds__(256) void qgemm_split_reduce_kernel(const float* __
     }
 }
 
-// K splits for an N x K weight matrix: enough workgroups to fill the chip when N alone gives few column tiles
-// (a 2560-wide projection is 10 tiles).  Depends on N and K only -- not on M -- so that the summation order of a
-// row does not change with how many rows share the launch.
-int qgemm_f16_splits(int N, int K) {
+// K splits for an N x K weight matrix and M rows: enough workgroups to fill the chip when N alone gives few column
+// tiles (a 2560-wide projection is 10 tiles).  M enters only through its class (up to 128 rows, up to 256, more), so
+// that the summation order of a row does not change with how many rows share the launch within a class; short
+// prompts (one row tile) get up to 16 splits, because there the launch is bound by how many workgroups stream weights.
+int qgemm_f16_splits(int N, int K, int M) {
     const int ntiles = (N + QF_TN - 1) / QF_TN, nblk = K / 256;
-    int s = 64 / ntiles;  // 4 row tiles (512 rows) x ntiles x s ~ 256 workgroups
-    s = s > 8 ? 8 : s;
+    const int row_tiles = M <= 128 ? 1 : (M <= 256 ? 2 : 4);
+    int s = 256 / (ntiles * row_tiles);
+    const int cap = row_tiles == 1 ? 16 : 8;
+    s = s > cap ? cap : s;
     s = s > nblk / 2 ? nblk / 2 : s;
     return s < 1 ? 1 : s;
 }
@@ -744,7 +747,7 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     _Float16* Xh = static_cast<_Float16*>(workspace);
     float* rowscale = reinterpret_cast<float*>(Xh + (int64_t)mp * K);
     const int nblk = K / 256;
-    int splits = split_ws ? qgemm_f16_splits(N, K) : 1;
+    int splits = split_ws ? qgemm_f16_splits(N, K, M) : 1;
     while (splits > 1 && (size_t)splits * M * N * sizeof(float) > split_ws_bytes) --splits;
     const int bps = (nblk + splits - 1) / splits;
     splits = (nblk + bps - 1) / bps;  // no empty split
@@ -863,7 +866,7 @@ int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* 
 int64_t ptm_qgemm_f16_f32_workspace_bytes(int M, int K, int N) {
     if (M <= 0 || K <= 0 || N <= 0) return 0;
     const int64_t base = (ptm_qgemm_f16_workspace_bytes(M, K) + 255) & ~(int64_t)255;
-    const int splits = qgemm_f16_splits(N, K);
+    const int splits = qgemm_f16_splits(N, K, M);
     return base + (splits > 1 ? (int64_t)splits * M * N * 4 : 0);
 }
 
@@ -872,7 +875,7 @@ int ptm_qgemm_f16_f32(uint32_t ggml_type, const void* W, const float* X_f32, flo
     if (M <= 0 || K <= 0 || N <= 0) return PTM_E_SHAPE;
     if (!workspace) return PTM_E_NULL;
     const int64_t base = (ptm_qgemm_f16_workspace_bytes(M, K) + 255) & ~(int64_t)255;
-    const int splits = qgemm_f16_splits(N, K);
+    const int splits = qgemm_f16_splits(N, K, M);
     return qgemm_f16_impl(ggml_type, W, X_f32, true, Y, M, K, N, stride, workspace, accumulate != 0,
                           splits > 1 ? reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + base) : nullptr,
                           splits > 1 ? (size_t)splits * M * N * 4 : 0, false, as_stream(stream));

@@ -193,8 +193,9 @@ def test_qgemm_f16_f32_rows_and_accumulate(dev, po, qt, M, K, N):
     rms = np.sqrt((ref.astype(np.float64) ** 2).mean())
     assert np.abs(Y.cpu().numpy() - ref).max() / rms <= PREFILL_TOL
     assert np.array_equal(bits(Ya.cpu().numpy()), bits(y0 + Y.cpu().numpy()))   # Y += is one fp32 add of the same product
-    # a row's result does not depend on how many rows share the launch (the K split is a function of N and K only)
-    m3 = min(3, M)
+    # a row's result does not depend on how many rows share the launch, within a row class (the K split is a function
+    # of N, K and of whether M is at most 128, at most 256, or more)
+    m3 = min(3, M) if M <= 128 else 129
     Y3 = torch.empty((m3, N), device="cuda")
     ops.matmul_q_f16_f32(qt, Wd, Xd[:m3].contiguous(), Y3, m3, K, N, W.shape[1], ws)
     torch.cuda.synchronize()
@@ -386,7 +387,8 @@ def test_q8_rounding_noise_floor_of_the_oracle(po, seeds):
 
 
 def test_prefill_chunking_does_not_change_the_result(dev, seeds):
-    """Chunks only bound the scratch: rows are independent in every GEMM (the K split depends on N and K only) and
+    """Chunks only bound the scratch: rows are independent in every GEMM (the K split depends on N, K and the row class,
+    here always "at most 128 rows") and
     attention reads the cache in the same tiles, so any chunk size that stays on the same attention kernel gives
     bit-identical logits; chunks under 16 rows use the fp32 attention kernel and agree within the end-to-end bars."""
     from prometorch_amd.decode import Decoder
