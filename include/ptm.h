@@ -320,6 +320,13 @@ int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_r
  * out_tokens.  Stop tokens are the caller's business: generate in short runs and cut at the first one. */
 int ptm_decode_sampling_begin(ptm_decoder* d, const ptm_sampling* params);
 int ptm_decode_sample(ptm_decoder* d, int token_id, int n, const float* uniforms_host, int64_t* out_tokens);
+/* The whole serving loop of api_handlers.h:848-923 in one call: the prompt (all but its last token through
+ * ptm_decode_prefill), then sample / stop check / feed back for up to max_new tokens; a stop token ends the output and
+ * is not part of it.  out_tokens must hold max_new ids; uniforms_host max_new draws.  On return past_len counts the
+ * prompt and every generated token that was fed back (the last generated token is not fed yet). */
+int ptm_decode_generate(ptm_decoder* d, const int32_t* prompt, int n_prompt, const ptm_sampling* params,
+                        const float* uniforms_host, int max_new, const int32_t* stop_ids, int n_stop,
+                        int64_t* out_tokens, int* n_out);
 int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_out);
 /* Device pointers to the last step's logits [vocab] and final-normed hidden [hidden]. */
 const float* ptm_decode_logits(ptm_decoder* d);

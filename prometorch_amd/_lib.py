@@ -97,6 +97,8 @@ SIGNATURES = {
     "ptm_embedding_rows": (i32, [vp, vp, i64, vp, i32, i32, i32, vp, vp]),
     "ptm_qknorm_rope_kvwrite_rows": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, i32, vp]),
     "ptm_prefill_attention": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, vp]),
+    "ptm_decode_generate": (i32, [vp, C.POINTER(C.c_int32), i32, C.POINTER(Sampling), C.POINTER(f32), i32, C.POINTER(C.c_int32),
+                                  i32, C.POINTER(i64), C.POINTER(i32)]),
     "ptm_decode_sampling_begin": (i32, [vp, C.POINTER(Sampling)]),
     "ptm_decode_sample": (i32, [vp, i32, i32, C.POINTER(f32), C.POINTER(i64)]),
     "ptm_sampler_workspace_bytes": (i64, []),

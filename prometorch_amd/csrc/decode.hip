@@ -459,6 +459,48 @@ int ptm_decode_sample(ptm_decoder* d, int token_id, int n, const float* uniforms
     return PTM_OK;
 }
 
+int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_rows, int64_t* next_token);
+
+// The serving loop (promeserve/api_handlers.h:848-923) in one call: prompt, then sample / check for a stop token /
+// feed back until max_new tokens or a stop token (which is not part of the output).  Tokens are generated in chained
+// runs of 16 steps; when a stop token turns up inside a run the steps after it are dropped (the cache rows they wrote
+// lie beyond past_len and are overwritten by whatever comes next).
+int ptm_decode_generate(ptm_decoder* d, const int32_t* prompt, int n_prompt, const ptm_sampling* params,
+                        const float* uniforms_host, int max_new, const int32_t* stop_ids, int n_stop, int64_t* out_tokens,
+                        int* n_out) {
+    if (!d || !prompt || !params || !uniforms_host || !out_tokens || !n_out || (n_stop > 0 && !stop_ids)) return PTM_E_NULL;
+    if (n_prompt <= 0 || max_new <= 0 || n_stop < 0) return PTM_E_SHAPE;
+    if (d->status != PTM_OK) return PTM_E_STATE;
+    if (d->past_len + n_prompt - 1 + max_new > d->cfg.max_seq) return PTM_E_RANGE;
+    *n_out = 0;
+    int rc;
+    if (n_prompt > 1) {
+        int64_t unused;
+        if ((rc = ptm_decode_prefill(d, prompt, n_prompt - 1, 0, &unused)) != PTM_OK) return rc;
+    } else if (prompt[0] < 0 || prompt[0] >= d->cfg.vocab) {
+        return PTM_E_RANGE;
+    }
+    if ((rc = ptm_decode_sampling_begin(d, params)) != PTM_OK) return rc;
+    int token = prompt[n_prompt - 1], produced = 0;
+    while (produced < max_new) {
+        const int run = max_new - produced < 16 ? max_new - produced : 16;
+        if ((rc = ptm_decode_sample(d, token, run, uniforms_host + produced, out_tokens + produced)) != PTM_OK) return rc;
+        for (int i = 0; i < run; ++i) {
+            const int64_t t = out_tokens[produced + i];
+            for (int k = 0; k < n_stop; ++k)
+                if (t == stop_ids[k]) {
+                    d->past_len -= run - (i + 1);  // steps i+1.. of the run fed the stop token and what followed it
+                    *n_out = produced + i;
+                    return PTM_OK;
+                }
+        }
+        produced += run;
+        token = (int)out_tokens[produced - 1];
+    }
+    *n_out = produced;
+    return PTM_OK;
+}
+
 int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_rows, int64_t* next_token) {
     if (!d || !tokens || !next_token) return PTM_E_NULL;
     if (d->status != PTM_OK) return PTM_E_STATE;

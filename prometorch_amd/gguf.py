@@ -239,6 +239,21 @@ class GGUFModel:
         check(self.L.ptm_decode_prefill(self.h, buf, n, chunk_rows, C.byref(out)), "decode_prefill")
         return out.value
 
+    def generate(self, prompt, uniforms, temperature: float, top_k: int, top_p: float, repeat_penalty: float = 1.0,
+                 stop_ids=()) -> list:
+        """Prompt, then up to len(uniforms) sampled tokens, ending before the first stop token (the serving loop of
+        promeserve/api_handlers.h:848-923 with everything but the token ids kept on the device)."""
+        from ._lib import Sampling
+        n, m, ns = len(prompt), len(uniforms), len(stop_ids)
+        pa = (C.c_int32 * n)(*[int(t) for t in prompt])
+        ua = (C.c_float * m)(*[float(u) for u in uniforms])
+        sa = (C.c_int32 * max(1, ns))(*[int(t) for t in stop_ids])
+        out = (C.c_int64 * m)()
+        n_out = C.c_int()
+        check(self.L.ptm_decode_generate(self.h, pa, n, Sampling(temperature, top_k, top_p, repeat_penalty), ua, m, sa, ns, out,
+                                         C.byref(n_out)), "decode_generate")
+        return list(out[:n_out.value])
+
     def sampling_begin(self, temperature: float, top_k: int, top_p: float, repeat_penalty: float = 1.0) -> None:
         """Start a sampled generation: store the parameters, forget previously generated tokens."""
         from ._lib import Sampling

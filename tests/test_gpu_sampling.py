@@ -181,3 +181,59 @@ def test_decoder_sampling_errors(dev, seeds):
         dec.sample(1, [0.5] * 33)                  # would overflow the cache
     assert len(dec.sample(1, [0.5] * 4)) == 4
     dec.close()
+
+
+def test_generate_loop_with_stop_tokens(dev, po, seeds):
+    """ptm_decode_generate against the reference's loop restated with the oracle: sample, stop on a stop id (not
+    emitted), feed back; and the decoder's position afterwards counts exactly the tokens that were fed."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = build_tiny(seeds)
+    params = (0.9, 30, 0.95, 1.2)
+    us = ops.mt19937_uniforms(42, 0, 50)
+
+    def oracle_loop(prompt, stops, min_gap=1e-4):
+        om = po.OracleModel(cfg, layers, head, 96, kv_fp16=True)
+        for t in prompt[:-1]:
+            om.step(t)
+        tok, gen, clear = prompt[-1], [], 0
+        for st in range(len(us)):
+            om.step(tok)
+            lg = po.repetition_penalty(om.logits, gen, params[3]) if gen else om.logits
+            tok, gap = po.sample_token(lg, params[0], params[1], params[2], us[st])
+            if gap > min_gap and clear == st:
+                clear = st + 1          # draws so far all sit clear of their interval edges
+            if tok in stops:
+                break
+            gen.append(tok)
+        return gen, om, clear
+
+    # a one-token prompt: no prefill, the decode path alone, which follows the oracle to ~1e-6 -- the loop logic exactly
+    prompt = [int(synth.rng_for(83).integers(0, cfg["vocab"]))]
+    free_run, _, clear = oracle_loop(prompt, ())
+    assert clear == len(us), "a draw sits on an interval edge: pick other draws"
+    dec = Decoder(cfg, layers, head, max_seq=96, kv_fp16=True, use_graph=True)
+    assert dec.generate(prompt, us, *params) == free_run
+    for cut in (0, 5, 15, 16, 17, 33, 49):  # a stop at the first token, inside a run of 16, on its edges, at the very end
+        stop = free_run[cut]
+        first = free_run.index(stop)
+        want, om, _ = oracle_loop(prompt, (stop, cfg["vocab"] + 5))
+        assert want == free_run[:first]
+        dec.set_past_len(0)
+        got = dec.generate(prompt, us, *params, stop_ids=(stop, cfg["vocab"] + 5))
+        assert got == want, cut
+        # position: the prompt and every generated token were fed; one more step must see exactly that context
+        probe = 11
+        t_o = om.step(probe)
+        t_g = dec.step(probe)
+        assert t_g == t_o and np.abs(dec.logits() - om.logits).max() / om.logits.std() <= 1e-3, cut
+    # a longer prompt goes through the prefill GEMMs (fp16 operands): the streams agree while the draws stay clear of
+    # the interval edges by more than that noise
+    prompt = [int(t) for t in synth.rng_for(84).integers(0, cfg["vocab"], 9)]
+    want, _, clear = oracle_loop(prompt, (), min_gap=3e-2)
+    dec.set_past_len(0)
+    got = dec.generate(prompt, us, *params)
+    assert len(got) == len(us) and got[:clear] == want[:clear] and clear >= 3
+    dec.set_past_len(0)
+    with pytest.raises(PtmError):
+        dec.generate(prompt, [0.5] * 200, *params)          # does not fit the cache
+    dec.close()
