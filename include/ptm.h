@@ -176,7 +176,11 @@ int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const 
                           const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
                           float* partial_lse, float* partial_max, const float* rope_table,
                           int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
-                          float scale, float eps, int add_one, int kv_fp16, ptm_stream_t stream);
+                          float scale, float eps, int add_one, int kv_fp16, int rope_interleaved,
+                          ptm_stream_t stream);
+/* q_norm_w / k_norm_w may both be NULL (models without QK-norm).  rope_interleaved: 0 rotates the NeoX pairs
+ * (d, d + head_dim/2) of qwen / gemma / phi (rope_apply_fused_neox, hot_loops.cpp:2035-2061), 1 the pairs
+ * (2d, 2d + 1) of llama / mistral (rope_apply_fused, hot_loops.cpp:1962-2030); config.rope_neox, gguf_model.h:98. */
 
 /* out = silu(gate) * up. launch_silu_mul (CUDAOps.h:416-418). */
 int ptm_silu_mul(const float* gate, const float* up, float* out, int64_t n, ptm_stream_t stream);
@@ -260,7 +264,7 @@ int ptm_embedding_rows(const float* table_f32, const void* table_q6k, int64_t q6
 int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
                                  void* K_cache, void* V_cache, const float* rope_table, int rows, int n_heads,
                                  int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float eps, int add_one,
-                                 int kv_fp16, ptm_stream_t stream);
+                                 int kv_fp16, int rope_interleaved, ptm_stream_t stream);
 /* Causal GQA attention of prompt row r over cache positions [0, pos0 + r] (the rows' own K/V already appended);
  * O [rows][n_heads*head_dim].  launch_causal_attention (gguf_model.h:7400; CUDAInference.cu:202-315). */
 int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cache, float* O, int rows, int n_heads,
@@ -277,7 +281,7 @@ typedef struct {
 
 typedef struct {
     ptm_qweight q, k, v, o, gate, up, down;
-    const float *attn_norm, *ffn_norm, *q_norm, *k_norm; /* device fp32 */
+    const float *attn_norm, *ffn_norm, *q_norm, *k_norm; /* device fp32; q_norm and k_norm both NULL: no QK-norm */
     void *k_cache, *v_cache; /* device [max_seq][kv_dim], fp16 or fp32 per kv_fp16 */
 } ptm_layer;
 
@@ -290,6 +294,7 @@ typedef struct {
     const ptm_layer* layers;      /* HOST array of n_layers descriptors (copied) */
     const float* out_norm;        /* device */
     ptm_qweight lm_head;
+    int32_t rope_interleaved;     /* 0: NeoX rotation pairs (qwen3); 1: pairs (2d, 2d+1) (llama, mistral) */
 } ptm_decode_config;
 
 typedef struct ptm_decoder ptm_decoder;

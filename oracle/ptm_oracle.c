@@ -339,6 +339,21 @@ void po_rope_apply_neox(float* q, float* k, const float* c, const float* s,
     for (int64_t h = 0; h < n_kv_heads; ++h) rope_neox_head(k + h * head_dim, c, s, head_dim / 2);
 }
 
+/* interleaved pairs (2d, 2d+1): the rotation of llama / mistral (reference: rope_apply_fused, hot_loops.cpp:1962-2030;
+ * the reference build contracts x0*c - x1*s and x0*s + x1*c into one fused multiply-add each, as below) */
+static void rope_norm_head(float* h, const float* c, const float* s, int64_t half) {
+    for (int64_t d = 0; d < half; ++d) {
+        const float a = h[2 * d], b = h[2 * d + 1];
+        h[2 * d] = fmaf(a, c[d], -(b * s[d]));
+        h[2 * d + 1] = fmaf(a, s[d], b * c[d]);
+    }
+}
+void po_rope_apply_norm(float* q, float* k, const float* c, const float* s,
+                        int64_t n_heads, int64_t n_kv_heads, int64_t head_dim) {
+    for (int64_t h = 0; h < n_heads; ++h) rope_norm_head(q + h * head_dim, c, s, head_dim / 2);
+    for (int64_t h = 0; h < n_kv_heads; ++h) rope_norm_head(k + h * head_dim, c, s, head_dim / 2);
+}
+
 /* ---- vector exp (reference: VectorizedOps.h:56-97; Cephes polynomial) ------------ */
 static inline __m256 exp8(__m256 x) {
     x = _mm256_max_ps(_mm256_min_ps(x, _mm256_set1_ps(88.3762626647949f)), _mm256_set1_ps(-88.3762626647949f));
@@ -450,9 +465,12 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
         qgemv(&L->q, xn, qb);
         qgemv(&L->k, xn, kb);
         qgemv(&L->v, xn, vb);
-        for (int64_t h = 0; h < nh; ++h) po_rmsnorm_vec(qb + h * hd, L->q_norm, m->eps, 0, hd, qb + h * hd);
-        for (int64_t h = 0; h < nkv; ++h) po_rmsnorm_vec(kb + h * hd, L->k_norm, m->eps, 0, hd, kb + h * hd);
-        po_rope_apply_neox(qb, kb, rc, rs, nh, nkv, hd);
+        if (L->q_norm) { /* QK-norm only where the model has it (gguf_model.h:3441-3450) */
+            for (int64_t h = 0; h < nh; ++h) po_rmsnorm_vec(qb + h * hd, L->q_norm, m->eps, 0, hd, qb + h * hd);
+            for (int64_t h = 0; h < nkv; ++h) po_rmsnorm_vec(kb + h * hd, L->k_norm, m->eps, 0, hd, kb + h * hd);
+        }
+        if (m->rope_interleaved) po_rope_apply_norm(qb, kb, rc, rs, nh, nkv, hd); /* gguf_model.h:3464-3470 */
+        else po_rope_apply_neox(qb, kb, rc, rs, nh, nkv, hd);
         float* kc = L->k_cache + past * kvd;
         float* vc = L->v_cache + past * kvd;
         for (int64_t j = 0; j < kvd; ++j) {

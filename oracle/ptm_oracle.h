@@ -15,7 +15,7 @@
  *   po_q4k_gemv            golden y from the compiled reference (bit-exact) + exact int dots vs numpy
  *   po_q6k_gemv            golden y from the compiled reference (bit-exact) + float64 dot of dequant
  *   po_rmsnorm_*           compiled reference + float64 numpy
- *   po_rope_*              compiled reference + float64 closed form (NeoX pairing)
+ *   po_rope_*              compiled reference + float64 closed form (NeoX and interleaved pairing)
  *   po_exp256              compiled reference + float64 exp
  *   po_attn_head, po_silu_mul, po_argmax, po_decode_step
  *                          golden logits / token ids of the compiled reference's
@@ -63,6 +63,8 @@ void po_q4k_row_isums(const void* row, const int8_t* qs, int64_t K, int32_t* isu
 void po_rmsnorm_seq(const float* x, const float* gamma, float eps, int add_one, int64_t H, float* out);
 void po_rmsnorm_vec(const float* x, const float* gamma, float eps, int add_one, int64_t H, float* out);
 void po_rope_precompute(float* c, float* s, int64_t pos, int64_t head_dim, float base);
+void po_rope_apply_norm(float* q, float* k, const float* c, const float* s, int64_t n_heads, int64_t n_kv_heads,
+                        int64_t head_dim);
 void po_rope_apply_neox(float* q, float* k, const float* c, const float* s,
                         int64_t n_heads, int64_t n_kv_heads, int64_t head_dim);
 void po_exp256(const float* in, float* out, int64_t n8);
@@ -79,7 +81,7 @@ typedef struct {
 
 typedef struct {
     po_qweight q, k, v, o, gate, up, down;
-    const float *attn_norm, *ffn_norm, *q_norm, *k_norm;
+    const float *attn_norm, *ffn_norm, *q_norm, *k_norm; /* q_norm, k_norm: NULL for models without QK-norm */
     float *k_cache, *v_cache; /* [max_seq][kv_dim] fp32 storage */
 } po_layer;
 
@@ -92,6 +94,7 @@ typedef struct {
     const float* out_norm;
     po_qweight lm_head;
     int64_t seq_len;
+    int rope_interleaved;   /* 0: NeoX pairs (d, d + half) as qwen / gemma / phi; 1: pairs (2d, 2d + 1) as llama / mistral */
 } po_model;
 
 /* One decode step (forward_decode_cpu order, Q4_K_M fallbacks); writes logits[vocab],

@@ -40,7 +40,7 @@ class Layer(C.Structure):
 class Model(C.Structure):
     _fields_ = [(n, _i64) for n in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")] + \
                [("rope_base", _f32), ("eps", _f32), ("kv_fp16", _i32), ("embedding", _vp),
-                ("layers", C.POINTER(Layer)), ("out_norm", _vp), ("lm_head", QW), ("seq_len", _i64)]
+                ("layers", C.POINTER(Layer)), ("out_norm", _vp), ("lm_head", QW), ("seq_len", _i64), ("rope_interleaved", _i32)]
 
 
 _lib = None
@@ -71,6 +71,7 @@ def lib():
         L.po_rmsnorm_vec.argtypes = [_vp, _vp, _f32, _i32, _i64, _vp]
         L.po_rope_precompute.argtypes = [_vp, _vp, _i64, _i64, _f32]
         L.po_rope_apply_neox.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
+        L.po_rope_apply_norm.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
         L.po_exp256.argtypes = [_vp, _vp, _i64]
         L.po_attn_head.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp, _vp]
         L.po_silu_mul.argtypes = [_vp, _vp, _i64]
@@ -151,6 +152,14 @@ def rope_tables(pos, head_dim, base):
     return c, s
 
 
+def rope_norm(q, k, c, s, n_heads, n_kv_heads, head_dim):
+    """Interleaved pairs (2d, 2d + 1): llama / mistral."""
+    q = np.array(q, np.float32, copy=True)
+    k = np.array(k, np.float32, copy=True)
+    lib().po_rope_apply_norm(_p(q), _p(k), _p(c), _p(s), n_heads, n_kv_heads, head_dim)
+    return q, k
+
+
 def rope_neox(q, k, c, s, n_heads, n_kv_heads, head_dim):
     q = np.array(q, np.float32, copy=True)
     k = np.array(k, np.float32, copy=True)
@@ -229,6 +238,7 @@ class OracleModel:
     """Host-side model for po_decode_step; keeps every numpy buffer alive."""
 
     def __init__(self, cfg: dict, layers: list, head: dict, max_seq: int, kv_fp16: bool, embedding=None):
+        """cfg may carry 'rope_interleaved' (llama-style rotation pairs); layers without 'q_norm' / 'k_norm' have no QK-norm."""
         self.cfg = cfg
         self._keep = []
         kvd = cfg["n_kv_heads"] * cfg["head_dim"]
@@ -241,6 +251,9 @@ class OracleModel:
                 self._keep.append(Wc)
                 setattr(self.layers[i], name, qw)
             for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+                if L.get(name) is None:
+                    setattr(self.layers[i], name, None)
+                    continue
                 a = np.ascontiguousarray(L[name], np.float32)
                 self._keep.append(a)
                 setattr(self.layers[i], name, a.ctypes.data)
@@ -270,6 +283,7 @@ class OracleModel:
         self.m.out_norm = on.ctypes.data
         self.m.lm_head = lm
         self.m.seq_len = 0
+        self.m.rope_interleaved = int(bool(cfg.get("rope_interleaved", False)))
         self.logits = np.empty(cfg["vocab"], np.float32)
         self.hidden = np.empty(cfg["hidden"], np.float32)
 
@@ -309,6 +323,8 @@ def ref():
         R.ref_rmsnorm_inplace.argtypes = [_vp, _vp, _f32, _i32, _i64]
         R.ref_rope_precompute.argtypes = [_vp, _vp, _i64, _i64, _f32]
         R.ref_rope_apply_neox.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
+        R.ref_rope_apply_norm.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
+        R.ref_model_set_arch.argtypes = [_vp, _i32, _i32]
         R.ref_exp256.argtypes = [_vp, _vp, _i64]
         R.ref_num_threads.restype = _i32
         R.ref_model_create.restype = _vp
@@ -363,6 +379,8 @@ class RefModel:
         self.cfg = cfg
         self.h = R.ref_model_create(cfg["vocab"], cfg["hidden"], cfg["n_layers"], cfg["n_heads"], cfg["n_kv_heads"],
                                     cfg["head_dim"], cfg["inter"], cfg["rope_base"], cfg["eps"], max_seq)
+        if cfg.get("rope_interleaved") or layers[0].get("q_norm") is None:
+            R.ref_model_set_arch(self.h, int(layers[0].get("q_norm") is not None), int(not cfg.get("rope_interleaved")))
         names = ("q", "k", "v", "o", "gate", "up", "down")
         for i, L in enumerate(layers):
             for w, name in enumerate(names):
@@ -372,6 +390,8 @@ class RefModel:
                 K = W.shape[1] // (144 if qt == 12 else 210) * 256
                 R.ref_model_set_weight(self.h, i, w, _p(W), qt, W.shape[0], K)
             for w, name in enumerate(("attn_norm", "ffn_norm", "q_norm", "k_norm")):
+                if L.get(name) is None:
+                    continue
                 a = np.ascontiguousarray(L[name], np.float32)
                 R.ref_model_set_norm(self.h, i, w, _p(a), a.size)
         lm = np.ascontiguousarray(head["lm_head"], np.uint8)

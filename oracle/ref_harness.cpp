@@ -77,6 +77,10 @@ void ref_exp256(const float* in, float* out, int64_t n8) {
     for (int64_t i = 0; i < n8; ++i)
         _mm256_storeu_ps(out + 8 * i, at::native::vec::exp256_ps(_mm256_loadu_ps(in + 8 * i)));
 }
+void ref_rope_apply_norm(float* qv, float* kv, const float* c, const float* s,
+                         int64_t n_heads, int64_t n_kv_heads, int64_t head_dim) {
+    at::native::hot::rope_apply_fused(qv, kv, c, s, n_heads, n_kv_heads, head_dim);
+}
 int ref_num_threads() { return c10::get_thread_pool().num_threads(); }
 
 // ---------------------------------------------------------------------------------
@@ -102,6 +106,13 @@ void* ref_model_create(int64_t vocab, int64_t hidden, int64_t n_layers, int64_t 
     r->m.use_cuda_ = false;
     r->m.kv_cache.allocate(n_layers, max_seq, n_kv_heads * head_dim, false);
     return r;
+}
+// llama-style models: no per-head QK-norm (the norm tensors stay undefined: never call ref_model_set_norm with which 2, 3)
+// and interleaved rotation pairs (config.rope_neox, gguf_model.h:98)
+void ref_model_set_arch(void* h, int has_qk_norm, int rope_neox) {
+    auto& c = static_cast<RefModel*>(h)->m.config;
+    c.has_qk_norm = has_qk_norm != 0;
+    c.rope_neox = rope_neox != 0;
 }
 void ref_model_destroy(void* h) {
     auto* r = static_cast<RefModel*>(h);

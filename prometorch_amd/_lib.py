@@ -31,7 +31,8 @@ class Layer(C.Structure):
 class DecodeConfig(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")] + \
                [("rope_freq_base", f32), ("rms_eps", f32), ("kv_fp16", C.c_int32), ("use_graph", C.c_int32),
-                ("embedding_f32", vp), ("layers", C.POINTER(Layer)), ("out_norm", vp), ("lm_head", QWeight)]
+                ("embedding_f32", vp), ("layers", C.POINTER(Layer)), ("out_norm", vp), ("lm_head", QWeight),
+                ("rope_interleaved", C.c_int32)]
 
 
 class Sampling(C.Structure):
@@ -74,7 +75,7 @@ SIGNATURES = {
     "ptm_flash_decode_kv_chunk_size": (i32, []),
     "ptm_flash_decode_num_splits": (i32, [i32]),
     "ptm_flash_decode": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, i32, vp]),
-    "ptm_attn_decode_fused": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, f32, i32, i32, vp]),
+    "ptm_attn_decode_fused": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, f32, i32, i32, i32, vp]),
     "ptm_silu_mul": (i32, [vp, vp, vp, i64, vp]),
     "ptm_embedding_row": (i32, [vp, vp, vp, i32, vp]),
     "ptm_embedding_row_q6k": (i32, [vp, vp, vp, i32, i64, vp]),
@@ -95,7 +96,7 @@ SIGNATURES = {
     "ptm_qgemm_f16_f32_workspace_bytes": (i64, [i32, i32, i32]),
     "ptm_qgemm_f16_f32": (i32, [u32, vp, vp, vp, i32, i32, i32, i64, vp, i32, vp]),
     "ptm_embedding_rows": (i32, [vp, vp, i64, vp, i32, i32, i32, vp, vp]),
-    "ptm_qknorm_rope_kvwrite_rows": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, i32, vp]),
+    "ptm_qknorm_rope_kvwrite_rows": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, i32, i32, vp]),
     "ptm_prefill_attention": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, vp]),
     "ptm_decode_generate": (i32, [vp, C.POINTER(C.c_int32), i32, C.POINTER(Sampling), C.POINTER(f32), i32, C.POINTER(C.c_int32),
                                   i32, C.POINTER(i64), C.POINTER(i32)]),

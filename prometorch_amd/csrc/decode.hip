@@ -160,7 +160,7 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
         // QK-norm + RoPE + K/V append + split-KV attention in one launch, plus the small merge launch
         PTM_TRY(ptm_attn_decode_fused(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn, d->pO,
                                       d->pL, d->pM, d->rope, c.n_heads, c.n_kv_heads, hd, d->d_past,
-                                      c.max_seq, 1.0f / sqrtf((float)hd), c.rms_eps, 0, c.kv_fp16, s));
+                                      c.max_seq, 1.0f / sqrtf((float)hd), c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, s));
         PTM_TRY(gemv_any(L.o, d->attn, d->x, true, s));  // x += Wo . attn
         if (L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
             L.gate.row_stride_bytes == L.up.row_stride_bytes && L.gate.rows == L.up.rows) {
@@ -271,7 +271,7 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
         PTM_TRY(gemm(L.k, d->pf_x, d->pf_k, false, true));
         PTM_TRY(gemm(L.v, d->pf_x, d->pf_v, false, true));
         PTM_TRY(ptm_qknorm_rope_kvwrite_rows(d->pf_q, d->pf_k, d->pf_v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->rope, M,
-                                             c.n_heads, c.n_kv_heads, hd, pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, s));
+                                             c.n_heads, c.n_kv_heads, hd, pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, s));
         PTM_TRY(ptm_prefill_attention(d->pf_q, L.k_cache, L.v_cache, d->pf_attn, M, c.n_heads, c.n_kv_heads, hd, pos0,
                                       c.max_seq, 1.0f / sqrtf((float)hd), c.kv_fp16, s));
         PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true, false));  // x += attn . Wo^T
@@ -306,7 +306,8 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     if (!c.embedding_f32 && c.lm_head.ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
     for (int i = 0; i < c.n_layers; ++i) {
         const ptm_layer& L = c.layers[i];
-        if (!L.attn_norm || !L.ffn_norm || !L.q_norm || !L.k_norm || !L.k_cache || !L.v_cache) return PTM_E_NULL;
+        if (!L.attn_norm || !L.ffn_norm || !L.k_cache || !L.v_cache) return PTM_E_NULL;
+        if ((L.q_norm == nullptr) != (L.k_norm == nullptr)) return PTM_E_NULL;  // QK-norm: both or neither
         if ((rc = qw_check(L.q, qd, H)) || (rc = qw_check(L.k, kvd, H)) || (rc = qw_check(L.v, kvd, H)) ||
             (rc = qw_check(L.o, H, qd)) || (rc = qw_check(L.gate, c.inter, H)) || (rc = qw_check(L.up, c.inter, H)) ||
             (rc = qw_check(L.down, H, c.inter)))

@@ -263,6 +263,7 @@ struct AttnArgs {
     const int64_t* d_past;
     int n_heads, n_kv_heads, max_seq, add_one;
     float scale, eps;
+    int rope_interleaved;  // 0: NeoX pairs (d, d + HD/2); 1: pairs (2d, 2d + 1) as llama / mistral rotate (hot_loops.cpp:1962-2030)
 };
 
 // one wave: RMSNorm (optional) + NeoX rotation of a head held as pairs (t, t+HD/2); results to dst[HD]
@@ -345,16 +346,18 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     const float* cs = a.rope + past * HD;
     const float* qwp = has_norm ? a.qw : a.Q;  // a valid address either way; unused without norm weights
     const float* kwp = has_norm ? a.kw : a.Q;
+    // lane lh owns rotation pair lh: elements (i0, i1) of a head
+    const int i0 = a.rope_interleaved ? 2 * lh : lh, i1 = a.rope_interleaved ? 2 * lh + 1 : lh + HALF;
     float qx0[G], qx1[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         const float* src = a.Q + (int64_t)(kvh * G + g) * HD;
-        qx0[g] = src[lh];
-        qx1[g] = src[lh + HALF];
+        qx0[g] = src[i0];
+        qx1[g] = src[i1];
     }
-    const float qn0 = qwp[lh], qn1 = qwp[lh + HALF], kn0 = kwp[lh], kn1 = kwp[lh + HALF];
+    const float qn0 = qwp[i0], qn1 = qwp[i1], kn0 = kwp[i0], kn1 = kwp[i1];
     const float rc = cs[lh], rsn = cs[HALF + lh];
-    float kx0 = a.K[(int64_t)kvh * HD + lh], kx1 = a.K[(int64_t)kvh * HD + lh + HALF];
+    float kx0 = a.K[(int64_t)kvh * HD + i0], kx1 = a.K[(int64_t)kvh * HD + i1];
     float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
     issue_order_fence();
     // ---- ... then the cached K/V rows of this wave's positions (the new position is not cached: clamp below it) ----
@@ -391,8 +394,8 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
             x1 = x1 * rs * (qn1 + one);
         }
         if (on) {
-            s_q[wave][g][lane] = fmaf(x0, rc, -(x1 * rsn));
-            s_q[wave][g][lane + HALF] = fmaf(x0, rsn, x1 * rc);
+            s_q[wave][g][i0] = fmaf(x0, rc, -(x1 * rsn));
+            s_q[wave][g][i1] = fmaf(x0, rsn, x1 * rc);
         }
     }
     if (owner) {  // workgroup-uniform
@@ -410,23 +413,23 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
         if constexpr (KV16) {
             const __half h0 = __float2half_rn(r0), h1 = __float2half_rn(r1), g0 = __float2half_rn(vx0), g1 = __float2half_rn(vx1);
             if (on && wave == 0) {
-                static_cast<__half*>(a.Kc)[rowoff + lane] = h0;
-                static_cast<__half*>(a.Kc)[rowoff + lane + HALF] = h1;
+                static_cast<__half*>(a.Kc)[rowoff + i0] = h0;
+                static_cast<__half*>(a.Kc)[rowoff + i1] = h1;
                 static_cast<__half*>(a.Vc)[rowoff + lane] = g0;
                 static_cast<__half*>(a.Vc)[rowoff + lane + HALF] = g1;
             }
             r0 = __half2float(h0); r1 = __half2float(h1); vx0 = __half2float(g0); vx1 = __half2float(g1);
         } else {
             if (on && wave == 0) {
-                static_cast<float*>(a.Kc)[rowoff + lane] = r0;
-                static_cast<float*>(a.Kc)[rowoff + lane + HALF] = r1;
+                static_cast<float*>(a.Kc)[rowoff + i0] = r0;
+                static_cast<float*>(a.Kc)[rowoff + i1] = r1;
                 static_cast<float*>(a.Vc)[rowoff + lane] = vx0;
                 static_cast<float*>(a.Vc)[rowoff + lane + HALF] = vx1;
             }
         }
         if (on) {
-            s_new[wave][0][lane] = r0;
-            s_new[wave][0][lane + HALF] = r1;
+            s_new[wave][0][i0] = r0;
+            s_new[wave][0][i1] = r1;
             s_new[wave][1][lane] = vx0;
             s_new[wave][1][lane + HALF] = vx1;
         }
@@ -595,7 +598,7 @@ int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const 
                           const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
                           float* partial_lse, float* partial_max, const float* rope_table,
                           int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
-                          float scale, float eps, int add_one, int kv_fp16, ptm_stream_t stream) {
+                          float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, ptm_stream_t stream) {
     if (!Q || !K || !V || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max ||
         !rope_table || !d_past_len)
         return PTM_E_NULL;
@@ -604,7 +607,7 @@ int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const 
     if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
     if (!aligned16(K_cache) || !aligned16(V_cache) || !aligned16(partial_O) || !aligned16(O)) return PTM_E_ALIGN;
     AttnArgs a{Q, K, V, q_norm_w, k_norm_w, rope_table, K_cache, V_cache, partial_O, partial_lse, partial_max,
-               d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps};
+               d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps, rope_interleaved ? 1 : 0};
     const int G = n_heads / n_kv_heads;
     const dim3 grid(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
     hipStream_t s = as_stream(stream);

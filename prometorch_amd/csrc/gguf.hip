@@ -371,8 +371,11 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
     const char* arch_c = ptm_gguf_get_string(m->file, "general.architecture");
     if (!arch_c) { ptm_model_free(m); return PTM_E_FORMAT; }
     const std::string arch = arch_c;
-    // the decode step built here is the qwen3 one: RMSNorm, per-head QK-norm, NeoX RoPE, SwiGLU, no biases
-    if (arch != "qwen3") { ptm_model_free(m); return PTM_E_UNSUPPORTED; }
+    // two decode steps are built here, both RMSNorm + SwiGLU without biases: qwen3 (per-head QK-norm, rotation pairs
+    // half a head apart) and llama, which mistral files also carry (no QK-norm, interleaved pairs (2d, 2d+1));
+    // gguf_model.h:202-217 makes the same split by architecture name
+    const bool is_llama = arch == "llama";
+    if (arch != "qwen3" && !is_llama) { ptm_model_free(m); return PTM_E_UNSUPPORTED; }
     auto geti = [&](const char* key, int64_t def, bool required) -> int64_t {
         int64_t v = def;
         const int r = ptm_gguf_get_int(m->file, (arch + "." + key).c_str(), &v);
@@ -399,6 +402,7 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
     c.max_seq = max_seq;
     c.kv_fp16 = kv_fp16 ? 1 : 0;
     c.use_graph = use_graph ? 1 : 0;
+    c.rope_interleaved = is_llama ? 1 : 0;
     // vocabulary size from the embedding table [hidden x vocab]
     ptm_gguf_tensor emb{};
     PTM_L(ptm_gguf_find_tensor(m->file, "token_embd.weight", &emb));
@@ -439,8 +443,13 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
         PTM_L(load_matrix(m, p + "attn_k.weight", kvd, c.hidden, &L.k));
         PTM_L(load_matrix(m, p + "attn_v.weight", kvd, c.hidden, &L.v));
         PTM_L(load_matrix(m, p + "attn_output.weight", c.hidden, qd, &L.o));
-        PTM_L(load_vector(m, p + "attn_q_norm.weight", c.head_dim, &L.q_norm));
-        PTM_L(load_vector(m, p + "attn_k_norm.weight", c.head_dim, &L.k_norm));
+        if (is_llama) {
+            L.q_norm = nullptr;
+            L.k_norm = nullptr;
+        } else {
+            PTM_L(load_vector(m, p + "attn_q_norm.weight", c.head_dim, &L.q_norm));
+            PTM_L(load_vector(m, p + "attn_k_norm.weight", c.head_dim, &L.k_norm));
+        }
         PTM_L(load_vector(m, p + "ffn_norm.weight", c.hidden, &L.ffn_norm));
         PTM_L(load_matrix(m, p + "ffn_gate.weight", c.inter, c.hidden, &L.gate));
         PTM_L(load_matrix(m, p + "ffn_up.weight", c.inter, c.hidden, &L.up));

@@ -57,7 +57,7 @@ __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restri
                                                                  const float* __restrict__ kw, void* __restrict__ Kc,
                                                                  void* __restrict__ Vc, const float* __restrict__ rope,
                                                                  int n_heads, int n_kv_heads, int head_dim, int64_t pos0,
-                                                                 float eps, int add_one) {
+                                                                 float eps, int add_one, int rope_interleaved) {
     const int m = blockIdx.x, hb = blockIdx.y;
     const bool is_k = hb >= n_heads;
     const int h = is_k ? hb - n_heads : hb;
@@ -68,7 +68,8 @@ __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restri
     const float* nw = is_k ? kw : qw;
     const int half = head_dim / 2, t = threadIdx.x;
     const bool on = t < half;
-    float x0 = on ? vec[t] : 0.0f, x1 = on ? vec[t + half] : 0.0f;
+    const int i0 = rope_interleaved ? 2 * t : t, i1 = rope_interleaved ? 2 * t + 1 : t + half;  // rotation pair t
+    float x0 = on ? vec[i0] : 0.0f, x1 = on ? vec[i1] : 0.0f;
     if (nw) {
         float ss = fmaf(x0, x0, 0.0f);
         ss = fmaf(x1, x1, ss);
@@ -76,31 +77,31 @@ __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restri
         const float rs = 1.0f / sqrtf(ss / (float)head_dim + eps);
         const float one = add_one ? 1.0f : 0.0f;
         if (on) {
-            x0 = x0 * rs * (nw[t] + one);
-            x1 = x1 * rs * (nw[t + half] + one);
+            x0 = x0 * rs * (nw[i0] + one);
+            x1 = x1 * rs * (nw[i1] + one);
         }
     }
     if (!on) return;
     const float* cs = rope + pos * head_dim;
     const float c = cs[t], s = cs[half + t];
     const float r0 = fmaf(x0, c, -(x1 * s)), r1 = fmaf(x0, s, x1 * c);  // hot_loops.cpp:2035-2061
-    vec[t] = r0;
-    vec[t + half] = r1;
+    vec[i0] = r0;
+    vec[i1] = r1;
     if (is_k) {
         const int64_t off = pos * kv_dim + (int64_t)h * head_dim;
         const float v0 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t], v1 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t + half];
         if constexpr (KV16) {
             __half* kc = static_cast<__half*>(Kc) + off;
             __half* vc = static_cast<__half*>(Vc) + off;
-            kc[t] = __float2half_rn(r0);
-            kc[t + half] = __float2half_rn(r1);
+            kc[i0] = __float2half_rn(r0);
+            kc[i1] = __float2half_rn(r1);
             vc[t] = __float2half_rn(v0);
             vc[t + half] = __float2half_rn(v1);
         } else {
             float* kc = static_cast<float*>(Kc) + off;
             float* vc = static_cast<float*>(Vc) + off;
-            kc[t] = r0;
-            kc[t + half] = r1;
+            kc[i0] = r0;
+            kc[i1] = r1;
             vc[t] = v0;
             vc[t + half] = v1;
         }
@@ -420,7 +421,7 @@ int ptm_embedding_rows(const float* table_f32, const void* table_q6k, int64_t q6
 int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
                                  void* K_cache, void* V_cache, const float* rope_table, int rows, int n_heads,
                                  int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float eps, int add_one,
-                                 int kv_fp16, ptm_stream_t stream) {
+                                 int kv_fp16, int rope_interleaved, ptm_stream_t stream) {
     if (!Q || !K || !V || !K_cache || !V_cache || !rope_table) return PTM_E_NULL;
     if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
     if (rows <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || head_dim <= 0 || (head_dim & 1) || head_dim > 128)
@@ -430,10 +431,10 @@ int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float
     const dim3 grid(rows, n_heads + n_kv_heads);
     if (kv_fp16)
         hipLaunchKernelGGL(qknorm_rope_kv_rows_kernel<true>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
-                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one);
+                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0);
     else
         hipLaunchKernelGGL(qknorm_rope_kv_rows_kernel<false>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
-                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one);
+                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0);
     return launch_status();
 }
 

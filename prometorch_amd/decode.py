@@ -24,7 +24,8 @@ class Decoder:
     """Greedy batch-1 decoder over caller-provided quantised weights.
 
     layers: list of dicts with (qtype, uint8[rows, stride]) per projection name and fp32 norm
-    vectors 'attn_norm', 'ffn_norm', 'q_norm', 'k_norm'; head: {'lm_head': uint8 Q6_K table,
+    vectors 'attn_norm', 'ffn_norm', 'q_norm', 'k_norm' (the last two None for a model without QK-norm;
+    cfg['rope_interleaved'] selects llama-style rotation pairs); head: {'lm_head': uint8 Q6_K table,
     'out_norm': fp32}.  The token-embedding is the tied Q6_K table unless embedding_f32 is given."""
 
     def __init__(self, cfg: dict, layers: list, head: dict, max_seq: int, kv_fp16: bool = True,
@@ -47,6 +48,9 @@ class Decoder:
                 bb = 144 if qt == 12 else 210
                 setattr(arr[i], name, QWeight(t.data_ptr(), qt, W.shape[0], W.shape[1] // bb * 256, W.shape[1]))
             for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+                if Ld.get(name) is None:  # q_norm / k_norm: a model without QK-norm
+                    setattr(arr[i], name, None)
+                    continue
                 t = torch.from_numpy(np.ascontiguousarray(Ld[name], np.float32)).cuda()
                 self._keep.append(t)
                 setattr(arr[i], name, t.data_ptr())
@@ -68,6 +72,7 @@ class Decoder:
         c.rms_eps = cfg["eps"]
         c.kv_fp16 = int(kv_fp16)
         c.use_graph = int(use_graph)
+        c.rope_interleaved = int(bool(cfg.get("rope_interleaved", False)))
         if embedding_f32 is not None:
             e = embedding_f32 if isinstance(embedding_f32, torch.Tensor) else torch.from_numpy(embedding_f32)
             e = e.to(device="cuda", dtype=torch.float32).contiguous()

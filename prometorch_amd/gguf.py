@@ -95,8 +95,9 @@ def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "q
             qt, W = L[k]
             cols = W.shape[1] // (144 if qt == Q4_K else 210) * 256
             ts.append((p + gname + ".weight", qt, [cols, W.shape[0]], W))
-        ts.append((p + "attn_q_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["q_norm"], np.float32)))
-        ts.append((p + "attn_k_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["k_norm"], np.float32)))
+        if L.get("q_norm") is not None:  # absent in a llama-style model
+            ts.append((p + "attn_q_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["q_norm"], np.float32)))
+            ts.append((p + "attn_k_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["k_norm"], np.float32)))
         ts.append((p + "ffn_norm.weight", F32, [H], np.asarray(L["ffn_norm"], np.float32)))
     write_gguf(path, md, ts, alignment=alignment)
 
@@ -206,7 +207,8 @@ class GGUFModel:
         c = DecodeConfig()
         check(self.L.ptm_model_config(m, C.byref(c)), "model_config")
         self.cfg = {k: getattr(c, k) for k in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")}
-        self.cfg.update(rope_base=c.rope_freq_base, eps=c.rms_eps, kv_fp16=bool(c.kv_fp16), tied=not bool(c.embedding_f32))
+        self.cfg.update(rope_base=c.rope_freq_base, eps=c.rms_eps, kv_fp16=bool(c.kv_fp16), tied=not bool(c.embedding_f32),
+                        rope_interleaved=bool(c.rope_interleaved))
 
     def layer(self, i: int) -> Layer:
         out = Layer()

@@ -212,13 +212,13 @@ def launch_flash_decode_fp16_graph(Q, K_cache_fp16, V_cache_fp16, O, partial_O, 
 
 def attn_decode_fused(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, partial_O, partial_lse, partial_max,
                       rope_table, n_heads, n_kv_heads, head_dim, d_past_len, max_seq, scale, eps, add_one=False,
-                      kv_fp16=True, stream=None):
+                      kv_fp16=True, stream=None, rope_interleaved=False):
     """launch_fused_qknorm_rope_kvwrite_graph + launch_flash_decode(_fp16)_graph fused (one launch + a small merge launch)
     (CUDAOps.h:653-673; issued back to back at gguf_model.h:2785-2832)."""
     check(_L().ptm_attn_decode_fused(_ptr(Q), _ptr(K), _ptr(V), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(K_cache),
                                     _ptr(V_cache), _ptr(O), _ptr(partial_O), _ptr(partial_lse), _ptr(partial_max),
                                     _ptr(rope_table), n_heads, n_kv_heads, head_dim, _ptr(d_past_len),
-                                    max_seq, scale, eps, int(add_one), int(kv_fp16), _stream(stream)),
+                                    max_seq, scale, eps, int(add_one), int(kv_fp16), int(rope_interleaved), _stream(stream)),
           "attn_decode_fused")
 
 
@@ -308,11 +308,12 @@ def embedding_rows(table_f32, table_q6k, q6k_row_stride_bytes, d_tokens, rows, h
 
 
 def qknorm_rope_kvwrite_rows(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, rope, rows, n_heads, n_kv_heads, head_dim,
-                             pos0, max_seq, eps, add_one, kv_fp16, stream=None):
+                             pos0, max_seq, eps, add_one, kv_fp16, stream=None, rope_interleaved=False):
     """launch_fused_qknorm_rope_kvwrite (CUDAOps.h:563-570) over `rows` prompt rows at positions pos0 + r."""
     check(_L().ptm_qknorm_rope_kvwrite_rows(_ptr(Q), _ptr(K), _ptr(V), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(K_cache),
                                             _ptr(V_cache), _ptr(rope), rows, n_heads, n_kv_heads, head_dim, pos0, max_seq,
-                                            eps, int(add_one), int(kv_fp16), _stream(stream)), "qknorm_rope_kvwrite_rows")
+                                            eps, int(add_one), int(kv_fp16), int(rope_interleaved), _stream(stream)),
+          "qknorm_rope_kvwrite_rows")
 
 
 def prefill_attention(Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, head_dim, pos0, max_seq, scale, kv_fp16,

@@ -171,6 +171,20 @@ def make_kv_prefill(seed: int, layer: int, cfg: dict, n_pos: int):
     return k, v
 
 
+def tiny_llama(seed: int):
+    """The TINY shapes as a llama-style model: no per-head QK-norm, interleaved rotation pairs.  The attention-input
+    norm weights are a tenth of TINY's: with random weights and no QK-norm the Q.K scores would otherwise run to the
+    hundreds, softmax would pick one position outright and neither the rotation nor the cache would matter."""
+    cfg = dict(TINY)
+    cfg["rope_interleaved"] = True
+    layers = [make_layer(seed, i, cfg) for i in range(cfg["n_layers"])]
+    for L in layers:
+        L["q_norm"] = None
+        L["k_norm"] = None
+        L["attn_norm"] = (np.float32(0.1) * L["attn_norm"]).astype(np.float32)
+    return cfg, layers, make_head(seed, cfg)
+
+
 # ---- sampling cases: (vocab, logit kind, temperature, top_k, top_p), in the order the golden run draws them ----
 SAMPLING_CASES = (
     [(1000, "normal", 0.8, 40, 0.9), (1000, "normal", 1.0, 0, 1.0), (1000, "normal", 0.7, 1, 1.0),

@@ -82,6 +82,7 @@ def main():
     ap.add_argument("--full", action="store_true")
     ap.add_argument("--sampling-only", action="store_true", help="write golden_sampling.npz and nothing else")
     ap.add_argument("--tokenizer-only", action="store_true", help="write golden_tokenizer.json and nothing else")
+    ap.add_argument("--llama-only", action="store_true", help="write golden_llama.npz and nothing else")
     args = ap.parse_args()
     assert po.have_ref(), "build oracle/_ref first: make -C oracle ref"
     if args.sampling_only:
@@ -91,6 +92,10 @@ def main():
     if args.tokenizer_only:
         make_tokenizer_golden()
         print("wrote golden_tokenizer.json")
+        return
+    if args.llama_only:
+        make_llama_golden()
+        print("wrote golden_llama.npz")
         return
     R = po.ref()
     meta = {"made_with": "oracle/_ref/libptm_ref.so (g++ -O2 -std=c++17 -mavx2 -mfma; see oracle/Makefile)",
@@ -214,6 +219,7 @@ def main():
     np.savez_compressed(os.path.join(OUT, "golden_small.npz"), **g)
     make_sampling()
     make_tokenizer_golden()
+    make_llama_golden()
 
     if args.full:
         make_full(meta)
@@ -298,6 +304,32 @@ def make_tokenizer_golden():
     os.environ.pop("PT_NO_THINK", None)
     with open(os.path.join(OUT, "golden_tokenizer.json"), "w") as f:
         json.dump(out, f, indent=0, sort_keys=True)
+
+
+def make_llama_golden():
+    """The reference's forward_decode_cpu on a llama-style tiny model (synth.tiny_llama): no QK-norm, interleaved
+    rotation pairs; 12 greedy steps after a 19-position cache, plus the rotation alone."""
+    R = po.ref()
+    cfg, layers, head = synth.tiny_llama(SEEDS["tiny"])
+    emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    rm = po.RefModel(cfg, layers, head, 64, emb)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(SEEDS["tiny"], i, cfg, 19)
+        rm.set_kv(i, k, v)
+    tok, toks, lg = 3, [], []
+    for _ in range(12):
+        tok = rm.step(tok)
+        toks.append(tok)
+        lg.append(rm.logits.copy())
+    rm.close()
+    g = {"tokens": np.array(toks, np.int64), "logits": np.stack(lg)}
+    r = synth.rng_for(SEEDS["blocks"], 77)
+    q = (3 * r.standard_normal(32 * 128, dtype=np.float32)).astype(np.float32)
+    k = (3 * r.standard_normal(8 * 128, dtype=np.float32)).astype(np.float32)
+    c, s = po.rope_tables(2049, 128, 5.0e5)
+    R.ref_rope_apply_norm(q.ctypes.data, k.ctypes.data, c.ctypes.data, s.ctypes.data, 32, 8, 128)
+    g["rope_norm_q"], g["rope_norm_k"] = q, k
+    np.savez_compressed(os.path.join(OUT, "golden_llama.npz"), **g)
 
 
 def make_full(meta):

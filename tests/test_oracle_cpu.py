@@ -205,3 +205,33 @@ def test_tiny_decode_bit_exact_vs_reference(po, golden, seeds):
         tok = om.step(tok)
         assert tok == int(golden["tiny_tokens"][st])
         assert np.array_equal(bits(om.logits), bits(golden["tiny_logits"][st])), st
+
+
+def test_llama_style_decode_and_rope_match_the_reference(po, seeds):
+    """No QK-norm + interleaved rotation pairs (llama / mistral): oracle bit-identical to the compiled reference's
+    forward_decode_cpu and rope_apply_fused (golden_llama.npz), and the rotation against float64."""
+    import os
+    from prometorch_amd import synth
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_llama.npz"))
+    cfg, layers, head = synth.tiny_llama(seeds["tiny"])
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(seeds["tiny"], i, cfg, 19)
+        om.set_kv(i, k, v)
+    tok = 3
+    for st in range(12):
+        tok = om.step(tok)
+        assert tok == int(g["tokens"][st])
+        assert np.array_equal(om.logits.view(np.uint32), g["logits"][st].view(np.uint32)), st
+    r = synth.rng_for(seeds["blocks"], 77)
+    q = (3 * r.standard_normal(32 * 128, dtype=np.float32)).astype(np.float32)
+    k = (3 * r.standard_normal(8 * 128, dtype=np.float32)).astype(np.float32)
+    c, s = po.rope_tables(2049, 128, 5.0e5)
+    qr, kr = po.rope_norm(q, k, c, s, 32, 8, 128)
+    assert np.array_equal(qr.view(np.uint32), g["rope_norm_q"].view(np.uint32))
+    assert np.array_equal(kr.view(np.uint32), g["rope_norm_k"].view(np.uint32))
+    # float64: pairs (2d, 2d+1) rotate by theta_d = pos * base^(-2d/hd)
+    th = 2049.0 * 5.0e5 ** (-np.arange(64) / 64.0)
+    q64 = q.astype(np.float64).reshape(32, 64, 2)
+    want = np.stack([q64[..., 0] * np.cos(th) - q64[..., 1] * np.sin(th), q64[..., 0] * np.sin(th) + q64[..., 1] * np.cos(th)], -1)
+    assert np.abs(qr.reshape(32, 64, 2) - want).max() <= 2e-3 * np.abs(want).max()   # fp32 angles of ~2e3 rad
