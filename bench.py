@@ -236,6 +236,21 @@ def main():
     gemv["copy_256MiB"] = {"bytes_read": ca.numel() * 4, "bytes_written": ca.numel() * 4, "us": msc * 1e3,
                            "GBs": 2 * ca.numel() * 4 / msc / 1e6}
     del ca, cb
+    # pure streaming reads of the GEMV footprints (cold: 36 distinct spans of a 1 GB buffer; the lm_head once per launch):
+    # the ceiling that launches of this size can reach on this part, beside the nominal 8 TB/s
+    span = 2 * I * stride4
+    pool = torch.empty(36 * span, dtype=torch.uint8, device="cuda")
+    parts = torch.empty(ops.stream_read_partials(V * stride6), dtype=torch.int32, device="cuda")
+    ceil = {}
+    for name, nb in (("14MB_one_q4k_matrix", I * stride4), ("28MB_gate_up", span)):
+        msr = event_time_ms(lambda i: ops.stream_read_xor(pool[(i % 36) * span:], nb, parts), 360, torch)
+        ceil[name] = {"bytes": nb, "us": msr * 1e3, "GBs": nb / msr / 1e6}
+    msr = event_time_ms(lambda i: ops.stream_read_xor(lm, V * stride6, parts), 40, torch)
+    ceil["319MB_lm_head"] = {"bytes": V * stride6, "us": msr * 1e3, "GBs": V * stride6 / msr / 1e6}
+    gemv["stream_read_ceiling"] = ceil
+    roof["frac_of_stream_read"] = roof["achieved"] / ceil["28MB_gate_up"]["GBs"]
+    log("stream-read ceiling: " + ", ".join("%s %.2f us" % (k, v["us"]) for k, v in ceil.items()))
+    del pool, parts
     # prompt prefill through all layers: 512 tokens from an empty context (row-batched GEMMs + causal attention)
     prompt = [int(t) for t in synth.rng_for(SEED, 9).integers(0, V, 512)]
     layer_params = H * (2 * cfg["n_heads"] * cfg["head_dim"] + 2 * cfg["n_kv_heads"] * cfg["head_dim"] + 3 * I)
@@ -292,6 +307,7 @@ def main():
 def cpu_baseline(cfg, layers, head, kvs, n_tokens, gpu_tokens, warmup):
     """Time the reference CPU decode path on this host for n_tokens tokens of the same workload."""
     from oracle import pyoracle as po
+    from prometorch_amd import synth
     kind = "port"
     model = None
     if po.have_ref():
@@ -315,8 +331,21 @@ def cpu_baseline(cfg, layers, head, kvs, n_tokens, gpu_tokens, warmup):
     log("cpu baseline (%s, %d threads): %.2f tok/s" % (kind, cores, n_tokens / dt))
     if hasattr(model, "close"):
         model.close()
+    # the same host on configs[0]: one Q4_K GEMV 9728x2560 through the reference's dispatcher (or the port's), cycling
+    # the 36 layers' gate matrices (504 MB, beyond the host caches)
+    gemv = po.ref_gemv if kind == "reference" else po.gemv
+    xg = synth.make_x(synth.rng_for(SEED, 11), cfg["hidden"])
+    gemv(12, layers[0]["gate"][1], xg)
+    t = time.perf_counter()
+    n_gemv = 3 * len(layers)
+    for i in range(n_gemv):
+        gemv(12, layers[i % len(layers)]["gate"][1], xg)
+    dtg = (time.perf_counter() - t) / n_gemv
+    wbytes = layers[0]["gate"][1].size + 4 * cfg["hidden"] + 4 * cfg["inter"]
+    log("cpu baseline GEMV 9728x2560: %.1f us, %.1f GB/s" % (dtg * 1e6, wbytes / dtg / 1e9))
     return {"value": n_tokens / dt, "unit": "tok/s", "cores": int(cores), "kind": kind,
-            "sample": "%d greedy tokens of the same 36-layer model after 1 warm-up token, KV prefilled to %d (fp32 KV on the CPU)" % (n_tokens, N_PREFILL)}
+            "sample": "%d greedy tokens of the same 36-layer model after 1 warm-up token, KV prefilled to %d (fp32 KV on the CPU)" % (n_tokens, N_PREFILL),
+            "cfg0_q4k_gemv_9728x2560": {"us": dtg * 1e6, "GBs": wbytes / dtg / 1e9, "launches": n_gemv}}
 
 
 if __name__ == "__main__":

@@ -219,6 +219,12 @@ int ptm_mt19937_uniforms(uint32_t seed, int64_t skip, int64_t n, float* out_host
 int ptm_add(const float* a, const float* b, float* out, int64_t n, ptm_stream_t stream);
 int ptm_copy(const float* in, float* out, int64_t n, ptm_stream_t stream);
 
+/* Measurement aid with no counterpart in the reference: a pure streaming read of `bytes` (a multiple of 16, 16-byte
+ * aligned) with 16-byte loads.  out_partials[i], i < ptm_stream_read_partials(bytes), receives the XOR of all 32-bit
+ * words of the i-th 32 KiB span.  Its time is the ceiling for a kernel that streams weights of that footprint. */
+int64_t ptm_stream_read_partials(int64_t bytes);
+int ptm_stream_read_xor(const void* src, int64_t bytes, uint32_t* out_partials, ptm_stream_t stream);
+
 /* ---- prefill: quantised-weight GEMM, Y[M,N] = X[M,K] . W[N,K]^T ------------------ */
 /* The reference has no quantised GEMM: matmul_q loops M single-row GEMVs
  * (gguf_model.h:7029-7036, :7056-7061).  These read each weight tile once per 64 rows of X and
