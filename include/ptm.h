@@ -41,7 +41,7 @@ enum {
     PTM_E_NOT_FOUND = -10   /* no tensor / metadata key of that name */
 };
 
-enum { PTM_TYPE_Q4_K = 12, PTM_TYPE_Q6_K = 14 }; /* ggml type ids, gguf_dequant.h:29-58 */
+enum { PTM_TYPE_Q5_0 = 6, PTM_TYPE_Q8_0 = 8, PTM_TYPE_Q4_K = 12, PTM_TYPE_Q5_K = 13, PTM_TYPE_Q6_K = 14 }; /* ggml type ids, gguf_dequant.h:29-58 */
 
 const char* ptm_strerror(int code);
 int ptm_last_hip_error(void);
@@ -89,10 +89,26 @@ int ptm_q6k_gemv_argmax(const void* W, const float* x, float* logits, int K, int
                         int64_t row_stride_bytes, int64_t* out_index, void* workspace,
                         ptm_stream_t stream);
 /* Type dispatcher mirroring cpu_quant_gemv (cpu_quant_gemv.h:1635-1688) and gemv_scratch
- * (gguf_model.h:3117-3140): 12 -> Q4_K, 14 -> Q6_K; anything else returns PTM_E_UNSUPPORTED
- * and launches nothing (the reference silently no-ops). */
+ * (gguf_model.h:3117-3140): 12 -> Q4_K, 14 -> Q6_K, 13 -> Q5_K, 8 -> Q8_0, 6 -> Q5_0; anything else returns
+ * PTM_E_UNSUPPORTED and launches nothing (the reference silently no-ops).  ptm_quant_gemv_supported mirrors
+ * cpu_quant_gemv_supported (cpu_quant_gemv.h:1691-1694). */
 int ptm_quant_gemv(uint32_t ggml_type, const void* W, const float* x, float* y, int K, int N,
                    int64_t row_stride_bytes, int accumulate, ptm_stream_t stream);
+int ptm_quant_gemv_supported(uint32_t ggml_type);
+
+/* The dispatcher's other formats, fp32 activations, y (+)= W.x (q8_0_gemv_avx2 cpu_quant_gemv.h:784-826, q5k_gemv_avx2
+ * :1091-1185, q5_0_gemv_scalar :1572-1630).  K a multiple of 32 (Q8_0: 34-byte blocks; Q5_0: 22-byte blocks; W and the
+ * row stride 2-byte aligned) or of 256 (Q5_K: 176-byte super-blocks, 4-byte aligned); x 16-byte aligned.  No file of
+ * the decode path's models holds these types: the kernels are plain row-per-wave ones, not tuned. */
+int ptm_q8_0_gemv(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes, int accumulate,
+                  ptm_stream_t stream);
+int ptm_q5k_gemv(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes, int accumulate,
+                 ptm_stream_t stream);
+int ptm_q5_0_gemv(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes, int accumulate,
+                  ptm_stream_t stream);
+/* dequantize_q8_0 / dequantize_q5_k (gguf_dequant.h:237-255, :348-388), bit-exact. */
+int ptm_dequant_q8_0(const void* blocks, float* out, int64_t n_elems, ptm_stream_t stream);
+int ptm_dequant_q5k(const void* blocks, float* out, int64_t n_elems, ptm_stream_t stream);
 
 /* Two / three Q4_K projections of the same x in one launch.
  * Replace launch_q4km_fused_gate_up_gemv (CUDAOps.h:453-458) and

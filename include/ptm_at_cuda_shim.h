@@ -33,6 +33,8 @@ inline void launch_quantize_q8_1(const float* x, void* y_q8, int K, cudaStream_t
 inline void launch_q4km_q8_gemv(const void* w, const void* x_q8, float* y, int K, int N, int64_t stride, cudaStream_t s = nullptr) { (void)ptm_q4k_gemv_q8(w, x_q8, y, K, N, stride, 0, s); }
 /* CUDAOps.h:498-501 */
 inline void launch_q6k_gemv(const void* w, const float* x, float* y, int K, int N, int64_t stride, cudaStream_t s = nullptr) { (void)ptm_q6k_gemv(w, x, y, K, N, stride, 0, s); }
+/* CUDAOps.h:503-507 */
+inline void launch_q5k_gemv(const void* w, const float* x, float* y, int K, int N, int64_t stride, cudaStream_t s = nullptr) { (void)ptm_q5k_gemv(w, x, y, K, N, stride, 0, s); }
 /* CUDAOps.h:453-458 */
 inline void launch_q4km_fused_gate_up_gemv(const void* wg, const void* wu, const float* x, float* yg, float* yu, int K, int Ng, int Nu, int64_t stride, cudaStream_t s = nullptr) { (void)ptm_q4k_fused_gate_up_gemv(wg, wu, x, yg, yu, K, Ng, Nu, stride, s); }
 /* CUDAOps.h:578-583 */

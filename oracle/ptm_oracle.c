@@ -286,10 +286,124 @@ void po_q6k_gemv_f32(const void* W, const float* x, float* y, int64_t K, int64_t
     free(row);
 }
 
+/* ---- the dispatcher's other block formats: Q8_0 (34 B / 32 values), Q5_K (176 B / 256), Q5_0 (22 B / 32) ----------
+ * fp32 activations in all three.  The 8-lane sums are written lane by lane: lane i of the reference's vector
+ * accumulator sees elements i, i+8, ... of each run of 32, and the lanes meet in the order of its hsum_avx. */
+static inline float hsum8_lanes(const float* a) { /* ((a0+a4)+(a1+a5)) + ((a2+a6)+(a3+a7)) */
+    const float s0 = a[0] + a[4], s1 = a[1] + a[5], s2 = a[2] + a[6], s3 = a[3] + a[7];
+    return (s0 + s1) + (s2 + s3);
+}
+
+/* reference: gguf_dequant.h:237-255 */
+void po_dequantize_q8_0(const void* src, float* dst, int64_t n) {
+    const uint8_t* p = (const uint8_t*)src;
+    for (int64_t b = 0; b < n / 32; ++b, p += 34, dst += 32) {
+        const float d = ld_f16(p);
+        const int8_t* q = (const int8_t*)(p + 2);
+        for (int j = 0; j < 32; ++j) dst[j] = d * (float)q[j];
+    }
+}
+
+/* the 5-bit quant e (0..255) of a Q5_K block: nibble from qs, fifth bit from qh */
+static inline int q5k_quant(const uint8_t* p, int e) {
+    const int pair = e >> 6, hi = (e >> 5) & 1, l = e & 31;
+    const uint8_t b = p[48 + 32 * pair + l];
+    const int nib = hi ? (b >> 4) : (b & 0xf);
+    return nib + (((p[16 + l] >> (2 * pair + hi)) & 1) ? 16 : 0);
+}
+
+/* reference: gguf_dequant.h:348-388 */
+void po_dequantize_q5_k(const void* src, float* dst, int64_t n) {
+    const uint8_t* p = (const uint8_t*)src;
+    for (int64_t b = 0; b < n / 256; ++b, p += 176, dst += 256) {
+        const float d = ld_f16(p), dmin = ld_f16(p + 2);
+        for (int sb = 0; sb < 8; ++sb) {
+            uint8_t sc, m;
+            po_get_scale_min_k4(sb, p + 4, &sc, &m);
+            const float ds = d * (float)sc, ms = dmin * (float)m;
+            for (int l = 0; l < 32; ++l) dst[32 * sb + l] = ds * (float)q5k_quant(p, 32 * sb + l) - ms;
+        }
+    }
+}
+
+/* reference: cpu_quant_gemv.h:784-826 (acc += (d*q) * x per lane, fused) */
+void po_q8_0_gemv(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride) {
+    const uint8_t* base = (const uint8_t*)W;
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; ++n) {
+        const uint8_t* p = base + n * stride;
+        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int64_t b = 0; b < K / 32; ++b, p += 34) {
+            const float d = ld_f16(p);
+            const int8_t* q = (const int8_t*)(p + 2);
+            for (int l = 0; l < 32; l += 8)
+                for (int i = 0; i < 8; ++i) acc[i] = fmaf(d * (float)q[l + i], x[32 * b + l + i], acc[i]);
+        }
+        y[n] = hsum8_lanes(acc);
+    }
+}
+
+/* reference: cpu_quant_gemv.h:1091-1185.  Per 32-wide sub-block the lanes first gather sum(q*x) and sum(x), then
+ * acc += d_sb * sum(q*x); acc -= m_sb * sum(x), low-nibble sub-block before the high-nibble one of each pair. */
+void po_q5k_gemv(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride) {
+    const uint8_t* base = (const uint8_t*)W;
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; ++n) {
+        const uint8_t* p = base + n * stride;
+        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int64_t b = 0; b < K / 256; ++b, p += 176) {
+            const float d = ld_f16(p), dmin = ld_f16(p + 2);
+            for (int sb = 0; sb < 8; ++sb) {
+                uint8_t sc, m;
+                po_get_scale_min_k4(sb, p + 4, &sc, &m);
+                const float ds = d * (float)sc, ms = dmin * (float)m;
+                const float* xx = x + 256 * b + 32 * sb;
+                float qx[8] = {0, 0, 0, 0, 0, 0, 0, 0}, sx[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                for (int l = 0; l < 32; l += 8)
+                    for (int i = 0; i < 8; ++i) {
+                        qx[i] = fmaf((float)q5k_quant(p, 32 * sb + l + i), xx[l + i], qx[i]);
+                        sx[i] = sx[i] + xx[l + i];
+                    }
+                for (int i = 0; i < 8; ++i) {
+                    acc[i] = fmaf(ds, qx[i], acc[i]);
+                    acc[i] = fmaf(-ms, sx[i], acc[i]);
+                }
+            }
+        }
+        y[n] = hsum8_lanes(acc);
+    }
+}
+
+/* reference: cpu_quant_gemv.h:1572-1630: one running sum per row, elements j and j+16 of a block alternating;
+ * d*q is exact in fp32 (11-bit by 5-bit), and the reference build (g++ -O2 -mfma, contraction on) fuses the
+ * multiply by x with the add */
+void po_q5_0_gemv(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride) {
+    const uint8_t* base = (const uint8_t*)W;
+    for (int64_t n = 0; n < N; ++n) {
+        const uint8_t* p = base + n * stride;
+        float acc = 0.0f;
+        for (int64_t b = 0; b < K / 32; ++b, p += 22) {
+            const float d = ld_f16(p);
+            uint32_t qh;
+            memcpy(&qh, p + 2, 4);
+            for (int j = 0; j < 16; ++j) {
+                const int q0 = ((p[6 + j] & 0xf) | (((qh >> j) & 1) << 4)) - 16;
+                const int q1 = ((p[6 + j] >> 4) | (((qh >> (j + 16)) & 1) << 4)) - 16;
+                acc = fmaf(d * (float)q0, x[32 * b + j], acc);
+                acc = fmaf(d * (float)q1, x[32 * b + j + 16], acc);
+            }
+        }
+        y[n] = acc;
+    }
+}
+
 void po_cpu_quant_gemv(uint32_t type, const void* W, const float* x, float* y,
                        int64_t K, int64_t N, int64_t stride) {
     if (type == PO_Q4_K) po_q4k_gemv(W, x, y, K, N, stride);
     else if (type == PO_Q6_K) po_q6k_gemv(W, x, y, K, N, stride);
+    else if (type == PO_Q8_0) po_q8_0_gemv(W, x, y, K, N, stride);
+    else if (type == PO_Q5_K) po_q5k_gemv(W, x, y, K, N, stride);
+    else if (type == PO_Q5_0) po_q5_0_gemv(W, x, y, K, N, stride);
     /* any other type: no-op, as reference cpu_quant_gemv.h:1684-1686 */
 }
 

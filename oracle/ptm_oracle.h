@@ -14,6 +14,9 @@
  *   po_quantize_x_q8       golden vectors from the compiled reference (bit-exact) + numpy rint invariants
  *   po_q4k_gemv            golden y from the compiled reference (bit-exact) + exact int dots vs numpy
  *   po_q6k_gemv            golden y from the compiled reference (bit-exact) + float64 dot of dequant
+ *   po_q8_0_gemv, po_q5k_gemv, po_q5_0_gemv, po_dequantize_q8_0, po_dequantize_q5_k
+ *                          golden y / values from the compiled reference's dispatcher and dequantisers
+ *                          (golden_formats.npz, bit-exact) + closed-form numpy dequantisation and its float64 dot
  *   po_rmsnorm_*           compiled reference + float64 numpy
  *   po_rope_*              compiled reference + float64 closed form (NeoX and interleaved pairing)
  *   po_exp256              compiled reference + float64 exp
@@ -39,13 +42,18 @@
 extern "C" {
 #endif
 
-enum { PO_Q4_K = 12, PO_Q6_K = 14 };
+enum { PO_Q5_0 = 6, PO_Q8_0 = 8, PO_Q4_K = 12, PO_Q5_K = 13, PO_Q6_K = 14 };
 
 float po_fp16_to_fp32(uint16_t h);
 uint16_t po_fp32_to_fp16(float f); /* round-to-nearest-even, IEEE */
 void po_get_scale_min_k4(int j, const uint8_t* q, uint8_t* sc, uint8_t* m);
 void po_dequantize_q4_k(const void* src, float* dst, int64_t n);
 void po_dequantize_q6_k(const void* src, float* dst, int64_t n);
+void po_dequantize_q8_0(const void* src, float* dst, int64_t n);   /* gguf_dequant.h:237 */
+void po_dequantize_q5_k(const void* src, float* dst, int64_t n);   /* gguf_dequant.h:348 */
+void po_q8_0_gemv(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride); /* cpu_quant_gemv.h:784 */
+void po_q5k_gemv(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride);  /* cpu_quant_gemv.h:1091 */
+void po_q5_0_gemv(const void* W, const float* x, float* y, int64_t K, int64_t N, int64_t stride); /* cpu_quant_gemv.h:1572 */
 
 /* Q8 activation blocks, flat: d[K/32], sum[K/32], qs[K] */
 void po_quantize_x_q8(const float* x, int64_t K, float* d, float* sum, int8_t* qs);

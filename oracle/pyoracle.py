@@ -63,8 +63,8 @@ def lib():
         for name in ("po_q4k_gemv", "po_q4k_gemv_f32", "po_q6k_gemv", "po_q6k_gemv_f32"):
             getattr(L, name).argtypes = [_vp, _vp, _vp, _i64, _i64, _i64]
         L.po_cpu_quant_gemv.argtypes = [_u32, _vp, _vp, _vp, _i64, _i64, _i64]
-        L.po_dequantize_q4_k.argtypes = [_vp, _vp, _i64]
-        L.po_dequantize_q6_k.argtypes = [_vp, _vp, _i64]
+        for name in ("po_dequantize_q4_k", "po_dequantize_q6_k", "po_dequantize_q8_0", "po_dequantize_q5_k"):
+            getattr(L, name).argtypes = [_vp, _vp, _i64]
         L.po_quantize_x_q8.argtypes = [_vp, _i64, _vp, _vp, _vp]
         L.po_q4k_row_isums.argtypes = [_vp, _vp, _i64, _vp]
         L.po_rmsnorm_seq.argtypes = [_vp, _vp, _f32, _i32, _i64, _vp]
@@ -94,12 +94,29 @@ def fp16_to_fp32(h: int) -> float:
     return lib().po_fp16_to_fp32(h)
 
 
+# ggml type id -> (bytes per block, values per block): gguf_dequant.h:29-58
+BLOCK = {12: (144, 256), 14: (210, 256), 13: (176, 256), 8: (34, 32), 6: (22, 32)}
+_DEQUANT = {12: "dequantize_q4_k", 14: "dequantize_q6_k", 8: "dequantize_q8_0", 13: "dequantize_q5_k"}
+
+
 def dequant(qtype: int, raw: np.ndarray) -> np.ndarray:
     raw = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1)
-    bb = 144 if qtype == 12 else 210
-    n = raw.size // bb * 256
+    bb, per = BLOCK[qtype]
+    n = raw.size // bb * per
     out = np.empty(n, dtype=np.float32)
-    (lib().po_dequantize_q4_k if qtype == 12 else lib().po_dequantize_q6_k)(_p(raw), _p(out), n)
+    getattr(lib(), "po_" + _DEQUANT[qtype])(_p(raw), _p(out), n)
+    return out
+
+
+def ref_dequant(qtype: int, raw: np.ndarray) -> np.ndarray:
+    """The compiled reference's dequantiser (only where oracle/_ref is built)."""
+    raw = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1)
+    bb, per = BLOCK[qtype]
+    n = raw.size // bb * per
+    out = np.empty(n, dtype=np.float32)
+    fn = getattr(ref(), "ref_" + _DEQUANT[qtype])
+    fn.argtypes = [_vp, _vp, _i64]
+    fn(_p(raw), _p(out), n)
     return out
 
 
@@ -118,9 +135,9 @@ def gemv(qtype: int, W: np.ndarray, x: np.ndarray, variant: str = "ref") -> np.n
     fp32 for Q6_K); 'f32': exact-math fp32-activation cross-check."""
     W = np.ascontiguousarray(W, dtype=np.uint8)
     N, stride = W.shape
-    K = stride // (144 if qtype == 12 else 210) * 256
+    K = x.size if qtype not in (12, 14) else stride // BLOCK[qtype][0] * 256
     x = np.ascontiguousarray(x, dtype=np.float32)
-    assert x.size == K
+    assert x.size == K and stride >= K // BLOCK[qtype][1] * BLOCK[qtype][0]
     y = np.empty(N, np.float32)
     if variant == "ref":
         lib().po_cpu_quant_gemv(qtype, _p(W), _p(x), _p(y), K, N, stride)
@@ -363,8 +380,8 @@ def ref():
 def ref_gemv(qtype, W, x):
     W = np.ascontiguousarray(W, np.uint8)
     N, stride = W.shape
-    K = stride // (144 if qtype == 12 else 210) * 256
     x = np.ascontiguousarray(x, np.float32)
+    K = x.size
     y = np.empty(N, np.float32)
     ref().ref_cpu_quant_gemv(qtype, _p(W), _p(x), _p(y), K, N, stride)
     return y

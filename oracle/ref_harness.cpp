@@ -29,6 +29,9 @@ void ref_get_scale_min_k4(int j, const uint8_t* s, uint8_t* d, uint8_t* m) { g::
 void ref_dequantize_q4_k(const void* src, float* dst, int64_t n) { g::dequantize_q4_k(src, dst, n); }
 // torch/io/gguf_dequant.h:395
 void ref_dequantize_q6_k(const void* src, float* dst, int64_t n) { g::dequantize_q6_k(src, dst, n); }
+// torch/io/gguf_dequant.h:237, :348
+void ref_dequantize_q8_0(const void* src, float* dst, int64_t n) { g::dequantize_q8_0(src, dst, n); }
+void ref_dequantize_q5_k(const void* src, float* dst, int64_t n) { g::dequantize_q5_k(src, dst, n); }
 
 // torch/io/cpu_quant_gemv.h:147 — the Q8Block struct is alignas(32) (64 B); unpack to flat arrays.
 void ref_quantize_x_q8(const float* x, int64_t K, float* d_out, float* sum_out, int8_t* qs_out) {

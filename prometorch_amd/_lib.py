@@ -52,6 +52,12 @@ SIGNATURES = {
     "ptm_device_cus": (i32, []),
     "ptm_dequant_q4k": (i32, [vp, vp, i64, vp]),
     "ptm_dequant_q6k": (i32, [vp, vp, i64, vp]),
+    "ptm_dequant_q8_0": (i32, [vp, vp, i64, vp]),
+    "ptm_dequant_q5k": (i32, [vp, vp, i64, vp]),
+    "ptm_q8_0_gemv": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
+    "ptm_q5k_gemv": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
+    "ptm_q5_0_gemv": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
+    "ptm_quant_gemv_supported": (i32, [u32]),
     "ptm_dequant_q4k_to_fp16": (i32, [vp, vp, i32, i32, i64, vp]),
     "ptm_q8_bytes": (i64, [i32]),
     "ptm_quantize_q8": (i32, [vp, vp, i32, vp]),

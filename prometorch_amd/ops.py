@@ -49,6 +49,16 @@ def dequant_q6k(blocks, out, n_elems, stream=None):
     check(_L().ptm_dequant_q6k(_ptr(blocks), _ptr(out), n_elems, _stream(stream)), "dequant_q6k")
 
 
+def dequant_q8_0(blocks, out, n_elems, stream=None):
+    """dequantize_q8_0 (gguf_dequant.h:237-255)"""
+    check(_L().ptm_dequant_q8_0(_ptr(blocks), _ptr(out), n_elems, _stream(stream)), "dequant_q8_0")
+
+
+def dequant_q5k(blocks, out, n_elems, stream=None):
+    """dequantize_q5_k (gguf_dequant.h:348-388)"""
+    check(_L().ptm_dequant_q5k(_ptr(blocks), _ptr(out), n_elems, _stream(stream)), "dequant_q5k")
+
+
 def launch_dequant_q4k_to_fp16(weights, out_fp16, K, N, row_stride_bytes, stream=None):
     """CUDAOps.h:477-480"""
     check(_L().ptm_dequant_q4k_to_fp16(_ptr(weights), _ptr(out_fp16), K, N, row_stride_bytes, _stream(stream)),
@@ -107,6 +117,11 @@ def quant_gemv(quant_type, weights, x, y, K, N, row_stride_bytes, stream=None, a
     """cpu_quant_gemv / gemv_scratch dispatch (cpu_quant_gemv.h:1635-1688, gguf_model.h:3117-3140)."""
     check(_L().ptm_quant_gemv(quant_type, _ptr(weights), _ptr(x), _ptr(y), K, N, row_stride_bytes, int(accumulate),
                              _stream(stream)), "quant_gemv")
+
+
+def quant_gemv_supported(quant_type) -> bool:
+    """cpu_quant_gemv_supported (cpu_quant_gemv.h:1691-1694)"""
+    return bool(_L().ptm_quant_gemv_supported(quant_type))
 
 
 def launch_q4km_fused_gate_up_gemv(w_gate, w_up, x, y_gate, y_up, K, N_gate, N_up, row_stride_bytes, stream=None):

@@ -59,8 +59,44 @@ def make_q6k(rng: np.random.Generator, rows: int, cols: int, d_scale: float = 0.
     return blk.reshape(rows, cols // 256 * 210)
 
 
+def make_q5k(rng: np.random.Generator, rows: int, cols: int, d_scale: float = 0.01) -> np.ndarray:
+    """[rows, cols/256*176] uint8 of Q5_K super-blocks: d, dmin, 6-bit scales/mins as Q4_K, 32 bytes of fifth bits,
+    128 bytes of nibbles, all uniform."""
+    nb = rows * (cols // 256)
+    blk = np.empty((nb, 176), dtype=np.uint8)
+    dd = (np.abs(rng.standard_normal((nb, 2), dtype=np.float32)) * np.float32(d_scale)).astype(np.float16)
+    blk[:, 0:4] = dd.view(np.uint8).reshape(nb, 4)
+    sm = rng.integers(0, 64, size=(nb, 16), dtype=np.uint8)
+    blk[:, 4:16] = pack_scales_k4(sm[:, :8], sm[:, 8:])
+    blk[:, 16:176] = rng.integers(0, 256, size=(nb, 160), dtype=np.uint8)
+    return blk.reshape(rows, cols // 256 * 176)
+
+
+def make_q8_0(rng: np.random.Generator, rows: int, cols: int, d_scale: float = 0.002) -> np.ndarray:
+    """[rows, cols/32*34] uint8 of Q8_0 blocks: d = fp16(|N(0,1)|*d_scale), 32 int8 quants uniform -127..127."""
+    nb = rows * (cols // 32)
+    blk = np.empty((nb, 34), dtype=np.uint8)
+    d = (np.abs(rng.standard_normal((nb, 1), dtype=np.float32)) * np.float32(d_scale)).astype(np.float16)
+    blk[:, 0:2] = d.view(np.uint8).reshape(nb, 2)
+    blk[:, 2:34] = rng.integers(-127, 128, size=(nb, 32), dtype=np.int8).view(np.uint8)
+    return blk.reshape(rows, cols // 32 * 34)
+
+
+def make_q5_0(rng: np.random.Generator, rows: int, cols: int, d_scale: float = 0.01) -> np.ndarray:
+    """[rows, cols/32*22] uint8 of Q5_0 blocks: d = fp16(|N(0,1)|*d_scale), 32 fifth bits, 16 bytes of nibbles."""
+    nb = rows * (cols // 32)
+    blk = np.empty((nb, 22), dtype=np.uint8)
+    d = (np.abs(rng.standard_normal((nb, 1), dtype=np.float32)) * np.float32(d_scale)).astype(np.float16)
+    blk[:, 0:2] = d.view(np.uint8).reshape(nb, 2)
+    blk[:, 2:22] = rng.integers(0, 256, size=(nb, 20), dtype=np.uint8)
+    return blk.reshape(rows, cols // 32 * 22)
+
+
+Q5_0, Q8_0, Q5_K = 6, 8, 13
+
+
 def make_weight(rng, qtype: int, rows: int, cols: int) -> np.ndarray:
-    return make_q4k(rng, rows, cols) if qtype == Q4_K else make_q6k(rng, rows, cols)
+    return {Q4_K: make_q4k, Q6_K: make_q6k, Q5_K: make_q5k, Q8_0: make_q8_0, Q5_0: make_q5_0}[qtype](rng, rows, cols)
 
 
 def make_x(rng: np.random.Generator, n: int) -> np.ndarray:

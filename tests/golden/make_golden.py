@@ -83,6 +83,7 @@ def main():
     ap.add_argument("--sampling-only", action="store_true", help="write golden_sampling.npz and nothing else")
     ap.add_argument("--tokenizer-only", action="store_true", help="write golden_tokenizer.json and nothing else")
     ap.add_argument("--llama-only", action="store_true", help="write golden_llama.npz and nothing else")
+    ap.add_argument("--formats-only", action="store_true", help="write golden_formats.npz and nothing else")
     args = ap.parse_args()
     assert po.have_ref(), "build oracle/_ref first: make -C oracle ref"
     if args.sampling_only:
@@ -96,6 +97,10 @@ def main():
     if args.llama_only:
         make_llama_golden()
         print("wrote golden_llama.npz")
+        return
+    if args.formats_only:
+        make_formats_golden()
+        print("wrote golden_formats.npz")
         return
     R = po.ref()
     meta = {"made_with": "oracle/_ref/libptm_ref.so (g++ -O2 -std=c++17 -mavx2 -mfma; see oracle/Makefile)",
@@ -220,6 +225,7 @@ def main():
     make_sampling()
     make_tokenizer_golden()
     make_llama_golden()
+    make_formats_golden()
 
     if args.full:
         make_full(meta)
@@ -304,6 +310,23 @@ def make_tokenizer_golden():
     os.environ.pop("PT_NO_THINK", None)
     with open(os.path.join(OUT, "golden_tokenizer.json"), "w") as f:
         json.dump(out, f, indent=0, sort_keys=True)
+
+
+FORMAT_CASES = [(13, 24, 512), (13, 3, 2560), (8, 24, 512), (8, 5, 96), (6, 24, 512), (6, 7, 32)]  # (ggml type, N, K)
+
+
+def make_formats_golden():
+    """The reference's dispatcher on its other block formats (Q5_K, Q8_0, Q5_0: cpu_quant_gemv.h:1635-1688) and its
+    dequantisers of the first two, on seeded blocks (synth.make_weight / make_x from SEEDS['blocks'], type, N, K)."""
+    g = {}
+    for qt, N, K in FORMAT_CASES:
+        r = synth.rng_for(SEEDS["blocks"], qt, N, K)
+        W = synth.make_weight(r, qt, N, K)
+        x = synth.make_x(r, K)
+        g["y_%d_%d_%d" % (qt, N, K)] = po.ref_gemv(qt, W, x)
+        if qt != 6:
+            g["dq_%d_%d_%d" % (qt, N, K)] = po.ref_dequant(qt, W)
+    np.savez_compressed(os.path.join(OUT, "golden_formats.npz"), **g)
 
 
 def make_llama_golden():

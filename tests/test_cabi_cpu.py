@@ -65,7 +65,13 @@ def test_host_side_validation_codes():
     assert L.ptm_q4k_gemv(16, 16, 16, 65536, 4, 144 * 256, 0, None) == E_UNSUP
     assert L.ptm_q6k_gemv(16, 16, 16, 256, 4, 209, 0, None) == E_SHAPE
     assert L.ptm_q6k_gemv(17, 16, 16, 256, 4, 210, 0, None) == E_ALIGN
-    assert L.ptm_quant_gemv(13, 16, 16, 16, 256, 4, 176, 0, None) == E_UNSUP  # Q5_K: not on this path
+    assert L.ptm_quant_gemv(10, 16, 16, 16, 256, 4, 84, 0, None) == E_UNSUP   # Q2_K: not in the reference's dispatcher either
+    assert L.ptm_quant_gemv(13, 16, 16, 16, 250, 4, 176, 0, None) == E_SHAPE  # Q5_K: K not a multiple of 256
+    assert L.ptm_quant_gemv(13, 18, 16, 16, 256, 4, 176, 0, None) == E_ALIGN  # Q5_K blocks are read as dwords
+    assert L.ptm_quant_gemv(8, 16, 16, 16, 48, 4, 68, 0, None) == E_SHAPE     # Q8_0: K not a multiple of 32
+    assert L.ptm_quant_gemv(8, 17, 16, 16, 64, 4, 68, 0, None) == E_ALIGN
+    assert L.ptm_quant_gemv(6, 16, 16, 16, 64, 4, 43, 0, None) == E_SHAPE     # Q5_0: stride below two 22-byte blocks
+    assert [t for t in range(32) if L.ptm_quant_gemv_supported(t)] == [6, 8, 12, 13, 14]  # cpu_quant_gemv.h:1691-1694
     assert L.ptm_flash_decode(16, 16, 16, 16, 16, 16, 16, 32, 8, 96, 16, 128, 1.0, 1, None) == E_UNSUP
     assert L.ptm_flash_decode(16, 16, 16, 16, 16, 16, 16, 30, 8, 128, 16, 128, 1.0, 1, None) == E_SHAPE
     assert L.ptm_dequant_q4k(16, 16, 100, None) == E_SHAPE
