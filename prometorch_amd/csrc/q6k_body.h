@@ -148,23 +148,24 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
 #endif
     __syncthreads();
 
+    // Passes roll: as soon as a block of pass p has been consumed its registers are refilled with the same slot of
+    // pass p + 1, so a lane group keeps NB - 1 .. NB blocks in flight while it computes; the last pass only consumes.
     float acc = 0.0f;
-#pragma unroll
-    for (int u = 0; u < NB; ++u) {
-        const int b = sub + (u << a.log2S);
-        const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
-        acc += b < nblk ? t : 0.0f;
-    }
-    for (int i0 = NB; i0 < nb_max; i0 += NB) {
-#pragma unroll
-        for (int u = 0; u < NB; ++u)
-            blk[u] = q6k_load(row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 210, j, qh_off, sc_off);
+    int i0 = 0;
+    for (; i0 + NB < nb_max; i0 += NB) {
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
             const int b = sub + ((i0 + u) << a.log2S);
             const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
             acc += b < nblk ? t : 0.0f;
+            blk[u] = q6k_load(row + (int64_t)min(sub + ((i0 + NB + u) << a.log2S), nblk - 1) * 210, j, qh_off, sc_off);
         }
+    }
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        const int b = sub + ((i0 + u) << a.log2S);
+        const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
+        acc += b < nblk ? t : 0.0f;
     }
     float p = sum8(acc);
     if (S >= 2) p += dpp_f<0x128>(p);
@@ -196,6 +197,10 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
     }
 }
 
+// Lane groups per row: the fewest that still give the chip enough workgroups, with a group's blocks in at most two
+// rolling passes (the vocabulary projection 151936 x 2560 then runs one group per row, two passes of 5 blocks:
+// 94 -> 88 us with the argmax against two groups per row and one pass, for half the stagings of x).
+// PTM_Q6K_LOG2S (0..3) forces the split and PTM_Q6K_TWO_PASS=0 restores the one-pass rule, for tuning runs.
 inline int q6k_pick_log2S(int rows, int nblk) {
     static const int forced = [] {
         const char* e = getenv("PTM_Q6K_LOG2S");
@@ -207,7 +212,8 @@ inline int q6k_pick_log2S(int rows, int nblk) {
         const int S = 1 << l;
         const int wgs = (rows * S + 31) / 32;
         const int nb = (nblk + S - 1) / S;
-        if (nb <= Q6K_U && wgs >= 600) break;
+        static const int passes = [] { const char* e = getenv("PTM_Q6K_TWO_PASS"); return (e && e[0] == '0') ? 1 : 2; }();
+        if (nb <= passes * Q6K_U && wgs >= 600) break;
         if (nb <= 1) break;
         ++l;
     }
