@@ -199,7 +199,6 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
     __shared__ float s_p[SAMPLER_MAX_CAND];                   // x, then p, in index order
     __shared__ uint32_t s_idx[SAMPLER_MAX_CAND];
     __shared__ uint8_t s_keep[SAMPLER_MAX_CAND];
-    __shared__ int s_token;
     const int tid = threadIdx.x;
     // every load whose address is known goes out first, in one round trip; the draw follows as soon as the step is known
     const ptm_sampling p = sampler_params(a);
@@ -358,7 +357,6 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
                 }
             }
         }
-        s_token = token;
         if (o.out_token) *o.out_token = token;
         if (o.counts_rw && token >= 0) o.counts_rw[token] += 1;
         if (o.adv.d_step) {

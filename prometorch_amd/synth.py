@@ -173,13 +173,13 @@ def layer_shapes(cfg: dict) -> dict:
 NORM_SCALE = {"attn": 0.1, "ffn": 1.0e-3, "qk": 1.0, "out": 1.0}
 
 
-def make_layer(seed: int, layer: int, cfg: dict, norm_scale: dict | None = None) -> dict:
+def make_layer(seed: int, layer: int, cfg: dict, norm_scale: dict | None = None, mats=None) -> dict:
     """One decoder layer's seven weight matrices plus its four norm vectors
-    (gamma = scale * (1 + 0.1*N(0,1)), scale per NORM_SCALE)."""
+    (gamma = scale * (1 + 0.1*N(0,1)), scale per NORM_SCALE).  mats: (name, quant type) pairs, LAYER_MATS by default."""
     ns = dict(NORM_SCALE if norm_scale is None else norm_scale)
     shp = layer_shapes(cfg)
     out = {}
-    for i, (name, qt) in enumerate(LAYER_MATS):
+    for i, (name, qt) in enumerate(LAYER_MATS if mats is None else mats):
         out[name] = (qt, make_weight(rng_for(seed, 1, layer, i), qt, *shp[name]))
     g = rng_for(seed, 2, layer)
     for name, n, sc in (("attn_norm", cfg["hidden"], ns["attn"]), ("ffn_norm", cfg["hidden"], ns["ffn"]),
@@ -205,6 +205,23 @@ def make_kv_prefill(seed: int, layer: int, cfg: dict, n_pos: int):
     k = g.standard_normal((n_pos, kvd), dtype=np.float32).astype(np.float16)
     v = g.standard_normal((n_pos, kvd), dtype=np.float32).astype(np.float16)
     return k, v
+
+
+# Type mixes a Q4_K_M file really holds besides LAYER_MATS (about half of its layers keep attn_v and ffn_down in
+# Q4_K), and one it does not, to reach the remaining branches of the step (a Q6_K q beside Q4_K k and v, Q6_K o and gate)
+MIX_ALL_Q4K = tuple((n, Q4_K) for n, _ in LAYER_MATS)
+MIX_ODD = (("q", Q6_K), ("k", Q4_K), ("v", Q4_K), ("o", Q6_K), ("gate", Q6_K), ("up", Q4_K), ("down", Q6_K))
+
+
+MIXED_FEED = tuple((131 * i + 3) % 1024 for i in range(32))  # tokens fed to tiny_mixed step by step
+
+
+def tiny_mixed(seed: int):
+    """The TINY shapes with three layers of different type mixes: LAYER_MATS, MIX_ALL_Q4K, MIX_ODD."""
+    cfg = dict(TINY)
+    cfg["n_layers"] = 3
+    layers = [make_layer(seed, i, cfg, mats=m) for i, m in enumerate((LAYER_MATS, MIX_ALL_Q4K, MIX_ODD))]
+    return cfg, layers, make_head(seed, cfg)
 
 
 def tiny_llama(seed: int):

@@ -83,6 +83,7 @@ def main():
     ap.add_argument("--sampling-only", action="store_true", help="write golden_sampling.npz and nothing else")
     ap.add_argument("--tokenizer-only", action="store_true", help="write golden_tokenizer.json and nothing else")
     ap.add_argument("--llama-only", action="store_true", help="write golden_llama.npz and nothing else")
+    ap.add_argument("--mixed-only", action="store_true", help="write golden_mixed.npz and nothing else")
     ap.add_argument("--formats-only", action="store_true", help="write golden_formats.npz and nothing else")
     args = ap.parse_args()
     assert po.have_ref(), "build oracle/_ref first: make -C oracle ref"
@@ -97,6 +98,10 @@ def main():
     if args.llama_only:
         make_llama_golden()
         print("wrote golden_llama.npz")
+        return
+    if args.mixed_only:
+        make_mixed_golden()
+        print("wrote golden_mixed.npz")
         return
     if args.formats_only:
         make_formats_golden()
@@ -226,6 +231,7 @@ def main():
     make_tokenizer_golden()
     make_llama_golden()
     make_formats_golden()
+    make_mixed_golden()
 
     if args.full:
         make_full(meta)
@@ -327,6 +333,23 @@ def make_formats_golden():
         if qt != 6:
             g["dq_%d_%d_%d" % (qt, N, K)] = po.ref_dequant(qt, W)
     np.savez_compressed(os.path.join(OUT, "golden_formats.npz"), **g)
+
+
+def make_mixed_golden():
+    """The reference's forward_decode_cpu on synth.tiny_mixed: layers whose q/k/v share a type (fused QKV, 8-lane
+    norm, gguf_model.h:3342-3350) beside layers where they do not, Q4_K and Q6_K in every projection role."""
+    cfg, layers, head = synth.tiny_mixed(SEEDS["tiny"])
+    emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    rm = po.RefModel(cfg, layers, head, 64, emb)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(SEEDS["tiny"], i, cfg, 19)
+        rm.set_kv(i, k, v)
+    toks, lg = [], []
+    for st in range(12):   # fed tokens are fixed (synth.MIXED_FEED): the greedy loop of this model settles on one token
+        toks.append(rm.step(synth.MIXED_FEED[st]))
+        lg.append(rm.logits.copy())
+    rm.close()
+    np.savez_compressed(os.path.join(OUT, "golden_mixed.npz"), tokens=np.array(toks, np.int64), logits=np.stack(lg))
 
 
 def make_llama_golden():

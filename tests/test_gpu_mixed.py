@@ -1,0 +1,112 @@
+"""GPU: layers of different quant-type mixes in one model (synth.tiny_mixed) -- the Q4_K_M mix, an all-Q4_K layer
+(about half the layers of a real Q4_K_M file keep attn_v and ffn_down in Q4_K) and an odd mix that reaches the
+remaining branches of the step (Q6_K q beside Q4_K k/v, Q6_K o and gate) -- against the compiled reference's golden
+run, the oracle, the prompt path and a .gguf round trip.  Bars as in test_gpu_decode / test_gpu_prefill."""
+import os
+
+import numpy as np
+import pytest
+
+from conftest import GOLDEN_DIR, bits
+from prometorch_amd import gguf, synth
+from test_gpu_decode import LOGIT_TOL, LOGIT_TOL_FLIP, check_step_errors
+from test_gpu_prefill import check_kv_rows, check_logits, follow
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def golden_mixed():
+    return np.load(os.path.join(GOLDEN_DIR, "golden_mixed.npz"))
+
+
+def mixed_with_cache(seeds, n=19):
+    cfg, layers, head = synth.tiny_mixed(seeds["tiny"])
+    return cfg, layers, head, [synth.make_kv_prefill(seeds["tiny"], i, cfg, n) for i in range(cfg["n_layers"])]
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_mixed_decode_fp32_kv_vs_reference_golden(dev, golden_mixed, seeds, use_graph):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = mixed_with_cache(seeds)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False, use_graph=use_graph)
+    for i, (k, v) in enumerate(kv):
+        dec.set_kv(i, k, v)
+    dec.set_past_len(19)
+    errs = []
+    for st in range(12):
+        tok = dec.step(synth.MIXED_FEED[st])
+        ref = golden_mixed["logits"][st]
+        errs.append(np.abs(dec.logits() - ref).max() / ref.std())
+        assert tok == int(golden_mixed["tokens"][st]), st
+    check_step_errors(errs)
+    dec.close()
+
+
+def test_mixed_decode_fp16_kv_vs_oracle(dev, po, seeds):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = mixed_with_cache(seeds)
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=True)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=True)
+    for i, (k, v) in enumerate(kv):
+        om.set_kv(i, k, v)
+        dec.set_kv(i, k, v)
+    dec.set_past_len(19)
+    errs = []
+    for st in range(24):
+        tok_o = om.step(synth.MIXED_FEED[st])
+        tok_g = dec.step(synth.MIXED_FEED[st])
+        errs.append(np.abs(dec.logits() - om.logits).max() / om.logits.std())
+        assert tok_g == tok_o, st
+    # The all-Q4_K layer rounds the inputs of all seven projections to int8 where the Q4_K_M mix rounds five, and
+    # the model is a layer deeper: steps in which one activation lands on the other side of a rounding boundary
+    # (see test_gpu_decode) are more frequent here (3 of 24 measured, up to 1.4e-2), so the count of such steps is
+    # not bounded, only their size, and the typical step must hold the tight bar
+    errs = np.asarray(errs)
+    assert errs.max() <= LOGIT_TOL_FLIP and np.median(errs) <= LOGIT_TOL, errs
+    dec.close()
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+@pytest.mark.parametrize("pos0,n,chunk", [(0, 23, 0), (19, 12, 5)])
+def test_mixed_prefill_vs_oracle_token_by_token(dev, po, seeds, kv_fp16, pos0, n, chunk):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = synth.tiny_mixed(seeds["tiny"])
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=kv_fp16)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=kv_fp16, use_graph=True)
+    if pos0:
+        for i in range(cfg["n_layers"]):
+            k, v = synth.make_kv_prefill(seeds["tiny"], i, cfg, pos0)
+            om.set_kv(i, k, v)
+            dec.set_kv(i, k, v)
+        dec.set_past_len(pos0)
+    prompt = [int(t) for t in synth.rng_for(68, pos0, n).integers(0, cfg["vocab"], n)]
+    for t in prompt:
+        tok_o = om.step(t)
+    tok_g = dec.prefill(prompt, chunk_rows=chunk)
+    for li in range(cfg["n_layers"]):
+        for nm, gpu_c, cpu_c in (("k", dec.k_cache[li], om.k_cache[li]), ("v", dec.v_cache[li], om.v_cache[li])):
+            check_kv_rows(gpu_c[pos0:pos0 + n].float().cpu().numpy(), cpu_c[pos0:pos0 + n], li, nm)
+    check_logits(dec.logits(), om.logits, tok_g, tok_o, "prefill")
+    follow(dec, om, tok_o, 6)
+    dec.close()
+
+
+def test_mixed_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_mixed, tmp_path):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = mixed_with_cache(seeds)
+    path = str(tmp_path / "tiny_mixed.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head)
+    m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
+    d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
+    for i, (k, v) in enumerate(kv):
+        m.set_kv(i, k, v)
+        d.set_kv(i, k, v)
+    m.set_past_len(19)
+    d.set_past_len(19)
+    for st in range(12):
+        tm, td = m.step(synth.MIXED_FEED[st]), d.step(synth.MIXED_FEED[st])
+        assert tm == td == int(golden_mixed["tokens"][st]), st
+        assert np.array_equal(bits(m.logits()), bits(d.logits())), st
+    m.close()
+    d.close()

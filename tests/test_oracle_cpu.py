@@ -235,3 +235,19 @@ def test_llama_style_decode_and_rope_match_the_reference(po, seeds):
     q64 = q.astype(np.float64).reshape(32, 64, 2)
     want = np.stack([q64[..., 0] * np.cos(th) - q64[..., 1] * np.sin(th), q64[..., 0] * np.sin(th) + q64[..., 1] * np.cos(th)], -1)
     assert np.abs(qr.reshape(32, 64, 2) - want).max() <= 2e-3 * np.abs(want).max()   # fp32 angles of ~2e3 rad
+
+
+def test_mixed_type_layers_match_the_reference(po, seeds):
+    """Layers whose q/k/v share a type (the reference fuses them behind its 8-lane norm) beside layers where they do
+    not, Q4_K and Q6_K in every projection role (synth.tiny_mixed): oracle bit-identical to the compiled reference's
+    forward_decode_cpu (golden_mixed.npz)."""
+    import os
+    from prometorch_amd import synth
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_mixed.npz"))
+    cfg, layers, head = synth.tiny_mixed(seeds["tiny"])
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)
+    for i in range(cfg["n_layers"]):
+        om.set_kv(i, *synth.make_kv_prefill(seeds["tiny"], i, cfg, 19))
+    for st in range(12):
+        assert om.step(synth.MIXED_FEED[st]) == int(g["tokens"][st]), st
+        assert np.array_equal(bits(om.logits), bits(g["logits"][st])), st
