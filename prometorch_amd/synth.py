@@ -224,6 +224,23 @@ def tiny_mixed(seed: int):
     return cfg, layers, make_head(seed, cfg)
 
 
+LLAMA3_8B = dict(vocab=128256, hidden=4096, n_layers=32, n_heads=32, n_kv_heads=8, head_dim=128,
+                 inter=14336, rope_base=5.0e5, eps=1.0e-5, rope_interleaved=True)
+
+
+def llama3_8b_like(seed: int, n_layers: int = 2, vocab: int = 32000):
+    """Llama-3-8B layer shapes (no QK-norm, interleaved rotation), a few layers and a reduced vocabulary so that the
+    CPU oracle can step it; attention-input norm gains reduced as in tiny_llama."""
+    cfg = dict(LLAMA3_8B)
+    cfg["n_layers"], cfg["vocab"] = n_layers, vocab
+    layers = [make_layer(seed, i, cfg) for i in range(n_layers)]
+    for L in layers:
+        L["q_norm"] = None
+        L["k_norm"] = None
+        L["attn_norm"] = (np.float32(0.1) * L["attn_norm"]).astype(np.float32)
+    return cfg, layers, make_head(seed, cfg)
+
+
 def tiny_llama(seed: int):
     """The TINY shapes as a llama-style model: no per-head QK-norm, interleaved rotation pairs.  The attention-input
     norm weights are a tenth of TINY's: with random weights and no QK-norm the Q.K scores would otherwise run to the

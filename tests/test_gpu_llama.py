@@ -270,3 +270,61 @@ def test_llama_sensitive_step_is_the_oracles_own(po, seeds):
     print("oracle vs perturbed oracle, 6 steps after the prompt: rms", np.round(errs[:, 1], 4), flush=True)
     assert errs[2, 1] > E2E_RMS_TOL and errs[2, 0] > E2E_MAX_TOL
     assert np.median(errs[:, 1]) <= E2E_RMS_TOL and np.median(errs[:, 0]) <= E2E_MAX_TOL
+
+
+def test_llama3_8b_layer_shapes_decode_and_prefill_vs_oracle(dev, po, seeds):
+    """Two layers of Llama-3-8B size (4096 hidden, 14336 intermediate, 32/8 heads of 128, base 5e5, eps 1e-5) over
+    a 32000-token vocabulary: 12 decode steps at positions 300.. and a 40-token prompt against the oracle.
+    After the prompt the two sides hold cache rows that differ by the fp16 GEMM's error, and single steps of this
+    random model amplify such differences to the size of the logits themselves (its attention without QK-norm is
+    close to a hard maximum).  The yardstick for those steps is therefore the oracle against ITSELF with its input
+    embedding perturbed by 5e-4 relative, stepped beside the other two: the GPU must stay within twice that."""
+    from prometorch_amd.decode import Decoder
+    from test_gpu_decode import LOGIT_TOL, LOGIT_TOL_FLIP
+    cfg, layers, head = synth.llama3_8b_like(seeds["cfg4"])
+    table = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    noise = synth.rng_for(71).standard_normal(table.shape, dtype=np.float32)
+    om = po.OracleModel(cfg, layers, head, 512, kv_fp16=True, embedding=table)
+    ob = po.OracleModel(cfg, layers, head, 512, kv_fp16=True, embedding=table * (1 + np.float32(5e-4) * noise))
+    dec = Decoder(cfg, layers, head, max_seq=512, kv_fp16=True, use_graph=True)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(seeds["cfg4"], i, cfg, 300)
+        om.set_kv(i, k, v)
+        ob.set_kv(i, k, v)
+        dec.set_kv(i, k, v)
+    dec.set_past_len(300)
+    tok, errs = 11, []
+    for st in range(12):
+        tok_o = om.step(tok)
+        ob.step(tok)
+        tok_g = dec.step(tok)
+        err, rms, margin = logit_errors(dec.logits(), om.logits)
+        errs.append(err)
+        if margin > 2 * err:
+            assert tok_g == tok_o, (st, margin, err)
+        tok = tok_o
+    errs = np.asarray(errs)
+    print("decode steps: logit err/std", np.array2string(errs, precision=2), flush=True)
+    assert errs.max() <= LOGIT_TOL_FLIP and np.median(errs) <= LOGIT_TOL, errs
+    # a 40-token prompt behind those 312 positions, then 6 more steps on the rows the prefill wrote
+    prompt = [int(t) for t in synth.rng_for(69).integers(0, cfg["vocab"], 40)]
+    for t in prompt:
+        tok_o = om.step(t)
+        ob.step(t)
+    tok_g = dec.prefill(prompt)
+    check_kv_rows(dec.k_cache[0][312:352].float().cpu().numpy(), om.k_cache[0][312:352], 0, "k")
+    check_kv_rows(dec.v_cache[0][312:352].float().cpu().numpy(), om.v_cache[0][312:352], 0, "v")
+    check_logits(dec.logits(), om.logits, tok_g, tok_o, "prefill")
+    tok = tok_o
+    for st in range(6):
+        tok_o = om.step(tok)
+        ob.step(tok)
+        tok_g = dec.step(tok)
+        err, rms, margin = logit_errors(dec.logits(), om.logits)
+        perr, prms, _ = logit_errors(ob.logits, om.logits)
+        print("  after the prompt, step %d: GPU err %.3f rms %.4f; perturbed oracle err %.3f rms %.4f" % (st, err, rms, perr, prms), flush=True)
+        assert err <= max(E2E_MAX_TOL, 2 * perr) and rms <= max(E2E_RMS_TOL, 2 * prms), (st, err, rms, perr, prms)
+        if margin > 2 * err:
+            assert tok_g == tok_o, (st, margin, err)
+        tok = tok_o
+    dec.close()
