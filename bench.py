@@ -77,6 +77,8 @@ def main():
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--llama-steps", type=int, default=64,
+                    help="decode steps of the Llama-3-8B-shaped extra measurement (0 = skip)")
     ap.add_argument("--layers", type=int, default=36, help=argparse.SUPPRESS)  # debugging only; 36 is the workload
     args = ap.parse_args()
     if args.gpus != 1:
@@ -279,6 +281,36 @@ def main():
     del dec
     torch.cuda.empty_cache()
 
+    # ---- a second model family on the same decoder: Llama-3-8B-shaped Q4_K_M (no QK-norm, interleaved rotation) -----
+    llama = None
+    if args.llama_steps > 0:
+        t0 = time.perf_counter()
+        lcfg = dict(synth.LLAMA3_8B)
+        _, llayers, lhead = synth.llama3_8b_like(SEED + 1, n_layers=lcfg["n_layers"], vocab=lcfg["vocab"])
+        ldec = Decoder(lcfg, llayers, lhead, max_seq=MAX_SEQ, kv_fp16=True, use_graph=True)
+        for i in range(lcfg["n_layers"]):
+            ldec.set_kv(i, *synth.make_kv_prefill(SEED + 1, i, lcfg, N_PREFILL))
+        ldec.set_past_len(N_PREFILL)
+        ltok = 1
+        for _ in range(args.warmup):
+            ltok = ldec.step(ltok)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.llama_steps):
+            ltok = ldec.step(ltok)
+        torch.cuda.synchronize()
+        ldt = time.perf_counter() - t1
+        llama = {"workload": "batch-1 greedy decode, Llama-3-8B-shaped Q4_K_M (32 layers, 4096 hidden, 14336 intermediate, "
+                             "128256 vocabulary), fp16 KV prefilled %d, %d new tokens, host-synchronous" % (N_PREFILL, args.llama_steps),
+                 "tok_s": args.llama_steps / ldt, "ms_per_token": ldt / args.llama_steps * 1e3,
+                 "token_hbm_frac": (32 * 138_903_552 + 128256 * 3360 + 32 * 2 * (N_PREFILL + args.warmup + args.llama_steps / 2) * 1024 * 2)
+                                   / (ldt / args.llama_steps) / 1e9 / HBM_PEAK_GBS,
+                 "a100_published_deepseek_r1_8b_tok_s": 51.1}
+        log("llama-3-8B shape: %.1f tok/s (%.3f ms/token), set up in %.1fs" % (llama["tok_s"], llama["ms_per_token"], t1 - t0))
+        ldec.close()
+        del ldec, llayers, lhead
+        torch.cuda.empty_cache()
+
     # ---- CPU baseline on this host: bounded sample of the same workload ---------------------------
     cpu = None
     if args.cpu_tokens > 0:
@@ -296,6 +328,7 @@ def main():
         "roofline": roof, "cpu_baseline": cpu, "gemv": gemv,
         "chained_tok_s": chained_tok_s, "chained_tokens_identical": bool(tokens_equal),
         "sampled_tok_s": sampled_tok_s, "sampled_chained_tok_s": sampled_chained_tok_s,
+        "llama3_8b_shape": llama,
         "a100_published_tok_s": 82.6, "x_a100_published": tok_s / 82.6,
         "token_hbm_frac": per_token_bytes / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
     }

@@ -13,6 +13,7 @@
 //   down-proj GEMV accumulating into the residual
 #include "ptm_common.h"
 
+#include <cstring>
 #include <new>
 #include <vector>
 
@@ -91,6 +92,8 @@ struct ptm_decoder {
     int64_t* d_next = nullptr;
     int64_t* d_tokens = nullptr;
     int64_t* h_pinned = nullptr;  // [max_seq] pinned host staging for token ids
+    float* h_uniforms = nullptr;  // [max_seq] pinned host staging for the sampler's draws (a copy from pageable memory
+                                  // goes through the runtime's own staging and can stall for hundreds of microseconds)
     int64_t past_len = 0;
     int status = PTM_OK;
     // prefill scratch for up to pf_rows prompt rows at a time (allocated on the first prefill)
@@ -351,6 +354,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
 
     if ((rc = hip_status(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     if ((rc = hip_status(hipHostMalloc((void**)&d->h_pinned, 8 * (size_t)c.max_seq, hipHostMallocDefault))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
+    if ((rc = hip_status(hipHostMalloc((void**)&d->h_uniforms, 4 * (size_t)c.max_seq, hipHostMallocDefault))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     {
         std::vector<float> tab((size_t)c.max_seq * c.head_dim);
         ptm_rope_table_host(tab.data(), c.max_seq, c.head_dim, c.rope_freq_base);
@@ -370,6 +374,7 @@ void ptm_decode_destroy(ptm_decoder* d) {
     if (d->exec_s) (void)hipGraphExecDestroy(d->exec_s);
     if (d->graph_s) (void)hipGraphDestroy(d->graph_s);
     if (d->h_pinned) (void)hipHostFree(d->h_pinned);
+    if (d->h_uniforms) (void)hipHostFree(d->h_uniforms);
     if (d->pf_slab) (void)hipFree(d->pf_slab);
     if (d->slab) (void)hipFree(d->slab);
     if (d->stream) (void)hipStreamDestroy(d->stream);
@@ -450,7 +455,8 @@ int ptm_decode_sample(ptm_decoder* d, int token_id, int n, const float* uniforms
     if (!d || !uniforms_host || !out_tokens) return PTM_E_NULL;
     if (!d->sampling_set) return PTM_E_STATE;
     if (n <= 0 || n > d->cfg.max_seq) return PTM_E_SHAPE;
-    int rc = hip_status(hipMemcpyAsync(d->d_uniforms, uniforms_host, 4 * (size_t)n, hipMemcpyHostToDevice, d->stream));
+    memcpy(d->h_uniforms, uniforms_host, 4 * (size_t)n);  // the previous call's copy has completed: every call ends synchronised
+    int rc = hip_status(hipMemcpyAsync(d->d_uniforms, d->h_uniforms, 4 * (size_t)n, hipMemcpyHostToDevice, d->stream));
     if (rc != PTM_OK) return rc;
     if ((rc = run_steps(d, token_id, n, true)) != PTM_OK) return rc;
     for (int i = 0; i < n; ++i) {

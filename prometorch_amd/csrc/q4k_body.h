@@ -244,26 +244,26 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
         issue_order_fence();
         between();
 
+        // passes roll: a consumed block's registers are refilled from the next pass at once, so a lane group keeps
+        // NB - 1 .. NB blocks in flight while it computes; the last pass only consumes
         float acc = 0.0f;
-#pragma unroll
-        for (int u = 0; u < NB; ++u) {
-            const int b = sub + (u << a.log2S);
-            const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
-            acc += b < nblk ? t : 0.0f;
-        }
-        for (int i0 = NB; i0 < nb_max; i0 += NB) {
-#pragma unroll
-            for (int u = 0; u < NB; ++u) {
-                const uint8_t* p = row + (int64_t)min(sub + ((i0 + u) << a.log2S), nblk - 1) * 144;
-                hdr[u] = *reinterpret_cast<const uint4*>(p);
-                qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
-            }
+        int i0 = 0;
+        for (; i0 + NB < nb_max; i0 += NB) {
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
                 const int b = sub + ((i0 + u) << a.log2S);
                 const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
                 acc += b < nblk ? t : 0.0f;
+                const uint8_t* p = row + (int64_t)min(sub + ((i0 + NB + u) << a.log2S), nblk - 1) * 144;
+                hdr[u] = *reinterpret_cast<const uint4*>(p);
+                qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
             }
+        }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int b = sub + ((i0 + u) << a.log2S);
+            const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
+            acc += b < nblk ? t : 0.0f;
         }
         // reduce: 8 lanes of the group, then the S groups of the row
         float p = sum8(acc);

@@ -24,23 +24,25 @@ __global__ __launch_bounds__(Q6K_THREADS) void q6k_gemv_kernel(const Q6KArgs a) 
     q6k_gemv_body<ACC, ARGMAX, NORM, XCH, NB>(a, lds_raw, blockIdx.x);
 }
 
-// Few rows, long rows (a down projection: 2560 x 9728): with 4 rows per workgroup every workgroup would stage the
-// whole activation vector for 4 rows' worth of weights, and the staging traffic through L2 would exceed the weights'.
-// Here a workgroup is `waves` rows (one wave per row, its 8 lane groups striding the row's super-blocks), sized so
-// that the launch is one workgroup per CU (or two): x is staged once per CU.  XL = float4 loads of x per thread.
+// Few rows, long rows (a down projection: 2560 x 9728, 4096 x 14336): with 4 rows per workgroup every workgroup
+// would stage the whole activation vector for 4 rows' worth of weights, and the staging traffic through L2 would
+// exceed the weights'.  Here a workgroup is `waves` waves of 8 >> LOG2S rows each (a row's super-blocks strided over
+// 1 << LOG2S lane groups), sized so that the launch is one workgroup per CU: x is staged once per CU.
+// XL = float4 loads of x per thread.
 enum { Q6K_TALL_MAX_WAVES = 12 };
-template <bool ACC, int NB, int XL>
+template <bool ACC, int NB, int XL, int LOG2S>
 __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(const Q6KArgs a) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
+    constexpr int S = 1 << LOG2S, ROWS_PER_WAVE = 8 >> LOG2S;
     float* xf = reinterpret_cast<float*>(lds_raw);
     float* xsum16 = xf + a.K;
     const int tid = threadIdx.x, nthr = blockDim.x;
-    const int lane = tid & 63, wave = tid >> 6, j = lane & 7, sub = lane >> 3;
-    const int r = blockIdx.x * (nthr >> 6) + wave;
+    const int lane = tid & 63, wave = tid >> 6, j = lane & 7, grp = lane >> 3, sub = grp & (S - 1);
+    const int r = (blockIdx.x * (nthr >> 6) + wave) * ROWS_PER_WAVE + (grp >> LOG2S);
     const bool live = r < a.N;
     const int rr = live ? r : a.N - 1;
     const int nblk = a.K / 256, n4 = a.K / 4;
-    const int nb_max = (nblk + 7) >> 3;
+    const int nb_max = (nblk + S - 1) >> LOG2S;
     const uint8_t* row = a.W + (int64_t)rr * a.stride;
     const int qh_off = 128 + 32 * (j >> 2) + 16 * (j & 1);
     const int sc_off = 192 + 8 * (j >> 2) + 2 * ((j & 3) >> 1) + (j & 1);
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(
     issue_order_fence();
     Q6Blk blk[NB];
 #pragma unroll
-    for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + 8 * u, nblk - 1) * 210, j, qh_off, sc_off);
+    for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + S * u, nblk - 1) * 210, j, qh_off, sc_off);
     issue_order_fence();
     // x and its per-16 sums to LDS: 4 consecutive lanes hold one group of 16 (n4 and nthr are multiples of 64, so
     // the range test is wave-uniform)
@@ -72,55 +74,74 @@ __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(
     }
     __syncthreads();
 
+    // rolling passes, as in q6k_gemv_body
     float acc = 0.0f;
+    int i0 = 0;
+    for (; i0 + NB < nb_max; i0 += NB) {
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int b = sub + S * (i0 + u);
+            const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
+            acc += b < nblk ? t : 0.0f;
+            blk[u] = q6k_load(row + (int64_t)min(sub + S * (i0 + NB + u), nblk - 1) * 210, j, qh_off, sc_off);
+        }
+    }
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-        const int b = sub + 8 * u;
+        const int b = sub + S * (i0 + u);
         const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
         acc += b < nblk ? t : 0.0f;
     }
-    for (int i0 = NB; i0 < nb_max; i0 += NB) {
-#pragma unroll
-        for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + 8 * (i0 + u), nblk - 1) * 210, j, qh_off, sc_off);
-#pragma unroll
-        for (int u = 0; u < NB; ++u) {
-            const int b = sub + 8 * (i0 + u);
-            const float t = q6k_block_term(blk[u], xf, xsum16, min(b, nblk - 1), j);
-            acc += b < nblk ? t : 0.0f;
-        }
-    }
-    // same reduction order as the S = 8 path of q6k_gemv_body
+    // same reduction order as q6k_gemv_body
     float p = sum8(acc);
     p += dpp_f<0x128>(p);
     p += __shfl_xor(p, 16, 64);
-    p += __shfl_xor(p, 32, 64);
-    if (live && lane == 0) {
+    if (S >= 8) p += __shfl_xor(p, 32, 64);
+    if (live && sub == 0 && j == 0) {
         if constexpr (ACC) a.y[rr] += p;
         else a.y[rr] = p;
     }
 }
 
-// waves per workgroup for the tall kernel, or 0 when the shape is not one for it: rows that fill the chip once at
-// one workgroup per CU (measured: 2560 x 9728 10.25 -> 9.75 us; at two workgroups per CU, 4096 x 14336, the 4-row
-// tiles are faster: 20.9 against 23.2 us).  PTM_Q6K_TALL=0 switches it off, for tuning runs.
-inline int q6k_tall_waves(int N, int K) {
+// Shape of a tall launch: waves per workgroup and lane groups per row, or waves = 0 when the shape is not one for
+// it.  Rows that fill the chip once at one workgroup per CU: 8 lane groups per row while that needs at most 12 waves
+// (2560 x 9728: 10 waves, 10.25 -> 9.75 us against 4-row tiles), else 4 groups per row and two rows per wave
+// (4096 x 14336: 8 waves of 2 rows).  PTM_Q6K_TALL=0 switches it off, for tuning runs.
+struct Q6KTall { int waves, log2S; };
+inline Q6KTall q6k_tall_shape(int N, int K) {
     static const bool off = [] { const char* e = getenv("PTM_Q6K_TALL"); return e && e[0] == '0'; }();
-    if (off || K < 4096 || K > 14336) return 0;
-    if (q6k_pick_log2S(N, K / 256) != 3) return 0;   // only where the row tiles would be 4 rows anyway
-    const int w = (N + 255) / 256;
-    const int waves = w < 2 ? 2 : w;
-    if (waves > Q6K_TALL_MAX_WAVES) return 0;
-    return K / 4 <= 8 * 64 * waves ? waves : 0;      // x in at most 8 loads per thread
+    if (off || K < 4096 || K > 14336) return {0, 0};
+    if (q6k_pick_log2S(N, K / 256) != 3) return {0, 0};   // only where the row tiles would be 4 rows anyway
+    const int rows_per_wg = (N + 255) / 256;
+    for (int l = 3; l >= 2; --l) {
+        const int rpw = 8 >> l;
+        int waves = (rows_per_wg + rpw - 1) / rpw;
+        if (waves < 2) waves = 2;
+        if (waves > Q6K_TALL_MAX_WAVES) continue;
+        if (K / 4 > 8 * 64 * waves) continue;            // x in at most 8 loads per thread
+        return {waves, l};
+    }
+    return {0, 0};
 }
 
-template <bool ACC, int NB>
+template <bool ACC, int NB, int LOG2S>
 static int q6k_launch_tall_nb(const Q6KArgs& a, int waves, hipStream_t s) {
-    const int grid = (a.N + waves - 1) / waves;
+    const int rows_per_wg = waves * (8 >> LOG2S);
+    const int grid = (a.N + rows_per_wg - 1) / rows_per_wg;
     const size_t lds = (size_t)a.K * 4 + (size_t)a.K / 4;
     const int xl = (a.K / 4 + 64 * waves - 1) / (64 * waves);
-    if (xl <= 4) hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 4>), dim3(grid), dim3(64 * waves), lds, s, a);
-    else hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8>), dim3(grid), dim3(64 * waves), lds, s, a);
+    if (xl <= 4) hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 4, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
+    else hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
     return launch_status();
+}
+template <bool ACC, int LOG2S>
+static int q6k_launch_tall(const Q6KArgs& a, int waves, hipStream_t s) {
+    // blocks in flight per lane group: as many as the registers allow rather than the tightest fit (a padded slot
+    // repeats a load that hits in L1; two blocks in flight leave the memory pipe idle)
+    const int nb = (a.K / 256 + (1 << LOG2S) - 1) >> LOG2S;
+    if (nb <= 2) return q6k_launch_tall_nb<ACC, 2, LOG2S>(a, waves, s);
+    if (nb == 3) return q6k_launch_tall_nb<ACC, 3, LOG2S>(a, waves, s);
+    return q6k_launch_tall_nb<ACC, 5, LOG2S>(a, waves, s);
 }
 
 // Final argmax over the per-workgroup (value, index) pairs: one workgroup of 1024 threads; every thread issues its
@@ -227,12 +248,9 @@ static int q6k_launch(Q6KArgs& a, hipStream_t s) {
     const int grid = q6k_workgroups(a.N, a.K);
     const size_t lds = (size_t)a.K * 4 + (size_t)a.K / 4;
     if constexpr (!ARGMAX && !NORM) {
-        if (const int waves = q6k_tall_waves(a.N, a.K)) {
-            const int nb = (a.K / 256 + 7) / 8;
-            if (nb <= 2) return q6k_launch_tall_nb<ACC, 2>(a, waves, s);
-            if (nb <= 3) return q6k_launch_tall_nb<ACC, 3>(a, waves, s);
-            return q6k_launch_tall_nb<ACC, 5>(a, waves, s);
-        }
+        const Q6KTall tall = q6k_tall_shape(a.N, a.K);
+        if (tall.waves > 0)
+            return tall.log2S == 3 ? q6k_launch_tall<ACC, 3>(a, tall.waves, s) : q6k_launch_tall<ACC, 2>(a, tall.waves, s);
         // long rows (down projection): all of x is requested before the weights
         if (a.K > 4096 && a.K <= 3 * 4096) return q6k_launch_xch<ACC, false, false, 3>(a, grid, lds, s);
     }

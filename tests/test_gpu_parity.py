@@ -538,7 +538,8 @@ def test_stream_read_xor_matches_numpy(dev, nbytes):
         ops.stream_read_xor(cu(data), nbytes + 8, out)
 
 
-@pytest.mark.parametrize("N,K,accumulate", [(2500, 9728, True), (300, 4096, False), (77, 14336, True), (3000, 6912, False)])
+@pytest.mark.parametrize("N,K,accumulate", [(2500, 9728, True), (300, 4096, False), (77, 14336, True), (3000, 6912, False),
+                                            (4096, 14336, True), (3300, 8192, False), (5119, 13824, False)])  # two rows per wave
 def test_q6k_long_rows_few_rows_vs_oracle(dev, po, N, K, accumulate):
     """Shapes served by the one-row-per-wave kernel (whole x staged once per workgroup): ragged row counts, both
     store modes, and a row stride wider than the row."""
