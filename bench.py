@@ -114,6 +114,12 @@ def main():
     torch.cuda.synchronize()
     log("uploaded in %.1fs" % (time.time() - t0))
 
+    # The host loops below are timed per token; a full collection of the interpreter's object graph (tens of
+    # milliseconds once torch is imported) landing inside one of them would be charged to that loop
+    import gc
+    gc.collect()
+    gc.disable()
+
     # ---- timed region: W warm-up tokens, then exactly K tokens, host-synchronous per token ----
     dec.set_past_len(N_PREFILL)
     tok = 1
@@ -159,6 +165,7 @@ def main():
     dec.sample(1, us)
     sampled_chained_tok_s = (args.warmup + args.steps) / (time.perf_counter() - t1)
     log("sampled (device top-k/top-p): %.1f tok/s per-token sync, %.1f tok/s chained" % (sampled_tok_s, sampled_chained_tok_s))
+    gc.enable()
 
     # ---- roofline of the dominant kernel, live, HIP events on the launching stream --------------
     H, I = cfg["hidden"], cfg["inter"]

@@ -92,8 +92,8 @@ struct ptm_decoder {
     int64_t* d_next = nullptr;
     int64_t* d_tokens = nullptr;
     int64_t* h_pinned = nullptr;  // [max_seq] pinned host staging for token ids
-    float* h_uniforms = nullptr;  // [max_seq] pinned host staging for the sampler's draws (a copy from pageable memory
-                                  // goes through the runtime's own staging and can stall for hundreds of microseconds)
+    float* h_uniforms = nullptr;  // [max_seq] pinned host staging for the sampler's draws (an "async" copy from the
+                                  // caller's pageable memory would be staged by the runtime synchronously)
     int64_t past_len = 0;
     int status = PTM_OK;
     // prefill scratch for up to pf_rows prompt rows at a time (allocated on the first prefill)
