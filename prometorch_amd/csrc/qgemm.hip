@@ -508,31 +508,39 @@ struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh
 // of the current block, followed by the next block's weights, and written to the other LDS buffer during steps
 // 3..6, so the block ends with the next tile complete behind the only workgroup barrier of the block.  (After the
 // last block the same code re-fetches the last tile into the idle buffer: no conditionals in the steady-state loop.)
-template <typename Tile, int MT>
-__global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
+// WAVES = 4: a wave owns 64 columns (two 32-column tiles) and all MT row tiles.  WAVES = 8 (MT = 4): waves w and w + 4
+// own one 32-column tile each of the same 64 columns, so a SIMD holds two waves and one's dequantisation and LDS reads
+// run under the other's MFMAs (the two pipes of a single wave barely overlap); no weight is dequantised twice, the X
+// tile in LDS is read by twice as many waves.
+template <typename Tile, int MT, int WAVES = 4>
+__global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
                                                         const float* __restrict__ rowscale, float* Y, int M, int K, int N,
                                                         int accumulate, int blocks_per_split, float* partials) {
     // W and Xh are deliberately not __restrict__: loads through a restrict pointer may be moved across the
     // compiler fences below, and the prefetch distance of this loop depends on those fences
     constexpr int TM = 32 * MT;                     // rows of X per workgroup (MT tiles of 32)
+    constexpr int NT = 2 / (WAVES / 4);             // 32-column tiles per wave
+    constexpr int RS = 2 * WAVES;                   // rows of the X tile that one fetch instruction of the workgroup covers
+    constexpr int NPIECE = TM / RS;                 // 16-byte pieces of the X tile per thread
+    static_assert(WAVES == 4 || (WAVES == 8 && MT == 4), "wave layouts");
     extern __shared__ __align__(16) uint8_t s_a[];  // [2][TM * QF_PITCH]
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3;
     const int j = lane & 31, kh = lane >> 5;
     const int m0 = blockIdx.y * TM;
-    const int n_base = blockIdx.x * QF_TN + wave * 64;
+    const int n_base = blockIdx.x * QF_TN + wave * 64 + (WAVES == 8 ? 32 * (tid >> 8) : 0);
     // split K: workgroup z of the grid sums super-blocks [blk0, blk0 + nblk) into its own M x N partial
     const int blk0 = blockIdx.z * blocks_per_split;
     const int nblk = min(K / 256 - blk0, blocks_per_split);
-    const uint8_t* wrow[2];
+    const uint8_t* wrow[NT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < NT; ++t)
         wrow[t] = W + (int64_t)min(n_base + 32 * t + j, N - 1) * stride + (int64_t)blk0 * Tile::kBlockBytes;
 
-    f32x16 acc[MT][2];
+    f32x16 acc[MT][NT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mt][t][r] = 0.0f;
 
@@ -547,14 +555,14 @@ __global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const
     uint4 x0, x1, x2, x3, x4, x5, x6, x7, x8, x9, x10, x11, x12, x13, x14, x15;
     // prologue: tile of block 0 -> LDS buffer 0, weights of block 0, fragments of step 0
 #pragma unroll
-    for (int p = 0; p < 4 * MT; ++p)
-        *reinterpret_cast<uint4*>(x_dst + 8 * p * QF_PITCH) = *reinterpret_cast<const uint4*>(x_src + 8 * p * x_row_bytes);
-    Tile cur[2], nxt[2];
+    for (int p = 0; p < NPIECE; ++p)
+        *reinterpret_cast<uint4*>(x_dst + RS * p * QF_PITCH) = *reinterpret_cast<const uint4*>(x_src + RS * p * x_row_bytes);
+    Tile cur[NT], nxt[NT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) cur[t].load(wrow[t], kh);
-    h8 bf[2][2], bn[2][2];
+    for (int t = 0; t < NT; ++t) cur[t].load(wrow[t], kh);
+    h8 bf[NT][2], bn[NT][2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) cur[t].frags(0, kh, bf[t][0], bf[t][1]);
+    for (int t = 0; t < NT; ++t) cur[t].frags(0, kh, bf[t][0], bf[t][1]);
     __syncthreads();
 
     for (int blk = 0; blk < nblk; ++blk) {
@@ -570,25 +578,25 @@ __global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const
                 af[ks][mt] = *reinterpret_cast<const h8*>(a_cur + (mt * 32 + j) * QF_PITCH + 32 * kh + 16 * ks);
 #pragma unroll
         for (int s = 0; s < 8; ++s) {  // unrolled: the sub-block index selects registers
-#define QF_LD(p) (*reinterpret_cast<const uint4*>(x_from + 8 * (p) * x_row_bytes))
-#define QF_ST(p, v) (*reinterpret_cast<uint4*>(x_nxt + 8 * (p) * QF_PITCH) = (v))
+#define QF_LD(p) (*reinterpret_cast<const uint4*>(x_from + RS * (p) * x_row_bytes))
+#define QF_ST(p, v) (*reinterpret_cast<uint4*>(x_nxt + RS * (p) * QF_PITCH) = (v))
             if (s == 0) {
                 // All fetches of the block are issued here, tile pieces FIRST: loads return in order, so a wait for a
                 // piece must not have the weight loads (HBM latency, one cache line per lane) in front of it.  The
                 // pieces are written to LDS in steps 3..6 with the weights still in flight; the weights are first
                 // needed at step 7.
                 x0 = QF_LD(0); x1 = QF_LD(1); x2 = QF_LD(2); x3 = QF_LD(3);
-                if constexpr (MT >= 2) { x4 = QF_LD(4); x5 = QF_LD(5); x6 = QF_LD(6); x7 = QF_LD(7); }
-                if constexpr (MT >= 4) {
+                if constexpr (NPIECE >= 8) { x4 = QF_LD(4); x5 = QF_LD(5); x6 = QF_LD(6); x7 = QF_LD(7); }
+                if constexpr (NPIECE >= 16) {
                     x8 = QF_LD(8); x9 = QF_LD(9); x10 = QF_LD(10); x11 = QF_LD(11); x12 = QF_LD(12);
                     x13 = QF_LD(13); x14 = QF_LD(14); x15 = QF_LD(15);
                 }
 #pragma unroll
-                for (int t = 0; t < 2; ++t) nxt[t].load(wrow[t] + (int64_t)nb * Tile::kBlockBytes, kh);
+                for (int t = 0; t < NT; ++t) nxt[t].load(wrow[t] + (int64_t)nb * Tile::kBlockBytes, kh);
             }
             if (s == 3) { QF_ST(0, x0); QF_ST(1, x1); QF_ST(2, x2); QF_ST(3, x3); }
-            if constexpr (MT >= 2) { if (s == 4) { QF_ST(4, x4); QF_ST(5, x5); QF_ST(6, x6); QF_ST(7, x7); } }
-            if constexpr (MT >= 4) {
+            if constexpr (NPIECE >= 8) { if (s == 4) { QF_ST(4, x4); QF_ST(5, x5); QF_ST(6, x6); QF_ST(7, x7); } }
+            if constexpr (NPIECE >= 16) {
                 if (s == 5) { QF_ST(8, x8); QF_ST(9, x9); QF_ST(10, x10); QF_ST(11, x11); }
                 if (s == 6) { QF_ST(12, x12); QF_ST(13, x13); QF_ST(14, x14); QF_ST(15, x15); }
             }
@@ -607,10 +615,10 @@ __global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const
             }
 #if defined(PTM_EXP) && PTM_EXP == 11
 #pragma unroll
-            for (int t = 0; t < 2; ++t) { bn[t][0] = bf[t][1]; bn[t][1] = bf[t][0]; }
+            for (int t = 0; t < NT; ++t) { bn[t][0] = bf[t][1]; bn[t][1] = bf[t][0]; }
 #else
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < NT; ++t) {
                 if (s < 7) cur[t].frags(s + 1, kh, bn[t][0], bn[t][1]);
                 else nxt[t].frags(0, kh, bn[t][0], bn[t][1]);
             }
@@ -620,7 +628,7 @@ __global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                    for (int t = 0; t < 2; ++t)
+                    for (int t = 0; t < NT; ++t)
 #if defined(PTM_EXP) && PTM_EXP == 12
                         acc[mt][t][0] += (float)af[ks][mt][0] * (float)bf[t][ks][0];
 #else
@@ -629,13 +637,13 @@ __global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const
             // issue order: one MFMA, then the vector work that fits under it (a 32x32x16 MFMA occupies the matrix pipe
             // for 32 cycles = 8 vector instructions), so that neither pipe waits for the other
 #pragma unroll
-            for (int i = 0; i < 4 * MT; ++i) {
+            for (int i = 0; i < 2 * NT * MT; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
                 __builtin_amdgcn_sched_group_barrier(0x002, 24 / MT, 0);   // VALU
             }
 #pragma unroll
-            for (int t = 0; t < 2; ++t) { bf[t][0] = bn[t][0]; bf[t][1] = bn[t][1]; }
+            for (int t = 0; t < NT; ++t) { bf[t][0] = bn[t][0]; bf[t][1] = bn[t][1]; }
             if (s < 7) {
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks)
@@ -644,7 +652,7 @@ __global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const
             }
         }
 #pragma unroll
-        for (int t = 0; t < 2; ++t) cur[t] = nxt[t];
+        for (int t = 0; t < NT; ++t) cur[t] = nxt[t];
         __syncthreads();  // next tile complete, this tile no longer read
     }
     // C layout of the 32x32 tile: column j = lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4
@@ -656,7 +664,7 @@ __global__ __launch_bounds__(256, (MT <= 2 ? 2 : 1)) void qgemm_f16_kernel(const
             if (m < M) {
                 const float rs = rowscale[m];
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
+                for (int t = 0; t < NT; ++t) {
                     const int n = n_base + 32 * t + j;
                     if (n < N) {
                         const float v = acc[mt][t][r] * rs;
@@ -716,7 +724,7 @@ int qgemm_f16_splits(int N, int K, int M) {
 static int qgemm_f16_row_tiles(bool q4, int M, int N, int splits) {
     if (M <= 64) return 2;
     const int wgs = ((N + QF_TN - 1) / QF_TN) * ((M + 127) / 128) * splits;
-    return (q4 && wgs < 200) ? 2 : 4;
+    return (q4 && wgs < 128) ? 2 : 4;  // 512 x 2560 x 9728 (152 workgroups): 60 us with 128 rows, 70 with 64; 512 x 4096 x 4096 (64): 80 / 68
 }
 
 static int qgemm_check(const void* W, const void* X, const void* Y, int M, int K, int N, int64_t stride, int blk_bytes) {
@@ -771,13 +779,21 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
         const int big = 2 * 128 * QF_PITCH, small = 2 * 64 * QF_PITCH;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
         raised = true;
     }
     const dim3 grid((N + QF_TN - 1) / QF_TN, (M + tm - 1) / tm, splits);
     const uint8_t* Wb = static_cast<const uint8_t*>(W);
-    if (q4 && MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    // 128-row tiles run with eight waves (PTM_QGEMM_WAVES=4 restores four, for tuning runs): 512 x 4096 x 14336
+    // 104 -> 92-94 us (Q4_K), 321 -> 308 us for 512 x 14336 x 4096 (Q6_K)
+    static const int waves_env = [] { const char* e = getenv("PTM_QGEMM_WAVES"); return e ? atoi(e) : 0; }();
+    const bool eight = MT == 4 && waves_env != 4;
+    if (eight && q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    else if (eight) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    else if (q4 && MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
