@@ -296,7 +296,8 @@ int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cac
 /* ---- batch-1 decode runtime (GGUFModel::forward_decode, gguf_model.h:2575-3113) --- */
 typedef struct {
     const void* data;         /* device, raw super-blocks */
-    uint32_t ggml_type;       /* PTM_TYPE_Q4_K or PTM_TYPE_Q6_K */
+    uint32_t ggml_type;       /* PTM_TYPE_Q4_K / Q6_K (fused kernels) or Q5_K / Q8_0 / Q5_0 (plain kernels; prompts of a
+                               * decoder holding any of these are stepped token by token) */
     int32_t rows, cols;       /* N, K */
     int64_t row_stride_bytes;
 } ptm_qweight; /* the device half of QuantizedWeight, gguf_model.h:336-385 */
@@ -399,7 +400,8 @@ const void* ptm_gguf_array_data(const ptm_gguf* g, const char* key);
  * uploads every blk.N.{attn_q,attn_k,attn_v,attn_output,ffn_gate,ffn_up,ffn_down}.weight and
  * output.weight (or the tied token_embd.weight) verbatim (gguf_model.h:1177-1360), norm vectors as
  * fp32, allocates zeroed KV caches for max_seq positions and creates the decode runtime.
- * Matrices must be Q4_K or Q6_K; other architectures, biases and other types: PTM_E_UNSUPPORTED. */
+ * Matrices may be of any type the GEMV dispatcher takes (Q4_K, Q6_K: the tuned path; Q5_K, Q8_0, Q5_0: plain
+ * kernels); other architectures, biases and other types: PTM_E_UNSUPPORTED. */
 typedef struct ptm_model ptm_model;
 int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_graph, ptm_model** out);
 ptm_decoder* ptm_model_decoder(ptm_model* m); /* owned by the model */

@@ -217,7 +217,7 @@ def argmax(x):
 def _qw(qtype, W):
     W = np.ascontiguousarray(W, np.uint8)
     N, stride = W.shape
-    return QW(W.ctypes.data, qtype, N, stride // (144 if qtype == 12 else 210) * 256, stride), W
+    return QW(W.ctypes.data, qtype, N, stride // BLOCK[qtype][0] * BLOCK[qtype][1], stride), W
 
 
 class MT19937:
@@ -404,7 +404,7 @@ class RefModel:
                 qt, W = L[name]
                 W = np.ascontiguousarray(W, np.uint8)
                 self._keep.append(W)
-                K = W.shape[1] // (144 if qt == 12 else 210) * 256
+                K = W.shape[1] // BLOCK[qt][0] * BLOCK[qt][1]
                 R.ref_model_set_weight(self.h, i, w, _p(W), qt, W.shape[0], K)
             for w, name in enumerate(("attn_norm", "ffn_norm", "q_norm", "k_norm")):
                 if L.get(name) is None:

@@ -135,7 +135,9 @@ static at::Tensor vec_tensor(const float* src, int64_t n) {
 static void set_qw(torch::io::QuantizedWeight& w, const void* data, uint32_t type, int64_t rows, int64_t cols) {
     w.cpu_data = const_cast<void*>(data);
     w.rows = rows; w.cols = cols; w.quant_type = type;
-    w.row_stride_bytes = cols / 256 * (type == 12 ? 144 : 210);
+    // block sizes of the dispatcher's formats (torch/io/gguf_dequant.h:29-58)
+    const int64_t blk_bytes = type == 12 ? 144 : type == 14 ? 210 : type == 13 ? 176 : type == 8 ? 34 : 22;
+    w.row_stride_bytes = cols / (type == 8 || type == 6 ? 32 : 256) * blk_bytes;
     w.total_bytes = rows * w.row_stride_bytes;
     w.valid = true; w.mmap_owned = true; w.owns_cpu_data = false;
 }

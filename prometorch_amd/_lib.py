@@ -19,6 +19,16 @@ class PtmError(RuntimeError):
         self.code = code
 
 
+# ggml type id -> (bytes per block, values per block) of the formats the GEMV dispatcher takes (gguf_dequant.h:29-58)
+BLOCK = {12: (144, 256), 14: (210, 256), 13: (176, 256), 8: (34, 32), 6: (22, 32)}
+
+
+def weight_cols(qtype: int, row_bytes: int) -> int:
+    """Values per row of a matrix whose rows are row_bytes of qtype blocks."""
+    b, per = BLOCK[qtype]
+    return row_bytes // b * per
+
+
 class QWeight(C.Structure):
     _fields_ = [("data", vp), ("ggml_type", u32), ("rows", C.c_int32), ("cols", C.c_int32), ("row_stride_bytes", i64)]
 

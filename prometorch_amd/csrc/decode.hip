@@ -91,6 +91,7 @@ struct ptm_decoder {
     int64_t* d_past = nullptr;
     int64_t* d_next = nullptr;
     int64_t* d_tokens = nullptr;
+    bool untuned_types = false;   // some matrix is Q5_K / Q8_0 / Q5_0: no row-batched GEMM for it, prompts go token by token
     int64_t* h_pinned = nullptr;  // [max_seq] pinned host staging for token ids
     float* h_uniforms = nullptr;  // [max_seq] pinned host staging for the sampler's draws (an "async" copy from the
                                   // caller's pageable memory would be staged by the runtime synchronously)
@@ -108,10 +109,15 @@ struct ptm_decoder {
     int* pf_tokens = nullptr;
 };
 
+static bool tuned_type(uint32_t t) { return t == PTM_TYPE_Q4_K || t == PTM_TYPE_Q6_K; }
+
+// Every type of the GEMV dispatcher is accepted.  Q4_K and Q6_K take the fused kernels of the decode path; Q5_K, Q8_0 and
+// Q5_0 matrices go through a separate RMSNorm and the dispatcher's plain kernels, and a model that holds any of them
+// is prefilled token by token (as the reference prefills every model: matmul_q is a loop of GEMVs, gguf_model.h:7029-7036).
 static int qw_check(const ptm_qweight& w, int rows, int cols) {
     if (!w.data) return PTM_E_NULL;
     if (w.rows != rows || w.cols != cols) return PTM_E_SHAPE;
-    if (w.ggml_type != PTM_TYPE_Q4_K && w.ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
+    if (!ptm_quant_gemv_supported(w.ggml_type)) return PTM_E_UNSUPPORTED;
     return PTM_OK;
 }
 
@@ -121,7 +127,9 @@ static int gemv_any(const ptm_qweight& w, const float* x_f32, float* y, bool acc
         const int N = w.rows;
         return q4k_gemv_multi(1, &W, &y, &N, x_f32, false, nullptr, 0.f, 0, w.cols, w.row_stride_bytes, acc, s);
     }
-    return q6k_gemv_impl(w.data, x_f32, y, w.cols, w.rows, w.row_stride_bytes, acc, nullptr, 0.f, 0, s);
+    if (w.ggml_type == PTM_TYPE_Q6_K)
+        return q6k_gemv_impl(w.data, x_f32, y, w.cols, w.rows, w.row_stride_bytes, acc, nullptr, 0.f, 0, s);
+    return ptm_quant_gemv(w.ggml_type, w.data, x_f32, y, w.cols, w.rows, w.row_stride_bytes, acc ? 1 : 0, s);
 }
 
 // Enqueue one token step on d->stream. Everything it reads that changes per token is in device memory.
@@ -148,7 +156,10 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
                 else { i6 = i; ++n6; }
             }
             const int64_t s4 = (int64_t)(H / 256) * 144;
-            if (n6 == 1 && n4 >= 1 && H <= 16384) {
+            if (!tuned_type(L.q.ggml_type) || !tuned_type(L.k.ggml_type) || !tuned_type(L.v.ggml_type)) {
+                PTM_TRY(ptm_rms_norm(d->x, L.attn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+                for (int i = 0; i < 3; ++i) PTM_TRY(gemv_any(*w[i], d->xn, y[i], false, s));
+            } else if (n6 == 1 && n4 >= 1 && H <= 16384) {
                 // the Q4_K_M mix (q, k in Q4_K; v in Q6_K): all three projections in one launch
                 PTM_TRY(rmsnorm_mixed_gemv(n4, W4, y4, N4, s4, w[i6]->data, y[i6], w[i6]->rows, w[i6]->row_stride_bytes,
                                            d->x, L.attn_norm, c.rms_eps, 0, H, s));
@@ -321,6 +332,9 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->cfg = c;
     d->layers.assign(c.layers, c.layers + c.n_layers);
     d->cfg.layers = d->layers.data();
+    for (const ptm_layer& L : d->layers)
+        for (const ptm_qweight* w : {&L.q, &L.k, &L.v, &L.o, &L.gate, &L.up, &L.down})
+            if (!tuned_type(w->ggml_type)) d->untuned_types = true;
 
     const int S = ptm_flash_decode_num_splits(c.max_seq);
     auto up16 = [](size_t b) { return (b + 255) & ~(size_t)255; };
@@ -516,6 +530,13 @@ int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_r
     for (int i = 0; i < n; ++i)
         if (tokens[i] < 0 || tokens[i] >= d->cfg.vocab) return PTM_E_RANGE;
     const ptm_decode_config& c = d->cfg;
+    if (d->untuned_types) {
+        // no row-batched GEMM for these types: the prompt is stepped, each step a full decode step whose token is dropped
+        int rc = PTM_OK;
+        for (int i = 0; i < n && rc == PTM_OK; ++i) rc = run_steps(d, tokens[i], 1);
+        if (rc == PTM_OK) *next_token = d->h_pinned[0];
+        return rc;
+    }
     if (chunk_rows <= 0) chunk_rows = 2048;  // measured: 2048-row chunks run a 4096-token prompt 1.4x faster than 512-row ones
     if (chunk_rows > 2048) chunk_rows = 2048;  // bounds the row scratch (and the launch grids) whatever the prompt length
     if (chunk_rows > n) chunk_rows = n;

@@ -127,6 +127,9 @@ static int64_t tensor_bytes(uint32_t ggml_type, uint64_t n_elems) {
         case 1: return (int64_t)n_elems * 2;                               // F16
         case PTM_TYPE_Q4_K: return n_elems % 256 ? -1 : (int64_t)(n_elems / 256) * 144;
         case PTM_TYPE_Q6_K: return n_elems % 256 ? -1 : (int64_t)(n_elems / 256) * 210;
+        case PTM_TYPE_Q5_K: return n_elems % 256 ? -1 : (int64_t)(n_elems / 256) * 176;
+        case PTM_TYPE_Q8_0: return n_elems % 32 ? -1 : (int64_t)(n_elems / 32) * 34;
+        case PTM_TYPE_Q5_0: return n_elems % 32 ? -1 : (int64_t)(n_elems / 32) * 22;
         default: return -1;  // a type this reader does not size; the tensor stays listed with nbytes = -1
     }
 }
@@ -335,15 +338,23 @@ static int load_matrix(ptm_model* m, const std::string& name, int64_t rows, int6
     ptm_gguf_tensor t{};
     int rc = ptm_gguf_find_tensor(m->file, name.c_str(), &t);
     if (rc != PTM_OK) return rc;
-    if (t.ggml_type != PTM_TYPE_Q4_K && t.ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
-    if (t.n_dims != 2 || t.dims[0] != cols || t.dims[1] != rows || t.nbytes <= 0) return PTM_E_SHAPE;
+    int blk_bytes = 0, blk_vals = 0;
+    switch (t.ggml_type) {  // the GEMV dispatcher's formats (gguf_dequant.h:29-58)
+        case PTM_TYPE_Q4_K: blk_bytes = 144; blk_vals = 256; break;
+        case PTM_TYPE_Q6_K: blk_bytes = 210; blk_vals = 256; break;
+        case PTM_TYPE_Q5_K: blk_bytes = 176; blk_vals = 256; break;
+        case PTM_TYPE_Q8_0: blk_bytes = 34; blk_vals = 32; break;
+        case PTM_TYPE_Q5_0: blk_bytes = 22; blk_vals = 32; break;
+        default: return PTM_E_UNSUPPORTED;
+    }
+    if (t.n_dims != 2 || t.dims[0] != cols || t.dims[1] != rows || t.nbytes <= 0 || cols % blk_vals != 0) return PTM_E_SHAPE;
     void* d = nullptr;
     if ((rc = upload(m, t.data, (size_t)t.nbytes, &d)) != PTM_OK) return rc;
     w->data = d;
     w->ggml_type = t.ggml_type;
     w->rows = (int32_t)rows;
     w->cols = (int32_t)cols;
-    w->row_stride_bytes = cols / 256 * (t.ggml_type == PTM_TYPE_Q4_K ? 144 : 210);
+    w->row_stride_bytes = cols / blk_vals * blk_bytes;
     return PTM_OK;
 }
 
@@ -424,8 +435,13 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
         void* table = nullptr;
         const int64_t n = (int64_t)c.vocab * c.hidden;
         PTM_L(upload(m, nullptr, (size_t)n * 4, &table));
-        PTM_L(ew.ggml_type == PTM_TYPE_Q4_K ? ptm_dequant_q4k(ew.data, static_cast<float*>(table), n, nullptr)
-                                            : ptm_dequant_q6k(ew.data, static_cast<float*>(table), n, nullptr));
+        switch (ew.ggml_type) {
+            case PTM_TYPE_Q4_K: PTM_L(ptm_dequant_q4k(ew.data, static_cast<float*>(table), n, nullptr)); break;
+            case PTM_TYPE_Q6_K: PTM_L(ptm_dequant_q6k(ew.data, static_cast<float*>(table), n, nullptr)); break;
+            case PTM_TYPE_Q5_K: PTM_L(ptm_dequant_q5k(ew.data, static_cast<float*>(table), n, nullptr)); break;
+            case PTM_TYPE_Q8_0: PTM_L(ptm_dequant_q8_0(ew.data, static_cast<float*>(table), n, nullptr)); break;
+            default: ptm_model_free(m); return PTM_E_UNSUPPORTED;  // the reference has no Q5_0 dequantiser either
+        }
         PTM_L(hip_status(hipDeviceSynchronize()));
         c.embedding_f32 = static_cast<const float*>(table);
     }

@@ -45,8 +45,7 @@ class Decoder:
                 qt, W = Ld[name]
                 t = _upload_bytes(W)
                 self._keep.append(t)
-                bb = 144 if qt == 12 else 210
-                setattr(arr[i], name, QWeight(t.data_ptr(), qt, W.shape[0], W.shape[1] // bb * 256, W.shape[1]))
+                setattr(arr[i], name, QWeight(t.data_ptr(), qt, W.shape[0], _lib.weight_cols(qt, W.shape[1]), W.shape[1]))
             for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
                 if Ld.get(name) is None:  # q_norm / k_norm: a model without QK-norm
                     setattr(arr[i], name, None)

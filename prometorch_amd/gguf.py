@@ -93,7 +93,7 @@ def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "q
         ts.append((p + "attn_norm.weight", F32, [H], np.asarray(L["attn_norm"], np.float32)))
         for k, gname in names.items():
             qt, W = L[k]
-            cols = W.shape[1] // (144 if qt == Q4_K else 210) * 256
+            cols = _lib.weight_cols(qt, W.shape[1])
             ts.append((p + gname + ".weight", qt, [cols, W.shape[0]], W))
         if L.get("q_norm") is not None:  # absent in a llama-style model
             ts.append((p + "attn_q_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["q_norm"], np.float32)))

@@ -213,6 +213,20 @@ MIX_ALL_Q4K = tuple((n, Q4_K) for n, _ in LAYER_MATS)
 MIX_ODD = (("q", Q6_K), ("k", Q4_K), ("v", Q4_K), ("o", Q6_K), ("gate", Q6_K), ("up", Q4_K), ("down", Q6_K))
 
 
+# The dispatcher's other formats in every projection role: a Q8_0 layer, a Q5_K layer, and a layer mixing all five types
+MIX_Q8_0 = tuple((n, Q8_0) for n, _ in LAYER_MATS)
+MIX_Q5_K = tuple((n, Q5_K) for n, _ in LAYER_MATS)
+MIX_FIVE = (("q", Q5_0), ("k", Q8_0), ("v", Q5_K), ("o", Q4_K), ("gate", Q5_K), ("up", Q8_0), ("down", Q5_0))
+
+
+def tiny_formats(seed: int):
+    """The TINY shapes with three layers in the GEMV dispatcher's other formats: MIX_Q8_0, MIX_Q5_K, MIX_FIVE."""
+    cfg = dict(TINY)
+    cfg["n_layers"] = 3
+    layers = [make_layer(seed, i, cfg, mats=m) for i, m in enumerate((MIX_Q8_0, MIX_Q5_K, MIX_FIVE))]
+    return cfg, layers, make_head(seed, cfg)
+
+
 MIXED_FEED = tuple((131 * i + 3) % 1024 for i in range(32))  # tokens fed to tiny_mixed step by step
 
 

@@ -101,7 +101,7 @@ def main():
         return
     if args.mixed_only:
         make_mixed_golden()
-        print("wrote golden_mixed.npz")
+        print("wrote golden_mixed.npz, golden_formats_model.npz")
         return
     if args.formats_only:
         make_formats_golden()
@@ -337,8 +337,14 @@ def make_formats_golden():
 
 def make_mixed_golden():
     """The reference's forward_decode_cpu on synth.tiny_mixed: layers whose q/k/v share a type (fused QKV, 8-lane
-    norm, gguf_model.h:3342-3350) beside layers where they do not, Q4_K and Q6_K in every projection role."""
-    cfg, layers, head = synth.tiny_mixed(SEEDS["tiny"])
+    norm, gguf_model.h:3342-3350) beside layers where they do not, Q4_K and Q6_K in every projection role; and on
+    synth.tiny_formats: Q8_0, Q5_K and Q5_0 matrices through the same step (golden_formats_model.npz)."""
+    for maker, fname in ((synth.tiny_mixed, "golden_mixed.npz"), (synth.tiny_formats, "golden_formats_model.npz")):
+        _model_golden(maker, fname)
+
+
+def _model_golden(maker, fname):
+    cfg, layers, head = maker(SEEDS["tiny"])
     emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
     rm = po.RefModel(cfg, layers, head, 64, emb)
     for i in range(cfg["n_layers"]):
@@ -349,7 +355,7 @@ def make_mixed_golden():
         toks.append(rm.step(synth.MIXED_FEED[st]))
         lg.append(rm.logits.copy())
     rm.close()
-    np.savez_compressed(os.path.join(OUT, "golden_mixed.npz"), tokens=np.array(toks, np.int64), logits=np.stack(lg))
+    np.savez_compressed(os.path.join(OUT, fname), tokens=np.array(toks, np.int64), logits=np.stack(lg))
 
 
 def make_llama_golden():

@@ -110,3 +110,75 @@ def test_mixed_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_mixed, t
         assert np.array_equal(bits(m.logits()), bits(d.logits())), st
     m.close()
     d.close()
+
+
+# ---- the dispatcher's other formats (Q8_0, Q5_K, Q5_0) through the decoder: plain kernels, prompts stepped token by token ----
+@pytest.fixture(scope="module")
+def golden_formats_model():
+    return np.load(os.path.join(GOLDEN_DIR, "golden_formats_model.npz"))
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_other_formats_decode_fp32_kv_vs_reference_golden(dev, golden_formats_model, seeds, use_graph):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = synth.tiny_formats(seeds["tiny"])
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False, use_graph=use_graph)
+    for i in range(cfg["n_layers"]):
+        dec.set_kv(i, *synth.make_kv_prefill(seeds["tiny"], i, cfg, 19))
+    dec.set_past_len(19)
+    errs = []
+    for st in range(12):
+        tok = dec.step(synth.MIXED_FEED[st])
+        ref = golden_formats_model["logits"][st]
+        errs.append(np.abs(dec.logits() - ref).max() / ref.std())
+        assert tok == int(golden_formats_model["tokens"][st]), st
+    check_step_errors(errs)
+    dec.close()
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+def test_other_formats_prompt_and_generation_vs_oracle(dev, po, seeds, kv_fp16):
+    """A decoder holding Q8_0 / Q5_K / Q5_0 matrices has no row-batched GEMM: its prefill steps the prompt, so the
+    logits and cache rows agree with the oracle as closely as single steps do."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = synth.tiny_formats(seeds["tiny"])
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=kv_fp16)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=kv_fp16, use_graph=True)
+    prompt = [int(t) for t in synth.rng_for(70).integers(0, cfg["vocab"], 17)]
+    for t in prompt:
+        tok_o = om.step(t)
+    tok_g = dec.prefill(prompt)
+    assert tok_g == tok_o
+    assert np.abs(dec.logits() - om.logits).max() <= LOGIT_TOL_FLIP * om.logits.std()
+    for li in range(cfg["n_layers"]):
+        k_gpu = dec.k_cache[li][:17].float().cpu().numpy()
+        assert np.abs(k_gpu - om.k_cache[li][:17]).max() <= 2e-3 * np.abs(om.k_cache[li][:17]).max()
+    errs = []
+    for st in range(10):
+        tok_o = om.step(tok_o)
+        tok_g = dec.step(tok_g)
+        errs.append(np.abs(dec.logits() - om.logits).max() / om.logits.std())
+        assert tok_g == tok_o, st
+    check_step_errors(errs)
+    dec.close()
+
+
+def test_other_formats_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_formats_model, tmp_path):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = synth.tiny_formats(seeds["tiny"])
+    path = str(tmp_path / "tiny_formats.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head)
+    m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
+    d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(seeds["tiny"], i, cfg, 19)
+        m.set_kv(i, k, v)
+        d.set_kv(i, k, v)
+    m.set_past_len(19)
+    d.set_past_len(19)
+    for st in range(12):
+        tm, td = m.step(synth.MIXED_FEED[st]), d.step(synth.MIXED_FEED[st])
+        assert tm == td == int(golden_formats_model["tokens"][st]), st
+        assert np.array_equal(bits(m.logits()), bits(d.logits())), st
+    m.close()
+    d.close()

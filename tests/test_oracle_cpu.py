@@ -237,14 +237,15 @@ def test_llama_style_decode_and_rope_match_the_reference(po, seeds):
     assert np.abs(qr.reshape(32, 64, 2) - want).max() <= 2e-3 * np.abs(want).max()   # fp32 angles of ~2e3 rad
 
 
-def test_mixed_type_layers_match_the_reference(po, seeds):
+@pytest.mark.parametrize("maker,fname", [("tiny_mixed", "golden_mixed.npz"), ("tiny_formats", "golden_formats_model.npz")])
+def test_mixed_type_layers_match_the_reference(po, seeds, maker, fname):
     """Layers whose q/k/v share a type (the reference fuses them behind its 8-lane norm) beside layers where they do
-    not, Q4_K and Q6_K in every projection role (synth.tiny_mixed): oracle bit-identical to the compiled reference's
-    forward_decode_cpu (golden_mixed.npz)."""
+    not, Q4_K and Q6_K in every projection role (synth.tiny_mixed), and layers in the dispatcher's other formats
+    (Q8_0, Q5_K, Q5_0: synth.tiny_formats): oracle bit-identical to the compiled reference's forward_decode_cpu."""
     import os
     from prometorch_amd import synth
-    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_mixed.npz"))
-    cfg, layers, head = synth.tiny_mixed(seeds["tiny"])
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", fname))
+    cfg, layers, head = getattr(synth, maker)(seeds["tiny"])
     om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)
     for i in range(cfg["n_layers"]):
         om.set_kv(i, *synth.make_kv_prefill(seeds["tiny"], i, cfg, 19))
