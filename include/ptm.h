@@ -394,7 +394,8 @@ int ptm_gguf_get_array(const ptm_gguf* g, const char* key, uint32_t* elem_type, 
 int ptm_gguf_array_string(const ptm_gguf* g, const char* key, int64_t i, const char** data, int64_t* len);
 const void* ptm_gguf_array_data(const ptm_gguf* g, const char* key);
 
-/* From a .gguf file to a ready decoder: reads the `qwen3` hyper-parameters
+/* From a .gguf file to a ready decoder: reads the `qwen3` or `llama` (no QK-norm tensors, interleaved rotation
+ * pairs: gguf_model.h:202-217) hyper-parameters
  * (<arch>.block_count, embedding_length, feed_forward_length, attention.head_count(_kv),
  * attention.key_length, rope.freq_base, attention.layer_norm_rms_epsilon; gguf_model.h:126-181),
  * uploads every blk.N.{attn_q,attn_k,attn_v,attn_output,ffn_gate,ffn_up,ffn_down}.weight and
