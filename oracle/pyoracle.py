@@ -280,7 +280,7 @@ class OracleModel:
             self.v_cache.append(vc)
             self.layers[i].k_cache = kc.ctypes.data
             self.layers[i].v_cache = vc.ctypes.data
-        lm, lmW = _qw(14, head["lm_head"])
+        lm, lmW = _qw(head.get("lm_head_type", 14), head["lm_head"])
         on = np.ascontiguousarray(head["out_norm"], np.float32)
         self._keep += [lmW, on]
         self.m = Model()
@@ -414,7 +414,7 @@ class RefModel:
         lm = np.ascontiguousarray(head["lm_head"], np.uint8)
         on = np.ascontiguousarray(head["out_norm"], np.float32)
         self._keep += [lm, on]
-        R.ref_model_set_output(self.h, _p(on), _p(lm), 14)
+        R.ref_model_set_output(self.h, _p(on), _p(lm), head.get("lm_head_type", 14))
         emb = np.ascontiguousarray(embedding, np.float32)
         R.ref_model_set_embedding(self.h, _p(emb))
         self.logits = np.empty(cfg["vocab"], np.float32)

@@ -25,7 +25,7 @@ class Decoder:
 
     layers: list of dicts with (qtype, uint8[rows, stride]) per projection name and fp32 norm
     vectors 'attn_norm', 'ffn_norm', 'q_norm', 'k_norm' (the last two None for a model without QK-norm;
-    cfg['rope_interleaved'] selects llama-style rotation pairs); head: {'lm_head': uint8 Q6_K table,
+    cfg['rope_interleaved'] selects llama-style rotation pairs); head: {'lm_head': uint8 table (Q6_K unless 'lm_head_type' says otherwise),
     'out_norm': fp32}.  The token-embedding is the tied Q6_K table unless embedding_f32 is given."""
 
     def __init__(self, cfg: dict, layers: list, head: dict, max_seq: int, kv_fp16: bool = True,
@@ -81,7 +81,7 @@ class Decoder:
             c.embedding_f32 = None
         c.layers = arr
         c.out_norm = on.data_ptr()
-        c.lm_head = QWeight(lm.data_ptr(), 14, cfg["vocab"], cfg["hidden"], head["lm_head"].shape[1])
+        c.lm_head = QWeight(lm.data_ptr(), head.get("lm_head_type", 14), cfg["vocab"], cfg["hidden"], head["lm_head"].shape[1])
         self._cfg = c
         torch.cuda.synchronize()
         h = C.c_void_p()

@@ -83,9 +83,10 @@ def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "q
         md = {k: v for k, v in md.items() if not k.startswith("tokenizer.")}
         md.update(tokenizer)
     H = cfg["hidden"]
-    ts = [("token_embd.weight", Q6_K, [H, cfg["vocab"]], head["lm_head"])]
+    lm_type = head.get("lm_head_type", Q6_K)
+    ts = [("token_embd.weight", lm_type, [H, cfg["vocab"]], head["lm_head"])]
     if not tied:
-        ts.append(("output.weight", Q6_K, [H, cfg["vocab"]], head["lm_head"]))
+        ts.append(("output.weight", lm_type, [H, cfg["vocab"]], head["lm_head"]))
     ts.append(("output_norm.weight", F32, [H], np.asarray(head["out_norm"], np.float32)))
     names = {"q": "attn_q", "k": "attn_k", "v": "attn_v", "o": "attn_output", "gate": "ffn_gate", "up": "ffn_up", "down": "ffn_down"}
     for i, L in enumerate(layers):

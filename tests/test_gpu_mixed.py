@@ -182,3 +182,27 @@ def test_other_formats_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_
         assert np.array_equal(bits(m.logits()), bits(d.logits())), st
     m.close()
     d.close()
+
+
+@pytest.mark.parametrize("lm_type,tied", [(8, True), (13, True), (8, False), (12, True)])
+def test_other_lm_head_types_from_gguf_vs_oracle(dev, po, seeds, tmp_path, lm_type, tied):
+    """token_embd / output in Q8_0, Q5_K or Q4_K (a Q8_0 file keeps both in Q8_0): the loader dequantises the embedding
+    table to fp32 on the device and the vocabulary projection goes through the dispatcher."""
+    cfg, layers, head = synth.tiny_formats(seeds["tiny"])
+    head = dict(head)
+    head["lm_head_type"] = lm_type
+    head["lm_head"] = synth.make_weight(synth.rng_for(seeds["tiny"], 3, lm_type), lm_type, cfg["vocab"], cfg["hidden"])
+    emb = po.dequant(lm_type, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False, embedding=emb)
+    path = str(tmp_path / "lm.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head, tied=tied)
+    m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
+    errs, tok_o = [], 5
+    tok_g = 5
+    for st in range(10):
+        tok_o = om.step(tok_o)
+        tok_g = m.step(tok_g)
+        errs.append(np.abs(m.logits() - om.logits).max() / om.logits.std())
+        assert tok_g == tok_o, st
+    check_step_errors(errs)
+    m.close()
