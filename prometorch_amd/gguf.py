@@ -204,6 +204,7 @@ class GGUFModel:
         check(self.L.ptm_model_load_gguf(path.encode(), max_seq, int(kv_fp16), int(use_graph), C.byref(m)),
               f"model_load_gguf({path})")
         self.m = m
+        self._path = path
         self.h = self.L.ptm_model_decoder(m)
         c = DecodeConfig()
         check(self.L.ptm_model_config(m, C.byref(c)), "model_config")
@@ -257,6 +258,35 @@ class GGUFModel:
                                          C.byref(n_out)), "decode_generate")
         return list(out[:n_out.value])
 
+    # the reference's stop strings besides the file's eos id (GGUFModel::is_stop_token, gguf_model.h:5132-5139)
+    STOP_TOKENS = ("<|im_end|>", "<|endoftext|>", "<end_of_turn>", "<|eot_id|>", "</s>", "<|end|>")
+
+    def chat(self, prompt: str, system=None, max_new: int = 256, temperature: float = 0.7, top_k: int = 40,
+             top_p: float = 0.9, repeat_penalty: float = 1.1, seed: int = 42, no_think: bool = False) -> str:
+        """One chat turn from text to text on a fresh context: the file's chat template and tokenizer, prompt prefill,
+        sampled decode on the device until a stop token (promeserve/api_handlers.h:848-923), the reply decoded."""
+        from . import ops
+        from .tokenizer import Tokenizer, chat_template
+        if getattr(self, "_tok", None) is None:
+            self._file = GGUFFile(self._path)
+            self._tok = Tokenizer.from_gguf(self._file)
+            stops = {self._tok.special_ids()["eos"]}
+            for t in self.STOP_TOKENS:
+                ids = self._tok.encode(t, use_bos=False)
+                if len(ids) == 1:
+                    stops.add(ids[0])
+            self._stops = sorted(i for i in stops if i >= 0)
+        arch = self._file.get_string("general.architecture")
+        name = self._file.get_string("general.name") or ""
+        ids = self._tok.encode(chat_template(arch, prompt, model_name=name, system=system, no_think=no_think))
+        room = self.cfg["max_seq"] - len(ids)
+        if room <= 0:
+            raise ValueError("prompt of %d tokens does not fit a context of %d" % (len(ids), self.cfg["max_seq"]))
+        self.set_past_len(0)
+        out = self.generate(ids, ops.mt19937_uniforms(seed, 0, min(max_new, room)), temperature, top_k, top_p,
+                            repeat_penalty, stop_ids=self._stops)
+        return self._tok.decode(out).decode("utf-8", errors="replace")
+
     def sampling_begin(self, temperature: float, top_k: int, top_p: float, repeat_penalty: float = 1.0) -> None:
         """Start a sampled generation: store the parameters, forget previously generated tokens."""
         from ._lib import Sampling
@@ -284,6 +314,10 @@ class GGUFModel:
         return out.cpu().numpy()
 
     def close(self) -> None:
+        if getattr(self, "_tok", None) is not None:
+            self._tok.close()
+            self._file.close()
+            self._tok = self._file = None
         if getattr(self, "m", None):
             self.L.ptm_model_free(self.m)
             self.m = None

@@ -115,3 +115,34 @@ def test_text_to_text_through_one_file(dev, po, seeds, tmp_path):
     reply = tk.decode(got)
     assert isinstance(reply, bytes) and len(reply) > 0
     m.close(); tk.close(); f.close()
+
+
+def test_chat_is_the_manual_path_in_one_call(dev, seeds, tmp_path):
+    """GGUFModel.chat = chat template + tokenizer + ptm_decode_generate with the file's stop tokens + decode."""
+    from prometorch_amd import ops
+    from prometorch_amd.tokenizer import Tokenizer, chat_template
+    cfg, layers, head, _ = build_tiny(seeds)
+    tok_md = synth.make_tokenizer("gpt2", vocab_size=cfg["vocab"])
+    path = str(tmp_path / "chat.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head, tokenizer=tok_md)
+    m = gguf.GGUFModel(path, max_seq=160, kv_fp16=True)
+    reply = m.chat("Hello there, what's 2+2?", system="Be brief.", max_new=24, temperature=0.8, top_k=40, top_p=0.9,
+                   repeat_penalty=1.1, seed=42)
+    assert isinstance(reply, str)
+    with gguf.GGUFFile(path) as f:
+        tk = Tokenizer.from_gguf(f)
+        ids = tk.encode(chat_template(f.get_string("general.architecture"), "Hello there, what's 2+2?",
+                                      model_name=f.get_string("general.name") or "", system="Be brief."))
+        stops = sorted({tk.special_ids()["eos"]} | {tk.encode(t, use_bos=False)[0] for t in m.STOP_TOKENS
+                                                    if len(tk.encode(t, use_bos=False)) == 1})
+        m.set_past_len(0)
+        want = m.generate(ids, ops.mt19937_uniforms(42, 0, 24), 0.8, 40, 0.9, 1.1, stop_ids=[s for s in stops if s >= 0])
+        assert reply == tk.decode(want).decode("utf-8", errors="replace")
+        assert all(t not in stops for t in want)
+        # a second turn starts from an empty context again and, with the same seed, repeats the first
+        assert m.chat("Hello there, what's 2+2?", system="Be brief.", max_new=24, temperature=0.8, top_k=40, top_p=0.9,
+                      repeat_penalty=1.1, seed=42) == reply
+        tk.close()
+    with pytest.raises(ValueError):
+        m.chat("x " * 400, max_new=8)
+    m.close()
