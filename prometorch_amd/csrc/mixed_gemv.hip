@@ -52,12 +52,32 @@ int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const in
     a4.gamma = gamma;
     a4.eps = eps;
     a4.add_one = add_one;
-    a4.log2S = q4k_pick_log2S(total, K / 256, 3);
-    Q6KArgs a6{static_cast<const uint8_t*>(W6), x, y6, K, N6, q6k_pick_log2S(N6, K / 256), stride6, nullptr, nullptr,
+    // Lane groups per row of the two parts.  Every workgroup stages x and gamma (20 KB for 2560 values) for a few KB of
+    // weights, so the launch wants few, fat workgroups: the smallest split that still gives the chip 1.5 workgroups
+    // per CU, the Q6_K rows (fewer, and more arithmetic per byte) one step finer than the Q4_K ones.  Qwen3-4B and
+    // Llama-3-8B shapes both land on 2 and 4 groups per row (448 workgroups): 617 -> 633 tok/s and 518 -> 523 tok/s
+    // against the per-kernel rules of the single-type GEMVs (4 and 8 groups, 896 workgroups).
+    // PTM_MIXED_L4 / PTM_MIXED_L6 (0..3) override, for tuning runs.
+    static const int l4_env = [] { const char* e = getenv("PTM_MIXED_L4"); return e ? atoi(e) : -1; }();
+    static const int l6_env = [] { const char* e = getenv("PTM_MIXED_L6"); return e ? atoi(e) : -1; }();
+    int l4 = 3, l6 = 3;
+    for (int l = 0; l <= 3; ++l) {
+        const int t6 = l + 1 < 3 ? l + 1 : 3;
+        if ((total + (32 >> l) - 1) / (32 >> l) + (N6 + (32 >> t6) - 1) / (32 >> t6) >= 384 || l == 3) {
+            l4 = l;
+            l6 = t6;
+            break;
+        }
+    }
+    if (l4_env >= 0 && l4_env <= 3) l4 = l4_env;
+    if (l6_env >= 0 && l6_env <= 3) l6 = l6_env;
+    a4.log2S = l4;
+    Q6KArgs a6{static_cast<const uint8_t*>(W6), x, y6, K, N6, l6, stride6, nullptr, nullptr,
                gamma, eps, add_one, nullptr};
-    const int n6 = q6k_workgroups(N6, K), n4w = q4k_workgroups(total, a4.log2S);
+    const int n6 = (N6 + (32 >> l6) - 1) / (32 >> l6), n4w = q4k_workgroups(total, a4.log2S);
     const size_t lds = (size_t)K * 4 + (size_t)K / 4;  // the Q6_K body's fp32 x + per-16 sums; Q4_K needs less
-    const int nb6 = q6k_blocks_per_pass(N6, K);
+    static const int cand6[] = {2, 3, 5};
+    const int nb6 = pick_blocks_per_pass((K / 256 + (1 << l6) - 1) >> l6, cand6, 3);
     const dim3 grid(n6 + n4w);
     switch (q4k_blocks_per_pass(K / 256, a4.log2S)) {
         case 2: mixed_launch6<2>(nb6, grid, lds, s, a4, a6, n6); break;
