@@ -17,6 +17,14 @@
 #include <new>
 #include <vector>
 
+// flash_decode.hip: ptm_attn_decode_fused that also leaves the output as Q8 activation blocks (not part of the C ABI)
+extern "C" int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                                        const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8,
+                                        float* partial_O, float* partial_lse, float* partial_max, const float* rope_table,
+                                        int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                                        float scale, float eps, int add_one, int kv_fp16, int rope_interleaved,
+                                        ptm_stream_t stream);
+
 namespace ptm {
 int q4k_gemv_multi(int n_mat, const void* const* W, float* const* y, const int* N, const void* x, bool x_is_q8,
                    const float* gamma, float eps, int add_one, int K, int64_t stride, bool accumulate, hipStream_t s);
@@ -172,10 +180,21 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
             }
         }
         // QK-norm + RoPE + K/V append + split-KV attention in one launch, plus the small merge launch
-        PTM_TRY(ptm_attn_decode_fused(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn, d->pO,
-                                      d->pL, d->pM, d->rope, c.n_heads, c.n_kv_heads, hd, d->d_past,
-                                      c.max_seq, 1.0f / sqrtf((float)hd), c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, s));
-        PTM_TRY(gemv_any(L.o, d->attn, d->x, true, s));  // x += Wo . attn
+        // a Q4_K output projection takes the attention output as the Q8 blocks the merge kernel leaves beside the fp32
+        // vector: its prologue then copies 1.25 bytes per value instead of fetching and quantising 4
+        const bool o_q8 = L.o.ggml_type == PTM_TYPE_Q4_K;
+        PTM_TRY(ptm_attn_decode_fused_q8(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn,
+                                         o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM, d->rope, c.n_heads, c.n_kv_heads, hd,
+                                         d->d_past, c.max_seq, 1.0f / sqrtf((float)hd), c.rms_eps, 0, c.kv_fp16,
+                                         c.rope_interleaved, s));
+        if (o_q8) {  // x += Wo . attn
+            const void* W = L.o.data;
+            float* y = d->x;
+            const int N = L.o.rows;
+            PTM_TRY(q4k_gemv_multi(1, &W, &y, &N, d->xq8, true, nullptr, 0.f, 0, L.o.cols, L.o.row_stride_bytes, true, s));
+        } else {
+            PTM_TRY(gemv_any(L.o, d->attn, d->x, true, s));
+        }
         if (L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
             L.gate.row_stride_bytes == L.up.row_stride_bytes && L.gate.rows == L.up.rows) {
             PTM_TRY(q4k_gate_up_silu(L.gate.data, L.up.data, d->x, false, L.ffn_norm, c.rms_eps, 0, d->act, H,
@@ -346,7 +365,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
                  o_up = take(4 * (size_t)c.inter), o_logits = take(4 * (size_t)c.vocab),
                  o_pO = take(4 * (size_t)S * c.n_heads * c.head_dim), o_pL = take(4 * (size_t)S * c.n_heads),
                  o_pM = take(4 * (size_t)S * c.n_heads), o_rope = take(4 * (size_t)c.max_seq * c.head_dim),
-                 o_xq8 = take((size_t)ptm_q8_bytes(H > c.inter ? H : c.inter)),
+                 o_xq8 = take((size_t)ptm_q8_bytes(qd > (H > c.inter ? H : c.inter) ? qd : (H > c.inter ? H : c.inter))),
                  o_ws = take((size_t)ptm_argmax_workspace_bytes(c.vocab)), o_tok = take(256), o_past = take(256),
                  o_next = take(256), o_step = take(256), o_tokens = take(8 * (size_t)c.max_seq),
                  o_samp = take(256), o_counts = take(4 * (size_t)c.vocab), o_unif = take(4 * (size_t)c.max_seq),

@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
                                                                  const float* __restrict__ pL,
                                                                  const float* __restrict__ pM, float* __restrict__ O,
                                                                  int n_heads, const int64_t* __restrict__ d_past,
-                                                                 int max_seq) {
+                                                                 int max_seq, uint8_t* __restrict__ q8_out) {
     constexpr int NOUT = HD / 4, NSLOT = 256 / NOUT;
     __shared__ __align__(16) float4 s_stage[256];
     __shared__ float s_red[8];
@@ -231,16 +231,31 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
         }
         const float dsum = (s_red[4] + s_red[5]) + (s_red[6] + s_red[7]);
         const float inv = 1.0f / (dsum + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
-        reinterpret_cast<float4*>(O)[(int64_t)h * NOUT + tid] = make_float4(t.x * inv, t.y * inv, t.z * inv, t.w * inv);
+        const float4 o4 = make_float4(t.x * inv, t.y * inv, t.z * inv, t.w * inv);
+        reinterpret_cast<float4*>(O)[(int64_t)h * NOUT + tid] = o4;
+        if (q8_out) {
+            // the same vector as Q8 blocks (int8 qs[K] | float d[K/32] | float sum[K/32], K = n_heads * HD) for a Q4_K
+            // output projection, whose prologue then copies 1.25 bytes per value instead of quantising 4
+            const int K = n_heads * HD;
+            float d, sm;
+            const uint32_t packed = q8_quantize4(o4, d, sm);  // 8 consecutive lanes hold one block of 32
+            reinterpret_cast<uint32_t*>(q8_out)[(int64_t)h * NOUT + tid] = packed;
+            if ((tid & 7) == 0) {
+                float* dd = reinterpret_cast<float*>(q8_out + K);
+                const int blk = h * (HD / 32) + (tid >> 3);
+                dd[blk] = d;
+                dd[K / 32 + blk] = sm;
+            }
+        }
     }
 }
 
 static int fd_merge(int head_dim, int n_heads, hipStream_t s, const float* pO, const float* pL, const float* pM, float* O,
-                    const int64_t* d_past, int max_seq) {
+                    const int64_t* d_past, int max_seq, uint8_t* q8_out = nullptr) {
     if (head_dim == 128)
-        hipLaunchKernelGGL(flash_decode_merge_kernel<128>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq);
+        hipLaunchKernelGGL(flash_decode_merge_kernel<128>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq, q8_out);
     else
-        hipLaunchKernelGGL(flash_decode_merge_kernel<64>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq);
+        hipLaunchKernelGGL(flash_decode_merge_kernel<64>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq, q8_out);
     return launch_status();
 }
 
@@ -594,11 +609,13 @@ int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, f
     return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq);
 }
 
-int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const float* q_norm_w,
-                          const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
-                          float* partial_lse, float* partial_max, const float* rope_table,
-                          int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
-                          float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, ptm_stream_t stream) {
+// ptm_attn_decode_fused that can also leave the output as Q8 activation blocks (o_q8, may be NULL) for a Q4_K output
+// projection.  The decode runtime's entry; not declared in the public header.
+int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                             const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8, float* partial_O,
+                             float* partial_lse, float* partial_max, const float* rope_table,
+                             int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                             float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, ptm_stream_t stream) {
     if (!Q || !K || !V || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max ||
         !rope_table || !d_past_len)
         return PTM_E_NULL;
@@ -615,7 +632,19 @@ int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const 
     if (kv_fp16) rc = head_dim == 128 ? attn_launch_g<true, 128>(G, grid, s, a) : attn_launch_g<true, 64>(G, grid, s, a);
     else rc = head_dim == 128 ? attn_launch_g<false, 128>(G, grid, s, a) : attn_launch_g<false, 64>(G, grid, s, a);
     if (rc != PTM_OK) return rc;
-    return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq);
+    if (o_q8 && (reinterpret_cast<uintptr_t>(o_q8) & 15u)) return PTM_E_ALIGN;
+    return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
+                    static_cast<uint8_t*>(o_q8));
+}
+
+int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                          const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
+                          float* partial_lse, float* partial_max, const float* rope_table,
+                          int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                          float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, ptm_stream_t stream) {
+    return ptm_attn_decode_fused_q8(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, nullptr, partial_O, partial_lse,
+                                    partial_max, rope_table, n_heads, n_kv_heads, head_dim, d_past_len, max_seq, scale,
+                                    eps, add_one, kv_fp16, rope_interleaved, stream);
 }
 
 }  // extern "C"

@@ -557,3 +557,38 @@ def test_q6k_long_rows_few_rows_vs_oracle(dev, po, N, K, accumulate):
     pad = np.full((N, W.shape[1] + 210), 0x5A, np.uint8)
     pad[:, :W.shape[1]] = W
     assert np.array_equal(gpu_gemv(14, pad, x), gpu_gemv(14, W, x))
+
+
+@pytest.mark.parametrize("nh,nkv,hd,past", [(32, 8, 128, 2100), (4, 2, 64, 19), (16, 2, 64, 63)])
+def test_attn_decode_fused_q8_output_is_the_quantised_fp32_output(dev, nh, nkv, hd, past):
+    """The decoder's internal attention entry also leaves the output as Q8 activation blocks for a Q4_K output
+    projection: bit-identical to quantising the fp32 output with the stand-alone quantiser."""
+    import ctypes as C
+    from prometorch_amd import _lib
+    L = _lib.load()
+    fn = L.ptm_attn_decode_fused_q8
+    vp = C.c_void_p
+    fn.restype = C.c_int
+    fn.argtypes = [vp] * 13 + [C.c_int, C.c_int, C.c_int, vp, C.c_int, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int, vp]
+    max_seq = ((past + 1 + 63) // 64 + 1) * 64
+    r = synth.rng_for(49, nh, hd, past)
+    kvd, qd = nkv * hd, nh * hd
+    Kc = cu(r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16))
+    Vc = cu(r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16))
+    S = ops.flash_decode_num_splits(max_seq)
+    pO, pL, pM = torch.empty(S * qd, device="cuda"), torch.empty(S * nh, device="cuda"), torch.empty(S * nh, device="cuda")
+    table = ops.rope_table(max_seq, hd, 1e6).cuda()
+    O = torch.empty(qd, device="cuda")
+    q8 = torch.zeros(ops.q8_bytes(qd), dtype=torch.uint8, device="cuda")
+    d_past = torch.full((1,), past, dtype=torch.int64, device="cuda")
+    Q, K, V = cu(synth.make_x(r, qd) * 3), cu(synth.make_x(r, kvd) * 3), cu(synth.make_x(r, kvd))
+    qw, kw = cu(1 + 0.1 * synth.make_x(r, hd)), cu(1 + 0.1 * synth.make_x(r, hd))
+    p = lambda t: t.data_ptr()
+    rc = fn(p(Q), p(K), p(V), p(qw), p(kw), p(Kc), p(Vc), p(O), p(q8), p(pO), p(pL), p(pM), p(table), nh, nkv, hd,
+            p(d_past), max_seq, 1.0 / np.sqrt(hd), 1e-6, 0, 1, 0, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    want = torch.zeros_like(q8)
+    ops.launch_quantize_q8(O, want, qd)
+    torch.cuda.synchronize()
+    assert torch.equal(q8, want)
