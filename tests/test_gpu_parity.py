@@ -592,3 +592,29 @@ def test_attn_decode_fused_q8_output_is_the_quantised_fp32_output(dev, nh, nkv, 
     ops.launch_quantize_q8(O, want, qd)
     torch.cuda.synchronize()
     assert torch.equal(q8, want)
+
+
+def test_gemv_random_shapes_vs_oracle(dev, po):
+    """A fixed pseudo-random sweep over row counts, row lengths, formats and store modes: every launch rule (lane
+    groups per row, blocks per pass, rolling passes, the one-workgroup-per-CU kernel, the plain formats) is met by
+    shapes nobody picked by hand."""
+    r = np.random.default_rng(20251125)
+    worst = {}
+    for case in range(48):
+        qt = int(r.choice([12, 12, 14, 14, 13, 8, 6]))
+        K = int(r.integers(1, 65)) * 256 if case % 3 else int(r.choice([256, 2560, 4096, 9728, 14336]))
+        N = int(r.integers(1, 6000)) if case % 4 else int(r.choice([1, 31, 32, 33, 2560, 4096]))
+        accumulate = bool(r.integers(0, 2))
+        rr = synth.rng_for(36, case)
+        W = synth.make_weight(rr, qt, N, K)
+        x = synth.make_x(rr, K)
+        ref = po.gemv(qt, W, x)
+        if accumulate:
+            y0 = synth.make_x(rr, N)
+            y = gpu_gemv(qt, W, x, accumulate=True, y0=y0) - y0
+            e = float(np.abs(y - ref).max() / max(np.sqrt((ref.astype(np.float64) ** 2).mean()), np.abs(y0).max(), 1e-30))
+        else:
+            e = rel_err(gpu_gemv(qt, W, x), ref)
+        worst[qt] = max(worst.get(qt, 0.0), e)
+        assert e <= GEMV_TOL * 1e-1, (case, qt, N, K, accumulate, e)
+    print("worst rel err per type:", {k: "%.1e" % v for k, v in worst.items()})

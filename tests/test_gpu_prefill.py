@@ -464,3 +464,27 @@ def test_qwen3_4b_shape_prefill_64_tokens(dev, po, seeds):
         check_kv_rows(dec.v_cache[li][:64].float().cpu().numpy(), om.v_cache[li][:64], li, "v")
     follow(dec, om, tok_o, 8)
     dec.close()
+
+
+def test_qgemm_f16_random_shapes_vs_oracle(dev, po):
+    """A fixed pseudo-random sweep of the fast prefill GEMM over row counts (both tile heights, ragged last tiles),
+    widths and lengths (split and unsplit K), both weight types, against the oracle's row-by-row GEMVs."""
+    r = np.random.default_rng(20251126)
+    worst = 0.0
+    for case in range(12):
+        qt = int(r.choice([12, 14]))
+        M = int(r.integers(1, 400)) if case % 3 else int(r.choice([1, 64, 65, 128, 129, 256, 257]))
+        K = int(r.integers(1, 17)) * 256
+        N = int(r.integers(1, 1600))
+        rr = synth.rng_for(72, case)
+        W = synth.make_weight(rr, qt, N, K)
+        x = rr.standard_normal((M, K), dtype=np.float32)
+        ref = np.stack([po.gemv(qt, W, x[m]) for m in range(M)])
+        ws = torch.empty(ops.qgemm_f16_f32_workspace_bytes(M, K, N), dtype=torch.uint8, device="cuda")
+        Y = torch.full((M, N), -3.0, device="cuda")
+        ops.matmul_q_f16_f32(qt, cu(W), cu(x), Y, M, K, N, W.shape[1], ws)
+        torch.cuda.synchronize()
+        e = float(np.abs(Y.cpu().numpy() - ref).max() / np.sqrt((ref.astype(np.float64) ** 2).mean()))
+        worst = max(worst, e)
+        assert e <= PREFILL_TOL, (case, qt, M, K, N, e)
+    print("worst error / rms(y): %.2e" % worst)
