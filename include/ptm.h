@@ -234,6 +234,11 @@ int ptm_mt19937_uniforms(uint32_t seed, int64_t skip, int64_t n, float* out_host
 /* out = a + b; out = in. launch_add / launch_copy (CUDAOps.h:63, :83). */
 int ptm_add(const float* a, const float* b, float* out, int64_t n, ptm_stream_t stream);
 int ptm_copy(const float* in, float* out, int64_t n, ptm_stream_t stream);
+/* The q / k / v projection biases of a qwen2-style layer: Q[r][:] += q_bias, K[r][:] += k_bias, V[r][:] += v_bias for
+ * `rows` rows of q_dim / kv_dim / kv_dim values, in one launch where the reference issues three launch_add calls
+ * (gguf_model.h:2768-2779; CPU path :3413-3438): one fp32 add per element, before QK-norm and rotation. */
+int ptm_add_qkv_bias(float* Q, float* K, float* V, const float* q_bias, const float* k_bias, const float* v_bias, int rows,
+                     int q_dim, int kv_dim, ptm_stream_t stream);
 
 /* Measurement aid with no counterpart in the reference: a pure streaming read of `bytes` (a multiple of 16, 16-byte
  * aligned) with 16-byte loads.  out_partials[i], i < ptm_stream_read_partials(bytes), receives the XOR of all 32-bit
@@ -306,6 +311,8 @@ typedef struct {
     ptm_qweight q, k, v, o, gate, up, down;
     const float *attn_norm, *ffn_norm, *q_norm, *k_norm; /* device fp32; q_norm and k_norm both NULL: no QK-norm */
     void *k_cache, *v_cache; /* device [max_seq][kv_dim], fp16 or fp32 per kv_fp16 */
+    const float *q_bias, *k_bias, *v_bias; /* device fp32 [q_dim], [kv_dim], [kv_dim] (qwen2; LayerWeights::attn_*_bias,
+                                            * gguf_model.h:410-412); all three or all NULL */
 } ptm_layer;
 
 typedef struct {
@@ -394,7 +401,8 @@ int ptm_gguf_get_array(const ptm_gguf* g, const char* key, uint32_t* elem_type, 
 int ptm_gguf_array_string(const ptm_gguf* g, const char* key, int64_t i, const char** data, int64_t* len);
 const void* ptm_gguf_array_data(const ptm_gguf* g, const char* key);
 
-/* From a .gguf file to a ready decoder: reads the `qwen3` or `llama` (no QK-norm tensors, interleaved rotation
+/* From a .gguf file to a ready decoder: reads the `qwen3`, `qwen2` (no QK-norm tensors; blk.N.attn_{q,k,v}.bias
+ * vectors where the file has them, gguf_model.h:6750-6754) or `llama` (no QK-norm tensors, interleaved rotation
  * pairs: gguf_model.h:202-217) hyper-parameters
  * (<arch>.block_count, embedding_length, feed_forward_length, attention.head_count(_kv),
  * attention.key_length, rope.freq_base, attention.layer_norm_rms_epsilon; gguf_model.h:126-181),
@@ -402,7 +410,7 @@ const void* ptm_gguf_array_data(const ptm_gguf* g, const char* key);
  * output.weight (or the tied token_embd.weight) verbatim (gguf_model.h:1177-1360), norm vectors as
  * fp32, allocates zeroed KV caches for max_seq positions and creates the decode runtime.
  * Matrices may be of any type the GEMV dispatcher takes (Q4_K, Q6_K: the tuned path; Q5_K, Q8_0, Q5_0: plain
- * kernels); other architectures, biases and other types: PTM_E_UNSUPPORTED. */
+ * kernels); other architectures and other types: PTM_E_UNSUPPORTED. */
 typedef struct ptm_model ptm_model;
 int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_graph, ptm_model** out);
 ptm_decoder* ptm_model_decoder(ptm_model* m); /* owned by the model */

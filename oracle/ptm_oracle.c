@@ -579,6 +579,10 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
         qgemv(&L->q, xn, qb);
         qgemv(&L->k, xn, kb);
         qgemv(&L->v, xn, vb);
+        if (L->q_bias) { /* gguf_model.h:3413-3438: one fp32 add per element, before the per-head norm */
+            for (int64_t j = 0; j < qd; ++j) qb[j] += L->q_bias[j];
+            for (int64_t j = 0; j < kvd; ++j) { kb[j] += L->k_bias[j]; vb[j] += L->v_bias[j]; }
+        }
         if (L->q_norm) { /* QK-norm only where the model has it (gguf_model.h:3441-3450) */
             for (int64_t h = 0; h < nh; ++h) po_rmsnorm_vec(qb + h * hd, L->q_norm, m->eps, 0, hd, qb + h * hd);
             for (int64_t h = 0; h < nkv; ++h) po_rmsnorm_vec(kb + h * hd, L->k_norm, m->eps, 0, hd, kb + h * hd);

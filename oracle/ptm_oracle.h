@@ -91,6 +91,7 @@ typedef struct {
     po_qweight q, k, v, o, gate, up, down;
     const float *attn_norm, *ffn_norm, *q_norm, *k_norm; /* q_norm, k_norm: NULL for models without QK-norm */
     float *k_cache, *v_cache; /* [max_seq][kv_dim] fp32 storage */
+    const float *q_bias, *k_bias, *v_bias; /* added to the projections' outputs (qwen2); all three or all NULL */
 } po_layer;
 
 typedef struct {

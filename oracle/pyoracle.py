@@ -34,7 +34,8 @@ class QW(C.Structure):
 
 class Layer(C.Structure):
     _fields_ = [(n, QW) for n in ("q", "k", "v", "o", "gate", "up", "down")] + \
-               [(n, _vp) for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "k_cache", "v_cache")]
+               [(n, _vp) for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "k_cache", "v_cache",
+                                   "q_bias", "k_bias", "v_bias")]
 
 
 class Model(C.Structure):
@@ -255,7 +256,8 @@ class OracleModel:
     """Host-side model for po_decode_step; keeps every numpy buffer alive."""
 
     def __init__(self, cfg: dict, layers: list, head: dict, max_seq: int, kv_fp16: bool, embedding=None):
-        """cfg may carry 'rope_interleaved' (llama-style rotation pairs); layers without 'q_norm' / 'k_norm' have no QK-norm."""
+        """cfg may carry 'rope_interleaved' (llama-style rotation pairs); layers without 'q_norm' / 'k_norm' have no QK-norm;
+        layers with 'q_bias', 'k_bias', 'v_bias' add them to the projections (qwen2)."""
         self.cfg = cfg
         self._keep = []
         kvd = cfg["n_kv_heads"] * cfg["head_dim"]
@@ -267,7 +269,7 @@ class OracleModel:
                 qw, Wc = _qw(qt, W)
                 self._keep.append(Wc)
                 setattr(self.layers[i], name, qw)
-            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias"):
                 if L.get(name) is None:
                     setattr(self.layers[i], name, None)
                     continue
@@ -406,7 +408,7 @@ class RefModel:
                 self._keep.append(W)
                 K = W.shape[1] // BLOCK[qt][0] * BLOCK[qt][1]
                 R.ref_model_set_weight(self.h, i, w, _p(W), qt, W.shape[0], K)
-            for w, name in enumerate(("attn_norm", "ffn_norm", "q_norm", "k_norm")):
+            for w, name in enumerate(("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias")):
                 if L.get(name) is None:
                     continue
                 a = np.ascontiguousarray(L[name], np.float32)

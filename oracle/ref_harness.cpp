@@ -149,12 +149,13 @@ void ref_model_set_weight(void* h, int64_t layer, int which, const void* data, u
                                         &L.q_ffn_gate, &L.q_ffn_up, &L.q_ffn_down};
     set_qw(*w[which], data, type, rows, cols);
 }
-// which: 0 attn_norm, 1 ffn_norm, 2 q_norm, 3 k_norm
+// which: 0 attn_norm, 1 ffn_norm, 2 q_norm, 3 k_norm, 4 / 5 / 6 attn_q / attn_k / attn_v bias (gguf_model.h:410-412)
 void ref_model_set_norm(void* h, int64_t layer, int which, const float* gamma, int64_t n) {
     auto& L = static_cast<RefModel*>(h)->m.layers[layer];
     at::Tensor t = vec_tensor(gamma, n);
     if (which == 0) L.attn_norm = t; else if (which == 1) L.ffn_norm = t;
-    else if (which == 2) L.attn_q_norm = t; else L.attn_k_norm = t;
+    else if (which == 2) L.attn_q_norm = t; else if (which == 3) L.attn_k_norm = t;
+    else if (which == 4) L.attn_q_bias = t; else if (which == 5) L.attn_k_bias = t; else L.attn_v_bias = t;
 }
 void ref_model_set_output(void* h, const float* out_norm, const void* lm_head, uint32_t type) {
     auto& m = static_cast<RefModel*>(h)->m;

@@ -35,7 +35,8 @@ class QWeight(C.Structure):
 
 class Layer(C.Structure):
     _fields_ = [(n, QWeight) for n in ("q", "k", "v", "o", "gate", "up", "down")] + \
-               [(n, vp) for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "k_cache", "v_cache")]
+               [(n, vp) for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "k_cache", "v_cache",
+                                  "q_bias", "k_bias", "v_bias")]
 
 
 class DecodeConfig(C.Structure):
@@ -97,6 +98,7 @@ SIGNATURES = {
     "ptm_embedding_row_q6k": (i32, [vp, vp, vp, i32, i64, vp]),
     "ptm_argmax": (i32, [vp, vp, i64, vp]),
     "ptm_add": (i32, [vp, vp, vp, i64, vp]),
+    "ptm_add_qkv_bias": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp]),
     "ptm_copy": (i32, [vp, vp, i64, vp]),
     "ptm_stream_read_partials": (i64, [i64]),
     "ptm_stream_read_xor": (i32, [vp, i64, vp, vp]),

@@ -179,6 +179,7 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
                 if (n4 > 0) PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->x, false, L.attn_norm, c.rms_eps, 0, H, s4, false, s));
             }
         }
+        if (L.q_bias) PTM_TRY(ptm_add_qkv_bias(d->q, d->k, d->v, L.q_bias, L.k_bias, L.v_bias, 1, c.n_heads * hd, c.n_kv_heads * hd, s));
         // QK-norm + RoPE + K/V append + split-KV attention in one launch, plus the small merge launch
         // a Q4_K output projection takes the attention output as the Q8 blocks the merge kernel leaves beside the fp32
         // vector: its prologue then copies 1.25 bytes per value instead of fetching and quantising 4
@@ -303,6 +304,7 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
         PTM_TRY(gemm(L.q, d->pf_x, d->pf_q, false, true));
         PTM_TRY(gemm(L.k, d->pf_x, d->pf_k, false, true));
         PTM_TRY(gemm(L.v, d->pf_x, d->pf_v, false, true));
+        if (L.q_bias) PTM_TRY(ptm_add_qkv_bias(d->pf_q, d->pf_k, d->pf_v, L.q_bias, L.k_bias, L.v_bias, M, qd, kvd, s));
         PTM_TRY(ptm_qknorm_rope_kvwrite_rows(d->pf_q, d->pf_k, d->pf_v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->rope, M,
                                              c.n_heads, c.n_kv_heads, hd, pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, s));
         PTM_TRY(ptm_prefill_attention(d->pf_q, L.k_cache, L.v_cache, d->pf_attn, M, c.n_heads, c.n_kv_heads, hd, pos0,
@@ -341,6 +343,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
         const ptm_layer& L = c.layers[i];
         if (!L.attn_norm || !L.ffn_norm || !L.k_cache || !L.v_cache) return PTM_E_NULL;
         if ((L.q_norm == nullptr) != (L.k_norm == nullptr)) return PTM_E_NULL;  // QK-norm: both or neither
+        if ((L.q_bias == nullptr) != (L.k_bias == nullptr) || (L.q_bias == nullptr) != (L.v_bias == nullptr)) return PTM_E_NULL;
         if ((rc = qw_check(L.q, qd, H)) || (rc = qw_check(L.k, kvd, H)) || (rc = qw_check(L.v, kvd, H)) ||
             (rc = qw_check(L.o, H, qd)) || (rc = qw_check(L.gate, c.inter, H)) || (rc = qw_check(L.up, c.inter, H)) ||
             (rc = qw_check(L.down, H, c.inter)))

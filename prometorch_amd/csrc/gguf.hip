@@ -382,11 +382,12 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
     const char* arch_c = ptm_gguf_get_string(m->file, "general.architecture");
     if (!arch_c) { ptm_model_free(m); return PTM_E_FORMAT; }
     const std::string arch = arch_c;
-    // two decode steps are built here, both RMSNorm + SwiGLU without biases: qwen3 (per-head QK-norm, rotation pairs
-    // half a head apart) and llama, which mistral files also carry (no QK-norm, interleaved pairs (2d, 2d+1));
-    // gguf_model.h:202-217 makes the same split by architecture name
+    // three decode steps are built here, all RMSNorm + SwiGLU: qwen3 (per-head QK-norm, rotation pairs half a head
+    // apart), qwen2 (no QK-norm, the same pairs, bias vectors on q / k / v) and llama, which mistral files also carry
+    // (no QK-norm, interleaved pairs (2d, 2d+1)); gguf_model.h:194-217 makes the same split by architecture name
     const bool is_llama = arch == "llama";
-    if (arch != "qwen3" && !is_llama) { ptm_model_free(m); return PTM_E_UNSUPPORTED; }
+    const bool has_qk_norm = arch == "qwen3";
+    if (arch != "qwen3" && arch != "qwen2" && !is_llama) { ptm_model_free(m); return PTM_E_UNSUPPORTED; }
     auto geti = [&](const char* key, int64_t def, bool required) -> int64_t {
         int64_t v = def;
         const int r = ptm_gguf_get_int(m->file, (arch + "." + key).c_str(), &v);
@@ -453,13 +454,17 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
         ptm_layer& L = m->layers[(size_t)i];
         const std::string p = "blk." + std::to_string(i) + ".";
         ptm_gguf_tensor bias{};
-        if (ptm_gguf_find_tensor(m->file, (p + "attn_q.bias").c_str(), &bias) == PTM_OK) { ptm_model_free(m); return PTM_E_UNSUPPORTED; }
+        if (ptm_gguf_find_tensor(m->file, (p + "attn_q.bias").c_str(), &bias) == PTM_OK) {  // gguf_model.h:6750-6754
+            PTM_L(load_vector(m, p + "attn_q.bias", qd, &L.q_bias));
+            PTM_L(load_vector(m, p + "attn_k.bias", kvd, &L.k_bias));
+            PTM_L(load_vector(m, p + "attn_v.bias", kvd, &L.v_bias));
+        }
         PTM_L(load_vector(m, p + "attn_norm.weight", c.hidden, &L.attn_norm));
         PTM_L(load_matrix(m, p + "attn_q.weight", qd, c.hidden, &L.q));
         PTM_L(load_matrix(m, p + "attn_k.weight", kvd, c.hidden, &L.k));
         PTM_L(load_matrix(m, p + "attn_v.weight", kvd, c.hidden, &L.v));
         PTM_L(load_matrix(m, p + "attn_output.weight", c.hidden, qd, &L.o));
-        if (is_llama) {
+        if (!has_qk_norm) {
             L.q_norm = nullptr;
             L.k_norm = nullptr;
         } else {

@@ -237,6 +237,21 @@ __global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, c
     if (i < n) o[i] = a[i] + b[i];
 }
 
+// Q[r][j] += bq[j], K[r][j] += bk[j], V[r][j] += bv[j] for `rows` rows in one launch (element e of a row of
+// q_dim + 2 kv_dim values picks its segment)
+__global__ __launch_bounds__(256) void qkv_bias_kernel(float* __restrict__ Q, float* __restrict__ K, float* __restrict__ V,
+                                                       const float* __restrict__ bq, const float* __restrict__ bk,
+                                                       const float* __restrict__ bv, int64_t rows, int q_dim, int kv_dim) {
+    const int w = q_dim + 2 * kv_dim;
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= rows * w) return;
+    const int64_t r = e / w;
+    const int j = (int)(e - r * w);
+    if (j < q_dim) Q[r * q_dim + j] += bq[j];
+    else if (j < q_dim + kv_dim) K[r * kv_dim + (j - q_dim)] += bk[j - q_dim];
+    else V[r * kv_dim + (j - q_dim - kv_dim)] += bv[j - q_dim - kv_dim];
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ a, float* __restrict__ o, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) o[i] = a[i];
@@ -488,6 +503,17 @@ int ptm_add(const float* a, const float* b, float* out, int64_t n, ptm_stream_t 
     if (n < 0) return PTM_E_SHAPE;
     if (n == 0) return PTM_OK;
     hipLaunchKernelGGL(add_kernel, dim3(nblk256(n)), dim3(256), 0, as_stream(stream), a, b, out, n);
+    return launch_status();
+}
+
+int ptm_add_qkv_bias(float* Q, float* K, float* V, const float* q_bias, const float* k_bias, const float* v_bias, int rows,
+                     int q_dim, int kv_dim, ptm_stream_t stream) {
+    if (!Q || !K || !V || !q_bias || !k_bias || !v_bias) return PTM_E_NULL;
+    if (rows < 0 || q_dim <= 0 || kv_dim <= 0) return PTM_E_SHAPE;
+    if (rows == 0) return PTM_OK;
+    const int64_t n = (int64_t)rows * (q_dim + 2 * (int64_t)kv_dim);
+    hipLaunchKernelGGL(qkv_bias_kernel, dim3(nblk256(n)), dim3(256), 0, as_stream(stream), Q, K, V, q_bias, k_bias, v_bias,
+                       (int64_t)rows, q_dim, kv_dim);
     return launch_status();
 }
 

@@ -24,7 +24,8 @@ class Decoder:
     """Greedy batch-1 decoder over caller-provided quantised weights.
 
     layers: list of dicts with (qtype, uint8[rows, stride]) per projection name and fp32 norm
-    vectors 'attn_norm', 'ffn_norm', 'q_norm', 'k_norm' (the last two None for a model without QK-norm;
+    vectors 'attn_norm', 'ffn_norm', 'q_norm', 'k_norm' (the last two None for a model without QK-norm; optional
+    'q_bias', 'k_bias', 'v_bias' added to the projections' outputs;
     cfg['rope_interleaved'] selects llama-style rotation pairs); head: {'lm_head': uint8 table (Q6_K unless 'lm_head_type' says otherwise),
     'out_norm': fp32}.  The token-embedding is the tied Q6_K table unless embedding_f32 is given."""
 
@@ -46,8 +47,8 @@ class Decoder:
                 t = _upload_bytes(W)
                 self._keep.append(t)
                 setattr(arr[i], name, QWeight(t.data_ptr(), qt, W.shape[0], _lib.weight_cols(qt, W.shape[1]), W.shape[1]))
-            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
-                if Ld.get(name) is None:  # q_norm / k_norm: a model without QK-norm
+            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias"):
+                if Ld.get(name) is None:  # q_norm / k_norm: a model without QK-norm; biases: qwen2-style only
                     setattr(arr[i], name, None)
                     continue
                 t = torch.from_numpy(np.ascontiguousarray(Ld[name], np.float32)).cuda()

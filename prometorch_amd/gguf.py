@@ -99,6 +99,10 @@ def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "q
         if L.get("q_norm") is not None:  # absent in a llama-style model
             ts.append((p + "attn_q_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["q_norm"], np.float32)))
             ts.append((p + "attn_k_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["k_norm"], np.float32)))
+        for k in ("q", "k", "v"):
+            if L.get(k + "_bias") is not None:  # qwen2-style projections
+                b = np.asarray(L[k + "_bias"], np.float32)
+                ts.append((p + f"attn_{k}.bias", F32, [b.size], b))
         ts.append((p + "ffn_norm.weight", F32, [H], np.asarray(L["ffn_norm"], np.float32)))
     write_gguf(path, md, ts, alignment=alignment)
 

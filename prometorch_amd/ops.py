@@ -285,6 +285,12 @@ def launch_add(a, b, out, n, stream=None):
     check(_L().ptm_add(_ptr(a), _ptr(b), _ptr(out), n, _stream(stream)), "add")
 
 
+def add_qkv_bias(Q, K, V, q_bias, k_bias, v_bias, rows, q_dim, kv_dim, stream=None):
+    """The three launch_add calls of a qwen2-style layer (gguf_model.h:2768-2779) as one launch, for `rows` rows."""
+    check(_L().ptm_add_qkv_bias(_ptr(Q), _ptr(K), _ptr(V), _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), rows, q_dim, kv_dim,
+                                _stream(stream)), "add_qkv_bias")
+
+
 def launch_copy(input, output, n, stream=None):
     """CUDAOps.h:83"""
     check(_L().ptm_copy(_ptr(input), _ptr(output), n, _stream(stream)), "copy")

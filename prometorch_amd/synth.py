@@ -269,6 +269,23 @@ def tiny_llama(seed: int):
     return cfg, layers, make_head(seed, cfg)
 
 
+def tiny_qwen2(seed: int):
+    """The TINY shapes as a qwen2-style model: no per-head QK-norm, NeoX rotation pairs, and bias vectors on the q, k and
+    v projections (N(0,1) scaled to the size of the projections' outputs, so that dropping one changes the tokens).
+    Attention-input norm gains reduced as in tiny_llama."""
+    cfg = dict(TINY)
+    layers = [make_layer(seed, i, cfg) for i in range(cfg["n_layers"])]
+    qd, kvd = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    for i, L in enumerate(layers):
+        L["q_norm"] = None
+        L["k_norm"] = None
+        L["attn_norm"] = (np.float32(0.1) * L["attn_norm"]).astype(np.float32)
+        g = rng_for(seed, 5, i)
+        for name, n in (("q_bias", qd), ("k_bias", kvd), ("v_bias", kvd)):
+            L[name] = (np.float32(0.5) * g.standard_normal(n, dtype=np.float32)).astype(np.float32)
+    return cfg, layers, make_head(seed, cfg)
+
+
 # ---- sampling cases: (vocab, logit kind, temperature, top_k, top_p), in the order the golden run draws them ----
 SAMPLING_CASES = (
     [(1000, "normal", 0.8, 40, 0.9), (1000, "normal", 1.0, 0, 1.0), (1000, "normal", 0.7, 1, 1.0),

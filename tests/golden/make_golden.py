@@ -82,6 +82,7 @@ def main():
     ap.add_argument("--full", action="store_true")
     ap.add_argument("--sampling-only", action="store_true", help="write golden_sampling.npz and nothing else")
     ap.add_argument("--tokenizer-only", action="store_true", help="write golden_tokenizer.json and nothing else")
+    ap.add_argument("--qwen2-only", action="store_true", help="write golden_qwen2.npz and nothing else")
     ap.add_argument("--llama-only", action="store_true", help="write golden_llama.npz and nothing else")
     ap.add_argument("--mixed-only", action="store_true", help="write golden_mixed.npz and nothing else")
     ap.add_argument("--formats-only", action="store_true", help="write golden_formats.npz and nothing else")
@@ -94,6 +95,10 @@ def main():
     if args.tokenizer_only:
         make_tokenizer_golden()
         print("wrote golden_tokenizer.json")
+        return
+    if args.qwen2_only:
+        make_qwen2_golden()
+        print("wrote golden_qwen2.npz")
         return
     if args.llama_only:
         make_llama_golden()
@@ -230,6 +235,7 @@ def main():
     make_sampling()
     make_tokenizer_golden()
     make_llama_golden()
+    make_qwen2_golden()
     make_formats_golden()
     make_mixed_golden()
 
@@ -382,6 +388,24 @@ def make_llama_golden():
     R.ref_rope_apply_norm(q.ctypes.data, k.ctypes.data, c.ctypes.data, s.ctypes.data, 32, 8, 128)
     g["rope_norm_q"], g["rope_norm_k"] = q, k
     np.savez_compressed(os.path.join(OUT, "golden_llama.npz"), **g)
+
+
+def make_qwen2_golden():
+    """The reference's forward_decode_cpu on a qwen2-style tiny model (synth.tiny_qwen2): q / k / v biases, no QK-norm,
+    NeoX rotation; 12 greedy steps after a 19-position cache."""
+    cfg, layers, head = synth.tiny_qwen2(SEEDS["tiny"])
+    emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    rm = po.RefModel(cfg, layers, head, 64, emb)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(SEEDS["tiny"], i, cfg, 19)
+        rm.set_kv(i, k, v)
+    tok, toks, lg = 3, [], []
+    for _ in range(12):
+        tok = rm.step(tok)
+        toks.append(tok)
+        lg.append(rm.logits.copy())
+    rm.close()
+    np.savez_compressed(os.path.join(OUT, "golden_qwen2.npz"), tokens=np.array(toks, np.int64), logits=np.stack(lg))
 
 
 def make_full(meta):

@@ -71,6 +71,25 @@ def test_model_file_has_the_reference_tensor_names(tmp_path):
         assert t["type"] == qt and t["dims"] == [cfg["inter"], cfg["hidden"]] and np.array_equal(t["data"], W.reshape(-1))
 
 
+def test_qwen2_model_file_carries_the_bias_vectors(tmp_path):
+    """blk.N.attn_{q,k,v}.bias as F32 vectors, the names the reference looks up (gguf_model.h:6750-6753)."""
+    from prometorch_amd import synth
+    cfg, layers, head = synth.tiny_qwen2(5)
+    path = str(tmp_path / "q2.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head, arch="qwen2")
+    with gguf.GGUFFile(path) as g:
+        assert g.get_string("general.architecture") == "qwen2"
+        assert g.get_int("qwen2.attention.head_count_kv") == cfg["n_kv_heads"]
+        for i in range(cfg["n_layers"]):
+            for k, n in (("q", cfg["n_heads"] * cfg["head_dim"]), ("k", cfg["n_kv_heads"] * cfg["head_dim"]),
+                         ("v", cfg["n_kv_heads"] * cfg["head_dim"])):
+                t = g.tensor(f"blk.{i}.attn_{k}.bias")
+                assert t["type"] == 0 and t["dims"] == [n]
+                assert np.array_equal(t["data"].view(np.float32), layers[i][k + "_bias"])
+        with pytest.raises(Exception):
+            g.tensor("blk.0.attn_q_norm.weight")
+
+
 def test_malformed_files_are_refused(tmp_path):
     good = str(tmp_path / "g.gguf")
     gguf.write_gguf(good, {"general.architecture": "qwen3"}, [("c", gguf.F32, [8], np.zeros(8, np.float32))])

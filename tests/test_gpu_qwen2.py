@@ -1,0 +1,181 @@
+"""GPU parity of the qwen2-style variant of the decode path: bias vectors added to the q / k / v projections before
+the rotation (torch/io/gguf_model.h:2768-2779 on the GPU, :3413-3438 on the CPU), no per-head QK-norm, NeoX rotation
+pairs.  The compiled reference's forward_decode_cpu run of synth.tiny_qwen2 is golden_qwen2.npz.  Bars are those of
+the qwen3-style tests: tokens identical, logits within LOGIT_TOL of the spread (decode), the prefill bars of
+test_gpu_prefill for the prompt path, bit-identical results between a .gguf load and the direct decoder."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import bits
+from prometorch_amd import gguf, ops, synth
+from test_gpu_decode import check_step_errors
+from test_gpu_llama import follow_sensitive
+from test_gpu_prefill import check_kv_rows, check_logits
+
+pytestmark = pytest.mark.gpu
+
+
+def cu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.fixture(scope="module")
+def golden_qwen2():
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_qwen2.npz"))
+
+
+def tiny_qwen2_with_cache(seeds, n=19):
+    cfg, layers, head = synth.tiny_qwen2(seeds["tiny"])
+    kv = [synth.make_kv_prefill(seeds["tiny"], i, cfg, n) for i in range(cfg["n_layers"])]
+    return cfg, layers, head, kv
+
+
+@pytest.mark.parametrize("rows,qd,kvd", [(1, 4096, 1024), (7, 256, 128), (33, 512, 512)])
+def test_add_qkv_bias_is_one_fp32_add_per_element(dev, rows, qd, kvd):
+    r = synth.rng_for(91, rows, qd)
+    Q, K, V = (r.standard_normal((rows, n), dtype=np.float32) for n in (qd, kvd, kvd))
+    bq, bk, bv = (r.standard_normal(n, dtype=np.float32) for n in (qd, kvd, kvd))
+    dQ, dK, dV = cu(Q), cu(K), cu(V)
+    ops.add_qkv_bias(dQ, dK, dV, cu(bq), cu(bk), cu(bv), rows, qd, kvd)
+    for got, want in ((dQ, Q + bq), (dK, K + bk), (dV, V + bv)):
+        assert np.array_equal(bits(got.cpu().numpy()), bits(want))
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_qwen2_decode_fp32_kv_vs_reference_golden(dev, golden_qwen2, seeds, use_graph):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_qwen2_with_cache(seeds)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False, use_graph=use_graph)
+    for i, (k, v) in enumerate(kv):
+        dec.set_kv(i, k, v)
+    dec.set_past_len(19)
+    tok, errs = 3, []
+    for st in range(12):
+        tok = dec.step(tok)
+        ref = golden_qwen2["logits"][st]
+        errs.append(np.abs(dec.logits() - ref).max() / ref.std())
+        assert tok == int(golden_qwen2["tokens"][st]), st
+    check_step_errors(errs)
+    dec.close()
+
+
+def test_qwen2_decode_fp16_kv_vs_oracle_and_chained_greedy(dev, po, seeds):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_qwen2_with_cache(seeds)
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=True)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=True)
+    dec2 = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=True)
+    for i, (k, v) in enumerate(kv):
+        om.set_kv(i, k, v)
+        dec.set_kv(i, k, v)
+        dec2.set_kv(i, k, v)
+    dec.set_past_len(19)
+    dec2.set_past_len(19)
+    tok_o = tok_g = 3
+    want, errs = [], []
+    for st in range(24):
+        tok_o = om.step(tok_o)
+        tok_g = dec.step(tok_g)
+        want.append(tok_o)
+        errs.append(np.abs(dec.logits() - om.logits).max() / om.logits.std())
+        assert tok_g == tok_o, st
+    check_step_errors(errs)
+    assert dec2.greedy(3, 24) == want
+    # the appended K rows carry the k bias, the V rows the v bias
+    for gpu_c, cpu_c in ((dec.k_cache[0], om.k_cache[0]), (dec.v_cache[1], om.v_cache[1])):
+        got, ref = gpu_c[19:43].float().cpu().numpy(), cpu_c[19:43]
+        assert np.abs(got - ref).max() <= 2e-3 * np.abs(ref).max()
+    dec.close()
+    dec2.close()
+
+
+def test_qwen2_biases_are_not_ignored(dev, seeds, golden_qwen2):
+    """The same weights without the bias vectors give other logits at the first step: the golden run exercises them."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_qwen2_with_cache(seeds)
+    bare = [{k: v for k, v in L.items() if not k.endswith("_bias")} for L in layers]
+    dec = Decoder(cfg, bare, head, max_seq=64, kv_fp16=False, use_graph=False)
+    for i, (k, v) in enumerate(kv):
+        dec.set_kv(i, k, v)
+    dec.set_past_len(19)
+    dec.step(3)
+    ref = golden_qwen2["logits"][0]
+    assert np.abs(dec.logits() - ref).max() > 0.05 * ref.std()
+    dec.close()
+
+
+def test_decoder_wants_all_three_biases_or_none(dev, seeds):
+    from prometorch_amd._lib import PtmError
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = synth.tiny_qwen2(seeds["tiny"])
+    bad = [dict(L) for L in layers]
+    bad[1]["v_bias"] = None
+    with pytest.raises(PtmError) as e:
+        Decoder(cfg, bad, head, max_seq=64, kv_fp16=False)
+    assert e.value.code == -1
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+@pytest.mark.parametrize("pos0,n,chunk", [(0, 23, 0), (0, 23, 7), (19, 12, 5)])
+def test_qwen2_prefill_vs_oracle_token_by_token(dev, po, seeds, kv_fp16, pos0, n, chunk):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = synth.tiny_qwen2(seeds["tiny"])
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=kv_fp16)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=kv_fp16, use_graph=True)
+    if pos0:
+        for i in range(cfg["n_layers"]):
+            k, v = synth.make_kv_prefill(seeds["tiny"], i, cfg, pos0)
+            om.set_kv(i, k, v)
+            dec.set_kv(i, k, v)
+        dec.set_past_len(pos0)
+    prompt = [int(t) for t in synth.rng_for(68, pos0, n).integers(0, cfg["vocab"], n)]
+    for t in prompt:
+        tok_o = om.step(t)
+    tok_g = dec.prefill(prompt, chunk_rows=chunk)
+    for li in range(cfg["n_layers"]):
+        for nm, gpu_c, cpu_c in (("k", dec.k_cache[li], om.k_cache[li]), ("v", dec.v_cache[li], om.v_cache[li])):
+            check_kv_rows(gpu_c[pos0:pos0 + n].float().cpu().numpy(), cpu_c[pos0:pos0 + n], li, nm)
+    check_logits(dec.logits(), om.logits, tok_g, tok_o, "prefill")
+    follow_sensitive(dec, om, tok_o, 6)
+    dec.close()
+
+
+def test_qwen2_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_qwen2, tmp_path):
+    """general.architecture = qwen2: blk.N.attn_{q,k,v}.bias vectors loaded, no QK-norm tensors, NeoX rotation."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_qwen2_with_cache(seeds)
+    path = str(tmp_path / "tiny_qwen2.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head, arch="qwen2")
+    f = gguf.GGUFFile(path)
+    assert np.array_equal(f.tensor("blk.1.attn_k.bias")["data"].view(np.float32), layers[1]["k_bias"])
+    f.close()
+    m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
+    assert m.cfg["rope_interleaved"] is False
+    assert m.layer(0).q_bias and m.layer(0).v_bias and not m.layer(0).q_norm
+    d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
+    for i, (k, v) in enumerate(kv):
+        m.set_kv(i, k, v)
+        d.set_kv(i, k, v)
+    m.set_past_len(19)
+    d.set_past_len(19)
+    tm = td = 3
+    for st in range(12):
+        tm = m.step(tm)
+        td = d.step(td)
+        assert tm == td == int(golden_qwen2["tokens"][st]), st
+        assert np.array_equal(bits(m.logits()), bits(d.logits())), st
+    m.close()
+    d.close()
+    # a file with only two of the three bias vectors: missing tensor
+    part = [dict(L) for L in layers]
+    for L in part:
+        L["v_bias"] = None
+    p2 = str(tmp_path / "partial.gguf")
+    gguf.model_to_gguf(p2, cfg, part, head, arch="qwen2")
+    from prometorch_amd._lib import PtmError
+    with pytest.raises(PtmError) as e:
+        gguf.GGUFModel(p2, max_seq=64)
+    assert e.value.code == -10

@@ -237,6 +237,39 @@ def test_llama_style_decode_and_rope_match_the_reference(po, seeds):
     assert np.abs(qr.reshape(32, 64, 2) - want).max() <= 2e-3 * np.abs(want).max()   # fp32 angles of ~2e3 rad
 
 
+def test_qwen2_style_biases_match_the_reference(po, seeds):
+    """q / k / v bias vectors, no QK-norm, NeoX rotation (qwen2): oracle bit-identical to the compiled reference's
+    forward_decode_cpu (golden_qwen2.npz); with any one of the three vectors zeroed the logits differ, so the golden run
+    does exercise each of them."""
+    import os
+    from prometorch_amd import synth
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_qwen2.npz"))
+    cfg, layers, head = synth.tiny_qwen2(seeds["tiny"])
+
+    def run(layers, steps):
+        om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)
+        for i in range(cfg["n_layers"]):
+            k, v = synth.make_kv_prefill(seeds["tiny"], i, cfg, 19)
+            om.set_kv(i, k, v)
+        tok, toks, lg = 3, [], []
+        for _ in range(steps):
+            tok = om.step(tok)
+            toks.append(tok)
+            lg.append(om.logits.copy())
+        return toks, np.stack(lg)
+
+    toks, lg = run(layers, 12)
+    assert toks == [int(t) for t in g["tokens"]]
+    assert np.array_equal(lg.view(np.uint32), g["logits"].view(np.uint32))
+    sigma = float(g["logits"][0].std())
+    for drop in ("q_bias", "k_bias", "v_bias"):
+        alt = [dict(L) for L in layers]
+        for L in alt:
+            L[drop] = np.zeros_like(L[drop])
+        _, l1 = run(alt, 1)
+        assert np.abs(l1[0] - g["logits"][0]).max() > 1e-2 * sigma, drop
+
+
 @pytest.mark.parametrize("maker,fname", [("tiny_mixed", "golden_mixed.npz"), ("tiny_formats", "golden_formats_model.npz")])
 def test_mixed_type_layers_match_the_reference(po, seeds, maker, fname):
     """Layers whose q/k/v share a type (the reference fuses them behind its 8-lane norm) beside layers where they do
