@@ -165,6 +165,9 @@ int ptm_qknorm_rope_kvwrite(float* Q, float* K, const float* V, const float* q_n
 /* Host-side helper: fill table[max_seq][head_dim] with the reference's fp32 cos/sin
  * (hot_loops.cpp:1853-1876: freq = 1/powf(base, 2d/hd), theta = pos*freq). table is a HOST pointer. */
 int ptm_rope_table_host(float* table, int max_seq, int head_dim, float rope_freq_base);
+/* The same with linear position scaling: theta = (pos / scale) * freq when scale is positive and not 1
+ * (the `scale` argument of rope_precompute, hot_loops.cpp:1853-1860; ModelConfig::rope_scale, gguf_model.h:71). */
+int ptm_rope_table_host_scaled(float* table, int max_seq, int head_dim, float rope_freq_base, float scale);
 /* fp32 rows -> fp16 cache rows. launch_fp16_kv_cache_write (CUDAOps.h:635-638). */
 int ptm_fp16_kv_cache_write(const float* src, void* dst_cache_fp16, int64_t num_new_rows, int64_t cols,
                             int64_t offset_row, ptm_stream_t stream);
@@ -325,6 +328,7 @@ typedef struct {
     const float* out_norm;        /* device */
     ptm_qweight lm_head;
     int32_t rope_interleaved;     /* 0: NeoX rotation pairs (qwen3); 1: pairs (2d, 2d+1) (llama, mistral) */
+    float rope_scale;             /* linear position scaling, theta = (pos / rope_scale) * freq (gguf_model.h:71); 0 or 1: none */
 } ptm_decode_config;
 
 typedef struct ptm_decoder ptm_decoder;

@@ -432,7 +432,11 @@ void po_rmsnorm_vec(const float* x, const float* gamma, float eps, int add_one, 
 
 /* ---- RoPE (reference: hot_loops.cpp:1853-1876, :2035-2061) ----------------------- */
 void po_rope_precompute(float* c, float* s, int64_t pos, int64_t head_dim, float base) {
-    const float p = (float)pos;
+    po_rope_precompute_scaled(c, s, pos, head_dim, base, 1.0f);
+}
+/* linear position scaling: theta = (pos / scale) * freq when scale is positive and not 1 (hot_loops.cpp:1858-1860) */
+void po_rope_precompute_scaled(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale) {
+    const float p = (scale > 0.0f && scale != 1.0f) ? (float)pos / scale : (float)pos;
     for (int64_t d = 0; d < head_dim / 2; ++d) {
         const float inv = 1.0f / powf(base, 2.0f * (float)d / (float)head_dim);
         const float th = p * inv;
@@ -568,7 +572,7 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
     else po_dequantize_q6_k((const uint8_t*)m->lm_head.data + token * m->lm_head.stride, x, H);
 
     float rc[256], rs[256];
-    po_rope_precompute(rc, rs, past, hd, m->rope_base);
+    po_rope_precompute_scaled(rc, rs, past, hd, m->rope_base, m->rope_scale);
     const float scale = 1.0f / sqrtf((float)hd);
 
     for (int64_t li = 0; li < m->n_layers; ++li) {

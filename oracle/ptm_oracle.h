@@ -71,6 +71,7 @@ void po_q4k_row_isums(const void* row, const int8_t* qs, int64_t K, int32_t* isu
 void po_rmsnorm_seq(const float* x, const float* gamma, float eps, int add_one, int64_t H, float* out);
 void po_rmsnorm_vec(const float* x, const float* gamma, float eps, int add_one, int64_t H, float* out);
 void po_rope_precompute(float* c, float* s, int64_t pos, int64_t head_dim, float base);
+void po_rope_precompute_scaled(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale);
 void po_rope_apply_norm(float* q, float* k, const float* c, const float* s, int64_t n_heads, int64_t n_kv_heads,
                         int64_t head_dim);
 void po_rope_apply_neox(float* q, float* k, const float* c, const float* s,
@@ -104,6 +105,7 @@ typedef struct {
     po_qweight lm_head;
     int64_t seq_len;
     int rope_interleaved;   /* 0: NeoX pairs (d, d + half) as qwen / gemma / phi; 1: pairs (2d, 2d + 1) as llama / mistral */
+    float rope_scale;       /* linear position scaling (ModelConfig::rope_scale, gguf_model.h:71); 0 or 1: none */
 } po_model;
 
 /* One decode step (forward_decode_cpu order, Q4_K_M fallbacks); writes logits[vocab],

@@ -41,7 +41,8 @@ class Layer(C.Structure):
 class Model(C.Structure):
     _fields_ = [(n, _i64) for n in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")] + \
                [("rope_base", _f32), ("eps", _f32), ("kv_fp16", _i32), ("embedding", _vp),
-                ("layers", C.POINTER(Layer)), ("out_norm", _vp), ("lm_head", QW), ("seq_len", _i64), ("rope_interleaved", _i32)]
+                ("layers", C.POINTER(Layer)), ("out_norm", _vp), ("lm_head", QW), ("seq_len", _i64), ("rope_interleaved", _i32),
+                ("rope_scale", _f32)]
 
 
 _lib = None
@@ -71,6 +72,7 @@ def lib():
         L.po_rmsnorm_seq.argtypes = [_vp, _vp, _f32, _i32, _i64, _vp]
         L.po_rmsnorm_vec.argtypes = [_vp, _vp, _f32, _i32, _i64, _vp]
         L.po_rope_precompute.argtypes = [_vp, _vp, _i64, _i64, _f32]
+        L.po_rope_precompute_scaled.argtypes = [_vp, _vp, _i64, _i64, _f32, _f32]
         L.po_rope_apply_neox.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
         L.po_rope_apply_norm.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
         L.po_exp256.argtypes = [_vp, _vp, _i64]
@@ -163,10 +165,10 @@ def rmsnorm(x, gamma, eps, seq=False):
     return out
 
 
-def rope_tables(pos, head_dim, base):
+def rope_tables(pos, head_dim, base, scale=1.0):
     c = np.empty(head_dim // 2, np.float32)
     s = np.empty(head_dim // 2, np.float32)
-    lib().po_rope_precompute(_p(c), _p(s), pos, head_dim, base)
+    lib().po_rope_precompute_scaled(_p(c), _p(s), pos, head_dim, base, scale)
     return c, s
 
 
@@ -303,6 +305,7 @@ class OracleModel:
         self.m.lm_head = lm
         self.m.seq_len = 0
         self.m.rope_interleaved = int(bool(cfg.get("rope_interleaved", False)))
+        self.m.rope_scale = float(cfg.get("rope_scale", 1.0))
         self.logits = np.empty(cfg["vocab"], np.float32)
         self.hidden = np.empty(cfg["hidden"], np.float32)
 
@@ -341,6 +344,8 @@ def ref():
                                                 _i64, _i64, _i64, _i64, _i64]
         R.ref_rmsnorm_inplace.argtypes = [_vp, _vp, _f32, _i32, _i64]
         R.ref_rope_precompute.argtypes = [_vp, _vp, _i64, _i64, _f32]
+        R.ref_rope_precompute_scaled.argtypes = [_vp, _vp, _i64, _i64, _f32, _f32]
+        R.ref_model_set_rope_scale.argtypes = [_vp, _f32]
         R.ref_rope_apply_neox.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
         R.ref_rope_apply_norm.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
         R.ref_model_set_arch.argtypes = [_vp, _i32, _i32]
@@ -400,6 +405,8 @@ class RefModel:
                                     cfg["head_dim"], cfg["inter"], cfg["rope_base"], cfg["eps"], max_seq)
         if cfg.get("rope_interleaved") or layers[0].get("q_norm") is None:
             R.ref_model_set_arch(self.h, int(layers[0].get("q_norm") is not None), int(not cfg.get("rope_interleaved")))
+        if cfg.get("rope_scale", 1.0) != 1.0:
+            R.ref_model_set_rope_scale(self.h, float(cfg["rope_scale"]))
         names = ("q", "k", "v", "o", "gate", "up", "down")
         for i, L in enumerate(layers):
             for w, name in enumerate(names):

@@ -117,6 +117,11 @@ void ref_model_set_arch(void* h, int has_qk_norm, int rope_neox) {
     c.has_qk_norm = has_qk_norm != 0;
     c.rope_neox = rope_neox != 0;
 }
+// linear rotary position scaling (ModelConfig::rope_scale, gguf_model.h:71, read from rope.scaling.* at :136-156)
+void ref_model_set_rope_scale(void* h, float scale) { static_cast<RefModel*>(h)->m.config.rope_scale = scale; }
+void ref_rope_precompute_scaled(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale) {
+    at::native::hot::rope_precompute(c, s, pos, head_dim, base, scale, nullptr, 1.0f);
+}
 void ref_model_destroy(void* h) {
     auto* r = static_cast<RefModel*>(h);
     // weights are caller-owned: detach before QuantizedWeight could free them

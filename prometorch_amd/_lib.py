@@ -43,7 +43,7 @@ class DecodeConfig(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")] + \
                [("rope_freq_base", f32), ("rms_eps", f32), ("kv_fp16", C.c_int32), ("use_graph", C.c_int32),
                 ("embedding_f32", vp), ("layers", C.POINTER(Layer)), ("out_norm", vp), ("lm_head", QWeight),
-                ("rope_interleaved", C.c_int32)]
+                ("rope_interleaved", C.c_int32), ("rope_scale", f32)]
 
 
 class Sampling(C.Structure):
@@ -88,6 +88,7 @@ SIGNATURES = {
     "ptm_per_head_rms_norm": (i32, [vp, vp, i32, i32, i32, f32, i32, vp]),
     "ptm_qknorm_rope_kvwrite": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, vp, f32, i32, i32, i32, vp]),
     "ptm_rope_table_host": (i32, [vp, i32, i32, f32]),
+    "ptm_rope_table_host_scaled": (i32, [vp, i32, i32, f32, f32]),
     "ptm_fp16_kv_cache_write": (i32, [vp, vp, i64, i64, i64, vp]),
     "ptm_flash_decode_kv_chunk_size": (i32, []),
     "ptm_flash_decode_num_splits": (i32, [i32]),

@@ -393,7 +393,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     if ((rc = hip_status(hipHostMalloc((void**)&d->h_uniforms, 4 * (size_t)c.max_seq, hipHostMallocDefault))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     {
         std::vector<float> tab((size_t)c.max_seq * c.head_dim);
-        ptm_rope_table_host(tab.data(), c.max_seq, c.head_dim, c.rope_freq_base);
+        ptm_rope_table_host_scaled(tab.data(), c.max_seq, c.head_dim, c.rope_freq_base, c.rope_scale);
         if ((rc = hip_status(hipMemcpy(d->rope, tab.data(), tab.size() * 4, hipMemcpyHostToDevice))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     }
     hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, d->stream, d->d_token, 0, d->d_past, (int64_t)0, d->d_step);

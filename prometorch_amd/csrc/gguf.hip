@@ -408,6 +408,18 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
     double fv = 10000.0;
     (void)ptm_gguf_get_float(m->file, (arch + ".rope.freq_base").c_str(), &fv);
     c.rope_freq_base = (float)fv;
+    {   // linear position scaling: rope.scaling.type == "linear" with a factor above 1, else the older
+        // rope.scale_linear key (gguf_model.h:136-156); other scaling types leave the positions as they are
+        c.rope_scale = 1.0f;
+        const char* st = ptm_gguf_get_string(m->file, (arch + ".rope.scaling.type").c_str());
+        double f = 0.0;
+        if (st && std::string(st) == "linear" &&
+            ptm_gguf_get_float(m->file, (arch + ".rope.scaling.factor").c_str(), &f) == PTM_OK && (float)f > 1.0f)
+            c.rope_scale = (float)f;
+        if (c.rope_scale == 1.0f && ptm_gguf_get_float(m->file, (arch + ".rope.scale_linear").c_str(), &f) == PTM_OK &&
+            (float)f > 1.0f)
+            c.rope_scale = (float)f;
+    }
     fv = 1e-6;
     (void)ptm_gguf_get_float(m->file, (arch + ".attention.layer_norm_rms_epsilon").c_str(), &fv);
     c.rms_eps = (float)fv;

@@ -442,13 +442,19 @@ int ptm_qknorm_rope_kvwrite(float* Q, float* K, const float* V, const float* q_n
 }
 
 int ptm_rope_table_host(float* table, int max_seq, int head_dim, float base) {
+    return ptm_rope_table_host_scaled(table, max_seq, head_dim, base, 1.0f);
+}
+
+int ptm_rope_table_host_scaled(float* table, int max_seq, int head_dim, float base, float scale) {
     if (!table) return PTM_E_NULL;
     if (max_seq <= 0 || head_dim <= 0 || (head_dim & 1)) return PTM_E_SHAPE;
     const int half = head_dim / 2;
+    const bool scaled = scale > 0.0f && scale != 1.0f;  // hot_loops.cpp:1858-1860
     for (int pos = 0; pos < max_seq; ++pos) {
+        const float p = scaled ? (float)pos / scale : (float)pos;
         for (int d = 0; d < half; ++d) {
             const float inv = 1.0f / std::pow(base, 2.0f * (float)d / (float)head_dim);
-            const float th = (float)pos * inv;
+            const float th = p * inv;
             table[(int64_t)pos * head_dim + d] = std::cos(th);
             table[(int64_t)pos * head_dim + half + d] = std::sin(th);
         }

@@ -73,6 +73,7 @@ class Decoder:
         c.kv_fp16 = int(kv_fp16)
         c.use_graph = int(use_graph)
         c.rope_interleaved = int(bool(cfg.get("rope_interleaved", False)))
+        c.rope_scale = float(cfg.get("rope_scale", 1.0))
         if embedding_f32 is not None:
             e = embedding_f32 if isinstance(embedding_f32, torch.Tensor) else torch.from_numpy(embedding_f32)
             e = e.to(device="cuda", dtype=torch.float32).contiguous()

@@ -66,10 +66,10 @@ def write_gguf(path: str, metadata: dict, tensors: list, alignment: int = 32, ve
 
 
 def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "qwen3", tied: bool = True,
-                  alignment: int = 32, tokenizer: dict | None = None) -> None:
+                  alignment: int = 32, tokenizer: dict | None = None, extra_metadata: dict | None = None) -> None:
     """Write a decoder (the dict form prometorch_amd.decode.Decoder takes) as a GGUF file with the
     tensor names and metadata keys a qwen3 GGUF carries.  tokenizer: tokenizer.ggml.* metadata to store
-    (default: a three-token placeholder)."""
+    (default: a three-token placeholder); extra_metadata: further keys, written as given."""
     md = {
         "general.architecture": arch, "general.name": "synthetic",
         f"{arch}.block_count": cfg["n_layers"], f"{arch}.embedding_length": cfg["hidden"],
@@ -79,9 +79,14 @@ def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "q
         f"{arch}.attention.layer_norm_rms_epsilon": float(cfg["eps"]), f"{arch}.context_length": 4096,
         "tokenizer.ggml.model": "gpt2", "tokenizer.ggml.tokens": ["a", "b", "c"], "tokenizer.ggml.token_type": [1, 1, 1],
     }
+    if cfg.get("rope_scale", 1.0) != 1.0:  # linear position scaling, the keys llama3 / qwen2 files use
+        md[f"{arch}.rope.scaling.type"] = "linear"
+        md[f"{arch}.rope.scaling.factor"] = float(cfg["rope_scale"])
     if tokenizer:
         md = {k: v for k, v in md.items() if not k.startswith("tokenizer.")}
         md.update(tokenizer)
+    if extra_metadata:
+        md.update(extra_metadata)
     H = cfg["hidden"]
     lm_type = head.get("lm_head_type", Q6_K)
     ts = [("token_embd.weight", lm_type, [H, cfg["vocab"]], head["lm_head"])]
@@ -214,7 +219,7 @@ class GGUFModel:
         check(self.L.ptm_model_config(m, C.byref(c)), "model_config")
         self.cfg = {k: getattr(c, k) for k in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")}
         self.cfg.update(rope_base=c.rope_freq_base, eps=c.rms_eps, kv_fp16=bool(c.kv_fp16), tied=not bool(c.embedding_f32),
-                        rope_interleaved=bool(c.rope_interleaved))
+                        rope_interleaved=bool(c.rope_interleaved), rope_scale=c.rope_scale)
 
     def layer(self, i: int) -> Layer:
         out = Layer()

@@ -188,10 +188,11 @@ def launch_fused_qknorm_rope_kvwrite_graph(Q, K, V, q_norm_w, k_norm_w, K_cache,
                                       _stream(stream)), "qknorm_rope_kvwrite")
 
 
-def rope_table(max_seq, head_dim, rope_freq_base):
-    """Host-computed cos/sin rows [max_seq, head_dim] (hot_loops.cpp:1853-1876), returned as a CPU tensor."""
+def rope_table(max_seq, head_dim, rope_freq_base, scale=1.0):
+    """Host-computed cos/sin rows [max_seq, head_dim] (hot_loops.cpp:1853-1876), returned as a CPU tensor; scale: linear
+    position scaling, theta = (pos / scale) * freq."""
     t = torch.empty(max_seq, head_dim, dtype=torch.float32)
-    check(_L().ptm_rope_table_host(t.data_ptr(), max_seq, head_dim, rope_freq_base), "rope_table_host")
+    check(_L().ptm_rope_table_host_scaled(t.data_ptr(), max_seq, head_dim, rope_freq_base, scale), "rope_table_host")
     return t
 
 

@@ -387,6 +387,22 @@ def make_llama_golden():
     c, s = po.rope_tables(2049, 128, 5.0e5)
     R.ref_rope_apply_norm(q.ctypes.data, k.ctypes.data, c.ctypes.data, s.ctypes.data, 32, 8, 128)
     g["rope_norm_q"], g["rope_norm_k"] = q, k
+    # linear position scaling (rope.scaling.type = linear): the same model at scale 4, and the table alone
+    cfg4 = dict(cfg, rope_scale=4.0)
+    rm = po.RefModel(cfg4, layers, head, 64, emb)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(SEEDS["tiny"], i, cfg, 19)
+        rm.set_kv(i, k, v)
+    tok, toks, lg = 3, [], []
+    for _ in range(12):
+        tok = rm.step(tok)
+        toks.append(tok)
+        lg.append(rm.logits.copy())
+    rm.close()
+    g["scaled_tokens"], g["scaled_logits"] = np.array(toks, np.int64), np.stack(lg)
+    c4, s4 = np.empty(64, np.float32), np.empty(64, np.float32)
+    R.ref_rope_precompute_scaled(c4.ctypes.data, s4.ctypes.data, 2049, 128, 5.0e5, 4.0)
+    g["scaled_cos"], g["scaled_sin"] = c4, s4
     np.savez_compressed(os.path.join(OUT, "golden_llama.npz"), **g)
 
 

@@ -249,6 +249,48 @@ def test_llama_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_llama, t
     assert e.value.code == -10
 
 
+def test_linear_rope_scaling_vs_reference_golden(dev, po, seeds, golden_llama, tmp_path):
+    """rope.scaling.type = linear, factor 4: theta = (pos / 4) * freq (hot_loops.cpp:1858-1860).  The host table equals the
+    reference's bit for bit, a decoder built with cfg['rope_scale'] and one loaded from a .gguf file carrying the scaling
+    keys follow the compiled reference's run at that scale; the older rope.scale_linear key is read too."""
+    from prometorch_amd.decode import Decoder
+    tab = ops.rope_table(2050, 128, 5.0e5, 4.0).numpy()
+    assert np.array_equal(bits(tab[2049, :64]), bits(golden_llama["scaled_cos"]))
+    assert np.array_equal(bits(tab[2049, 64:]), bits(golden_llama["scaled_sin"]))
+    assert np.array_equal(ops.rope_table(64, 128, 5.0e5, 1.0).numpy(), ops.rope_table(64, 128, 5.0e5).numpy())
+    cfg, layers, head, kv = tiny_llama_with_cache(seeds)
+    cfg = dict(cfg, rope_scale=4.0)
+    path = str(tmp_path / "scaled.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head, arch="llama")
+    m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
+    assert m.cfg["rope_scale"] == 4.0
+    d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
+    for i, (k, v) in enumerate(kv):
+        m.set_kv(i, k, v)
+        d.set_kv(i, k, v)
+    m.set_past_len(19)
+    d.set_past_len(19)
+    tm = td = 3
+    errs = []
+    for st in range(12):
+        tm = m.step(tm)
+        td = d.step(td)
+        ref = golden_llama["scaled_logits"][st]
+        errs.append(np.abs(d.logits() - ref).max() / ref.std())
+        assert tm == td == int(golden_llama["scaled_tokens"][st]), st
+        assert np.array_equal(bits(m.logits()), bits(d.logits())), st
+    check_step_errors(errs)
+    m.close()
+    d.close()
+    # legacy key; a scaling type other than linear leaves the positions alone
+    for md, want in (({"llama.rope.scale_linear": 2.0}, 2.0), ({"llama.rope.scaling.type": "yarn", "llama.rope.scaling.factor": 8.0}, 1.0)):
+        p2 = str(tmp_path / f"k{want}.gguf")
+        gguf.model_to_gguf(p2, dict(cfg, rope_scale=1.0), layers, head, arch="llama", extra_metadata=md)
+        m2 = gguf.GGUFModel(p2, max_seq=64, kv_fp16=False)
+        assert m2.cfg["rope_scale"] == want
+        m2.close()
+
+
 def test_llama_sensitive_step_is_the_oracles_own(po, seeds):
     """CPU only, the yardstick for follow_sensitive: the oracle against itself with its input embedding perturbed by
     5e-4 relative exceeds the end-to-end bars at the same step after the same prompt, and holds them at the median."""

@@ -235,6 +235,22 @@ def test_llama_style_decode_and_rope_match_the_reference(po, seeds):
     q64 = q.astype(np.float64).reshape(32, 64, 2)
     want = np.stack([q64[..., 0] * np.cos(th) - q64[..., 1] * np.sin(th), q64[..., 0] * np.sin(th) + q64[..., 1] * np.cos(th)], -1)
     assert np.abs(qr.reshape(32, 64, 2) - want).max() <= 2e-3 * np.abs(want).max()   # fp32 angles of ~2e3 rad
+    # linear position scaling: theta = (pos / scale) * freq -- table and a 12-step run at scale 4 against the reference's
+    c4, s4 = po.rope_tables(2049, 128, 5.0e5, 4.0)
+    assert np.array_equal(c4.view(np.uint32), g["scaled_cos"].view(np.uint32))
+    assert np.array_equal(s4.view(np.uint32), g["scaled_sin"].view(np.uint32))
+    th4 = (2049.0 / 4.0) * 5.0e5 ** (-np.arange(64) / 64.0)
+    assert np.abs(c4 - np.cos(th4)).max() <= 1e-3 and np.abs(s4 - np.sin(th4)).max() <= 1e-3
+    om = po.OracleModel(dict(cfg, rope_scale=4.0), layers, head, 64, kv_fp16=False)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(seeds["tiny"], i, cfg, 19)
+        om.set_kv(i, k, v)
+    tok = 3
+    for st in range(12):
+        tok = om.step(tok)
+        assert tok == int(g["scaled_tokens"][st])
+        assert np.array_equal(om.logits.view(np.uint32), g["scaled_logits"][st].view(np.uint32)), st
+    assert np.abs(g["scaled_logits"][0] - g["logits"][0]).max() > g["logits"][0].std()   # the scale is not a no-op
 
 
 def test_qwen2_style_biases_match_the_reference(po, seeds):
