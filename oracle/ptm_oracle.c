@@ -495,7 +495,14 @@ void po_exp256(const float* in, float* out, int64_t n8) {
 /* ---- single-token attention for one head (reference: gguf_model.h:3510-3636) ----- */
 void po_attn_head(const float* q, const float* k, const float* v, int64_t T, int64_t kv_dim,
                   int64_t head_dim, float scale, float* sc, float* out) {
-    for (int64_t t = 0; t < T; ++t) {
+    po_attn_head_window(q, k, v, T, 0, kv_dim, head_dim, scale, sc, out);
+}
+/* positions before t_start are masked the way the reference masks them (gguf_model.h:3528-3530): their scores are
+ * -inf and every loop still runs over [0, T), so the 8-wide groups of the softmax keep their alignment */
+void po_attn_head_window(const float* q, const float* k, const float* v, int64_t T, int64_t t_start, int64_t kv_dim,
+                         int64_t head_dim, float scale, float* sc, float* out) {
+    for (int64_t t = 0; t < t_start; ++t) sc[t] = -INFINITY;
+    for (int64_t t = t_start; t < T; ++t) {
         const float* kt = k + t * kv_dim;
         __m256 a = _mm256_setzero_ps();
         int64_t d = 0;
@@ -530,6 +537,16 @@ void po_attn_head(const float* q, const float* k, const float* v, int64_t T, int
 }
 
 /* ---- SiLU(gate)*up in place (reference: gguf_model.h:3728-3763) ------------------ */
+/* tanh-approximated GELU times up (gguf_model.h:3730-3738): the expression as written there, libm tanhf */
+void po_gelu_mul(float* gate, const float* up, int64_t n) {
+    for (int64_t j = 0; j < n; ++j) {
+        const float g = gate[j];
+        const float c = 0.7978845608028654f;
+        const float x3 = g * g * g;
+        const float t = tanhf(c * (g + 0.044715f * x3));
+        gate[j] = 0.5f * g * (1.0f + t) * up[j];
+    }
+}
 void po_silu_mul(float* gate, const float* up, int64_t n) {
     int64_t j = 0;
     for (; j + 8 <= n; j += 8) {
@@ -571,12 +588,20 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
     if (m->embedding) memcpy(x, m->embedding + token * H, sizeof(float) * H);
     else po_dequantize_q6_k((const uint8_t*)m->lm_head.data + token * m->lm_head.stride, x, H);
 
+    if (m->scale_embeddings) { /* gguf_model.h:3252-3265 */
+        const float es = sqrtf((float)H);
+        for (int64_t j = 0; j < H; ++j) x[j] *= es;
+    }
+
     float rc[256], rs[256];
-    po_rope_precompute_scaled(rc, rs, past, hd, m->rope_base, m->rope_scale);
     const float scale = 1.0f / sqrtf((float)hd);
 
     for (int64_t li = 0; li < m->n_layers; ++li) {
         po_layer* L = &m->layers[li];
+        /* local (sliding-window) layers have their own rotation base and window start (gguf_model.h:265-302, :3490-3500) */
+        const int global = m->swa_window <= 0 || m->swa_pattern <= 0 || ((li + 1) % m->swa_pattern) == 0;
+        po_rope_precompute_scaled(rc, rs, past, hd, global ? m->rope_base : m->rope_swa_base, global ? m->rope_scale : 1.0f);
+        const int64_t t_start = (!global && T > m->swa_window) ? T - m->swa_window : 0;
         const int fuse_qkv = L->q.type == L->k.type && L->q.type == L->v.type;
         if (fuse_qkv) po_rmsnorm_vec(x, L->attn_norm, m->eps, 0, H, xn);
         else po_rmsnorm_seq(x, L->attn_norm, m->eps, 0, H, xn);
@@ -605,18 +630,21 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
 #pragma omp for schedule(static)
             for (int64_t h = 0; h < nh; ++h) {
                 const int64_t kvh = h / (nh / nkv);
-                po_attn_head(qb + h * hd, L->k_cache + kvh * hd, L->v_cache + kvh * hd, T, kvd, hd,
-                             scale, sc, ab + h * hd);
+                po_attn_head_window(qb + h * hd, L->k_cache + kvh * hd, L->v_cache + kvh * hd, T, t_start, kvd, hd,
+                                    scale, sc, ab + h * hd);
             }
             free(sc);
         }
         qgemv(&L->o, ab, hb);
+        if (L->post_attn_norm) po_rmsnorm_vec(hb, L->post_attn_norm, m->eps, 0, H, hb); /* gguf_model.h:3656-3663 */
         for (int64_t j = 0; j < H; ++j) x2[j] = x[j] + hb[j];
         po_rmsnorm_vec(x2, L->ffn_norm, m->eps, 0, H, xn);
         qgemv(&L->gate, xn, gb);
         qgemv(&L->up, xn, ub);
-        po_silu_mul(gb, ub, inter);
+        if (m->ffn_gelu) po_gelu_mul(gb, ub, inter);
+        else po_silu_mul(gb, ub, inter);
         qgemv(&L->down, gb, hb);
+        if (L->post_ffn_norm) po_rmsnorm_vec(hb, L->post_ffn_norm, m->eps, 0, H, hb); /* gguf_model.h:3787-3791 */
         for (int64_t j = 0; j < H; ++j) x[j] = x2[j] + hb[j];
     }
     po_rmsnorm_vec(x, m->out_norm, m->eps, 0, H, xn);

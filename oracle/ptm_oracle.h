@@ -81,7 +81,10 @@ void po_exp256(const float* in, float* out, int64_t n8);
  * block of row 0, row pitch kv_dim floats; scores is scratch[T] */
 void po_attn_head(const float* q, const float* k, const float* v, int64_t T, int64_t kv_dim,
                   int64_t head_dim, float scale, float* scores, float* out);
+void po_attn_head_window(const float* q, const float* k, const float* v, int64_t T, int64_t t_start, int64_t kv_dim,
+                         int64_t head_dim, float scale, float* scores, float* out);
 void po_silu_mul(float* gate, const float* up, int64_t n);
+void po_gelu_mul(float* gate, const float* up, int64_t n);
 int64_t po_argmax(const float* x, int64_t n);
 
 typedef struct {
@@ -93,6 +96,7 @@ typedef struct {
     const float *attn_norm, *ffn_norm, *q_norm, *k_norm; /* q_norm, k_norm: NULL for models without QK-norm */
     float *k_cache, *v_cache; /* [max_seq][kv_dim] fp32 storage */
     const float *q_bias, *k_bias, *v_bias; /* added to the projections' outputs (qwen2); all three or all NULL */
+    const float *post_attn_norm, *post_ffn_norm; /* gemma2 / gemma3: RMSNorm of a branch's output before the residual add */
 } po_layer;
 
 typedef struct {
@@ -106,6 +110,12 @@ typedef struct {
     int64_t seq_len;
     int rope_interleaved;   /* 0: NeoX pairs (d, d + half) as qwen / gemma / phi; 1: pairs (2d, 2d + 1) as llama / mistral */
     float rope_scale;       /* linear position scaling (ModelConfig::rope_scale, gguf_model.h:71); 0 or 1: none */
+    /* gemma family (gguf_model.h:74-88, :184-197): embedding rows times sqrt(hidden); tanh-GELU instead of SiLU in the
+     * feed-forward gate; layers li with (li + 1) % swa_pattern != 0 attend to the last swa_window positions only and
+     * rotate with rope_swa_base and no position scaling (swa_window or swa_pattern 0: every layer is global) */
+    int scale_embeddings, ffn_gelu;
+    int64_t swa_window, swa_pattern;
+    float rope_swa_base;
 } po_model;
 
 /* One decode step (forward_decode_cpu order, Q4_K_M fallbacks); writes logits[vocab],

@@ -35,14 +35,15 @@ class QW(C.Structure):
 class Layer(C.Structure):
     _fields_ = [(n, QW) for n in ("q", "k", "v", "o", "gate", "up", "down")] + \
                [(n, _vp) for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "k_cache", "v_cache",
-                                   "q_bias", "k_bias", "v_bias")]
+                                   "q_bias", "k_bias", "v_bias", "post_attn_norm", "post_ffn_norm")]
 
 
 class Model(C.Structure):
     _fields_ = [(n, _i64) for n in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")] + \
                [("rope_base", _f32), ("eps", _f32), ("kv_fp16", _i32), ("embedding", _vp),
                 ("layers", C.POINTER(Layer)), ("out_norm", _vp), ("lm_head", QW), ("seq_len", _i64), ("rope_interleaved", _i32),
-                ("rope_scale", _f32)]
+                ("rope_scale", _f32), ("scale_embeddings", _i32), ("ffn_gelu", _i32), ("swa_window", _i64),
+                ("swa_pattern", _i64), ("rope_swa_base", _f32)]
 
 
 _lib = None
@@ -271,7 +272,8 @@ class OracleModel:
                 qw, Wc = _qw(qt, W)
                 self._keep.append(Wc)
                 setattr(self.layers[i], name, qw)
-            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias"):
+            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias", "post_attn_norm",
+                         "post_ffn_norm"):
                 if L.get(name) is None:
                     setattr(self.layers[i], name, None)
                     continue
@@ -306,6 +308,11 @@ class OracleModel:
         self.m.seq_len = 0
         self.m.rope_interleaved = int(bool(cfg.get("rope_interleaved", False)))
         self.m.rope_scale = float(cfg.get("rope_scale", 1.0))
+        self.m.scale_embeddings = int(bool(cfg.get("scale_embeddings", False)))
+        self.m.ffn_gelu = int(bool(cfg.get("ffn_gelu", False)))
+        self.m.swa_window = int(cfg.get("swa_window", 0))
+        self.m.swa_pattern = int(cfg.get("swa_pattern", 0))
+        self.m.rope_swa_base = float(cfg.get("rope_swa_base", 10000.0))
         self.logits = np.empty(cfg["vocab"], np.float32)
         self.hidden = np.empty(cfg["hidden"], np.float32)
 
@@ -346,6 +353,7 @@ def ref():
         R.ref_rope_precompute.argtypes = [_vp, _vp, _i64, _i64, _f32]
         R.ref_rope_precompute_scaled.argtypes = [_vp, _vp, _i64, _i64, _f32, _f32]
         R.ref_model_set_rope_scale.argtypes = [_vp, _f32]
+        R.ref_model_set_gemma.argtypes = [_vp, _i32, _i32, _i32, _i64, _i64, _f32]
         R.ref_rope_apply_neox.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
         R.ref_rope_apply_norm.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
         R.ref_model_set_arch.argtypes = [_vp, _i32, _i32]
@@ -407,6 +415,10 @@ class RefModel:
             R.ref_model_set_arch(self.h, int(layers[0].get("q_norm") is not None), int(not cfg.get("rope_interleaved")))
         if cfg.get("rope_scale", 1.0) != 1.0:
             R.ref_model_set_rope_scale(self.h, float(cfg["rope_scale"]))
+        if any(cfg.get(k) for k in ("scale_embeddings", "ffn_gelu", "swa_window")) or layers[0].get("post_attn_norm") is not None:
+            R.ref_model_set_gemma(self.h, int(bool(cfg.get("scale_embeddings"))), int(bool(cfg.get("ffn_gelu"))),
+                                  int(layers[0].get("post_attn_norm") is not None), int(cfg.get("swa_window", 0)),
+                                  int(cfg.get("swa_pattern", 0)), float(cfg.get("rope_swa_base", 10000.0)))
         names = ("q", "k", "v", "o", "gate", "up", "down")
         for i, L in enumerate(layers):
             for w, name in enumerate(names):
@@ -415,7 +427,8 @@ class RefModel:
                 self._keep.append(W)
                 K = W.shape[1] // BLOCK[qt][0] * BLOCK[qt][1]
                 R.ref_model_set_weight(self.h, i, w, _p(W), qt, W.shape[0], K)
-            for w, name in enumerate(("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias")):
+            for w, name in enumerate(("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias",
+                                      "post_attn_norm", "post_ffn_norm")):
                 if L.get(name) is None:
                     continue
                 a = np.ascontiguousarray(L[name], np.float32)

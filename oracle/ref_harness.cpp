@@ -117,6 +117,17 @@ void ref_model_set_arch(void* h, int has_qk_norm, int rope_neox) {
     c.has_qk_norm = has_qk_norm != 0;
     c.rope_neox = rope_neox != 0;
 }
+// gemma-family switches of ModelConfig (gguf_model.h:74-88, :184-197): embedding scaling, tanh-GELU gate, post-norms,
+// alternating sliding-window layers with their own rotation base
+void ref_model_set_gemma(void* h, int scale_embeddings, int ffn_gelu, int has_post_norm, int64_t swa_window,
+                         int64_t swa_pattern, float rope_swa_base) {
+    auto& c = static_cast<RefModel*>(h)->m.config;
+    c.scale_embeddings = scale_embeddings != 0;
+    c.ffn_gelu = ffn_gelu != 0;
+    c.has_post_norm = has_post_norm != 0;
+    c.swa_window = swa_window; c.swa_pattern = swa_pattern;
+    c.rope_swa_freq_base = rope_swa_base; c.rope_swa_scale = 1.0f;
+}
 // linear rotary position scaling (ModelConfig::rope_scale, gguf_model.h:71, read from rope.scaling.* at :136-156)
 void ref_model_set_rope_scale(void* h, float scale) { static_cast<RefModel*>(h)->m.config.rope_scale = scale; }
 void ref_rope_precompute_scaled(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale) {
@@ -154,13 +165,15 @@ void ref_model_set_weight(void* h, int64_t layer, int which, const void* data, u
                                         &L.q_ffn_gate, &L.q_ffn_up, &L.q_ffn_down};
     set_qw(*w[which], data, type, rows, cols);
 }
-// which: 0 attn_norm, 1 ffn_norm, 2 q_norm, 3 k_norm, 4 / 5 / 6 attn_q / attn_k / attn_v bias (gguf_model.h:410-412)
+// which: 0 attn_norm, 1 ffn_norm, 2 q_norm, 3 k_norm, 4 / 5 / 6 attn_q / attn_k / attn_v bias (gguf_model.h:410-412),
+// 7 post_attention_norm, 8 post_ffw_norm
 void ref_model_set_norm(void* h, int64_t layer, int which, const float* gamma, int64_t n) {
     auto& L = static_cast<RefModel*>(h)->m.layers[layer];
     at::Tensor t = vec_tensor(gamma, n);
     if (which == 0) L.attn_norm = t; else if (which == 1) L.ffn_norm = t;
     else if (which == 2) L.attn_q_norm = t; else if (which == 3) L.attn_k_norm = t;
-    else if (which == 4) L.attn_q_bias = t; else if (which == 5) L.attn_k_bias = t; else L.attn_v_bias = t;
+    else if (which == 4) L.attn_q_bias = t; else if (which == 5) L.attn_k_bias = t; else if (which == 6) L.attn_v_bias = t;
+    else if (which == 7) L.post_attention_norm = t; else L.post_ffw_norm = t;
 }
 void ref_model_set_output(void* h, const float* out_norm, const void* lm_head, uint32_t type) {
     auto& m = static_cast<RefModel*>(h)->m;

@@ -286,6 +286,22 @@ def tiny_qwen2(seed: int):
     return cfg, layers, make_head(seed, cfg)
 
 
+def tiny_gemma(seed: int, n_layers: int = 4):
+    """The TINY shapes as a gemma3-style model: embedding rows times sqrt(hidden), per-head QK-norm, NeoX rotation,
+    tanh-GELU gate, RMSNorm on each branch's output before the residual add, and alternating attention: layers li with
+    (li + 1) % 3 != 0 see only the last 8 positions and rotate with base 1e4, the others see everything and rotate with
+    base 1e6 and positions divided by 8.  Four layers: local, local, global, local.  The embedding scale of 16 is undone in
+    the first norm gains' scale so that activations stay where the other tiny models have them."""
+    cfg = dict(TINY, n_layers=n_layers, scale_embeddings=True, ffn_gelu=True, swa_window=8, swa_pattern=3, rope_swa_base=1.0e4,
+               rope_scale=8.0)
+    layers = [make_layer(seed, i, cfg) for i in range(n_layers)]
+    for i, L in enumerate(layers):
+        g = rng_for(seed, 6, i)
+        for name in ("post_attn_norm", "post_ffn_norm"):
+            L[name] = (np.float32(0.5) * (np.float32(1.0) + np.float32(0.1) * g.standard_normal(cfg["hidden"], dtype=np.float32))).astype(np.float32)
+    return cfg, layers, make_head(seed, cfg)
+
+
 # ---- sampling cases: (vocab, logit kind, temperature, top_k, top_p), in the order the golden run draws them ----
 SAMPLING_CASES = (
     [(1000, "normal", 0.8, 40, 0.9), (1000, "normal", 1.0, 0, 1.0), (1000, "normal", 0.7, 1, 1.0),

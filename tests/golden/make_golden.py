@@ -82,6 +82,7 @@ def main():
     ap.add_argument("--full", action="store_true")
     ap.add_argument("--sampling-only", action="store_true", help="write golden_sampling.npz and nothing else")
     ap.add_argument("--tokenizer-only", action="store_true", help="write golden_tokenizer.json and nothing else")
+    ap.add_argument("--gemma-only", action="store_true", help="write golden_gemma.npz and nothing else")
     ap.add_argument("--qwen2-only", action="store_true", help="write golden_qwen2.npz and nothing else")
     ap.add_argument("--llama-only", action="store_true", help="write golden_llama.npz and nothing else")
     ap.add_argument("--mixed-only", action="store_true", help="write golden_mixed.npz and nothing else")
@@ -95,6 +96,10 @@ def main():
     if args.tokenizer_only:
         make_tokenizer_golden()
         print("wrote golden_tokenizer.json")
+        return
+    if args.gemma_only:
+        make_gemma_golden()
+        print("wrote golden_gemma.npz")
         return
     if args.qwen2_only:
         make_qwen2_golden()
@@ -236,6 +241,7 @@ def main():
     make_tokenizer_golden()
     make_llama_golden()
     make_qwen2_golden()
+    make_gemma_golden()
     make_formats_golden()
     make_mixed_golden()
 
@@ -422,6 +428,25 @@ def make_qwen2_golden():
         lg.append(rm.logits.copy())
     rm.close()
     np.savez_compressed(os.path.join(OUT, "golden_qwen2.npz"), tokens=np.array(toks, np.int64), logits=np.stack(lg))
+
+
+def make_gemma_golden():
+    """The reference's forward_decode_cpu on a gemma3-style tiny model (synth.tiny_gemma): scaled embeddings, GELU gate,
+    post-norms, sliding-window layers with their own rotation base; 16 greedy steps after a 19-position cache (the
+    window of 8 is exceeded from the first step)."""
+    cfg, layers, head = synth.tiny_gemma(SEEDS["tiny"])
+    emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    rm = po.RefModel(cfg, layers, head, 64, emb)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(SEEDS["tiny"], i, cfg, 19)
+        rm.set_kv(i, k, v)
+    tok, toks, lg = 3, [], []
+    for _ in range(16):
+        tok = rm.step(tok)
+        toks.append(tok)
+        lg.append(rm.logits.copy())
+    rm.close()
+    np.savez_compressed(os.path.join(OUT, "golden_gemma.npz"), tokens=np.array(toks, np.int64), logits=np.stack(lg))
 
 
 def make_full(meta):

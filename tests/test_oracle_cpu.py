@@ -286,6 +286,51 @@ def test_qwen2_style_biases_match_the_reference(po, seeds):
         assert np.abs(l1[0] - g["logits"][0]).max() > 1e-2 * sigma, drop
 
 
+def test_gemma_style_decode_matches_the_reference(po, seeds):
+    """Scaled embeddings, tanh-GELU gate, post-norms, sliding-window layers with their own rotation base and linear
+    position scaling on the global ones (gemma3): oracle bit-identical to the compiled reference's forward_decode_cpu
+    (golden_gemma.npz); switching any one of the features off moves the first step's logits, so the run exercises each."""
+    import os
+    from prometorch_amd import synth
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_gemma.npz"))
+    cfg, layers, head = synth.tiny_gemma(seeds["tiny"])
+
+    def run(cfg, layers, steps):
+        om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)
+        for i in range(cfg["n_layers"]):
+            k, v = synth.make_kv_prefill(seeds["tiny"], i, cfg, 19)
+            om.set_kv(i, k, v)
+        tok, toks, lg = 3, [], []
+        for _ in range(steps):
+            tok = om.step(tok)
+            toks.append(tok)
+            lg.append(om.logits.copy())
+        return toks, np.stack(lg)
+
+    toks, lg = run(cfg, layers, 16)
+    assert toks == [int(t) for t in g["tokens"]]
+    assert np.array_equal(lg.view(np.uint32), g["logits"].view(np.uint32))
+    sigma = float(g["logits"][0].std())
+    for key, off in (("scale_embeddings", False), ("ffn_gelu", False), ("swa_window", 0), ("rope_swa_base", 1.0e6), ("rope_scale", 1.0)):
+        _, l1 = run(dict(cfg, **{key: off}), layers, 1)
+        assert np.abs(l1[0] - g["logits"][0]).max() > 1e-2 * sigma, key
+    for name in ("post_attn_norm", "post_ffn_norm"):
+        _, l1 = run(cfg, [{k: v for k, v in L.items() if k != name} for L in layers], 1)
+        assert np.abs(l1[0] - g["logits"][0]).max() > 1e-2 * sigma, name
+
+
+def test_gelu_gate_against_float64(po):
+    r = np.random.default_rng(3)
+    gate = (3 * r.standard_normal(4096)).astype(np.float32)
+    up = r.standard_normal(4096).astype(np.float32)
+    got = gate.copy()
+    po.lib().po_gelu_mul.argtypes = [po._vp, po._vp, po._i64]
+    po.lib().po_gelu_mul(po._p(got), po._p(up), got.size)
+    g64 = gate.astype(np.float64)
+    want = 0.5 * g64 * (1 + np.tanh(np.sqrt(2 / np.pi) * (g64 + 0.044715 * g64 ** 3))) * up
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("maker,fname", [("tiny_mixed", "golden_mixed.npz"), ("tiny_formats", "golden_formats_model.npz")])
 def test_mixed_type_layers_match_the_reference(po, seeds, maker, fname):
     """Layers whose q/k/v share a type (the reference fuses them behind its 8-lane norm) beside layers where they do
