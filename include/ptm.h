@@ -197,12 +197,28 @@ int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const 
                           int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
                           float scale, float eps, int add_one, int kv_fp16, int rope_interleaved,
                           ptm_stream_t stream);
+/* The same over a sliding window: only the last `window` positions, the new one included, are attended to
+ * (window <= 0: all).  The local layers of gemma3 (attn_start, gguf_model.h:3490-3500). */
+int ptm_attn_decode_fused_window(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                                 const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
+                                 float* partial_lse, float* partial_max, const float* rope_table,
+                                 int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                                 float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
+                                 ptm_stream_t stream);
 /* q_norm_w / k_norm_w may both be NULL (models without QK-norm).  rope_interleaved: 0 rotates the NeoX pairs
  * (d, d + head_dim/2) of qwen / gemma / phi (rope_apply_fused_neox, hot_loops.cpp:2035-2061), 1 the pairs
  * (2d, 2d + 1) of llama / mistral (rope_apply_fused, hot_loops.cpp:1962-2030); config.rope_neox, gguf_model.h:98. */
 
 /* out = silu(gate) * up. launch_silu_mul (CUDAOps.h:416-418). */
 int ptm_silu_mul(const float* gate, const float* up, float* out, int64_t n, ptm_stream_t stream);
+/* gemma-family glue.  out = gelu_tanh(gate) * up, the expression of the reference's CPU step (gguf_model.h:3730-3738;
+ * config.ffn_gelu).  x[r][:] += RMSNorm(h[r][:]) * weight: a branch's post-norm and its residual add
+ * (post_attention_norm / post_ffw_norm, gguf_model.h:3656-3680, :3787-3807).  x *= factor: embedding rows times
+ * sqrt(hidden) (config.scale_embeddings, gguf_model.h:3252-3265; launch_mul_scalar, CUDAOps.h:67). */
+int ptm_gelu_mul(const float* gate, const float* up, float* out, int64_t n, ptm_stream_t stream);
+int ptm_rms_norm_add(const float* h, const float* weight, float* x, int rows, int hidden, float eps, int add_one,
+                     ptm_stream_t stream);
+int ptm_scale(float* x, float factor, int64_t n, ptm_stream_t stream);
 /* out[hidden] = emb_table[*d_token_id][:]. launch_embedding_lookup (CUDAOps.h:149-152). */
 int ptm_embedding_row(const float* emb_table, float* out, const int* d_token_id, int hidden,
                       ptm_stream_t stream);
@@ -300,6 +316,11 @@ int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float
 int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cache, float* O, int rows, int n_heads,
                           int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float scale, int kv_fp16,
                           ptm_stream_t stream);
+/* The same over a sliding window: row r sees positions (pos0 + r - window, pos0 + r] only (window <= 0: everything).
+ * The local layers of gemma3 (attn_start, gguf_model.h:3490-3500); windowed calls run on the fp32 kernel. */
+int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void* V_cache, float* O, int rows, int n_heads,
+                                 int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float scale, int kv_fp16,
+                                 int window, ptm_stream_t stream);
 
 /* ---- batch-1 decode runtime (GGUFModel::forward_decode, gguf_model.h:2575-3113) --- */
 typedef struct {
@@ -316,6 +337,8 @@ typedef struct {
     void *k_cache, *v_cache; /* device [max_seq][kv_dim], fp16 or fp32 per kv_fp16 */
     const float *q_bias, *k_bias, *v_bias; /* device fp32 [q_dim], [kv_dim], [kv_dim] (qwen2; LayerWeights::attn_*_bias,
                                             * gguf_model.h:410-412); all three or all NULL */
+    const float *post_attn_norm, *post_ffn_norm; /* device fp32 [hidden] (gemma2 / gemma3: RMSNorm of the attention / the
+                                                  * feed-forward branch's output before the residual add); each may be NULL */
 } ptm_layer;
 
 typedef struct {
@@ -329,6 +352,11 @@ typedef struct {
     ptm_qweight lm_head;
     int32_t rope_interleaved;     /* 0: NeoX rotation pairs (qwen3); 1: pairs (2d, 2d+1) (llama, mistral) */
     float rope_scale;             /* linear position scaling, theta = (pos / rope_scale) * freq (gguf_model.h:71); 0 or 1: none */
+    /* gemma family (ModelConfig, gguf_model.h:74-88): embedding rows times sqrt(hidden); tanh-GELU instead of SiLU on the
+     * gate; layers li with (li + 1) % swa_pattern != 0 attend to the last swa_window positions only and rotate with
+     * rope_swa_freq_base without position scaling (swa_window or swa_pattern 0: no local layers) */
+    int32_t scale_embeddings, ffn_gelu, swa_window, swa_pattern;
+    float rope_swa_freq_base;
 } ptm_decode_config;
 
 typedef struct ptm_decoder ptm_decoder;

@@ -196,13 +196,15 @@ def exp256(x):
     return out
 
 
-def attn_head(q, kc, vc, T, kv_dim, head_dim, scale, col0=0):
-    """kc, vc: fp32 [>=T, kv_dim]; col0 = kv_head*head_dim."""
+def attn_head(q, kc, vc, T, kv_dim, head_dim, scale, col0=0, t_start=0):
+    """kc, vc: fp32 [>=T, kv_dim]; col0 = kv_head*head_dim; positions before t_start are masked."""
     q = np.ascontiguousarray(q, np.float32)
     sc = np.empty(T + 8, np.float32)
     out = np.empty(head_dim, np.float32)
-    lib().po_attn_head(_p(q), C.c_void_p(kc.ctypes.data + 4 * col0), C.c_void_p(vc.ctypes.data + 4 * col0),
-                       T, kv_dim, head_dim, scale, _p(sc), _p(out))
+    L = lib()
+    L.po_attn_head_window.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32, _vp, _vp]
+    L.po_attn_head_window(_p(q), C.c_void_p(kc.ctypes.data + 4 * col0), C.c_void_p(vc.ctypes.data + 4 * col0),
+                          T, t_start, kv_dim, head_dim, scale, _p(sc), _p(out))
     return out
 
 

@@ -36,14 +36,15 @@ class QWeight(C.Structure):
 class Layer(C.Structure):
     _fields_ = [(n, QWeight) for n in ("q", "k", "v", "o", "gate", "up", "down")] + \
                [(n, vp) for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "k_cache", "v_cache",
-                                  "q_bias", "k_bias", "v_bias")]
+                                  "q_bias", "k_bias", "v_bias", "post_attn_norm", "post_ffn_norm")]
 
 
 class DecodeConfig(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")] + \
                [("rope_freq_base", f32), ("rms_eps", f32), ("kv_fp16", C.c_int32), ("use_graph", C.c_int32),
                 ("embedding_f32", vp), ("layers", C.POINTER(Layer)), ("out_norm", vp), ("lm_head", QWeight),
-                ("rope_interleaved", C.c_int32), ("rope_scale", f32)]
+                ("rope_interleaved", C.c_int32), ("rope_scale", f32), ("scale_embeddings", C.c_int32),
+                ("ffn_gelu", C.c_int32), ("swa_window", C.c_int32), ("swa_pattern", C.c_int32), ("rope_swa_freq_base", f32)]
 
 
 class Sampling(C.Structure):
@@ -94,12 +95,17 @@ SIGNATURES = {
     "ptm_flash_decode_num_splits": (i32, [i32]),
     "ptm_flash_decode": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, i32, vp]),
     "ptm_attn_decode_fused": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, f32, i32, i32, i32, vp]),
+    "ptm_attn_decode_fused_window": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, f32, i32, i32, i32, i32, vp]),
     "ptm_silu_mul": (i32, [vp, vp, vp, i64, vp]),
     "ptm_embedding_row": (i32, [vp, vp, vp, i32, vp]),
     "ptm_embedding_row_q6k": (i32, [vp, vp, vp, i32, i64, vp]),
     "ptm_argmax": (i32, [vp, vp, i64, vp]),
     "ptm_add": (i32, [vp, vp, vp, i64, vp]),
     "ptm_add_qkv_bias": (i32, [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp]),
+    "ptm_gelu_mul": (i32, [vp, vp, vp, i64, vp]),
+    "ptm_rms_norm_add": (i32, [vp, vp, vp, i32, i32, f32, i32, vp]),
+    "ptm_scale": (i32, [vp, f32, i64, vp]),
+    "ptm_prefill_attention_window": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, i32, vp]),
     "ptm_copy": (i32, [vp, vp, i64, vp]),
     "ptm_stream_read_partials": (i64, [i64]),
     "ptm_stream_read_xor": (i32, [vp, i64, vp, vp]),

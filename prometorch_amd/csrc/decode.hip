@@ -18,6 +18,12 @@
 #include <vector>
 
 // flash_decode.hip: ptm_attn_decode_fused that also leaves the output as Q8 activation blocks (not part of the C ABI)
+extern "C" int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                                         const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8,
+                                         float* partial_O, float* partial_lse, float* partial_max, const float* rope_table,
+                                         int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                                         float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
+                                         ptm_stream_t stream);
 extern "C" int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, const float* q_norm_w,
                                         const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8,
                                         float* partial_O, float* partial_lse, float* partial_max, const float* rope_table,
@@ -92,6 +98,8 @@ struct ptm_decoder {
     float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr, *act = nullptr,
           *gate = nullptr, *up = nullptr, *logits = nullptr, *pO = nullptr, *pL = nullptr, *pM = nullptr,
           *rope = nullptr;
+    float* hb = nullptr;        // [hidden] a branch's output in front of its post-norm
+    float* rope_swa = nullptr;  // rotation table of the sliding-window layers (their own base, no position scaling)
     uint8_t* xq8 = nullptr;
     void* amax_ws = nullptr;
     int* d_token = nullptr;
@@ -109,7 +117,7 @@ struct ptm_decoder {
     void* pf_slab = nullptr;
     int pf_rows = 0;
     float *pf_x = nullptr, *pf_q = nullptr, *pf_k = nullptr, *pf_v = nullptr, *pf_attn = nullptr,
-          *pf_gate = nullptr, *pf_up = nullptr;
+          *pf_gate = nullptr, *pf_up = nullptr, *pf_h = nullptr;
     void* pf_ws = nullptr;   // fp16 rows for Q4_K matrices (Q8-rounded)
     void* pf_ws2 = nullptr;  // fp16 rows for Q6_K matrices (plain)
     float* pf_split = nullptr;  // K-split partial sums of the GEMMs
@@ -140,6 +148,12 @@ static int gemv_any(const ptm_qweight& w, const float* x_f32, float* y, bool acc
     return ptm_quant_gemv(w.ggml_type, w.data, x_f32, y, w.cols, w.rows, w.row_stride_bytes, acc ? 1 : 0, s);
 }
 
+// gemma3's alternating layers: li is local (sliding window, own rotation base) unless (li + 1) % swa_pattern == 0
+// (ModelConfig::layer_is_global, gguf_model.h:265-281)
+static inline bool layer_is_local(const ptm_decode_config& c, int li) {
+    return c.swa_window > 0 && c.swa_pattern > 0 && ((li + 1) % c.swa_pattern) != 0;
+}
+
 // Enqueue one token step on d->stream. Everything it reads that changes per token is in device memory.
 static int enqueue_step(ptm_decoder* d, bool sample = false) {
     const ptm_decode_config& c = d->cfg;
@@ -149,9 +163,11 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
 #define PTM_TRY(call) do { rc = (call); if (rc != PTM_OK) return rc; } while (0)
     if (c.embedding_f32) PTM_TRY(ptm_embedding_row(c.embedding_f32, d->x, d->d_token, H, s));
     else PTM_TRY(ptm_embedding_row_q6k(c.lm_head.data, d->x, d->d_token, H, c.lm_head.row_stride_bytes, s));
+    if (c.scale_embeddings) PTM_TRY(ptm_scale(d->x, sqrtf((float)H), H, s));
 
     for (int li = 0; li < c.n_layers; ++li) {
         const ptm_layer& L = d->layers[li];
+        const bool local = layer_is_local(c, li);  // sliding-window layer: own rotation table, attention window
         // attention RMSNorm is recomputed inside each projection kernel (no separate launch):
         // the Q4_K projections share one launch, Q6_K ones get their own
         {
@@ -184,19 +200,22 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
         // a Q4_K output projection takes the attention output as the Q8 blocks the merge kernel leaves beside the fp32
         // vector: its prologue then copies 1.25 bytes per value instead of fetching and quantising 4
         const bool o_q8 = L.o.ggml_type == PTM_TYPE_Q4_K;
-        PTM_TRY(ptm_attn_decode_fused_q8(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn,
-                                         o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM, d->rope, c.n_heads, c.n_kv_heads, hd,
-                                         d->d_past, c.max_seq, 1.0f / sqrtf((float)hd), c.rms_eps, 0, c.kv_fp16,
-                                         c.rope_interleaved, s));
-        if (o_q8) {  // x += Wo . attn
+        PTM_TRY(ptm_attn_decode_fused_win(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn,
+                                          o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM, local ? d->rope_swa : d->rope,
+                                          c.n_heads, c.n_kv_heads, hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd),
+                                          c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, local ? c.swa_window : 0, s));
+        // x += Wo . attn, or with a post-norm: h = Wo . attn, x += RMSNorm(h) * w
+        float* o_dst = L.post_attn_norm ? d->hb : d->x;
+        const bool o_acc = !L.post_attn_norm;
+        if (o_q8) {
             const void* W = L.o.data;
-            float* y = d->x;
             const int N = L.o.rows;
-            PTM_TRY(q4k_gemv_multi(1, &W, &y, &N, d->xq8, true, nullptr, 0.f, 0, L.o.cols, L.o.row_stride_bytes, true, s));
+            PTM_TRY(q4k_gemv_multi(1, &W, &o_dst, &N, d->xq8, true, nullptr, 0.f, 0, L.o.cols, L.o.row_stride_bytes, o_acc, s));
         } else {
-            PTM_TRY(gemv_any(L.o, d->attn, d->x, true, s));
+            PTM_TRY(gemv_any(L.o, d->attn, o_dst, o_acc, s));
         }
-        if (L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
+        if (L.post_attn_norm) PTM_TRY(ptm_rms_norm_add(d->hb, L.post_attn_norm, d->x, 1, H, c.rms_eps, 0, s));
+        if (!c.ffn_gelu && L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
             L.gate.row_stride_bytes == L.up.row_stride_bytes && L.gate.rows == L.up.rows) {
             PTM_TRY(q4k_gate_up_silu(L.gate.data, L.up.data, d->x, false, L.ffn_norm, c.rms_eps, 0, d->act, H,
                                      L.gate.rows, L.gate.row_stride_bytes, s));
@@ -204,9 +223,15 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
             PTM_TRY(ptm_rms_norm(d->x, L.ffn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
             PTM_TRY(gemv_any(L.gate, d->xn, d->gate, false, s));
             PTM_TRY(gemv_any(L.up, d->xn, d->up, false, s));
-            PTM_TRY(ptm_silu_mul(d->gate, d->up, d->act, c.inter, s));
+            if (c.ffn_gelu) PTM_TRY(ptm_gelu_mul(d->gate, d->up, d->act, c.inter, s));
+            else PTM_TRY(ptm_silu_mul(d->gate, d->up, d->act, c.inter, s));
         }
-        PTM_TRY(gemv_any(L.down, d->act, d->x, true, s));  // x += Wdown . act
+        if (L.post_ffn_norm) {
+            PTM_TRY(gemv_any(L.down, d->act, d->hb, false, s));
+            PTM_TRY(ptm_rms_norm_add(d->hb, L.post_ffn_norm, d->x, 1, H, c.rms_eps, 0, s));
+        } else {
+            PTM_TRY(gemv_any(L.down, d->act, d->x, true, s));  // x += Wdown . act
+        }
     }
     if (sample) {
         // logits (final RMSNorm in the lm_head prologue), then the sampler, whose last kernel does the step bookkeeping
@@ -248,6 +273,7 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
     size_t off = 0;
     auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
     const size_t R = (size_t)rows;
+    const size_t o_h = take(4 * R * H);
     const size_t o_x = take(4 * R * H), o_q = take(4 * R * qd), o_k = take(4 * R * kvd),
                  o_v = take(4 * R * kvd), o_attn = take(4 * R * qd), o_gate = take(4 * R * I), o_up = take(4 * R * I),
                  o_ws = take((size_t)ptm_qgemm_f16_workspace_bytes(rows, (int)kmax)),
@@ -266,6 +292,7 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
     const int rc = hip_status(hipMalloc(&d->pf_slab, off));
     if (rc != PTM_OK) return rc;
     uint8_t* b = static_cast<uint8_t*>(d->pf_slab);
+    d->pf_h = (float*)(b + o_h);
     d->pf_x = (float*)(b + o_x); d->pf_q = (float*)(b + o_q); d->pf_k = (float*)(b + o_k);
     d->pf_v = (float*)(b + o_v); d->pf_attn = (float*)(b + o_attn); d->pf_gate = (float*)(b + o_gate);
     d->pf_up = (float*)(b + o_up); d->pf_ws = b + o_ws; d->pf_ws2 = b + o_ws2; d->pf_tokens = (int*)(b + o_tok);
@@ -284,6 +311,7 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
     PTM_TRY(hip_status(hipMemcpyAsync(d->pf_tokens, tokens_host, 4 * (size_t)M, hipMemcpyHostToDevice, s)));
     PTM_TRY(ptm_embedding_rows(c.embedding_f32, c.embedding_f32 ? nullptr : c.lm_head.data, c.lm_head.row_stride_bytes,
                                d->pf_tokens, M, H, c.vocab, d->pf_x, s));
+    if (c.scale_embeddings) PTM_TRY(ptm_scale(d->pf_x, sqrtf((float)H), (int64_t)M * H, s));
     // Q4_K matrices take their rows from pf_ws (Q8-rounded fp16), Q6_K ones from pf_ws2 (plain fp16).  RMSNorm and
     // SiLU.up are fused into the conversion (one launch fills both forms); a product whose rows are already in its
     // workspace skips the conversion.
@@ -298,6 +326,7 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
     };
     for (int li = 0; li < c.n_layers; ++li) {
         const ptm_layer& L = d->layers[li];
+        const bool local = layer_is_local(c, li);
         PTM_TRY(qgemm_f16_prepare_fused(1, d->pf_x, L.attn_norm, c.rms_eps, 0,
                                         uses(PTM_TYPE_Q4_K, {&L.q, &L.k, &L.v}) ? d->pf_ws : nullptr,
                                         uses(PTM_TYPE_Q6_K, {&L.q, &L.k, &L.v}) ? d->pf_ws2 : nullptr, M, H, s));
@@ -305,19 +334,36 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
         PTM_TRY(gemm(L.k, d->pf_x, d->pf_k, false, true));
         PTM_TRY(gemm(L.v, d->pf_x, d->pf_v, false, true));
         if (L.q_bias) PTM_TRY(ptm_add_qkv_bias(d->pf_q, d->pf_k, d->pf_v, L.q_bias, L.k_bias, L.v_bias, M, qd, kvd, s));
-        PTM_TRY(ptm_qknorm_rope_kvwrite_rows(d->pf_q, d->pf_k, d->pf_v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->rope, M,
+        PTM_TRY(ptm_qknorm_rope_kvwrite_rows(d->pf_q, d->pf_k, d->pf_v, L.q_norm, L.k_norm, L.k_cache, L.v_cache,
+                                             local ? d->rope_swa : d->rope, M,
                                              c.n_heads, c.n_kv_heads, hd, pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, s));
-        PTM_TRY(ptm_prefill_attention(d->pf_q, L.k_cache, L.v_cache, d->pf_attn, M, c.n_heads, c.n_kv_heads, hd, pos0,
-                                      c.max_seq, 1.0f / sqrtf((float)hd), c.kv_fp16, s));
-        PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true, false));  // x += attn . Wo^T
+        PTM_TRY(ptm_prefill_attention_window(d->pf_q, L.k_cache, L.v_cache, d->pf_attn, M, c.n_heads, c.n_kv_heads, hd, pos0,
+                                             c.max_seq, 1.0f / sqrtf((float)hd), c.kv_fp16, local ? c.swa_window : 0, s));
+        if (L.post_attn_norm) {
+            PTM_TRY(gemm(L.o, d->pf_attn, d->pf_h, false, false));
+            PTM_TRY(ptm_rms_norm_add(d->pf_h, L.post_attn_norm, d->pf_x, M, H, c.rms_eps, 0, s));
+        } else {
+            PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true, false));  // x += attn . Wo^T
+        }
         PTM_TRY(qgemm_f16_prepare_fused(1, d->pf_x, L.ffn_norm, c.rms_eps, 0,
                                         uses(PTM_TYPE_Q4_K, {&L.gate, &L.up}) ? d->pf_ws : nullptr,
                                         uses(PTM_TYPE_Q6_K, {&L.gate, &L.up}) ? d->pf_ws2 : nullptr, M, H, s));
         PTM_TRY(gemm(L.gate, d->pf_x, d->pf_gate, false, true));
         PTM_TRY(gemm(L.up, d->pf_x, d->pf_up, false, true));
-        PTM_TRY(qgemm_f16_prepare_fused(2, d->pf_gate, d->pf_up, 0.0f, 0, L.down.ggml_type == PTM_TYPE_Q4_K ? d->pf_ws : nullptr,
-                                        L.down.ggml_type == PTM_TYPE_Q6_K ? d->pf_ws2 : nullptr, M, I, s));
-        PTM_TRY(gemm(L.down, d->pf_gate, d->pf_x, true, true));  // x += act . Wdown^T
+        bool act_ready = true;
+        if (c.ffn_gelu) {  // GELU.up as a launch of its own; the down product then converts its rows itself
+            PTM_TRY(ptm_gelu_mul(d->pf_gate, d->pf_up, d->pf_gate, (int64_t)M * I, s));
+            act_ready = false;
+        } else {
+            PTM_TRY(qgemm_f16_prepare_fused(2, d->pf_gate, d->pf_up, 0.0f, 0, L.down.ggml_type == PTM_TYPE_Q4_K ? d->pf_ws : nullptr,
+                                            L.down.ggml_type == PTM_TYPE_Q6_K ? d->pf_ws2 : nullptr, M, I, s));
+        }
+        if (L.post_ffn_norm) {
+            PTM_TRY(gemm(L.down, d->pf_gate, d->pf_h, false, act_ready));
+            PTM_TRY(ptm_rms_norm_add(d->pf_h, L.post_ffn_norm, d->pf_x, M, H, c.rms_eps, 0, s));
+        } else {
+            PTM_TRY(gemm(L.down, d->pf_gate, d->pf_x, true, act_ready));  // x += act . Wdown^T
+        }
     }
     (void)qd; (void)kvd;
     return PTM_OK;
@@ -335,6 +381,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
         (c.n_heads % c.n_kv_heads))
         return PTM_E_SHAPE;
     if (c.head_dim != 64 && c.head_dim != 128) return PTM_E_UNSUPPORTED;
+    if (c.swa_window < 0 || c.swa_pattern < 0 || (c.swa_window > 0 && !(c.rope_swa_freq_base > 0.0f))) return PTM_E_SHAPE;
     const int H = c.hidden, qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim;
     int rc = qw_check(c.lm_head, c.vocab, H);
     if (rc != PTM_OK) return rc;
@@ -368,6 +415,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
                  o_up = take(4 * (size_t)c.inter), o_logits = take(4 * (size_t)c.vocab),
                  o_pO = take(4 * (size_t)S * c.n_heads * c.head_dim), o_pL = take(4 * (size_t)S * c.n_heads),
                  o_pM = take(4 * (size_t)S * c.n_heads), o_rope = take(4 * (size_t)c.max_seq * c.head_dim),
+                 o_hb = take(4 * (size_t)H), o_rope_swa = take(c.swa_window > 0 ? 4 * (size_t)c.max_seq * c.head_dim : 0),
                  o_xq8 = take((size_t)ptm_q8_bytes(qd > (H > c.inter ? H : c.inter) ? qd : (H > c.inter ? H : c.inter))),
                  o_ws = take((size_t)ptm_argmax_workspace_bytes(c.vocab)), o_tok = take(256), o_past = take(256),
                  o_next = take(256), o_step = take(256), o_tokens = take(8 * (size_t)c.max_seq),
@@ -380,6 +428,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->act = (float*)(base + o_act); d->gate = (float*)(base + o_gate); d->up = (float*)(base + o_up);
     d->logits = (float*)(base + o_logits); d->pO = (float*)(base + o_pO); d->pL = (float*)(base + o_pL);
     d->pM = (float*)(base + o_pM); d->rope = (float*)(base + o_rope); d->xq8 = base + o_xq8;
+    d->hb = (float*)(base + o_hb); d->rope_swa = c.swa_window > 0 ? (float*)(base + o_rope_swa) : d->rope;
     d->amax_ws = base + o_ws; d->d_token = (int*)(base + o_tok); d->d_past = (int64_t*)(base + o_past);
     d->d_next = (int64_t*)(base + o_next); d->d_step = (int*)(base + o_step);
     d->d_tokens = (int64_t*)(base + o_tokens);
@@ -395,6 +444,10 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
         std::vector<float> tab((size_t)c.max_seq * c.head_dim);
         ptm_rope_table_host_scaled(tab.data(), c.max_seq, c.head_dim, c.rope_freq_base, c.rope_scale);
         if ((rc = hip_status(hipMemcpy(d->rope, tab.data(), tab.size() * 4, hipMemcpyHostToDevice))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
+        if (c.swa_window > 0) {  // ModelConfig::layer_rope_freq_base / layer_rope_scale, gguf_model.h:297-302
+            ptm_rope_table_host_scaled(tab.data(), c.max_seq, c.head_dim, c.rope_swa_freq_base, 1.0f);
+            if ((rc = hip_status(hipMemcpy(d->rope_swa, tab.data(), tab.size() * 4, hipMemcpyHostToDevice))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
+        }
     }
     hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, d->stream, d->d_token, 0, d->d_past, (int64_t)0, d->d_step);
     if ((rc = hip_status(hipStreamSynchronize(d->stream))) != PTM_OK) { ptm_decode_destroy(d); return rc; }

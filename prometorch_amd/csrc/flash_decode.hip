@@ -279,6 +279,7 @@ struct AttnArgs {
     int n_heads, n_kv_heads, max_seq, add_one;
     float scale, eps;
     int rope_interleaved;  // 0: NeoX pairs (d, d + HD/2); 1: pairs (2d, 2d + 1) as llama / mistral rotate (hot_loops.cpp:1962-2030)
+    int window;            // > 0: only the last `window` positions are attended to (gemma3 local layers, gguf_model.h:3490-3500)
 };
 
 // one wave: RMSNorm (optional) + NeoX rotation of a head held as pairs (t, t+HD/2); results to dst[HD]
@@ -349,6 +350,17 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     const int64_t t0 = (int64_t)split * FD_CHUNK;
     if (t0 >= total) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t t_begin = (a.window > 0 && total > a.window) ? total - a.window : 0;
+    if (t0 + FD_CHUNK <= t_begin) {
+        // a chunk wholly in front of the window: an empty partial (weight exp(-inf - M) = 0 in the merge)
+        for (int e = tid; e < G * HD; e += FD_THREADS) {
+            const int g = e / HD, d = e % HD;
+            const int64_t oi = (int64_t)split * a.n_heads + kvh * G + g;
+            a.pO[oi * HD + d] = 0.0f;
+            if (d == 0) { a.pM[oi] = -INFINITY; a.pL[oi] = 0.0f; }
+        }
+        return;
+    }
     const int dl = lane % LPP, pl = lane / LPP;
     const int kv_dim = a.n_kv_heads * HD;
     const int64_t col = (int64_t)kvh * HD + dl * 8;
@@ -469,8 +481,8 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
 #pragma unroll
             for (int i = 0; i < 8; ++i) { kreg[pass][i] = s_new[wave][0][dl * 8 + i]; vreg[pass][i] = s_new[wave][1][dl * 8 + i]; }
         }
-        const bool valid = t < total;
-        if (!valid) {  // rows past the end carry weight 0; keep 0 * garbage from producing NaN
+        const bool valid = t < total && t >= t_begin;
+        if (!valid) {  // rows past the end or in front of the window carry weight 0; keep 0 * garbage from producing NaN
 #pragma unroll
             for (int i = 0; i < 8; ++i) vreg[pass][i] = 0.0f;
         }
@@ -611,11 +623,13 @@ int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, f
 
 // ptm_attn_decode_fused that can also leave the output as Q8 activation blocks (o_q8, may be NULL) for a Q4_K output
 // projection.  The decode runtime's entry; not declared in the public header.
-int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, const float* q_norm_w,
-                             const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8, float* partial_O,
-                             float* partial_lse, float* partial_max, const float* rope_table,
-                             int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
-                             float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, ptm_stream_t stream) {
+// window > 0: only the last `window` positions (the new one included) are attended to.
+int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                              const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8, float* partial_O,
+                              float* partial_lse, float* partial_max, const float* rope_table,
+                              int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                              float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
+                              ptm_stream_t stream) {
     if (!Q || !K || !V || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max ||
         !rope_table || !d_past_len)
         return PTM_E_NULL;
@@ -624,7 +638,7 @@ int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, con
     if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
     if (!aligned16(K_cache) || !aligned16(V_cache) || !aligned16(partial_O) || !aligned16(O)) return PTM_E_ALIGN;
     AttnArgs a{Q, K, V, q_norm_w, k_norm_w, rope_table, K_cache, V_cache, partial_O, partial_lse, partial_max,
-               d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps, rope_interleaved ? 1 : 0};
+               d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps, rope_interleaved ? 1 : 0, window > 0 ? window : 0};
     const int G = n_heads / n_kv_heads;
     const dim3 grid(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
     hipStream_t s = as_stream(stream);
@@ -637,6 +651,16 @@ int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, con
                     static_cast<uint8_t*>(o_q8));
 }
 
+int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                             const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8, float* partial_O,
+                             float* partial_lse, float* partial_max, const float* rope_table,
+                             int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                             float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, ptm_stream_t stream) {
+    return ptm_attn_decode_fused_win(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, o_q8, partial_O, partial_lse,
+                                     partial_max, rope_table, n_heads, n_kv_heads, head_dim, d_past_len, max_seq, scale,
+                                     eps, add_one, kv_fp16, rope_interleaved, 0, stream);
+}
+
 int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const float* q_norm_w,
                           const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
                           float* partial_lse, float* partial_max, const float* rope_table,
@@ -645,6 +669,17 @@ int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const 
     return ptm_attn_decode_fused_q8(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, nullptr, partial_O, partial_lse,
                                     partial_max, rope_table, n_heads, n_kv_heads, head_dim, d_past_len, max_seq, scale,
                                     eps, add_one, kv_fp16, rope_interleaved, stream);
+}
+
+int ptm_attn_decode_fused_window(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                                 const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
+                                 float* partial_lse, float* partial_max, const float* rope_table,
+                                 int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                                 float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
+                                 ptm_stream_t stream) {
+    return ptm_attn_decode_fused_win(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, nullptr, partial_O, partial_lse,
+                                     partial_max, rope_table, n_heads, n_kv_heads, head_dim, d_past_len, max_seq, scale,
+                                     eps, add_one, kv_fp16, rope_interleaved, window, stream);
 }
 
 }  // extern "C"

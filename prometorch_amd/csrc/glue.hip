@@ -123,6 +123,37 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
     }
 }
 
+// x[r][:] += RMSNorm(h[r][:]) * w: the post-norm of a gemma2 / gemma3 branch and its residual add
+// (gguf_model.h:3656-3680, :3787-3807); one workgroup per row
+__global__ __launch_bounds__(256) void rms_norm_add_kernel(const float* __restrict__ h, const float* __restrict__ w,
+                                                           float* __restrict__ x, int hidden, float eps, int add_one) {
+    __shared__ float red[4];
+    const float* hr = h + (int64_t)blockIdx.x * hidden;
+    float* xr = x + (int64_t)blockIdx.x * hidden;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < hidden; i += 256) ss = fmaf(hr[i], hr[i], ss);
+    ss = block_sum256(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)hidden + eps);
+    const float one = add_one ? 1.0f : 0.0f;
+    for (int i = threadIdx.x; i < hidden; i += 256) xr[i] = xr[i] + hr[i] * rs * (w[i] + one);
+}
+
+__global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ x, float s, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) x[i] *= s;
+}
+
+// tanh-approximated GELU(gate) * up, the expression of gguf_model.h:3730-3738
+__global__ __launch_bounds__(256) void gelu_mul_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                       float* __restrict__ o, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float x = g[i];
+    const float x3 = x * x * x;
+    const float t = tanhf(0.7978845608028654f * (x + 0.044715f * x3));
+    o[i] = 0.5f * x * (1.0f + t) * u[i];
+}
+
 // in-place per-head RMSNorm: one wave per (row, head)
 __global__ __launch_bounds__(64) void per_head_rms_norm_kernel(float* __restrict__ data, const float* __restrict__ w,
                                                                int head_dim, float eps, int add_one) {
@@ -501,6 +532,31 @@ int ptm_argmax(const float* in, int64_t* out, int64_t n, ptm_stream_t stream) {
     if (!in || !out) return PTM_E_NULL;
     if (n <= 0) return PTM_E_SHAPE;
     hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, as_stream(stream), in, out, n);
+    return launch_status();
+}
+
+int ptm_rms_norm_add(const float* h, const float* weight, float* x, int rows, int hidden, float eps, int add_one,
+                     ptm_stream_t stream) {
+    if (!h || !weight || !x) return PTM_E_NULL;
+    if (rows < 0 || hidden <= 0) return PTM_E_SHAPE;
+    if (rows == 0) return PTM_OK;
+    hipLaunchKernelGGL(rms_norm_add_kernel, dim3(rows), dim3(256), 0, as_stream(stream), h, weight, x, hidden, eps, add_one);
+    return launch_status();
+}
+
+int ptm_scale(float* x, float factor, int64_t n, ptm_stream_t stream) {
+    if (!x) return PTM_E_NULL;
+    if (n < 0) return PTM_E_SHAPE;
+    if (n == 0) return PTM_OK;
+    hipLaunchKernelGGL(scale_kernel, dim3(nblk256(n)), dim3(256), 0, as_stream(stream), x, factor, n);
+    return launch_status();
+}
+
+int ptm_gelu_mul(const float* gate, const float* up, float* out, int64_t n, ptm_stream_t stream) {
+    if (!gate || !up || !out) return PTM_E_NULL;
+    if (n < 0) return PTM_E_SHAPE;
+    if (n == 0) return PTM_OK;
+    hipLaunchKernelGGL(gelu_mul_kernel, dim3(nblk256(n)), dim3(256), 0, as_stream(stream), gate, up, out, n);
     return launch_status();
 }
 

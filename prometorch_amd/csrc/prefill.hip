@@ -130,7 +130,8 @@ __device__ __forceinline__ void pf_load8(const void* base, int64_t elem_off, flo
 template <bool KV16, int HD, int G>
 __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restrict__ Q, const void* __restrict__ Kc,
                                                            const void* __restrict__ Vc, float* __restrict__ O, int rows,
-                                                           int n_heads, int n_kv_heads, int64_t pos0, float scale) {
+                                                           int n_heads, int n_kv_heads, int64_t pos0, float scale,
+                                                           int window) {
     constexpr int LPP = HD / 8, PPW = 64 / LPP;  // lanes per position, positions per wave and pass
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = blockIdx.x * 4 + wave, kvh = blockIdx.y;
@@ -139,6 +140,8 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restri
     const int kv_dim = n_kv_heads * HD;
     const int64_t col = (int64_t)kvh * HD + dl * 8;
     const int64_t limit = pos0 + m;  // last position this row may attend to (itself)
+    // window > 0: the row sees positions (limit - window, limit] only (gemma3 local layers, gguf_model.h:3490-3500)
+    const int64_t lo = (window > 0 && limit + 1 > window) ? limit + 1 - window : 0;
 
     float q[G][8];
 #pragma unroll
@@ -156,14 +159,15 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restri
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[g][i] = 0.0f;
     }
-    const int64_t n_pass = limit / PPW + 1;
+    const int64_t n_pass = limit / PPW + 1, pass0 = lo / PPW;
     float kn[8], vn[8];
     {
-        const int64_t tc = pl <= limit ? pl : limit;
+        const int64_t tf = pass0 * PPW + pl;
+        const int64_t tc = tf <= limit ? tf : limit;
         pf_load8<KV16>(Kc, tc * kv_dim + col, kn);
         pf_load8<KV16>(Vc, tc * kv_dim + col, vn);
     }
-    for (int64_t pass = 0; pass < n_pass; ++pass) {
+    for (int64_t pass = pass0; pass < n_pass; ++pass) {
         float k[8], v[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) { k[i] = kn[i]; v[i] = vn[i]; }
@@ -174,7 +178,7 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restri
             pf_load8<KV16>(Kc, tc * kv_dim + col, kn);
             pf_load8<KV16>(Vc, tc * kv_dim + col, vn);
         }
-        const bool valid = t <= limit;
+        const bool valid = t <= limit && t >= lo;
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float d = 0.0f;
@@ -197,7 +201,7 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restri
     for (int g = 0; g < G; ++g) {
         float M = mrun[g];
         for (int off = LPP; off < 64; off <<= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
-        const float w = pf_exp(mrun[g] - M);  // M is finite: position 0 is always valid for slot 0
+        const float w = pf_exp(mrun[g] - M);  // M is finite: the row's own position is valid for one of the slots
         float l = lsum[g] * w;
         for (int off = LPP; off < 64; off <<= 1) l += __shfl_xor(l, off, 64);
         const float inv = 1.0f / (l + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
@@ -389,8 +393,8 @@ static int prefill_attn_mfma_launch(int G, hipStream_t s, const float* Q, const 
 
 template <bool KV16, int HD>
 static int prefill_attn_launch(int G, dim3 grid, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* O,
-                               int rows, int n_heads, int n_kv_heads, int64_t pos0, float scale) {
-#define PTM_PA(GG) hipLaunchKernelGGL((prefill_attn_kernel<KV16, HD, GG>), grid, dim3(256), 0, s, Q, Kc, Vc, O, rows, n_heads, n_kv_heads, pos0, scale)
+                               int rows, int n_heads, int n_kv_heads, int64_t pos0, float scale, int window) {
+#define PTM_PA(GG) hipLaunchKernelGGL((prefill_attn_kernel<KV16, HD, GG>), grid, dim3(256), 0, s, Q, Kc, Vc, O, rows, n_heads, n_kv_heads, pos0, scale, window)
     switch (G) {
         case 1: PTM_PA(1); break;
         case 2: PTM_PA(2); break;
@@ -441,6 +445,13 @@ int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float
 int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cache, float* O, int rows, int n_heads,
                           int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float scale, int kv_fp16,
                           ptm_stream_t stream) {
+    return ptm_prefill_attention_window(Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, head_dim, pos0, max_seq, scale,
+                                        kv_fp16, 0, stream);
+}
+
+int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void* V_cache, float* O, int rows, int n_heads,
+                                 int n_kv_heads, int head_dim, int64_t pos0, int max_seq, float scale, int kv_fp16,
+                                 int window, ptm_stream_t stream) {
     if (!Q || !K_cache || !V_cache || !O) return PTM_E_NULL;
     if (rows <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
     if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
@@ -450,14 +461,16 @@ int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cac
     const int G = n_heads / n_kv_heads;
     const dim3 grid((rows + 3) / 4, n_kv_heads);
     hipStream_t s = as_stream(stream);
-    if (kv_fp16 && rows >= PTM_PREFILL_MFMA_MIN_ROWS && (G == 1 || G == 2 || G == 4 || G == 8))
+    if (window < 0) window = 0;
+    // the matrix-core kernel walks every tile from position 0; windowed layers take the fp32 kernel, which starts at the window
+    if (window == 0 && kv_fp16 && rows >= PTM_PREFILL_MFMA_MIN_ROWS && (G == 1 || G == 2 || G == 4 || G == 8))
         return head_dim == 128 ? prefill_attn_mfma_launch<128>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
                                : prefill_attn_mfma_launch<64>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
     if (kv_fp16)
-        return head_dim == 128 ? prefill_attn_launch<true, 128>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
-                               : prefill_attn_launch<true, 64>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
-    return head_dim == 128 ? prefill_attn_launch<false, 128>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
-                           : prefill_attn_launch<false, 64>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
+        return head_dim == 128 ? prefill_attn_launch<true, 128>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
+                               : prefill_attn_launch<true, 64>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
+    return head_dim == 128 ? prefill_attn_launch<false, 128>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
+                           : prefill_attn_launch<false, 64>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
 }
 
 }  // extern "C"

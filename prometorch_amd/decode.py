@@ -25,7 +25,8 @@ class Decoder:
 
     layers: list of dicts with (qtype, uint8[rows, stride]) per projection name and fp32 norm
     vectors 'attn_norm', 'ffn_norm', 'q_norm', 'k_norm' (the last two None for a model without QK-norm; optional
-    'q_bias', 'k_bias', 'v_bias' added to the projections' outputs;
+    'q_bias', 'k_bias', 'v_bias' added to the projections' outputs; optional 'post_attn_norm', 'post_ffn_norm' and the cfg keys
+    'scale_embeddings', 'ffn_gelu', 'swa_window', 'swa_pattern', 'rope_swa_base', 'rope_scale' of a gemma-style model;
     cfg['rope_interleaved'] selects llama-style rotation pairs); head: {'lm_head': uint8 table (Q6_K unless 'lm_head_type' says otherwise),
     'out_norm': fp32}.  The token-embedding is the tied Q6_K table unless embedding_f32 is given."""
 
@@ -47,7 +48,8 @@ class Decoder:
                 t = _upload_bytes(W)
                 self._keep.append(t)
                 setattr(arr[i], name, QWeight(t.data_ptr(), qt, W.shape[0], _lib.weight_cols(qt, W.shape[1]), W.shape[1]))
-            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias"):
+            for name in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias", "post_attn_norm",
+                         "post_ffn_norm"):
                 if Ld.get(name) is None:  # q_norm / k_norm: a model without QK-norm; biases: qwen2-style only
                     setattr(arr[i], name, None)
                     continue
@@ -74,6 +76,11 @@ class Decoder:
         c.use_graph = int(use_graph)
         c.rope_interleaved = int(bool(cfg.get("rope_interleaved", False)))
         c.rope_scale = float(cfg.get("rope_scale", 1.0))
+        c.scale_embeddings = int(bool(cfg.get("scale_embeddings", False)))
+        c.ffn_gelu = int(bool(cfg.get("ffn_gelu", False)))
+        c.swa_window = int(cfg.get("swa_window", 0))
+        c.swa_pattern = int(cfg.get("swa_pattern", 0))
+        c.rope_swa_freq_base = float(cfg.get("rope_swa_base", 10000.0))
         if embedding_f32 is not None:
             e = embedding_f32 if isinstance(embedding_f32, torch.Tensor) else torch.from_numpy(embedding_f32)
             e = e.to(device="cuda", dtype=torch.float32).contiguous()

@@ -228,14 +228,37 @@ def launch_flash_decode_fp16_graph(Q, K_cache_fp16, V_cache_fp16, O, partial_O, 
 
 def attn_decode_fused(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, partial_O, partial_lse, partial_max,
                       rope_table, n_heads, n_kv_heads, head_dim, d_past_len, max_seq, scale, eps, add_one=False,
-                      kv_fp16=True, stream=None, rope_interleaved=False):
+                      kv_fp16=True, stream=None, rope_interleaved=False, window=0):
     """launch_fused_qknorm_rope_kvwrite_graph + launch_flash_decode(_fp16)_graph fused (one launch + a small merge launch)
-    (CUDAOps.h:653-673; issued back to back at gguf_model.h:2785-2832)."""
-    check(_L().ptm_attn_decode_fused(_ptr(Q), _ptr(K), _ptr(V), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(K_cache),
-                                    _ptr(V_cache), _ptr(O), _ptr(partial_O), _ptr(partial_lse), _ptr(partial_max),
-                                    _ptr(rope_table), n_heads, n_kv_heads, head_dim, _ptr(d_past_len),
-                                    max_seq, scale, eps, int(add_one), int(kv_fp16), int(rope_interleaved), _stream(stream)),
+    (CUDAOps.h:653-673; issued back to back at gguf_model.h:2785-2832).  window > 0: only the last `window` positions."""
+    check(_L().ptm_attn_decode_fused_window(_ptr(Q), _ptr(K), _ptr(V), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(K_cache),
+                                           _ptr(V_cache), _ptr(O), _ptr(partial_O), _ptr(partial_lse), _ptr(partial_max),
+                                           _ptr(rope_table), n_heads, n_kv_heads, head_dim, _ptr(d_past_len),
+                                           max_seq, scale, eps, int(add_one), int(kv_fp16), int(rope_interleaved),
+                                           int(window), _stream(stream)),
           "attn_decode_fused")
+
+
+def gelu_mul(gate, up, out, n, stream=None):
+    """tanh-GELU(gate) * up (gguf_model.h:3730-3738)."""
+    check(_L().ptm_gelu_mul(_ptr(gate), _ptr(up), _ptr(out), n, _stream(stream)), "gelu_mul")
+
+
+def rms_norm_add(h, weight, x, rows, hidden, eps, add_one=False, stream=None):
+    """x[r] += RMSNorm(h[r]) * weight: a gemma post-norm with its residual add (gguf_model.h:3656-3680)."""
+    check(_L().ptm_rms_norm_add(_ptr(h), _ptr(weight), _ptr(x), rows, hidden, eps, int(add_one), _stream(stream)), "rms_norm_add")
+
+
+def scale(x, factor, n, stream=None):
+    check(_L().ptm_scale(_ptr(x), factor, n, _stream(stream)), "scale")
+
+
+def prefill_attention_window(Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, head_dim, pos0, max_seq, scale, kv_fp16, window,
+                             stream=None):
+    """Causal attention of prompt rows over the last `window` positions each (gguf_model.h:3490-3500)."""
+    check(_L().ptm_prefill_attention_window(_ptr(Q), _ptr(K_cache), _ptr(V_cache), _ptr(O), rows, n_heads, n_kv_heads, head_dim,
+                                           pos0, max_seq, scale, int(kv_fp16), int(window), _stream(stream)),
+          "prefill_attention_window")
 
 
 def launch_silu_mul(gate, up, output, n, stream=None):

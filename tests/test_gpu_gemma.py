@@ -1,0 +1,220 @@
+"""GPU parity of the gemma3-style variant of the decode path (torch/io/gguf_model.h:74-88, :184-197): embedding rows
+times sqrt(hidden), tanh-GELU gate, RMSNorm of each branch's output before the residual add, and alternating layers --
+local ones attend to the last swa_window positions and rotate with their own base, global ones see everything and
+rotate with linearly scaled positions.  The compiled reference's forward_decode_cpu run of synth.tiny_gemma is
+golden_gemma.npz.  Bars are those of the qwen3-style tests."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import bits
+from prometorch_amd import ops, synth
+from test_gpu_decode import check_step_errors
+from test_gpu_llama import follow_sensitive
+from test_gpu_prefill import check_kv_rows, check_logits
+
+pytestmark = pytest.mark.gpu
+
+
+def cu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.fixture(scope="module")
+def golden_gemma():
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_gemma.npz"))
+
+
+def tiny_gemma_with_cache(seeds, n=19):
+    cfg, layers, head = synth.tiny_gemma(seeds["tiny"])
+    kv = [synth.make_kv_prefill(seeds["tiny"], i, cfg, n) for i in range(cfg["n_layers"])]
+    return cfg, layers, head, kv
+
+
+def test_gelu_mul_rms_norm_add_and_scale(dev, po):
+    r = synth.rng_for(93)
+    gate = (3 * r.standard_normal(9728, dtype=np.float32)).astype(np.float32)
+    up = r.standard_normal(9728, dtype=np.float32)
+    want = gate.copy()
+    po.lib().po_gelu_mul.argtypes = [po._vp, po._vp, po._i64]
+    po.lib().po_gelu_mul(po._p(want), po._p(up), want.size)
+    out = torch.empty(9728, device="cuda")
+    ops.gelu_mul(cu(gate), cu(up), out, 9728)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()   # tanhf of the device library
+    for rows, H in ((1, 2560), (5, 256)):
+        h = r.standard_normal((rows, H), dtype=np.float32)
+        x = r.standard_normal((rows, H), dtype=np.float32)
+        w = (1 + 0.1 * r.standard_normal(H, dtype=np.float32)).astype(np.float32)
+        dx = cu(x)
+        ops.rms_norm_add(cu(h), cu(w), dx, rows, H, 1e-6)
+        want = np.stack([x[i] + po.rmsnorm(h[i], w, 1e-6, seq=False) for i in range(rows)])
+        assert np.abs(dx.cpu().numpy() - want).max() <= 2e-6 * np.abs(want).max()
+    v = r.standard_normal(2560, dtype=np.float32)
+    dv = cu(v)
+    ops.scale(dv, float(np.sqrt(np.float32(2560))), 2560)
+    assert np.array_equal(bits(dv.cpu().numpy()), bits(v * np.sqrt(np.float32(2560))))
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+@pytest.mark.parametrize("nh,nkv,hd,past,window", [(32, 8, 128, 2048, 1024), (4, 2, 64, 19, 8), (8, 4, 128, 130, 64),
+                                                  (8, 8, 128, 5, 8), (16, 2, 64, 200, 1), (32, 8, 128, 511, 512)])
+def test_attn_decode_fused_window_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past, window):
+    """QK-norm + NeoX rotation + KV append + attention over the last `window` positions + merge, three tokens in a row:
+    chunks wholly in front of the window are skipped, the chunk the window starts in is masked position by position."""
+    max_seq = ((past + 3 + 63) // 64 + 1) * 64
+    r = synth.rng_for(48, nh, hd, past)
+    kvd = nkv * hd
+    kf = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    vf = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    dt = torch.float16 if kv_fp16 else torch.float32
+    Kc, Vc = cu(kf).to(dt), cu(vf).to(dt)
+    Kc[past:] = float("nan")
+    Vc[past:] = float("nan")
+    S = ops.flash_decode_num_splits(max_seq)
+    pO = torch.full((S * nh * hd,), float("nan"), device="cuda")
+    pL = torch.full((S * nh,), float("nan"), device="cuda")
+    pM = torch.full((S * nh,), float("nan"), device="cuda")
+    table = ops.rope_table(max_seq, hd, 1e4).cuda()
+    O = torch.empty(nh * hd, device="cuda")
+    d_past = torch.zeros(1, dtype=torch.int64, device="cuda")
+    scale = 1.0 / np.sqrt(hd)
+    qw = (1 + 0.1 * r.standard_normal(hd, dtype=np.float32)).astype(np.float32)
+    kw = (1 + 0.1 * r.standard_normal(hd, dtype=np.float32)).astype(np.float32)
+    for step in range(3):
+        pos = past + step
+        q = synth.make_x(r, nh * hd).astype(np.float32)
+        k = synth.make_x(r, kvd).astype(np.float32)
+        v = synth.make_x(r, kvd)
+        qn = np.concatenate([po.rmsnorm(q[h * hd:(h + 1) * hd], qw, 1e-6, seq=False) for h in range(nh)])
+        kn = np.concatenate([po.rmsnorm(k[h * hd:(h + 1) * hd], kw, 1e-6, seq=False) for h in range(nkv)])
+        c, s = po.rope_tables(pos, hd, 1e4)
+        qr, kr = po.rope_neox(qn, kn, c, s, nh, nkv, hd)
+        kf[pos] = kr.astype(np.float16).astype(np.float32) if kv_fp16 else kr
+        vf[pos] = v.astype(np.float16).astype(np.float32) if kv_fp16 else v
+        t_start = max(0, pos + 1 - window)
+        want = np.concatenate([po.attn_head(qr[h * hd:(h + 1) * hd], kf, vf, pos + 1, kvd, hd, scale,
+                                            col0=(h // (nh // nkv)) * hd, t_start=t_start) for h in range(nh)])
+        full = np.concatenate([po.attn_head(qr[h * hd:(h + 1) * hd], kf, vf, pos + 1, kvd, hd, scale,
+                                            col0=(h // (nh // nkv)) * hd) for h in range(nh)])
+        d_past.fill_(pos)
+        ops.attn_decode_fused(cu(q), cu(k), cu(v), cu(qw), cu(kw), Kc, Vc, O, pO, pL, pM, table, nh, nkv, hd, d_past,
+                              max_seq, scale, 1e-6, kv_fp16=kv_fp16, window=window)
+        torch.cuda.synchronize()
+        got = O.cpu().numpy()
+        assert np.all(np.isfinite(got)), (step, pos)
+        assert np.abs(got - want).max() <= 3e-5 * max(np.abs(want).max(), 1e-3) + 1e-6, (step, pos)
+        if t_start > 0:
+            assert np.abs(got - full).max() > 1e-3 * np.abs(full).max()   # the window does cut something off
+        kf[pos] = Kc[pos].float().cpu().numpy()
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+@pytest.mark.parametrize("rows,nh,nkv,hd,pos0,window", [(23, 4, 2, 64, 0, 8), (40, 8, 4, 128, 100, 64), (7, 8, 8, 128, 30, 1),
+                                                       (64, 16, 4, 64, 0, 1024)])
+def test_prefill_attention_window_vs_oracle(dev, po, kv_fp16, rows, nh, nkv, hd, pos0, window):
+    r = synth.rng_for(49, rows, hd, pos0)
+    kvd, max_seq = nkv * hd, pos0 + rows + 3
+    kf = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    vf = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    q = r.standard_normal((rows, nh * hd), dtype=np.float32)
+    dt = torch.float16 if kv_fp16 else torch.float32
+    O = torch.empty(rows, nh * hd, device="cuda")
+    scale = 1.0 / np.sqrt(hd)
+    ops.prefill_attention_window(cu(q), cu(kf).to(dt), cu(vf).to(dt), O, rows, nh, nkv, hd, pos0, max_seq, scale, kv_fp16, window)
+    got = O.cpu().numpy()
+    for m in range(rows):
+        T = pos0 + m + 1
+        want = np.concatenate([po.attn_head(q[m, h * hd:(h + 1) * hd], kf, vf, T, kvd, hd, scale, col0=(h // (nh // nkv)) * hd,
+                                            t_start=max(0, T - window)) for h in range(nh)])
+        assert np.abs(got[m] - want).max() <= 3e-5 * max(np.abs(want).max(), 1e-3) + 1e-6, m
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_gemma_decode_fp32_kv_vs_reference_golden(dev, golden_gemma, seeds, use_graph):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_gemma_with_cache(seeds)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False, use_graph=use_graph)
+    for i, (k, v) in enumerate(kv):
+        dec.set_kv(i, k, v)
+    dec.set_past_len(19)
+    tok, errs = 3, []
+    for st in range(16):
+        tok = dec.step(tok)
+        ref = golden_gemma["logits"][st]
+        errs.append(np.abs(dec.logits() - ref).max() / ref.std())
+        assert tok == int(golden_gemma["tokens"][st]), st
+    check_step_errors(errs)
+    dec.close()
+
+
+@pytest.mark.parametrize("past", [19, 3])
+def test_gemma_decode_fp16_kv_vs_oracle_and_chained_greedy(dev, po, seeds, past):
+    """past = 3: the window of 8 is crossed during the run."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_gemma_with_cache(seeds, past)
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=True)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=True)
+    dec2 = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=True)
+    for i, (k, v) in enumerate(kv):
+        om.set_kv(i, k, v)
+        dec.set_kv(i, k, v)
+        dec2.set_kv(i, k, v)
+    dec.set_past_len(past)
+    dec2.set_past_len(past)
+    tok_o = tok_g = 3
+    want, errs = [], []
+    for st in range(24):
+        tok_o = om.step(tok_o)
+        tok_g = dec.step(tok_g)
+        want.append(tok_o)
+        errs.append(np.abs(dec.logits() - om.logits).max() / om.logits.std())
+        assert tok_g == tok_o, st
+    check_step_errors(errs)
+    assert dec2.greedy(3, 24) == want
+    dec.close()
+    dec2.close()
+
+
+@pytest.mark.parametrize("feature", ["scale_embeddings", "ffn_gelu", "swa_window", "rope_swa_base", "post_attn_norm", "post_ffn_norm"])
+def test_gemma_features_are_not_ignored(dev, seeds, golden_gemma, feature):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_gemma_with_cache(seeds)
+    if feature.startswith("post_"):
+        layers = [{k: v for k, v in L.items() if k != feature} for L in layers]
+    else:
+        cfg = dict(cfg, **{feature: {"scale_embeddings": False, "ffn_gelu": False, "swa_window": 0, "rope_swa_base": 1.0e6}[feature]})
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False, use_graph=False)
+    for i, (k, v) in enumerate(kv):
+        dec.set_kv(i, k, v)
+    dec.set_past_len(19)
+    dec.step(3)
+    ref = golden_gemma["logits"][0]
+    assert np.abs(dec.logits() - ref).max() > 1e-2 * ref.std()
+    dec.close()
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+@pytest.mark.parametrize("pos0,n,chunk", [(0, 23, 0), (0, 23, 7), (19, 12, 5)])
+def test_gemma_prefill_vs_oracle_token_by_token(dev, po, seeds, kv_fp16, pos0, n, chunk):
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = synth.tiny_gemma(seeds["tiny"])
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=kv_fp16)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=kv_fp16, use_graph=True)
+    if pos0:
+        for i in range(cfg["n_layers"]):
+            k, v = synth.make_kv_prefill(seeds["tiny"], i, cfg, pos0)
+            om.set_kv(i, k, v)
+            dec.set_kv(i, k, v)
+        dec.set_past_len(pos0)
+    prompt = [int(t) for t in synth.rng_for(69, pos0, n).integers(0, cfg["vocab"], n)]
+    for t in prompt:
+        tok_o = om.step(t)
+    tok_g = dec.prefill(prompt, chunk_rows=chunk)
+    for li in range(cfg["n_layers"]):
+        for nm, gpu_c, cpu_c in (("k", dec.k_cache[li], om.k_cache[li]), ("v", dec.v_cache[li], om.v_cache[li])):
+            check_kv_rows(gpu_c[pos0:pos0 + n].float().cpu().numpy(), cpu_c[pos0:pos0 + n], li, nm)
+    check_logits(dec.logits(), om.logits, tok_g, tok_o, "prefill")
+    follow_sensitive(dec, om, tok_o, 6)
+    dec.close()
