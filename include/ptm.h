@@ -177,13 +177,20 @@ int ptm_fp16_kv_cache_write(const float* src, void* dst_cache_fp16, int64_t num_
  * Scratch (caller-owned): partial_O [S*n_heads*head_dim], partial_lse [S*n_heads] (sum of exp),
  * partial_max [S*n_heads] with S = ptm_flash_decode_num_splits(max_seq).
  * Replaces launch_flash_decode(_fp16)(_graph) + flash_decode_num_splits / _kv_chunk_size
- * (CUDAOps.h:543-557, :641-673). head_dim must be 64 or 128. */
+ * (CUDAOps.h:543-557, :641-673). head_dim must be 64, 128 or 256. */
 int ptm_flash_decode_kv_chunk_size(void);
 int ptm_flash_decode_num_splits(int total_seq);
 int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, float* O,
                      float* partial_O, float* partial_lse, float* partial_max, int n_heads,
                      int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq, float scale,
                      int kv_fp16, ptm_stream_t stream);
+/* The same over a sliding window (window > 0: only the last `window` positions, gguf_model.h:3490-3500); o_q8, when not
+ * NULL, also receives the output as Q8 activation blocks (ptm_q8_bytes(n_heads * head_dim), 16-byte aligned) for a Q4_K
+ * output projection. */
+int ptm_flash_decode_window(const float* Q, const void* K_cache, const void* V_cache, float* O, void* o_q8,
+                            float* partial_O, float* partial_lse, float* partial_max, int n_heads, int n_kv_heads,
+                            int head_dim, const int64_t* d_past_len, int max_seq, float scale, int kv_fp16, int window,
+                            ptm_stream_t stream);
 
 /* The two operators above fused: one launch does per-head QK-norm + NeoX RoPE of Q and of the new K
  * row, the K/V append at row *d_past_len and the split-KV attention over rows [0, *d_past_len]; a

@@ -95,6 +95,7 @@ SIGNATURES = {
     "ptm_flash_decode_num_splits": (i32, [i32]),
     "ptm_flash_decode": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, i32, vp]),
     "ptm_attn_decode_fused": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, f32, i32, i32, i32, vp]),
+    "ptm_flash_decode_window": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, i32, i32, vp]),
     "ptm_attn_decode_fused_window": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, f32, i32, i32, i32, i32, vp]),
     "ptm_silu_mul": (i32, [vp, vp, vp, i64, vp]),
     "ptm_embedding_row": (i32, [vp, vp, vp, i32, vp]),

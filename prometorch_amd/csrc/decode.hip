@@ -200,6 +200,15 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
         // a Q4_K output projection takes the attention output as the Q8 blocks the merge kernel leaves beside the fp32
         // vector: its prologue then copies 1.25 bytes per value instead of fetching and quantising 4
         const bool o_q8 = L.o.ggml_type == PTM_TYPE_Q4_K;
+        if (hd == 256) {
+            // heads this wide (gemma3) take the plain pair of launches: norm + rotation + K/V append, then split-KV attention
+            PTM_TRY(ptm_qknorm_rope_kvwrite(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, c.n_heads, c.n_kv_heads,
+                                            hd, d->d_past, c.max_seq, 0.0f, local ? d->rope_swa : d->rope, c.rms_eps, 0,
+                                            c.rope_interleaved ? 0 : 1, c.kv_fp16, s));
+            PTM_TRY(ptm_flash_decode_window(d->q, L.k_cache, L.v_cache, d->attn, o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM,
+                                            c.n_heads, c.n_kv_heads, hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd),
+                                            c.kv_fp16, local ? c.swa_window : 0, s));
+        } else
         PTM_TRY(ptm_attn_decode_fused_win(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn,
                                           o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM, local ? d->rope_swa : d->rope,
                                           c.n_heads, c.n_kv_heads, hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd),
@@ -380,7 +389,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
         c.max_seq <= 0 || (c.hidden % 256) || (c.inter % 256) || ((c.n_heads * c.head_dim) % 256) ||
         (c.n_heads % c.n_kv_heads))
         return PTM_E_SHAPE;
-    if (c.head_dim != 64 && c.head_dim != 128) return PTM_E_UNSUPPORTED;
+    if (c.head_dim != 64 && c.head_dim != 128 && c.head_dim != 256) return PTM_E_UNSUPPORTED;
     if (c.swa_window < 0 || c.swa_pattern < 0 || (c.swa_window > 0 && !(c.rope_swa_freq_base > 0.0f))) return PTM_E_SHAPE;
     const int H = c.hidden, qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim;
     int rc = qw_check(c.lm_head, c.vocab, H);

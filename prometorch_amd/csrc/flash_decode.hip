@@ -48,7 +48,7 @@ template <bool KV16, int HD, int G>
 __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     const float* __restrict__ Q, const void* __restrict__ Kc, const void* __restrict__ Vc,
     float* __restrict__ pO, float* __restrict__ pL, float* __restrict__ pM, int n_heads, int n_kv_heads,
-    const int64_t* __restrict__ d_past, int max_seq, float scale) {
+    const int64_t* __restrict__ d_past, int max_seq, float scale, int window) {
     constexpr int LPP = HD / 8;         // lanes per position (each lane owns 8 dims)
     constexpr int PPW = 64 / LPP;       // positions per wave per pass
     constexpr int PPB = PPW * 4;        // positions per workgroup per pass
@@ -62,6 +62,17 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     const int64_t t0 = (int64_t)split * FD_CHUNK;
     if (t0 >= total) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // window > 0: only positions [total - window, total) count; a chunk wholly in front of them leaves an empty partial
+    const int64_t t_begin = (window > 0 && total > window) ? total - window : 0;
+    if (t0 + FD_CHUNK <= t_begin) {
+        for (int e = tid; e < G * HD; e += FD_THREADS) {
+            const int g = e / HD, d = e % HD;
+            const int64_t oi = (int64_t)split * n_heads + kvh * G + g;
+            pO[oi * HD + d] = 0.0f;
+            if (d == 0) { pM[oi] = -INFINITY; pL[oi] = 0.0f; }
+        }
+        return;
+    }
     const int dl = lane % LPP, pl = lane / LPP;
     const int kv_dim = n_kv_heads * HD;
     const int64_t col = (int64_t)kvh * HD + dl * 8;
@@ -89,13 +100,13 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
         const int tl = pass * PPB + wave * PPW + pl;
-        const bool valid = t0 + tl < total;
+        const bool valid = t0 + tl < total && t0 + tl >= t_begin;
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float d = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], kreg[pass][i], d);
-            d = (LPP == 16) ? sum16(d) : sum8(d);
+            d = sum_lanes<LPP>(d);
             if (dl == 0) s_p[g][tl] = valid ? d * scale : -INFINITY;
         }
     }
@@ -252,7 +263,9 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
 
 static int fd_merge(int head_dim, int n_heads, hipStream_t s, const float* pO, const float* pL, const float* pM, float* O,
                     const int64_t* d_past, int max_seq, uint8_t* q8_out = nullptr) {
-    if (head_dim == 128)
+    if (head_dim == 256)
+        hipLaunchKernelGGL(flash_decode_merge_kernel<256>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq, q8_out);
+    else if (head_dim == 128)
         hipLaunchKernelGGL(flash_decode_merge_kernel<128>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq, q8_out);
     else
         hipLaunchKernelGGL(flash_decode_merge_kernel<64>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq, q8_out);
@@ -491,7 +504,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
             float d = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], kreg[pass][i], d);
-            d = (LPP == 16) ? sum16(d) : sum8(d);
+            d = sum_lanes<LPP>(d);
             sc[g][pass] = valid ? d * a.scale : -INFINITY;
         }
     }
@@ -574,10 +587,10 @@ static int attn_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
 template <bool KV16, int HD>
 static int fd_launch_g(int G, dim3 grid, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* pO,
                        float* pL, float* pM, int n_heads, int n_kv_heads, const int64_t* d_past, int max_seq,
-                       float scale) {
+                       float scale, int window = 0) {
 #define PTM_FD(GG)                                                                                              \
     hipLaunchKernelGGL((flash_decode_partial_kernel<KV16, HD, GG>), grid, dim3(FD_THREADS), 0, s, Q, Kc, Vc, pO, \
-                       pL, pM, n_heads, n_kv_heads, d_past, max_seq, scale)
+                       pL, pM, n_heads, n_kv_heads, d_past, max_seq, scale, window)
     switch (G) {
         case 1: PTM_FD(1); break;
         case 2: PTM_FD(2); break;
@@ -601,24 +614,32 @@ int ptm_flash_decode_num_splits(int total_seq) { return total_seq <= 0 ? 0 : (to
 int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, float* O, float* partial_O,
                      float* partial_lse, float* partial_max, int n_heads, int n_kv_heads, int head_dim,
                      const int64_t* d_past_len, int max_seq, float scale, int kv_fp16, ptm_stream_t stream) {
+    return ptm_flash_decode_window(Q, K_cache, V_cache, O, nullptr, partial_O, partial_lse, partial_max, n_heads, n_kv_heads,
+                                   head_dim, d_past_len, max_seq, scale, kv_fp16, 0, stream);
+}
+
+int ptm_flash_decode_window(const float* Q, const void* K_cache, const void* V_cache, float* O, void* o_q8,
+                            float* partial_O, float* partial_lse, float* partial_max, int n_heads, int n_kv_heads,
+                            int head_dim, const int64_t* d_past_len, int max_seq, float scale, int kv_fp16, int window,
+                            ptm_stream_t stream) {
     if (!Q || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max || !d_past_len)
         return PTM_E_NULL;
     if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
-    if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return PTM_E_UNSUPPORTED;
     if (!aligned16(Q) || !aligned16(K_cache) || !aligned16(V_cache)) return PTM_E_ALIGN;
+    if (o_q8 && (reinterpret_cast<uintptr_t>(o_q8) & 15u)) return PTM_E_ALIGN;
+    if (window < 0) window = 0;
     const int G = n_heads / n_kv_heads;
     const dim3 grid(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
     hipStream_t s = as_stream(stream);
     int rc;
-    if (kv_fp16) {
-        rc = head_dim == 128 ? fd_launch_g<true, 128>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale)
-                             : fd_launch_g<true, 64>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale);
-    } else {
-        rc = head_dim == 128 ? fd_launch_g<false, 128>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale)
-                             : fd_launch_g<false, 64>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale);
-    }
+#define PTM_FDW(KV, HDV) fd_launch_g<KV, HDV>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale, window)
+    if (kv_fp16) rc = head_dim == 256 ? PTM_FDW(true, 256) : head_dim == 128 ? PTM_FDW(true, 128) : PTM_FDW(true, 64);
+    else rc = head_dim == 256 ? PTM_FDW(false, 256) : head_dim == 128 ? PTM_FDW(false, 128) : PTM_FDW(false, 64);
+#undef PTM_FDW
     if (rc != PTM_OK) return rc;
-    return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq);
+    return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
+                    static_cast<uint8_t*>(o_q8));
 }
 
 // ptm_attn_decode_fused that can also leave the output as Q8 activation blocks (o_q8, may be NULL) for a Q4_K output

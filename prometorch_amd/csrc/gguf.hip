@@ -385,9 +385,13 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
     // three decode steps are built here, all RMSNorm + SwiGLU: qwen3 (per-head QK-norm, rotation pairs half a head
     // apart), qwen2 (no QK-norm, the same pairs, bias vectors on q / k / v) and llama, which mistral files also carry
     // (no QK-norm, interleaved pairs (2d, 2d+1)); gguf_model.h:194-217 makes the same split by architecture name
+    // gemma3 (gguf_model.h:157-197): QK-norm, NeoX pairs, embedding rows times sqrt(hidden), tanh-GELU gate, post-norm
+    // vectors, sliding-window layers (every sliding_window_pattern-th layer global, 6 when the key is missing) with
+    // their own rotation base
     const bool is_llama = arch == "llama";
-    const bool has_qk_norm = arch == "qwen3";
-    if (arch != "qwen3" && arch != "qwen2" && !is_llama) { ptm_model_free(m); return PTM_E_UNSUPPORTED; }
+    const bool is_gemma3 = arch == "gemma3";
+    const bool has_qk_norm = arch == "qwen3" || is_gemma3;
+    if (arch != "qwen3" && arch != "qwen2" && !is_llama && !is_gemma3) { ptm_model_free(m); return PTM_E_UNSUPPORTED; }
     auto geti = [&](const char* key, int64_t def, bool required) -> int64_t {
         int64_t v = def;
         const int r = ptm_gguf_get_int(m->file, (arch + "." + key).c_str(), &v);
@@ -427,6 +431,16 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
     c.kv_fp16 = kv_fp16 ? 1 : 0;
     c.use_graph = use_graph ? 1 : 0;
     c.rope_interleaved = is_llama ? 1 : 0;
+    if (is_gemma3) {
+        c.scale_embeddings = 1;
+        c.ffn_gelu = 1;
+        c.swa_window = (int32_t)geti("attention.sliding_window", 0, false);
+        c.swa_pattern = (int32_t)geti("attention.sliding_window_pattern", 0, false);
+        if (c.swa_window > 0 && c.swa_pattern == 0) c.swa_pattern = 6;  // gguf_model.h:166-170
+        double fb = 10000.0;
+        (void)ptm_gguf_get_float(m->file, (arch + ".rope.freq_base_swa").c_str(), &fb);
+        c.rope_swa_freq_base = (float)fb;
+    }
     // vocabulary size from the embedding table [hidden x vocab]
     ptm_gguf_tensor emb{};
     PTM_L(ptm_gguf_find_tensor(m->file, "token_embd.weight", &emb));
@@ -482,6 +496,10 @@ int ptm_model_load_gguf(const char* path, int max_seq, int kv_fp16, int use_grap
         } else {
             PTM_L(load_vector(m, p + "attn_q_norm.weight", c.head_dim, &L.q_norm));
             PTM_L(load_vector(m, p + "attn_k_norm.weight", c.head_dim, &L.k_norm));
+        }
+        if (is_gemma3) {  // LayerWeights::post_attention_norm / post_ffw_norm
+            PTM_L(load_vector(m, p + "post_attention_norm.weight", c.hidden, &L.post_attn_norm));
+            PTM_L(load_vector(m, p + "post_ffw_norm.weight", c.hidden, &L.post_ffn_norm));
         }
         PTM_L(load_vector(m, p + "ffn_norm.weight", c.hidden, &L.ffn_norm));
         PTM_L(load_matrix(m, p + "ffn_gate.weight", c.inter, c.hidden, &L.gate));

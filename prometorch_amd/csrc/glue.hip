@@ -189,22 +189,38 @@ __global__ __launch_bounds__(64) void qknorm_rope_kvwrite_kernel(float* __restri
     float* vec = (is_k ? K : Q) + (int64_t)h * head_dim;
     const float* nw = is_k ? kw : qw;
     const int half = head_dim / 2;
-    const int t = threadIdx.x;
-    const bool on = t < half;
-    const int i0 = neox ? t : 2 * t, i1 = neox ? t + half : 2 * t + 1;
-    float x0 = on ? vec[i0] : 0.0f, x1 = on ? vec[i1] : 0.0f;
+    // thread t owns rotation pairs t and t + 64 (the second only for heads wider than 128)
+    float x0[2], x1[2];
+    int i0[2], i1[2];
+    bool on[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int t = threadIdx.x + 64 * j;
+        on[j] = t < half;
+        i0[j] = neox ? t : 2 * t;
+        i1[j] = neox ? t + half : 2 * t + 1;
+        x0[j] = on[j] ? vec[i0[j]] : 0.0f;
+        x1[j] = on[j] ? vec[i1[j]] : 0.0f;
+    }
     if (nw) {
-        float ss = fmaf(x0, x0, 0.0f);
-        ss = fmaf(x1, x1, ss);
+        float ss = fmaf(x0[0], x0[0], 0.0f);
+        ss = fmaf(x1[0], x1[0], ss);
+        ss = fmaf(x0[1], x0[1], ss);
+        ss = fmaf(x1[1], x1[1], ss);
         ss = sum64(ss);
         const float rs = 1.0f / sqrtf(ss / (float)head_dim + eps);
         const float one = add_one ? 1.0f : 0.0f;
-        if (on) {
-            x0 = x0 * rs * (nw[i0] + one);
-            x1 = x1 * rs * (nw[i1] + one);
-        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            if (on[j]) {
+                x0[j] = x0[j] * rs * (nw[i0[j]] + one);
+                x1[j] = x1[j] * rs * (nw[i1[j]] + one);
+            }
     }
-    if (on) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        if (!on[j]) continue;
+        const int t = threadIdx.x + 64 * j;
         float c, s;
         if (table) {
             c = table[pos * head_dim + t];
@@ -215,27 +231,27 @@ __global__ __launch_bounds__(64) void qknorm_rope_kvwrite_kernel(float* __restri
             c = cosf(th);
             s = sinf(th);
         }
-        const float r0 = fmaf(x0, c, -(x1 * s));
-        const float r1 = fmaf(x0, s, x1 * c);
-        vec[i0] = r0;
-        vec[i1] = r1;
+        const float r0 = fmaf(x0[j], c, -(x1[j] * s));
+        const float r1 = fmaf(x0[j], s, x1[j] * c);
+        vec[i0[j]] = r0;
+        vec[i1[j]] = r1;
         if (is_k) {
             const int64_t row = pos * (int64_t)(n_kv_heads * head_dim) + (int64_t)h * head_dim;
-            const float v0 = V[h * head_dim + i0], v1 = V[h * head_dim + i1];
+            const float v0 = V[h * head_dim + i0[j]], v1 = V[h * head_dim + i1[j]];
             if constexpr (KV16) {
                 __half* kc = static_cast<__half*>(Kc) + row;
                 __half* vc = static_cast<__half*>(Vc) + row;
-                kc[i0] = __float2half_rn(r0);
-                kc[i1] = __float2half_rn(r1);
-                vc[i0] = __float2half_rn(v0);
-                vc[i1] = __float2half_rn(v1);
+                kc[i0[j]] = __float2half_rn(r0);
+                kc[i1[j]] = __float2half_rn(r1);
+                vc[i0[j]] = __float2half_rn(v0);
+                vc[i1[j]] = __float2half_rn(v1);
             } else {
                 float* kc = static_cast<float*>(Kc) + row;
                 float* vc = static_cast<float*>(Vc) + row;
-                kc[i0] = r0;
-                kc[i1] = r1;
-                vc[i0] = v0;
-                vc[i1] = v1;
+                kc[i0[j]] = r0;
+                kc[i1[j]] = r1;
+                vc[i0[j]] = v0;
+                vc[i1[j]] = v1;
             }
         }
     }
@@ -459,7 +475,7 @@ int ptm_qknorm_rope_kvwrite(float* Q, float* K, const float* V, const float* q_n
     if (!Q || !K || !V || !K_cache || !V_cache || !d_past_len) return PTM_E_NULL;
     if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
     if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || head_dim <= 0 || (head_dim & 1)) return PTM_E_SHAPE;
-    if (head_dim > 128) return PTM_E_UNSUPPORTED;
+    if (head_dim > 256) return PTM_E_UNSUPPORTED;
     const dim3 grid(n_heads + n_kv_heads);
     if (kv_fp16)
         hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<true>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w,

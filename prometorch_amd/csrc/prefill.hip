@@ -66,44 +66,62 @@ __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restri
     float* vec = is_k ? K + (int64_t)m * kv_dim + (int64_t)h * head_dim
                       : Q + ((int64_t)m * n_heads + h) * head_dim;
     const float* nw = is_k ? kw : qw;
-    const int half = head_dim / 2, t = threadIdx.x;
-    const bool on = t < half;
-    const int i0 = rope_interleaved ? 2 * t : t, i1 = rope_interleaved ? 2 * t + 1 : t + half;  // rotation pair t
-    float x0 = on ? vec[i0] : 0.0f, x1 = on ? vec[i1] : 0.0f;
+    const int half = head_dim / 2;
+    const float* cs = rope + pos * head_dim;
+    // thread t owns rotation pairs t and t + 64 (the second only for heads wider than 128)
+    float x0[2], x1[2];
+    int i0[2], i1[2];
+    bool on[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int t = threadIdx.x + 64 * j;
+        on[j] = t < half;
+        i0[j] = rope_interleaved ? 2 * t : t;
+        i1[j] = rope_interleaved ? 2 * t + 1 : t + half;
+        x0[j] = on[j] ? vec[i0[j]] : 0.0f;
+        x1[j] = on[j] ? vec[i1[j]] : 0.0f;
+    }
     if (nw) {
-        float ss = fmaf(x0, x0, 0.0f);
-        ss = fmaf(x1, x1, ss);
+        float ss = fmaf(x0[0], x0[0], 0.0f);
+        ss = fmaf(x1[0], x1[0], ss);
+        ss = fmaf(x0[1], x0[1], ss);
+        ss = fmaf(x1[1], x1[1], ss);
         ss = sum64(ss);
         const float rs = 1.0f / sqrtf(ss / (float)head_dim + eps);
         const float one = add_one ? 1.0f : 0.0f;
-        if (on) {
-            x0 = x0 * rs * (nw[i0] + one);
-            x1 = x1 * rs * (nw[i1] + one);
-        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            if (on[j]) {
+                x0[j] = x0[j] * rs * (nw[i0[j]] + one);
+                x1[j] = x1[j] * rs * (nw[i1[j]] + one);
+            }
     }
-    if (!on) return;
-    const float* cs = rope + pos * head_dim;
-    const float c = cs[t], s = cs[half + t];
-    const float r0 = fmaf(x0, c, -(x1 * s)), r1 = fmaf(x0, s, x1 * c);  // hot_loops.cpp:2035-2061
-    vec[i0] = r0;
-    vec[i1] = r1;
-    if (is_k) {
-        const int64_t off = pos * kv_dim + (int64_t)h * head_dim;
-        const float v0 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t], v1 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t + half];
-        if constexpr (KV16) {
-            __half* kc = static_cast<__half*>(Kc) + off;
-            __half* vc = static_cast<__half*>(Vc) + off;
-            kc[i0] = __float2half_rn(r0);
-            kc[i1] = __float2half_rn(r1);
-            vc[t] = __float2half_rn(v0);
-            vc[t + half] = __float2half_rn(v1);
-        } else {
-            float* kc = static_cast<float*>(Kc) + off;
-            float* vc = static_cast<float*>(Vc) + off;
-            kc[i0] = r0;
-            kc[i1] = r1;
-            vc[t] = v0;
-            vc[t + half] = v1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        if (!on[j]) continue;
+        const int t = threadIdx.x + 64 * j;
+        const float c = cs[t], s = cs[half + t];
+        const float r0 = fmaf(x0[j], c, -(x1[j] * s)), r1 = fmaf(x0[j], s, x1[j] * c);  // hot_loops.cpp:2035-2061
+        vec[i0[j]] = r0;
+        vec[i1[j]] = r1;
+        if (is_k) {
+            const int64_t off = pos * kv_dim + (int64_t)h * head_dim;
+            const float v0 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t], v1 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t + half];
+            if constexpr (KV16) {
+                __half* kc = static_cast<__half*>(Kc) + off;
+                __half* vc = static_cast<__half*>(Vc) + off;
+                kc[i0[j]] = __float2half_rn(r0);
+                kc[i1[j]] = __float2half_rn(r1);
+                vc[t] = __float2half_rn(v0);
+                vc[t + half] = __float2half_rn(v1);
+            } else {
+                float* kc = static_cast<float*>(Kc) + off;
+                float* vc = static_cast<float*>(Vc) + off;
+                kc[i0[j]] = r0;
+                kc[i1[j]] = r1;
+                vc[t] = v0;
+                vc[t + half] = v1;
+            }
         }
     }
 }
@@ -184,7 +202,7 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restri
             float d = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) d = fmaf(q[g][i], k[i], d);
-            d = (LPP == 16) ? sum16(d) : sum8(d);
+            d = sum_lanes<LPP>(d);
             const float s = valid ? d * scale : -INFINITY;
             const float mnew = fmaxf(mrun[g], s);
             const float muse = mnew == -INFINITY ? 0.0f : mnew;
@@ -428,7 +446,7 @@ int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float
                                  int kv_fp16, int rope_interleaved, ptm_stream_t stream) {
     if (!Q || !K || !V || !K_cache || !V_cache || !rope_table) return PTM_E_NULL;
     if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
-    if (rows <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || head_dim <= 0 || (head_dim & 1) || head_dim > 128)
+    if (rows <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || head_dim <= 0 || (head_dim & 1) || head_dim > 256)
         return PTM_E_SHAPE;
     if (pos0 < 0 || pos0 + rows > max_seq) return PTM_E_RANGE;  // never write outside the cache
     if (n_heads + n_kv_heads > 65535) return PTM_E_UNSUPPORTED;
@@ -454,7 +472,7 @@ int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void
                                  int window, ptm_stream_t stream) {
     if (!Q || !K_cache || !V_cache || !O) return PTM_E_NULL;
     if (rows <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
-    if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return PTM_E_UNSUPPORTED;
     if (pos0 < 0 || pos0 + rows > max_seq) return PTM_E_RANGE;
     if (!aligned16(Q) || !aligned16(K_cache) || !aligned16(V_cache) || !aligned16(O)) return PTM_E_ALIGN;
     if (n_kv_heads > 65535) return PTM_E_UNSUPPORTED;
@@ -463,6 +481,10 @@ int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void
     hipStream_t s = as_stream(stream);
     if (window < 0) window = 0;
     // the matrix-core kernel walks every tile from position 0; windowed layers take the fp32 kernel, which starts at the window
+    if (head_dim == 256) {  // wide heads (gemma3): the fp32 kernel only
+        return kv_fp16 ? prefill_attn_launch<true, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
+                       : prefill_attn_launch<false, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
+    }
     if (window == 0 && kv_fp16 && rows >= PTM_PREFILL_MFMA_MIN_ROWS && (G == 1 || G == 2 || G == 4 || G == 8))
         return head_dim == 128 ? prefill_attn_mfma_launch<128>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
                                : prefill_attn_mfma_launch<64>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);

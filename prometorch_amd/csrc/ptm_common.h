@@ -66,6 +66,20 @@ __device__ __forceinline__ float sum16(float v) {
     v += dpp_f<0x140>(v);
     return v;
 }
+// all-reduce over each half of the wave (lanes 0..31, 32..63)
+__device__ __forceinline__ float sum32(float v) {
+    v = sum16(v);
+    v += __shfl_xor(v, 16, 64);
+    return v;
+}
+// sum over groups of LPP = 8, 16 or 32 consecutive lanes
+template <int LPP>
+__device__ __forceinline__ float sum_lanes(float v) {
+    static_assert(LPP == 8 || LPP == 16 || LPP == 32, "lane group of 8, 16 or 32");
+    if constexpr (LPP == 8) return sum8(v);
+    else if constexpr (LPP == 16) return sum16(v);
+    else return sum32(v);
+}
 // all-reduce over the whole wave64
 __device__ __forceinline__ float sum64(float v) {
     v = sum16(v);

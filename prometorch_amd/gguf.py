@@ -79,6 +79,11 @@ def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "q
         f"{arch}.attention.layer_norm_rms_epsilon": float(cfg["eps"]), f"{arch}.context_length": 4096,
         "tokenizer.ggml.model": "gpt2", "tokenizer.ggml.tokens": ["a", "b", "c"], "tokenizer.ggml.token_type": [1, 1, 1],
     }
+    if cfg.get("swa_window", 0) > 0:  # gemma3's alternating local / global layers
+        md[f"{arch}.attention.sliding_window"] = int(cfg["swa_window"])
+        if cfg.get("swa_pattern", 6) != 6:
+            md[f"{arch}.attention.sliding_window_pattern"] = int(cfg["swa_pattern"])
+        md[f"{arch}.rope.freq_base_swa"] = float(cfg.get("rope_swa_base", 10000.0))
     if cfg.get("rope_scale", 1.0) != 1.0:  # linear position scaling, the keys llama3 / qwen2 files use
         md[f"{arch}.rope.scaling.type"] = "linear"
         md[f"{arch}.rope.scaling.factor"] = float(cfg["rope_scale"])
@@ -104,6 +109,9 @@ def model_to_gguf(path: str, cfg: dict, layers: list, head: dict, arch: str = "q
         if L.get("q_norm") is not None:  # absent in a llama-style model
             ts.append((p + "attn_q_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["q_norm"], np.float32)))
             ts.append((p + "attn_k_norm.weight", F32, [cfg["head_dim"]], np.asarray(L["k_norm"], np.float32)))
+        for key, gname in (("post_attn_norm", "post_attention_norm"), ("post_ffn_norm", "post_ffw_norm")):
+            if L.get(key) is not None:  # gemma2 / gemma3
+                ts.append((p + gname + ".weight", F32, [H], np.asarray(L[key], np.float32)))
         for k in ("q", "k", "v"):
             if L.get(k + "_bias") is not None:  # qwen2-style projections
                 b = np.asarray(L[k + "_bias"], np.float32)
@@ -219,7 +227,9 @@ class GGUFModel:
         check(self.L.ptm_model_config(m, C.byref(c)), "model_config")
         self.cfg = {k: getattr(c, k) for k in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "max_seq")}
         self.cfg.update(rope_base=c.rope_freq_base, eps=c.rms_eps, kv_fp16=bool(c.kv_fp16), tied=not bool(c.embedding_f32),
-                        rope_interleaved=bool(c.rope_interleaved), rope_scale=c.rope_scale)
+                        rope_interleaved=bool(c.rope_interleaved), rope_scale=c.rope_scale,
+                        scale_embeddings=bool(c.scale_embeddings), ffn_gelu=bool(c.ffn_gelu), swa_window=c.swa_window,
+                        swa_pattern=c.swa_pattern, rope_swa_base=c.rope_swa_freq_base)
 
     def layer(self, i: int) -> Layer:
         out = Layer()

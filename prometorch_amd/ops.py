@@ -239,6 +239,14 @@ def attn_decode_fused(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, O, partial_
           "attn_decode_fused")
 
 
+def flash_decode_window(Q, K_cache, V_cache, O, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, head_dim, d_past_len,
+                        max_seq, scale, kv_fp16=True, window=0, o_q8=None, stream=None):
+    """launch_flash_decode(_fp16)_graph over the last `window` positions (0: all); head_dim 64, 128 or 256."""
+    check(_L().ptm_flash_decode_window(_ptr(Q), _ptr(K_cache), _ptr(V_cache), _ptr(O), _ptr(o_q8), _ptr(partial_O),
+                                      _ptr(partial_lse), _ptr(partial_max), n_heads, n_kv_heads, head_dim, _ptr(d_past_len),
+                                      max_seq, scale, int(kv_fp16), int(window), _stream(stream)), "flash_decode_window")
+
+
 def gelu_mul(gate, up, out, n, stream=None):
     """tanh-GELU(gate) * up (gguf_model.h:3730-3738)."""
     check(_L().ptm_gelu_mul(_ptr(gate), _ptr(up), _ptr(out), n, _stream(stream)), "gelu_mul")

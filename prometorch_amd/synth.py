@@ -286,14 +286,17 @@ def tiny_qwen2(seed: int):
     return cfg, layers, make_head(seed, cfg)
 
 
-def tiny_gemma(seed: int, n_layers: int = 4):
+def tiny_gemma(seed: int, n_layers: int = 4, head_dim: int = 64):
     """The TINY shapes as a gemma3-style model: embedding rows times sqrt(hidden), per-head QK-norm, NeoX rotation,
     tanh-GELU gate, RMSNorm on each branch's output before the residual add, and alternating attention: layers li with
     (li + 1) % 3 != 0 see only the last 8 positions and rotate with base 1e4, the others see everything and rotate with
-    base 1e6 and positions divided by 8.  Four layers: local, local, global, local.  The embedding scale of 16 is undone in
+    base 1e6 and positions divided by 8.  Four layers: local, local, global, local.  head_dim = 256 gives gemma3's head
+    width.  The embedding scale of 16 is undone in
     the first norm gains' scale so that activations stay where the other tiny models have them."""
     cfg = dict(TINY, n_layers=n_layers, scale_embeddings=True, ffn_gelu=True, swa_window=8, swa_pattern=3, rope_swa_base=1.0e4,
                rope_scale=8.0)
+    if head_dim != cfg["head_dim"]:  # gemma3's heads are 256 wide: two query heads on one kv head, q_dim 512
+        cfg.update(head_dim=head_dim, n_heads=2, n_kv_heads=1)
     layers = [make_layer(seed, i, cfg) for i in range(n_layers)]
     for i, L in enumerate(layers):
         g = rng_for(seed, 6, i)

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from conftest import bits
-from prometorch_amd import ops, synth
+from prometorch_amd import gguf, ops, synth
 from test_gpu_decode import check_step_errors
 from test_gpu_llama import follow_sensitive
 from test_gpu_prefill import check_kv_rows, check_logits
@@ -218,3 +218,115 @@ def test_gemma_prefill_vs_oracle_token_by_token(dev, po, seeds, kv_fp16, pos0, n
     check_logits(dec.logits(), om.logits, tok_g, tok_o, "prefill")
     follow_sensitive(dec, om, tok_o, 6)
     dec.close()
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+@pytest.mark.parametrize("nh,nkv,hd,past,window", [(8, 4, 256, 2048, 1024), (8, 4, 256, 2048, 0), (2, 1, 256, 19, 8), (4, 4, 128, 300, 100)])
+def test_flash_decode_window_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past, window):
+    """The plain split-KV attention (the path of 256-wide heads) over a window, with the Q8 copy of its output."""
+    T = past + 1
+    max_seq = ((T + 127) // 64) * 64
+    r = synth.rng_for(50, nh, hd, past)
+    kvd = nkv * hd
+    kf = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    vf = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    q = synth.make_x(r, nh * hd)
+    scale = 1.0 / np.sqrt(hd)
+    t_start = max(0, T - window) if window else 0
+    want = np.concatenate([po.attn_head(q[h * hd:(h + 1) * hd], kf, vf, T, kvd, hd, scale, col0=(h // (nh // nkv)) * hd,
+                                        t_start=t_start) for h in range(nh)])
+    dt = torch.float16 if kv_fp16 else torch.float32
+    Kc, Vc = cu(kf).to(dt), cu(vf).to(dt)
+    Kc[T:] = float("nan")
+    Vc[T:] = float("nan")
+    S = ops.flash_decode_num_splits(max_seq)
+    pO = torch.full((S * nh * hd,), float("nan"), device="cuda")
+    pL = torch.full((S * nh,), float("nan"), device="cuda")
+    pM = torch.full((S * nh,), float("nan"), device="cuda")
+    O = torch.empty(nh * hd, device="cuda")
+    q8 = torch.zeros(ops.q8_bytes(nh * hd), dtype=torch.uint8, device="cuda")
+    d_past = torch.tensor([past], dtype=torch.int64, device="cuda")
+    ops.flash_decode_window(cu(q), Kc, Vc, O, pO, pL, pM, nh, nkv, hd, d_past, max_seq, scale, kv_fp16=kv_fp16, window=window, o_q8=q8)
+    torch.cuda.synchronize()
+    got = O.cpu().numpy()
+    assert np.all(np.isfinite(got))
+    assert np.abs(got - want).max() <= 3e-5 * max(np.abs(want).max(), 1e-3) + 1e-6
+    K = nh * hd
+    raw = q8.cpu().numpy()
+    qs = raw[:K].view(np.int8).astype(np.float32)
+    d = raw[K:K + 4 * (K // 32)].view(np.float32)
+    assert np.abs(qs * np.repeat(d, 32) - got).max() <= 0.51 * d.max()   # the Q8 blocks are this vector, rounded
+
+
+@pytest.mark.parametrize("kv_fp16", [True, False])
+def test_gemma_wide_heads_decode_and_prefill_vs_oracle(dev, po, seeds, kv_fp16):
+    """head_dim 256 (gemma3's width): decode from a cache, chained greedy, and a prompt through the row-batched path."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head = synth.tiny_gemma(seeds["tiny"], head_dim=256)
+    kv = [synth.make_kv_prefill(seeds["tiny"], i, cfg, 19) for i in range(cfg["n_layers"])]
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=kv_fp16)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=kv_fp16, use_graph=True)
+    dec2 = Decoder(cfg, layers, head, max_seq=64, kv_fp16=kv_fp16, use_graph=True)
+    for i, (k, v) in enumerate(kv):
+        om.set_kv(i, k, v)
+        dec.set_kv(i, k, v)
+        dec2.set_kv(i, k, v)
+    dec.set_past_len(19)
+    dec2.set_past_len(19)
+    tok_o = tok_g = 3
+    want, errs = [], []
+    for st in range(16):
+        tok_o = om.step(tok_o)
+        tok_g = dec.step(tok_g)
+        want.append(tok_o)
+        errs.append(np.abs(dec.logits() - om.logits).max() / om.logits.std())
+        assert tok_g == tok_o, st
+    check_step_errors(errs)
+    assert dec2.greedy(3, 16) == want
+    dec.close()
+    dec2.close()
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=kv_fp16)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=kv_fp16, use_graph=True)
+    prompt = [int(t) for t in synth.rng_for(70).integers(0, cfg["vocab"], 23)]
+    for t in prompt:
+        tok_o = om.step(t)
+    tok_g = dec.prefill(prompt, chunk_rows=7)
+    for li in range(cfg["n_layers"]):
+        for nm, gpu_c, cpu_c in (("k", dec.k_cache[li], om.k_cache[li]), ("v", dec.v_cache[li], om.v_cache[li])):
+            check_kv_rows(gpu_c[:23].float().cpu().numpy(), cpu_c[:23], li, nm)
+    check_logits(dec.logits(), om.logits, tok_g, tok_o, "prefill")
+    follow_sensitive(dec, om, tok_o, 6)
+    dec.close()
+
+
+def test_gemma3_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_gemma, tmp_path):
+    """general.architecture = gemma3: sliding_window / sliding_window_pattern / rope.freq_base_swa / rope.scaling.* keys and
+    the post_attention_norm / post_ffw_norm vectors are read; scaled embeddings and the GELU gate follow from the name."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_gemma_with_cache(seeds)
+    path = str(tmp_path / "tiny_gemma3.gguf")
+    gguf.model_to_gguf(path, cfg, layers, head, arch="gemma3")
+    m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
+    for key in ("scale_embeddings", "ffn_gelu", "swa_window", "swa_pattern", "rope_swa_base", "rope_scale"):
+        assert m.cfg[key] == cfg[key], key
+    assert m.layer(2).post_attn_norm and m.layer(2).post_ffn_norm and m.layer(2).q_norm
+    d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
+    for i, (k, v) in enumerate(kv):
+        m.set_kv(i, k, v)
+        d.set_kv(i, k, v)
+    m.set_past_len(19)
+    d.set_past_len(19)
+    tm = td = 3
+    for st in range(16):
+        tm = m.step(tm)
+        td = d.step(td)
+        assert tm == td == int(golden_gemma["tokens"][st]), st
+        assert np.array_equal(bits(m.logits()), bits(d.logits())), st
+    m.close()
+    d.close()
+    # without the pattern key every sixth layer is global: the four-layer model is all local then
+    p2 = str(tmp_path / "default_pattern.gguf")
+    gguf.model_to_gguf(p2, dict(cfg, swa_pattern=6), layers, head, arch="gemma3")
+    m2 = gguf.GGUFModel(p2, max_seq=64, kv_fp16=False)
+    assert m2.cfg["swa_pattern"] == 6
+    m2.close()

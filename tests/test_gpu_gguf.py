@@ -51,8 +51,8 @@ def test_gguf_model_decodes_like_direct_decoder(dev, seeds, golden, tmp_path, ti
 
 def test_gguf_model_refuses_what_it_cannot_run(dev, seeds, tmp_path):
     cfg, layers, head, _ = build_tiny(seeds)
-    p = str(tmp_path / "gemma3.gguf")
-    gguf.model_to_gguf(p, cfg, layers, head, arch="gemma3")  # post-norms, GeGLU, sliding windows: not a step built here
+    p = str(tmp_path / "phi3.gguf")
+    gguf.model_to_gguf(p, cfg, layers, head, arch="phi3")  # fused qkv / gate-up tensors, per-frequency factors: not a step built here
     with pytest.raises(PtmError) as e:
         gguf.GGUFModel(p, max_seq=64)
     assert e.value.code == -4

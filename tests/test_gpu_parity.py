@@ -395,7 +395,7 @@ def test_rope_interleaved_pairs(dev):
 
 @pytest.mark.parametrize("kv_fp16", [True, False])
 @pytest.mark.parametrize("nh,nkv,hd,T", [(32, 8, 128, 2049), (32, 8, 128, 2176), (4, 2, 64, 20), (8, 8, 128, 1),
-                                         (16, 2, 64, 64), (8, 8, 64, 65)])
+                                         (16, 2, 64, 64), (8, 8, 64, 65), (8, 4, 256, 2049), (2, 1, 256, 70), (4, 4, 256, 1)])
 def test_flash_decode_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, T):
     max_seq = max(64, ((T + 127) // 64) * 64)
     r = synth.rng_for(44, nh, hd, T)
