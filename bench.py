@@ -77,6 +77,8 @@ def main():
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--gemma-steps", type=int, default=64,
+                    help="decode steps of the Gemma-3-4B-shaped extra (0: skip it)")
     ap.add_argument("--llama-steps", type=int, default=64,
                     help="decode steps of the Llama-3-8B-shaped extra measurement (0 = skip)")
     ap.add_argument("--layers", type=int, default=36, help=argparse.SUPPRESS)  # debugging only; 36 is the workload
@@ -318,6 +320,38 @@ def main():
         del ldec, llayers, lhead
         torch.cuda.empty_cache()
 
+    # ---- a third family: Gemma-3-4B-shaped Q4_K_M (256-wide heads, post-norms, GELU gate, sliding-window layers) ----
+    gemma = None
+    if args.gemma_steps > 0:
+        t0 = time.perf_counter()
+        gcfg = dict(synth.GEMMA3_4B)
+        _, glayers, ghead = synth.gemma3_4b_like(SEED + 2, n_layers=gcfg["n_layers"], vocab=gcfg["vocab"])
+        gdec = Decoder(gcfg, glayers, ghead, max_seq=MAX_SEQ, kv_fp16=True, use_graph=True)
+        for i in range(gcfg["n_layers"]):
+            gdec.set_kv(i, *synth.make_kv_prefill(SEED + 2, i, gcfg, N_PREFILL))
+        gdec.set_past_len(N_PREFILL)
+        gtok = 1
+        for _ in range(args.warmup):
+            gtok = gdec.step(gtok)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.gemma_steps):
+            gtok = gdec.step(gtok)
+        torch.cuda.synchronize()
+        gdt = time.perf_counter() - t1
+        g_T = N_PREFILL + args.warmup + args.gemma_steps / 2
+        g_bytes = 34 * 60_518_400 + 262144 * 2100 + 2 * (29 * 1024 + 5 * g_T) * 1024 * 2
+        gemma = {"workload": "batch-1 greedy decode, Gemma-3-4B-shaped Q4_K_M (34 layers, 2560 hidden, 8 x 256 heads on 4 kv heads, "
+                             "10240 intermediate, 262144 vocabulary, window 1024 on 29 layers), fp16 KV prefilled %d, %d new tokens, "
+                             "host-synchronous" % (N_PREFILL, args.gemma_steps),
+                 "tok_s": args.gemma_steps / gdt, "ms_per_token": gdt / args.gemma_steps * 1e3,
+                 "token_hbm_frac": g_bytes / (gdt / args.gemma_steps) / 1e9 / HBM_PEAK_GBS,
+                 "a100_published_gemma3_4b_tok_s": 81.4}
+        log("gemma-3-4B shape: %.1f tok/s (%.3f ms/token), set up in %.1fs" % (gemma["tok_s"], gemma["ms_per_token"], t1 - t0))
+        gdec.close()
+        del gdec, glayers, ghead
+        torch.cuda.empty_cache()
+
     # ---- CPU baseline on this host: bounded sample of the same workload ---------------------------
     cpu = None
     if args.cpu_tokens > 0:
@@ -336,6 +370,7 @@ def main():
         "chained_tok_s": chained_tok_s, "chained_tokens_identical": bool(tokens_equal),
         "sampled_tok_s": sampled_tok_s, "sampled_chained_tok_s": sampled_chained_tok_s,
         "llama3_8b_shape": llama,
+        "gemma3_4b_shape": gemma,
         "a100_published_tok_s": 82.6, "x_a100_published": tok_s / 82.6,
         "token_hbm_frac": per_token_bytes / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
     }

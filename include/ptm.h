@@ -441,7 +441,8 @@ int ptm_gguf_array_string(const ptm_gguf* g, const char* key, int64_t i, const c
 const void* ptm_gguf_array_data(const ptm_gguf* g, const char* key);
 
 /* From a .gguf file to a ready decoder: reads the `qwen3`, `qwen2` (no QK-norm tensors; blk.N.attn_{q,k,v}.bias
- * vectors where the file has them, gguf_model.h:6750-6754) or `llama` (no QK-norm tensors, interleaved rotation
+ * vectors where the file has them, gguf_model.h:6750-6754), `gemma3` (sliding-window keys, post-norm vectors, scaled
+ * embeddings and GELU gate: gguf_model.h:157-197) or `llama` (no QK-norm tensors, interleaved rotation
  * pairs: gguf_model.h:202-217) hyper-parameters
  * (<arch>.block_count, embedding_length, feed_forward_length, attention.head_count(_kv),
  * attention.key_length, rope.freq_base, attention.layer_norm_rms_epsilon; gguf_model.h:126-181),

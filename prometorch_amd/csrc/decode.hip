@@ -35,7 +35,7 @@ namespace ptm {
 int q4k_gemv_multi(int n_mat, const void* const* W, float* const* y, const int* N, const void* x, bool x_is_q8,
                    const float* gamma, float eps, int add_one, int K, int64_t stride, bool accumulate, hipStream_t s);
 int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8, const float* gamma, float eps,
-                     int add_one, float* act, int K, int N, int64_t stride, hipStream_t s);
+                     int add_one, float* act, int K, int N, int64_t stride, hipStream_t s, bool gelu);
 int q6k_gemv_impl(const void* W, const float* x, float* y, int K, int N, int64_t stride, bool accumulate,
                   const float* gamma, float eps, int add_one, hipStream_t s);
 void q6k_init_attributes();
@@ -224,10 +224,10 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
             PTM_TRY(gemv_any(L.o, d->attn, o_dst, o_acc, s));
         }
         if (L.post_attn_norm) PTM_TRY(ptm_rms_norm_add(d->hb, L.post_attn_norm, d->x, 1, H, c.rms_eps, 0, s));
-        if (!c.ffn_gelu && L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
+        if (L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
             L.gate.row_stride_bytes == L.up.row_stride_bytes && L.gate.rows == L.up.rows) {
             PTM_TRY(q4k_gate_up_silu(L.gate.data, L.up.data, d->x, false, L.ffn_norm, c.rms_eps, 0, d->act, H,
-                                     L.gate.rows, L.gate.row_stride_bytes, s));
+                                     L.gate.rows, L.gate.row_stride_bytes, s, c.ffn_gelu != 0));
         } else {
             PTM_TRY(ptm_rms_norm(d->x, L.ffn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
             PTM_TRY(gemv_any(L.gate, d->xn, d->gate, false, s));

@@ -21,6 +21,7 @@ struct Q4KArgs {
     const float* gamma;  // RMSNorm weight (NORM)
     float eps;
     int add_one;
+    int gelu;            // MODE 1: tanh-GELU(gate) * up (gemma) instead of SiLU(gate) * up
 };
 
 enum { Q4K_THREADS = 256, Q4K_U = 10 };
@@ -192,6 +193,13 @@ __device__ __forceinline__ float q4k_block_term(const uint4 hdr, const uint4 qv,
     return fmaf(w, (float)isum, -c);
 }
 
+__device__ __forceinline__ float gelu_mul_ref(float g, float u) {
+    // reference: gguf_model.h:3730-3738
+    const float x3 = g * g * g;
+    const float t = tanhf(0.7978845608028654f * (g + 0.044715f * x3));
+    return 0.5f * g * (1.0f + t) * u;
+}
+
 __device__ __forceinline__ float silu_mul_ref(float g, float u) {
     // reference: gguf_model.h:3741-3755 (clamp, libm exp, 1/(1+e), g*sig, *u)
     float ng = 0.0f - g;
@@ -277,7 +285,7 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
             if (S == 1) other = dpp_f<0x128>(p);
             else if (S == 2) other = __shfl_xor(p, 16, 64);
             else other = __shfl_xor(p, 32, 64);
-            if (live && mat == 0 && sub == 0 && j == 0) a.y[0][local] = silu_mul_ref(p, other);
+            if (live && mat == 0 && sub == 0 && j == 0) a.y[0][local] = a.gelu ? gelu_mul_ref(p, other) : silu_mul_ref(p, other);
         } else {
             float* y = mat == 0 ? a.y[0] : (mat == 1 ? a.y[1] : a.y[2]);
             if (live && sub == 0 && j == 0) {

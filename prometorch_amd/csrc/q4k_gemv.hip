@@ -87,7 +87,7 @@ int q4k_gemv_multi(int n_mat, const void* const* W, float* const* y, const int* 
 }
 
 int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8, const float* gamma, float eps,
-                     int add_one, float* act, int K, int N, int64_t stride, hipStream_t s) {
+                     int add_one, float* act, int K, int N, int64_t stride, hipStream_t s, bool gelu) {
     int rc = q4k_check(wg, x, act, K, N, stride);
     if (rc != PTM_OK) return rc;
     rc = q4k_check(wu, x, act, K, N, stride);
@@ -106,6 +106,7 @@ int q4k_gate_up_silu(const void* wg, const void* wu, const void* x, bool x_is_q8
     a.gamma = gamma;
     a.eps = eps;
     a.add_one = add_one;
+    a.gelu = gelu ? 1 : 0;
     if (gamma) {
         if (x_is_q8) return PTM_E_UNSUPPORTED;
         if (!aligned16(gamma)) return PTM_E_ALIGN;
@@ -178,7 +179,7 @@ int ptm_q4k_fused_rmsnorm_gate_up_silu(const float* x, const float* norm_w, cons
                                        const void* w_up, float* act, int K, int N, int64_t stride, float eps,
                                        int add_one, ptm_stream_t stream) {
     if (!norm_w) return PTM_E_NULL;
-    return q4k_gate_up_silu(w_gate, w_up, x, false, norm_w, eps, add_one, act, K, N, stride, as_stream(stream));
+    return q4k_gate_up_silu(w_gate, w_up, x, false, norm_w, eps, add_one, act, K, N, stride, as_stream(stream), false);
 }
 
 }  // extern "C"

@@ -255,6 +255,24 @@ def llama3_8b_like(seed: int, n_layers: int = 2, vocab: int = 32000):
     return cfg, layers, make_head(seed, cfg)
 
 
+GEMMA3_4B = dict(vocab=262144, hidden=2560, n_layers=34, n_heads=8, n_kv_heads=4, head_dim=256, inter=10240,
+                 rope_base=1.0e6, eps=1.0e-6, scale_embeddings=True, ffn_gelu=True, swa_window=1024, swa_pattern=6,
+                 rope_swa_base=1.0e4, rope_scale=8.0)
+
+
+def gemma3_4b_like(seed: int, n_layers: int = 2, vocab: int = 32000):
+    """Gemma-3-4B layer shapes (256-wide heads, post-norms, GELU gate, five local layers of window 1024 per global one),
+    optionally with fewer layers and a reduced vocabulary so that the CPU oracle can step it."""
+    cfg = dict(GEMMA3_4B)
+    cfg["n_layers"], cfg["vocab"] = n_layers, vocab
+    layers = [make_layer(seed, i, cfg) for i in range(n_layers)]
+    for i, L in enumerate(layers):
+        g = rng_for(seed, 6, i)
+        for name in ("post_attn_norm", "post_ffn_norm"):
+            L[name] = (np.float32(0.5) * (np.float32(1.0) + np.float32(0.1) * g.standard_normal(cfg["hidden"], dtype=np.float32))).astype(np.float32)
+    return cfg, layers, make_head(seed, cfg)
+
+
 def tiny_llama(seed: int):
     """The TINY shapes as a llama-style model: no per-head QK-norm, interleaved rotation pairs.  The attention-input
     norm weights are a tenth of TINY's: with random weights and no QK-norm the Q.K scores would otherwise run to the

@@ -330,3 +330,42 @@ def test_gemma3_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_gemma, 
     m2 = gguf.GGUFModel(p2, max_seq=64, kv_fp16=False)
     assert m2.cfg["swa_pattern"] == 6
     m2.close()
+
+
+def test_gemma3_4b_layer_shapes_decode_and_prefill_vs_oracle(dev, po, seeds):
+    """Two layers of Gemma-3-4B size (2560 hidden, 8 heads of 256 on 4 kv heads, 10240 intermediate, window 1024, bases
+    1e4 / 1e6 with positions divided by 8) over a 32000-token vocabulary, the second layer global: 8 decode steps behind
+    1100 cached positions (past the window) and a 40-token prompt, against the oracle."""
+    from prometorch_amd.decode import Decoder
+    from test_gpu_decode import LOGIT_TOL, LOGIT_TOL_FLIP
+    from test_gpu_prefill import logit_errors
+    cfg, layers, head = synth.gemma3_4b_like(seeds["cfg4"])
+    cfg["swa_pattern"] = 2
+    om = po.OracleModel(cfg, layers, head, 1280, kv_fp16=True)
+    dec = Decoder(cfg, layers, head, max_seq=1280, kv_fp16=True, use_graph=True)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(seeds["cfg4"], i, cfg, 1100)
+        om.set_kv(i, k, v)
+        dec.set_kv(i, k, v)
+    dec.set_past_len(1100)
+    tok, errs = 11, []
+    for st in range(8):
+        tok_o = om.step(tok)
+        tok_g = dec.step(tok)
+        err, rms, margin = logit_errors(dec.logits(), om.logits)
+        errs.append(err)
+        if margin > 2 * err:
+            assert tok_g == tok_o, (st, margin, err)
+        tok = tok_o
+    errs = np.asarray(errs)
+    print("decode steps: logit err/std", np.array2string(errs, precision=2), flush=True)
+    assert errs.max() <= LOGIT_TOL_FLIP and np.median(errs) <= LOGIT_TOL, errs
+    prompt = [int(t) for t in synth.rng_for(72).integers(0, cfg["vocab"], 40)]
+    for t in prompt:
+        tok_o = om.step(t)
+    tok_g = dec.prefill(prompt)
+    for li in range(2):
+        check_kv_rows(dec.k_cache[li][1108:1148].float().cpu().numpy(), om.k_cache[li][1108:1148], li, "k")
+        check_kv_rows(dec.v_cache[li][1108:1148].float().cpu().numpy(), om.v_cache[li][1108:1148], li, "v")
+    check_logits(dec.logits(), om.logits, tok_g, tok_o, "prefill")
+    dec.close()
