@@ -130,11 +130,49 @@ __global__ __launch_bounds__(256) void rms_norm_add_kernel(const float* __restri
     __shared__ float red[4];
     const float* hr = h + (int64_t)blockIdx.x * hidden;
     float* xr = x + (int64_t)blockIdx.x * hidden;
+    const float one = add_one ? 1.0f : 0.0f;
+    if ((hidden & 3) == 0 && hidden <= 4 * 256 * 4) {
+        // rows of up to 4096 values: every load goes out before the reduction, one memory round trip
+        const int nv = hidden >> 2;
+        float4 hv[4], xv[4], wv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            const int ic = i < nv ? i : 0;
+            hv[j] = reinterpret_cast<const float4*>(hr)[ic];
+            xv[j] = reinterpret_cast<const float4*>(xr)[ic];
+            wv[j] = reinterpret_cast<const float4*>(w)[ic];
+        }
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (threadIdx.x + 256 * j < nv) {
+                ss = fmaf(hv[j].x, hv[j].x, ss);
+                ss = fmaf(hv[j].y, hv[j].y, ss);
+                ss = fmaf(hv[j].z, hv[j].z, ss);
+                ss = fmaf(hv[j].w, hv[j].w, ss);
+            }
+        }
+        ss = block_sum256(ss, red);
+        const float rs = 1.0f / sqrtf(ss / (float)hidden + eps);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < nv) {
+                float4 r;
+                r.x = xv[j].x + hv[j].x * rs * (wv[j].x + one);
+                r.y = xv[j].y + hv[j].y * rs * (wv[j].y + one);
+                r.z = xv[j].z + hv[j].z * rs * (wv[j].z + one);
+                r.w = xv[j].w + hv[j].w * rs * (wv[j].w + one);
+                reinterpret_cast<float4*>(xr)[i] = r;
+            }
+        }
+        return;
+    }
     float ss = 0.0f;
     for (int i = threadIdx.x; i < hidden; i += 256) ss = fmaf(hr[i], hr[i], ss);
     ss = block_sum256(ss, red);
     const float rs = 1.0f / sqrtf(ss / (float)hidden + eps);
-    const float one = add_one ? 1.0f : 0.0f;
     for (int i = threadIdx.x; i < hidden; i += 256) xr[i] = xr[i] + hr[i] * rs * (w[i] + one);
 }
 
@@ -555,6 +593,7 @@ int ptm_rms_norm_add(const float* h, const float* weight, float* x, int rows, in
                      ptm_stream_t stream) {
     if (!h || !weight || !x) return PTM_E_NULL;
     if (rows < 0 || hidden <= 0) return PTM_E_SHAPE;
+    if ((hidden & 3) == 0 && (!aligned16(h) || !aligned16(weight) || !aligned16(x))) return PTM_E_ALIGN;
     if (rows == 0) return PTM_OK;
     hipLaunchKernelGGL(rms_norm_add_kernel, dim3(rows), dim3(256), 0, as_stream(stream), h, weight, x, hidden, eps, add_one);
     return launch_status();
