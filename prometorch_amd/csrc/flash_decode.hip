@@ -576,7 +576,11 @@ static int attn_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
     switch (G) {
         case 1: PTM_AT(1); break;
         case 2: PTM_AT(2); break;
+        case 3: PTM_AT(3); break;
         case 4: PTM_AT(4); break;
+        case 5: PTM_AT(5); break;
+        case 6: PTM_AT(6); break;
+        case 7: PTM_AT(7); break;
         case 8: PTM_AT(8); break;
         default: return PTM_E_UNSUPPORTED;
     }
@@ -594,7 +598,11 @@ static int fd_launch_g(int G, dim3 grid, hipStream_t s, const float* Q, const vo
     switch (G) {
         case 1: PTM_FD(1); break;
         case 2: PTM_FD(2); break;
+        case 3: PTM_FD(3); break;
         case 4: PTM_FD(4); break;
+        case 5: PTM_FD(5); break;
+        case 6: PTM_FD(6); break;
+        case 7: PTM_FD(7); break;
         case 8: PTM_FD(8); break;
         default: return PTM_E_UNSUPPORTED;
     }

@@ -416,7 +416,11 @@ static int prefill_attn_launch(int G, dim3 grid, hipStream_t s, const float* Q, 
     switch (G) {
         case 1: PTM_PA(1); break;
         case 2: PTM_PA(2); break;
+        case 3: PTM_PA(3); break;
         case 4: PTM_PA(4); break;
+        case 5: PTM_PA(5); break;
+        case 6: PTM_PA(6); break;
+        case 7: PTM_PA(7); break;
         case 8: PTM_PA(8); break;
         default: return PTM_E_UNSUPPORTED;
     }

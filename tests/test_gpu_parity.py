@@ -395,7 +395,7 @@ def test_rope_interleaved_pairs(dev):
 
 @pytest.mark.parametrize("kv_fp16", [True, False])
 @pytest.mark.parametrize("nh,nkv,hd,T", [(32, 8, 128, 2049), (32, 8, 128, 2176), (4, 2, 64, 20), (8, 8, 128, 1),
-                                         (16, 2, 64, 64), (8, 8, 64, 65), (8, 4, 256, 2049), (2, 1, 256, 70), (4, 4, 256, 1)])
+                                         (16, 2, 64, 64), (8, 8, 64, 65), (8, 4, 256, 2049), (2, 1, 256, 70), (4, 4, 256, 1), (28, 4, 128, 2049), (6, 2, 64, 100), (5, 1, 128, 65), (6, 2, 256, 90)])
 def test_flash_decode_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, T):
     max_seq = max(64, ((T + 127) // 64) * 64)
     r = synth.rng_for(44, nh, hd, T)
@@ -469,6 +469,7 @@ def test_elementwise_embedding_argmax(dev, po):
 @pytest.mark.parametrize("nh,nkv,hd,past", [(32, 8, 128, 2048), (32, 8, 128, 2111), (32, 8, 128, 2112), (4, 2, 64, 19),
                                             (8, 8, 128, 0), (16, 2, 64, 63), (8, 1, 64, 64), (8, 8, 64, 130), (4, 2, 64, 29),
                                             (4, 2, 64, 31), (16, 2, 64, 61), (32, 8, 128, 14), (32, 8, 128, 62), (4, 4, 128, 5),
+                                            (28, 4, 128, 2100), (40, 8, 128, 300), (12, 2, 128, 70), (24, 8, 64, 19),  # 7, 5, 6, 3 query heads per kv head
                                             (32, 8, 128, 20000)])   # past the ~12 k positions where the reference's kernel stops
 def test_attn_decode_fused_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past):
     """QK-norm + RoPE + KV append + attention + merge in one launch, three tokens in a row, against the oracle's pieces in the reference's order."""
