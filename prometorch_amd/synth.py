@@ -255,6 +255,28 @@ def llama3_8b_like(seed: int, n_layers: int = 2, vocab: int = 32000):
     return cfg, layers, make_head(seed, cfg)
 
 
+QWEN25_7B = dict(vocab=152064, hidden=3584, n_layers=28, n_heads=28, n_kv_heads=4, head_dim=128, inter=18944,
+                 rope_base=1.0e6, eps=1.0e-6)
+
+
+def qwen25_7b_like(seed: int, n_layers: int = 2, vocab: int = 32000):
+    """Qwen2.5-7B layer shapes (7 query heads per kv head, q / k / v biases, no QK-norm; 14 and 74 super-blocks per row),
+    a few layers and a reduced vocabulary so that the CPU oracle can step it; attention-input norm gains reduced as in
+    tiny_llama."""
+    cfg = dict(QWEN25_7B)
+    cfg["n_layers"], cfg["vocab"] = n_layers, vocab
+    layers = [make_layer(seed, i, cfg) for i in range(n_layers)]
+    qd, kvd = cfg["n_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    for i, L in enumerate(layers):
+        L["q_norm"] = None
+        L["k_norm"] = None
+        L["attn_norm"] = (np.float32(0.1) * L["attn_norm"]).astype(np.float32)
+        g = rng_for(seed, 5, i)
+        for name, n in (("q_bias", qd), ("k_bias", kvd), ("v_bias", kvd)):
+            L[name] = (np.float32(0.5) * g.standard_normal(n, dtype=np.float32)).astype(np.float32)
+    return cfg, layers, make_head(seed, cfg)
+
+
 GEMMA3_4B = dict(vocab=262144, hidden=2560, n_layers=34, n_heads=8, n_kv_heads=4, head_dim=256, inter=10240,
                  rope_base=1.0e6, eps=1.0e-6, scale_embeddings=True, ffn_gelu=True, swa_window=1024, swa_pattern=6,
                  rope_swa_base=1.0e4, rope_scale=8.0)

@@ -179,3 +179,43 @@ def test_qwen2_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_qwen2, t
     with pytest.raises(PtmError) as e:
         gguf.GGUFModel(p2, max_seq=64)
     assert e.value.code == -10
+
+
+def test_qwen25_7b_layer_shapes_decode_and_prefill_vs_oracle(dev, po, seeds):
+    """Two layers of Qwen2.5-7B size (3584 hidden = 14 super-blocks, 18944 intermediate = 74, 28 query heads on 4 kv heads,
+    biases) over a 32000-token vocabulary: 8 decode steps behind 300 cached positions and a 40-token prompt against the
+    oracle.  Bars as for the Llama-3-8B-shaped test: the median step within LOGIT_TOL, every step within LOGIT_TOL_FLIP,
+    tokens equal wherever the oracle's margin exceeds twice the error."""
+    from prometorch_amd.decode import Decoder
+    from test_gpu_decode import LOGIT_TOL, LOGIT_TOL_FLIP
+    from test_gpu_prefill import logit_errors
+    cfg, layers, head = synth.qwen25_7b_like(seeds["cfg4"])
+    om = po.OracleModel(cfg, layers, head, 512, kv_fp16=True)
+    dec = Decoder(cfg, layers, head, max_seq=512, kv_fp16=True, use_graph=True)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(seeds["cfg4"], i, cfg, 300)
+        om.set_kv(i, k, v)
+        dec.set_kv(i, k, v)
+    dec.set_past_len(300)
+    tok, errs = 11, []
+    for st in range(8):
+        tok_o = om.step(tok)
+        tok_g = dec.step(tok)
+        err, rms, margin = logit_errors(dec.logits(), om.logits)
+        errs.append(err)
+        if margin > 2 * err:
+            assert tok_g == tok_o, (st, margin, err)
+        tok = tok_o
+    errs = np.asarray(errs)
+    print("decode steps: logit err/std", np.array2string(errs, precision=2), flush=True)
+    assert errs.max() <= LOGIT_TOL_FLIP and np.median(errs) <= LOGIT_TOL, errs
+    prompt = [int(t) for t in synth.rng_for(73).integers(0, cfg["vocab"], 40)]
+    for t in prompt:
+        tok_o = om.step(t)
+    tok_g = dec.prefill(prompt)
+    for li in range(2):
+        check_kv_rows(dec.k_cache[li][308:348].float().cpu().numpy(), om.k_cache[li][308:348], li, "k")
+        check_kv_rows(dec.v_cache[li][308:348].float().cpu().numpy(), om.v_cache[li][308:348], li, "v")
+    err, rms, margin = logit_errors(dec.logits(), om.logits)
+    print("prefill: logit err/std %.2e margin %.2e" % (err, margin), flush=True)
+    dec.close()
