@@ -205,7 +205,9 @@ int ptm_attn_decode_fused(const float* Q, const float* K, const float* V, const 
                           float scale, float eps, int add_one, int kv_fp16, int rope_interleaved,
                           ptm_stream_t stream);
 /* The same over a sliding window: only the last `window` positions, the new one included, are attended to
- * (window <= 0: all).  The local layers of gemma3 (attn_start, gguf_model.h:3490-3500). */
+ * (window <= 0: all).  The local layers of gemma3 (attn_start, gguf_model.h:3490-3500).  Both entries take head_dim
+ * 64, 128 or 256; 256-wide heads run the split-KV kernel of ptm_flash_decode with the norm / rotation / append
+ * prologue in front of it. */
 int ptm_attn_decode_fused_window(const float* Q, const float* K, const float* V, const float* q_norm_w,
                                  const float* k_norm_w, void* K_cache, void* V_cache, float* O, float* partial_O,
                                  float* partial_lse, float* partial_max, const float* rope_table,

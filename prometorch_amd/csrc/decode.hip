@@ -200,15 +200,6 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
         // a Q4_K output projection takes the attention output as the Q8 blocks the merge kernel leaves beside the fp32
         // vector: its prologue then copies 1.25 bytes per value instead of fetching and quantising 4
         const bool o_q8 = L.o.ggml_type == PTM_TYPE_Q4_K;
-        if (hd == 256) {
-            // heads this wide (gemma3) take the plain pair of launches: norm + rotation + K/V append, then split-KV attention
-            PTM_TRY(ptm_qknorm_rope_kvwrite(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, c.n_heads, c.n_kv_heads,
-                                            hd, d->d_past, c.max_seq, 0.0f, local ? d->rope_swa : d->rope, c.rms_eps, 0,
-                                            c.rope_interleaved ? 0 : 1, c.kv_fp16, s));
-            PTM_TRY(ptm_flash_decode_window(d->q, L.k_cache, L.v_cache, d->attn, o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM,
-                                            c.n_heads, c.n_kv_heads, hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd),
-                                            c.kv_fp16, local ? c.swa_window : 0, s));
-        } else
         PTM_TRY(ptm_attn_decode_fused_win(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn,
                                           o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM, local ? d->rope_swa : d->rope,
                                           c.n_heads, c.n_kv_heads, hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd),

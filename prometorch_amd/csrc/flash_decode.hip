@@ -43,20 +43,34 @@ __device__ __forceinline__ void load8(const void* base, int64_t elem_off, float 
     }
 }
 
-// grid (max_splits, n_kv_heads); G = query heads per kv head; HD = head_dim
-template <bool KV16, int HD, int G>
+// What a FUSED launch of the kernel below does first: per-head RMSNorm (optional) + rotation of the raw q heads and, in
+// the workgroup whose chunk holds the new position, of the raw k row, and the K/V append.
+struct FdFuse {
+    const float *K, *V, *qw, *kw, *rope;  // raw new k / v rows [kv_dim], norm weights (both or neither), table [max_seq][HD]
+    float eps;
+    int add_one, rope_interleaved;
+};
+
+// grid (max_splits, n_kv_heads); G = query heads per kv head; HD = head_dim.  FUSED: Q holds the raw projections and
+// the caches are appended to (the one-launch form for heads wider than the fused kernel further down covers).
+template <bool KV16, int HD, int G, bool FUSED = false>
 __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
-    const float* __restrict__ Q, const void* __restrict__ Kc, const void* __restrict__ Vc,
+    const float* __restrict__ Q, void* __restrict__ Kc, void* __restrict__ Vc,
     float* __restrict__ pO, float* __restrict__ pL, float* __restrict__ pM, int n_heads, int n_kv_heads,
-    const int64_t* __restrict__ d_past, int max_seq, float scale, int window) {
+    const int64_t* __restrict__ d_past, int max_seq, float scale, int window, const FdFuse f) {
     constexpr int LPP = HD / 8;         // lanes per position (each lane owns 8 dims)
     constexpr int PPW = 64 / LPP;       // positions per wave per pass
     constexpr int PPB = PPW * 4;        // positions per workgroup per pass
     constexpr int NPASS = FD_CHUNK / PPB;
     __shared__ float s_p[G][FD_CHUNK];
     __shared__ float s_o[4][G][HD];
+    __shared__ float s_q[FUSED ? G : 1][FUSED ? HD : 1];
+    __shared__ float s_new[2][FUSED ? HD : 1];
 
     int64_t total = *d_past + 1;
+    if constexpr (FUSED) {
+        if (total <= 0 || total > max_seq) return;  // never touch memory outside the cache
+    }
     if (total > max_seq) total = max_seq;
     const int split = blockIdx.x, kvh = blockIdx.y;
     const int64_t t0 = (int64_t)split * FD_CHUNK;
@@ -76,24 +90,106 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     const int dl = lane % LPP, pl = lane / LPP;
     const int kv_dim = n_kv_heads * HD;
     const int64_t col = (int64_t)kvh * HD + dl * 8;
+    const int64_t past = total - 1;
 
-    float q[G][8];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const float4 a = *reinterpret_cast<const float4*>(Q + (int64_t)(kvh * G + g) * HD + dl * 8);
-        const float4 b = *reinterpret_cast<const float4*>(Q + (int64_t)(kvh * G + g) * HD + dl * 8 + 4);
-        q[g][0] = a.x; q[g][1] = a.y; q[g][2] = a.z; q[g][3] = a.w;
-        q[g][4] = b.x; q[g][5] = b.y; q[g][6] = b.z; q[g][7] = b.w;
-    }
-
-    // ---- all K and V rows of the chunk are requested up front: one HBM round trip ----
+    // ---- all K and V rows of the chunk are requested up front: one HBM round trip (FUSED: the new position's row is
+    // not in the cache yet, it comes from LDS below) ----
     float kreg[NPASS][8], vreg[NPASS][8];
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
         const int64_t t = t0 + pass * PPB + wave * PPW + pl;
-        const int64_t tc = t < total ? t : total - 1;
+        const int64_t last = FUSED ? (past > 0 ? past - 1 : 0) : total - 1;
+        const int64_t tc = t <= last ? t : last;
         load8<KV16>(Kc, tc * kv_dim + col, kreg[pass]);
         load8<KV16>(Vc, tc * kv_dim + col, vreg[pass]);
+    }
+
+    float q[G][8];
+    if constexpr (FUSED) {
+        constexpr int HALF = HD / 2;
+        const bool owner = past >= t0 && past < t0 + FD_CHUNK;
+        const float* cs = f.rope + past * HD;
+        const float one = f.add_one ? 1.0f : 0.0f;
+        // wave w prepares heads w, w + 4, ...: the G query heads, then (owner only) the new k row; a lane owns rotation
+        // pairs lane and lane + 64
+        for (int it = wave; it < G + (owner ? 1 : 0); it += 4) {
+            const bool is_k = it == G;
+            const float* src = is_k ? f.K + (int64_t)kvh * HD : Q + (int64_t)(kvh * G + it) * HD;
+            const float* nw = is_k ? f.kw : f.qw;
+            float x0[2], x1[2];
+            int i0[2], i1[2];
+            bool on[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int t = lane + 64 * j;
+                on[j] = t < HALF;
+                i0[j] = f.rope_interleaved ? 2 * t : t;
+                i1[j] = f.rope_interleaved ? 2 * t + 1 : t + HALF;
+                x0[j] = on[j] ? src[i0[j]] : 0.0f;
+                x1[j] = on[j] ? src[i1[j]] : 0.0f;
+            }
+            if (nw) {
+                float ss = fmaf(x0[0], x0[0], 0.0f);
+                ss = fmaf(x1[0], x1[0], ss);
+                ss = fmaf(x0[1], x0[1], ss);
+                ss = fmaf(x1[1], x1[1], ss);
+                ss = sum64(ss);
+                const float rs = 1.0f / sqrtf(ss / (float)HD + f.eps);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (on[j]) {
+                        x0[j] = x0[j] * rs * (nw[i0[j]] + one);
+                        x1[j] = x1[j] * rs * (nw[i1[j]] + one);
+                    }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (!on[j]) continue;
+                const int t = lane + 64 * j;
+                const float c = cs[t], sn = cs[HALF + t];
+                float r0 = fmaf(x0[j], c, -(x1[j] * sn)), r1 = fmaf(x0[j], sn, x1[j] * c);
+                if (!is_k) {
+                    s_q[it][i0[j]] = r0;
+                    s_q[it][i1[j]] = r1;
+                } else {
+                    const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;
+                    float v0 = f.V[(int64_t)kvh * HD + t], v1 = f.V[(int64_t)kvh * HD + t + HALF];
+                    if constexpr (KV16) {
+                        const __half h0 = __float2half_rn(r0), h1 = __float2half_rn(r1), g0 = __float2half_rn(v0), g1 = __float2half_rn(v1);
+                        __half* kc = static_cast<__half*>(Kc) + rowoff;
+                        __half* vc = static_cast<__half*>(Vc) + rowoff;
+                        kc[i0[j]] = h0; kc[i1[j]] = h1; vc[t] = g0; vc[t + HALF] = g1;
+                        r0 = __half2float(h0); r1 = __half2float(h1); v0 = __half2float(g0); v1 = __half2float(g1);
+                    } else {
+                        float* kc = static_cast<float*>(Kc) + rowoff;
+                        float* vc = static_cast<float*>(Vc) + rowoff;
+                        kc[i0[j]] = r0; kc[i1[j]] = r1; vc[t] = v0; vc[t + HALF] = v1;
+                    }
+                    s_new[0][i0[j]] = r0; s_new[0][i1[j]] = r1;
+                    s_new[1][t] = v0; s_new[1][t + HALF] = v1;
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) q[g][i] = s_q[g][dl * 8 + i];
+#pragma unroll
+        for (int pass = 0; pass < NPASS; ++pass) {
+            if (t0 + pass * PPB + wave * PPW + pl == past) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { kreg[pass][i] = s_new[0][dl * 8 + i]; vreg[pass][i] = s_new[1][dl * 8 + i]; }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float4 a = *reinterpret_cast<const float4*>(Q + (int64_t)(kvh * G + g) * HD + dl * 8);
+            const float4 b = *reinterpret_cast<const float4*>(Q + (int64_t)(kvh * G + g) * HD + dl * 8 + 4);
+            q[g][0] = a.x; q[g][1] = a.y; q[g][2] = a.z; q[g][3] = a.w;
+            q[g][4] = b.x; q[g][5] = b.y; q[g][6] = b.z; q[g][7] = b.w;
+        }
     }
 
     // ---- scores ----
@@ -588,13 +684,14 @@ static int attn_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
     return launch_status();
 }
 
-template <bool KV16, int HD>
+template <bool KV16, int HD, bool FUSED = false>
 static int fd_launch_g(int G, dim3 grid, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* pO,
                        float* pL, float* pM, int n_heads, int n_kv_heads, const int64_t* d_past, int max_seq,
-                       float scale, int window = 0) {
-#define PTM_FD(GG)                                                                                              \
-    hipLaunchKernelGGL((flash_decode_partial_kernel<KV16, HD, GG>), grid, dim3(FD_THREADS), 0, s, Q, Kc, Vc, pO, \
-                       pL, pM, n_heads, n_kv_heads, d_past, max_seq, scale, window)
+                       float scale, int window = 0, const FdFuse& f = FdFuse{}) {
+#define PTM_FD(GG)                                                                                                     \
+    hipLaunchKernelGGL((flash_decode_partial_kernel<KV16, HD, GG, FUSED>), grid, dim3(FD_THREADS), 0, s, Q,             \
+                       const_cast<void*>(Kc), const_cast<void*>(Vc), pO, pL, pM, n_heads, n_kv_heads, d_past, max_seq, \
+                       scale, window, f)
     switch (G) {
         case 1: PTM_FD(1); break;
         case 2: PTM_FD(2); break;
@@ -664,8 +761,21 @@ int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, co
         return PTM_E_NULL;
     if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
     if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
-    if (head_dim != 64 && head_dim != 128) return PTM_E_UNSUPPORTED;
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return PTM_E_UNSUPPORTED;
     if (!aligned16(K_cache) || !aligned16(V_cache) || !aligned16(partial_O) || !aligned16(O)) return PTM_E_ALIGN;
+    if (head_dim == 256) {
+        // heads this wide (gemma3): the plain split-KV kernel with the norm / rotation / append prologue in front
+        if (o_q8 && (reinterpret_cast<uintptr_t>(o_q8) & 15u)) return PTM_E_ALIGN;
+        const FdFuse f{K, V, q_norm_w, k_norm_w, rope_table, eps, add_one, rope_interleaved ? 1 : 0};
+        const dim3 grid256(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
+        const int G256 = n_heads / n_kv_heads;
+        const int w = window > 0 ? window : 0;
+        const int rc256 = kv_fp16 ? fd_launch_g<true, 256, true>(G256, grid256, as_stream(stream), Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale, w, f)
+                                  : fd_launch_g<false, 256, true>(G256, grid256, as_stream(stream), Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale, w, f);
+        if (rc256 != PTM_OK) return rc256;
+        return fd_merge(head_dim, n_heads, as_stream(stream), partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
+                        static_cast<uint8_t*>(o_q8));
+    }
     AttnArgs a{Q, K, V, q_norm_w, k_norm_w, rope_table, K_cache, V_cache, partial_O, partial_lse, partial_max,
                d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps, rope_interleaved ? 1 : 0, window > 0 ? window : 0};
     const int G = n_heads / n_kv_heads;
