@@ -81,6 +81,20 @@ def test_host_side_validation_codes():
     assert L.ptm_q8_bytes(2560) == 2560 + 640
     assert L.ptm_flash_decode_num_splits(2176) == 34 and L.ptm_flash_decode_kv_chunk_size() == 64
     assert L.ptm_decode_create(None, None) == E_NULL
+    # the qwen2 / gemma3 additions
+    assert L.ptm_add_qkv_bias(16, 16, 16, 16, 16, None, 1, 256, 64, None) == E_NULL
+    assert L.ptm_add_qkv_bias(16, 16, 16, 16, 16, 16, 1, 0, 64, None) == E_SHAPE
+    assert L.ptm_add_qkv_bias(16, 16, 16, 16, 16, 16, 0, 256, 64, None) == 0            # no rows: nothing to do
+    assert L.ptm_rms_norm_add(16, 16, None, 1, 256, 1e-6, 0, None) == E_NULL
+    assert L.ptm_rms_norm_add(16, 16, 20, 1, 256, 1e-6, 0, None) == E_ALIGN            # rows are read as float4
+    assert L.ptm_gelu_mul(16, None, 16, 8, None) == E_NULL and L.ptm_gelu_mul(16, 16, 16, -1, None) == E_SHAPE
+    assert L.ptm_scale(None, 2.0, 8, None) == E_NULL and L.ptm_scale(16, 2.0, 0, None) == 0
+    assert L.ptm_flash_decode_window(16, 16, 16, 16, None, 16, 16, 16, 32, 8, 96, 16, 128, 1.0, 1, 8, None) == E_UNSUP
+    assert L.ptm_flash_decode_window(16, 16, 16, 16, 24, 16, 16, 16, 8, 4, 256, 16, 128, 1.0, 1, 8, None) == E_ALIGN  # Q8 copy
+    assert L.ptm_prefill_attention_window(16, 16, 16, 16, 4, 4, 2, 96, 0, 16, 0.1, 0, 8, None) == E_UNSUP
+    assert L.ptm_prefill_attention_window(16, 16, 16, 16, 4, 4, 2, 256, 14, 16, 0.1, 0, 8, None) == -6  # rows run past the cache
+    assert L.ptm_attn_decode_fused_window(16, 16, 16, 16, None, 16, 16, 16, 16, 16, 16, 16, 8, 4, 256, 16, 128, 1.0, 1e-6, 0,
+                                          1, 0, 8, None) == E_NULL                    # QK-norm weights: both or neither
 
 
 def test_rope_table_host_matches_oracle(po):
@@ -90,6 +104,12 @@ def test_rope_table_host_matches_oracle(po):
         c, s = po.rope_tables(pos, 128, 1e6)
         assert np.array_equal(t[pos, :64].view(np.uint32), c.view(np.uint32))
         assert np.array_equal(t[pos, 64:].view(np.uint32), s.view(np.uint32))
+    # linear position scaling, 256-wide heads
+    t = ops.rope_table(70, 256, 1e6, 8.0).numpy()
+    for pos in (0, 7, 69):
+        c, s = po.rope_tables(pos, 256, 1e6, 8.0)
+        assert np.array_equal(t[pos, :128].view(np.uint32), c.view(np.uint32))
+        assert np.array_equal(t[pos, 128:].view(np.uint32), s.view(np.uint32))
 
 
 def test_synth_generators_are_deterministic_and_in_range():
