@@ -23,6 +23,12 @@
  *   po_attn_head, po_silu_mul, po_argmax, po_decode_step
  *                          golden logits / token ids of the compiled reference's
  *                          forward_decode_cpu on a tiny and the full-size model
+ *   po_decode_step's model switches (no QK-norm, interleaved pairs, position scaling, q / k / v biases, scaled
+ *                          embeddings, GELU gate via po_gelu_mul, post-norms, sliding windows via
+ *                          po_attn_head_window with per-layer rotation bases): golden logits of the compiled
+ *                          reference on one tiny model per switch family (golden_llama / qwen2 / gemma .npz, each
+ *                          switch shown to move the logits) and on ten models with all switches drawn at random
+ *                          (golden_random_arch.npz), bit-exact; po_gelu_mul also against float64
  *   po_mt19937_*, po_uniform01   the 10000th output of the default-seeded generator (4123659995, ISO C++
  *                          [rand.predef]) + the tokens the compiled reference's sample_token draws with its
  *                          mt19937(42) (golden_sampling.npz)

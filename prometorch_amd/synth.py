@@ -345,6 +345,50 @@ def tiny_gemma(seed: int, n_layers: int = 4, head_dim: int = 64):
     return cfg, layers, make_head(seed, cfg)
 
 
+def random_model(seed):
+    """A small decoder with every architectural switch drawn at random: head width, query heads per kv head, QK-norm or
+    none, rotation pairing, position scaling, q / k / v biases, the gemma features each on its own, the type of every
+    matrix from the tuned pair."""
+    r = rng_for(97, seed)
+    hd = int(r.choice([64, 128, 256]))
+    G = int(r.integers(1, 9))
+    nkv = int(r.integers(1, 3))
+    nh = G * nkv
+    while (nh * hd) % 256:   # q_dim must hold whole super-blocks
+        nkv += 1
+        nh = G * nkv
+    cfg = dict(vocab=512, hidden=int(r.choice([256, 512, 768])), n_layers=int(r.integers(2, 5)), n_heads=nh, n_kv_heads=nkv,
+               head_dim=hd, inter=256 * int(r.integers(1, 5)), rope_base=float(r.choice([1.0e4, 1.0e6])), eps=1.0e-6)
+    if r.random() < 0.5:
+        cfg["rope_interleaved"] = True
+    if r.random() < 0.4:
+        cfg["rope_scale"] = float(r.choice([2.0, 8.0]))
+    if r.random() < 0.5:
+        cfg["scale_embeddings"] = True
+    if r.random() < 0.5:
+        cfg["ffn_gelu"] = True
+    if r.random() < 0.5:
+        cfg.update(swa_window=int(r.integers(1, 40)), swa_pattern=int(r.integers(1, 4)), rope_swa_base=1.0e4)
+    qk_norm, bias = r.random() < 0.5, r.random() < 0.5
+    post = [r.random() < 0.5, r.random() < 0.5]
+    layers = []
+    for i in range(cfg["n_layers"]):
+        mats = tuple((n, int(r.choice([Q4_K, Q6_K]))) for n in ("q", "k", "v", "o", "gate", "up", "down"))
+        L = make_layer(1000 + seed, i, cfg, mats=mats)
+        L["attn_norm"] = (np.float32(0.1) * L["attn_norm"]).astype(np.float32)
+        if not qk_norm:
+            L["q_norm"] = L["k_norm"] = None
+        g = rng_for(98, seed, i)
+        if bias:
+            for name, n in (("q_bias", nh * hd), ("k_bias", nkv * hd), ("v_bias", nkv * hd)):
+                L[name] = (np.float32(0.5) * g.standard_normal(n, dtype=np.float32)).astype(np.float32)
+        for on, name in zip(post, ("post_attn_norm", "post_ffn_norm")):
+            if on:
+                L[name] = (np.float32(0.5) * (1 + np.float32(0.1) * g.standard_normal(cfg["hidden"], dtype=np.float32))).astype(np.float32)
+        layers.append(L)
+    return cfg, layers, make_head(1000 + seed, cfg)
+
+
 # ---- sampling cases: (vocab, logit kind, temperature, top_k, top_p), in the order the golden run draws them ----
 SAMPLING_CASES = (
     [(1000, "normal", 0.8, 40, 0.9), (1000, "normal", 1.0, 0, 1.0), (1000, "normal", 0.7, 1, 1.0),

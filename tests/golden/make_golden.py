@@ -82,6 +82,7 @@ def main():
     ap.add_argument("--full", action="store_true")
     ap.add_argument("--sampling-only", action="store_true", help="write golden_sampling.npz and nothing else")
     ap.add_argument("--tokenizer-only", action="store_true", help="write golden_tokenizer.json and nothing else")
+    ap.add_argument("--random-only", action="store_true", help="write golden_random_arch.npz and nothing else")
     ap.add_argument("--gemma-only", action="store_true", help="write golden_gemma.npz and nothing else")
     ap.add_argument("--qwen2-only", action="store_true", help="write golden_qwen2.npz and nothing else")
     ap.add_argument("--llama-only", action="store_true", help="write golden_llama.npz and nothing else")
@@ -96,6 +97,10 @@ def main():
     if args.tokenizer_only:
         make_tokenizer_golden()
         print("wrote golden_tokenizer.json")
+        return
+    if args.random_only:
+        make_random_arch_golden()
+        print("wrote golden_random_arch.npz")
         return
     if args.gemma_only:
         make_gemma_golden()
@@ -242,6 +247,7 @@ def main():
     make_llama_golden()
     make_qwen2_golden()
     make_gemma_golden()
+    make_random_arch_golden()
     make_formats_golden()
     make_mixed_golden()
 
@@ -447,6 +453,27 @@ def make_gemma_golden():
         lg.append(rm.logits.copy())
     rm.close()
     np.savez_compressed(os.path.join(OUT, "golden_gemma.npz"), tokens=np.array(toks, np.int64), logits=np.stack(lg))
+
+
+def make_random_arch_golden():
+    """The reference's forward_decode_cpu on synth.random_model(0..9): ten decoders whose architectural switches (head width,
+    heads per kv head, QK-norm, rotation pairing and scaling, biases, the gemma features, per-matrix types) are drawn at
+    random; 4 steps each behind 11 cached positions."""
+    out = {}
+    for seed in range(10):
+        cfg, layers, head = synth.random_model(seed)
+        emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+        rm = po.RefModel(cfg, layers, head, 32, emb)
+        for i in range(cfg["n_layers"]):
+            k, v = synth.make_kv_prefill(1000 + seed, i, cfg, 11)
+            rm.set_kv(i, k, v)
+        tok, lg = 5, []
+        for _ in range(4):
+            tok = rm.step(tok)
+            lg.append(rm.logits.copy())
+        rm.close()
+        out["logits_%d" % seed] = np.stack(lg)
+    np.savez_compressed(os.path.join(OUT, "golden_random_arch.npz"), **out)
 
 
 def make_full(meta):

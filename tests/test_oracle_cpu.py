@@ -319,6 +319,26 @@ def test_gemma_style_decode_matches_the_reference(po, seeds):
         assert np.abs(l1[0] - g["logits"][0]).max() > 1e-2 * sigma, name
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_architectures_match_the_reference(po, seed):
+    """synth.random_model draws every architectural switch at random (head width, heads per kv head, QK-norm, rotation
+    pairing and scaling, biases, scaled embeddings, GELU, post-norms, sliding windows, per-matrix types): the oracle's
+    logits over 4 steps are bit-identical to the compiled reference's (golden_random_arch.npz), so the switches are
+    pinned in combination, not only one at a time."""
+    import os
+    from prometorch_amd import synth
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_random_arch.npz"))
+    cfg, layers, head = synth.random_model(seed)
+    om = po.OracleModel(cfg, layers, head, 32, kv_fp16=False)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(1000 + seed, i, cfg, 11)
+        om.set_kv(i, k, v)
+    tok = 5
+    for st in range(4):
+        tok = om.step(tok)
+        assert np.array_equal(om.logits.view(np.uint32), g["logits_%d" % seed][st].view(np.uint32)), st
+
+
 def test_gelu_gate_against_float64(po):
     r = np.random.default_rng(3)
     gate = (3 * r.standard_normal(4096)).astype(np.float32)
