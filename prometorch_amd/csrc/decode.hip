@@ -350,14 +350,11 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
                                         uses(PTM_TYPE_Q6_K, {&L.gate, &L.up}) ? d->pf_ws2 : nullptr, M, H, s));
         PTM_TRY(gemm(L.gate, d->pf_x, d->pf_gate, false, true));
         PTM_TRY(gemm(L.up, d->pf_x, d->pf_up, false, true));
-        bool act_ready = true;
-        if (c.ffn_gelu) {  // GELU.up as a launch of its own; the down product then converts its rows itself
-            PTM_TRY(ptm_gelu_mul(d->pf_gate, d->pf_up, d->pf_gate, (int64_t)M * I, s));
-            act_ready = false;
-        } else {
-            PTM_TRY(qgemm_f16_prepare_fused(2, d->pf_gate, d->pf_up, 0.0f, 0, L.down.ggml_type == PTM_TYPE_Q4_K ? d->pf_ws : nullptr,
-                                            L.down.ggml_type == PTM_TYPE_Q6_K ? d->pf_ws2 : nullptr, M, I, s));
-        }
+        const bool act_ready = true;
+        // SiLU.up (or, flagged through the add_one slot, GELU.up) fused into the conversion for the down projection
+        PTM_TRY(qgemm_f16_prepare_fused(2, d->pf_gate, d->pf_up, 0.0f, c.ffn_gelu ? 1 : 0,
+                                        L.down.ggml_type == PTM_TYPE_Q4_K ? d->pf_ws : nullptr,
+                                        L.down.ggml_type == PTM_TYPE_Q6_K ? d->pf_ws2 : nullptr, M, I, s));
         if (L.post_ffn_norm) {
             PTM_TRY(gemm(L.down, d->pf_gate, d->pf_h, false, act_ready));
             PTM_TRY(ptm_rms_norm_add(d->pf_h, L.post_ffn_norm, d->pf_x, M, H, c.rms_eps, 0, s));

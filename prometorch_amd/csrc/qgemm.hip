@@ -346,7 +346,8 @@ __global__ __launch_bounds__(256) void qgemm_prepare_rows_f16_kernel(const void*
 
 // The same conversion fused with what precedes a projection in the prompt pass, so that the fp32 intermediate is never
 // written: PRE 1 = RMSNorm of the row (x * rs * (gamma + add_one), the arithmetic and reduction order of
-// rms_norm_kernel), PRE 2 = SiLU(gate) * up (the arithmetic of silu_mul_kernel).  Writes the Q8-rounded form (for Q4_K
+// rms_norm_kernel), PRE 2 = SiLU(gate) * up (the arithmetic of silu_mul_kernel), or tanh-GELU(gate) * up (that of
+// gelu_mul_kernel) when add_one, which has no other meaning for PRE 2, is set.  Writes the Q8-rounded form (for Q4_K
 // matrices) and / or the plain form (for Q6_K matrices) in one pass; either output may be NULL.
 template <int PRE>
 __global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* __restrict__ X, const float* __restrict__ X2,
@@ -380,7 +381,13 @@ __global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* _
         if constexpr (PRE == 1) {
             r.x = a.x * rs * (b.x + one); r.y = a.y * rs * (b.y + one); r.z = a.z * rs * (b.z + one); r.w = a.w * rs * (b.w + one);
         } else {
-            auto silu_mul = [](float g, float u) {
+            const bool gelu = add_one != 0;
+            auto silu_mul = [gelu](float g, float u) {
+                if (gelu) {
+                    const float x3 = g * g * g;
+                    const float t = tanhf(0.7978845608028654f * (g + 0.044715f * x3));
+                    return 0.5f * g * (1.0f + t) * u;
+                }
                 float ng = 0.0f - g;
                 ng = fminf(fmaxf(ng, -88.0f), 88.0f);
                 return (g * (1.0f / (1.0f + expf(ng)))) * u;
