@@ -162,6 +162,14 @@ int ptm_qknorm_rope_kvwrite(float* Q, float* K, const float* V, const float* q_n
                             int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
                             float rope_freq_base, const float* rope_table, float eps, int add_one,
                             int neox, int kv_fp16, ptm_stream_t stream);
+/* The same with the position given by the host, for callers outside a captured graph: the rotation uses `position`, the
+ * K and V rows land in cache row `cache_offset_row` (the two may differ).  Replaces the non-graph
+ * launch_fused_qknorm_rope_kvwrite (CUDAOps.h:563-570; FlashDecoding.cu:256-395).  max_seq: height of the caches (and of
+ * rope_table when given); a row or position outside it returns PTM_E_RANGE. */
+int ptm_qknorm_rope_kvwrite_pos(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
+                                void* K_cache, void* V_cache, int n_heads, int n_kv_heads, int head_dim, int position,
+                                int64_t cache_offset_row, int max_seq, float rope_freq_base, const float* rope_table,
+                                float eps, int add_one, int neox, int kv_fp16, ptm_stream_t stream);
 /* Host-side helper: fill table[max_seq][head_dim] with the reference's fp32 cos/sin
  * (hot_loops.cpp:1853-1876: freq = 1/powf(base, 2d/hd), theta = pos*freq). table is a HOST pointer. */
 int ptm_rope_table_host(float* table, int max_seq, int head_dim, float rope_freq_base);
@@ -184,6 +192,12 @@ int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, f
                      float* partial_O, float* partial_lse, float* partial_max, int n_heads,
                      int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq, float scale,
                      int kv_fp16, ptm_stream_t stream);
+/* The same with the row count given by the host: attends rows [0, total_seq) of caches holding at least total_seq rows;
+ * scratch sized with ptm_flash_decode_num_splits(total_seq) or more.  Replaces the non-graph launch_flash_decode /
+ * launch_flash_decode_fp16 (CUDAOps.h:543-549, :641-647). */
+int ptm_flash_decode_pos(const float* Q, const void* K_cache, const void* V_cache, float* O, float* partial_O,
+                         float* partial_lse, float* partial_max, int n_heads, int n_kv_heads, int head_dim, int total_seq,
+                         float scale, int kv_fp16, ptm_stream_t stream);
 /* The same over a sliding window (window > 0: only the last `window` positions, gguf_model.h:3490-3500); o_q8, when not
  * NULL, also receives the output as Q8 activation blocks (ptm_q8_bytes(n_heads * head_dim), 16-byte aligned) for a Q4_K
  * output projection. */
@@ -267,6 +281,30 @@ int ptm_copy(const float* in, float* out, int64_t n, ptm_stream_t stream);
  * (gguf_model.h:2768-2779; CPU path :3413-3438): one fp32 add per element, before QK-norm and rotation. */
 int ptm_add_qkv_bias(float* Q, float* K, float* V, const float* q_bias, const float* k_bias, const float* v_bias, int rows,
                      int q_dim, int kv_dim, ptm_stream_t stream);
+
+/* ---- unquantised operators the reference's host code calls beside the k-quant kernels ------------------------
+ * out = a * factor (launch_mul_scalar, CUDAOps.h:67; in place when out == a). */
+int ptm_mul_scalar(const float* a, float factor, float* out, int64_t n, ptm_stream_t stream);
+/* fp32 rows [num_new_rows][cols] copied into a cache [.][cols] from row offset_row (launch_kv_cache_write,
+ * CUDAOps.h:410-413; KVCache::append, gguf_model.h:520-525). */
+int ptm_kv_cache_write(const float* src, float* dst_cache, int64_t num_new_rows, int64_t cols, int64_t offset_row,
+                       ptm_stream_t stream);
+/* out[a_rows + b_rows][cols] = rows of a, then rows of b (launch_concat, CUDAOps.h:404-407). */
+int ptm_concat_rows(const float* a, const float* b, float* out, int64_t a_rows, int64_t b_rows, int64_t cols,
+                    ptm_stream_t stream);
+/* In-place rotation of data[seq_len][n_heads * head_dim], row s at position position_offset + s (launch_rope,
+ * CUDAOps.h:392-395; CUDAInference.cu:149-189 rotates the interleaved pairs (2d, 2d + 1): neox = 0; neox != 0 rotates
+ * (d, d + head_dim / 2) as the reference's CPU path does for qwen / gemma / phi).  rope_table (device, table_rows rows as
+ * ptm_rope_table_host fills them) gives the host-libm angles; NULL computes them on the device from rope_freq_base. */
+int ptm_rope(float* data, int seq_len, int n_heads, int head_dim, int position_offset, float rope_freq_base,
+             const float* rope_table, int table_rows, int neox, ptm_stream_t stream);
+/* y[N] = W . x for unquantised weights.  fp32: k_major = 0 is W[N][K] row-major (launch_gemv, CUDAOps.h:188-192),
+ * k_major != 0 is W[K][N] (launch_inference_gemv, CUDAOps.h:422-424).  fp16: k_major = 0 is W[N][K] row-major
+ * (launch_fp16_gemv, CUDAOps.h:493-495; launch_cublas_hgemv with row_major), k_major != 0 the [K][N] order that
+ * ptm_dequant_q4k_to_fp16 writes (launch_cublas_hgemv's default, CUDAOps.h:484-489); round_x != 0 rounds x to fp16 first,
+ * as launch_cublas_hgemv does.  fp32 accumulation.  Plain kernels, not tuned: no Q4_K_M model takes these paths. */
+int ptm_f32_gemv(const float* W, const float* x, float* y, int K, int N, int k_major, ptm_stream_t stream);
+int ptm_f16_gemv(const void* W_fp16, const float* x, float* y, int K, int N, int k_major, int round_x, ptm_stream_t stream);
 
 /* Measurement aid with no counterpart in the reference: a pure streaming read of `bytes` (a multiple of 16, 16-byte
  * aligned) with 16-byte loads.  out_partials[i], i < ptm_stream_read_partials(bytes), receives the XOR of all 32-bit
@@ -370,9 +408,15 @@ typedef struct {
 
 typedef struct ptm_decoder ptm_decoder;
 
-/* Allocates scratch, the RoPE table, the decode stream and device scalars once; nothing is
- * allocated afterwards.  The KV caches and weights stay caller-owned. */
+/* Allocates the decode scratch, the RoPE table, the decode stream and device scalars once: no decode step allocates
+ * afterwards.  The row scratch of prompt prefill is separate: ptm_decode_reserve_prefill allocates it up front, otherwise
+ * the first ptm_decode_prefill (or one with more rows per chunk than any before) does.  The KV caches and weights stay
+ * caller-owned.  Each matrix is read with its own row_stride_bytes (at least a dense row, 16-byte multiples for Q4_K, even for
+ * Q6_K; the Q4_K matrices among q / k / v share one stride), PTM_E_SHAPE otherwise. */
 int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out);
+/* Allocate the prefill row scratch for chunks of up to `rows` prompt rows (capped at 2048) now, so that no later
+ * ptm_decode_prefill with chunk_rows <= rows allocates. */
+int ptm_decode_reserve_prefill(ptm_decoder* d, int rows);
 void ptm_decode_destroy(ptm_decoder* d);
 /* Set the number of positions already present in the KV caches (after prefill). */
 int ptm_decode_set_past_len(ptm_decoder* d, int64_t past_len);
@@ -387,7 +431,8 @@ int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token);
  * prompt token are left for ptm_decode_logits.  Rows go through the layers in chunks of chunk_rows
  * (<= 0 or above 2048: 2048) with the fast quantised GEMM, row-batched QK-norm + RoPE + KV append and causal attention.
  * The counterpart of GGUFModel::forward(tokens, use_cache = true) (gguf_model.h:2510-2571); row m equals
- * a decode step of token m up to the fp16 rounding of the GEMM operands.  Allocates its scratch on first use. */
+ * a decode step of token m up to the fp16 rounding of the GEMM operands.  Allocates its row scratch on first use unless
+ * ptm_decode_reserve_prefill has reserved enough rows. */
 int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_rows, int64_t* next_token);
 /* Sampled generation (the decode loop of promeserve/api_handlers.h:848-923 with the sampling kept on the GPU).
  * ptm_decode_sampling_begin starts a generation: stores the parameters and forgets the tokens generated so far

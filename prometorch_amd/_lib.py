@@ -88,6 +88,14 @@ SIGNATURES = {
     "ptm_rms_norm": (i32, [vp, vp, vp, i32, i32, f32, i32, vp, vp]),
     "ptm_per_head_rms_norm": (i32, [vp, vp, i32, i32, i32, f32, i32, vp]),
     "ptm_qknorm_rope_kvwrite": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, i32, f32, vp, f32, i32, i32, i32, vp]),
+    "ptm_qknorm_rope_kvwrite_pos": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, vp, f32, i32, i32, i32, vp]),
+    "ptm_flash_decode_pos": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp]),
+    "ptm_mul_scalar": (i32, [vp, f32, vp, i64, vp]),
+    "ptm_kv_cache_write": (i32, [vp, vp, i64, i64, i64, vp]),
+    "ptm_concat_rows": (i32, [vp, vp, vp, i64, i64, i64, vp]),
+    "ptm_rope": (i32, [vp, i32, i32, i32, i32, f32, vp, i32, i32, vp]),
+    "ptm_f32_gemv": (i32, [vp, vp, vp, i32, i32, i32, vp]),
+    "ptm_f16_gemv": (i32, [vp, vp, vp, i32, i32, i32, i32, vp]),
     "ptm_rope_table_host": (i32, [vp, i32, i32, f32]),
     "ptm_rope_table_host_scaled": (i32, [vp, i32, i32, f32, f32]),
     "ptm_fp16_kv_cache_write": (i32, [vp, vp, i64, i64, i64, vp]),
@@ -118,6 +126,7 @@ SIGNATURES = {
     "ptm_decode_create": (i32, [C.POINTER(DecodeConfig), C.POINTER(vp)]),
     "ptm_decode_destroy": (None, [vp]),
     "ptm_decode_set_past_len": (i32, [vp, i64]),
+    "ptm_decode_reserve_prefill": (i32, [vp, i32]),
     "ptm_decode_step": (i32, [vp, i32, C.POINTER(i64)]),
     "ptm_decode_greedy": (i32, [vp, i32, i32, C.POINTER(i64)]),
     "ptm_decode_prefill": (i32, [vp, C.POINTER(C.c_int32), i32, i32, C.POINTER(i64)]),

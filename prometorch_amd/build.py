@@ -8,7 +8,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libptm_hip.so")
-SOURCES = ["glue.hip", "q4k_gemv.hip", "q6k_gemv.hip", "flash_decode.hip", "mixed_gemv.hip", "qgemm.hip", "decode.hip", "dispatch.hip", "other_gemv.hip", "gguf.hip", "prefill.hip", "sampler.hip", "tokenizer.hip"]
+SOURCES = ["glue.hip", "q4k_gemv.hip", "q6k_gemv.hip", "flash_decode.hip", "mixed_gemv.hip", "qgemm.hip", "decode.hip", "dispatch.hip", "other_gemv.hip", "gguf.hip", "prefill.hip", "sampler.hip", "tokenizer.hip", "plain_ops.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",

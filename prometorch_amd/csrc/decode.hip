@@ -134,6 +134,9 @@ static int qw_check(const ptm_qweight& w, int rows, int cols) {
     if (!w.data) return PTM_E_NULL;
     if (w.rows != rows || w.cols != cols) return PTM_E_SHAPE;
     if (!ptm_quant_gemv_supported(w.ggml_type)) return PTM_E_UNSUPPORTED;
+    // the row stride is the descriptor's own (rows may be padded); it must hold a row and keep the rows aligned
+    if (w.ggml_type == PTM_TYPE_Q4_K && (w.row_stride_bytes < (int64_t)(cols / 256) * 144 || (w.row_stride_bytes & 15))) return PTM_E_SHAPE;
+    if (w.ggml_type == PTM_TYPE_Q6_K && (w.row_stride_bytes < (int64_t)(cols / 256) * 210 || (w.row_stride_bytes & 1))) return PTM_E_SHAPE;
     return PTM_OK;
 }
 
@@ -179,7 +182,8 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
                 if (w[i]->ggml_type == PTM_TYPE_Q4_K) { W4[n4] = w[i]->data; y4[n4] = y[i]; N4[n4] = w[i]->rows; ++n4; }
                 else { i6 = i; ++n6; }
             }
-            const int64_t s4 = (int64_t)(H / 256) * 144;
+            int64_t s4 = 0;  // the Q4_K projections of one launch share a row stride (checked at create)
+            for (int i = 0; i < 3; ++i) if (w[i]->ggml_type == PTM_TYPE_Q4_K) { s4 = w[i]->row_stride_bytes; break; }
             if (!tuned_type(L.q.ggml_type) || !tuned_type(L.k.ggml_type) || !tuned_type(L.v.ggml_type)) {
                 PTM_TRY(ptm_rms_norm(d->x, L.attn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
                 for (int i = 0; i < 3; ++i) PTM_TRY(gemv_any(*w[i], d->xn, y[i], false, s));
@@ -392,6 +396,13 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
             (rc = qw_check(L.o, H, qd)) || (rc = qw_check(L.gate, c.inter, H)) || (rc = qw_check(L.up, c.inter, H)) ||
             (rc = qw_check(L.down, H, c.inter)))
             return rc;
+        // q / k / v in Q4_K go through one launch with one row stride
+        int64_t s4 = -1;
+        for (const ptm_qweight* w : {&L.q, &L.k, &L.v}) {
+            if (w->ggml_type != PTM_TYPE_Q4_K) continue;
+            if (s4 >= 0 && w->row_stride_bytes != s4) return PTM_E_SHAPE;
+            s4 = w->row_stride_bytes;
+        }
     }
     ptm_decoder* d = new (std::nothrow) ptm_decoder();
     if (!d) return PTM_E_STATE;
@@ -592,6 +603,17 @@ int ptm_decode_generate(ptm_decoder* d, const int32_t* prompt, int n_prompt, con
     }
     *n_out = produced;
     return PTM_OK;
+}
+
+int ptm_decode_reserve_prefill(ptm_decoder* d, int rows) {
+    if (!d) return PTM_E_NULL;
+    if (d->status != PTM_OK) return PTM_E_STATE;
+    if (rows <= 0) return PTM_E_SHAPE;
+    if (d->untuned_types) return PTM_OK;  // such models are prefilled token by token: no row scratch
+    if (rows > 2048) rows = 2048;
+    const int rc = hip_status(hipStreamSynchronize(d->stream));  // the slab may be replaced: nothing may still use it
+    if (rc != PTM_OK) return rc;
+    return prefill_alloc(d, rows);
 }
 
 int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_rows, int64_t* next_token) {

@@ -57,7 +57,7 @@ template <bool KV16, int HD, int G, bool FUSED = false>
 __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     const float* __restrict__ Q, void* __restrict__ Kc, void* __restrict__ Vc,
     float* __restrict__ pO, float* __restrict__ pL, float* __restrict__ pM, int n_heads, int n_kv_heads,
-    const int64_t* __restrict__ d_past, int max_seq, float scale, int window, const FdFuse f) {
+    const int64_t* __restrict__ d_past, int64_t past_host, int max_seq, float scale, int window, const FdFuse f) {
     constexpr int LPP = HD / 8;         // lanes per position (each lane owns 8 dims)
     constexpr int PPW = 64 / LPP;       // positions per wave per pass
     constexpr int PPB = PPW * 4;        // positions per workgroup per pass
@@ -67,7 +67,8 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     __shared__ float s_q[FUSED ? G : 1][FUSED ? HD : 1];
     __shared__ float s_new[2][FUSED ? HD : 1];
 
-    int64_t total = *d_past + 1;
+    // d_past == NULL: the position is the host argument (launch_flash_decode's total_seq, CUDAOps.h:543-549)
+    int64_t total = (d_past ? *d_past : past_host) + 1;
     if constexpr (FUSED) {
         if (total <= 0 || total > max_seq) return;  // never touch memory outside the cache
     }
@@ -271,7 +272,8 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
                                                                  const float* __restrict__ pL,
                                                                  const float* __restrict__ pM, float* __restrict__ O,
                                                                  int n_heads, const int64_t* __restrict__ d_past,
-                                                                 int max_seq, uint8_t* __restrict__ q8_out) {
+                                                                 int64_t past_host, int max_seq,
+                                                                 uint8_t* __restrict__ q8_out) {
     constexpr int NOUT = HD / 4, NSLOT = 256 / NOUT;
     __shared__ __align__(16) float4 s_stage[256];
     __shared__ float s_red[8];
@@ -282,7 +284,7 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
     // are clamped into the allocation (ns_max chunks) and dropped by selects below, so the kernel makes one
     // memory round trip, not one for the position and a second for the data.
     const int ns_max = (max_seq + FD_CHUNK - 1) / FD_CHUNK;
-    const int64_t past = *d_past;
+    const int64_t past = d_past ? *d_past : past_host;
     float4 v[8];
     float mm[8];
 #pragma unroll
@@ -358,13 +360,13 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
 }
 
 static int fd_merge(int head_dim, int n_heads, hipStream_t s, const float* pO, const float* pL, const float* pM, float* O,
-                    const int64_t* d_past, int max_seq, uint8_t* q8_out = nullptr) {
+                    const int64_t* d_past, int max_seq, uint8_t* q8_out = nullptr, int64_t past_host = 0) {
     if (head_dim == 256)
-        hipLaunchKernelGGL(flash_decode_merge_kernel<256>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq, q8_out);
+        hipLaunchKernelGGL(flash_decode_merge_kernel<256>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out);
     else if (head_dim == 128)
-        hipLaunchKernelGGL(flash_decode_merge_kernel<128>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq, q8_out);
+        hipLaunchKernelGGL(flash_decode_merge_kernel<128>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out);
     else
-        hipLaunchKernelGGL(flash_decode_merge_kernel<64>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, max_seq, q8_out);
+        hipLaunchKernelGGL(flash_decode_merge_kernel<64>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out);
     return launch_status();
 }
 
@@ -687,11 +689,11 @@ static int attn_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
 template <bool KV16, int HD, bool FUSED = false>
 static int fd_launch_g(int G, dim3 grid, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* pO,
                        float* pL, float* pM, int n_heads, int n_kv_heads, const int64_t* d_past, int max_seq,
-                       float scale, int window = 0, const FdFuse& f = FdFuse{}) {
+                       float scale, int window = 0, const FdFuse& f = FdFuse{}, int64_t past_host = 0) {
 #define PTM_FD(GG)                                                                                                     \
     hipLaunchKernelGGL((flash_decode_partial_kernel<KV16, HD, GG, FUSED>), grid, dim3(FD_THREADS), 0, s, Q,             \
-                       const_cast<void*>(Kc), const_cast<void*>(Vc), pO, pL, pM, n_heads, n_kv_heads, d_past, max_seq, \
-                       scale, window, f)
+                       const_cast<void*>(Kc), const_cast<void*>(Vc), pO, pL, pM, n_heads, n_kv_heads, d_past, past_host, \
+                       max_seq, scale, window, f)
     switch (G) {
         case 1: PTM_FD(1); break;
         case 2: PTM_FD(2); break;
@@ -723,11 +725,11 @@ int ptm_flash_decode(const float* Q, const void* K_cache, const void* V_cache, f
                                    head_dim, d_past_len, max_seq, scale, kv_fp16, 0, stream);
 }
 
-int ptm_flash_decode_window(const float* Q, const void* K_cache, const void* V_cache, float* O, void* o_q8,
+static int flash_decode_any(const float* Q, const void* K_cache, const void* V_cache, float* O, void* o_q8,
                             float* partial_O, float* partial_lse, float* partial_max, int n_heads, int n_kv_heads,
-                            int head_dim, const int64_t* d_past_len, int max_seq, float scale, int kv_fp16, int window,
-                            ptm_stream_t stream) {
-    if (!Q || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max || !d_past_len)
+                            int head_dim, const int64_t* d_past_len, int64_t past_host, int max_seq, float scale, int kv_fp16,
+                            int window, ptm_stream_t stream) {
+    if (!Q || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max)
         return PTM_E_NULL;
     if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return PTM_E_UNSUPPORTED;
@@ -738,13 +740,31 @@ int ptm_flash_decode_window(const float* Q, const void* K_cache, const void* V_c
     const dim3 grid(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
     hipStream_t s = as_stream(stream);
     int rc;
-#define PTM_FDW(KV, HDV) fd_launch_g<KV, HDV>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale, window)
+#define PTM_FDW(KV, HDV) fd_launch_g<KV, HDV>(G, grid, s, Q, K_cache, V_cache, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, d_past_len, max_seq, scale, window, FdFuse{}, past_host)
     if (kv_fp16) rc = head_dim == 256 ? PTM_FDW(true, 256) : head_dim == 128 ? PTM_FDW(true, 128) : PTM_FDW(true, 64);
     else rc = head_dim == 256 ? PTM_FDW(false, 256) : head_dim == 128 ? PTM_FDW(false, 128) : PTM_FDW(false, 64);
 #undef PTM_FDW
     if (rc != PTM_OK) return rc;
     return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
-                    static_cast<uint8_t*>(o_q8));
+                    static_cast<uint8_t*>(o_q8), past_host);
+}
+
+int ptm_flash_decode_window(const float* Q, const void* K_cache, const void* V_cache, float* O, void* o_q8,
+                            float* partial_O, float* partial_lse, float* partial_max, int n_heads, int n_kv_heads,
+                            int head_dim, const int64_t* d_past_len, int max_seq, float scale, int kv_fp16, int window,
+                            ptm_stream_t stream) {
+    if (!d_past_len) return PTM_E_NULL;
+    return flash_decode_any(Q, K_cache, V_cache, O, o_q8, partial_O, partial_lse, partial_max, n_heads, n_kv_heads, head_dim,
+                            d_past_len, 0, max_seq, scale, kv_fp16, window, stream);
+}
+
+// Position from the host: attends rows [0, total_seq) of caches that hold at least total_seq rows.
+int ptm_flash_decode_pos(const float* Q, const void* K_cache, const void* V_cache, float* O, float* partial_O,
+                         float* partial_lse, float* partial_max, int n_heads, int n_kv_heads, int head_dim, int total_seq,
+                         float scale, int kv_fp16, ptm_stream_t stream) {
+    if (total_seq <= 0) return PTM_E_RANGE;
+    return flash_decode_any(Q, K_cache, V_cache, O, nullptr, partial_O, partial_lse, partial_max, n_heads, n_kv_heads,
+                            head_dim, nullptr, (int64_t)total_seq - 1, total_seq, scale, kv_fp16, 0, stream);
 }
 
 // ptm_attn_decode_fused that can also leave the output as Q8 activation blocks (o_q8, may be NULL) for a Q4_K output

@@ -217,10 +217,15 @@ __global__ __launch_bounds__(64) void qknorm_rope_kvwrite_kernel(float* __restri
                                                                  const float* __restrict__ kw, void* __restrict__ Kc,
                                                                  void* __restrict__ Vc, int n_heads, int n_kv_heads,
                                                                  int head_dim, const int64_t* __restrict__ d_past,
+                                                                 int64_t pos_host, int64_t row_host,
                                                                  int max_seq, float base, const float* __restrict__ table,
                                                                  float eps, int add_one, int neox) {
-    const int64_t pos = *d_past;
-    if (pos < 0 || pos >= max_seq) return;  // never write outside the cache
+    // d_past != NULL: position and cache row both come from device memory (graph-replayable); otherwise from the host
+    // arguments, where the rotation position and the cache row may differ (launch_fused_qknorm_rope_kvwrite's
+    // `position` / `cache_offset_row`, CUDAOps.h:563-570)
+    const int64_t pos = d_past ? *d_past : pos_host;
+    const int64_t crow = d_past ? pos : row_host;
+    if (pos < 0 || crow < 0 || crow >= max_seq || (table && pos >= max_seq)) return;  // never touch memory outside the cache / table
     const int hb = blockIdx.x;
     const bool is_k = hb >= n_heads;
     const int h = is_k ? hb - n_heads : hb;
@@ -274,7 +279,7 @@ __global__ __launch_bounds__(64) void qknorm_rope_kvwrite_kernel(float* __restri
         vec[i0[j]] = r0;
         vec[i1[j]] = r1;
         if (is_k) {
-            const int64_t row = pos * (int64_t)(n_kv_heads * head_dim) + (int64_t)h * head_dim;
+            const int64_t row = crow * (int64_t)(n_kv_heads * head_dim) + (int64_t)h * head_dim;
             const float v0 = V[h * head_dim + i0[j]], v1 = V[h * head_dim + i1[j]];
             if constexpr (KV16) {
                 __half* kc = static_cast<__half*>(Kc) + row;
@@ -506,24 +511,45 @@ int ptm_per_head_rms_norm(float* data, const float* weight, int rows, int n_head
     return launch_status();
 }
 
-int ptm_qknorm_rope_kvwrite(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
-                            void* K_cache, void* V_cache, int n_heads, int n_kv_heads, int head_dim,
-                            const int64_t* d_past_len, int max_seq, float rope_freq_base, const float* rope_table,
-                            float eps, int add_one, int neox, int kv_fp16, ptm_stream_t stream) {
-    if (!Q || !K || !V || !K_cache || !V_cache || !d_past_len) return PTM_E_NULL;
+static int qknorm_rope_kvwrite_any(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
+                                   void* K_cache, void* V_cache, int n_heads, int n_kv_heads, int head_dim,
+                                   const int64_t* d_past_len, int64_t pos_host, int64_t row_host, int max_seq,
+                                   float rope_freq_base, const float* rope_table, float eps, int add_one, int neox,
+                                   int kv_fp16, ptm_stream_t stream) {
+    if (!Q || !K || !V || !K_cache || !V_cache) return PTM_E_NULL;
     if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
     if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || head_dim <= 0 || (head_dim & 1)) return PTM_E_SHAPE;
     if (head_dim > 256) return PTM_E_UNSUPPORTED;
     const dim3 grid(n_heads + n_kv_heads);
     if (kv_fp16)
         hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<true>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w,
-                           k_norm_w, K_cache, V_cache, n_heads, n_kv_heads, head_dim, d_past_len, max_seq,
+                           k_norm_w, K_cache, V_cache, n_heads, n_kv_heads, head_dim, d_past_len, pos_host, row_host, max_seq,
                            rope_freq_base, rope_table, eps, add_one, neox);
     else
         hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<false>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w,
-                           k_norm_w, K_cache, V_cache, n_heads, n_kv_heads, head_dim, d_past_len, max_seq,
+                           k_norm_w, K_cache, V_cache, n_heads, n_kv_heads, head_dim, d_past_len, pos_host, row_host, max_seq,
                            rope_freq_base, rope_table, eps, add_one, neox);
     return launch_status();
+}
+
+int ptm_qknorm_rope_kvwrite(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
+                            void* K_cache, void* V_cache, int n_heads, int n_kv_heads, int head_dim,
+                            const int64_t* d_past_len, int max_seq, float rope_freq_base, const float* rope_table,
+                            float eps, int add_one, int neox, int kv_fp16, ptm_stream_t stream) {
+    if (!d_past_len) return PTM_E_NULL;
+    return qknorm_rope_kvwrite_any(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, n_heads, n_kv_heads, head_dim, d_past_len,
+                                   0, 0, max_seq, rope_freq_base, rope_table, eps, add_one, neox, kv_fp16, stream);
+}
+
+int ptm_qknorm_rope_kvwrite_pos(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
+                                void* K_cache, void* V_cache, int n_heads, int n_kv_heads, int head_dim, int position,
+                                int64_t cache_offset_row, int max_seq, float rope_freq_base, const float* rope_table,
+                                float eps, int add_one, int neox, int kv_fp16, ptm_stream_t stream) {
+    if (position < 0 || cache_offset_row < 0 || cache_offset_row >= max_seq || (rope_table && position >= max_seq))
+        return PTM_E_RANGE;
+    return qknorm_rope_kvwrite_any(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, n_heads, n_kv_heads, head_dim, nullptr,
+                                   position, cache_offset_row, max_seq, rope_freq_base, rope_table, eps, add_one, neox,
+                                   kv_fp16, stream);
 }
 
 int ptm_rope_table_host(float* table, int max_seq, int head_dim, float base) {

@@ -181,6 +181,9 @@ __global__ __launch_bounds__(1024) void argmax_partials_kernel(const float* pv, 
     if (threadIdx.x == 0) {
         for (int w = 1; w < 16; ++w)
             if (bv[w] > v || (bv[w] == v && bi[w] < idx)) { v = bv[w]; idx = bi[w]; }
+        // every comparison against NaN is false: with all-NaN logits no candidate ever replaces the start value.  Publish
+        // row 0 then (as the standalone argmax does), never an index outside the table the next step's embedding reads.
+        if (idx == 0x7fffffff) idx = 0;
         *out = (int64_t)idx;
         if (adv.d_token) {
             if (step < adv.cap) adv.tokens_out[step] = (int64_t)idx;

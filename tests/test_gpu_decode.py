@@ -150,3 +150,43 @@ def test_cfg4_qwen3_4b_shape_128_greedy_tokens(dev, po, golden_cfg4, seeds):
     dec.set_past_len(2048)
     assert dec.greedy(1, 128) == want_ref
     dec.close()
+
+
+def test_padded_row_strides_are_honoured(dev, seeds):
+    """Every matrix with 16 bytes of padding behind each row: the decode step and the prompt path read each matrix
+    with its descriptor's stride, so logits are bit-identical to the dense layout; q / k strides that differ are refused."""
+    from prometorch_amd import _lib
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = build_tiny(seeds)
+    padded = []
+    for Ld in layers:
+        P = dict(Ld)
+        for name in ("q", "k", "v", "o", "gate", "up", "down"):
+            qt, W = Ld[name]
+            P[name] = (qt, np.ascontiguousarray(np.pad(W, ((0, 0), (0, 16)), constant_values=0xA5)))
+        padded.append(P)
+    outs = []
+    for ls in (layers, padded):
+        dec = Decoder(cfg, ls, head, max_seq=64, kv_fp16=True, use_graph=True)
+        for i, (k, v) in enumerate(kv):
+            dec.set_kv(i, k, v)
+        dec.set_past_len(19)
+        toks, lg = [], []
+        t = 3
+        for _ in range(4):
+            t = dec.step(t)
+            toks.append(t)
+            lg.append(dec.logits())
+        t = dec.prefill([5, 9, 200, 31, 7, 7, 64, 2])
+        toks.append(t)
+        lg.append(dec.logits())
+        outs.append((toks, lg))
+        dec.close()
+    assert outs[0][0] == outs[1][0]
+    for a, b in zip(outs[0][1], outs[1][1]):
+        assert np.array_equal(bits(a), bits(b))
+    bad = [dict(L) for L in padded]
+    bad[0]["k"] = layers[0]["k"]   # q padded, k dense: one launch cannot serve two strides
+    with pytest.raises(_lib.PtmError) as e:
+        Decoder(cfg, bad, head, max_seq=64, kv_fp16=True, use_graph=True)
+    assert e.value.code == -2

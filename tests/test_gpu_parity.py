@@ -619,3 +619,18 @@ def test_gemv_random_shapes_vs_oracle(dev, po):
         worst[qt] = max(worst.get(qt, 0.0), e)
         assert e <= GEMV_TOL * 1e-1, (case, qt, N, K, accumulate, e)
     print("worst rel err per type:", {k: "%.1e" % v for k, v in worst.items()})
+
+
+def test_fused_argmax_of_nan_logits_publishes_a_row_inside_the_table(dev):
+    """All-NaN logits (a NaN anywhere in the hidden state): no comparison is ever true; the fused lm_head tail must still
+    publish an index inside [0, N), because the next captured step reads that row of the embedding table."""
+    N, K = 1024, 256
+    W = synth.make_weight(synth.rng_for(3), 14, N, K)
+    Wd = torch.from_numpy(W).cuda()
+    xd = torch.full((K,), float("nan"), device="cuda")
+    logits = torch.zeros(N, device="cuda")
+    idx = torch.full((1,), -7, dtype=torch.int64, device="cuda")
+    ws = torch.empty(ops.argmax_workspace_bytes(N), dtype=torch.uint8, device="cuda")
+    ops.q6k_gemv_argmax(Wd, xd, logits, K, N, W.shape[1], idx, ws)
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(logits).all()) and 0 <= int(idx.item()) < N
