@@ -88,6 +88,15 @@ int64_t ptm_argmax_workspace_bytes(int N);
 int ptm_q6k_gemv_argmax(const void* W, const float* x, float* logits, int K, int N,
                         int64_t row_stride_bytes, int64_t* out_index, void* workspace,
                         ptm_stream_t stream);
+/* The same for callers that cannot allocate device memory (code under hipGraph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no workspace argument, the per-workgroup partials live in a device array inside the
+ * library (512 KiB per GPU, held until the process ends).  No counterpart in the reference.  N above
+ * ptm_q6k_gemv_argmax_noalloc_max_rows() (262144) returns PTM_E_RANGE.  Calls no hipMalloc / hipFree.  All calls on one
+ * GPU share that GPU's array: calls that overlap in time on one GPU (different streams) race; calls ordered on one
+ * stream do not.  Same results as ptm_q6k_gemv_argmax. */
+int ptm_q6k_gemv_argmax_noalloc_max_rows(void);
+int ptm_q6k_gemv_argmax_noalloc(const void* W, const float* x, float* logits, int K, int N, int64_t row_stride_bytes,
+                                int64_t* out_index, ptm_stream_t stream);
 /* Type dispatcher mirroring cpu_quant_gemv (cpu_quant_gemv.h:1635-1688) and gemv_scratch
  * (gguf_model.h:3117-3140): 12 -> Q4_K, 14 -> Q6_K, 13 -> Q5_K, 8 -> Q8_0, 6 -> Q5_0; anything else returns
  * PTM_E_UNSUPPORTED and launches nothing (the reference silently no-ops).  ptm_quant_gemv_supported mirrors

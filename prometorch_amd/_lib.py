@@ -78,6 +78,8 @@ SIGNATURES = {
     "ptm_q6k_gemv": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
     "ptm_argmax_workspace_bytes": (i64, [i32]),
     "ptm_q6k_gemv_argmax": (i32, [vp, vp, vp, i32, i32, i64, vp, vp, vp]),
+    "ptm_q6k_gemv_argmax_noalloc_max_rows": (i32, []),
+    "ptm_q6k_gemv_argmax_noalloc": (i32, [vp, vp, vp, i32, i32, i64, vp, vp]),
     "ptm_quant_gemv": (i32, [u32, vp, vp, vp, i32, i32, i64, i32, vp]),
     "ptm_q4k_fused_gate_up_gemv": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i64, vp]),
     "ptm_q4k_fused_qkv_gemv": (i32, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i64, vp]),

@@ -16,6 +16,8 @@
 // count the loads in flight and each block is consumed as soon as it has arrived.
 #include "q6k_body.h"
 
+#include <mutex>
+
 namespace ptm {
 
 template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
@@ -312,6 +314,54 @@ int64_t ptm_argmax_workspace_bytes(int N) {
 int ptm_q6k_gemv_argmax(const void* W, const float* x, float* logits, int K, int N, int64_t stride,
                         int64_t* out_index, void* workspace, ptm_stream_t stream) {
     return q6k_gemv_argmax_impl(W, x, nullptr, 0.f, 0, nullptr, logits, K, N, stride, out_index, workspace,
+                                ArgmaxAdvance{nullptr, nullptr, nullptr, nullptr, 0}, as_stream(stream));
+}
+
+}  // extern "C"
+
+// ---- the same operator for callers that cannot allocate device memory ------------------------------------------
+// The per-workgroup (value, index) pairs of the fused argmax live in a device array of this library instead of a
+// caller-provided workspace.  Every GPU the library runs on holds its own copy of the array, at its own address,
+// until the process ends; host code only ever uses the address looked up below, never the array's name.
+enum { PTM_NOALLOC_MAX_ROWS = 262144 };  // 8 bytes per 4 rows: 512 KiB
+static __device__ __align__(256) unsigned char scratch[(PTM_NOALLOC_MAX_ROWS / 4) * 8];
+
+namespace {
+enum { MAX_DEVICES = 64 };
+void* g_scratch_ptr[MAX_DEVICES];  // per device, filled on the first call with that device current
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (no allocation: a symbol lookup), or NULL with *rc set.
+void* scratch_on_current_device(int* rc) {
+    int dev = -1;
+    *rc = hip_status(hipGetDevice(&dev));
+    if (*rc != PTM_OK) return nullptr;
+    if (dev < 0 || dev >= MAX_DEVICES) { *rc = PTM_E_UNSUPPORTED; return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        *rc = hip_status(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (*rc != PTM_OK) return nullptr;
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" {
+
+int ptm_q6k_gemv_argmax_noalloc_max_rows(void) { return PTM_NOALLOC_MAX_ROWS; }
+
+int ptm_q6k_gemv_argmax_noalloc(const void* W, const float* x, float* logits, int K, int N, int64_t stride,
+                                int64_t* out_index, ptm_stream_t stream) {
+    if (N > PTM_NOALLOC_MAX_ROWS) return PTM_E_RANGE;  // the array holds the partials of at most that many rows
+    if (N > 0 && ptm_argmax_workspace_bytes(N) > (int64_t)sizeof(scratch)) return PTM_E_RANGE;
+    int rc = PTM_OK;
+    void* ws = scratch_on_current_device(&rc);
+    if (!ws) return rc;
+    // every workgroup of the GEMV overwrites its own pair and the finishing kernel reads exactly those: nothing in the
+    // array has to start at zero, whatever an earlier call left there
+    return q6k_gemv_argmax_impl(W, x, nullptr, 0.f, 0, nullptr, logits, K, N, stride, out_index, ws,
                                 ArgmaxAdvance{nullptr, nullptr, nullptr, nullptr, 0}, as_stream(stream));
 }
 
