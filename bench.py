@@ -9,9 +9,10 @@ cache prefilled with 2048 seeded positions), i.e. BASELINE.json configs[3].  Wei
 scratch are resident in HBM before the timed region starts.  One JSON line is printed on stdout.
 
 Besides the token rate the line carries
-  roofline      the dominant kernel (fused RMSNorm + Q4_K gate/up GEMV + SiLU, 2 x 9728 x 2560),
-                algorithmic bytes per launch / average launch duration measured with HIP events on
-                the launching stream, cycling over the 36 layers' distinct weights (1 GB footprint)
+  roofline      the kernel that costs most per token - of the fused RMSNorm + Q4_K gate/up GEMV + SiLU (2 x 9728 x 2560)
+                and the Q6_K down projection (2560 x 9728), both reported under roofline.kernels: algorithmic bytes per
+                launch / average launch duration measured with HIP events on the launching stream, cycling over the
+                36 layers' distinct weights; traffic from the rocprofv3 counter summary under profiles/
   gemv          the same measurement for configs[0] (Q4_K 9728x2560) and configs[1] (Q6_K lm_head)
   cpu_baseline  the reference's CPU path (oracle/_ref build if present, else this repo's C port)
                 timed on this host for a bounded number of tokens of the same workload
@@ -30,10 +31,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the fused gate/up kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
-# script (KiB per dispatch: 13830.1 read, 38.0 written), reads scaled by 1.9998 = what FETCH_SIZE reports for
-# the 256 MiB copy this script also launches (profiles/decode_qwen3_4b_hbm_traffic_pmc.md).
-GATE_UP_TRAFFIC_BYTES = int((13830.1 * 1.9998 + 38.0) * 1024)
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "decode_qwen3_4b_hbm_traffic_pmc.md")
 SEED = 25
 N_PREFILL = 2048
 MAX_SEQ = 2304
@@ -41,6 +39,38 @@ MAX_SEQ = 2304
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def measured_traffic():
+    """HBM bytes per launch of the decode kernels, as the rocprofv3 FETCH_SIZE / WRITE_SIZE summary under profiles/ records
+    them: its lines `TRAFFIC <kernel key> fetch_kib=<..> write_kib=<..>` (KiB per dispatch), `FETCH_SCALE <factor>` (what
+    FETCH_SIZE reads for a copy of known size) and `MEASURED_AT <commit>`.  Returns ({key: bytes}, commit) or ({}, None)."""
+    import re
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return {}, None
+    scale = re.search(r"^FETCH_SCALE\s+([0-9.]+)", text, re.M)
+    commit = re.search(r"^MEASURED_AT\s+(\S+)", text, re.M)
+    out = {}
+    for key, f, w in re.findall(r"^TRAFFIC\s+(\S+)\s+fetch_kib=([0-9.]+)\s+write_kib=([0-9.]+)", text, re.M):
+        out[key] = int((float(f) * float(scale.group(1) if scale else 1.0) + float(w)) * 1024)
+    return out, (commit.group(1) if commit else None)
+
+
+def bench_lib():
+    """libptm_bench.so (bench_kernels.hip): the streaming-read kernel used as the achievable ceiling; not part of the product
+    library."""
+    import ctypes as C
+    path = os.path.join(ROOT, "libptm_bench.so")
+    if not os.path.exists(path):
+        raise ImportError(path + " is not built: python -c 'import __graft_entry__ as g; g.build()'")
+    L = C.CDLL(path)
+    L.bench_stream_read_partials.restype = C.c_int64
+    L.bench_stream_read_partials.argtypes = [C.c_int64]
+    L.bench_stream_read_xor.restype = C.c_int
+    L.bench_stream_read_xor.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
+    return L
 
 
 def event_time_ms(fn, iters, torch):
@@ -91,7 +121,8 @@ def main():
         sys.exit(2)
 
     import torch
-    from prometorch_amd import _lib, ops, synth
+    from prometorch_amd import _lib, ops
+    from prometorch_amd.testing import synth
     from prometorch_amd.decode import Decoder
 
     _lib.load()  # fails loudly when the HIP library is not built
@@ -183,12 +214,7 @@ def main():
         ops.fused_rmsnorm_gate_up_silu(x, Ld.ffn_norm, Ld.gate.data, Ld.up.data, act, H, I, stride4, 1e-6, False)
 
     ms = event_time_ms(run_gate_up, 360, torch)
-    roof = {"bound": "hbm", "kernel": "q4k_gemv_kernel<fused rmsnorm + gate/up + silu> 2x9728x2560",
-            "achieved": gate_up_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": gate_up_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "traffic": GATE_UP_TRAFFIC_BYTES if args.layers == 36 else None,
-            "bytes_per_launch": gate_up_bytes, "us_per_launch": ms * 1e3}
-    log("gate/up fused: %.2f us/launch, %.0f GB/s" % (ms * 1e3, roof["achieved"]))
+    log("gate/up fused: %.2f us/launch, %.0f GB/s" % (ms * 1e3, gate_up_bytes / (ms * 1e-3) / 1e9))
 
     gemv = {}
     # configs[0]: single Q4_K GEMV 9728x2560 (x quantised in the kernel), cold (36 distinct matrices) and warm
@@ -219,11 +245,29 @@ def main():
     del Wbig, ybig
     # down projection Q6_K 2560x9728
     xa = torch.randn(I, device="cuda")
-    yd = torch.empty(H, device="cuda")
+    yd = torch.zeros(H, device="cuda")
     strided = I // 256 * 210
     b2 = H * strided + 4 * I + 4 * H
-    ms2 = event_time_ms(lambda i: ops.launch_q6k_gemv(L0[i % nL].down.data, xa, yd, I, H, strided), 360, torch)
+    ms2 = event_time_ms(lambda i: ops.launch_q6k_gemv(L0[i % nL].down.data, xa, yd, I, H, strided, accumulate=True), 360, torch)
     gemv["q6k_down_2560x9728"] = {"bytes": b2, "us": ms2 * 1e3, "GBs": b2 / ms2 / 1e6, "frac": b2 / ms2 / 1e6 / HBM_PEAK_GBS}
+    # The two GEMV kernels that share the top of the per-token budget (36 launches each): fused RMSNorm + Q4_K gate/up + SiLU
+    # and the Q6_K down projection accumulating into the residual.  `roofline` is the one that costs more per token.
+    traffic, traffic_commit = measured_traffic()
+    kernels = {
+        "gate_up": {"kernel": "q4k_gemv_kernel<fused rmsnorm + gate/up + silu> 2x9728x2560", "bytes_per_launch": gate_up_bytes,
+                    "us_per_launch": ms * 1e3, "launches_per_token": nL},
+        "down": {"kernel": "q6k_gemv_tall_kernel<accumulate> 2560x9728", "bytes_per_launch": b2, "us_per_launch": ms2 * 1e3,
+                 "launches_per_token": nL},
+    }
+    for key, kq in kernels.items():
+        kq["achieved"] = kq["bytes_per_launch"] / kq["us_per_launch"] / 1e3
+        kq["frac"] = kq["achieved"] / HBM_PEAK_GBS
+        kq["traffic"] = traffic.get(key) if args.layers == 36 else None
+    dom = max(kernels, key=lambda k: kernels[k]["us_per_launch"] * kernels[k]["launches_per_token"])
+    roof = {"bound": "hbm", "kernel": kernels[dom]["kernel"], "achieved": kernels[dom]["achieved"], "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": kernels[dom]["frac"], "traffic": kernels[dom]["traffic"],
+            "bytes_per_launch": kernels[dom]["bytes_per_launch"], "us_per_launch": kernels[dom]["us_per_launch"],
+            "traffic_measured_at": traffic_commit, "kernels": kernels}
     # configs[4] (prefill): Llama-3-8B gate projection 14336x4096 (Q4_K), 512 bf16 rows, both GEMM kernels
     Mq, Kq, Nq = 512, 4096, 14336
     Wq = torch.from_numpy(synth.make_q4k(synth.rng_for(SEED, 5), Nq, Kq)).cuda()
@@ -251,15 +295,23 @@ def main():
     # the ceiling that launches of this size can reach on this part, beside the nominal 8 TB/s
     span = 2 * I * stride4
     pool = torch.empty(36 * span, dtype=torch.uint8, device="cuda")
-    parts = torch.empty(ops.stream_read_partials(V * stride6), dtype=torch.int32, device="cuda")
+    BL = bench_lib()
+    parts = torch.empty(BL.bench_stream_read_partials(V * stride6), dtype=torch.int32, device="cuda")
+
+    def stream_read(ptr, nb):
+        rc = BL.bench_stream_read_xor(ptr, nb, parts.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+
     ceil = {}
-    for name, nb in (("14MB_one_q4k_matrix", I * stride4), ("28MB_gate_up", span)):
-        msr = event_time_ms(lambda i: ops.stream_read_xor(pool[(i % 36) * span:], nb, parts), 360, torch)
+    for name, nb in (("14MB_one_q4k_matrix", I * stride4), ("20MB_q6k_down", H * strided), ("28MB_gate_up", span)):
+        msr = event_time_ms(lambda i: stream_read(pool[(i % 36) * span:].data_ptr(), nb), 360, torch)
         ceil[name] = {"bytes": nb, "us": msr * 1e3, "GBs": nb / msr / 1e6}
-    msr = event_time_ms(lambda i: ops.stream_read_xor(lm, V * stride6, parts), 40, torch)
+    msr = event_time_ms(lambda i: stream_read(lm, V * stride6), 40, torch)
     ceil["319MB_lm_head"] = {"bytes": V * stride6, "us": msr * 1e3, "GBs": V * stride6 / msr / 1e6}
     gemv["stream_read_ceiling"] = ceil
-    roof["frac_of_stream_read"] = roof["achieved"] / ceil["28MB_gate_up"]["GBs"]
+    kernels["gate_up"]["frac_of_stream_read"] = kernels["gate_up"]["achieved"] / ceil["28MB_gate_up"]["GBs"]
+    kernels["down"]["frac_of_stream_read"] = kernels["down"]["achieved"] / ceil["20MB_q6k_down"]["GBs"]
+    roof["frac_of_stream_read"] = kernels[dom]["frac_of_stream_read"]
     log("stream-read ceiling: " + ", ".join("%s %.2f us" % (k, v["us"]) for k, v in ceil.items()))
     del pool, parts
     # prompt prefill through all layers: 512 tokens from an empty context (row-batched GEMMs + causal attention)
@@ -382,7 +434,7 @@ def main():
 def cpu_baseline(cfg, layers, head, kvs, n_tokens, gpu_tokens, warmup):
     """Time the reference CPU decode path on this host for n_tokens tokens of the same workload."""
     from oracle import pyoracle as po
-    from prometorch_amd import synth
+    from prometorch_amd.testing import synth
     kind = "port"
     model = None
     if po.have_ref():

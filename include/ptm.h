@@ -315,12 +315,6 @@ int ptm_rope(float* data, int seq_len, int n_heads, int head_dim, int position_o
 int ptm_f32_gemv(const float* W, const float* x, float* y, int K, int N, int k_major, ptm_stream_t stream);
 int ptm_f16_gemv(const void* W_fp16, const float* x, float* y, int K, int N, int k_major, int round_x, ptm_stream_t stream);
 
-/* Measurement aid with no counterpart in the reference: a pure streaming read of `bytes` (a multiple of 16, 16-byte
- * aligned) with 16-byte loads.  out_partials[i], i < ptm_stream_read_partials(bytes), receives the XOR of all 32-bit
- * words of the i-th 32 KiB span.  Its time is the ceiling for a kernel that streams weights of that footprint. */
-int64_t ptm_stream_read_partials(int64_t bytes);
-int ptm_stream_read_xor(const void* src, int64_t bytes, uint32_t* out_partials, ptm_stream_t stream);
-
 /* ---- prefill: quantised-weight GEMM, Y[M,N] = X[M,K] . W[N,K]^T ------------------ */
 /* The reference has no quantised GEMM: matmul_q loops M single-row GEMVs
  * (gguf_model.h:7029-7036, :7056-7061).  These read each weight tile once per 64 rows of X and

@@ -263,6 +263,46 @@ int64_t ref_chat_template(const char* architecture, const char* model_name, cons
     memcpy(out, s.data(), (size_t)std::min<int64_t>(cap, (int64_t)s.size()));
     return (int64_t)s.size();
 }
+// ---------------------------------------------------------------------------------
+// The reference's own loader: GGUFModel::load (torch/io/gguf_model.h:2038-2089: ModelConfig::parse :122-263, tokenizer,
+// load_weights :6770-6886, load_quantized_mmap :1747-1975) on a .gguf file, then forward_decode_cpu on what it loaded.
+// The handle is stepped with ref_model_decode and released with ref_model_free_loaded (the weights belong to the
+// reference's mapping here, not to the caller).
+// ---------------------------------------------------------------------------------
+void* ref_model_load_gguf(const char* gguf_path, int64_t max_seq) {
+    auto* r = new RefModel();
+    try {
+        r->m.load(gguf_path);
+    } catch (...) {
+        delete r;
+        return nullptr;
+    }
+    r->m.use_cuda_ = false;
+    r->m.kv_cache.allocate(r->m.config.num_layers, max_seq, r->m.config.num_kv_heads * r->m.config.head_dim, false);
+    return r;
+}
+void ref_model_free_loaded(void* h) { delete static_cast<RefModel*>(h); }
+// What the reference's parser made of the file's metadata and tensors.  ints[16]: vocab, hidden, layers, heads, kv heads,
+// head_dim, intermediate, tie_word_embeddings, has_qk_norm, rope_neox, scale_embeddings, ffn_gelu, has_post_norm, swa_window,
+// swa_pattern, use_quant_gemv_; floats[5]: rope_freq_base, rms_norm_eps, rope_scale, rope_swa_freq_base, rope_swa_scale;
+// types[7 * layers + 1]: ggml type of q, k, v, o, gate, up, down per layer as load_quantized_mmap registered them, then of
+// the output matrix (0xffffffff: not registered as a quantised weight)
+void ref_model_describe(void* h, int64_t* ints, float* floats, uint32_t* types) {
+    auto& m = static_cast<RefModel*>(h)->m;
+    const auto& c = m.config;
+    const int64_t iv[16] = {c.vocab_size, c.hidden_size, c.num_layers, c.num_heads, c.num_kv_heads, c.head_dim,
+                            c.intermediate_size, c.tie_word_embeddings, c.has_qk_norm, c.rope_neox, c.scale_embeddings,
+                            c.ffn_gelu, c.has_post_norm, c.swa_window, c.swa_pattern, m.use_quant_gemv_};
+    std::memcpy(ints, iv, sizeof iv);
+    const float fv[5] = {c.rope_freq_base, c.rms_norm_eps, c.rope_scale, c.rope_swa_freq_base, c.rope_swa_scale};
+    std::memcpy(floats, fv, sizeof fv);
+    size_t k = 0;
+    for (auto& L : m.layers)
+        for (auto* w : {&L.q_attn_q, &L.q_attn_k, &L.q_attn_v, &L.q_attn_output, &L.q_ffn_gate, &L.q_ffn_up, &L.q_ffn_down})
+            types[k++] = w->valid ? w->quant_type : 0xffffffffu;
+    types[k] = m.q_output_weight.valid ? m.q_output_weight.quant_type : 0xffffffffu;
+}
+
 // what the reference's reader sees of a file: tensor count, and name / type / dims / first bytes of tensor i
 int64_t ref_gguf_n_tensors(const char* gguf_path) {
     g::GGUFReader reader;

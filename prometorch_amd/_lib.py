@@ -118,8 +118,6 @@ SIGNATURES = {
     "ptm_scale": (i32, [vp, f32, i64, vp]),
     "ptm_prefill_attention_window": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i64, i32, f32, i32, i32, vp]),
     "ptm_copy": (i32, [vp, vp, i64, vp]),
-    "ptm_stream_read_partials": (i64, [i64]),
-    "ptm_stream_read_xor": (i32, [vp, i64, vp, vp]),
     "ptm_qgemm_workspace_bytes": (i64, [i32, i32]),
     "ptm_qgemm_q4k": (i32, [vp, vp, vp, i32, i32, i32, i64, vp, vp]),
     "ptm_qgemm_q6k": (i32, [vp, vp, vp, i32, i32, i32, i64, vp, vp]),

@@ -14,10 +14,7 @@
 
 namespace ptm {
 
-#ifndef PTM_FD_CHUNK
-#define PTM_FD_CHUNK 64
-#endif
-enum { FD_CHUNK = PTM_FD_CHUNK, FD_THREADS = 256 };
+enum { FD_CHUNK = 64, FD_THREADS = 256 };
 
 // e^x through the hardware base-2 exponential (v_exp_f32, 1 ulp): softmax weights need no more, and the libm
 // expf expands to a dozen instructions on a path whose cost is instruction count.  -inf gives 0.
@@ -505,16 +502,8 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     for (int pass = 0; pass < NPASS; ++pass) {
         const int64_t t = t0 + pass * PPB + wave * PPW + pl;
         const int64_t tc = t < past ? t : last_cached;
-#if defined(PTM_EXP) && PTM_EXP == 8
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { kreg[pass][i] = 0.01f * i; vreg[pass][i] = 0.02f * i; }
-#elif defined(PTM_EXP) && PTM_EXP == 9
-        load8<KV16>(a.Kc, ((int64_t)kvh * a.max_seq + tc) * HD + dl * 8, kreg[pass]);
-        load8<KV16>(a.Vc, ((int64_t)kvh * a.max_seq + tc) * HD + dl * 8, vreg[pass]);
-#else
         load8<KV16>(a.Kc, tc * kv_dim + col, kreg[pass]);
         load8<KV16>(a.Vc, tc * kv_dim + col, vreg[pass]);
-#endif
     }
     issue_order_fence();
 
@@ -654,11 +643,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
         const float m0 = s_m[0][g], m1 = s_m[1][g], m2 = s_m[2][g], m3 = s_m[3][g];
         const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));  // finite: the chunk holds at least one valid position
         const float w0 = fast_exp(m0 - M), w1 = fast_exp(m1 - M), w2 = fast_exp(m2 - M), w3 = fast_exp(m3 - M);
-#if defined(PTM_EXP) && PTM_EXP == 7
-        const float o = ((w0 * s_o[0][g][d] + w1 * s_o[1][g][d]) + w2 * s_o[2][g][d]) + w3 * s_o[3][g][d];
-#else
         const float o = (w0 * s_o[0][g][d] + w1 * s_o[1][g][d]) + (w2 * s_o[2][g][d] + w3 * s_o[3][g][d]);
-#endif
         const int64_t oi = (int64_t)split * a.n_heads + kvh * G + g;
         a.pO[oi * HD + d] = o;
         if (d == 0) {

@@ -347,34 +347,6 @@ __global__ __launch_bounds__(256) void copy_kernel(const float* __restrict__ a, 
     if (i < n) o[i] = a[i];
 }
 
-// Streaming read of `n16` 16-byte words: the ceiling a weight-streaming kernel of the same footprint is measured
-// against.  Eight independent 16-byte loads per lane, consecutive lanes on consecutive words; the XOR of a
-// workgroup's words is its one output, so the loads cannot be dropped and the result can be checked.
-#ifndef PTM_STREAM_WPL
-#define PTM_STREAM_WPL 8
-#endif
-enum { STREAM_READ_WORDS_PER_LANE = PTM_STREAM_WPL, STREAM_READ_WORDS_PER_WG = 256 * STREAM_READ_WORDS_PER_LANE };
-__global__ __launch_bounds__(256) void stream_read_xor_kernel(const uint4* __restrict__ p, int64_t n16,
-                                                              uint32_t* __restrict__ out) {
-    __shared__ uint32_t part[4];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t base = (int64_t)blockIdx.x * STREAM_READ_WORDS_PER_WG + wave * (64 * STREAM_READ_WORDS_PER_LANE) + lane;
-    uint4 v[STREAM_READ_WORDS_PER_LANE];
-#pragma unroll
-    for (int i = 0; i < STREAM_READ_WORDS_PER_LANE; ++i) {
-        const int64_t idx = base + i * 64;
-        v[i] = idx < n16 ? p[idx] : make_uint4(0, 0, 0, 0);
-    }
-    uint32_t s = 0;
-#pragma unroll
-    for (int i = 0; i < STREAM_READ_WORDS_PER_LANE; ++i) s ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s ^= __shfl_xor(s, o);
-    if (lane == 0) part[wave] = s;
-    __syncthreads();
-    if (threadIdx.x == 0) out[blockIdx.x] = part[0] ^ part[1] ^ part[2] ^ part[3];
-}
-
 __global__ __launch_bounds__(256) void embedding_row_kernel(const float* __restrict__ table, float* __restrict__ out,
                                                             const int* __restrict__ d_tok, int hidden) {
     const int i = blockIdx.x * 256 + threadIdx.x;
@@ -665,20 +637,6 @@ int ptm_copy(const float* in, float* out, int64_t n, ptm_stream_t stream) {
     if (n < 0) return PTM_E_SHAPE;
     if (n == 0) return PTM_OK;
     hipLaunchKernelGGL(copy_kernel, dim3(nblk256(n)), dim3(256), 0, as_stream(stream), in, out, n);
-    return launch_status();
-}
-
-int64_t ptm_stream_read_partials(int64_t bytes) {
-    return bytes <= 0 ? 0 : (bytes / 16 + STREAM_READ_WORDS_PER_WG - 1) / STREAM_READ_WORDS_PER_WG;
-}
-
-int ptm_stream_read_xor(const void* src, int64_t bytes, uint32_t* out_partials, ptm_stream_t stream) {
-    if (!src || !out_partials) return PTM_E_NULL;
-    if (bytes <= 0 || bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(src) & 15) != 0) return PTM_E_SHAPE;
-    const int64_t wgs = ptm_stream_read_partials(bytes);
-    if (wgs > 0x7fffffff) return PTM_E_RANGE;
-    hipLaunchKernelGGL(stream_read_xor_kernel, dim3((unsigned)wgs), dim3(256), 0, as_stream(stream),
-                       static_cast<const uint4*>(src), bytes / 16, out_partials);
     return launch_status();
 }
 

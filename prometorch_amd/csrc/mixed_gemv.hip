@@ -57,9 +57,6 @@ int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const in
     // per CU, the Q6_K rows (fewer, and more arithmetic per byte) one step finer than the Q4_K ones.  Qwen3-4B and
     // Llama-3-8B shapes both land on 2 and 4 groups per row (448 workgroups): 617 -> 633 tok/s and 518 -> 523 tok/s
     // against the per-kernel rules of the single-type GEMVs (4 and 8 groups, 896 workgroups).
-    // PTM_MIXED_L4 / PTM_MIXED_L6 (0..3) override, for tuning runs.
-    static const int l4_env = [] { const char* e = getenv("PTM_MIXED_L4"); return e ? atoi(e) : -1; }();
-    static const int l6_env = [] { const char* e = getenv("PTM_MIXED_L6"); return e ? atoi(e) : -1; }();
     int l4 = 3, l6 = 3;
     for (int l = 0; l <= 3; ++l) {
         const int t6 = l + 1 < 3 ? l + 1 : 3;
@@ -69,8 +66,6 @@ int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const in
             break;
         }
     }
-    if (l4_env >= 0 && l4_env <= 3) l4 = l4_env;
-    if (l6_env >= 0 && l6_env <= 3) l6 = l6_env;
     a4.log2S = l4;
     Q6KArgs a6{static_cast<const uint8_t*>(W6), x, y6, K, N6, l6, stride6, nullptr, nullptr,
                gamma, eps, add_one, nullptr};

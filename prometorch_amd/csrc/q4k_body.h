@@ -3,8 +3,6 @@
 #pragma once
 #include "ptm_common.h"
 
-#include <cstdlib>
-
 namespace ptm {
 
 struct Q4KArgs {
@@ -162,9 +160,6 @@ __device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KAr
 // contribution of one super-block to lane j's chain (sub-block j of the block)
 __device__ __forceinline__ float q4k_block_term(const uint4 hdr, const uint4 qv, const uint8_t* __restrict__ lds,
                                                 int K, int b, int j) {
-#if defined(PTM_EXP) && (PTM_EXP == 1 || PTM_EXP == 3)
-    return __int_as_float((hdr.x ^ qv.x ^ qv.y ^ qv.z ^ qv.w ^ hdr.y) & 0x3fffffff);
-#endif
     const int8_t* xq = reinterpret_cast<const int8_t*>(lds);
     const float* xd = reinterpret_cast<const float*>(lds + K);
     const float* xs = xd + K / 32;
@@ -297,13 +292,8 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
 
     // ---- activation loads first, then the first tile's weight loads, then the activation prologue ----
     __shared__ float red[4];
-#if defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3)
-    Q4KStage stg;
-    run_tile(wg * tpw, [] {});
-#else
     const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a, lds, red);
     run_tile(wg * tpw, [&] { q4k_stage_finish<XQ8, NORM>(stg, a, lds, red); });
-#endif
     // further tiles reuse the staged activations: the quantisation of x is paid once per workgroup
     for (int k = 1; k < tpw; ++k) {
         const int tile = wg * tpw + k;
@@ -313,14 +303,7 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
 }
 
 // lane groups per row: enough workgroups to cover the chip, and all of a group's blocks in one pass
-// PTM_Q4K_LOG2S / PTM_Q6K_LOG2S (0..3) override the heuristic, for tuning runs.
-inline int tuning_env(const char* name) {
-    const char* e = getenv(name);
-    return (e && e[0] >= '0' && e[0] <= '3' && e[1] == 0) ? e[0] - '0' : -1;
-}
 inline int q4k_pick_log2S(int total_rows, int nblk, int max_log2S) {
-    static const int forced = tuning_env("PTM_Q4K_LOG2S");
-    if (forced >= 0) return forced < max_log2S ? forced : max_log2S;
     int l = 0;
     while (l < max_log2S) {
         const int S = 1 << l;
@@ -337,14 +320,9 @@ inline int q4k_workgroups(int total_rows, int log2S) {
     return (total_rows + rows_per_wg - 1) / rows_per_wg;
 }
 // Row tiles per workgroup: beyond ~1200 tiles a workgroup walks several, so that the activation prologue (every
-// workgroup quantises the whole vector) is amortised.  PTM_Q4K_TPW (1..9) overrides, for tuning runs.
+// workgroup quantises the whole vector) is amortised.
 inline int q4k_tiles_per_wg(int n_tiles) {
-    static const int forced = [] {
-        const char* e = getenv("PTM_Q4K_TPW");
-        return (e && e[0] >= '1' && e[0] <= '9' && e[1] == 0) ? e[0] - '0' : 0;
-    }();
-    if (forced > 0) return forced;
-    static const int max_wgs = [] { const char* e = getenv("PTM_Q4K_MAXWG"); return e ? atoi(e) : 1280; }();
+    const int max_wgs = 1280;
     int t = 1;
     while (t < 8 && (n_tiles + t - 1) / t > max_wgs) ++t;
     return t;

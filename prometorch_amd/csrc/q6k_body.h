@@ -3,8 +3,6 @@
 #pragma once
 #include "ptm_common.h"
 
-#include <cstdlib>
-
 namespace ptm {
 
 struct Q6KArgs {
@@ -68,9 +66,6 @@ __device__ __forceinline__ void realign16(const uint4 w, uint32_t tail, uint32_t
 // contribution of block b to lane j's chain
 __device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __restrict__ xf,
                                                 const float* __restrict__ xsum16, int b, int j) {
-#if defined(PTM_EXP) && (PTM_EXP == 1 || PTM_EXP == 3)
-    return __uint_as_float((k.ql.x ^ k.ql.y ^ k.ql.z ^ k.ql.w ^ k.qh.x ^ k.qh.y ^ k.qh.z ^ k.qh.w ^ k.sc_lo ^ k.sc_hi ^ k.d ^ k.ql_t ^ k.qh_t) & 0x3fffffffu);
-#endif
     const int half = j >> 2, jj = j & 3, which32 = jj >> 1, l16 = jj & 1;
     const int hshift = 2 * which32;
     const int xo = 128 * half + 32 * which32 + 16 * l16;  // x offset of the low-nibble 16; high-nibble +64
@@ -133,19 +128,13 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
         if ((tid & 3) == 0) xsum16[i >> 2] = sm;
     };
     // activation loads first (loads complete in issue order), then the first pass of weight loads
-#if defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3 || PTM_EXP == 4 || PTM_EXP == 5)
-    XStage<XCH> stg;
-#else
     const XStage<XCH> stg = stage_issue<NORM, XCH>(a.x, a.gamma, a.K, a.eps, a.add_one, red, emit);
-#endif
     Q6Blk blk[NB];
     issue_order_fence();
 #pragma unroll
     for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off, sc_off);
     issue_order_fence();
-#if !(defined(PTM_EXP) && (PTM_EXP == 2 || PTM_EXP == 3 || PTM_EXP == 4 || PTM_EXP == 5))
     stage_finish<NORM, XCH>(stg, a.K, a.eps, a.add_one, red, emit);
-#endif
     __syncthreads();
 
     // Passes roll: as soon as a block of pass p has been consumed its registers are refilled with the same slot of
@@ -200,20 +189,13 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
 // Lane groups per row: the fewest that still give the chip enough workgroups, with a group's blocks in at most two
 // rolling passes (the vocabulary projection 151936 x 2560 then runs one group per row, two passes of 5 blocks:
 // 94 -> 88 us with the argmax against two groups per row and one pass, for half the stagings of x).
-// PTM_Q6K_LOG2S (0..3) forces the split and PTM_Q6K_TWO_PASS=0 restores the one-pass rule, for tuning runs.
 inline int q6k_pick_log2S(int rows, int nblk) {
-    static const int forced = [] {
-        const char* e = getenv("PTM_Q6K_LOG2S");
-        return (e && e[0] >= '0' && e[0] <= '3' && e[1] == 0) ? e[0] - '0' : -1;
-    }();
-    if (forced >= 0) return forced;
     int l = 0;
     while (l < 3) {
         const int S = 1 << l;
         const int wgs = (rows * S + 31) / 32;
         const int nb = (nblk + S - 1) / S;
-        static const int passes = [] { const char* e = getenv("PTM_Q6K_TWO_PASS"); return (e && e[0] == '0') ? 1 : 2; }();
-        if (nb <= passes * Q6K_U && wgs >= 600) break;
+        if (nb <= 2 * Q6K_U && wgs >= 600) break;
         if (nb <= 1) break;
         ++l;
     }

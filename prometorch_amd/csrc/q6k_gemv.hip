@@ -108,11 +108,10 @@ __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(
 // Shape of a tall launch: waves per workgroup and lane groups per row, or waves = 0 when the shape is not one for
 // it.  Rows that fill the chip once at one workgroup per CU: 8 lane groups per row while that needs at most 12 waves
 // (2560 x 9728: 10 waves, 10.25 -> 9.75 us against 4-row tiles), else 4 groups per row and two rows per wave
-// (4096 x 14336: 8 waves of 2 rows).  PTM_Q6K_TALL=0 switches it off, for tuning runs.
+// (4096 x 14336: 8 waves of 2 rows).
 struct Q6KTall { int waves, log2S; };
 inline Q6KTall q6k_tall_shape(int N, int K) {
-    static const bool off = [] { const char* e = getenv("PTM_Q6K_TALL"); return e && e[0] == '0'; }();
-    if (off || K < 4096 || K > 14336) return {0, 0};
+    if (K < 4096 || K > 14336) return {0, 0};
     if (q6k_pick_log2S(N, K / 256) != 3) return {0, 0};   // only where the row tiles would be 4 rows anyway
     const int rows_per_wg = (N + 255) / 256;
     for (int l = 3; l >= 2; --l) {

@@ -620,27 +620,18 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) v
                     for (int mt = 0; mt < MT; ++mt)
                         an[ks][mt] = *reinterpret_cast<const h8*>(a_cur + (mt * 32 + j) * QF_PITCH + 64 * (s + 1) + 32 * kh + 16 * ks);
             }
-#if defined(PTM_EXP) && PTM_EXP == 11
-#pragma unroll
-            for (int t = 0; t < NT; ++t) { bn[t][0] = bf[t][1]; bn[t][1] = bf[t][0]; }
-#else
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 if (s < 7) cur[t].frags(s + 1, kh, bn[t][0], bn[t][1]);
                 else nxt[t].frags(0, kh, bn[t][0], bn[t][1]);
             }
-#endif
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                     for (int t = 0; t < NT; ++t)
-#if defined(PTM_EXP) && PTM_EXP == 12
-                        acc[mt][t][0] += (float)af[ks][mt][0] * (float)bf[t][ks][0];
-#else
                         acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks][mt], bf[t][ks], acc[mt][t], 0, 0, 0);
-#endif
             // issue order: one MFMA, then the vector work that fits under it (a 32x32x16 MFMA occupies the matrix pipe
             // for 32 cycles = 8 vector instructions), so that neither pipe waits for the other
 #pragma unroll
@@ -777,8 +768,7 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     }
     // rows per workgroup: 64 (two workgroups share a CU, so one's memory waits hide behind the other's arithmetic) or
     // 128 (half the dequantisation work per product)
-    static const int mt_env = [] { const char* e = getenv("PTM_QGEMM_MT"); return e ? atoi(e) : 0; }();
-    const int MT = (mt_env == 2 || mt_env == 4) ? mt_env : qgemm_f16_row_tiles(q4, M, N, splits);
+    const int MT = qgemm_f16_row_tiles(q4, M, N, splits);
     const int tm = 32 * MT;
     const size_t lds = 2 * (size_t)tm * QF_PITCH;  // 132 KB / 66 KB: above the default 64 KB cap of dynamic LDS
     static bool raised = false;
@@ -794,10 +784,9 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     }
     const dim3 grid((N + QF_TN - 1) / QF_TN, (M + tm - 1) / tm, splits);
     const uint8_t* Wb = static_cast<const uint8_t*>(W);
-    // 128-row tiles run with eight waves (PTM_QGEMM_WAVES=4 restores four, for tuning runs): 512 x 4096 x 14336
-    // 104 -> 92-94 us (Q4_K), 321 -> 308 us for 512 x 14336 x 4096 (Q6_K)
-    static const int waves_env = [] { const char* e = getenv("PTM_QGEMM_WAVES"); return e ? atoi(e) : 0; }();
-    const bool eight = MT == 4 && waves_env != 4;
+    // 128-row tiles run with eight waves: 512 x 4096 x 14336 104 -> 92-94 us (Q4_K) against four waves,
+    // 321 -> 308 us for 512 x 14336 x 4096 (Q6_K)
+    const bool eight = MT == 4;
     if (eight && q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (eight) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (q4 && MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);

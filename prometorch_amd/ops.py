@@ -328,15 +328,6 @@ def launch_copy(input, output, n, stream=None):
     check(_L().ptm_copy(_ptr(input), _ptr(output), n, _stream(stream)), "copy")
 
 
-def stream_read_partials(nbytes):
-    return int(_L().ptm_stream_read_partials(nbytes))
-
-
-def stream_read_xor(src, nbytes, out_partials, stream=None):
-    """Pure streaming read of nbytes from src (measurement ceiling); out_partials: uint32/int32[stream_read_partials]."""
-    check(_L().ptm_stream_read_xor(_ptr(src), nbytes, _ptr(out_partials), _stream(stream)), "stream_read_xor")
-
-
 # ---- prefill GEMM ---------------------------------------------------------------------
 def qgemm_workspace_bytes(M, K):
     return _L().ptm_qgemm_workspace_bytes(M, K)

@@ -22,7 +22,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 sys.path.insert(0, ROOT)
 from oracle import pyoracle as po  # noqa: E402
-from prometorch_amd import synth  # noqa: E402
+from prometorch_amd.testing import synth  # noqa: E402
 
 OUT = os.path.dirname(os.path.abspath(__file__))
 SEEDS = {"blocks": 101, "cfg1": 1001, "cfg2": 1002, "cfg3": 1003, "tiny": 7, "cfg4": 25, "ragged": 1005}
@@ -290,6 +290,7 @@ def make_tokenizer_golden():
     import tempfile
     import ctypes as C
     from prometorch_amd import gguf
+    from prometorch_amd.testing import gguf_writer
     R = po.ref()
     b64 = lambda b: base64.b64encode(b).decode()
     out = {"tokenizers": {}, "chat": []}
@@ -306,7 +307,7 @@ def make_tokenizer_golden():
         md["general.architecture"] = "qwen3"
         with tempfile.TemporaryDirectory() as d:
             path = os.path.join(d, "tok.gguf")
-            gguf.write_gguf(path, md, [("dummy", 0, [4], np.zeros(4, np.float32))])
+            gguf_writer.write_gguf(path, md, [("dummy", 0, [4], np.zeros(4, np.float32))])
             assert R.ref_gguf_n_tensors(path.encode()) == 1
             h = R.ref_tokenizer_load(path.encode())
         cases = []

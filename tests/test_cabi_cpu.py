@@ -114,7 +114,7 @@ def test_rope_table_host_matches_oracle(po):
 
 
 def test_synth_generators_are_deterministic_and_in_range():
-    from prometorch_amd import synth
+    from prometorch_amd.testing import synth
     a = synth.make_q4k(synth.rng_for(3), 4, 512)
     b = synth.make_q4k(synth.rng_for(3), 4, 512)
     assert np.array_equal(a, b) and a.shape == (4, 288)

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from conftest import GOLDEN_DIR, bits
-from prometorch_amd import synth
+from prometorch_amd.testing import synth
 
 CASES = [(13, 24, 512), (13, 3, 2560), (8, 24, 512), (8, 5, 96), (6, 24, 512), (6, 7, 32)]
 

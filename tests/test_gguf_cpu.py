@@ -6,7 +6,8 @@ import struct
 import numpy as np
 import pytest
 
-from prometorch_amd import gguf, synth
+from prometorch_amd import gguf
+from prometorch_amd.testing import gguf_writer, synth
 from prometorch_amd._lib import PtmError
 
 
@@ -25,7 +26,7 @@ def test_roundtrip_tensor_table_and_bytes(tmp_path, alignment):
     f32 = r.standard_normal(7, dtype=np.float32)
     f16 = r.standard_normal((3, 8), dtype=np.float32).astype(np.float16)
     path = str(tmp_path / "t.gguf")
-    gguf.write_gguf(path, {"general.architecture": "qwen3", "qwen3.block_count": 2, "qwen3.rope.freq_base": 1e6,
+    gguf_writer.write_gguf(path, {"general.architecture": "qwen3", "qwen3.block_count": 2, "qwen3.rope.freq_base": 1e6,
                            "some.flag": True, "some.big": 2 ** 40, "some.list": [1, 2, 3], "some.names": ["x", "yy"]},
                     [("a.weight", gguf.Q4_K, [512, 6], q4), ("b.weight", gguf.Q6_K, [256, 5], q6),
                      ("c", gguf.F32, [7], f32), ("d", gguf.F16, [8, 3], f16), ("e", 2, [32], b"\0" * 18)],
@@ -60,7 +61,7 @@ def test_roundtrip_tensor_table_and_bytes(tmp_path, alignment):
 def test_model_file_has_the_reference_tensor_names(tmp_path):
     cfg, layers, head = tiny_model()
     path = str(tmp_path / "m.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head)
+    gguf_writer.model_to_gguf(path, cfg, layers, head)
     with gguf.GGUFFile(path) as g:
         assert g.get_int("qwen3.embedding_length") == cfg["hidden"]
         for name in ("token_embd.weight", "output_norm.weight", "blk.0.attn_q.weight", "blk.1.ffn_down.weight",
@@ -73,10 +74,10 @@ def test_model_file_has_the_reference_tensor_names(tmp_path):
 
 def test_qwen2_model_file_carries_the_bias_vectors(tmp_path):
     """blk.N.attn_{q,k,v}.bias as F32 vectors, the names the reference looks up (gguf_model.h:6750-6753)."""
-    from prometorch_amd import synth
+    from prometorch_amd.testing import synth
     cfg, layers, head = synth.tiny_qwen2(5)
     path = str(tmp_path / "q2.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, arch="qwen2")
+    gguf_writer.model_to_gguf(path, cfg, layers, head, arch="qwen2")
     with gguf.GGUFFile(path) as g:
         assert g.get_string("general.architecture") == "qwen2"
         assert g.get_int("qwen2.attention.head_count_kv") == cfg["n_kv_heads"]
@@ -92,7 +93,7 @@ def test_qwen2_model_file_carries_the_bias_vectors(tmp_path):
 
 def test_malformed_files_are_refused(tmp_path):
     good = str(tmp_path / "g.gguf")
-    gguf.write_gguf(good, {"general.architecture": "qwen3"}, [("c", gguf.F32, [8], np.zeros(8, np.float32))])
+    gguf_writer.write_gguf(good, {"general.architecture": "qwen3"}, [("c", gguf.F32, [8], np.zeros(8, np.float32))])
     raw = open(good, "rb").read()
 
     def code_of(data):
@@ -113,6 +114,6 @@ def test_malformed_files_are_refused(tmp_path):
     assert e.value.code == -8
     # version 2 is accepted
     v2 = str(tmp_path / "v2.gguf")
-    gguf.write_gguf(v2, {"general.architecture": "qwen3"}, [("c", gguf.F32, [8], np.zeros(8, np.float32))], version=2)
+    gguf_writer.write_gguf(v2, {"general.architecture": "qwen3"}, [("c", gguf.F32, [8], np.zeros(8, np.float32))], version=2)
     with gguf.GGUFFile(v2) as g:
         assert g.version == 2

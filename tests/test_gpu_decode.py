@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 from conftest import bits
-from prometorch_amd import synth
+from prometorch_amd.testing import synth
 
 pytestmark = pytest.mark.gpu
 

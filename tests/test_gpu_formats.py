@@ -8,7 +8,8 @@ import pytest
 import torch
 
 from conftest import GOLDEN_DIR, bits
-from prometorch_amd import ops, synth
+from prometorch_amd import ops
+from prometorch_amd.testing import synth
 from prometorch_amd._lib import PtmError
 from test_gpu_parity import GEMV_TOL, cu, gpu_gemv, rel_err
 

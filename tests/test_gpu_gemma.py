@@ -10,7 +10,8 @@ import pytest
 import torch
 
 from conftest import bits
-from prometorch_amd import gguf, ops, synth
+from prometorch_amd import gguf, ops
+from prometorch_amd.testing import gguf_writer, synth
 from test_gpu_decode import check_step_errors
 from test_gpu_llama import follow_sensitive
 from test_gpu_prefill import check_kv_rows, check_logits
@@ -306,7 +307,7 @@ def test_gemma3_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_gemma, 
     from prometorch_amd.decode import Decoder
     cfg, layers, head, kv = tiny_gemma_with_cache(seeds)
     path = str(tmp_path / "tiny_gemma3.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, arch="gemma3")
+    gguf_writer.model_to_gguf(path, cfg, layers, head, arch="gemma3")
     m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
     for key in ("scale_embeddings", "ffn_gelu", "swa_window", "swa_pattern", "rope_swa_base", "rope_scale"):
         assert m.cfg[key] == cfg[key], key
@@ -327,7 +328,7 @@ def test_gemma3_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_gemma, 
     d.close()
     # without the pattern key every sixth layer is global: the four-layer model is all local then
     p2 = str(tmp_path / "default_pattern.gguf")
-    gguf.model_to_gguf(p2, dict(cfg, swa_pattern=6), layers, head, arch="gemma3")
+    gguf_writer.model_to_gguf(p2, dict(cfg, swa_pattern=6), layers, head, arch="gemma3")
     m2 = gguf.GGUFModel(p2, max_seq=64, kv_fp16=False)
     assert m2.cfg["swa_pattern"] == 6
     m2.close()

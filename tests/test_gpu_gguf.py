@@ -4,7 +4,8 @@ import numpy as np
 import pytest
 
 from conftest import bits
-from prometorch_amd import gguf, synth
+from prometorch_amd import gguf
+from prometorch_amd.testing import gguf_writer, synth
 from prometorch_amd._lib import PtmError
 
 pytestmark = pytest.mark.gpu
@@ -23,7 +24,7 @@ def test_gguf_model_decodes_like_direct_decoder(dev, seeds, golden, tmp_path, ti
     from prometorch_amd.decode import Decoder
     cfg, layers, head, kv = build_tiny(seeds)
     path = str(tmp_path / "tiny.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, tied=tied, alignment=64)
+    gguf_writer.model_to_gguf(path, cfg, layers, head, tied=tied, alignment=64)
     m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
     for k in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter"):
         assert m.cfg[k] == cfg[k], k
@@ -52,7 +53,7 @@ def test_gguf_model_decodes_like_direct_decoder(dev, seeds, golden, tmp_path, ti
 def test_gguf_model_refuses_what_it_cannot_run(dev, seeds, tmp_path):
     cfg, layers, head, _ = build_tiny(seeds)
     p = str(tmp_path / "phi3.gguf")
-    gguf.model_to_gguf(p, cfg, layers, head, arch="phi3")  # fused qkv / gate-up tensors, per-frequency factors: not a step built here
+    gguf_writer.model_to_gguf(p, cfg, layers, head, arch="phi3")  # fused qkv / gate-up tensors, per-frequency factors: not a step built here
     with pytest.raises(PtmError) as e:
         gguf.GGUFModel(p, max_seq=64)
     assert e.value.code == -4
@@ -61,7 +62,7 @@ def test_gguf_model_refuses_what_it_cannot_run(dev, seeds, tmp_path):
     qt, W = bad[1]["down"]
     bad[1]["down"] = (qt, W[:-1])
     p2 = str(tmp_path / "short.gguf")
-    gguf.model_to_gguf(p2, cfg, bad, head)
+    gguf_writer.model_to_gguf(p2, cfg, bad, head)
     with pytest.raises(PtmError) as e:
         gguf.GGUFModel(p2, max_seq=64)
     assert e.value.code == -2
@@ -69,7 +70,7 @@ def test_gguf_model_refuses_what_it_cannot_run(dev, seeds, tmp_path):
     p3 = str(tmp_path / "missing.gguf")
     cfg3 = dict(cfg)
     cfg3["n_layers"] = 3
-    gguf.model_to_gguf(p3, cfg3, layers, head)
+    gguf_writer.model_to_gguf(p3, cfg3, layers, head)
     with pytest.raises(PtmError) as e:
         gguf.GGUFModel(p3, max_seq=64)
     assert e.value.code == -10
@@ -85,7 +86,7 @@ def test_text_to_text_through_one_file(dev, po, seeds, tmp_path):
     tok_md = synth.make_tokenizer("gpt2", vocab_size=cfg["vocab"])
     assert len(tok_md["tokenizer.ggml.tokens"]) == cfg["vocab"]
     path = str(tmp_path / "chat.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, tokenizer=tok_md)
+    gguf_writer.model_to_gguf(path, cfg, layers, head, tokenizer=tok_md)
     f = gguf.GGUFFile(path)
     tk = Tokenizer.from_gguf(f)
     m = gguf.GGUFModel(path, max_seq=160, kv_fp16=True)
@@ -124,7 +125,7 @@ def test_chat_is_the_manual_path_in_one_call(dev, seeds, tmp_path):
     cfg, layers, head, _ = build_tiny(seeds)
     tok_md = synth.make_tokenizer("gpt2", vocab_size=cfg["vocab"])
     path = str(tmp_path / "chat.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, tokenizer=tok_md)
+    gguf_writer.model_to_gguf(path, cfg, layers, head, tokenizer=tok_md)
     m = gguf.GGUFModel(path, max_seq=160, kv_fp16=True)
     reply = m.chat("Hello there, what's 2+2?", system="Be brief.", max_new=24, temperature=0.8, top_k=40, top_p=0.9,
                    repeat_penalty=1.1, seed=42)

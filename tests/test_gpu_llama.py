@@ -11,7 +11,8 @@ import pytest
 import torch
 
 from conftest import bits
-from prometorch_amd import gguf, ops, synth
+from prometorch_amd import gguf, ops
+from prometorch_amd.testing import gguf_writer, synth
 from test_gpu_decode import check_step_errors
 from test_gpu_prefill import E2E_MAX_TOL, E2E_RMS_TOL, check_kv_rows, check_logits, logit_errors
 
@@ -223,7 +224,7 @@ def test_llama_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_llama, t
     from prometorch_amd.decode import Decoder
     cfg, layers, head, kv = tiny_llama_with_cache(seeds)
     path = str(tmp_path / "tiny_llama.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, arch="llama")
+    gguf_writer.model_to_gguf(path, cfg, layers, head, arch="llama")
     m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
     assert m.cfg["rope_interleaved"] is True
     d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
@@ -242,7 +243,7 @@ def test_llama_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_llama, t
     d.close()
     # the same tensors labelled qwen3 lack its QK-norm vectors: a missing tensor, not a silent llama-style run
     p2 = str(tmp_path / "mislabelled.gguf")
-    gguf.model_to_gguf(p2, cfg, layers, head, arch="qwen3")
+    gguf_writer.model_to_gguf(p2, cfg, layers, head, arch="qwen3")
     from prometorch_amd._lib import PtmError
     with pytest.raises(PtmError) as e:
         gguf.GGUFModel(p2, max_seq=64)
@@ -261,7 +262,7 @@ def test_linear_rope_scaling_vs_reference_golden(dev, po, seeds, golden_llama, t
     cfg, layers, head, kv = tiny_llama_with_cache(seeds)
     cfg = dict(cfg, rope_scale=4.0)
     path = str(tmp_path / "scaled.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, arch="llama")
+    gguf_writer.model_to_gguf(path, cfg, layers, head, arch="llama")
     m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
     assert m.cfg["rope_scale"] == 4.0
     d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
@@ -285,7 +286,7 @@ def test_linear_rope_scaling_vs_reference_golden(dev, po, seeds, golden_llama, t
     # legacy key; a scaling type other than linear leaves the positions alone
     for md, want in (({"llama.rope.scale_linear": 2.0}, 2.0), ({"llama.rope.scaling.type": "yarn", "llama.rope.scaling.factor": 8.0}, 1.0)):
         p2 = str(tmp_path / f"k{want}.gguf")
-        gguf.model_to_gguf(p2, dict(cfg, rope_scale=1.0), layers, head, arch="llama", extra_metadata=md)
+        gguf_writer.model_to_gguf(p2, dict(cfg, rope_scale=1.0), layers, head, arch="llama", extra_metadata=md)
         m2 = gguf.GGUFModel(p2, max_seq=64, kv_fp16=False)
         assert m2.cfg["rope_scale"] == want
         m2.close()

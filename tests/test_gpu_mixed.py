@@ -8,7 +8,8 @@ import numpy as np
 import pytest
 
 from conftest import GOLDEN_DIR, bits
-from prometorch_amd import gguf, synth
+from prometorch_amd import gguf
+from prometorch_amd.testing import gguf_writer, synth
 from test_gpu_decode import LOGIT_TOL, LOGIT_TOL_FLIP, check_step_errors
 from test_gpu_prefill import check_kv_rows, check_logits, follow
 
@@ -96,7 +97,7 @@ def test_mixed_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_mixed, t
     from prometorch_amd.decode import Decoder
     cfg, layers, head, kv = mixed_with_cache(seeds)
     path = str(tmp_path / "tiny_mixed.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head)
+    gguf_writer.model_to_gguf(path, cfg, layers, head)
     m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
     d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
     for i, (k, v) in enumerate(kv):
@@ -167,7 +168,7 @@ def test_other_formats_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_
     from prometorch_amd.decode import Decoder
     cfg, layers, head = synth.tiny_formats(seeds["tiny"])
     path = str(tmp_path / "tiny_formats.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head)
+    gguf_writer.model_to_gguf(path, cfg, layers, head)
     m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
     d = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False)
     for i in range(cfg["n_layers"]):
@@ -195,7 +196,7 @@ def test_other_lm_head_types_from_gguf_vs_oracle(dev, po, seeds, tmp_path, lm_ty
     emb = po.dequant(lm_type, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
     om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False, embedding=emb)
     path = str(tmp_path / "lm.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, tied=tied)
+    gguf_writer.model_to_gguf(path, cfg, layers, head, tied=tied)
     m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
     errs, tok_o = [], 5
     tok_g = 5

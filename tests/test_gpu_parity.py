@@ -9,7 +9,8 @@ import pytest
 import torch
 
 from conftest import bits, sha, sha_of
-from prometorch_amd import ops, synth
+from prometorch_amd import ops
+from prometorch_amd.testing import synth
 
 pytestmark = pytest.mark.gpu
 
@@ -519,24 +520,6 @@ def test_attn_decode_fused_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past):
         assert np.abs(krow - kf[pos]).max() <= (2e-3 if kv_fp16 else 2e-6) * np.abs(kf[pos]).max()
         assert np.array_equal(Vc[pos].float().cpu().numpy(), vf[pos])
         kf[pos] = krow                                               # continue from what the cache really holds
-
-
-@pytest.mark.parametrize("nbytes", [16, 32768, 32768 + 16, (1 << 20) + 48, 14008320])
-def test_stream_read_xor_matches_numpy(dev, nbytes):
-    """The measurement ceiling kernel reads every byte: per-32 KiB XORs equal numpy's."""
-    from prometorch_amd._lib import PtmError
-    data = synth.rng_for(48, nbytes).integers(0, 256, nbytes, dtype=np.uint8)
-    n = ops.stream_read_partials(nbytes)
-    assert n == (nbytes + 32767) // 32768
-    out = torch.full((n,), -1, dtype=torch.int32, device="cuda")
-    ops.stream_read_xor(cu(data), nbytes, out)
-    torch.cuda.synchronize()
-    words = np.zeros(n * 8192, np.uint32)
-    words[:nbytes // 4] = data.view(np.uint32)
-    want = np.bitwise_xor.reduce(words.reshape(n, 8192), axis=1)
-    assert np.array_equal(out.cpu().numpy().view(np.uint32), want)
-    with pytest.raises(PtmError):
-        ops.stream_read_xor(cu(data), nbytes + 8, out)
 
 
 @pytest.mark.parametrize("N,K,accumulate", [(2500, 9728, True), (300, 4096, False), (77, 14336, True), (3000, 6912, False),

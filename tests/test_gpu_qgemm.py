@@ -9,7 +9,8 @@ import pytest
 import torch
 
 from conftest import bits
-from prometorch_amd import ops, synth
+from prometorch_amd import ops
+from prometorch_amd.testing import synth
 from prometorch_amd._lib import PtmError
 
 pytestmark = pytest.mark.gpu

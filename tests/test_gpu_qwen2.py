@@ -10,7 +10,8 @@ import pytest
 import torch
 
 from conftest import bits
-from prometorch_amd import gguf, ops, synth
+from prometorch_amd import gguf, ops
+from prometorch_amd.testing import gguf_writer, synth
 from test_gpu_decode import check_step_errors
 from test_gpu_llama import follow_sensitive
 from test_gpu_prefill import check_kv_rows, check_logits
@@ -148,7 +149,7 @@ def test_qwen2_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_qwen2, t
     from prometorch_amd.decode import Decoder
     cfg, layers, head, kv = tiny_qwen2_with_cache(seeds)
     path = str(tmp_path / "tiny_qwen2.gguf")
-    gguf.model_to_gguf(path, cfg, layers, head, arch="qwen2")
+    gguf_writer.model_to_gguf(path, cfg, layers, head, arch="qwen2")
     f = gguf.GGUFFile(path)
     assert np.array_equal(f.tensor("blk.1.attn_k.bias")["data"].view(np.float32), layers[1]["k_bias"])
     f.close()
@@ -174,7 +175,7 @@ def test_qwen2_gguf_file_decodes_like_direct_decoder(dev, seeds, golden_qwen2, t
     for L in part:
         L["v_bias"] = None
     p2 = str(tmp_path / "partial.gguf")
-    gguf.model_to_gguf(p2, cfg, part, head, arch="qwen2")
+    gguf_writer.model_to_gguf(p2, cfg, part, head, arch="qwen2")
     from prometorch_amd._lib import PtmError
     with pytest.raises(PtmError) as e:
         gguf.GGUFModel(p2, max_seq=64)

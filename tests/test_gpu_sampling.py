@@ -8,7 +8,8 @@ import numpy as np
 import pytest
 import torch
 
-from prometorch_amd import ops, synth
+from prometorch_amd import ops
+from prometorch_amd.testing import synth
 from prometorch_amd._lib import PtmError
 
 pytestmark = pytest.mark.gpu

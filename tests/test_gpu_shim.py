@@ -9,7 +9,8 @@ import pytest
 import torch
 
 from conftest import ROOT
-from prometorch_amd import _lib, ops, synth
+from prometorch_amd import _lib, ops
+from prometorch_amd.testing import synth
 
 pytestmark = pytest.mark.gpu
 

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from conftest import bits, sha, sha_of
-from prometorch_amd import synth
+from prometorch_amd.testing import synth
 
 
 def test_fp16_all_values_vs_numpy_and_reference(po, golden):
@@ -211,7 +211,7 @@ def test_llama_style_decode_and_rope_match_the_reference(po, seeds):
     """No QK-norm + interleaved rotation pairs (llama / mistral): oracle bit-identical to the compiled reference's
     forward_decode_cpu and rope_apply_fused (golden_llama.npz), and the rotation against float64."""
     import os
-    from prometorch_amd import synth
+    from prometorch_amd.testing import synth
     g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_llama.npz"))
     cfg, layers, head = synth.tiny_llama(seeds["tiny"])
     om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)
@@ -258,7 +258,7 @@ def test_qwen2_style_biases_match_the_reference(po, seeds):
     forward_decode_cpu (golden_qwen2.npz); with any one of the three vectors zeroed the logits differ, so the golden run
     does exercise each of them."""
     import os
-    from prometorch_amd import synth
+    from prometorch_amd.testing import synth
     g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_qwen2.npz"))
     cfg, layers, head = synth.tiny_qwen2(seeds["tiny"])
 
@@ -291,7 +291,7 @@ def test_gemma_style_decode_matches_the_reference(po, seeds):
     position scaling on the global ones (gemma3): oracle bit-identical to the compiled reference's forward_decode_cpu
     (golden_gemma.npz); switching any one of the features off moves the first step's logits, so the run exercises each."""
     import os
-    from prometorch_amd import synth
+    from prometorch_amd.testing import synth
     g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_gemma.npz"))
     cfg, layers, head = synth.tiny_gemma(seeds["tiny"])
 
@@ -326,7 +326,7 @@ def test_random_architectures_match_the_reference(po, seed):
     logits over 4 steps are bit-identical to the compiled reference's (golden_random_arch.npz), so the switches are
     pinned in combination, not only one at a time."""
     import os
-    from prometorch_amd import synth
+    from prometorch_amd.testing import synth
     g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_random_arch.npz"))
     cfg, layers, head = synth.random_model(seed)
     om = po.OracleModel(cfg, layers, head, 32, kv_fp16=False)
@@ -357,7 +357,7 @@ def test_mixed_type_layers_match_the_reference(po, seeds, maker, fname):
     not, Q4_K and Q6_K in every projection role (synth.tiny_mixed), and layers in the dispatcher's other formats
     (Q8_0, Q5_K, Q5_0: synth.tiny_formats): oracle bit-identical to the compiled reference's forward_decode_cpu."""
     import os
-    from prometorch_amd import synth
+    from prometorch_amd.testing import synth
     g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", fname))
     cfg, layers, head = getattr(synth, maker)(seeds["tiny"])
     om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)

@@ -6,7 +6,7 @@ import os
 import numpy as np
 import pytest
 
-from prometorch_amd import synth
+from prometorch_amd.testing import synth
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_sampling.npz")
 

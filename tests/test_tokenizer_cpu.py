@@ -10,7 +10,8 @@ import os
 import numpy as np
 import pytest
 
-from prometorch_amd import gguf, synth
+from prometorch_amd import gguf
+from prometorch_amd.testing import gguf_writer, synth
 from prometorch_amd._lib import PtmError
 from prometorch_amd.tokenizer import Tokenizer, chat_template
 
@@ -27,7 +28,7 @@ def from_gguf(kind, tmp_path):
     md = synth.make_tokenizer(kind)
     md["general.architecture"] = "qwen3"
     path = str(tmp_path / f"tok_{kind}.gguf")
-    gguf.write_gguf(path, md, [("dummy", 0, [4], np.zeros(4, np.float32))])
+    gguf_writer.write_gguf(path, md, [("dummy", 0, [4], np.zeros(4, np.float32))])
     f = gguf.GGUFFile(path)
     return md, f, Tokenizer.from_gguf(f)
 
@@ -104,7 +105,7 @@ def test_chat_template_matches_the_reference(golden_tok):
 def test_gguf_arrays_malformed(tmp_path):
     md = {"general.architecture": "qwen3", "a.strings": ["x", "", "yz"], "a.ints": [1, -2, 3], "a.floats": [0.5, 1.5]}
     path = str(tmp_path / "arr.gguf")
-    gguf.write_gguf(path, md, [])
+    gguf_writer.write_gguf(path, md, [])
     with gguf.GGUFFile(path) as f:
         assert f.get_array("a.strings") == [b"x", b"", b"yz"]
         assert list(f.get_array("a.ints")) == [1, -2, 3] and list(f.get_array("a.floats")) == [0.5, 1.5]

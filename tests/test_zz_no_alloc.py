@@ -5,7 +5,8 @@ import numpy as np
 import pytest
 import torch
 
-from prometorch_amd import _lib, ops, synth
+from prometorch_amd import _lib, ops
+from prometorch_amd.testing import synth
 
 pytestmark = pytest.mark.gpu
 
