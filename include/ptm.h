@@ -77,6 +77,11 @@ int ptm_q4k_gemv(const void* W, const float* x, float* y, int K, int N, int64_t 
 /* Same with x already quantised by ptm_quantize_q8 (replaces launch_q4km_q8_gemv, CUDAOps.h:467-470). */
 int ptm_q4k_gemv_q8(const void* W, const void* x_q8, float* y, int K, int N, int64_t row_stride_bytes,
                     int accumulate, ptm_stream_t stream);
+/* Q4_K with fp32 activations, no Q8 rounding: y (+)= sum_k fma(d*sc, q, -(dmin*m)) * x_k, the arithmetic of the reference's
+ * scalar kernel (q4k_gemv_scalar, cpu_quant_gemv.h:689-767; its AVX2 twin q4k_gemv_avx2_float :62-134), which a host with
+ * AVX2 never dispatches to.  The exact-math cross-check of ptm_q4k_gemv; a plain row-per-wave kernel, not tuned. */
+int ptm_q4k_gemv_f32act(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes, int accumulate,
+                        ptm_stream_t stream);
 /* Q6_K with fp32 activations (cpu_quant_gemv.h:883-1020). Replaces launch_q6k_gemv (CUDAOps.h:498-501). */
 int ptm_q6k_gemv(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes,
                  int accumulate, ptm_stream_t stream);
@@ -185,6 +190,12 @@ int ptm_rope_table_host(float* table, int max_seq, int head_dim, float rope_freq
 /* The same with linear position scaling: theta = (pos / scale) * freq when scale is positive and not 1
  * (the `scale` argument of rope_precompute, hot_loops.cpp:1853-1860; ModelConfig::rope_scale, gguf_model.h:71). */
 int ptm_rope_table_host_scaled(float* table, int max_seq, int head_dim, float rope_freq_base, float scale);
+/* The same with phi3's LongRoPE terms (hot_loops.cpp:1861-1873; ModelConfig::rope_factors_for, gguf_model.h:285-296): the
+ * frequency of pair d is divided by factors[d] - row pos takes factors_short while pos + 1 <= orig_ctx and factors_long
+ * beyond (host arrays of head_dim / 2 floats; NULL: no factors for that range; orig_ctx <= 0: none at all) - and cos and sin
+ * are multiplied with attn_factor (0 or 1: not). */
+int ptm_rope_table_host_factors(float* table, int max_seq, int head_dim, float rope_freq_base, float scale,
+                                const float* factors_short, const float* factors_long, int orig_ctx, float attn_factor);
 /* fp32 rows -> fp16 cache rows. launch_fp16_kv_cache_write (CUDAOps.h:635-638). */
 int ptm_fp16_kv_cache_write(const float* src, void* dst_cache_fp16, int64_t num_new_rows, int64_t cols,
                             int64_t offset_row, ptm_stream_t stream);
@@ -407,6 +418,12 @@ typedef struct {
      * rope_swa_freq_base without position scaling (swa_window or swa_pattern 0: no local layers) */
     int32_t scale_embeddings, ffn_gelu, swa_window, swa_pattern;
     float rope_swa_freq_base;
+    /* phi3 LongRoPE (ModelConfig::rope_factors_short / _long / rope_orig_ctx / rope_attn_factor, gguf_model.h:89-96): HOST
+     * arrays of head_dim / 2 per-frequency factors (copied at create; NULL: none), the context length up to which the short
+     * set applies (0: no factors), and the factor cos / sin are scaled by (0 or 1: none); see ptm_rope_table_host_factors */
+    const float *rope_factors_short, *rope_factors_long;
+    int32_t rope_orig_ctx;
+    float rope_attn_factor;
 } ptm_decode_config;
 
 typedef struct ptm_decoder ptm_decoder;
@@ -427,6 +444,10 @@ int ptm_decode_set_past_len(ptm_decoder* d, int64_t past_len);
  * *next_token (host), advances past_len.  Synchronous like forward_decode + GPU argmax
  * (gguf_model.h:3107, :4850-4859). */
 int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token);
+/* One greedy step run as plain launches that also copies out the residual stream after every layer's attention branch and
+ * after its feed-forward branch: trace_device[n_layers][2][hidden] fp32 (device).  The hook the reference has as
+ * PT_DUMP_HIDDEN (gguf_model.h:3268-3289): for comparing a run layer by layer, not for serving. */
+int ptm_decode_step_trace(ptm_decoder* d, int token_id, int64_t* next_token, float* trace_device);
 /* n greedy steps feeding each output back in, without host round trips between tokens:
  * tokens_out[n] (host). */
 /* Prefill: run n prompt tokens (host array) through the model at once, append their K/V rows at positions
@@ -452,6 +473,10 @@ int ptm_decode_generate(ptm_decoder* d, const int32_t* prompt, int n_prompt, con
                         const float* uniforms_host, int max_new, const int32_t* stop_ids, int n_stop,
                         int64_t* out_tokens, int* n_out);
 int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_out);
+/* How the greedy (sampled = 0) or the sampled (1) token step runs: 0 plain launches so far (use_graph = 0, or no second
+ * step yet), 1 replaying its captured hipGraph, 2 plain launches because capturing or instantiating the graph failed
+ * once - not an error: the reference likewise falls back to eager launches (gguf_model.h:2660-2665, :3093-3104). */
+int ptm_decode_graph_state(const ptm_decoder* d, int sampled);
 /* Device pointers to the last step's logits [vocab] and final-normed hidden [hidden]. */
 const float* ptm_decode_logits(ptm_decoder* d);
 const float* ptm_decode_hidden(ptm_decoder* d);

@@ -436,12 +436,22 @@ void po_rope_precompute(float* c, float* s, int64_t pos, int64_t head_dim, float
 }
 /* linear position scaling: theta = (pos / scale) * freq when scale is positive and not 1 (hot_loops.cpp:1858-1860) */
 void po_rope_precompute_scaled(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale) {
+    po_rope_precompute_factors(c, s, pos, head_dim, base, scale, NULL, 1.0f);
+}
+/* per-frequency factors (phi3 LongRoPE: inv_freq[d] /= factor[d]) and the attention factor that scales cos and sin
+ * (hot_loops.cpp:1861-1873) */
+void po_rope_precompute_factors(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale,
+                                const float* factors, float attn_factor) {
     const float p = (scale > 0.0f && scale != 1.0f) ? (float)pos / scale : (float)pos;
+    const int apply_af = attn_factor > 0.0f && attn_factor != 1.0f;
     for (int64_t d = 0; d < head_dim / 2; ++d) {
-        const float inv = 1.0f / powf(base, 2.0f * (float)d / (float)head_dim);
+        float inv = 1.0f / powf(base, 2.0f * (float)d / (float)head_dim);
+        if (factors) inv /= factors[d];
         const float th = p * inv;
-        c[d] = cosf(th);
-        s[d] = sinf(th);
+        float cv = cosf(th), sv = sinf(th);
+        if (apply_af) { cv *= attn_factor; sv *= attn_factor; }
+        c[d] = cv;
+        s[d] = sv;
     }
 }
 static void rope_neox_head(float* h, const float* c, const float* s, int64_t half) {
@@ -580,6 +590,12 @@ static void qgemv(const po_qweight* w, const float* x, float* y) {
 }
 
 int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_out) {
+    return po_decode_step_trace(m, token, logits, hidden_out, NULL);
+}
+
+/* trace (optional): [n_layers][2][hidden], the residual stream after each layer's attention branch and after its
+ * feed-forward branch (what the reference prints under PT_DUMP_HIDDEN, gguf_model.h:3268-3289) */
+int64_t po_decode_step_trace(po_model* m, int64_t token, float* logits, float* hidden_out, float* trace) {
     const int64_t H = m->hidden, hd = m->head_dim, nh = m->n_heads, nkv = m->n_kv_heads;
     const int64_t qd = nh * hd, kvd = nkv * hd, inter = m->inter, past = m->seq_len, T = past + 1;
     float* buf = (float*)malloc(sizeof(float) * (4 * H + 2 * qd + 2 * kvd + 2 * inter));
@@ -600,7 +616,10 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
         po_layer* L = &m->layers[li];
         /* local (sliding-window) layers have their own rotation base and window start (gguf_model.h:265-302, :3490-3500) */
         const int global = m->swa_window <= 0 || m->swa_pattern <= 0 || ((li + 1) % m->swa_pattern) == 0;
-        po_rope_precompute_scaled(rc, rs, past, hd, global ? m->rope_base : m->rope_swa_base, global ? m->rope_scale : 1.0f);
+        /* ModelConfig::rope_factors_for(past_len + 1), gguf_model.h:285-296: the short factors up to the original context */
+        const float* factors = m->rope_orig_ctx <= 0 ? NULL : (past + 1 <= m->rope_orig_ctx ? m->rope_factors_short : m->rope_factors_long);
+        po_rope_precompute_factors(rc, rs, past, hd, global ? m->rope_base : m->rope_swa_base, global ? m->rope_scale : 1.0f,
+                                   factors, m->rope_attn_factor);
         const int64_t t_start = (!global && T > m->swa_window) ? T - m->swa_window : 0;
         const int fuse_qkv = L->q.type == L->k.type && L->q.type == L->v.type;
         if (fuse_qkv) po_rmsnorm_vec(x, L->attn_norm, m->eps, 0, H, xn);
@@ -638,6 +657,7 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
         qgemv(&L->o, ab, hb);
         if (L->post_attn_norm) po_rmsnorm_vec(hb, L->post_attn_norm, m->eps, 0, H, hb); /* gguf_model.h:3656-3663 */
         for (int64_t j = 0; j < H; ++j) x2[j] = x[j] + hb[j];
+        if (trace) memcpy(trace + (2 * li) * H, x2, sizeof(float) * H);
         po_rmsnorm_vec(x2, L->ffn_norm, m->eps, 0, H, xn);
         qgemv(&L->gate, xn, gb);
         qgemv(&L->up, xn, ub);
@@ -646,6 +666,7 @@ int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_
         qgemv(&L->down, gb, hb);
         if (L->post_ffn_norm) po_rmsnorm_vec(hb, L->post_ffn_norm, m->eps, 0, H, hb); /* gguf_model.h:3787-3791 */
         for (int64_t j = 0; j < H; ++j) x[j] = x2[j] + hb[j];
+        if (trace) memcpy(trace + (2 * li + 1) * H, x, sizeof(float) * H);
     }
     po_rmsnorm_vec(x, m->out_norm, m->eps, 0, H, xn);
     if (hidden_out) memcpy(hidden_out, xn, sizeof(float) * H);

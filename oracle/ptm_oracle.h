@@ -78,6 +78,8 @@ void po_rmsnorm_seq(const float* x, const float* gamma, float eps, int add_one, 
 void po_rmsnorm_vec(const float* x, const float* gamma, float eps, int add_one, int64_t H, float* out);
 void po_rope_precompute(float* c, float* s, int64_t pos, int64_t head_dim, float base);
 void po_rope_precompute_scaled(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale);
+void po_rope_precompute_factors(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale,
+                                const float* factors, float attn_factor);
 void po_rope_apply_norm(float* q, float* k, const float* c, const float* s, int64_t n_heads, int64_t n_kv_heads,
                         int64_t head_dim);
 void po_rope_apply_neox(float* q, float* k, const float* c, const float* s,
@@ -122,11 +124,20 @@ typedef struct {
     int scale_embeddings, ffn_gelu;
     int64_t swa_window, swa_pattern;
     float rope_swa_base;
+    /* phi3 LongRoPE (ModelConfig, gguf_model.h:89-96, :285-296): per-frequency factors [head_dim / 2], the short set while
+     * past + 1 <= rope_orig_ctx and the long set beyond (rope_orig_ctx 0: none; a NULL set: none for its range), and the
+     * factor cos and sin are multiplied with (0 or 1: none) */
+    const float *rope_factors_short, *rope_factors_long;
+    int64_t rope_orig_ctx;
+    float rope_attn_factor;
 } po_model;
 
 /* One decode step (forward_decode_cpu order, Q4_K_M fallbacks); writes logits[vocab],
  * advances seq_len, returns greedy argmax. hidden_out (optional) gets the final-normed hidden. */
 int64_t po_decode_step(po_model* m, int64_t token, float* logits, float* hidden_out);
+/* The same, also writing the residual stream after every layer's attention branch and after its feed-forward branch:
+ * trace[n_layers][2][hidden] (may be NULL). */
+int64_t po_decode_step_trace(po_model* m, int64_t token, float* logits, float* hidden_out, float* trace);
 int po_num_threads(void);
 
 /* ---- sampling (reference: GGUFModel::sample_token, gguf_model.h:7658-7751; penalty loop :4926-4938) ---- */

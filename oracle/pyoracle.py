@@ -43,7 +43,8 @@ class Model(C.Structure):
                [("rope_base", _f32), ("eps", _f32), ("kv_fp16", _i32), ("embedding", _vp),
                 ("layers", C.POINTER(Layer)), ("out_norm", _vp), ("lm_head", QW), ("seq_len", _i64), ("rope_interleaved", _i32),
                 ("rope_scale", _f32), ("scale_embeddings", _i32), ("ffn_gelu", _i32), ("swa_window", _i64),
-                ("swa_pattern", _i64), ("rope_swa_base", _f32)]
+                ("swa_pattern", _i64), ("rope_swa_base", _f32), ("rope_factors_short", _vp), ("rope_factors_long", _vp),
+                ("rope_orig_ctx", _i64), ("rope_attn_factor", _f32)]
 
 
 _lib = None
@@ -166,10 +167,13 @@ def rmsnorm(x, gamma, eps, seq=False):
     return out
 
 
-def rope_tables(pos, head_dim, base, scale=1.0):
+def rope_tables(pos, head_dim, base, scale=1.0, factors=None, attn_factor=1.0):
     c = np.empty(head_dim // 2, np.float32)
     s = np.empty(head_dim // 2, np.float32)
-    lib().po_rope_precompute_scaled(_p(c), _p(s), pos, head_dim, base, scale)
+    L = lib()
+    L.po_rope_precompute_factors.argtypes = [_vp, _vp, _i64, _i64, _f32, _f32, _vp, _f32]
+    f = None if factors is None else np.ascontiguousarray(factors, np.float32)
+    L.po_rope_precompute_factors(_p(c), _p(s), pos, head_dim, base, scale, None if f is None else _p(f), attn_factor)
     return c, s
 
 
@@ -315,6 +319,13 @@ class OracleModel:
         self.m.swa_window = int(cfg.get("swa_window", 0))
         self.m.swa_pattern = int(cfg.get("swa_pattern", 0))
         self.m.rope_swa_base = float(cfg.get("rope_swa_base", 10000.0))
+        for key in ("rope_factors_short", "rope_factors_long"):   # phi3 LongRoPE
+            if cfg.get(key) is not None:
+                f = np.ascontiguousarray(cfg[key], np.float32)
+                self._keep.append(f)
+                setattr(self.m, key, f.ctypes.data)
+        self.m.rope_orig_ctx = int(cfg.get("rope_orig_ctx", 0))
+        self.m.rope_attn_factor = float(cfg.get("rope_attn_factor", 1.0))
         self.logits = np.empty(cfg["vocab"], np.float32)
         self.hidden = np.empty(cfg["hidden"], np.float32)
 
@@ -326,6 +337,15 @@ class OracleModel:
 
     def step(self, token: int) -> int:
         return int(lib().po_decode_step(C.byref(self.m), token, _p(self.logits), _p(self.hidden)))
+
+    def step_trace(self, token: int):
+        """One step that also returns the residual stream after every layer's attention branch and feed-forward branch:
+        (token, trace[n_layers, 2, hidden])."""
+        L = lib()
+        L.po_decode_step_trace.restype = _i64
+        trace = np.empty((self.cfg["n_layers"], 2, self.cfg["hidden"]), np.float32)
+        tok = int(L.po_decode_step_trace(C.byref(self.m), token, _p(self.logits), _p(self.hidden), _p(trace)))
+        return tok, trace
 
 
 # ---- compiled reference (only where oracle/_ref has been built) --------------------------
@@ -355,6 +375,8 @@ def ref():
         R.ref_rope_precompute.argtypes = [_vp, _vp, _i64, _i64, _f32]
         R.ref_rope_precompute_scaled.argtypes = [_vp, _vp, _i64, _i64, _f32, _f32]
         R.ref_model_set_rope_scale.argtypes = [_vp, _f32]
+        R.ref_model_set_rope_factors.argtypes = [_vp, _vp, _i64, _vp, _i64, _i64, _f32]
+        R.ref_rope_precompute_factors.argtypes = [_vp, _vp, _i64, _i64, _f32, _f32, _vp, _f32]
         R.ref_model_set_gemma.argtypes = [_vp, _i32, _i32, _i32, _i64, _i64, _f32]
         R.ref_rope_apply_neox.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
         R.ref_rope_apply_norm.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64]
@@ -390,6 +412,10 @@ def ref():
         R.ref_chat_template.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p, _i64]
         R.ref_gguf_n_tensors.restype = _i64
         R.ref_gguf_n_tensors.argtypes = [C.c_char_p]
+        R.ref_model_load_gguf.restype = _vp
+        R.ref_model_load_gguf.argtypes = [C.c_char_p, _i64]
+        R.ref_model_free_loaded.argtypes = [_vp]
+        R.ref_model_describe.argtypes = [_vp, _vp, _vp, _vp]
         _ref = R
     return _ref
 
@@ -402,6 +428,50 @@ def ref_gemv(qtype, W, x):
     y = np.empty(N, np.float32)
     ref().ref_cpu_quant_gemv(qtype, _p(W), _p(x), _p(y), K, N, stride)
     return y
+
+
+LOADED_INT_FIELDS = ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "tied", "has_qk_norm",
+                     "rope_neox", "scale_embeddings", "ffn_gelu", "has_post_norm", "swa_window", "swa_pattern", "use_quant_gemv")
+LOADED_FLOAT_FIELDS = ("rope_base", "eps", "rope_scale", "rope_swa_base", "rope_swa_scale")
+
+
+class RefLoadedModel:
+    """The reference's GGUFModel::load on a .gguf file (its own metadata parser, tensor-name mapping and quantised-weight
+    registration), stepped with forward_decode_cpu."""
+
+    def __init__(self, path: str, max_seq: int):
+        R = ref()
+        self.h = R.ref_model_load_gguf(path.encode(), max_seq)
+        if not self.h:
+            raise RuntimeError("the reference could not load " + path)
+        ints = np.zeros(16, np.int64)
+        floats = np.zeros(5, np.float32)
+        self.ints, self.floats = ints, floats
+        n_layers = self._describe(None)
+        self.types = np.zeros(7 * n_layers + 1, np.uint32)
+        self._describe(self.types)
+        self.cfg = dict(zip(LOADED_INT_FIELDS, (int(v) for v in self.ints)))
+        self.cfg.update(zip(LOADED_FLOAT_FIELDS, (float(v) for v in self.floats)))
+        self.logits = np.empty(self.cfg["vocab"], np.float32)
+
+    def _describe(self, types):
+        R = ref()
+        scratch = np.zeros(7 * 4096 + 1, np.uint32) if types is None else types
+        R.ref_model_describe(self.h, _p(self.ints), _p(self.floats), _p(scratch))
+        return int(self.ints[2])
+
+    def set_kv(self, layer, k16, v16):
+        k = np.ascontiguousarray(k16.astype(np.float32))
+        v = np.ascontiguousarray(v16.astype(np.float32))
+        ref().ref_model_set_kv(self.h, layer, _p(k), _p(v), k.shape[0])
+
+    def step(self, token: int) -> int:
+        return int(ref().ref_model_decode(self.h, token, _p(self.logits)))
+
+    def close(self):
+        if self.h:
+            ref().ref_model_free_loaded(self.h)
+            self.h = None
 
 
 class RefModel:
@@ -417,6 +487,11 @@ class RefModel:
             R.ref_model_set_arch(self.h, int(layers[0].get("q_norm") is not None), int(not cfg.get("rope_interleaved")))
         if cfg.get("rope_scale", 1.0) != 1.0:
             R.ref_model_set_rope_scale(self.h, float(cfg["rope_scale"]))
+        if cfg.get("rope_orig_ctx", 0) > 0 or cfg.get("rope_attn_factor", 1.0) != 1.0:
+            fs = np.ascontiguousarray(cfg.get("rope_factors_short", []), np.float32)
+            fl = np.ascontiguousarray(cfg.get("rope_factors_long", []), np.float32)
+            R.ref_model_set_rope_factors(self.h, _p(fs), fs.size, _p(fl), fl.size, int(cfg.get("rope_orig_ctx", 0)),
+                                         float(cfg.get("rope_attn_factor", 1.0)))
         if any(cfg.get(k) for k in ("scale_embeddings", "ffn_gelu", "swa_window")) or layers[0].get("post_attn_norm") is not None:
             R.ref_model_set_gemma(self.h, int(bool(cfg.get("scale_embeddings"))), int(bool(cfg.get("ffn_gelu"))),
                                   int(layers[0].get("post_attn_norm") is not None), int(cfg.get("swa_window", 0)),

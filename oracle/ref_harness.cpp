@@ -133,6 +133,20 @@ void ref_model_set_rope_scale(void* h, float scale) { static_cast<RefModel*>(h)-
 void ref_rope_precompute_scaled(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale) {
     at::native::hot::rope_precompute(c, s, pos, head_dim, base, scale, nullptr, 1.0f);
 }
+// phi3 LongRoPE fields of ModelConfig (gguf_model.h:89-96): per-frequency factor sets, the context length up to which the
+// short set applies, and the factor cos / sin are scaled by
+void ref_model_set_rope_factors(void* h, const float* fshort, int64_t n_short, const float* flong, int64_t n_long,
+                                int64_t orig_ctx, float attn_factor) {
+    auto& c = static_cast<RefModel*>(h)->m.config;
+    c.rope_factors_short.assign(fshort, fshort + n_short);
+    c.rope_factors_long.assign(flong, flong + n_long);
+    c.rope_orig_ctx = orig_ctx;
+    c.rope_attn_factor = attn_factor;
+}
+void ref_rope_precompute_factors(float* c, float* s, int64_t pos, int64_t head_dim, float base, float scale,
+                                 const float* factors, float attn_factor) {
+    at::native::hot::rope_precompute(c, s, pos, head_dim, base, scale, factors, attn_factor);
+}
 void ref_model_destroy(void* h) {
     auto* r = static_cast<RefModel*>(h);
     // weights are caller-owned: detach before QuantizedWeight could free them

@@ -44,7 +44,8 @@ class DecodeConfig(C.Structure):
                [("rope_freq_base", f32), ("rms_eps", f32), ("kv_fp16", C.c_int32), ("use_graph", C.c_int32),
                 ("embedding_f32", vp), ("layers", C.POINTER(Layer)), ("out_norm", vp), ("lm_head", QWeight),
                 ("rope_interleaved", C.c_int32), ("rope_scale", f32), ("scale_embeddings", C.c_int32),
-                ("ffn_gelu", C.c_int32), ("swa_window", C.c_int32), ("swa_pattern", C.c_int32), ("rope_swa_freq_base", f32)]
+                ("ffn_gelu", C.c_int32), ("swa_window", C.c_int32), ("swa_pattern", C.c_int32), ("rope_swa_freq_base", f32),
+                ("rope_factors_short", vp), ("rope_factors_long", vp), ("rope_orig_ctx", C.c_int32), ("rope_attn_factor", f32)]
 
 
 class Sampling(C.Structure):
@@ -75,6 +76,7 @@ SIGNATURES = {
     "ptm_quantize_q8": (i32, [vp, vp, i32, vp]),
     "ptm_q4k_gemv": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
     "ptm_q4k_gemv_q8": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
+    "ptm_q4k_gemv_f32act": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
     "ptm_q6k_gemv": (i32, [vp, vp, vp, i32, i32, i64, i32, vp]),
     "ptm_argmax_workspace_bytes": (i64, [i32]),
     "ptm_q6k_gemv_argmax": (i32, [vp, vp, vp, i32, i32, i64, vp, vp, vp]),
@@ -100,6 +102,7 @@ SIGNATURES = {
     "ptm_f16_gemv": (i32, [vp, vp, vp, i32, i32, i32, i32, vp]),
     "ptm_rope_table_host": (i32, [vp, i32, i32, f32]),
     "ptm_rope_table_host_scaled": (i32, [vp, i32, i32, f32, f32]),
+    "ptm_rope_table_host_factors": (i32, [vp, i32, i32, f32, f32, vp, vp, i32, f32]),
     "ptm_fp16_kv_cache_write": (i32, [vp, vp, i64, i64, i64, vp]),
     "ptm_flash_decode_kv_chunk_size": (i32, []),
     "ptm_flash_decode_num_splits": (i32, [i32]),
@@ -129,6 +132,7 @@ SIGNATURES = {
     "ptm_decode_reserve_prefill": (i32, [vp, i32]),
     "ptm_decode_step": (i32, [vp, i32, C.POINTER(i64)]),
     "ptm_decode_greedy": (i32, [vp, i32, i32, C.POINTER(i64)]),
+    "ptm_decode_step_trace": (i32, [vp, i32, C.POINTER(i64), vp]),
     "ptm_decode_prefill": (i32, [vp, C.POINTER(C.c_int32), i32, i32, C.POINTER(i64)]),
     "ptm_qgemm_f16_f32_workspace_bytes": (i64, [i32, i32, i32]),
     "ptm_qgemm_f16_f32": (i32, [u32, vp, vp, vp, i32, i32, i32, i64, vp, i32, vp]),
@@ -142,6 +146,7 @@ SIGNATURES = {
     "ptm_sampler_workspace_bytes": (i64, []),
     "ptm_sample_token": (i32, [vp, i32, vp, C.POINTER(Sampling), vp, vp, vp, vp]),
     "ptm_mt19937_uniforms": (i32, [u32, i64, i64, C.POINTER(f32)]),
+    "ptm_decode_graph_state": (i32, [vp, i32]),
     "ptm_decode_logits": (vp, [vp]),
     "ptm_decode_hidden": (vp, [vp]),
     "ptm_decode_stream": (vp, [vp]),

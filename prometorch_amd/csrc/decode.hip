@@ -87,6 +87,7 @@ struct ptm_decoder {
     hipGraph_t graph_s = nullptr;     // one sampled step
     hipGraphExec_t exec_s = nullptr;
     bool captured_s = false;
+    bool eager_fallback = false, eager_fallback_s = false;  // capture or instantiation failed once: plain launches from then on
     // sampling state: parameters (host + device copy), occurrence counts of generated tokens, uniform draws
     ptm_sampling sampling{0.0f, 1, 1.0f, 1.0f};
     bool sampling_set = false;
@@ -158,7 +159,9 @@ static inline bool layer_is_local(const ptm_decode_config& c, int li) {
 }
 
 // Enqueue one token step on d->stream. Everything it reads that changes per token is in device memory.
-static int enqueue_step(ptm_decoder* d, bool sample = false) {
+// trace (optional, device [n_layers][2][hidden]): the residual stream after each layer's attention branch and after its
+// feed-forward branch, copied out between the launches (never part of a captured graph)
+static int enqueue_step(ptm_decoder* d, bool sample = false, float* trace = nullptr) {
     const ptm_decode_config& c = d->cfg;
     hipStream_t s = d->stream;
     const int H = c.hidden, hd = c.head_dim;
@@ -219,6 +222,7 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
             PTM_TRY(gemv_any(L.o, d->attn, o_dst, o_acc, s));
         }
         if (L.post_attn_norm) PTM_TRY(ptm_rms_norm_add(d->hb, L.post_attn_norm, d->x, 1, H, c.rms_eps, 0, s));
+        if (trace) PTM_TRY(ptm_copy(d->x, trace + (size_t)(2 * li) * H, H, s));
         if (L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
             L.gate.row_stride_bytes == L.up.row_stride_bytes && L.gate.rows == L.up.rows) {
             PTM_TRY(q4k_gate_up_silu(L.gate.data, L.up.data, d->x, false, L.ffn_norm, c.rms_eps, 0, d->act, H,
@@ -236,6 +240,7 @@ static int enqueue_step(ptm_decoder* d, bool sample = false) {
         } else {
             PTM_TRY(gemv_any(L.down, d->act, d->x, true, s));  // x += Wdown . act
         }
+        if (trace) PTM_TRY(ptm_copy(d->x, trace + (size_t)(2 * li + 1) * H, H, s));
     }
     if (sample) {
         // logits (final RMSNorm in the lm_head prologue), then the sampler, whose last kernel does the step bookkeeping
@@ -409,6 +414,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->cfg = c;
     d->layers.assign(c.layers, c.layers + c.n_layers);
     d->cfg.layers = d->layers.data();
+    d->cfg.rope_factors_short = d->cfg.rope_factors_long = nullptr;  // host arrays of the caller: read below, not kept
     for (const ptm_layer& L : d->layers)
         for (const ptm_qweight* w : {&L.q, &L.k, &L.v, &L.o, &L.gate, &L.up, &L.down})
             if (!tuned_type(w->ggml_type)) d->untuned_types = true;
@@ -450,10 +456,12 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     if ((rc = hip_status(hipHostMalloc((void**)&d->h_uniforms, 4 * (size_t)c.max_seq, hipHostMallocDefault))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     {
         std::vector<float> tab((size_t)c.max_seq * c.head_dim);
-        ptm_rope_table_host_scaled(tab.data(), c.max_seq, c.head_dim, c.rope_freq_base, c.rope_scale);
+        ptm_rope_table_host_factors(tab.data(), c.max_seq, c.head_dim, c.rope_freq_base, c.rope_scale, c.rope_factors_short,
+                                    c.rope_factors_long, c.rope_orig_ctx, c.rope_attn_factor);
         if ((rc = hip_status(hipMemcpy(d->rope, tab.data(), tab.size() * 4, hipMemcpyHostToDevice))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
         if (c.swa_window > 0) {  // ModelConfig::layer_rope_freq_base / layer_rope_scale, gguf_model.h:297-302
-            ptm_rope_table_host_scaled(tab.data(), c.max_seq, c.head_dim, c.rope_swa_freq_base, 1.0f);
+            ptm_rope_table_host_factors(tab.data(), c.max_seq, c.head_dim, c.rope_swa_freq_base, 1.0f, c.rope_factors_short,
+                                        c.rope_factors_long, c.rope_orig_ctx, c.rope_attn_factor);
             if ((rc = hip_status(hipMemcpy(d->rope_swa, tab.data(), tab.size() * 4, hipMemcpyHostToDevice))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
         }
     }
@@ -500,22 +508,30 @@ static int run_steps(ptm_decoder* d, int token, int n, bool sample = false) {
     hipGraph_t& graph = sample ? d->graph_s : d->graph;
     hipGraphExec_t& exec = sample ? d->exec_s : d->exec;
     int done = 0;
-    if (d->cfg.use_graph && !captured) {
+    bool& fell_back = sample ? d->eager_fallback_s : d->eager_fallback;
+    if (d->cfg.use_graph && !captured && !fell_back) {
         // first step eagerly (sets one-time kernel attributes outside capture), then capture
         if ((rc = enqueue_step(d, sample)) != PTM_OK) return d->status = rc;
         done = 1;
-        {
-            if ((rc = hip_status(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal))) != PTM_OK) return d->status = rc;
+        // A failed capture or instantiation is not an error of the decoder: the step runs as plain launches from then on,
+        // as the reference falls back to eager execution (gguf_model.h:2660-2665, :3093-3104).
+        hipGraph_t g = nullptr;
+        hipGraphExec_t ge = nullptr;
+        bool ok = hip_status(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal)) == PTM_OK;
+        if (ok) {
             const int rc_enq = enqueue_step(d, sample);
-            hipGraph_t g = nullptr;
-            rc = hip_status(hipStreamEndCapture(s, &g));
-            if (rc_enq != PTM_OK || rc != PTM_OK) {
-                if (g) (void)hipGraphDestroy(g);
-                return d->status = (rc_enq != PTM_OK ? rc_enq : rc);
-            }
+            const int rc_end = hip_status(hipStreamEndCapture(s, &g));  // always ends the capture, also after a failed launch
+            ok = rc_enq == PTM_OK && rc_end == PTM_OK && g != nullptr;
+            if (ok) ok = hip_status(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0)) == PTM_OK;
+        }
+        if (ok) {
             graph = g;
-            if ((rc = hip_status(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0))) != PTM_OK) return d->status = rc;
+            exec = ge;
             captured = true;
+        } else {
+            if (g) (void)hipGraphDestroy(g);
+            (void)hipGetLastError();  // the failure has been handled: do not let it surface at the next launch check
+            fell_back = true;
         }
     }
     for (; done < n; ++done) {
@@ -678,11 +694,35 @@ int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token) {
     return rc;
 }
 
+int ptm_decode_step_trace(ptm_decoder* d, int token_id, int64_t* next_token, float* trace_device) {
+    if (!d || !next_token || !trace_device) return PTM_E_NULL;
+    if (d->status != PTM_OK) return PTM_E_STATE;
+    if (token_id < 0 || token_id >= d->cfg.vocab) return PTM_E_RANGE;
+    if (d->past_len + 1 > d->cfg.max_seq) return PTM_E_RANGE;
+    hipStream_t s = d->stream;
+    hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, s, d->d_token, token_id, d->d_past, d->past_len, d->d_step);
+    int rc = launch_status();
+    if (rc != PTM_OK) return rc;
+    if ((rc = enqueue_step(d, false, trace_device)) != PTM_OK) return d->status = rc;
+    if ((rc = hip_status(hipMemcpyAsync(d->h_pinned, d->d_tokens, 8, hipMemcpyDeviceToHost, s))) != PTM_OK) return d->status = rc;
+    if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return d->status = rc;
+    d->past_len += 1;
+    *next_token = d->h_pinned[0];
+    return PTM_OK;
+}
+
 int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_out) {
     if (!d || !tokens_out) return PTM_E_NULL;
     const int rc = run_steps(d, first_token, n);
     if (rc == PTM_OK) for (int i = 0; i < n; ++i) tokens_out[i] = d->h_pinned[i];
     return rc;
+}
+
+int ptm_decode_graph_state(const ptm_decoder* d, int sampled) {
+    if (!d) return PTM_E_NULL;
+    if (sampled ? d->captured_s : d->captured) return 1;
+    if (sampled ? d->eager_fallback_s : d->eager_fallback) return 2;
+    return 0;
 }
 
 const float* ptm_decode_logits(ptm_decoder* d) { return d ? d->logits : nullptr; }

@@ -529,17 +529,28 @@ int ptm_rope_table_host(float* table, int max_seq, int head_dim, float base) {
 }
 
 int ptm_rope_table_host_scaled(float* table, int max_seq, int head_dim, float base, float scale) {
+    return ptm_rope_table_host_factors(table, max_seq, head_dim, base, scale, nullptr, nullptr, 0, 1.0f);
+}
+
+int ptm_rope_table_host_factors(float* table, int max_seq, int head_dim, float base, float scale, const float* factors_short,
+                                const float* factors_long, int orig_ctx, float attn_factor) {
     if (!table) return PTM_E_NULL;
     if (max_seq <= 0 || head_dim <= 0 || (head_dim & 1)) return PTM_E_SHAPE;
     const int half = head_dim / 2;
-    const bool scaled = scale > 0.0f && scale != 1.0f;  // hot_loops.cpp:1858-1860
+    const bool scaled = scale > 0.0f && scale != 1.0f;                 // hot_loops.cpp:1858-1860
+    const bool apply_af = attn_factor > 0.0f && attn_factor != 1.0f;   // hot_loops.cpp:1861
     for (int pos = 0; pos < max_seq; ++pos) {
         const float p = scaled ? (float)pos / scale : (float)pos;
+        // the reference picks the set by the sequence length after this token (gguf_model.h:285-296, called with past + 1)
+        const float* factors = orig_ctx <= 0 ? nullptr : (pos + 1 <= orig_ctx ? factors_short : factors_long);
         for (int d = 0; d < half; ++d) {
-            const float inv = 1.0f / std::pow(base, 2.0f * (float)d / (float)head_dim);
+            float inv = 1.0f / std::pow(base, 2.0f * (float)d / (float)head_dim);
+            if (factors) inv /= factors[d];
             const float th = p * inv;
-            table[(int64_t)pos * head_dim + d] = std::cos(th);
-            table[(int64_t)pos * head_dim + half + d] = std::sin(th);
+            float c = std::cos(th), s = std::sin(th);
+            if (apply_af) { c *= attn_factor; s *= attn_factor; }
+            table[(int64_t)pos * head_dim + d] = c;
+            table[(int64_t)pos * head_dim + half + d] = s;
         }
     }
     return PTM_OK;

@@ -107,6 +107,35 @@ struct FmtQ5_K {
     }
 };
 
+// Q4_K with fp32 activations, as the reference computes it where it has no AVX2 (q4k_gemv_scalar, cpu_quant_gemv.h:689-767):
+// every weight is dequantised as fma(d * sc, q, -(dmin * m)) and multiplied with x, no Q8 rounding of the activations.
+// The exact-math cross-check of the Q8-activation kernel, not a path of the decoder.  Run u is sub-block u & 7 of
+// super-block u >> 3: 32 nibbles of one 32-byte group (low nibbles for even, high for odd sub-blocks).
+struct FmtQ4_K_F32 {
+    static constexpr int BLOCK_BYTES = 144;
+    static __device__ __forceinline__ float term(const uint8_t* __restrict__ row, int u, const float* __restrict__ x) {
+        const int sb = u & 7, hi = sb & 1;
+        const uint8_t* p = row + (int64_t)(u >> 3) * 144;
+        const uint4 hdr = *reinterpret_cast<const uint4*>(p);
+        int sc, mn;
+        q4k_scale_min(hdr.y, hdr.z, hdr.w, sb, sc, mn);
+        const float d1 = h2f(hdr.x) * (float)sc, m1 = h2f(hdr.x >> 16) * (float)mn;
+        const uint8_t* qs = p + 16 + 32 * (sb >> 1);
+        const float* xb = x + 32 * u;
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            const uint32_t q = (*reinterpret_cast<const uint32_t*>(qs + 4 * w) >> (4 * hi)) & 0x0f0f0f0fu;
+            const float4 xv = *reinterpret_cast<const float4*>(xb + 4 * w);
+            s = fmaf(fmaf(d1, (float)(q & 0xffu), -m1), xv.x, s);
+            s = fmaf(fmaf(d1, (float)((q >> 8) & 0xffu), -m1), xv.y, s);
+            s = fmaf(fmaf(d1, (float)((q >> 16) & 0xffu), -m1), xv.z, s);
+            s = fmaf(fmaf(d1, (float)(q >> 24), -m1), xv.w, s);
+        }
+        return s;
+    }
+};
+
 // y[r] (+)= sum over the row's runs of 32; one wave per row, four rows per workgroup
 template <typename Fmt, bool ACC>
 __global__ __launch_bounds__(256) void rowwave_gemv_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x,
@@ -179,6 +208,11 @@ int ptm_q5_0_gemv(const void* W, const float* x, float* y, int K, int N, int64_t
 int ptm_q5k_gemv(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes, int accumulate,
                  ptm_stream_t stream) {
     return rowwave_launch<FmtQ5_K>(W, x, y, K, N, row_stride_bytes, 256, 4, accumulate != 0, as_stream(stream));
+}
+
+int ptm_q4k_gemv_f32act(const void* W, const float* x, float* y, int K, int N, int64_t row_stride_bytes, int accumulate,
+                        ptm_stream_t stream) {
+    return rowwave_launch<FmtQ4_K_F32>(W, x, y, K, N, row_stride_bytes, 256, 16, accumulate != 0, as_stream(stream));
 }
 
 int ptm_dequant_q8_0(const void* blocks, float* out, int64_t n, ptm_stream_t stream) {

@@ -81,6 +81,13 @@ class Decoder:
         c.swa_window = int(cfg.get("swa_window", 0))
         c.swa_pattern = int(cfg.get("swa_pattern", 0))
         c.rope_swa_freq_base = float(cfg.get("rope_swa_base", 10000.0))
+        for key in ("rope_factors_short", "rope_factors_long"):   # phi3 LongRoPE: host arrays, read by decode_create
+            if cfg.get(key) is not None:
+                f = np.ascontiguousarray(cfg[key], np.float32)
+                self._keep.append(f)
+                setattr(c, key, f.ctypes.data)
+        c.rope_orig_ctx = int(cfg.get("rope_orig_ctx", 0))
+        c.rope_attn_factor = float(cfg.get("rope_attn_factor", 1.0))
         if embedding_f32 is not None:
             e = embedding_f32 if isinstance(embedding_f32, torch.Tensor) else torch.from_numpy(embedding_f32)
             e = e.to(device="cuda", dtype=torch.float32).contiguous()
@@ -111,6 +118,14 @@ class Decoder:
         out = C.c_int64()
         check(self.L.ptm_decode_step(self.h, token, C.byref(out)), "decode_step")
         return out.value
+
+    def step_trace(self, token: int):
+        """One step as plain launches that also returns the residual stream after every layer's attention branch and after
+        its feed-forward branch: (token, trace[n_layers, 2, hidden])."""
+        trace = torch.empty(self.cfg["n_layers"], 2, self.cfg["hidden"], dtype=torch.float32, device="cuda")
+        out = C.c_int64()
+        check(self.L.ptm_decode_step_trace(self.h, token, C.byref(out), trace.data_ptr()), "decode_step_trace")
+        return out.value, trace.cpu().numpy()
 
     def prefill(self, tokens, chunk_rows: int = 0) -> int:
         """Run the prompt through the model in row batches, appending its K/V rows; returns the greedy next token

@@ -88,6 +88,9 @@ def main():
     ap.add_argument("--llama-only", action="store_true", help="write golden_llama.npz and nothing else")
     ap.add_argument("--mixed-only", action="store_true", help="write golden_mixed.npz and nothing else")
     ap.add_argument("--formats-only", action="store_true", help="write golden_formats.npz and nothing else")
+    ap.add_argument("--f32act-only", action="store_true", help="write golden_q4k_f32act.npz and nothing else")
+    ap.add_argument("--longrope-only", action="store_true", help="write golden_longrope.npz and nothing else")
+    ap.add_argument("--loader-only", action="store_true", help="write golden_loader.npz and nothing else")
     args = ap.parse_args()
     assert po.have_ref(), "build oracle/_ref first: make -C oracle ref"
     if args.sampling_only:
@@ -117,6 +120,15 @@ def main():
     if args.mixed_only:
         make_mixed_golden()
         print("wrote golden_mixed.npz, golden_formats_model.npz")
+        return
+    if args.f32act_only:
+        make_f32act_golden()
+        return
+    if args.longrope_only:
+        make_longrope_golden()
+        return
+    if args.loader_only:
+        make_loader_golden()
         return
     if args.formats_only:
         make_formats_golden()
@@ -454,6 +466,114 @@ def make_gemma_golden():
         lg.append(rm.logits.copy())
     rm.close()
     np.savez_compressed(os.path.join(OUT, "golden_gemma.npz"), tokens=np.array(toks, np.int64), logits=np.stack(lg))
+
+
+def make_f32act_golden():
+    """The reference's fp32-activation Q4_K kernel (q4k_gemv_scalar, cpu_quant_gemv.h:689-767) on seeded matrices:
+    96 x 2560 and, for the ragged end, 5 x 256."""
+    R = po.ref()
+    out = {}
+    for name, N, K in (("a", 96, 2560), ("b", 5, 256)):
+        r = synth.rng_for(SEEDS["blocks"], 31, N)
+        W = synth.make_q4k(r, N, K)
+        x = synth.make_x(r, K)
+        y = np.empty(N, np.float32)
+        R.ref_q4k_gemv_scalar(W.ctypes.data, x.ctypes.data, y.ctypes.data, K, N, W.shape[1])
+        out["y_" + name] = y
+    np.savez_compressed(os.path.join(OUT, "golden_q4k_f32act.npz"), **out)
+
+
+def longrope_cfg(seed):
+    """synth.TINY with phi3-style LongRoPE terms: per-frequency factors (a short and a long set), the short set valid up to a
+    22-token context - so a run that starts behind 19 cached positions crosses over after three steps - and an attention
+    factor on cos / sin."""
+    cfg = dict(synth.TINY)
+    r = synth.rng_for(seed, 55)
+    half = cfg["head_dim"] // 2
+    cfg["rope_factors_short"] = (1.0 + 0.25 * r.random(half)).astype(np.float32)
+    cfg["rope_factors_long"] = (1.0 + 8.0 * r.random(half)).astype(np.float32)
+    cfg["rope_orig_ctx"] = 22
+    cfg["rope_attn_factor"] = 1.19
+    return cfg
+
+
+def make_longrope_golden():
+    """The reference's rope_precompute with per-frequency factors and attn_factor (hot_loops.cpp:1853-1876), alone and inside
+    forward_decode_cpu (rope_factors_for(past + 1), gguf_model.h:285-296, :3456-3463): 12 steps behind 19 cached positions."""
+    R = po.ref()
+    cfg = longrope_cfg(SEEDS["tiny"])
+    layers = [synth.make_layer(SEEDS["tiny"], i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(SEEDS["tiny"], cfg)
+    g = {}
+    hd = cfg["head_dim"]
+    for pos in (0, 1, 21, 22, 2049):
+        for which in ("short", "long"):
+            c, s = np.empty(hd // 2, np.float32), np.empty(hd // 2, np.float32)
+            f = cfg["rope_factors_" + which]
+            R.ref_rope_precompute_factors(c.ctypes.data, s.ctypes.data, pos, hd, cfg["rope_base"], 1.0, f.ctypes.data,
+                                          cfg["rope_attn_factor"])
+            g["cos_%s_%d" % (which, pos)], g["sin_%s_%d" % (which, pos)] = c, s
+    emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
+    rm = po.RefModel(cfg, layers, head, 64, emb)
+    for i in range(cfg["n_layers"]):
+        k, v = synth.make_kv_prefill(SEEDS["tiny"], i, cfg, 19)
+        rm.set_kv(i, k, v)
+    tok, toks, lg = 3, [], []
+    for _ in range(12):
+        tok = rm.step(tok)
+        toks.append(tok)
+        lg.append(rm.logits.copy())
+    rm.close()
+    g["tokens"], g["logits"] = np.array(toks, np.int64), np.stack(lg)
+    np.savez_compressed(os.path.join(OUT, "golden_longrope.npz"), **g)
+    print("longrope tokens", toks)
+
+
+LOADER_FEED = (3, 17, 900, 41, 5, 5, 260, 77)   # tokens fed to the loaded models step by step
+
+
+def loader_cases(seed):
+    """(name, cfg, layers, head, writer keyword arguments) of the files the loader fixture covers: one per architecture the
+    loader accepts, tied and untied output matrices, and linear position scaling."""
+    t = dict(synth.TINY)
+    tl = [synth.make_layer(seed, i, t) for i in range(t["n_layers"])]
+    th = synth.make_head(seed, t)
+    lc, ll, lh = synth.tiny_llama(seed)
+    qc, ql, qh = synth.tiny_qwen2(seed)
+    gc, gl, gh = synth.tiny_gemma(seed)
+    return [("qwen3_tied", t, tl, th, dict(arch="qwen3", tied=True)),
+            ("qwen3_untied", t, tl, th, dict(arch="qwen3", tied=False, alignment=64)),
+            ("llama", lc, ll, lh, dict(arch="llama")),
+            ("llama_scaled", dict(lc, rope_scale=4.0), ll, lh, dict(arch="llama")),
+            ("qwen2", qc, ql, qh, dict(arch="qwen2")),
+            ("gemma3", gc, gl, gh, dict(arch="gemma3"))]
+
+
+def make_loader_golden():
+    """Files written by this repository's GGUF writer, read by the REFERENCE's own loader (GGUFModel::load,
+    gguf_model.h:2038-2089): what its parser made of the metadata (config fields), which matrices it registered as
+    quantised weights and with which type, and 8 steps of forward_decode_cpu logits behind a 19-position cache."""
+    import tempfile
+    from prometorch_amd.testing import gguf_writer
+    out = {}
+    with tempfile.TemporaryDirectory() as td:
+        for name, cfg, layers, head, kw in loader_cases(SEEDS["tiny"]):
+            path = os.path.join(td, name + ".gguf")
+            gguf_writer.model_to_gguf(path, cfg, layers, head, **kw)
+            rm = po.RefLoadedModel(path, 64)
+            for i in range(cfg["n_layers"]):
+                k, v = synth.make_kv_prefill(SEEDS["tiny"], i, cfg, 19)
+                rm.set_kv(i, k, v)
+            toks, lg = [], []
+            for tok in LOADER_FEED:
+                toks.append(rm.step(tok))
+                lg.append(rm.logits.copy())
+            out[name + "_ints"], out[name + "_floats"], out[name + "_types"] = rm.ints.copy(), rm.floats.copy(), rm.types.copy()
+            out[name + "_tokens"], out[name + "_logits"] = np.array(toks, np.int64), np.stack(lg)
+            out[name + "_sha"] = np.frombuffer(hashlib.sha256(open(path, "rb").read()).hexdigest().encode(), np.uint8)
+            rm.close()
+            print(name, dict(zip(po.LOADED_INT_FIELDS, rm.ints.tolist())), rm.floats.tolist(), toks, flush=True)
+    np.savez_compressed(os.path.join(OUT, "golden_loader.npz"), **out)
 
 
 def make_random_arch_golden():

@@ -80,3 +80,24 @@ def test_dispatcher_types_and_argument_errors(dev):
         ops.dequant_q5k(W, y, 100)                       # not a whole number of blocks
     with pytest.raises(PtmError):
         ops.dequant_q8_0(W, y, 48)
+
+
+@pytest.mark.parametrize("N,K,accumulate", [(96, 2560, False), (5, 256, True), (1000, 4096, False)])
+def test_q4k_fp32_activation_gemv_vs_oracle(dev, po, seeds, N, K, accumulate):
+    """ptm_q4k_gemv_f32act: Q4_K with fp32 activations (the reference's scalar kernel, cpu_quant_gemv.h:689-767) against
+    the oracle's restatement of it, which golden_q4k_f32act.npz pins to the compiled reference."""
+    from prometorch_amd import _lib
+    r = synth.rng_for(seeds["blocks"], 31, N)
+    W = synth.make_q4k(r, N, K)
+    x = synth.make_x(r, K)
+    want = po.gemv(12, W, x, "f32")
+    y0 = synth.make_x(r, N)
+    Wd, xd = torch.from_numpy(W).cuda(), torch.from_numpy(x).cuda()
+    y = torch.from_numpy(y0.copy()).cuda()
+    _lib.check(ops._L().ptm_q4k_gemv_f32act(Wd.data_ptr(), xd.data_ptr(), y.data_ptr(), K, N, W.shape[1], int(accumulate),
+                                            torch.cuda.current_stream().cuda_stream), "q4k_gemv_f32act")
+    torch.cuda.synchronize()
+    got = y.cpu().numpy() - (y0 if accumulate else 0)
+    rms = np.sqrt((want.astype(np.float64) ** 2).mean())
+    assert np.abs(got - want).max() / rms < (1e-3 if not accumulate else 1e-3 + 1e-6 * np.abs(y0).max() / rms)
+    assert np.abs(got - want).max() / rms < 2e-5 or accumulate   # measured ~1e-6: only the summation order differs

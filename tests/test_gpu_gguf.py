@@ -147,3 +147,59 @@ def test_chat_is_the_manual_path_in_one_call(dev, seeds, tmp_path):
     with pytest.raises(ValueError):
         m.chat("x " * 400, max_new=8)
     m.close()
+
+
+LOADER_CASES = ("qwen3_tied", "qwen3_untied", "llama", "llama_scaled", "qwen2", "gemma3")
+
+
+@pytest.mark.parametrize("case", LOADER_CASES)
+def test_loader_agrees_with_the_references_own_loader(dev, seeds, tmp_path, case):
+    """golden_loader.npz: the same files (byte-identical: sha256 checked) as the REFERENCE's GGUFModel::load read them -
+    its config fields, the type it registered for every matrix, and 8 steps of its forward_decode_cpu logits.
+    ptm_model_load_gguf must arrive at the same configuration, the same types, and logits within the decode bars."""
+    import hashlib
+    import os
+    import sys
+    from conftest import GOLDEN_DIR
+    sys.path.insert(0, GOLDEN_DIR)
+    import make_golden as mg   # the case list and the fed tokens live beside the script that wrote the fixture
+    g = np.load(os.path.join(GOLDEN_DIR, "golden_loader.npz"), allow_pickle=False)
+    name, cfg, layers, head, kw = [c for c in mg.loader_cases(seeds["tiny"]) if c[0] == case][0]
+    path = str(tmp_path / (case + ".gguf"))
+    gguf_writer.model_to_gguf(path, cfg, layers, head, **kw)
+    assert hashlib.sha256(open(path, "rb").read()).hexdigest() == bytes(g[case + "_sha"]).decode(), "not the file the reference read"
+    m = gguf.GGUFModel(path, max_seq=64, kv_fp16=False)
+    from oracle import pyoracle as po
+    ref_cfg = dict(zip(po.LOADED_INT_FIELDS, (int(v) for v in g[case + "_ints"])))
+    ref_cfg.update(zip(po.LOADED_FLOAT_FIELDS, (float(v) for v in g[case + "_floats"])))
+    for k in ("vocab", "hidden", "n_layers", "n_heads", "n_kv_heads", "head_dim", "inter", "swa_window"):
+        assert m.cfg[k] == ref_cfg[k], (k, m.cfg[k], ref_cfg[k])
+    assert m.cfg["tied"] == bool(ref_cfg["tied"])
+    assert m.cfg["rope_interleaved"] == (not ref_cfg["rope_neox"])
+    assert m.cfg["scale_embeddings"] == bool(ref_cfg["scale_embeddings"]) and m.cfg["ffn_gelu"] == bool(ref_cfg["ffn_gelu"])
+    assert np.float32(m.cfg["rope_base"]) == np.float32(ref_cfg["rope_base"]) and np.float32(m.cfg["eps"]) == np.float32(ref_cfg["eps"])
+    assert np.float32(m.cfg["rope_scale"] or 1.0) == np.float32(ref_cfg["rope_scale"])
+    if ref_cfg["swa_window"]:
+        assert m.cfg["swa_pattern"] == ref_cfg["swa_pattern"]
+        assert np.float32(m.cfg["rope_swa_base"]) == np.float32(ref_cfg["rope_swa_base"])
+    types = g[case + "_types"]
+    for i in range(cfg["n_layers"]):
+        Ld = m.layer(i)
+        got = [getattr(Ld, n).ggml_type for n in ("q", "k", "v", "o", "gate", "up", "down")]
+        assert got == [int(t) for t in types[7 * i:7 * i + 7]], (i, got)
+        assert bool(Ld.q_norm) == bool(ref_cfg["has_qk_norm"]) and bool(Ld.post_attn_norm) == bool(ref_cfg["has_post_norm"])
+    for i in range(cfg["n_layers"]):
+        m.set_kv(i, *synth.make_kv_prefill(seeds["tiny"], i, cfg, 19))
+    m.set_past_len(19)
+    errs = []
+    for st, tok in enumerate(mg.LOADER_FEED):
+        t = m.step(tok)
+        ref = g[case + "_logits"][st]
+        errs.append(float(np.abs(m.logits() - ref).max() / ref.std()))
+        assert t == int(g[case + "_tokens"][st]), (st, errs[-1])
+    errs = np.asarray(errs)
+    # llama-style models (no QK-norm) amplify the Q8 rounding noise of single steps more: their bars are the llama tests' own
+    loose = case.startswith("llama") or case == "qwen2"
+    assert errs.max() <= (5e-2 if loose else 2e-2), errs
+    assert int((errs > 1e-3).sum()) <= (8 if loose else 2), errs
+    m.close()

@@ -366,3 +366,68 @@ def test_mixed_type_layers_match_the_reference(po, seeds, maker, fname):
     for st in range(12):
         assert om.step(synth.MIXED_FEED[st]) == int(g["tokens"][st]), st
         assert np.array_equal(bits(om.logits), bits(g["logits"][st])), st
+
+
+def test_q4k_fp32_activation_variant_vs_reference_scalar_kernel(po, seeds):
+    """golden_q4k_f32act.npz: the compiled reference's q4k_gemv_scalar (fp32 activations, no Q8 rounding); the oracle's
+    restatement is bit-identical, and equals the float64 product of the dequantised matrix to fp32 rounding."""
+    import os
+    from conftest import GOLDEN_DIR
+    g = np.load(os.path.join(GOLDEN_DIR, "golden_q4k_f32act.npz"), allow_pickle=False)
+    for name, N, K in (("a", 96, 2560), ("b", 5, 256)):
+        r = synth.rng_for(seeds["blocks"], 31, N)
+        W = synth.make_q4k(r, N, K)
+        x = synth.make_x(r, K)
+        y = po.gemv(12, W, x, "f32")
+        assert np.array_equal(bits(y), bits(g["y_" + name])), name
+        want = po.dequant(12, W).reshape(N, K).astype(np.float64) @ x.astype(np.float64)
+        assert np.abs(y - want).max() / np.sqrt((want ** 2).mean()) < 1e-5
+
+
+def test_longrope_factors_vs_reference(po, seeds):
+    """golden_longrope.npz: the compiled reference's rope_precompute with per-frequency factors and attn_factor, and 12 steps
+    of its forward_decode_cpu on a model whose factor set switches from short to long inside the run.  The oracle is
+    bit-identical; the C ABI's host table builder too; factors that are all 1 with attn_factor 1 change nothing."""
+    import os
+    import sys
+    from conftest import GOLDEN_DIR
+    sys.path.insert(0, GOLDEN_DIR)
+    import make_golden as mg
+    from prometorch_amd import _lib
+    g = np.load(os.path.join(GOLDEN_DIR, "golden_longrope.npz"), allow_pickle=False)
+    cfg = mg.longrope_cfg(seeds["tiny"])
+    hd = cfg["head_dim"]
+    for pos in (0, 1, 21, 22, 2049):
+        for which in ("short", "long"):
+            c, s = po.rope_tables(pos, hd, cfg["rope_base"], 1.0, cfg["rope_factors_" + which], cfg["rope_attn_factor"])
+            assert np.array_equal(bits(c), bits(g["cos_%s_%d" % (which, pos)])), (which, pos)
+            assert np.array_equal(bits(s), bits(g["sin_%s_%d" % (which, pos)])), (which, pos)
+    # the product's host table: row pos takes the short set while pos + 1 <= orig_ctx
+    tab = np.empty((40, hd), np.float32)
+    fs, fl = cfg["rope_factors_short"], cfg["rope_factors_long"]
+    assert _lib.load().ptm_rope_table_host_factors(tab.ctypes.data, 40, hd, cfg["rope_base"], 1.0, fs.ctypes.data, fl.ctypes.data,
+                                                   cfg["rope_orig_ctx"], cfg["rope_attn_factor"]) == 0
+    for pos, which in ((0, "short"), (1, "short"), (21, "short"), (22, "long")):
+        assert np.array_equal(bits(tab[pos, :hd // 2]), bits(g["cos_%s_%d" % (which, pos)])), pos
+        assert np.array_equal(bits(tab[pos, hd // 2:]), bits(g["sin_%s_%d" % (which, pos)])), pos
+    plain = np.empty((40, hd), np.float32)
+    ones = np.ones(hd // 2, np.float32)
+    _lib.load().ptm_rope_table_host_factors(plain.ctypes.data, 40, hd, cfg["rope_base"], 1.0, ones.ctypes.data, ones.ctypes.data, 22, 1.0)
+    c0, s0 = po.rope_tables(17, hd, cfg["rope_base"])
+    assert np.array_equal(bits(plain[17, :hd // 2]), bits(c0)) and np.array_equal(bits(plain[17, hd // 2:]), bits(s0))
+    # the whole step
+    layers = [synth.make_layer(seeds["tiny"], i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(seeds["tiny"], cfg)
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)
+    for i in range(cfg["n_layers"]):
+        om.set_kv(i, *synth.make_kv_prefill(seeds["tiny"], i, cfg, 19))
+    tok = 3
+    for st in range(12):
+        tok = om.step(tok)
+        assert tok == int(g["tokens"][st]) and np.array_equal(bits(om.logits), bits(g["logits"][st])), st
+    # and the factors matter: the same model without them decodes to different logits
+    om2 = po.OracleModel(dict(synth.TINY), layers, head, 64, kv_fp16=False)
+    for i in range(cfg["n_layers"]):
+        om2.set_kv(i, *synth.make_kv_prefill(seeds["tiny"], i, cfg, 19))
+    om2.step(3)
+    assert np.abs(om2.logits - g["logits"][0]).max() / g["logits"][0].std() > 1e-2
