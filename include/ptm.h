@@ -276,9 +276,11 @@ int ptm_argmax(const float* in, int64_t* out, int64_t n, ptm_stream_t stream);
  * applied first: penalty once per earlier occurrence (counts[i]; NULL = none), temperature, top-k (ties at the
  * k-th value kept), softmax, top-p, inverse CDF in index order against the uniform draw *d_uniform (device
  * memory; the reference draws it from a static std::mt19937(42) through uniform_real_distribution<float>).
- * temperature < 1e-6: argmax of the penalised logits, no draw.  Implemented for 1 <= top_k <= 1024 and
- * top_k < vocab (PTM_E_UNSUPPORTED otherwise: sample on the host from ptm_decode_logits).  *out_token (device)
- * is -1 when more than 2048 logits tie at the top-k threshold.  workspace: ptm_sampler_workspace_bytes() device
+ * temperature < 1e-6: argmax of the penalised logits, no draw.  1 <= top_k <= 1024 (and below the vocabulary) runs on a
+ * gathered candidate list with the reference's sums in the reference's order; top-k off (top_k <= 0 or >= vocab) and
+ * larger top_k run as passes over the whole vocabulary whose sums are order-independent 64-bit fixed-point ones (they
+ * differ from the reference's sequential fp32 sums by rounding, ~1e-7 of the distribution).  *out_token (device)
+ * is -1 when more than 2048 logits tie at the threshold of a top_k <= 1024.  workspace: ptm_sampler_workspace_bytes() device
  * bytes, 8-byte aligned, contents irrelevant.  Replaces the 608 KB logits copy + CPU sampling per token. */
 typedef struct ptm_sampling {
     float temperature;

@@ -550,7 +550,6 @@ int ptm_decode_sampling_begin(ptm_decoder* d, const ptm_sampling* params) {
     if (d->status != PTM_OK) return PTM_E_STATE;
     const bool greedy = !(params->temperature >= 1e-6f);
     if (!greedy) {
-        if (params->top_k <= 0 || params->top_k >= d->cfg.vocab || params->top_k > 1024) return PTM_E_UNSUPPORTED;
         if (!(params->top_p > 0.0f)) return PTM_E_SHAPE;
     }
     hipStream_t s = d->stream;

@@ -32,9 +32,16 @@ enum {
     SW_COUNT = 5120,              // number of gathered candidates
     SW_CAND_KEY = 5128,           // [SAMPLER_MAX_CAND]
     SW_CAND_IDX = SW_CAND_KEY + SAMPLER_MAX_CAND,
-    SW_WORDS = SW_CAND_IDX + SAMPLER_MAX_CAND,
+    // the wide path (top-k off or beyond SAMPLER_MAX_TOPK): scalars, and a 2048-bin 64-bit mass histogram that shares the
+    // candidate arrays (the two paths never run in the same call)
+    SW_WIDE = SW_CAND_IDX + SAMPLER_MAX_CAND,
+    SW_MASS_HIST = SW_CAND_KEY,
+    SW_WORDS = SW_WIDE + 64,
     SW_CLEAR_WORDS = SW_COUNT + 8
 };
+// wide-path scalars (32-bit words from SW_WIDE): top-k threshold key, largest kept key, sum of exp (64-bit, 2^-32 units),
+// probability mass above the current prefix (64-bit, 2^-40 units), key prefix chosen so far, 1 when every eligible token stays
+enum { WS_THR = 0, WS_MAXKEY = 1, WS_SUMEXP = 2, WS_MASS_ABOVE = 4, WS_PREFIX = 6, WS_KEEP_ALL = 7, WS_TSTAR = 8, WS_NTIE = 9 };
 
 struct SamplerArgs {
     const float* logits;
@@ -371,10 +378,315 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Wide path: top-k off (top_k <= 0 or >= vocab) or a top-k beyond the candidate list.  The distribution then spans (almost)
+// the whole vocabulary, so nothing is gathered: every stage is a pass over the logits.  Sums that decide something (the
+// softmax denominator, the nucleus mass) are accumulated in 64-bit fixed point with integer atomics, so that the result does
+// not depend on the order in which workgroups arrive; they differ from the reference's sequential fp32 sums by rounding
+// (~1e-7 relative), which moves a token's CDF interval by that much.
+// ---------------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float wide_inv_sum(const uint32_t* w) {
+    const unsigned long long s = *reinterpret_cast<const unsigned long long*>(w + WS_SUMEXP);
+    return 1.0f / ((float)s * 2.3283064365386963e-10f);  // 2^-32
+}
+__device__ __forceinline__ unsigned long long shfl_down_u64(unsigned long long v, int off) {
+    const uint32_t lo = __shfl_down((uint32_t)v, off, 64), hi = __shfl_down((uint32_t)(v >> 32), off, 64);
+    return ((unsigned long long)hi << 32) | lo;
+}
+
+// thr: key of the k-th largest value when a top-k beyond the candidate list is active (else 0: everything is kept)
+__global__ __launch_bounds__(256) void sampler_wide_threshold_kernel(SamplerArgs a, int use_topk) {
+    __shared__ uint32_t s_scan[8];
+    uint32_t* w = a.ws + SW_WIDE;
+    uint32_t thr = 0;
+    if (use_topk) {
+        const ptm_sampling p = sampler_params(a);
+        int b0, b1, b2, k = sampler_k(p);
+        select_bin(a.ws + SW_HIST0, 2048, k, b0, k, s_scan);
+        select_bin(a.ws + SW_HIST1, 2048, k, b1, k, s_scan);
+        select_bin(a.ws + SW_HIST2, 1024, k, b2, k, s_scan);
+        thr = ((uint32_t)b0 << 21) | ((uint32_t)b1 << 10) | (uint32_t)b2;
+    }
+    if (threadIdx.x < 16) w[threadIdx.x] = threadIdx.x == WS_THR ? thr : 0u;
+    // the mass histogram shares the candidate arrays of the narrow path, which leaves anything there
+    for (int i = threadIdx.x; i < 2 * 2048; i += 256) a.ws[SW_MASS_HIST + i] = 0;
+}
+
+__global__ __launch_bounds__(256) void sampler_wide_max_kernel(SamplerArgs a) {
+    const ptm_sampling p = sampler_params(a);
+    uint32_t* w = a.ws + SW_WIDE;
+    const uint32_t thr = w[WS_THR];
+    uint32_t best = 0;
+    const int base = blockIdx.x * SAMPLER_ELEMS_PER_WG;
+#pragma unroll
+    for (int u = 0; u < SAMPLER_ELEMS_PER_WG / 256; ++u) {
+        const int i = base + threadIdx.x + 256 * u;
+        if (i < a.vocab) {
+            const uint32_t key = order_key(sampler_value(a, p, i));
+            if (key >= thr && key > best) best = key;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) best = max(best, (uint32_t)__shfl_down(best, off, 64));
+    if ((threadIdx.x & 63) == 0 && best) atomicMax(&w[WS_MAXKEY], best);
+}
+
+__global__ __launch_bounds__(256) void sampler_wide_sumexp_kernel(SamplerArgs a) {
+    const ptm_sampling p = sampler_params(a);
+    uint32_t* w = a.ws + SW_WIDE;
+    const uint32_t thr = w[WS_THR];
+    const float mx = key_value(w[WS_MAXKEY]);
+    unsigned long long acc = 0;
+    const int base = blockIdx.x * SAMPLER_ELEMS_PER_WG;
+#pragma unroll
+    for (int u = 0; u < SAMPLER_ELEMS_PER_WG / 256; ++u) {
+        const int i = base + threadIdx.x + 256 * u;
+        if (i < a.vocab) {
+            const float x = sampler_value(a, p, i);
+            if (order_key(x) >= thr) acc += (unsigned long long)(expf(x - mx) * 4294967296.0f);  // e <= 1
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) acc += shfl_down_u64(acc, off);
+    if ((threadIdx.x & 63) == 0 && acc) atomicAdd(reinterpret_cast<unsigned long long*>(w + WS_SUMEXP), acc);
+}
+
+// probability of a kept token as every wide kernel computes it
+__device__ __forceinline__ float wide_prob(float x, float mx, float inv) { return expf(x - mx) * inv; }
+__device__ __forceinline__ unsigned long long wide_mass(float pr) { return (unsigned long long)(pr * 1099511627776.0f); }  // 2^40
+
+// LEVEL 0/1/2: probability mass (2^-40 units) per key bin among the kept, eligible (p > 1e-10) tokens under the prefix
+template <int LEVEL>
+__global__ __launch_bounds__(256) void sampler_wide_mass_hist_kernel(SamplerArgs a) {
+    constexpr int NB = LEVEL == 2 ? 1024 : 2048;
+    __shared__ unsigned long long s_hist[NB];
+    const int tid = threadIdx.x;
+    const ptm_sampling p = sampler_params(a);
+    uint32_t* w = a.ws + SW_WIDE;
+    if (w[WS_KEEP_ALL]) return;
+    const uint32_t thr = w[WS_THR], prefix = w[WS_PREFIX];
+    const float mx = key_value(w[WS_MAXKEY]), inv = wide_inv_sum(w);
+    for (int i = tid; i < NB; i += 256) s_hist[i] = 0;
+    __syncthreads();
+    const int base = blockIdx.x * SAMPLER_ELEMS_PER_WG;
+#pragma unroll
+    for (int u = 0; u < SAMPLER_ELEMS_PER_WG / 256; ++u) {
+        const int i = base + tid + 256 * u;
+        if (i >= a.vocab) continue;
+        const float x = sampler_value(a, p, i);
+        const uint32_t key = order_key(x);
+        if (key < thr) continue;
+        const float pr = wide_prob(x, mx, inv);
+        if (!(pr > 1e-10f)) continue;
+        int bin;
+        if (LEVEL == 0) bin = (int)(key >> 21);
+        else if (LEVEL == 1) { if ((key >> 21) != prefix) continue; bin = (int)((key >> 10) & 0x7ffu); }
+        else { if ((key >> 10) != prefix) continue; bin = (int)(key & 0x3ffu); }
+        atomicAdd(&s_hist[bin], wide_mass(pr));
+    }
+    __syncthreads();
+    unsigned long long* g = reinterpret_cast<unsigned long long*>(a.ws + SW_MASS_HIST);
+    for (int i = tid; i < NB; i += 256)
+        if (s_hist[i]) atomicAdd(&g[i], s_hist[i]);
+}
+
+// Walk the level's bins from the top: the bin in which the accumulated mass reaches top_p becomes part of the key prefix, the
+// mass above it is carried on; the histogram is zeroed for the next level.  After level 2 the prefix is the key t* of the
+// last token value that enters the nucleus, and the number of tokens of that value that enter is fixed (the reference adds
+// tokens in descending order and stops as soon as the sum reaches top_p).
+template <int LEVEL>
+__global__ __launch_bounds__(256) void sampler_wide_select_kernel(SamplerArgs a) {
+    constexpr int NB = LEVEL == 2 ? 1024 : 2048, PER = NB / 256;
+    __shared__ unsigned long long s_wave[4];
+    __shared__ uint32_t s_found[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const ptm_sampling p = sampler_params(a);
+    uint32_t* w = a.ws + SW_WIDE;
+    unsigned long long* g = reinterpret_cast<unsigned long long*>(a.ws + SW_MASS_HIST);
+    if (w[WS_KEEP_ALL]) return;
+    const unsigned long long target = (unsigned long long)((double)p.top_p * 1099511627776.0);
+    const unsigned long long above0 = *reinterpret_cast<unsigned long long*>(w + WS_MASS_ABOVE);
+    unsigned long long h[PER], mine = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) { h[j] = g[NB - 1 - (tid * PER + j)]; mine += h[j]; }
+    unsigned long long incl = mine;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t lo = __shfl_up((uint32_t)incl, off, 64), hi = __shfl_up((uint32_t)(incl >> 32), off, 64);
+        if (lane >= off) incl += ((unsigned long long)hi << 32) | lo;
+    }
+    if (tid < 4) s_found[tid] = tid == 0 ? 0u : 0u;
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    for (int q = 0; q < wave; ++q) incl += s_wave[q];
+    const unsigned long long excl = incl - mine;
+    if (above0 + excl < target && above0 + incl >= target) {   // exactly one thread, if any
+        unsigned long long above = above0 + excl;
+        for (int j = 0; j < PER; ++j) {
+            if (above + h[j] >= target) {
+                const uint32_t bin = (uint32_t)(NB - 1 - (tid * PER + j));
+                s_found[0] = 1;
+                s_found[1] = bin;
+                *reinterpret_cast<unsigned long long*>(w + WS_MASS_ABOVE) = above;
+                break;
+            }
+            above += h[j];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PER; ++j) g[NB - 1 - (tid * PER + j)] = 0;   // clean for the next level / the next call
+    if (tid == 0) {
+        if (!s_found[0]) {
+            w[WS_KEEP_ALL] = 1;   // the eligible tokens together do not reach top_p: all of them stay (the reference's loop runs out)
+        } else {
+            const uint32_t bin = s_found[1];
+            const uint32_t prefix = LEVEL == 0 ? bin : LEVEL == 1 ? ((w[WS_PREFIX] << 11) | bin) : ((w[WS_PREFIX] << 10) | bin);
+            w[WS_PREFIX] = prefix;
+            if (LEVEL == 2) {
+                const float pstar = wide_prob(key_value(prefix), key_value(w[WS_MAXKEY]), wide_inv_sum(w));
+                const unsigned long long pf = wide_mass(pstar), above = *reinterpret_cast<unsigned long long*>(w + WS_MASS_ABOVE);
+                unsigned long long n = pf ? (target - above + pf - 1) / pf : 1;
+                w[WS_TSTAR] = prefix;
+                w[WS_NTIE] = (uint32_t)(n < 1 ? 1 : (n > 0xffffffffull ? 0xffffffffull : n));
+            }
+        }
+    }
+}
+
+// The draw: one workgroup, wave q walks the q-th sixteenth of the vocabulary in index order, 64 tokens at a time.
+// Walk 0 counts the tokens of the nucleus' last value per wave (the first WS_NTIE of them in index order stay), walk 1 sums
+// the kept probabilities per wave (the renormalisation of the reference's top-p step), walk 2 finds the first index whose
+// running sum reaches the draw.
+__global__ __launch_bounds__(1024) void sampler_wide_draw_kernel(SamplerArgs a, SamplerOut o) {
+    __shared__ uint32_t s_ties[16];
+    __shared__ float s_sum[16];
+    __shared__ int s_token[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const ptm_sampling p = sampler_params(a);
+    uint32_t* w = a.ws + SW_WIDE;
+    const int step = o.d_step ? *o.d_step : 0;
+    const int64_t past_now = o.adv.d_past ? *o.adv.d_past : 0;
+    const float r = o.uniforms[step];
+    const uint32_t thr = w[WS_THR];
+    const float mx = key_value(w[WS_MAXKEY]), inv = wide_inv_sum(w);
+    const bool nucleus = p.top_p < 1.0f;
+    const bool keep_all = w[WS_KEEP_ALL] != 0;
+    const uint32_t tstar = w[WS_TSTAR], ntie = w[WS_NTIE];
+    const int per_wave = ((a.vocab + 15) / 16 + 63) / 64 * 64;
+    const int lo = wave * per_wave, hi = min(a.vocab, lo + per_wave);
+    // walk 0: ties of the nucleus' last value in this wave's range
+    uint32_t my_ties = 0;
+    if (nucleus && !keep_all) {
+        for (int b = lo; b < hi; b += 64) {
+            const int i = b + lane;
+            const bool tie = i < hi && order_key(sampler_value(a, p, i)) == tstar;
+            my_ties += (uint32_t)__popcll(__ballot(tie));
+        }
+    }
+    if (lane == 0) s_ties[wave] = my_ties;
+    __syncthreads();
+    uint32_t tie_base = 0;
+    for (int q = 0; q < wave; ++q) tie_base += s_ties[q];
+    // kept probability of token i (0 when dropped); tie_rank counts the ties seen so far in index order
+    auto kept_prob = [&](int i, bool in, uint32_t& tie_seen) -> float {
+        float pr = 0.0f;
+        bool tie = false;
+        if (in) {
+            const float x = sampler_value(a, p, i);
+            const uint32_t key = order_key(x);
+            if (key >= thr) {
+                pr = wide_prob(x, mx, inv);
+                if (nucleus) {
+                    if (!(pr > 1e-10f)) pr = 0.0f;
+                    else if (!keep_all) {
+                        tie = key == tstar;
+                        if (key < tstar) pr = 0.0f;
+                    }
+                }
+            }
+        }
+        const unsigned long long tb = __ballot(tie);
+        if (tie) {
+            const uint32_t rank = tie_seen + (uint32_t)__popcll(tb & ((1ull << lane) - 1ull));
+            if (rank >= ntie) pr = 0.0f;
+        }
+        tie_seen += (uint32_t)__popcll(tb);
+        return pr;
+    };
+    // walk 1: sum of the kept probabilities (only the nucleus step renormalises)
+    float total = 1.0f;
+    if (nucleus) {
+        float acc = 0.0f;
+        uint32_t seen = tie_base;
+        for (int b = lo; b < hi; b += 64) acc += kept_prob(b + lane, b + lane < hi, seen);
+        acc = sum64(acc);
+        if (lane == 0) s_sum[wave] = acc;
+        __syncthreads();
+        total = 0.0f;
+        for (int q = 0; q < 16; ++q) total += s_sum[q];
+        __syncthreads();
+    }
+    const float scale = (nucleus && total > 0.0f) ? 1.0f / total : 1.0f;
+    // walk 2: per-wave sums first (to know where each wave's running sum starts), then the crossing
+    {
+        float acc = 0.0f;
+        uint32_t seen = tie_base;
+        for (int b = lo; b < hi; b += 64) acc += kept_prob(b + lane, b + lane < hi, seen) * scale;
+        acc = sum64(acc);
+        if (lane == 0) s_sum[wave] = acc;
+    }
+    __syncthreads();
+    float cum = 0.0f;
+    for (int q = 0; q < wave; ++q) cum += s_sum[q];
+    int found = 0x7fffffff;
+    // Every wave adds the same per-wave sums in the same order, so exactly one wave (if any) sees the running sum pass the
+    // draw inside its range; it looks for the index.  Its 64-wide scans round differently from the per-wave sum: should they
+    // never reach the draw, the wave's last kept token is the one that tipped the sum.
+    if (cum < r && cum + s_sum[wave] >= r) {
+        uint32_t seen = tie_base;
+        int last_kept = lo;
+        for (int b = lo; b < hi && found == 0x7fffffff; b += 64) {
+            const float v = kept_prob(b + lane, b + lane < hi, seen) * scale;
+            float incl = v;   // inclusive prefix sum over the wave, lane order = index order
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const float up = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += up;
+            }
+            const unsigned long long hit = __ballot(b + lane < hi && cum + incl >= r);
+            const unsigned long long any = __ballot(v > 0.0f);
+            if (any) last_kept = b + 63 - (int)__builtin_clzll(any);
+            if (hit) found = b + (int)__builtin_ctzll(hit);
+            cum += lane_f(incl, 63);
+        }
+        if (found == 0x7fffffff) found = last_kept;
+    }
+    if (lane == 0) s_token[wave] = found;
+    __syncthreads();
+    if (tid == 0) {
+        int token = a.vocab - 1;   // the running sum never reached the draw (rounding): the reference returns the last id
+        for (int q = 0; q < 16; ++q) if (s_token[q] != 0x7fffffff) { token = s_token[q]; break; }
+        if (r <= 0.0f) token = 0;
+        if (o.out_token) *o.out_token = token;
+        if (o.counts_rw) o.counts_rw[token] += 1;
+        if (o.adv.d_step) {
+            if (step < o.adv.cap) o.adv.tokens_out[step] = token;
+            *o.adv.d_token = token;
+            *o.adv.d_past = past_now + 1;
+            *o.adv.d_step = step + 1;
+        }
+    }
+    __syncthreads();
+    if (o.leave_clean) for (int i = tid; i < SW_CLEAR_WORDS; i += 1024) a.ws[i] = 0;
+}
+
+static bool sampler_is_wide(const ptm_sampling& p, int vocab) {
+    return p.temperature >= 1e-6f && (p.top_k <= 0 || p.top_k >= vocab || p.top_k > SAMPLER_MAX_TOPK);
+}
+
 static int sampler_check(const ptm_sampling& p, int vocab) {
     if (vocab <= 0) return PTM_E_SHAPE;
     if (!(p.temperature >= 1e-6f)) return PTM_OK;  // greedy: the other fields are not used
-    if (p.top_k <= 0 || p.top_k >= vocab || p.top_k > SAMPLER_MAX_TOPK) return PTM_E_UNSUPPORTED;
     if (!(p.top_p > 0.0f)) return PTM_E_SHAPE;
     return PTM_OK;
 }
@@ -393,6 +705,28 @@ int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const
     SamplerOut o{out_token, d_uniforms, d_step, counts_rw, adv, ws_kept_clean ? 1 : 0};
     const dim3 grid((vocab + SAMPLER_ELEMS_PER_WG - 1) / SAMPLER_ELEMS_PER_WG);
     if (!ws_kept_clean) hipLaunchKernelGGL(sampler_clear_kernel, dim3(4), dim3(256), 0, s, a.ws);
+    if (sampler_is_wide(host_params, vocab)) {
+        // top-k off, or a top-k beyond the candidate list: passes over the whole vocabulary instead of a gathered list
+        const int use_topk = host_params.top_k > 0 && host_params.top_k < vocab;
+        if (use_topk) {
+            hipLaunchKernelGGL(sampler_hist_kernel<0>, grid, dim3(256), 0, s, a);
+            hipLaunchKernelGGL(sampler_hist_kernel<1>, grid, dim3(256), 0, s, a);
+            hipLaunchKernelGGL(sampler_hist_kernel<2>, grid, dim3(256), 0, s, a);
+        }
+        hipLaunchKernelGGL(sampler_wide_threshold_kernel, dim3(1), dim3(256), 0, s, a, use_topk);
+        hipLaunchKernelGGL(sampler_wide_max_kernel, grid, dim3(256), 0, s, a);
+        hipLaunchKernelGGL(sampler_wide_sumexp_kernel, grid, dim3(256), 0, s, a);
+        if (host_params.top_p < 1.0f) {
+            hipLaunchKernelGGL(sampler_wide_mass_hist_kernel<0>, grid, dim3(256), 0, s, a);
+            hipLaunchKernelGGL(sampler_wide_select_kernel<0>, dim3(1), dim3(256), 0, s, a);
+            hipLaunchKernelGGL(sampler_wide_mass_hist_kernel<1>, grid, dim3(256), 0, s, a);
+            hipLaunchKernelGGL(sampler_wide_select_kernel<1>, dim3(1), dim3(256), 0, s, a);
+            hipLaunchKernelGGL(sampler_wide_mass_hist_kernel<2>, grid, dim3(256), 0, s, a);
+            hipLaunchKernelGGL(sampler_wide_select_kernel<2>, dim3(1), dim3(256), 0, s, a);
+        }
+        hipLaunchKernelGGL(sampler_wide_draw_kernel, dim3(1), dim3(1024), 0, s, a, o);
+        return launch_status();
+    }
     hipLaunchKernelGGL(sampler_hist_kernel<0>, grid, dim3(256), 0, s, a);
     hipLaunchKernelGGL(sampler_hist_kernel<1>, grid, dim3(256), 0, s, a);
     hipLaunchKernelGGL(sampler_hist_kernel<2>, grid, dim3(256), 0, s, a);

@@ -17,6 +17,15 @@ pytestmark = pytest.mark.gpu
 GAP_TOL = 1e-5
 
 
+
+def gap_tol(vocab, temperature, top_k):
+    """Over the whole vocabulary (top-k off) the reference's softmax denominator and running sums are sequential fp32 sums of
+    up to 151 936 terms, which drift from the exact sums by a few 1e-4 relative at that length (measured: the reference's
+    probabilities then add up to 1 +- 3e-4 in float64); the device sums there are order-independent fixed-point ones.  A draw
+    closer than this to an interval edge of the reference's CDF may land on a neighbouring token."""
+    return max(GAP_TOL, 3e-9 * vocab) if wide(vocab, temperature, top_k) else GAP_TOL
+
+
 def cu(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
@@ -31,8 +40,9 @@ def gpu_sample(x, temperature, top_k, top_p, r, counts=None, penalty=1.0):
     return int(out.item())
 
 
-def supported(vocab, temperature, top_k):
-    return temperature < 1e-6 or (1 <= top_k <= 1024 and top_k < vocab)
+def wide(vocab, temperature, top_k):
+    """top-k off or beyond the candidate list: the sampler's passes over the whole vocabulary"""
+    return temperature >= 1e-6 and not (1 <= top_k <= 1024 and top_k < vocab)
 
 
 def test_mt19937_uniforms_are_the_reference_sequence(po):
@@ -49,24 +59,24 @@ def test_sample_token_cases_vs_oracle_and_reference_golden(dev, po, golden_sampl
     for i, (vocab, kind, temperature, top_k, top_p) in enumerate(synth.SAMPLING_CASES):
         x = synth.sampling_logits(i)
         r = rng.uniform01() if temperature >= 1e-6 else 0.0
-        if not supported(vocab, temperature, top_k):
-            with pytest.raises(PtmError) as e:
-                gpu_sample(x, temperature, top_k, top_p, r)
-            assert e.value.code == -4
-            continue
         tok_o, gap = po.sample_token(x, temperature, top_k, top_p, r)
         assert tok_o == int(golden_sampling[i])        # the oracle is the compiled reference here
         tok_g = gpu_sample(x, temperature, top_k, top_p, r)
         print(i, vocab, kind, temperature, top_k, top_p, "r %.6f gap %.2e" % (r, gap), tok_g, tok_o, flush=True)
-        if gap > GAP_TOL:
-            assert tok_g == tok_o, i
+        if gap > gap_tol(vocab, temperature, top_k):
+            assert tok_g == tok_o, (i, wide(vocab, temperature, top_k))
             checked += 1
-    assert checked >= 30
+    assert checked >= 36
 
 
 @pytest.mark.parametrize("vocab,kind_case,temperature,top_k,top_p", [(1000, 0, 0.8, 40, 0.9), (151936, 12, 0.8, 40, 0.9),
                                                                       (151936, 18, 1.0, 1024, 0.95), (1000, 3, 1.3, 7, 1.0),
-                                                                      (151936, 19, 0.5, 2, 0.5)])
+                                                                      (151936, 19, 0.5, 2, 0.5),
+                                                                      # the wide path: top-k off, top-k beyond the list
+                                                                      (1000, 1, 1.0, 0, 1.0), (1000, 6, 0.8, 0, 0.9),
+                                                                      (1000, 9, 0.8, 1000, 0.95), (151936, 18, 0.6, 0, 0.9),
+                                                                      (151936, 12, 0.8, 5000, 0.9), (151936, 16, 1.0, 0, 1.0),
+                                                                      (151936, 12, 2.5, 0, 0.5), (1000, 3, 1.0, 0, 0.7)])
 def test_sample_token_many_draws(dev, po, vocab, kind_case, temperature, top_k, top_p):
     """The whole inverse CDF: 64 draws spread over (0, 1) plus the edges."""
     x = synth.sampling_logits(kind_case)
@@ -74,10 +84,22 @@ def test_sample_token_many_draws(dev, po, vocab, kind_case, temperature, top_k, 
     rs = list(np.random.default_rng(kind_case).random(60).astype(np.float32)) + [0.0, 1e-30, 0.99999994, 0.5]
     checked = 0
     for r in rs:
-        tok_o, gap = po.sample_token(x, temperature, top_k, top_p, float(r))
+        tok_o, gap, probs = po.sample_token(x, temperature, top_k, top_p, float(r), want_probs=True)
         tok_g = gpu_sample(x, temperature, top_k, top_p, float(r))
-        if gap > GAP_TOL or r == 0.0:
+        if gap > gap_tol(vocab, temperature, top_k) or r == 0.0:
             assert tok_g == tok_o, (float(r), gap)
+            checked += 1
+        elif wide(vocab, temperature, top_k):
+            # a flat distribution over 151 936 tokens has intervals narrower than the drift of the reference's own running
+            # sum: the drawn token must then be a kept one whose interval of the reference's distribution holds the draw
+            # to within that drift
+            tol = gap_tol(vocab, temperature, top_k)
+            cdf = np.cumsum(probs)   # fp32, in index order: the sum the reference walks
+            if tok_g == vocab - 1 and r > cdf[-1] - tol:
+                checked += 1   # a running sum that stops short of the draw: the reference's loop then returns the last id
+                continue
+            assert probs[tok_g] > 0 and cdf[tok_g] + tol >= r and (tok_g == 0 or cdf[tok_g - 1] - tol <= r), \
+                (float(r), tok_g, tok_o)
             checked += 1
     assert checked >= 55
 
@@ -121,7 +143,7 @@ def test_sample_token_greedy_ties_and_edges(dev, po):
 
 def test_sample_token_argument_errors(dev):
     x = np.zeros(100, np.float32)
-    for temperature, top_k, top_p in ((0.8, 0, 0.9), (0.8, 100, 0.9), (0.8, 2000, 0.9), (0.8, 40, 0.0)):
+    for temperature, top_k, top_p in ((0.8, 40, 0.0), (0.8, 0, -1.0)):
         with pytest.raises(PtmError):
             gpu_sample(x, temperature, top_k, top_p, 0.5)
 
@@ -134,7 +156,8 @@ def build_tiny(seeds):
 
 
 @pytest.mark.parametrize("use_graph", [True, False])
-@pytest.mark.parametrize("temperature,top_k,top_p,penalty", [(0.8, 40, 0.9, 1.1), (1.2, 8, 1.0, 1.0), (0.0, 40, 0.9, 1.3)])
+@pytest.mark.parametrize("temperature,top_k,top_p,penalty", [(0.8, 40, 0.9, 1.1), (1.2, 8, 1.0, 1.0), (0.0, 40, 0.9, 1.3),
+                                                             (0.9, 0, 0.92, 1.05), (1.1, 0, 1.0, 1.0)])  # top-k off
 def test_decoder_sampled_generation_vs_oracle_loop(dev, po, seeds, use_graph, temperature, top_k, top_p, penalty):
     """The reference's decode loop (api_handlers.h:848-923): penalise with the generated tokens, sample, feed back."""
     from prometorch_amd.decode import Decoder
@@ -176,7 +199,7 @@ def test_decoder_sampling_errors(dev, seeds):
     with pytest.raises(PtmError):
         dec.sample(1, [0.5])                       # no sampling_begin yet
     with pytest.raises(PtmError):
-        dec.sampling_begin(0.8, 0, 0.9)            # top-k off: not on the device
+        dec.sampling_begin(0.8, 40, 0.0)           # top-p must be positive
     dec.sampling_begin(0.8, 40, 0.9)
     with pytest.raises(PtmError):
         dec.sample(1, [0.5] * 33)                  # would overflow the cache
