@@ -373,9 +373,11 @@ static int fd_merge(int head_dim, int n_heads, hipStream_t s, const float* pO, c
 //   * every workgroup normalises/rotates the 4..8 query heads it needs itself (512..1024 values);
 //   * the workgroup whose chunk contains the new position also produces the new K/V row, writes it
 //     to the cache and uses it from LDS (the cache row is not yet visible to its own loads).
-// The split merge stays a second, small launch: doing it in the last-arriving workgroup needs
-// device-scope release/acquire fences in all ~270 workgroups, which measured slower on MI355X
-// (L2 write-back per fence across the 8 XCDs) than the extra launch.
+// The split merge stays a second, small launch.  Doing it in the workgroup of a kv head that arrives last was measured
+// twice on MI355X and lost both times: with device-scope release/acquire fences in all ~270 workgroups (an L2 write-back per
+// fence across the 8 XCDs), and with write-through partial stores, a relaxed device-scope arrival counter and one round of
+// 20 write-through-coherent loads per thread (store acknowledgement + atomic + load round trip behind the slowest workgroup:
+// 1579 against 1568 us per Qwen3-4B token with the second launch).
 // The kernel's cost is instruction latency (about one wave per SIMD, each with a long dependent chain), not the
 // 8.6 MB of KV it reads, so the arithmetic is kept short: hardware exp2 / rsq, no barrier before the final merge.
 // ---------------------------------------------------------------------------------------------

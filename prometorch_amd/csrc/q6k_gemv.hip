@@ -137,12 +137,12 @@ static int q6k_launch_tall_nb(const Q6KArgs& a, int waves, hipStream_t s) {
 }
 template <bool ACC, int LOG2S>
 static int q6k_launch_tall(const Q6KArgs& a, int waves, hipStream_t s) {
-    // blocks in flight per lane group: as many as the registers allow rather than the tightest fit (a padded slot
-    // repeats a load that hits in L1; two blocks in flight leave the memory pipe idle)
-    const int nb = (a.K / 256 + (1 << LOG2S) - 1) >> LOG2S;
-    if (nb <= 2) return q6k_launch_tall_nb<ACC, 2, LOG2S>(a, waves, s);
-    if (nb == 3) return q6k_launch_tall_nb<ACC, 3, LOG2S>(a, waves, s);
-    return q6k_launch_tall_nb<ACC, 5, LOG2S>(a, waves, s);
+    // ONE block in flight per lane group.  The whole launch is resident at once, and a workgroup that requests all of its
+    // blocks up front receives them in one burst, at a time set by its launch order, and only then starts its arithmetic:
+    // the last workgroup served ends a full arithmetic phase behind the end of the stream.  With one block at a time the
+    // requests of all workgroups interleave, every workgroup's arithmetic overlaps the stream, and the other waves of a
+    // SIMD cover a wave's wait (2560 x 9728: 7.5 us against 10.4 with five blocks up front; 2, 3, 4 in flight: 9.6, 9.7, 11.4).
+    return q6k_launch_tall_nb<ACC, 1, LOG2S>(a, waves, s);
 }
 
 // Final argmax over the per-workgroup (value, index) pairs: one workgroup of 1024 threads; every thread issues its
