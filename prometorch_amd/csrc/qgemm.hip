@@ -459,6 +459,8 @@ __device__ __forceinline__ void bytes_to_frags(const uint32_t (&b)[4], float bia
     __builtin_memcpy(&f1, &o[4], 16);
 }
 
+__device__ __forceinline__ void pin4(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
+
 // ---- per-type weight access: what a lane (column n, element half kh) fetches of a 256-wide super-block ----
 struct Q4Tile {  // Q4_K: header + the lane's 16 bytes of each of the 4 groups of 64
     uint4 hdr;
@@ -478,6 +480,14 @@ struct Q4Tile {  // Q4_K: header + the lane's 16 bytes of each of the 4 groups o
         const uint32_t b[4] = {(r.x >> sh) & 0x0f0f0f0fu, (r.y >> sh) & 0x0f0f0f0fu, (r.z >> sh) & 0x0f0f0f0fu,
                                (r.w >> sh) & 0x0f0f0f0fu};
         bytes_to_frags(b, 0.0f, dsc, -dmn, f0, f1);  // (d*sc)*q - dmin*m, the dequantised value (gguf_dequant.h:304-341)
+    }
+    // Nothing computed from these registers may be scheduled above this point: without it the scheduler fills the vector
+    // slots behind the first MFMAs of a block with the scale arithmetic of the block that was requested an instant
+    // before, and every block starts with a wait for its successor's weights.
+    __device__ __forceinline__ void pin() {
+        pin4(hdr);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) pin4(qs[g]);
     }
     static constexpr int kBlockBytes = 144;
     static constexpr bool kQ8Round = true;
@@ -506,6 +516,12 @@ struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh
         const uint32_t pair = scw[s >> 1] >> (16 * (s & 1));            // scales 2s and 2s+1
         const int sv = (int)(int8_t)((kh ? pair >> 8 : pair) & 0xffu);
         bytes_to_frags(b, 32.0f, h2f(d) * (float)sv, 0.0f, f0, f1);     // d*scale*(q-32) (gguf_dequant.h:395-430)
+    }
+    __device__ __forceinline__ void pin() {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) pin4(ql[c]);
+        pin4(qh[0]); pin4(qh[1]); pin4(sc);
+        asm volatile("" : "+v"(d));
     }
     static constexpr int kBlockBytes = 210;
     static constexpr bool kQ8Round = false;
@@ -598,6 +614,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) v
                     x8 = QF_LD(8); x9 = QF_LD(9); x10 = QF_LD(10); x11 = QF_LD(11); x12 = QF_LD(12);
                     x13 = QF_LD(13); x14 = QF_LD(14); x15 = QF_LD(15);
                 }
+                issue_order_fence();  // pieces before weights, as written
 #pragma unroll
                 for (int t = 0; t < NT; ++t) nxt[t].load(wrow[t] + (int64_t)nb * Tile::kBlockBytes, kh);
             }
@@ -610,6 +627,14 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) v
 #undef QF_LD
 #undef QF_ST
             issue_order_fence();  // the fetches stay HERE, two steps ahead of their use (the compiler would sink them to it)
+            // This step's X fragments were read from LDS during the previous step; nothing that consumes them may be hoisted
+            // above this point.  (An MFMA is no memory operation: without this the scheduler moves each MFMA up to right
+            // behind the LDS read of its operand, the fragments share ONE register quad, and every MFMA waits out the
+            // LDS latency of its own operand.)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) asm volatile("" : "+v"(af[ks][mt]));
             // X fragments of the NEXT step are read from LDS now and weight fragments of the next step are prepared
             // while this step's 16 MFMAs (all operands already in registers) run
             h8 an[2][MT];
@@ -623,7 +648,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) v
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 if (s < 7) cur[t].frags(s + 1, kh, bn[t][0], bn[t][1]);
-                else nxt[t].frags(0, kh, bn[t][0], bn[t][1]);
+                else { nxt[t].pin(); nxt[t].frags(0, kh, bn[t][0], bn[t][1]); }
             }
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks)
@@ -632,14 +657,6 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) v
 #pragma unroll
                     for (int t = 0; t < NT; ++t)
                         acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks][mt], bf[t][ks], acc[mt][t], 0, 0, 0);
-            // issue order: one MFMA, then the vector work that fits under it (a 32x32x16 MFMA occupies the matrix pipe
-            // for 32 cycles = 8 vector instructions), so that neither pipe waits for the other
-#pragma unroll
-            for (int i = 0; i < 2 * NT * MT; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
-                __builtin_amdgcn_sched_group_barrier(0x002, 24 / MT, 0);   // VALU
-            }
 #pragma unroll
             for (int t = 0; t < NT; ++t) { bf[t][0] = bn[t][0]; bf[t][1] = bn[t][1]; }
             if (s < 7) {
