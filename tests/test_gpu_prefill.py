@@ -410,6 +410,32 @@ def test_prefill_chunking_does_not_change_the_result(dev, seeds):
         assert outs[3][0] == outs[0][0]
 
 
+def test_reserved_prefill_allocates_nothing_and_changes_nothing(dev, seeds):
+    """ptm_decode_reserve_prefill sizes the row scratch ahead of time: a prefill of at most that many rows then leaves the
+    amount of free device memory untouched (no allocation after set-up), with logits bit-identical to a decoder that allocates
+    on first use; a longer prompt afterwards still works (the scratch grows)."""
+    from prometorch_amd.decode import Decoder
+    from prometorch_amd._lib import check
+    cfg, layers, head = build_tiny(seeds)
+    prompt = [int(t) for t in synth.rng_for(69).integers(0, cfg["vocab"], 40)]
+    plain = Decoder(cfg, layers, head, max_seq=96, kv_fp16=True, use_graph=False)
+    t_plain = plain.prefill(prompt)
+    lg_plain = plain.logits()
+    plain.close()
+    dec = Decoder(cfg, layers, head, max_seq=96, kv_fp16=True, use_graph=False)
+    check(dec.L.ptm_decode_reserve_prefill(dec.h, 48), "reserve_prefill")
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    tok = dec.prefill(prompt)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert tok == t_plain and np.array_equal(bits(dec.logits()), bits(lg_plain))
+    more = [int(t) for t in synth.rng_for(70).integers(0, cfg["vocab"], 50)]
+    dec.prefill(more)                                   # beyond the reservation: allowed, allocates
+    assert dec.L.ptm_decode_reserve_prefill(dec.h, 0) < 0   # a reservation of no rows is an error
+    dec.close()
+
+
 def test_prefill_then_prefill_continues_the_context(dev, po, seeds):
     """Two prefills in a row (a second user turn) equal one prefill of the concatenation."""
     from prometorch_amd.decode import Decoder
