@@ -107,7 +107,7 @@ __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(
 
 // Shape of a tall launch: waves per workgroup and lane groups per row, or waves = 0 when the shape is not one for
 // it.  Rows that fill the chip once at one workgroup per CU: 8 lane groups per row while that needs at most 12 waves
-// (2560 x 9728: 10 waves, 10.25 -> 9.75 us against 4-row tiles), else 4 groups per row and two rows per wave
+// (2560 x 9728: 10 waves), else 4 groups per row and two rows per wave
 // (4096 x 14336: 8 waves of 2 rows).
 struct Q6KTall { int waves, log2S; };
 inline Q6KTall q6k_tall_shape(int N, int K) {
@@ -142,6 +142,10 @@ static int q6k_launch_tall(const Q6KArgs& a, int waves, hipStream_t s) {
     // the last workgroup served ends a full arithmetic phase behind the end of the stream.  With one block at a time the
     // requests of all workgroups interleave, every workgroup's arithmetic overlaps the stream, and the other waves of a
     // SIMD cover a wave's wait (2560 x 9728: 7.5 us against 10.4 with five blocks up front; 2, 3, 4 in flight: 9.6, 9.7, 11.4).
+    // Where a lane group walks many blocks (4096 x 14336: 14 per group, two rows per wave) a second block in flight pays for
+    // itself: 15.8 us against 19.4 with one, 16.5 with three, 17.5 with five.
+    const int nb = (a.K / 256 + (1 << LOG2S) - 1) >> LOG2S;
+    if (nb > 6) return q6k_launch_tall_nb<ACC, 2, LOG2S>(a, waves, s);
     return q6k_launch_tall_nb<ACC, 1, LOG2S>(a, waves, s);
 }
 
