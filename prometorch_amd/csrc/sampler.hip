@@ -41,7 +41,10 @@ enum {
 };
 // wide-path scalars (32-bit words from SW_WIDE): top-k threshold key, largest kept key, sum of exp (64-bit, 2^-32 units),
 // probability mass above the current prefix (64-bit, 2^-40 units), key prefix chosen so far, 1 when every eligible token stays
-enum { WS_THR = 0, WS_MAXKEY = 1, WS_SUMEXP = 2, WS_MASS_ABOVE = 4, WS_PREFIX = 6, WS_KEEP_ALL = 7, WS_TSTAR = 8, WS_NTIE = 9 };
+// the narrow path's hand-over to its overflow kernel: 1 when more candidates tied at the threshold than the list holds, and the
+// threshold key itself (outside the words the wide threshold kernel zeroes)
+enum { WS_THR = 0, WS_MAXKEY = 1, WS_SUMEXP = 2, WS_MASS_ABOVE = 4, WS_PREFIX = 6, WS_KEEP_ALL = 7, WS_TSTAR = 8, WS_NTIE = 9,
+       WS_OVERFLOW = 16, WS_THR_SAVE = 17 };
 
 struct SamplerArgs {
     const float* logits;
@@ -160,6 +163,7 @@ __global__ __launch_bounds__(256) void sampler_gather_kernel(SamplerArgs a) {
     select_bin(a.ws + SW_HIST1, 2048, k, b1, k, s_scan);
     select_bin(a.ws + SW_HIST2, 1024, k, b2, k, s_scan);
     const uint32_t threshold = ((uint32_t)b0 << 21) | ((uint32_t)b1 << 10) | (uint32_t)b2;
+    if (blockIdx.x == 0 && tid == 0) a.ws[SW_WIDE + WS_THR_SAVE] = threshold;   // for the overflow kernel
     const int base = blockIdx.x * SAMPLER_ELEMS_PER_WG;
 #pragma unroll
     for (int u = 0; u < SAMPLER_ELEMS_PER_WG / 256; ++u) {
@@ -193,13 +197,25 @@ __device__ void bitonic_sort_u64(unsigned long long* v, int n) {
 }
 
 struct SamplerOut {
-    int64_t* out_token;       // chosen id (or -1: more than SAMPLER_MAX_CAND logits tie at the threshold)
+    int64_t* out_token;       // chosen id
     const float* uniforms;    // r of step s is uniforms[s]
     const int* d_step;        // NULL: s = 0
     int32_t* counts_rw;       // NULL, or the occurrence counts to bump for the chosen token
     ArgmaxAdvance adv;        // step bookkeeping of the decode loop (all NULL outside it)
     int leave_clean;          // zero the histograms and the candidate count for the next call (it then skips its clear launch)
 };
+
+// what the last thread of a draw does with the chosen id: result, occurrence count, the decode loop's step bookkeeping
+__device__ __forceinline__ void sampler_publish(const SamplerOut& o, int token, int step, int64_t past_now) {
+    if (o.out_token) *o.out_token = token;
+    if (o.counts_rw) o.counts_rw[token] += 1;
+    if (o.adv.d_step) {
+        if (step < o.adv.cap) o.adv.tokens_out[step] = token;
+        *o.adv.d_token = token;
+        *o.adv.d_past = past_now + 1;
+        *o.adv.d_step = step + 1;
+    }
+}
 
 __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, SamplerOut o) {
     __shared__ unsigned long long s_sort[SAMPLER_MAX_CAND];   // 16 KB
@@ -214,8 +230,14 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
     const int step = o.d_step ? *o.d_step : 0;
     const int64_t past_now = o.adv.d_past ? *o.adv.d_past : 0;
     const float r_draw = o.uniforms[step];
-    const bool overflow = total > SAMPLER_MAX_CAND;
-    const int m = overflow ? SAMPLER_MAX_CAND : (int)total;
+    if (total > SAMPLER_MAX_CAND) {
+        // more logits tie at the threshold than the candidate list holds: the kernel behind this one (sampler_overflow_kernel)
+        // draws from the whole vocabulary instead and publishes the token
+        if (tid == 0) a.ws[SW_WIDE + WS_OVERFLOW] = 1u;
+        if (o.leave_clean) for (int i = tid; i < SW_CLEAR_WORDS; i += 1024) a.ws[i] = 0;
+        return;
+    }
+    const int m = (int)total;
     if (m <= 64) {
         // The usual case (k candidates, k <= 64): one wave, one candidate per lane, no workgroup barrier.  Order by
         // counting, sequential sums by reading lane after lane -- the same additions in the same order as below.
@@ -291,6 +313,7 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
                 *o.adv.d_step = step + 1;
             }
             if (o.leave_clean) a.ws[SW_COUNT] = 0;
+            a.ws[SW_WIDE + WS_OVERFLOW] = 0u;
         }
         return;
     }
@@ -346,10 +369,9 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
         }
     }
     if (tid == 0) {
+        a.ws[SW_WIDE + WS_OVERFLOW] = 0u;
         int token;
-        if (overflow) {
-            token = -1;
-        } else if (greedy) {
+        if (greedy) {
             token = (int)s_idx[0];  // every candidate equals the maximum; index order -> the lowest index
         } else {
             const float r = r_draw;
@@ -364,14 +386,7 @@ __global__ __launch_bounds__(1024) void sampler_finish_kernel(SamplerArgs a, Sam
                 }
             }
         }
-        if (o.out_token) *o.out_token = token;
-        if (o.counts_rw && token >= 0) o.counts_rw[token] += 1;
-        if (o.adv.d_step) {
-            if (step < o.adv.cap) o.adv.tokens_out[step] = token;
-            *o.adv.d_token = token < 0 ? 0 : token;
-            *o.adv.d_past = past_now + 1;
-            *o.adv.d_step = step + 1;
-        }
+        sampler_publish(o, token, step, past_now);
     }
     if (o.leave_clean) {  // every thread read the candidate count long before (barriers above)
         for (int i = tid; i < SW_CLEAR_WORDS; i += 1024) a.ws[i] = 0;
@@ -557,7 +572,7 @@ __global__ __launch_bounds__(256) void sampler_wide_select_kernel(SamplerArgs a)
 // Walk 0 counts the tokens of the nucleus' last value per wave (the first WS_NTIE of them in index order stay), walk 1 sums
 // the kept probabilities per wave (the renormalisation of the reference's top-p step), walk 2 finds the first index whose
 // running sum reaches the draw.
-__global__ __launch_bounds__(1024) void sampler_wide_draw_kernel(SamplerArgs a, SamplerOut o) {
+__device__ __forceinline__ void sampler_wide_draw_body(const SamplerArgs& a, const SamplerOut& o) {
     __shared__ uint32_t s_ties[16];
     __shared__ float s_sum[16];
     __shared__ int s_token[16];
@@ -667,17 +682,125 @@ __global__ __launch_bounds__(1024) void sampler_wide_draw_kernel(SamplerArgs a, 
         int token = a.vocab - 1;   // the running sum never reached the draw (rounding): the reference returns the last id
         for (int q = 0; q < 16; ++q) if (s_token[q] != 0x7fffffff) { token = s_token[q]; break; }
         if (r <= 0.0f) token = 0;
-        if (o.out_token) *o.out_token = token;
-        if (o.counts_rw) o.counts_rw[token] += 1;
-        if (o.adv.d_step) {
-            if (step < o.adv.cap) o.adv.tokens_out[step] = token;
-            *o.adv.d_token = token;
-            *o.adv.d_past = past_now + 1;
-            *o.adv.d_step = step + 1;
-        }
+        sampler_publish(o, token, step, past_now);
     }
     __syncthreads();
     if (o.leave_clean) for (int i = tid; i < SW_CLEAR_WORDS; i += 1024) a.ws[i] = 0;
+}
+
+__global__ __launch_bounds__(1024) void sampler_wide_draw_kernel(SamplerArgs a, SamplerOut o) { sampler_wide_draw_body(a, o); }
+
+// Behind the narrow path's finish kernel, always launched, one workgroup: returns at once unless that kernel found more
+// logits tied at the top-k threshold than its candidate list holds (a flat or constant stretch of logits at the cut: the
+// reference keeps every tie, gguf_model.h:7682-7691).  Then it does what the wide path does for a large top-k -- largest
+// kept value, fixed-point softmax denominator, the nucleus' last value by a three-level walk over per-key-bin mass -- with
+// loops of this one workgroup over the vocabulary (a rare case: no launch-level parallelism spent on it), and ends in the
+// wide path's draw.  Greedy (k = 1 with the maximum tied that often): the lowest index among the maxima, as argmax gives.
+__global__ __launch_bounds__(1024) void sampler_overflow_kernel(SamplerArgs a, SamplerOut o) {
+    uint32_t* w = a.ws + SW_WIDE;
+    if (w[WS_OVERFLOW] == 0u) return;
+    __shared__ unsigned long long s_hist[2048];
+    __shared__ unsigned long long s_red64[16];
+    __shared__ uint32_t s_red32[16];
+    __shared__ uint32_t s_sel[2];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const ptm_sampling p = sampler_params(a);
+    const uint32_t thr = w[WS_THR_SAVE];
+    // largest kept key (and, for greedy, the lowest index that holds it)
+    uint32_t best = 0;
+    for (int i = tid; i < a.vocab; i += 1024) {
+        const uint32_t key = order_key(sampler_value(a, p, i));
+        if (key >= thr && key > best) best = key;
+    }
+    for (int off = 32; off > 0; off >>= 1) best = max(best, (uint32_t)__shfl_down(best, off, 64));
+    if (lane == 0) s_red32[wave] = best;
+    __syncthreads();
+    uint32_t mxkey = 0;
+    for (int q = 0; q < 16; ++q) mxkey = max(mxkey, s_red32[q]);
+    __syncthreads();
+    if (!(p.temperature >= 1e-6f)) {
+        uint32_t first = 0xffffffffu;
+        for (int i = tid; i < a.vocab; i += 1024)
+            if (order_key(sampler_value(a, p, i)) == mxkey) { first = (uint32_t)i; break; }
+        for (int off = 32; off > 0; off >>= 1) first = min(first, (uint32_t)__shfl_down(first, off, 64));
+        if (lane == 0) s_red32[wave] = first;
+        __syncthreads();
+        if (tid == 0) {
+            for (int q = 1; q < 16; ++q) first = min(first, s_red32[q]);
+            w[WS_OVERFLOW] = 0u;
+            sampler_publish(o, (int)first, o.d_step ? *o.d_step : 0, o.adv.d_past ? *o.adv.d_past : 0);
+        }
+        return;
+    }
+    const float mx = key_value(mxkey);
+    unsigned long long acc = 0;
+    for (int i = tid; i < a.vocab; i += 1024) {
+        const float x = sampler_value(a, p, i);
+        if (order_key(x) >= thr) acc += (unsigned long long)(expf(x - mx) * 4294967296.0f);
+    }
+    for (int off = 32; off > 0; off >>= 1) acc += shfl_down_u64(acc, off);
+    if (lane == 0) s_red64[wave] = acc;
+    __syncthreads();
+    unsigned long long sumexp = 0;
+    for (int q = 0; q < 16; ++q) sumexp += s_red64[q];
+    const float inv = 1.0f / ((float)sumexp * 2.3283064365386963e-10f);
+    uint32_t keep_all = 0, prefix = 0, ntie = 0;
+    if (p.top_p < 1.0f) {
+        const unsigned long long target = (unsigned long long)((double)p.top_p * 1099511627776.0);
+        unsigned long long above = 0;
+        for (int level = 0; level < 3 && !keep_all; ++level) {
+            const int nb = level == 2 ? 1024 : 2048;
+            __syncthreads();
+            for (int i = tid; i < nb; i += 1024) s_hist[i] = 0;
+            __syncthreads();
+            for (int i = tid; i < a.vocab; i += 1024) {
+                const float x = sampler_value(a, p, i);
+                const uint32_t key = order_key(x);
+                if (key < thr) continue;
+                const float pr = wide_prob(x, mx, inv);
+                if (!(pr > 1e-10f)) continue;
+                int bin;
+                if (level == 0) bin = (int)(key >> 21);
+                else if (level == 1) { if ((key >> 21) != prefix) continue; bin = (int)((key >> 10) & 0x7ffu); }
+                else { if ((key >> 10) != prefix) continue; bin = (int)(key & 0x3ffu); }
+                atomicAdd(&s_hist[bin], wide_mass(pr));
+            }
+            __syncthreads();
+            if (tid == 0) {   // from the top: the bin in which the accumulated mass reaches top_p
+                unsigned long long run = above;
+                uint32_t found = 0, bin = 0;
+                for (int b = nb - 1; b >= 0; --b) {
+                    if (run + s_hist[b] >= target) { found = 1; bin = (uint32_t)b; break; }
+                    run += s_hist[b];
+                }
+                s_sel[0] = found;
+                s_sel[1] = bin;
+                s_red64[0] = run;
+            }
+            __syncthreads();
+            if (!s_sel[0]) { keep_all = 1; break; }   // the eligible tokens together do not reach top_p: all of them stay
+            above = s_red64[0];
+            prefix = level == 0 ? s_sel[1] : level == 1 ? ((prefix << 11) | s_sel[1]) : ((prefix << 10) | s_sel[1]);
+        }
+        if (!keep_all) {
+            const unsigned long long pf = wide_mass(wide_prob(key_value(prefix), mx, inv));
+            const unsigned long long n = pf ? (target - above + pf - 1) / pf : 1;
+            ntie = (uint32_t)(n < 1 ? 1 : (n > 0xffffffffull ? 0xffffffffull : n));
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        w[WS_THR] = thr;
+        w[WS_MAXKEY] = mxkey;
+        *reinterpret_cast<unsigned long long*>(w + WS_SUMEXP) = sumexp;
+        w[WS_KEEP_ALL] = keep_all;
+        w[WS_TSTAR] = prefix;
+        w[WS_NTIE] = ntie;
+        w[WS_OVERFLOW] = 0u;
+    }
+    __threadfence_block();
+    __syncthreads();
+    sampler_wide_draw_body(a, o);
 }
 
 static bool sampler_is_wide(const ptm_sampling& p, int vocab) {
@@ -732,6 +855,7 @@ int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const
     hipLaunchKernelGGL(sampler_hist_kernel<2>, grid, dim3(256), 0, s, a);
     hipLaunchKernelGGL(sampler_gather_kernel, grid, dim3(256), 0, s, a);
     hipLaunchKernelGGL(sampler_finish_kernel, dim3(1), dim3(1024), 0, s, a, o);
+    hipLaunchKernelGGL(sampler_overflow_kernel, dim3(1), dim3(1024), 0, s, a, o);   // returns at once in the usual case
     return launch_status();
 }
 

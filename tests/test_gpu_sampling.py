@@ -40,6 +40,20 @@ def gpu_sample(x, temperature, top_k, top_p, r, counts=None, penalty=1.0):
     return int(out.item())
 
 
+def check_wide_draw(tok_g, tok_o, gap, probs, r, tol, vocab):
+    """The bar of the whole-vocabulary path: the reference's token when the draw is clear of its interval's edges, otherwise a
+    kept token whose interval of the reference's CDF (fp32, index order: the sum the reference walks) holds the draw to within
+    tol.  Where the reference's running sum stops short of the draw its loop returns the last id; the device's sum may reach
+    the draw there, and the other way round."""
+    cdf = np.cumsum(probs)
+    fell_off = cdf[-1] < r
+    if (gap > tol and not fell_off) or r == 0.0:
+        assert tok_g == tok_o, (float(r), gap)
+        return
+    assert (tok_g == vocab - 1 and r > cdf[-1] - tol) or \
+        (probs[tok_g] > 0 and cdf[tok_g] + tol >= r and (tok_g == 0 or cdf[tok_g - 1] - tol <= r)), (float(r), tok_g, tok_o)
+
+
 def wide(vocab, temperature, top_k):
     """top-k off or beyond the candidate list: the sampler's passes over the whole vocabulary"""
     return temperature >= 1e-6 and not (1 <= top_k <= 1024 and top_k < vocab)
@@ -86,20 +100,12 @@ def test_sample_token_many_draws(dev, po, vocab, kind_case, temperature, top_k, 
     for r in rs:
         tok_o, gap, probs = po.sample_token(x, temperature, top_k, top_p, float(r), want_probs=True)
         tok_g = gpu_sample(x, temperature, top_k, top_p, float(r))
-        if gap > gap_tol(vocab, temperature, top_k) or r == 0.0:
-            assert tok_g == tok_o, (float(r), gap)
+        if wide(vocab, temperature, top_k):
+            # a flat distribution over 151 936 tokens has intervals narrower than the drift of the reference's own running sum
+            check_wide_draw(tok_g, tok_o, gap, probs, r, gap_tol(vocab, temperature, top_k), vocab)
             checked += 1
-        elif wide(vocab, temperature, top_k):
-            # a flat distribution over 151 936 tokens has intervals narrower than the drift of the reference's own running
-            # sum: the drawn token must then be a kept one whose interval of the reference's distribution holds the draw
-            # to within that drift
-            tol = gap_tol(vocab, temperature, top_k)
-            cdf = np.cumsum(probs)   # fp32, in index order: the sum the reference walks
-            if tok_g == vocab - 1 and r > cdf[-1] - tol:
-                checked += 1   # a running sum that stops short of the draw: the reference's loop then returns the last id
-                continue
-            assert probs[tok_g] > 0 and cdf[tok_g] + tol >= r and (tok_g == 0 or cdf[tok_g - 1] - tol <= r), \
-                (float(r), tok_g, tok_o)
+        elif gap > GAP_TOL or r == 0.0:
+            assert tok_g == tok_o, (float(r), gap)
             checked += 1
     assert checked >= 55
 
@@ -135,10 +141,36 @@ def test_sample_token_greedy_ties_and_edges(dev, po):
     tok_o, _ = po.sample_token(x, 1.0, 2, 1.0, 0.5)
     assert gpu_sample(x, 1.0, 2, 1.0, 0.5) == tok_o
     flat = np.zeros(5000, np.float32)                                 # 5000 logits tie at the threshold: more than the list holds
-    assert gpu_sample(flat, 1.0, 4, 1.0, 0.5) == -1
+    tok_o, _ = po.sample_token(flat, 1.0, 4, 1.0, 0.5)                # the reference keeps every tie: uniform over all 5000
+    assert gpu_sample(flat, 1.0, 4, 1.0, 0.5) == tok_o
+    assert gpu_sample(flat, 0.0, 1, 1.0, 0.5) == 0                    # greedy over 5000 equal maxima: the lowest index
     flat2 = np.zeros(2048, np.float32)                                # exactly as many as it holds
     tok_o, _ = po.sample_token(flat2, 1.0, 4, 1.0, 0.5)
     assert gpu_sample(flat2, 1.0, 4, 1.0, 0.5) == tok_o
+
+
+@pytest.mark.parametrize("top_k,top_p", [(40, 1.0), (40, 0.9), (300, 0.5), (1, 1.0)])
+def test_more_ties_at_the_threshold_than_the_candidate_list_holds(dev, po, top_k, top_p):
+    """A plateau of 3000 equal logits at the top-k cut (above it a few larger ones, below it the rest): the reference keeps every
+    tie (gguf_model.h:7682-7691), so more than 2048 candidates survive and the draw comes from the overflow kernel, which walks
+    the whole vocabulary; the bar is the wide path's (order-independent sums)."""
+    rng = np.random.default_rng(91)
+    vocab = 20000
+    x = (rng.standard_normal(vocab) * 0.5 - 3.0).astype(np.float32)
+    plateau = rng.choice(vocab, 3000, replace=False)
+    x[plateau] = 1.25
+    x[plateau[:7]] = np.array([3.0, 2.5, 2.5, 2.0, 1.75, 1.5, 1.5], np.float32)   # 7 above the plateau: k = 40 cuts inside it
+    tol = max(GAP_TOL, 3e-9 * vocab)
+    checked = 0
+    for r in list(rng.random(24).astype(np.float32)) + [0.0, 0.99999994]:
+        tok_o, gap, probs = po.sample_token(x, 0.9, top_k, top_p, float(r), want_probs=True)
+        tok_g = gpu_sample(x, 0.9, top_k, top_p, float(r))
+        if top_k == 1:
+            assert tok_g == tok_o          # one maximum, no tie at k = 1: the narrow path
+            continue
+        check_wide_draw(tok_g, tok_o, gap, probs, r, tol, vocab)
+        checked += 1
+    assert top_k == 1 or checked >= 20
 
 
 def test_sample_token_argument_errors(dev):
