@@ -46,6 +46,9 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
                    int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, bool reuse_rows,
                    hipStream_t s);
 int qgemm_f16_splits(int N, int K, int M);
+size_t qgemm_f16_multi_split_bytes(int n, const int* N, const uint32_t* types, int K, int M);
+int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const int64_t* strides, const int* N, float* const* Y,
+                    int M, int K, void* ws_round, void* ws_plain, float* split_ws, size_t split_ws_bytes, hipStream_t s);
 int qgemm_f16_prepare_fused(int pre, const float* X, const float* X2, float eps, int add_one, void* ws_round, void* ws_plain,
                             int M, int K, hipStream_t s);
 int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
@@ -297,6 +300,15 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
         }
     }
     d->pf_split_bytes = 4 * split_elems;
+    for (int li = 0; li < c.n_layers; ++li) {  // q, k, v share one launch whose splits depend on the types, which vary by layer
+        const ptm_layer& L = d->layers[li];
+        const int N3[3] = {L.q.rows, L.k.rows, L.v.rows};
+        const uint32_t t3[3] = {L.q.ggml_type, L.k.ggml_type, L.v.ggml_type};
+        for (const int m : {128, 256, rows}) {
+            const size_t b = qgemm_f16_multi_split_bytes(3, N3, t3, (int)H, m < rows ? m : rows);
+            d->pf_split_bytes = b > d->pf_split_bytes ? b : d->pf_split_bytes;
+        }
+    }
     const size_t o_split = take(d->pf_split_bytes);
     const int rc = hip_status(hipMalloc(&d->pf_slab, off));
     if (rc != PTM_OK) return rc;
@@ -339,9 +351,14 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
         PTM_TRY(qgemm_f16_prepare_fused(1, d->pf_x, L.attn_norm, c.rms_eps, 0,
                                         uses(PTM_TYPE_Q4_K, {&L.q, &L.k, &L.v}) ? d->pf_ws : nullptr,
                                         uses(PTM_TYPE_Q6_K, {&L.q, &L.k, &L.v}) ? d->pf_ws2 : nullptr, M, H, s));
-        PTM_TRY(gemm(L.q, d->pf_x, d->pf_q, false, true));
-        PTM_TRY(gemm(L.k, d->pf_x, d->pf_k, false, true));
-        PTM_TRY(gemm(L.v, d->pf_x, d->pf_v, false, true));
+        {  // q, k, v in one launch
+            const uint32_t t3[3] = {L.q.ggml_type, L.k.ggml_type, L.v.ggml_type};
+            const void* W3[3] = {L.q.data, L.k.data, L.v.data};
+            const int64_t s3[3] = {L.q.row_stride_bytes, L.k.row_stride_bytes, L.v.row_stride_bytes};
+            const int N3[3] = {L.q.rows, L.k.rows, L.v.rows};
+            float* Y3[3] = {d->pf_q, d->pf_k, d->pf_v};
+            PTM_TRY(qgemm_f16_multi(3, t3, W3, s3, N3, Y3, M, H, d->pf_ws, d->pf_ws2, d->pf_split, d->pf_split_bytes, s));
+        }
         if (L.q_bias) PTM_TRY(ptm_add_qkv_bias(d->pf_q, d->pf_k, d->pf_v, L.q_bias, L.k_bias, L.v_bias, M, qd, kvd, s));
         PTM_TRY(ptm_qknorm_rope_kvwrite_rows(d->pf_q, d->pf_k, d->pf_v, L.q_norm, L.k_norm, L.k_cache, L.v_cache,
                                              local ? d->rope_swa : d->rope, M,

@@ -535,10 +535,12 @@ struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh
 // own one 32-column tile each of the same 64 columns, so a SIMD holds two waves and one's dequantisation and LDS reads
 // run under the other's MFMAs (the two pipes of a single wave barely overlap); no weight is dequantised twice, the X
 // tile in LDS is read by twice as many waves.
-template <typename Tile, int MT, int WAVES = 4>
-__global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
-                                                        const float* __restrict__ rowscale, float* Y, int M, int K, int N,
-                                                        int accumulate, int blocks_per_split, float* partials) {
+// (bx, by, bz) = (column tile, row tile, K split) of this workgroup; s_a = its dynamic LDS
+template <typename Tile, int MT, int WAVES>
+__device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride, const _Float16* Xh,
+                                               const float* __restrict__ rowscale, float* Y, int M, int K, int N,
+                                               int accumulate, int blocks_per_split, float* partials, int bx, int by, int bz,
+                                               uint8_t* s_a) {
     // W and Xh are deliberately not __restrict__: loads through a restrict pointer may be moved across the
     // compiler fences below, and the prefetch distance of this loop depends on those fences
     constexpr int TM = 32 * MT;                     // rows of X per workgroup (MT tiles of 32)
@@ -546,13 +548,12 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) v
     constexpr int RS = 2 * WAVES;                   // rows of the X tile that one fetch instruction of the workgroup covers
     constexpr int NPIECE = TM / RS;                 // 16-byte pieces of the X tile per thread
     static_assert(WAVES == 4 || (WAVES == 8 && MT == 4), "wave layouts");
-    extern __shared__ __align__(16) uint8_t s_a[];  // [2][TM * QF_PITCH]
-    const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3;
+    const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3;  // s_a: [2][TM * QF_PITCH]
     const int j = lane & 31, kh = lane >> 5;
-    const int m0 = blockIdx.y * TM;
-    const int n_base = blockIdx.x * QF_TN + wave * 64 + (WAVES == 8 ? 32 * (tid >> 8) : 0);
+    const int m0 = by * TM;
+    const int n_base = bx * QF_TN + wave * 64 + (WAVES == 8 ? 32 * (tid >> 8) : 0);
     // split K: workgroup z of the grid sums super-blocks [blk0, blk0 + nblk) into its own M x N partial
-    const int blk0 = blockIdx.z * blocks_per_split;
+    const int blk0 = bz * blocks_per_split;
     const int nblk = min(K / 256 - blk0, blocks_per_split);
     const uint8_t* wrow[NT];
 #pragma unroll
@@ -576,13 +577,30 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) v
     // the 16 pieces of the next tile in flight (scalars, not an array: they must stay in registers)
     static_assert(MT == 1 || MT == 2 || MT == 4, "row tiles per workgroup");
     uint4 x0, x1, x2, x3, x4, x5, x6, x7, x8, x9, x10, x11, x12, x13, x14, x15;
-    // prologue: tile of block 0 -> LDS buffer 0, weights of block 0, fragments of step 0
-#pragma unroll
-    for (int p = 0; p < NPIECE; ++p)
-        *reinterpret_cast<uint4*>(x_dst + RS * p * QF_PITCH) = *reinterpret_cast<const uint4*>(x_src + RS * p * x_row_bytes);
+    // prologue: tile of block 0 -> LDS buffer 0, weights of block 0, fragments of step 0.  The weight loads go out behind
+    // the tile's, before anything waits: one memory round trip for both, not two (a launch of two or three blocks per
+    // workgroup, as the K splits of the narrow projections are, is mostly this prologue)
+#define QF_LD0(p) (*reinterpret_cast<const uint4*>(x_src + RS * (p) * x_row_bytes))
+#define QF_ST0(p, v) (*reinterpret_cast<uint4*>(x_dst + RS * (p) * QF_PITCH) = (v))
+    x0 = QF_LD0(0); x1 = QF_LD0(1); x2 = QF_LD0(2); x3 = QF_LD0(3);
+    if constexpr (NPIECE >= 8) { x4 = QF_LD0(4); x5 = QF_LD0(5); x6 = QF_LD0(6); x7 = QF_LD0(7); }
+    if constexpr (NPIECE >= 16) {
+        x8 = QF_LD0(8); x9 = QF_LD0(9); x10 = QF_LD0(10); x11 = QF_LD0(11); x12 = QF_LD0(12);
+        x13 = QF_LD0(13); x14 = QF_LD0(14); x15 = QF_LD0(15);
+    }
+    issue_order_fence();
     Tile cur[NT], nxt[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) cur[t].load(wrow[t], kh);
+    issue_order_fence();
+    QF_ST0(0, x0); QF_ST0(1, x1); QF_ST0(2, x2); QF_ST0(3, x3);
+    if constexpr (NPIECE >= 8) { QF_ST0(4, x4); QF_ST0(5, x5); QF_ST0(6, x6); QF_ST0(7, x7); }
+    if constexpr (NPIECE >= 16) {
+        QF_ST0(8, x8); QF_ST0(9, x9); QF_ST0(10, x10); QF_ST0(11, x11); QF_ST0(12, x12);
+        QF_ST0(13, x13); QF_ST0(14, x14); QF_ST0(15, x15);
+    }
+#undef QF_LD0
+#undef QF_ST0
     h8 bf[NT][2], bn[NT][2];
 #pragma unroll
     for (int t = 0; t < NT; ++t) cur[t].frags(0, kh, bf[t][0], bf[t][1]);
@@ -670,29 +688,92 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) v
         for (int t = 0; t < NT; ++t) cur[t] = nxt[t];
         __syncthreads();  // next tile complete, this tile no longer read
     }
-    // C layout of the 32x32 tile: column j = lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4
+    // C layout of the 32x32 tile: column j = lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4.
+    // Every load of the epilogue is issued before the first store: a load behind a store to memory the compiler cannot tell
+    // apart waits for it, and 16 MT row scales (plus as many old values of Y when accumulating) fetched one by one between the
+    // stores are as many serial memory round trips, more than the main loop of a launch with few blocks per workgroup takes.
+    // (rowscale holds an entry for every padded row; rows >= M are never stored.)
+    float rsv[MT][16];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-            if (m < M) {
-                const float rs = rowscale[m];
+        for (int r = 0; r < 16; ++r) rsv[mt][r] = rowscale[m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3)];
 #pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const int n = n_base + 32 * t + j;
-                    if (n < N) {
-                        const float v = acc[mt][t][r] * rs;
-                        if (partials) {
-                            partials[((int64_t)blockIdx.z * M + m) * N + n] = v;
-                        } else {
-                            float* y = Y + (int64_t)m * N + n;
-                            *y = accumulate ? *y + v : v;
-                        }
-                    }
+    for (int t = 0; t < NT; ++t) {
+        const int n = n_base + 32 * t + j;
+        const bool n_ok = n < N;
+        const int nc = n_ok ? n : N - 1;
+        if (partials) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+                    if (m < M && n_ok) partials[((int64_t)bz * M + m) * N + n] = acc[mt][t][r] * rsv[mt][r];
+                }
+        } else if (accumulate) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                float old[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = min(m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3), M - 1);
+                    old[r] = Y[(int64_t)m * N + nc];
+                }
+                issue_order_fence();
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+                    if (m < M && n_ok) Y[(int64_t)m * N + n] = old[r] + acc[mt][t][r] * rsv[mt][r];
                 }
             }
+        } else {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+                    if (m < M && n_ok) Y[(int64_t)m * N + n] = acc[mt][t][r] * rsv[mt][r];
+                }
         }
+    }
+}
+
+template <typename Tile, int MT, int WAVES = 4>
+__global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
+                                                        const float* __restrict__ rowscale, float* Y, int M, int K, int N,
+                                                        int accumulate, int blocks_per_split, float* partials) {
+    extern __shared__ __align__(16) uint8_t qf_lds[];
+    qgemm_f16_body<Tile, MT, WAVES>(W, stride, Xh, rowscale, Y, M, K, N, accumulate, blocks_per_split, partials, blockIdx.x,
+                                    blockIdx.y, blockIdx.z, qf_lds);
+}
+
+// Up to three projections of the same rows in ONE launch of the eight-wave 128-row tile (q, k, v of a layer: in a Q4_K_M
+// file two Q4_K matrices and a Q6_K one).  Each matrix brings its own prepared rows (Q8-rounded for Q4_K, plain for
+// Q6_K), column tiles and K splits; blockIdx.x walks the (column tile, split) slots of the matrices one after the other.
+// Three narrow launches of two or three blocks per workgroup are mostly launch, prologue and epilogue; one launch pays
+// them once and fills the chip.
+struct QfMat {
+    const uint8_t* W;
+    int64_t stride;
+    const _Float16* Xh;
+    const float* rowscale;
+    float* Y;
+    float* partials;  // NULL: one split, written to Y
+    int N, bps, ntiles, slot_end, q6;
+};
+struct QfMulti { QfMat m[3]; int n_mat; };
+
+__global__ __launch_bounds__(512, 1) void qgemm_f16_multi_kernel(const QfMulti a, int M, int K) {
+    extern __shared__ __align__(16) uint8_t qf_lds[];
+    int i = 0;
+    if (a.n_mat > 1 && (int)blockIdx.x >= a.m[0].slot_end) i = 1;
+    if (a.n_mat > 2 && (int)blockIdx.x >= a.m[1].slot_end) i = 2;
+    const QfMat& q = i == 0 ? a.m[0] : (i == 1 ? a.m[1] : a.m[2]);
+    const int local = (int)blockIdx.x - (i == 0 ? 0 : (i == 1 ? a.m[0].slot_end : a.m[1].slot_end));
+    const int bx = local % q.ntiles, bz = local / q.ntiles;
+    if (q.q6) qgemm_f16_body<Q6Tile, 4, 8>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, blockIdx.y, bz, qf_lds);
+    else qgemm_f16_body<Q4Tile, 4, 8>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, blockIdx.y, bz, qf_lds);
 }
 
 // Y (+)= partials[0] + partials[1] + ... in that fixed order (deterministic, unlike atomics)
@@ -718,6 +799,33 @@ __global__ __launch_bounds__(256) void qgemm_split_reduce_kernel(const float* __
     }
 }
 
+// the same for the matrices of a multi-matrix launch: blockIdx.x walks the segments' 1024-element pieces
+struct QfRedSeg { const float* P; float* Y; int64_t total; int splits, blk_end; };
+struct QfRedMulti { QfRedSeg s[3]; int n; };
+__global__ __launch_bounds__(256) void qgemm_split_reduce_multi_kernel(const QfRedMulti a) {
+    int k = 0;
+    if (a.n > 1 && (int)blockIdx.x >= a.s[0].blk_end) k = 1;
+    if (a.n > 2 && (int)blockIdx.x >= a.s[1].blk_end) k = 2;
+    const QfRedSeg& g = k == 0 ? a.s[0] : (k == 1 ? a.s[1] : a.s[2]);
+    const int b = (int)blockIdx.x - (k == 0 ? 0 : (k == 1 ? a.s[0].blk_end : a.s[1].blk_end));
+    const int64_t i = ((int64_t)b * 256 + threadIdx.x) * 4;
+    if (i >= g.total) return;
+    if (i + 4 <= g.total && (g.total & 3) == 0) {
+        float4 v = *reinterpret_cast<const float4*>(g.P + i);
+        for (int z = 1; z < g.splits; ++z) {
+            const float4 w = *reinterpret_cast<const float4*>(g.P + z * g.total + i);
+            v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+        }
+        *reinterpret_cast<float4*>(g.Y + i) = v;
+    } else {
+        for (int64_t e = i; e < g.total && e < i + 4; ++e) {
+            float v = g.P[e];
+            for (int z = 1; z < g.splits; ++z) v += g.P[z * g.total + e];
+            g.Y[e] = v;
+        }
+    }
+}
+
 // K splits for an N x K weight matrix and M rows: enough workgroups to fill the chip when N alone gives few column
 // tiles (a 2560-wide projection is 10 tiles).  M enters only through its class (up to 128 rows, up to 256, more), so
 // that the summation order of a row does not change with how many rows share the launch within a class; short
@@ -730,6 +838,35 @@ int qgemm_f16_splits(int N, int K, int M) {
     s = s > cap ? cap : s;
     s = s > nblk / 2 ? nblk / 2 : s;
     return s < 1 ? 1 : s;
+}
+
+// K splits of the matrices of a multi-matrix launch.  All (column tile, split) slots of all matrices must fit one round of
+// the chip (256 workgroups over the row tiles of M's class, as above), and the launch lasts as long as its slowest
+// workgroup: starting from one split each, the matrix whose workgroups have the most work (blocks per split, a Q6_K block
+// weighing 1.6 Q4_K blocks: measured 8 against 5 us) gets its next split count until the slots run out.  A function of
+// the shapes, the types and M's class only, like qgemm_f16_splits.
+void qgemm_f16_multi_plan(int n, const int* N, const uint32_t* types, int K, int M, int* splits) {
+    const int nblk = K / 256;
+    const int row_tiles = M <= 128 ? 1 : (M <= 256 ? 2 : 4);
+    const int budget = 256 / row_tiles;
+    const int cap = (row_tiles == 1 ? 16 : 8) < nblk / 2 ? (row_tiles == 1 ? 16 : 8) : (nblk / 2 < 1 ? 1 : nblk / 2);
+    int ntile[3], slots = 0;
+    for (int i = 0; i < n; ++i) { splits[i] = 1; ntile[i] = (N[i] + QF_TN - 1) / QF_TN; slots += ntile[i]; }
+    for (;;) {
+        int j = -1;
+        float worst = 0.0f;
+        for (int i = 0; i < n; ++i) {
+            const float est = (float)((nblk + splits[i] - 1) / splits[i]) * (types[i] == PTM_TYPE_Q6_K ? 1.6f : 1.0f);
+            if (est > worst) { worst = est; j = i; }
+        }
+        if (j < 0) break;
+        const int bps = (nblk + splits[j] - 1) / splits[j];
+        if (bps <= 1) break;
+        const int next = (nblk + bps - 2) / (bps - 1);  // the fewest splits with fewer blocks each
+        if (next > cap || slots + ntile[j] * (next - splits[j]) > budget) break;
+        slots += ntile[j] * (next - splits[j]);
+        splits[j] = next;
+    }
 }
 
 // Rows per workgroup in tiles of 32: 4 (128 rows: each dequantised weight serves twice as many products) unless that
@@ -815,6 +952,80 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
         hipLaunchKernelGGL(qgemm_split_reduce_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, partials, splits,
                            Y, total, acc);
     }
+    return launch_status();
+}
+
+// Y[i] = X . W[i]^T for up to three Q4_K / Q6_K matrices over the same K whose rows are already prepared (ws_round for the
+// Q4_K ones, ws_plain for the Q6_K ones, as qgemm_f16_prepare_fused leaves them), in one launch plus one reduction.
+size_t qgemm_f16_multi_split_bytes(int n, const int* N, const uint32_t* types, int K, int M) {
+    int sp[3];
+    qgemm_f16_multi_plan(n, N, types, K, M, sp);
+    size_t e = 0;
+    for (int i = 0; i < n; ++i) if (sp[i] > 1) e += (size_t)sp[i] * M * N[i];
+    return 4 * e;
+}
+
+int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const int64_t* strides, const int* N, float* const* Y,
+                    int M, int K, void* ws_round, void* ws_plain, float* split_ws, size_t split_ws_bytes, hipStream_t s) {
+    if (n < 1 || n > 3) return PTM_E_SHAPE;
+    if (M <= 0 || K <= 0 || (K % 256) != 0) return PTM_E_SHAPE;
+    const int mp = qf_mpad(M);
+    if (mp / 128 > 65535) return PTM_E_UNSUPPORTED;
+    if (qgemm_f16_multi_split_bytes(n, N, types, K, M) > split_ws_bytes || !split_ws) return PTM_E_SHAPE;
+    int sp[3];
+    qgemm_f16_multi_plan(n, N, types, K, M, sp);
+    const int nblk = K / 256;
+    QfMulti a{};
+    QfRedMulti r{};
+    a.n_mat = n;
+    int slots = 0, red_blocks = 0;
+    float* part = split_ws;
+    // the Q6_K matrices first: their workgroups take longest and should be the first ones placed
+    int order[3], k = 0;
+    for (int i = 0; i < n; ++i) if (types[i] == PTM_TYPE_Q6_K) order[k++] = i;
+    for (int i = 0; i < n; ++i) if (types[i] != PTM_TYPE_Q6_K) order[k++] = i;
+    for (int o = 0; o < n; ++o) {
+        const int i = order[o];
+        const bool q6 = types[i] == PTM_TYPE_Q6_K;
+        if (!q6 && types[i] != PTM_TYPE_Q4_K) return PTM_E_UNSUPPORTED;
+        void* ws = q6 ? ws_plain : ws_round;
+        if (!W[i] || !Y[i] || !ws) return PTM_E_NULL;
+        if (N[i] <= 0 || strides[i] < (int64_t)nblk * (q6 ? 210 : 144)) return PTM_E_SHAPE;
+        if (q6 ? ((strides[i] & 1) || (reinterpret_cast<uintptr_t>(W[i]) & 1u)) : (!aligned16(W[i]) || (strides[i] & 15))) return PTM_E_ALIGN;
+        if (!aligned16(ws) || (reinterpret_cast<uintptr_t>(Y[i]) & 15u)) return PTM_E_ALIGN;
+        QfMat& m = a.m[o];
+        m.W = static_cast<const uint8_t*>(W[i]);
+        m.stride = strides[i];
+        m.Xh = static_cast<const _Float16*>(ws);
+        m.rowscale = reinterpret_cast<const float*>(m.Xh + (int64_t)mp * K);
+        m.Y = Y[i];
+        m.N = N[i];
+        m.bps = (nblk + sp[i] - 1) / sp[i];
+        const int splits = (nblk + m.bps - 1) / m.bps;  // no empty split
+        m.ntiles = (N[i] + QF_TN - 1) / QF_TN;
+        m.q6 = q6 ? 1 : 0;
+        m.partials = splits > 1 ? part : nullptr;
+        slots += m.ntiles * splits;
+        m.slot_end = slots;
+        if (splits > 1) {
+            QfRedSeg& g = r.s[r.n++];
+            g.P = part;
+            g.Y = Y[i];
+            g.total = (int64_t)M * N[i];
+            g.splits = splits;
+            red_blocks += (int)((g.total + 1023) / 1024);
+            g.blk_end = red_blocks;
+            part += (size_t)splits * M * N[i];
+        }
+    }
+    static bool raised = false;
+    if (!raised) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_multi_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  2 * 128 * QF_PITCH);
+        raised = true;
+    }
+    hipLaunchKernelGGL(qgemm_f16_multi_kernel, dim3(slots, (M + 127) / 128), dim3(512), 2 * (size_t)128 * QF_PITCH, s, a, M, K);
+    if (r.n > 0) hipLaunchKernelGGL(qgemm_split_reduce_multi_kernel, dim3(red_blocks), dim3(256), 0, s, r);
     return launch_status();
 }
 
