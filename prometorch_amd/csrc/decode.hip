@@ -44,7 +44,9 @@ int q6k_gemv_argmax_impl(const void* W, const float* x, const float* gamma, floa
                          const ArgmaxAdvance adv, hipStream_t s);
 int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
                    int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, bool reuse_rows,
-                   hipStream_t s);
+                   hipStream_t s, int* deferred_splits);
+int qgemm_f16_reduce_norm_prepare(const float* P, int splits, float* X, bool accumulate, const float* gamma, float eps,
+                                  int add_one, void* ws_round, void* ws_plain, int M, int K, hipStream_t s);
 int qgemm_f16_splits(int N, int K, int M);
 size_t qgemm_f16_multi_split_bytes(int n, const int* N, const uint32_t* types, int K, int M);
 int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const int64_t* strides, const int* N, float* const* Y,
@@ -337,10 +339,20 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
     // SiLU.up are fused into the conversion (one launch fills both forms); a product whose rows are already in its
     // workspace skips the conversion.
     auto ws_of = [&](const ptm_qweight& w) { return w.ggml_type == PTM_TYPE_Q4_K ? d->pf_ws : d->pf_ws2; };
-    auto gemm = [&](const ptm_qweight& w, const float* X, float* Y, bool acc, bool rows_ready) {
+    auto gemm = [&](const ptm_qweight& w, const float* X, float* Y, bool acc, bool rows_ready, int* deferred = nullptr) {
         return qgemm_f16_impl(w.ggml_type, w.data, X, true, Y, M, w.cols, w.rows, w.row_stride_bytes, ws_of(w), acc,
-                              d->pf_split, d->pf_split_bytes, rows_ready, s);
+                              d->pf_split, d->pf_split_bytes, rows_ready, s, deferred);
     };
+    // RMSNorm of the residual rows into the row workspaces; `pending` > 0: the projection before it left that many K-split
+    // partial sums in pf_split, which the same launch first adds to the residual rows
+    auto norm_rows = [&](int pending, const float* gamma, bool need4, bool need6) {
+        void* w4 = need4 ? d->pf_ws : nullptr;
+        void* w6 = need6 ? d->pf_ws2 : nullptr;
+        if (pending > 0)
+            return qgemm_f16_reduce_norm_prepare(d->pf_split, pending, d->pf_x, true, gamma, c.rms_eps, 0, w4, w6, M, H, s);
+        return qgemm_f16_prepare_fused(1, d->pf_x, gamma, c.rms_eps, 0, w4, w6, M, H, s);
+    };
+    int pending = 0;  // K-split partial sums of the last projection into pf_x that are still to be added
     auto uses = [](uint32_t type, std::initializer_list<const ptm_qweight*> ws) {
         for (const ptm_qweight* w : ws) if (w->ggml_type == type) return true;
         return false;
@@ -348,9 +360,8 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
     for (int li = 0; li < c.n_layers; ++li) {
         const ptm_layer& L = d->layers[li];
         const bool local = layer_is_local(c, li);
-        PTM_TRY(qgemm_f16_prepare_fused(1, d->pf_x, L.attn_norm, c.rms_eps, 0,
-                                        uses(PTM_TYPE_Q4_K, {&L.q, &L.k, &L.v}) ? d->pf_ws : nullptr,
-                                        uses(PTM_TYPE_Q6_K, {&L.q, &L.k, &L.v}) ? d->pf_ws2 : nullptr, M, H, s));
+        PTM_TRY(norm_rows(pending, L.attn_norm, uses(PTM_TYPE_Q4_K, {&L.q, &L.k, &L.v}), uses(PTM_TYPE_Q6_K, {&L.q, &L.k, &L.v})));
+        pending = 0;
         {  // q, k, v in one launch
             const uint32_t t3[3] = {L.q.ggml_type, L.k.ggml_type, L.v.ggml_type};
             const void* W3[3] = {L.q.data, L.k.data, L.v.data};
@@ -369,11 +380,10 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
             PTM_TRY(gemm(L.o, d->pf_attn, d->pf_h, false, false));
             PTM_TRY(ptm_rms_norm_add(d->pf_h, L.post_attn_norm, d->pf_x, M, H, c.rms_eps, 0, s));
         } else {
-            PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true, false));  // x += attn . Wo^T
+            PTM_TRY(gemm(L.o, d->pf_attn, d->pf_x, true, false, H <= 12288 ? &pending : nullptr));  // x += attn . Wo^T
         }
-        PTM_TRY(qgemm_f16_prepare_fused(1, d->pf_x, L.ffn_norm, c.rms_eps, 0,
-                                        uses(PTM_TYPE_Q4_K, {&L.gate, &L.up}) ? d->pf_ws : nullptr,
-                                        uses(PTM_TYPE_Q6_K, {&L.gate, &L.up}) ? d->pf_ws2 : nullptr, M, H, s));
+        PTM_TRY(norm_rows(pending, L.ffn_norm, uses(PTM_TYPE_Q4_K, {&L.gate, &L.up}), uses(PTM_TYPE_Q6_K, {&L.gate, &L.up})));
+        pending = 0;
         PTM_TRY(gemm(L.gate, d->pf_x, d->pf_gate, false, true));
         PTM_TRY(gemm(L.up, d->pf_x, d->pf_up, false, true));
         const bool act_ready = true;
@@ -385,7 +395,8 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
             PTM_TRY(gemm(L.down, d->pf_gate, d->pf_h, false, act_ready));
             PTM_TRY(ptm_rms_norm_add(d->pf_h, L.post_ffn_norm, d->pf_x, M, H, c.rms_eps, 0, s));
         } else {
-            PTM_TRY(gemm(L.down, d->pf_gate, d->pf_x, true, act_ready));  // x += act . Wdown^T
+            // x += act . Wdown^T; before another layer the sum of the K splits is left to that layer's first launch
+            PTM_TRY(gemm(L.down, d->pf_gate, d->pf_x, true, act_ready, (li + 1 < c.n_layers && H <= 12288) ? &pending : nullptr));
         }
     }
     (void)qd; (void)kvd;

@@ -396,6 +396,123 @@ __global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* _
         }
         return r;
     };
+    // Rows of up to 16384 values are computed once and kept in registers between the maximum and the store pass: all of a
+    // thread's loads go out together, and the exponentials of PRE 2 are paid once (the pass is otherwise two dependent
+    // sweeps over 2 x 4 K bytes per row).
+    constexpr int HOLD = 16;
+    const bool held = n4 <= HOLD * 256;
+    float4 hv[HOLD];
+    float amax = 0.0f;
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < HOLD; ++u) {
+            const int i = tid + 256 * u;
+            hv[u] = i < n4 ? value4(i) : make_float4(0.f, 0.f, 0.f, 0.f);
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(hv[u].x), fabsf(hv[u].y)), fmaxf(fabsf(hv[u].z), fabsf(hv[u].w))));
+        }
+    } else {
+        for (int i = tid; i < n4; i += 256) {
+            const float4 v = value4(i);
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
+    }
+    amax = max64(amax);
+    if ((tid & 63) == 0) red2[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red2[0], red2[1]), fmaxf(red2[2], red2[3]));
+    int e = 0;
+    if (amax > 16384.0f) { (void)frexpf(amax, &e); e -= 14; }
+    const float down = ldexpf(1.0f, -e);
+    if (tid == 0) {
+        if (rs_round) rs_round[m] = ldexpf(1.0f, e);
+        if (rs_plain) rs_plain[m] = ldexpf(1.0f, e);
+    }
+    auto store4 = [&](_Float16* dst, int i, float4 v) {
+        union { _Float16 h[4]; uint2 u; } o;
+        o.h[0] = (_Float16)(v.x * down);
+        o.h[1] = (_Float16)(v.y * down);
+        o.h[2] = (_Float16)(v.z * down);
+        o.h[3] = (_Float16)(v.w * down);
+        reinterpret_cast<uint2*>(dst)[i] = o.u;
+    };
+    auto emit4 = [&](int i, float4 v) {  // K % 256 == 0: whole waves, aligned groups of 8 lanes = one Q8 block
+        if (Xh_plain) store4(Xh_plain + (int64_t)m * K, i, v);
+        if (Xh_round) {
+            float d, sm;
+            const uint32_t pk = q8_quantize4(v, d, sm);
+            float4 q;
+            q.x = d * (float)(int)(int8_t)(pk & 0xff);
+            q.y = d * (float)(int)(int8_t)((pk >> 8) & 0xff);
+            q.z = d * (float)(int)(int8_t)((pk >> 16) & 0xff);
+            q.w = d * (float)(int)(int8_t)(pk >> 24);
+            store4(Xh_round + (int64_t)m * K, i, q);
+        }
+    };
+    if (held) {
+#pragma unroll
+        for (int u = 0; u < HOLD; ++u) {
+            const int i = tid + 256 * u;
+            if (i < n4) emit4(i, hv[u]);  // wave-uniform: n4 is a multiple of 64
+        }
+    } else {
+        for (int i = tid; i < n4; i += 256) emit4(i, value4(i));
+    }
+}
+
+// The K-split partial sums of a projection into the residual stream, folded into the conversion that follows it:
+// X[m] (+)= P[0][m] + P[1][m] + ... (the order of qgemm_split_reduce_kernel), then RMSNorm of the new row and its fp16
+// forms as qgemm_prepare_fused_kernel<1> produces them (same arithmetic, same reduction order: the row is staged in LDS
+// and walked with that kernel's two lane mappings).  One launch and one pass over the row instead of a reduction launch
+// and three sweeps of the conversion.
+__global__ __launch_bounds__(256) void qgemm_reduce_norm_prepare_kernel(const float* __restrict__ P, int splits, float* __restrict__ X,
+                                                                        int accumulate, const float* __restrict__ gamma, float eps,
+                                                                        int add_one, _Float16* __restrict__ Xh_round,
+                                                                        float* __restrict__ rs_round, _Float16* __restrict__ Xh_plain,
+                                                                        float* __restrict__ rs_plain, int M, int K) {
+    extern __shared__ __align__(16) float rn_row[];  // K floats
+    __shared__ float red[4];
+    __shared__ float red2[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const int n4 = K / 4;
+    if (m >= M) {  // padding rows: zeros
+        for (int i = tid; i < n4; i += 256) {
+            if (Xh_round) reinterpret_cast<uint2*>(Xh_round + (int64_t)m * K)[i] = make_uint2(0, 0);
+            if (Xh_plain) reinterpret_cast<uint2*>(Xh_plain + (int64_t)m * K)[i] = make_uint2(0, 0);
+        }
+        return;
+    }
+    const int64_t total = (int64_t)M * K;
+    float4* x4 = reinterpret_cast<float4*>(X + (int64_t)m * K);
+    for (int i = tid; i < n4; i += 256) {
+        // eight partial sums per batch, fetched unconditionally (the index clamped) so that they are in flight together
+        const float4 o = accumulate ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int z0 = 0; z0 < splits; z0 += 8) {
+            float4 b[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) b[u] = reinterpret_cast<const float4*>(P + min(z0 + u, splits - 1) * total + (int64_t)m * K)[i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (z0 + u == 0) a = b[u];
+                else if (z0 + u < splits) { a.x += b[u].x; a.y += b[u].y; a.z += b[u].z; a.w += b[u].w; }
+            }
+        }
+        if (accumulate) { a.x += o.x; a.y += o.y; a.z += o.z; a.w += o.w; }
+        x4[i] = a;
+        reinterpret_cast<float4*>(rn_row)[i] = a;
+    }
+    __syncthreads();
+    float ss = 0.0f;
+    for (int i = tid; i < K; i += 256) ss = fmaf(rn_row[i], rn_row[i], ss);
+    ss = block_sum256(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)K + eps);
+    const float one = add_one ? 1.0f : 0.0f;
+    auto value4 = [&](int i) {
+        const float4 a = reinterpret_cast<const float4*>(rn_row)[i], b = reinterpret_cast<const float4*>(gamma)[i];
+        float4 r;
+        r.x = a.x * rs * (b.x + one); r.y = a.y * rs * (b.y + one); r.z = a.z * rs * (b.z + one); r.w = a.w * rs * (b.w + one);
+        return r;
+    };
     float amax = 0.0f;
     for (int i = tid; i < n4; i += 256) {
         const float4 v = value4(i);
@@ -891,7 +1008,9 @@ static int qgemm_check(const void* W, const void* X, const void* Y, int M, int K
 // Y (+)= X . W^T with X bf16 or fp32 rows; shared by the C entry points and the prefill runtime.
 int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f32, float* Y, int M, int K, int N,
                    int64_t stride, void* workspace, bool accumulate, float* split_ws, size_t split_ws_bytes, bool reuse_rows,
-                   hipStream_t s) {
+                   hipStream_t s, int* deferred_splits) {
+    // deferred_splits (optional): where K was split, the partial sums are left in split_ws for the caller's next kernel to
+    // fold in (qgemm_f16_reduce_norm_prepare) and their count is returned here; 0 = Y is complete
     // reuse_rows: the workspace already holds these rows of X prepared by the previous call for a matrix of the
     // same type (same rounding rule), so the conversion pass is skipped
     if (ggml_type != PTM_TYPE_Q4_K && ggml_type != PTM_TYPE_Q6_K) return PTM_E_UNSUPPORTED;
@@ -947,11 +1066,30 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     else if (q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
-    if (partials) {
+    if (deferred_splits) *deferred_splits = partials ? splits : 0;
+    if (partials && !deferred_splits) {
         const int64_t total = (int64_t)M * N;
         hipLaunchKernelGGL(qgemm_split_reduce_kernel, dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, s, partials, splits,
                            Y, total, acc);
     }
+    return launch_status();
+}
+
+// X (+)= the `splits` partial sums a deferred qgemm_f16_impl left in P, then RMSNorm(X; gamma) into the row workspaces
+// (ws_round for Q4_K matrices, ws_plain for Q6_K ones; either may be NULL), as qgemm_f16_prepare_fused(1, ...) fills them.
+int qgemm_f16_reduce_norm_prepare(const float* P, int splits, float* X, bool accumulate, const float* gamma, float eps,
+                                  int add_one, void* ws_round, void* ws_plain, int M, int K, hipStream_t s) {
+    if (!P || !X || !gamma || (!ws_round && !ws_plain)) return PTM_E_NULL;
+    if (M <= 0 || K <= 0 || (K % 256) != 0 || splits < 1) return PTM_E_SHAPE;
+    if (K > 12288) return PTM_E_UNSUPPORTED;  // the row is staged in LDS (48 KB, within the default cap)
+    if (!aligned16(P) || !aligned16(X) || !aligned16(gamma) || !aligned16(ws_round) || !aligned16(ws_plain)) return PTM_E_ALIGN;
+    const int mp = qf_mpad(M);
+    _Float16* hr = static_cast<_Float16*>(ws_round);
+    _Float16* hp = static_cast<_Float16*>(ws_plain);
+    float* rr = hr ? reinterpret_cast<float*>(hr + (int64_t)mp * K) : nullptr;
+    float* rp = hp ? reinterpret_cast<float*>(hp + (int64_t)mp * K) : nullptr;
+    hipLaunchKernelGGL(qgemm_reduce_norm_prepare_kernel, dim3(mp), dim3(256), (size_t)K * 4, s, P, splits, X, accumulate ? 1 : 0,
+                       gamma, eps, add_one, hr, rr, hp, rp, M, K);
     return launch_status();
 }
 
@@ -1100,7 +1238,8 @@ int64_t ptm_qgemm_f16_workspace_bytes(int M, int K) {
 
 int ptm_qgemm_f16(uint32_t ggml_type, const void* W, const void* X_bf16, float* Y, int M, int K, int N, int64_t stride,
                   void* workspace, ptm_stream_t stream) {
-    return qgemm_f16_impl(ggml_type, W, X_bf16, false, Y, M, K, N, stride, workspace, false, nullptr, 0, false, as_stream(stream));
+    return qgemm_f16_impl(ggml_type, W, X_bf16, false, Y, M, K, N, stride, workspace, false, nullptr, 0, false, as_stream(stream),
+                          nullptr);
 }
 
 int64_t ptm_qgemm_f16_f32_workspace_bytes(int M, int K, int N) {
@@ -1118,7 +1257,7 @@ int ptm_qgemm_f16_f32(uint32_t ggml_type, const void* W, const float* X_f32, flo
     const int splits = qgemm_f16_splits(N, K, M);
     return qgemm_f16_impl(ggml_type, W, X_f32, true, Y, M, K, N, stride, workspace, accumulate != 0,
                           splits > 1 ? reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + base) : nullptr,
-                          splits > 1 ? (size_t)splits * M * N * 4 : 0, false, as_stream(stream));
+                          splits > 1 ? (size_t)splits * M * N * 4 : 0, false, as_stream(stream), nullptr);
 }
 
 }  // extern "C"
