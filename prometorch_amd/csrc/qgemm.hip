@@ -691,6 +691,8 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
     const uint8_t* x_src = reinterpret_cast<const uint8_t*>(Xh) + (int64_t)(m0 + (tid >> 5)) * x_row_bytes + 16 * (tid & 31) +
                            (int64_t)blk0 * 512;
     uint8_t* x_dst = s_a + (tid >> 5) * QF_PITCH + 16 * (tid & 31);
+    float* s_rs = reinterpret_cast<float*>(s_a + 2 * TM * QF_PITCH);  // the tile's TM row scales (every padded row has one)
+    if (tid < TM) s_rs[tid] = rowscale[m0 + tid];
     // the 16 pieces of the next tile in flight (scalars, not an array: they must stay in registers)
     static_assert(MT == 1 || MT == 2 || MT == 4, "row tiles per workgroup");
     uint4 x0, x1, x2, x3, x4, x5, x6, x7, x8, x9, x10, x11, x12, x13, x14, x15;
@@ -805,53 +807,39 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
         for (int t = 0; t < NT; ++t) cur[t] = nxt[t];
         __syncthreads();  // next tile complete, this tile no longer read
     }
-    // C layout of the 32x32 tile: column j = lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4.
-    // Every load of the epilogue is issued before the first store: a load behind a store to memory the compiler cannot tell
-    // apart waits for it, and 16 MT row scales (plus as many old values of Y when accumulating) fetched one by one between the
-    // stores are as many serial memory round trips, more than the main loop of a launch with few blocks per workgroup takes.
-    // (rowscale holds an entry for every padded row; rows >= M are never stored.)
-    float rsv[MT][16];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) rsv[mt][r] = rowscale[m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3)];
+    // C layout of the 32x32 tile: column j = lane % 32, rows 8 (r / 4) + 4 (lane / 32) + r % 4.  The row scales come from
+    // LDS (staged in the prologue), and when accumulating the 16 old values of a tile are fetched together before its 16
+    // stores: a load issued behind a store the compiler cannot tell apart from it is one serial memory round trip per value,
+    // more than the main loop of a launch with few blocks per workgroup takes.
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int n = n_base + 32 * t + j;
         const bool n_ok = n < N;
         const int nc = n_ok ? n : N - 1;
-        if (partials) {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-                    if (m < M && n_ok) partials[((int64_t)bz * M + m) * N + n] = acc[mt][t][r] * rsv[mt][r];
-                }
-        } else if (accumulate) {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                float old[16];
+        for (int mt = 0; mt < MT; ++mt) {
+            float old[16];
+            if (!partials && accumulate) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = min(m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3), M - 1);
                     old[r] = Y[(int64_t)m * N + nc];
                 }
                 issue_order_fence();
+            } else {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-                    if (m < M && n_ok) Y[(int64_t)m * N + n] = old[r] + acc[mt][t][r] * rsv[mt][r];
+                for (int r = 0; r < 16; ++r) old[r] = 0.0f;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int lr = mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+                const int m = m0 + lr;
+                const float v = acc[mt][t][r] * s_rs[lr];
+                if (m < M && n_ok) {
+                    if (partials) partials[((int64_t)bz * M + m) * N + n] = v;
+                    else Y[(int64_t)m * N + n] = accumulate ? old[r] + v : v;
                 }
             }
-        } else {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = m0 + mt * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-                    if (m < M && n_ok) Y[(int64_t)m * N + n] = acc[mt][t][r] * rsv[mt][r];
-                }
         }
     }
 }
@@ -1043,10 +1031,10 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     // 128 (half the dequantisation work per product)
     const int MT = qgemm_f16_row_tiles(q4, M, N, splits);
     const int tm = 32 * MT;
-    const size_t lds = 2 * (size_t)tm * QF_PITCH;  // 132 KB / 66 KB: above the default 64 KB cap of dynamic LDS
+    const size_t lds = 2 * (size_t)tm * QF_PITCH + 4 * (size_t)tm;  // 132 KB / 66 KB (two X tiles) + the row scales: above the default 64 KB cap of dynamic LDS
     static bool raised = false;
     if (!raised) {
-        const int big = 2 * 128 * QF_PITCH, small = 2 * 64 * QF_PITCH;
+        const int big = 2 * 128 * QF_PITCH + 4 * 128, small = 2 * 64 * QF_PITCH + 4 * 64;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
@@ -1159,10 +1147,10 @@ int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const in
     static bool raised = false;
     if (!raised) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_multi_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  2 * 128 * QF_PITCH);
+                                  2 * 128 * QF_PITCH + 4 * 128);
         raised = true;
     }
-    hipLaunchKernelGGL(qgemm_f16_multi_kernel, dim3(slots, (M + 127) / 128), dim3(512), 2 * (size_t)128 * QF_PITCH, s, a, M, K);
+    hipLaunchKernelGGL(qgemm_f16_multi_kernel, dim3(slots, (M + 127) / 128), dim3(512), 2 * (size_t)128 * QF_PITCH + 4 * 128, s, a, M, K);
     if (r.n > 0) hipLaunchKernelGGL(qgemm_split_reduce_multi_kernel, dim3(red_blocks), dim3(256), 0, s, r);
     return launch_status();
 }
