@@ -836,8 +836,8 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
                 const int m = m0 + lr;
                 const float v = acc[mt][t][r] * s_rs[lr];
                 if (m < M && n_ok) {
-                    if (partials) partials[((int64_t)bz * M + m) * N + n] = v;
-                    else Y[(int64_t)m * N + n] = accumulate ? old[r] + v : v;
+                    if (partials) __builtin_nontemporal_store(v, &partials[((int64_t)bz * M + m) * N + n]);
+                    else __builtin_nontemporal_store(accumulate ? old[r] + v : v, &Y[(int64_t)m * N + n]);
                 }
             }
         }
