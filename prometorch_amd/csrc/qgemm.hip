@@ -844,13 +844,38 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
     }
 }
 
+// Which tile a workgroup takes.  The hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its own
+// L2; taken as they come, the workgroups of one XCD are scattered over all column tiles, row tiles and K splits and share
+// almost nothing (the down projection of a 512-row prompt, 10 x 4 tiles x 6 splits, then pulls 200 MB through the L2s for
+// 30 MB of operands).  Here the workgroups an XCD receives form one contiguous run of the order "row tile fastest, then
+// column tile (or slot) within a band of 4 row tiles, then band, then K split": the 32 or so workgroups an XCD runs at a time
+// are then about 4 row tiles x 8 column tiles, so each weight piece serves 4 of them and each X tile 8 from one L2.
+__device__ __forceinline__ int qf_xcd_order(int hw, int nwg) {
+    const int xcd = hw & 7, slot = hw >> 3, per = nwg >> 3, rem = nwg & 7;
+    return xcd * per + (xcd < rem ? xcd : rem) + slot;
+}
+// position L of that order -> (column tile or slot, row tile, K split) on a gx x gy x gz grid
+__device__ __forceinline__ void qf_tile_of(int L, int gx, int gy, int& bx, int& by, int& bz) {
+    const int plane = gx * gy;
+    bz = L / plane;
+    const int r = L - bz * plane;
+    const int band = r / (4 * gx);
+    const int rows = min(4, gy - 4 * band);
+    const int within = r - band * 4 * gx;
+    by = 4 * band + within % rows;
+    bx = within / rows;
+}
+
 template <typename Tile, int MT, int WAVES = 4>
 __global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : (MT <= 2 ? 2 : 1))) void qgemm_f16_kernel(const uint8_t* W, int64_t stride, const _Float16* Xh,
                                                         const float* __restrict__ rowscale, float* Y, int M, int K, int N,
                                                         int accumulate, int blocks_per_split, float* partials) {
     extern __shared__ __align__(16) uint8_t qf_lds[];
-    qgemm_f16_body<Tile, MT, WAVES>(W, stride, Xh, rowscale, Y, M, K, N, accumulate, blocks_per_split, partials, blockIdx.x,
-                                    blockIdx.y, blockIdx.z, qf_lds);
+    const int hw = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const int L = qf_xcd_order(hw, gridDim.x * gridDim.y * gridDim.z);
+    int bx, by, bz;
+    qf_tile_of(L, gridDim.x, gridDim.y, bx, by, bz);
+    qgemm_f16_body<Tile, MT, WAVES>(W, stride, Xh, rowscale, Y, M, K, N, accumulate, blocks_per_split, partials, bx, by, bz, qf_lds);
 }
 
 // Up to three projections of the same rows in ONE launch of the eight-wave 128-row tile (q, k, v of a layer: in a Q4_K_M
@@ -871,14 +896,17 @@ struct QfMulti { QfMat m[3]; int n_mat; };
 
 __global__ __launch_bounds__(512, 1) void qgemm_f16_multi_kernel(const QfMulti a, int M, int K) {
     extern __shared__ __align__(16) uint8_t qf_lds[];
+    const int L = qf_xcd_order(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
+    int sx, by, unused;
+    qf_tile_of(L, gridDim.x, gridDim.y, sx, by, unused);  // sx: the (matrix, split, column tile) slot
     int i = 0;
-    if (a.n_mat > 1 && (int)blockIdx.x >= a.m[0].slot_end) i = 1;
-    if (a.n_mat > 2 && (int)blockIdx.x >= a.m[1].slot_end) i = 2;
+    if (a.n_mat > 1 && sx >= a.m[0].slot_end) i = 1;
+    if (a.n_mat > 2 && sx >= a.m[1].slot_end) i = 2;
     const QfMat& q = i == 0 ? a.m[0] : (i == 1 ? a.m[1] : a.m[2]);
-    const int local = (int)blockIdx.x - (i == 0 ? 0 : (i == 1 ? a.m[0].slot_end : a.m[1].slot_end));
+    const int local = sx - (i == 0 ? 0 : (i == 1 ? a.m[0].slot_end : a.m[1].slot_end));
     const int bx = local % q.ntiles, bz = local / q.ntiles;
-    if (q.q6) qgemm_f16_body<Q6Tile, 4, 8>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, blockIdx.y, bz, qf_lds);
-    else qgemm_f16_body<Q4Tile, 4, 8>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, blockIdx.y, bz, qf_lds);
+    if (q.q6) qgemm_f16_body<Q6Tile, 4, 8>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, by, bz, qf_lds);
+    else qgemm_f16_body<Q4Tile, 4, 8>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, by, bz, qf_lds);
 }
 
 // Y (+)= partials[0] + partials[1] + ... in that fixed order (deterministic, unlike atomics)
