@@ -16,6 +16,10 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
 ]
+# Per-file additions.  prefill.hip: its matrix-core attention rescales the output accumulators between MFMAs with vector
+# arithmetic, which cannot touch accumulation registers; with the accumulators there the compiler copies all 64 of them
+# out and back on every tile.  One wave per SIMD leaves room for them in ordinary registers.
+FILE_FLAGS = {"prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def build(verbose: bool = True, jobs: int = 8) -> str:
@@ -24,7 +28,7 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
     for src in SOURCES:
         obj = os.path.join(CSRC, "build", src.replace(".hip", ".o"))
         objs.append(obj)
-        cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [HIPCC, *FLAGS, *FILE_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

@@ -240,6 +240,7 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restri
 // ---- matrix-core version (fp16 cache) ----------------------------------------------------------------------------
 typedef _Float16 pf_h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 pf_h4 __attribute__((ext_vector_type(4)));
+typedef pf_h4 pf_h4_a4 __attribute__((aligned(4)));
 typedef float pf_f16v __attribute__((ext_vector_type(16)));
 
 // v_mfma_f32_32x32x16_f16 operand layout used below: A (32 x 16): lane l holds row l % 32, summation indices
@@ -247,8 +248,14 @@ typedef float pf_f16v __attribute__((ext_vector_type(16)));
 // l % 32, rows 8 (r / 4) + 4 (l / 32) + r % 4 for r = 0..15.  The summation index may be permuted freely as long as A
 // and B agree, which is used twice: the 16 head-dim elements of a step are [16 ks + 8 kh, +8) for lane half kh,
 // and the 16 positions of a P.V step are the ones the lane already holds in its S^T accumulator.
+// Eight waves in two groups of four: both groups hold the same 32 G-head query rows, group g takes the tiles of 32
+// positions with index = g mod 2 (its own staging buffers; the barriers are shared), and the two online-softmax states are
+// merged through LDS at the end.  A tile is one long dependent chain per wave (stage, barrier, 8 score MFMAs, softmax, 8
+// output MFMAs: about 1.4 us); splitting the positions halves the number of links of a row block's chain and gives each
+// SIMD a second wave to run under the first one's waits.  Tile parity is absolute, so a row's arithmetic does not depend
+// on how the prompt was chunked.
 template <int HD, int G>
-__global__ __launch_bounds__(256) void prefill_attn_mfma_kernel(const float* __restrict__ Q, const __half* __restrict__ Kc,
+__global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __restrict__ Q, const __half* __restrict__ Kc,
                                                                 const __half* __restrict__ Vc, float* __restrict__ O, int rows,
                                                                 int n_heads, int n_kv_heads, int64_t pos0, float scale) {
     constexpr int RPW = 32 / G;        // rows per wave (each with its G heads: 32 query vectors)
@@ -256,12 +263,16 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_kernel(const float* __r
     constexpr int KS = HD / 16;        // MFMA steps over the head dimension
     constexpr int DT = HD / 32;        // 32-wide tiles of the output's head dimension
     constexpr int KP = HD * 2 + 16;    // LDS pitch of a K row (bytes)
-    constexpr int VP = 64 + 8;         // LDS pitch of a V^T row: 32 positions of fp16 + padding
+    constexpr int VP = 64 + 4;         // LDS pitch of a V^T row: 32 positions of fp16 + one word, an ODD number of words
     constexpr int PCS = 32 * HD / 8 / 256;  // 16-byte pieces of a 32-position tile per thread (1 or 2)
     static_assert(PCS == 1 || PCS == 2, "tile smaller than the workgroup");
-    __shared__ __align__(16) uint8_t s_k[32 * KP];
-    __shared__ __align__(16) uint8_t s_vt[HD * VP];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ __align__(16) uint8_t s_k2[2][32 * KP];
+    __shared__ __align__(16) uint8_t s_vt2[2][HD * VP + 12];
+    __shared__ float s_merge[4][16 * DT + 2][64];  // group 1's accumulators, running maximum and sum, lane-contiguous
+    const int grp = threadIdx.x >> 8;
+    uint8_t* const s_k = s_k2[grp];
+    uint8_t* const s_vt = s_vt2[grp];
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, kh = lane >> 5;
     const int kvh = blockIdx.y;
     const int m_base = (gridDim.x - 1 - blockIdx.x) * BM;  // longest row blocks are scheduled first
@@ -292,28 +303,43 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_kernel(const float* __r
     const int last_row = (m_base + BM < rows ? m_base + BM : rows) - 1;
     const int64_t t_end = pos0 + last_row;  // last position any query of this workgroup attends to
     const int ntiles = (int)(t_end / 32) + 1;
-    // staging: piece q = tid + 256 i of a tile is position q / (HD / 8), elements 8 (q % (HD / 8)) .. +8
-    uint4 kreg0, kreg1, vreg0, vreg1;  // scalars, not arrays: they must stay in registers across the loop
-    kreg1 = vreg1 = make_uint4(0, 0, 0, 0);
-    auto piece_off = [&](int tile, int i) {
-        const int q = tid + 256 * i, p = q / (HD / 8), c = q % (HD / 8);
+    // staging: piece q = tid + 256 i of a tile is position q / (HD / 8), elements 8 (q % (HD / 8)) .. +8.
+    // Two tiles are kept in flight (register sets A and B, alternating): the rows come from HBM, and one tile's arithmetic
+    // is shorter than that round trip.  Every fetch is unconditional (tile indices past the end are clamped), so the
+    // number of loads in flight is static and waiting for set A does not wait for set B.
+    uint4 kA0, kA1, vA0, vA1, kB0, kB1, vB0, vB1;  // scalars, not arrays: they must stay in registers across the loop
+    kA1 = vA1 = kB1 = vB1 = make_uint4(0, 0, 0, 0);
+    // K piece i of a thread: position (tid + 256 i) / (HD / 8), elements 8 ((tid + 256 i) % (HD / 8)) .. +8 (a wave reads
+    // whole rows).  V pieces are laid out for the transposed LDS store, where the 64 lanes of a wave write one element
+    // each of rows 8 c + k at column p: a wave takes 16 positions x 4 element groups c, so that with the odd row pitch its
+    // lanes fall on all 32 banks (positions give 8 banks, the 4 groups are 8 banks apart); 4 positions x 16 groups, the K
+    // mapping, puts them on 4 (measured: bank conflicts were 59 % of the LDS cycles of the kernel).
+    auto k_piece = [&](int i, int& p, int& c) { const int q = tid + 256 * i; p = q / (HD / 8); c = q % (HD / 8); };
+    auto v_piece = [&](int i, int& p, int& c) { const int u = wave + 4 * i; p = 16 * (u & 1) + (lane & 15); c = 4 * (u >> 1) + (lane >> 4); };
+    auto piece_off = [&](int tile, int p, int c) {
         int64_t t = (int64_t)tile * 32 + p;
         t = t <= t_end ? t : t_end;  // rows past the end are masked below; never read past the appended rows
         return t * kv_dim + (int64_t)kvh * HD + 8 * c;
     };
-    auto fetch = [&](int tile) {
-        const int64_t o0 = piece_off(tile, 0);
-        kreg0 = *reinterpret_cast<const uint4*>(Kc + o0);
-        vreg0 = *reinterpret_cast<const uint4*>(Vc + o0);
+    auto fetch = [&](int tile, uint4& k0, uint4& v0, uint4& k1, uint4& v1) {
+        tile = tile < ntiles ? tile : ntiles - 1;
+        int p, c;
+        k_piece(0, p, c);
+        k0 = *reinterpret_cast<const uint4*>(Kc + piece_off(tile, p, c));
+        v_piece(0, p, c);
+        v0 = *reinterpret_cast<const uint4*>(Vc + piece_off(tile, p, c));
         if constexpr (PCS > 1) {
-            const int64_t o1 = piece_off(tile, 1);
-            kreg1 = *reinterpret_cast<const uint4*>(Kc + o1);
-            vreg1 = *reinterpret_cast<const uint4*>(Vc + o1);
+            k_piece(1, p, c);
+            k1 = *reinterpret_cast<const uint4*>(Kc + piece_off(tile, p, c));
+            v_piece(1, p, c);
+            v1 = *reinterpret_cast<const uint4*>(Vc + piece_off(tile, p, c));
         }
     };
     auto stage = [&](int i, const uint4& kr, const uint4& vr) {
-        const int q = tid + 256 * i, p = q / (HD / 8), c = q % (HD / 8);
+        int p, c;
+        k_piece(i, p, c);
         *reinterpret_cast<uint4*>(s_k + p * KP + 16 * c) = kr;
+        v_piece(i, p, c);
         uint8_t* vt = s_vt + (8 * c) * VP + 2 * p;  // transposed: V^T[d][position]
         *reinterpret_cast<uint16_t*>(vt + 0 * VP) = (uint16_t)vr.x;
         *reinterpret_cast<uint16_t*>(vt + 1 * VP) = (uint16_t)(vr.x >> 16);
@@ -324,38 +350,55 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_kernel(const float* __r
         *reinterpret_cast<uint16_t*>(vt + 6 * VP) = (uint16_t)vr.w;
         *reinterpret_cast<uint16_t*>(vt + 7 * VP) = (uint16_t)(vr.w >> 16);
     };
-    fetch(0);
-    for (int tile = 0; tile < ntiles; ++tile) {
+    // one tile: stage it from its register set, refill the set with the tile two further on, then the arithmetic
+    auto do_tile = [&](int tile, uint4& k0, uint4& v0, uint4& k1, uint4& v1) {
         __syncthreads();  // every wave has finished reading the previous tile
-        stage(0, kreg0, vreg0);
-        if constexpr (PCS > 1) stage(1, kreg1, vreg1);
+        stage(0, k0, v0);
+        if constexpr (PCS > 1) stage(1, k1, v1);
         __syncthreads();
-        if (tile + 1 < ntiles) fetch(tile + 1);  // in flight during this tile's arithmetic
+        fetch(tile + 4, k0, v0, k1, v1);  // the group's tile after next: in flight during two tiles' arithmetic
+        issue_order_fence();
 
+        // The eight K fragments are read together, so the score MFMAs wait once instead of each for its own read; the V^T
+        // fragments are requested behind the score MFMAs and arrive under the softmax arithmetic.
+        pf_h8 ka[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) ka[ks] = *reinterpret_cast<const pf_h8*>(s_k + j * KP + (16 * ks + 8 * kh) * 2);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(ka[ks]));  // no MFMA is moved up to behind its own read
         // S^T tile: rows = the tile's 32 positions, column = this lane's query vector
         pf_f16v sc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const pf_h8 a = *reinterpret_cast<const pf_h8*>(s_k + j * KP + (16 * ks + 8 * kh) * 2);
-            sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], sc, 0, 0, 0);
-        }
-        const int64_t t0 = (int64_t)tile * 32 + 4 * kh;
-        float mx = -INFINITY;
+        for (int ks = 0; ks < KS; ++ks) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks], qf[ks], sc, 0, 0, 0);
+        pf_h4 vlo[2][DT], vhi[2][DT];  // into the registers the K fragments leave
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int64_t t = t0 + 8 * (r >> 2) + (r & 3);
-            sc[r] = t <= limit ? sc[r] : -INFINITY;
-            mx = fmaxf(mx, sc[r]);
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const uint8_t* vrow = s_vt + (32 * dt + j) * VP + (16 * ks + 4 * kh) * 2;
+                vlo[ks][dt] = *reinterpret_cast<const pf_h4_a4*>(vrow);  // rows are 4-byte aligned
+                vhi[ks][dt] = *reinterpret_cast<const pf_h4_a4*>(vrow + 16);
+            }
+        // only the tiles on the diagonal hold positions some query of the workgroup must not see (workgroup-uniform)
+        if ((int64_t)tile * 32 + 31 > pos0 + m_base) {
+            const int lim = (int)(limit - (int64_t)tile * 32) - 4 * kh;  // position offsets of this lane: 8 (r / 4) + r % 4
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sc[r] = 8 * (r >> 2) + (r & 3) <= lim ? sc[r] : -INFINITY;
         }
+        float mx = sc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // the column's other 16 positions
-        const float m_new = fmaxf(m_run, mx);    // finite from the first tile on: position 0 is visible to every query
-        const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
+        const float m_new = fmaxf(m_run, mx);
+        // group 1 may have seen no visible position of a query yet (-inf): exponentials then take 0 as the reference and are 0
+        const float ms = m_new == -INFINITY ? 0.0f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m_run - ms);
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            sc[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
+            sc[r] = __builtin_amdgcn_exp2f(sc[r] - ms);
             psum += sc[r];
         }
         const pf_h8 pb0 = {(_Float16)sc[0], (_Float16)sc[1], (_Float16)sc[2], (_Float16)sc[3],
@@ -363,21 +406,56 @@ __global__ __launch_bounds__(256) void prefill_attn_mfma_kernel(const float* __r
         const pf_h8 pb1 = {(_Float16)sc[8], (_Float16)sc[9], (_Float16)sc[10], (_Float16)sc[11],
                            (_Float16)sc[12], (_Float16)sc[13], (_Float16)sc[14], (_Float16)sc[15]};
         l_run = fmaf(l_run, corr, psum);  // this lane's 16 positions of each tile; the two halves are added at the end
+        // a running maximum that no lane of the wave has raised leaves every correction at exactly 1: the rescale is skipped
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(m_new != m_run) != 0, 0)) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+        }
         m_run = m_new;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
         // O^T += V^T . P^T: step ks sums the positions of accumulator registers 8 ks .. 8 ks + 7
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const uint8_t* vrow = s_vt + (32 * dt + j) * VP + (16 * ks + 4 * kh) * 2;
-                const pf_h4 lo = *reinterpret_cast<const pf_h4*>(vrow), hi = *reinterpret_cast<const pf_h4*>(vrow + 16);
+                const pf_h4 lo = vlo[ks][dt], hi = vhi[ks][dt];
                 const pf_h8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ks ? pb1 : pb0, acc[dt], 0, 0, 0);
             }
+    };
+    // Group g walks tiles g, g + 2, g + 4, ...; a tile index past the end is a tile of masked positions (its fetch is
+    // clamped, its probabilities are exact zeros), so both groups run the same number of steps and meet at every barrier.
+    fetch(grp, kA0, vA0, kA1, vA1);
+    fetch(grp + 2, kB0, vB0, kB1, vB1);
+    // steps in pairs, with nothing conditional between them: the count of loads in flight at each wait stays static
+    const int nsteps = (ntiles + 1) / 2;
+    int st = 0;
+    for (; st + 1 < nsteps; st += 2) {
+        do_tile(2 * st + grp, kA0, vA0, kA1, vA1);
+        do_tile(2 * st + 2 + grp, kB0, vB0, kB1, vB1);
+    }
+    if (st < nsteps) do_tile(2 * st + grp, kA0, vA0, kA1, vA1);  // workgroup-uniform
+    // ---- merge the two groups' states (same lane of waves w and w + 4 = same query vector, same output elements) ----
+    if (grp == 1) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_merge[wave][16 * dt + r][lane] = acc[dt][r];
+        s_merge[wave][16 * DT][lane] = m_run;
+        s_merge[wave][16 * DT + 1][lane] = l_run;
+    }
+    __syncthreads();
+    if (grp == 1) return;
+    {
+        const float m1 = s_merge[wave][16 * DT][lane], l1 = s_merge[wave][16 * DT + 1][lane];
+        const float mm = fmaxf(m_run, m1);  // finite: tile 0 belongs to group 0 and holds position 0
+        const float c0 = __builtin_amdgcn_exp2f(m_run - mm), c1 = __builtin_amdgcn_exp2f(m1 - mm);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[dt][r] = fmaf(acc[dt][r], c0, s_merge[wave][16 * dt + r][lane] * c1);
+        l_run = fmaf(l_run, c0, l1 * c1);
     }
     const float l = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = 1.0f / (l + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
@@ -397,7 +475,7 @@ static int prefill_attn_mfma_launch(int G, hipStream_t s, const float* Q, const 
                                     int n_heads, int n_kv_heads, int64_t pos0, float scale) {
     const int bm = 128 / G;
     const dim3 grid((rows + bm - 1) / bm, n_kv_heads);
-#define PTM_PA(GG) hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG>), grid, dim3(256), 0, s, Q, static_cast<const __half*>(Kc), static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale)
+#define PTM_PA(GG) hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG>), grid, dim3(512), 0, s, Q, static_cast<const __half*>(Kc), static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale)
     switch (G) {
         case 1: PTM_PA(1); break;
         case 2: PTM_PA(2); break;
