@@ -357,7 +357,13 @@ def test_llama3_8b_layer_shapes_decode_and_prefill_vs_oracle(dev, po, seeds):
     tok_g = dec.prefill(prompt)
     check_kv_rows(dec.k_cache[0][312:352].float().cpu().numpy(), om.k_cache[0][312:352], 0, "k")
     check_kv_rows(dec.v_cache[0][312:352].float().cpu().numpy(), om.v_cache[0][312:352], 0, "v")
-    check_logits(dec.logits(), om.logits, tok_g, tok_o, "prefill")
+    # the prompt's last logits on the same yardstick as the steps behind it (the 40 rows went through the same amplification)
+    err, rms, margin = logit_errors(dec.logits(), om.logits)
+    perr, prms, _ = logit_errors(ob.logits, om.logits)
+    print("  prompt: GPU err %.3f rms %.4f; perturbed oracle err %.3f rms %.4f" % (err, rms, perr, prms), flush=True)
+    assert err <= max(E2E_MAX_TOL, 2 * perr) and rms <= max(E2E_RMS_TOL, 2 * prms), ("prefill", err, rms, perr, prms)
+    if margin > 2 * err:
+        assert tok_g == tok_o, ("prefill", margin, err)
     tok = tok_o
     for st in range(6):
         tok_o = om.step(tok)
