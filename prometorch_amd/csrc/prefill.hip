@@ -359,19 +359,23 @@ __global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __r
         fetch(tile + 4, k0, v0, k1, v1);  // the group's tile after next: in flight during two tiles' arithmetic
         issue_order_fence();
 
-        // The eight K fragments are read together, so the score MFMAs wait once instead of each for its own read; the V^T
+        // K fragments are read four at a time, so the score MFMAs wait twice for a batch instead of each for its own read
+        // (all eight at once would need 16 more registers than the 256 a wave of this 512-thread workgroup has); the V^T
         // fragments are requested behind the score MFMAs and arrive under the softmax arithmetic.
-        pf_h8 ka[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) ka[ks] = *reinterpret_cast<const pf_h8*>(s_k + j * KP + (16 * ks + 8 * kh) * 2);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(ka[ks]));  // no MFMA is moved up to behind its own read
         // S^T tile: rows = the tile's 32 positions, column = this lane's query vector
         pf_f16v sc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[ks], qf[ks], sc, 0, 0, 0);
+        for (int k0 = 0; k0 < KS; k0 += 4) {
+            pf_h8 ka[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ka[u] = *reinterpret_cast<const pf_h8*>(s_k + j * KP + (16 * (k0 + u) + 8 * kh) * 2);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(ka[u]));  // no MFMA is moved up to behind its own read
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[u], qf[k0 + u], sc, 0, 0, 0);
+        }
         pf_h4 vlo[2][DT], vhi[2][DT];  // into the registers the K fragments leave
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
