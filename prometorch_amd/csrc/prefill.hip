@@ -266,12 +266,15 @@ __global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __r
     constexpr int VP = 64 + 4;         // LDS pitch of a V^T row: 32 positions of fp16 + one word, an ODD number of words
     constexpr int PCS = 32 * HD / 8 / 256;  // 16-byte pieces of a 32-position tile per thread (1 or 2)
     static_assert(PCS == 1 || PCS == 2, "tile smaller than the workgroup");
-    __shared__ __align__(16) uint8_t s_k2[2][32 * KP];
-    __shared__ __align__(16) uint8_t s_vt2[2][HD * VP + 12];
-    __shared__ float s_merge[4][16 * DT + 2][64];  // group 1's accumulators, running maximum and sum, lane-contiguous
+    // LDS: per group a K tile and a transposed V tile; the merge buffer (group 1's accumulators, running maximum and sum,
+    // lane-contiguous) takes the same memory once the tiles are done, which keeps a workgroup under half the CU's LDS
+    constexpr int K_BYTES = 32 * KP, VT_BYTES = (HD * VP + 15) / 16 * 16, STAGE_BYTES = 2 * (K_BYTES + VT_BYTES);
+    constexpr int MERGE_BYTES = 4 * (16 * DT + 2) * 64 * 4;
+    __shared__ __align__(16) uint8_t s_raw[STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES];
+    float (*s_merge)[16 * DT + 2][64] = reinterpret_cast<float (*)[16 * DT + 2][64]>(s_raw);
     const int grp = threadIdx.x >> 8;
-    uint8_t* const s_k = s_k2[grp];
-    uint8_t* const s_vt = s_vt2[grp];
+    uint8_t* const s_k = s_raw + grp * (K_BYTES + VT_BYTES);
+    uint8_t* const s_vt = s_k + K_BYTES;
     const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, kh = lane >> 5;
     const int kvh = blockIdx.y;
@@ -441,6 +444,7 @@ __global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __r
     }
     if (st < nsteps) do_tile(2 * st + grp, kA0, vA0, kA1, vA1);  // workgroup-uniform
     // ---- merge the two groups' states (same lane of waves w and w + 4 = same query vector, same output elements) ----
+    __syncthreads();  // the merge buffer overlays the tiles: every wave has finished its last tile
     if (grp == 1) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
