@@ -50,7 +50,12 @@ int qgemm_f16_reduce_norm_prepare(const float* P, int splits, float* X, bool acc
 int qgemm_f16_splits(int N, int K, int M);
 size_t qgemm_f16_multi_split_bytes(int n, const int* N, const uint32_t* types, int K, int M);
 int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const int64_t* strides, const int* N, float* const* Y,
-                    int M, int K, void* ws_round, void* ws_plain, float* split_ws, size_t split_ws_bytes, hipStream_t s);
+                    int M, int K, void* ws_round, void* ws_plain, float* split_ws, size_t split_ws_bytes, hipStream_t s,
+                    const float** deferred_P, int* deferred_splits);
+int qknorm_rope_kv_rows_from_parts(const float* const* P, const int* splits, const float* const* bias, float* Q,
+                                   const float* q_norm_w, const float* k_norm_w, void* K_cache, void* V_cache,
+                                   const float* rope_table, int rows, int n_heads, int n_kv_heads, int head_dim, int64_t pos0,
+                                   int max_seq, float eps, int add_one, int kv_fp16, int rope_interleaved, hipStream_t s);
 int qgemm_f16_prepare_fused(int pre, const float* X, const float* X2, float eps, int add_one, void* ws_round, void* ws_plain,
                             int M, int K, hipStream_t s);
 int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
@@ -368,12 +373,15 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
             const int64_t s3[3] = {L.q.row_stride_bytes, L.k.row_stride_bytes, L.v.row_stride_bytes};
             const int N3[3] = {L.q.rows, L.k.rows, L.v.rows};
             float* Y3[3] = {d->pf_q, d->pf_k, d->pf_v};
-            PTM_TRY(qgemm_f16_multi(3, t3, W3, s3, N3, Y3, M, H, d->pf_ws, d->pf_ws2, d->pf_split, d->pf_split_bytes, s));
+            // the sum of the K splits (and the biases) is left to the next launch, which reads q, k, v once anyway
+            const float* P3[3];
+            int sp3[3];
+            PTM_TRY(qgemm_f16_multi(3, t3, W3, s3, N3, Y3, M, H, d->pf_ws, d->pf_ws2, d->pf_split, d->pf_split_bytes, s, P3, sp3));
+            const float* b3[3] = {L.q_bias, L.k_bias, L.v_bias};
+            PTM_TRY(qknorm_rope_kv_rows_from_parts(P3, sp3, L.q_bias ? b3 : nullptr, d->pf_q, L.q_norm, L.k_norm, L.k_cache,
+                                                   L.v_cache, local ? d->rope_swa : d->rope, M, c.n_heads, c.n_kv_heads, hd,
+                                                   pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, s));
         }
-        if (L.q_bias) PTM_TRY(ptm_add_qkv_bias(d->pf_q, d->pf_k, d->pf_v, L.q_bias, L.k_bias, L.v_bias, M, qd, kvd, s));
-        PTM_TRY(ptm_qknorm_rope_kvwrite_rows(d->pf_q, d->pf_k, d->pf_v, L.q_norm, L.k_norm, L.k_cache, L.v_cache,
-                                             local ? d->rope_swa : d->rope, M,
-                                             c.n_heads, c.n_kv_heads, hd, pos0, c.max_seq, c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, s));
         PTM_TRY(ptm_prefill_attention_window(d->pf_q, L.k_cache, L.v_cache, d->pf_attn, M, c.n_heads, c.n_kv_heads, hd, pos0,
                                              c.max_seq, 1.0f / sqrtf((float)hd), c.kv_fp16, local ? c.swa_window : 0, s));
         if (L.post_attn_norm) {

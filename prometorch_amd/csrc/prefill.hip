@@ -50,14 +50,40 @@ __global__ __launch_bounds__(256) void embedding_rows_kernel(const float* __rest
     out[(int64_t)m * hidden + i] = v;
 }
 
+// PART: q, k and v arrive as the K-split partial sums a multi-matrix GEMM launch left (per matrix: `splits` slabs of
+// rows x width floats, summed here in slab order, then the optional bias: the arithmetic of the split reduction and of
+// add_qkv_bias_kernel), and only what the attention reads is written: the rotated q rows and the cache rows.
+struct QkvParts {
+    const float* P[3];  // q, k, v; a matrix that was not split points at its finished rows (splits 1)
+    int splits[3];
+    const float* bias[3];  // NULL: none
+};
+__device__ __forceinline__ float qkv_part_load(const float* __restrict__ P, int splits, int64_t total, int64_t idx,
+                                               const float* __restrict__ bias, int col) {
+    // four slabs per batch, fetched unconditionally (the slab index clamped) so that they are in flight together
+    float a = 0.0f;
+    for (int z0 = 0; z0 < splits; z0 += 4) {
+        float b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) b[u] = P[(int64_t)min(z0 + u, splits - 1) * total + idx];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (z0 + u == 0) a = b[u];
+            else if (z0 + u < splits) a += b[u];
+        }
+    }
+    return bias ? a + bias[col] : a;
+}
+
 // grid (rows, n_heads + n_kv_heads), one wave; lane t owns the rotation pair (t, t + head_dim/2)
-template <bool KV16>
+template <bool KV16, bool PART>
 __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restrict__ Q, float* __restrict__ K,
                                                                  const float* __restrict__ V, const float* __restrict__ qw,
                                                                  const float* __restrict__ kw, void* __restrict__ Kc,
                                                                  void* __restrict__ Vc, const float* __restrict__ rope,
                                                                  int n_heads, int n_kv_heads, int head_dim, int64_t pos0,
-                                                                 float eps, int add_one, int rope_interleaved) {
+                                                                 float eps, int add_one, int rope_interleaved,
+                                                                 const QkvParts parts) {
     const int m = blockIdx.x, hb = blockIdx.y;
     const bool is_k = hb >= n_heads;
     const int h = is_k ? hb - n_heads : hb;
@@ -68,6 +94,17 @@ __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restri
     const float* nw = is_k ? kw : qw;
     const int half = head_dim / 2;
     const float* cs = rope + pos * head_dim;
+    const int rows = gridDim.x;
+    const int width = is_k ? kv_dim : n_heads * head_dim;       // row width of the matrix this head belongs to
+    const int64_t row_off = (int64_t)m * width + (int64_t)h * head_dim;
+    auto src = [&](int i) {
+        if constexpr (PART) {
+            const int w = is_k ? 1 : 0;
+            return qkv_part_load(parts.P[w], parts.splits[w], (int64_t)rows * width, row_off + i, parts.bias[w], h * head_dim + i);
+        } else {
+            return vec[i];
+        }
+    };
     // thread t owns rotation pairs t and t + 64 (the second only for heads wider than 128)
     float x0[2], x1[2];
     int i0[2], i1[2];
@@ -78,8 +115,8 @@ __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restri
         on[j] = t < half;
         i0[j] = rope_interleaved ? 2 * t : t;
         i1[j] = rope_interleaved ? 2 * t + 1 : t + half;
-        x0[j] = on[j] ? vec[i0[j]] : 0.0f;
-        x1[j] = on[j] ? vec[i1[j]] : 0.0f;
+        x0[j] = on[j] ? src(i0[j]) : 0.0f;
+        x1[j] = on[j] ? src(i1[j]) : 0.0f;
     }
     if (nw) {
         float ss = fmaf(x0[0], x0[0], 0.0f);
@@ -102,11 +139,20 @@ __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restri
         const int t = threadIdx.x + 64 * j;
         const float c = cs[t], s = cs[half + t];
         const float r0 = fmaf(x0[j], c, -(x1[j] * s)), r1 = fmaf(x0[j], s, x1[j] * c);  // hot_loops.cpp:2035-2061
-        vec[i0[j]] = r0;
-        vec[i1[j]] = r1;
+        if (!PART || !is_k) {  // the rotated fp32 K rows have no reader in the prompt pass
+            vec[i0[j]] = r0;
+            vec[i1[j]] = r1;
+        }
         if (is_k) {
             const int64_t off = pos * kv_dim + (int64_t)h * head_dim;
-            const float v0 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t], v1 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t + half];
+            float v0, v1;
+            if constexpr (PART) {
+                v0 = qkv_part_load(parts.P[2], parts.splits[2], (int64_t)rows * kv_dim, row_off + t, parts.bias[2], h * head_dim + t);
+                v1 = qkv_part_load(parts.P[2], parts.splits[2], (int64_t)rows * kv_dim, row_off + t + half, parts.bias[2], h * head_dim + t + half);
+            } else {
+                v0 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t];
+                v1 = V[(int64_t)m * kv_dim + (int64_t)h * head_dim + t + half];
+            }
             if constexpr (KV16) {
                 __half* kc = static_cast<__half*>(Kc) + off;
                 __half* vc = static_cast<__half*>(Vc) + off;
@@ -514,6 +560,36 @@ static int prefill_attn_launch(int G, dim3 grid, hipStream_t s, const float* Q, 
     return launch_status();
 }
 
+// QK-norm + rotation + cache append of M rows whose q, k, v are still K-split partial sums (P[i]: splits[i] slabs of
+// M x width_i floats; splits 1 = finished rows), optionally with biases: writes Q (rotated) and the cache rows only.
+int qknorm_rope_kv_rows_from_parts(const float* const* P, const int* splits, const float* const* bias, float* Q,
+                                   const float* q_norm_w, const float* k_norm_w, void* K_cache, void* V_cache,
+                                   const float* rope_table, int rows, int n_heads, int n_kv_heads, int head_dim, int64_t pos0,
+                                   int max_seq, float eps, int add_one, int kv_fp16, int rope_interleaved, hipStream_t s) {
+    if (!P || !splits || !Q || !K_cache || !V_cache || !rope_table) return PTM_E_NULL;
+    if ((q_norm_w == nullptr) != (k_norm_w == nullptr)) return PTM_E_NULL;
+    if (rows <= 0 || n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || head_dim <= 0 || (head_dim & 1) || head_dim > 256)
+        return PTM_E_SHAPE;
+    if (pos0 < 0 || pos0 + rows > max_seq) return PTM_E_RANGE;  // never write outside the cache
+    if (n_heads + n_kv_heads > 65535) return PTM_E_UNSUPPORTED;
+    QkvParts parts{};
+    for (int i = 0; i < 3; ++i) {
+        if (!P[i]) return PTM_E_NULL;
+        if (splits[i] < 1) return PTM_E_SHAPE;
+        parts.P[i] = P[i];
+        parts.splits[i] = splits[i];
+        parts.bias[i] = bias ? bias[i] : nullptr;
+    }
+    const dim3 grid(rows, n_heads + n_kv_heads);
+    if (kv_fp16)
+        hipLaunchKernelGGL((qknorm_rope_kv_rows_kernel<true, true>), grid, dim3(64), 0, s, Q, Q, Q, q_norm_w, k_norm_w,
+                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, parts);
+    else
+        hipLaunchKernelGGL((qknorm_rope_kv_rows_kernel<false, true>), grid, dim3(64), 0, s, Q, Q, Q, q_norm_w, k_norm_w,
+                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, parts);
+    return launch_status();
+}
+
 }  // namespace ptm
 
 using namespace ptm;
@@ -542,11 +618,11 @@ int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float
     if (n_heads + n_kv_heads > 65535) return PTM_E_UNSUPPORTED;
     const dim3 grid(rows, n_heads + n_kv_heads);
     if (kv_fp16)
-        hipLaunchKernelGGL(qknorm_rope_kv_rows_kernel<true>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
-                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0);
+        hipLaunchKernelGGL((qknorm_rope_kv_rows_kernel<true, false>), grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
+                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, QkvParts{});
     else
-        hipLaunchKernelGGL(qknorm_rope_kv_rows_kernel<false>, grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
-                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0);
+        hipLaunchKernelGGL((qknorm_rope_kv_rows_kernel<false, false>), grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
+                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, QkvParts{});
     return launch_status();
 }
 

@@ -1119,8 +1119,11 @@ size_t qgemm_f16_multi_split_bytes(int n, const int* N, const uint32_t* types, i
     return 4 * e;
 }
 
+// deferred_P / deferred_splits (optional, n entries each): instead of the reduction launch, where matrix i's partial sums lie
+// (its finished rows Y[i] when it was not split) and how many slabs there are, for the caller's next kernel to fold in.
 int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const int64_t* strides, const int* N, float* const* Y,
-                    int M, int K, void* ws_round, void* ws_plain, float* split_ws, size_t split_ws_bytes, hipStream_t s) {
+                    int M, int K, void* ws_round, void* ws_plain, float* split_ws, size_t split_ws_bytes, hipStream_t s,
+                    const float** deferred_P, int* deferred_splits) {
     if (n < 1 || n > 3) return PTM_E_SHAPE;
     if (M <= 0 || K <= 0 || (K % 256) != 0) return PTM_E_SHAPE;
     const int mp = qf_mpad(M);
@@ -1159,6 +1162,7 @@ int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const in
         m.ntiles = (N[i] + QF_TN - 1) / QF_TN;
         m.q6 = q6 ? 1 : 0;
         m.partials = splits > 1 ? part : nullptr;
+        if (deferred_P) { deferred_P[i] = splits > 1 ? part : Y[i]; deferred_splits[i] = splits; }
         slots += m.ntiles * splits;
         m.slot_end = slots;
         if (splits > 1) {
@@ -1179,7 +1183,7 @@ int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const in
         raised = true;
     }
     hipLaunchKernelGGL(qgemm_f16_multi_kernel, dim3(slots, (M + 127) / 128), dim3(512), 2 * (size_t)128 * QF_PITCH + 4 * 128, s, a, M, K);
-    if (r.n > 0) hipLaunchKernelGGL(qgemm_split_reduce_multi_kernel, dim3(red_blocks), dim3(256), 0, s, r);
+    if (r.n > 0 && !deferred_P) hipLaunchKernelGGL(qgemm_split_reduce_multi_kernel, dim3(red_blocks), dim3(256), 0, s, r);
     return launch_status();
 }
 
