@@ -75,8 +75,9 @@ def bench_lib():
 
 def event_time_ms(fn, iters, torch):
     """Average GPU duration of fn(i) over `iters` launches: the launches are captured into one graph
-    (so the host's per-call cost does not throttle them) and one replay is bracketed by HIP events
-    recorded on the stream the kernels run on."""
+    (so the host's per-call cost does not throttle them) and a replay is bracketed by HIP events
+    recorded on the stream the kernels run on; the median of three replays (a single short replay can
+    fall into a clock transient)."""
     st = torch.cuda.Stream()
     with torch.cuda.stream(st):
         for i in range(4):
@@ -88,12 +89,15 @@ def event_time_ms(fn, iters, torch):
                 fn(i)
         g.replay()
         st.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(st)
-        g.replay()
-        e1.record(st)
-        st.synchronize()
-    return e0.elapsed_time(e1) / iters
+        times = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st)
+            g.replay()
+            e1.record(st)
+            st.synchronize()
+            times.append(e0.elapsed_time(e1))
+    return sorted(times)[1] / iters
 
 
 def main():
