@@ -100,6 +100,39 @@ def event_time_ms(fn, iters, torch):
     return sorted(times)[1] / iters
 
 
+def only_kernel(which, torch, ops, synth):
+    """One prompt-pass kernel by itself, for counter passes: the cfg4 gate-projection GEMM (512 x 4096 x 14336, Q4_K) or the
+    causal attention of 512 / 2048 prompt rows at the Qwen3-4B head shape."""
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e3
+    if which == "prefill_gemm":
+        M, K, N = 512, 4096, 14336
+        W = torch.from_numpy(synth.make_q4k(synth.rng_for(SEED, 5), N, K)).cuda()
+        X = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+        Y = torch.empty(M, N, device="cuda")
+        ws = torch.empty(ops.qgemm_f16_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+        us = timed(lambda: ops.matmul_q_f16(12, W, X, Y, M, K, N, K // 256 * 144, ws), 6)
+        return {"only": which, "shape": [M, K, N], "us_with_row_conversion": us}
+    nh, nkv, hd, max_seq = 32, 8, 128, 2304
+    Kc = torch.randn(max_seq, nkv * hd, device="cuda").half()
+    Vc = torch.randn(max_seq, nkv * hd, device="cuda").half()
+    out = {"only": which}
+    for rows in (512, 2048):
+        Q = torch.randn(rows, nh * hd, device="cuda")
+        O = torch.empty_like(Q)
+        out["us_%d_rows" % rows] = timed(lambda: ops.prefill_attention(Q, Kc, Vc, O, rows, nh, nkv, hd, 0, max_seq, hd ** -0.5, True), 6)
+    return out
+
+
 def main():
     # stdout carries exactly one line, the JSON result: anything a native library prints to file descriptor 1 in the
     # meantime (the compiled reference reports its scratch allocation there) is sent to stderr instead
@@ -116,6 +149,9 @@ def main():
     ap.add_argument("--llama-steps", type=int, default=64,
                     help="decode steps of the Llama-3-8B-shaped extra measurement (0 = skip)")
     ap.add_argument("--layers", type=int, default=36, help=argparse.SUPPRESS)  # debugging only; 36 is the workload
+    ap.add_argument("--only", choices=["prefill_gemm", "prefill_attention"], default=None,
+                    help="launch just this prompt-pass kernel a few times and print its time: the target of the counter "
+                         "passes behind the figures quoted for it (rocprofv3 --pmc ... -- python3 bench.py --only ...)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU (batch-1 decode); --gpus %d is not supported" % args.gpus, file=sys.stderr)
@@ -134,6 +170,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
+    if args.only:
+        os.write(json_fd, (json.dumps(only_kernel(args.only, torch, ops, synth)) + "\n").encode())
+        return
     baseline = json.load(open(os.path.join(ROOT, "BASELINE.json")))
 
     cfg = dict(synth.QWEN3_4B)
@@ -279,11 +318,12 @@ def main():
     Yq = torch.empty(Mq, Nq, device="cuda")
     wsq = torch.empty(max(ops.qgemm_workspace_bytes(Mq, Kq), ops.qgemm_f16_workspace_bytes(Mq, Kq)), dtype=torch.uint8, device="cuda")
     flop = 2.0 * Mq * Kq * Nq
-    msf = event_time_ms(lambda i: ops.matmul_q_f16(12, Wq, Xq, Yq, Mq, Kq, Nq, Kq // 256 * 144, wsq), 20, torch)
+    # 100 launches per replay: shorter bursts of this matrix-core kernel are timed during the clock ramp (85-95 us against 78)
+    msf = event_time_ms(lambda i: ops.matmul_q_f16(12, Wq, Xq, Yq, Mq, Kq, Nq, Kq // 256 * 144, wsq), 100, torch)
     gemv["cfg4_q4k_prefill_gemm_512x4096x14336_f16_mfma"] = {
         "flop": flop, "us": msf * 1e3, "TFLOPs": flop / msf / 1e9, "frac_f16_mfma_peak": flop / msf / 1e9 / 2500.0,
         "numerics": "Q8-rounded activations and dequantised weights in fp16, fp32 accumulate; within 5e-3 of rms(y) of the reference GEMV per row"}
-    msq = event_time_ms(lambda i: ops.matmul_q(12, Wq, Xq, Yq, Mq, Kq, Nq, Kq // 256 * 144, wsq), 20, torch)
+    msq = event_time_ms(lambda i: ops.matmul_q(12, Wq, Xq, Yq, Mq, Kq, Nq, Kq // 256 * 144, wsq), 40, torch)
     gemv["cfg4_q4k_prefill_gemm_512x4096x14336_int8_mfma_exact"] = {
         "ops": flop, "us": msq * 1e3, "TOPs": flop / msq / 1e9, "frac_int8_mfma_peak": flop / msq / 1e9 / 5000.0,
         "numerics": "rows bit-identical to the reference GEMV"}
