@@ -300,7 +300,7 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
     size_t split_elems = 0;  // widest splits x N over the layer's matrices (all layers have the same shapes)
     for (const ptm_qweight* w : {&d->layers[0].q, &d->layers[0].k, &d->layers[0].v, &d->layers[0].o, &d->layers[0].gate,
                                  &d->layers[0].up, &d->layers[0].down}) {
-        for (const int m : {128, 256, rows}) {  // the split count depends on the row class: size for the widest use
+        for (const int m : {128, 256, 1024, rows}) {  // the split count depends on the row class: size for the widest use
             const int mm = m < rows ? m : rows;
             const size_t e = (size_t)qgemm_f16_splits(w->rows, w->cols, mm) * w->rows * (size_t)mm;
             split_elems = e > split_elems ? e : split_elems;
@@ -311,7 +311,7 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
         const ptm_layer& L = d->layers[li];
         const int N3[3] = {L.q.rows, L.k.rows, L.v.rows};
         const uint32_t t3[3] = {L.q.ggml_type, L.k.ggml_type, L.v.ggml_type};
-        for (const int m : {128, 256, rows}) {
+        for (const int m : {128, 256, 1024, rows}) {
             const size_t b = qgemm_f16_multi_split_bytes(3, N3, t3, (int)H, m < rows ? m : rows);
             d->pf_split_bytes = b > d->pf_split_bytes ? b : d->pf_split_bytes;
         }

@@ -959,13 +959,17 @@ __global__ __launch_bounds__(256) void qgemm_split_reduce_multi_kernel(const QfR
     }
 }
 
+// Row classes of the split rules: up to 128 rows, up to 256, up to 1024, more (2048-row chunks of long prompts: with 16 row
+// tiles per column tile, as many splits as a 512-row launch wants only multiply the partial sums).
+static inline int qf_row_class(int M) { return M <= 128 ? 1 : (M <= 256 ? 2 : (M <= 1024 ? 4 : 8)); }
+
 // K splits for an N x K weight matrix and M rows: enough workgroups to fill the chip when N alone gives few column
-// tiles (a 2560-wide projection is 10 tiles).  M enters only through its class (up to 128 rows, up to 256, more), so
+// tiles (a 2560-wide projection is 10 tiles).  M enters only through its class (up to 128 rows, up to 256, up to 1024, more), so
 // that the summation order of a row does not change with how many rows share the launch within a class; short
 // prompts (one row tile) get up to 16 splits, because there the launch is bound by how many workgroups stream weights.
 int qgemm_f16_splits(int N, int K, int M) {
     const int ntiles = (N + QF_TN - 1) / QF_TN, nblk = K / 256;
-    const int row_tiles = M <= 128 ? 1 : (M <= 256 ? 2 : 4);
+    const int row_tiles = qf_row_class(M);
     int s = 256 / (ntiles * row_tiles);
     const int cap = row_tiles == 1 ? 16 : 8;
     s = s > cap ? cap : s;
@@ -980,7 +984,7 @@ int qgemm_f16_splits(int N, int K, int M) {
 // the shapes, the types and M's class only, like qgemm_f16_splits.
 void qgemm_f16_multi_plan(int n, const int* N, const uint32_t* types, int K, int M, int* splits) {
     const int nblk = K / 256;
-    const int row_tiles = M <= 128 ? 1 : (M <= 256 ? 2 : 4);
+    const int row_tiles = qf_row_class(M);
     const int budget = 256 / row_tiles;
     const int cap = (row_tiles == 1 ? 16 : 8) < nblk / 2 ? (row_tiles == 1 ? 16 : 8) : (nblk / 2 < 1 ? 1 : nblk / 2);
     int ntile[3], slots = 0;
