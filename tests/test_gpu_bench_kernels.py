@@ -27,3 +27,23 @@ def test_stream_read_xor_matches_numpy(dev, nbytes):
     want = np.bitwise_xor.reduce(words.reshape(n, 8192), axis=1)
     assert np.array_equal(out.cpu().numpy().view(np.uint32), want)
     assert BL.bench_stream_read_xor(d.data_ptr(), nbytes + 8, out.data_ptr(), s) == -1
+
+
+@pytest.mark.parametrize("which,keys", [("prefill_gemm", ["us_with_row_conversion"]),
+                                        ("prefill_attention", ["us_512_rows", "us_2048_rows"])])
+def test_bench_single_kernel_mode(dev, which, keys):
+    """`bench.py --only <kernel>` (the target of the counter passes quoted in profiles/) runs in a child process and prints
+    one JSON line with positive times."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--only", which], capture_output=True, text=True, timeout=110)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [l for l in p.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1, p.stdout
+    out = json.loads(lines[0])
+    assert out["only"] == which
+    for k in keys:
+        assert 0.0 < out[k] < 1e5, out
