@@ -894,7 +894,8 @@ struct QfMat {
 };
 struct QfMulti { QfMat m[3]; int n_mat; };
 
-__global__ __launch_bounds__(512, 1) void qgemm_f16_multi_kernel(const QfMulti a, int M, int K) {
+template <int MT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, (WAVES == 8 ? 1 : 2)) void qgemm_f16_multi_kernel(const QfMulti a, int M, int K) {
     extern __shared__ __align__(16) uint8_t qf_lds[];
     const int L = qf_xcd_order(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
     int sx, by, unused;
@@ -905,8 +906,8 @@ __global__ __launch_bounds__(512, 1) void qgemm_f16_multi_kernel(const QfMulti a
     const QfMat& q = i == 0 ? a.m[0] : (i == 1 ? a.m[1] : a.m[2]);
     const int local = sx - (i == 0 ? 0 : (i == 1 ? a.m[0].slot_end : a.m[1].slot_end));
     const int bx = local % q.ntiles, bz = local / q.ntiles;
-    if (q.q6) qgemm_f16_body<Q6Tile, 4, 8>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, by, bz, qf_lds);
-    else qgemm_f16_body<Q4Tile, 4, 8>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, by, bz, qf_lds);
+    if (q.q6) qgemm_f16_body<Q6Tile, MT, WAVES>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, by, bz, qf_lds);
+    else qgemm_f16_body<Q4Tile, MT, WAVES>(q.W, q.stride, q.Xh, q.rowscale, q.Y, M, K, q.N, 0, q.bps, q.partials, bx, by, bz, qf_lds);
 }
 
 // Y (+)= partials[0] + partials[1] + ... in that fixed order (deterministic, unlike atomics)
@@ -1011,6 +1012,7 @@ void qgemm_f16_multi_plan(int n, const int* N, const uint32_t* types, int K, int
 // not fit its registers, so it is used only where the big tile would be half empty anyway.  A row's sum does not
 // depend on the choice (same K order).
 static int qgemm_f16_row_tiles(bool q4, int M, int N, int splits) {
+    if (M <= 32) return 1;  // short prompts: a quarter of the X tile traffic, LDS reads and MFMAs of the 128-row tile per block
     if (M <= 64) return 2;
     const int wgs = ((N + QF_TN - 1) / QF_TN) * ((M + 127) / 128) * splits;
     return (q4 && wgs < 128) ? 2 : 4;  // 512 x 2560 x 9728 (152 workgroups): 60 us with 128 rows, 70 with 64; 512 x 4096 x 4096 (64): 80 / 68
@@ -1083,6 +1085,8 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     if (eight && q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (eight) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (q4 && MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    else if (q4 && MT == 1) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 1>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    else if (MT == 1) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 1>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else if (MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
     else hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
@@ -1182,11 +1186,14 @@ int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const in
     }
     static bool raised = false;
     if (!raised) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_multi_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_multi_kernel<4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   2 * 128 * QF_PITCH + 4 * 128);
         raised = true;
     }
-    hipLaunchKernelGGL(qgemm_f16_multi_kernel, dim3(slots, (M + 127) / 128), dim3(512), 2 * (size_t)128 * QF_PITCH + 4 * 128, s, a, M, K);
+    if (M <= 32)  // short prompts: the 32-row tile (see qgemm_f16_row_tiles)
+        hipLaunchKernelGGL((qgemm_f16_multi_kernel<1, 4>), dim3(slots, 1), dim3(256), 2 * (size_t)32 * QF_PITCH + 4 * 32, s, a, M, K);
+    else
+        hipLaunchKernelGGL((qgemm_f16_multi_kernel<4, 8>), dim3(slots, (M + 127) / 128), dim3(512), 2 * (size_t)128 * QF_PITCH + 4 * 128, s, a, M, K);
     if (r.n > 0 && !deferred_P) hipLaunchKernelGGL(qgemm_split_reduce_multi_kernel, dim3(red_blocks), dim3(256), 0, s, r);
     return launch_status();
 }
