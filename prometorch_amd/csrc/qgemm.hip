@@ -349,17 +349,20 @@ __global__ __launch_bounds__(256) void qgemm_prepare_rows_f16_kernel(const void*
 // rms_norm_kernel), PRE 2 = SiLU(gate) * up (the arithmetic of silu_mul_kernel), or tanh-GELU(gate) * up (that of
 // gelu_mul_kernel) when add_one, which has no other meaning for PRE 2, is set.  Writes the Q8-rounded form (for Q4_K
 // matrices) and / or the plain form (for Q6_K matrices) in one pass; either output may be NULL.
-template <int PRE>
-__global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* __restrict__ X, const float* __restrict__ X2,
+// THREADS: 256, or 1024 for PRE 2 on short prompts (one workgroup per row: with few rows the launch lasts as long as one
+// row's dependent chain, which four times the threads shorten; the row maximum does not depend on the thread count).
+template <int PRE, int THREADS = 256>
+__global__ __launch_bounds__(THREADS) void qgemm_prepare_fused_kernel(const float* __restrict__ X, const float* __restrict__ X2,
                                                                   float eps, int add_one, _Float16* __restrict__ Xh_round,
                                                                   float* __restrict__ rs_round, _Float16* __restrict__ Xh_plain,
                                                                   float* __restrict__ rs_plain, int M, int K) {
+    static_assert(PRE == 2 || THREADS == 256, "the RMSNorm sum keeps the 256-thread reduction order");
     __shared__ float red[4];
-    __shared__ float red2[4];
+    __shared__ float red2[THREADS / 64];
     const int m = blockIdx.x, tid = threadIdx.x;
     const int n4 = K / 4;
     if (m >= M) {  // padding rows: zeros
-        for (int i = tid; i < n4; i += 256) {
+        for (int i = tid; i < n4; i += THREADS) {
             if (Xh_round) reinterpret_cast<uint2*>(Xh_round + (int64_t)m * K)[i] = make_uint2(0, 0);
             if (Xh_plain) reinterpret_cast<uint2*>(Xh_plain + (int64_t)m * K)[i] = make_uint2(0, 0);
         }
@@ -371,7 +374,7 @@ __global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* _
     const float one = add_one ? 1.0f : 0.0f;
     if constexpr (PRE == 1) {
         float ss = 0.0f;
-        for (int i = tid; i < K; i += 256) ss = fmaf(x[i], x[i], ss);
+        for (int i = tid; i < K; i += THREADS) ss = fmaf(x[i], x[i], ss);
         ss = block_sum256(ss, red);
         rs = 1.0f / sqrtf(ss / (float)K + eps);
     }
@@ -399,19 +402,19 @@ __global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* _
     // Rows of up to 16384 values are computed once and kept in registers between the maximum and the store pass: all of a
     // thread's loads go out together, and the exponentials of PRE 2 are paid once (the pass is otherwise two dependent
     // sweeps over 2 x 4 K bytes per row).
-    constexpr int HOLD = 16;
-    const bool held = n4 <= HOLD * 256;
+    constexpr int HOLD = 4096 / THREADS;
+    const bool held = n4 <= HOLD * THREADS;
     float4 hv[HOLD];
     float amax = 0.0f;
     if (held) {
 #pragma unroll
         for (int u = 0; u < HOLD; ++u) {
-            const int i = tid + 256 * u;
+            const int i = tid + THREADS * u;
             hv[u] = i < n4 ? value4(i) : make_float4(0.f, 0.f, 0.f, 0.f);
             amax = fmaxf(amax, fmaxf(fmaxf(fabsf(hv[u].x), fabsf(hv[u].y)), fmaxf(fabsf(hv[u].z), fabsf(hv[u].w))));
         }
     } else {
-        for (int i = tid; i < n4; i += 256) {
+        for (int i = tid; i < n4; i += THREADS) {
             const float4 v = value4(i);
             amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
         }
@@ -419,7 +422,12 @@ __global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* _
     amax = max64(amax);
     if ((tid & 63) == 0) red2[tid >> 6] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(red2[0], red2[1]), fmaxf(red2[2], red2[3]));
+    {
+        float t = red2[0];
+#pragma unroll
+        for (int w = 1; w < THREADS / 64; ++w) t = fmaxf(t, red2[w]);
+        amax = t;
+    }
     int e = 0;
     if (amax > 16384.0f) { (void)frexpf(amax, &e); e -= 14; }
     const float down = ldexpf(1.0f, -e);
@@ -451,11 +459,11 @@ __global__ __launch_bounds__(256) void qgemm_prepare_fused_kernel(const float* _
     if (held) {
 #pragma unroll
         for (int u = 0; u < HOLD; ++u) {
-            const int i = tid + 256 * u;
+            const int i = tid + THREADS * u;
             if (i < n4) emit4(i, hv[u]);  // wave-uniform: n4 is a multiple of 64
         }
     } else {
-        for (int i = tid; i < n4; i += 256) emit4(i, value4(i));
+        for (int i = tid; i < n4; i += THREADS) emit4(i, value4(i));
     }
 }
 
@@ -1211,6 +1219,7 @@ int qgemm_f16_prepare_fused(int pre, const float* X, const float* X2, float eps,
     float* rr = hr ? reinterpret_cast<float*>(hr + (int64_t)mp * K) : nullptr;
     float* rp = hp ? reinterpret_cast<float*>(hp + (int64_t)mp * K) : nullptr;
     if (pre == 1) hipLaunchKernelGGL(qgemm_prepare_fused_kernel<1>, dim3(mp), dim3(256), 0, s, X, X2, eps, add_one, hr, rr, hp, rp, M, K);
+    else if (pre == 2 && M <= 128) hipLaunchKernelGGL((qgemm_prepare_fused_kernel<2, 1024>), dim3(mp), dim3(1024), 0, s, X, X2, eps, add_one, hr, rr, hp, rp, M, K);
     else if (pre == 2) hipLaunchKernelGGL(qgemm_prepare_fused_kernel<2>, dim3(mp), dim3(256), 0, s, X, X2, eps, add_one, hr, rr, hp, rp, M, K);
     else return PTM_E_UNSUPPORTED;
     return launch_status();
