@@ -286,7 +286,14 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const float* __restri
 // ---- matrix-core version (fp16 cache) ----------------------------------------------------------------------------
 typedef _Float16 pf_h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 pf_h4 __attribute__((ext_vector_type(4)));
-typedef pf_h4 pf_h4_a4 __attribute__((aligned(4)));
+typedef short pf_s4 __attribute__((ext_vector_type(4)));
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i passes the address of four 16-bit values (a row i / 4 of the caller's
+// choice, columns 4 (i % 4) .. +3 of a 16-column block) and receives column i of the four rows: the transposition a V tile stored
+// position-major needs to become the A operand V^T[d][positions] of the MFMA.
+__device__ __forceinline__ pf_h4 lds_read_tr16(const uint8_t* p) {
+    typedef __attribute__((address_space(3))) pf_s4 lds_s4;
+    return __builtin_bit_cast(pf_h4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)p));
+}
 typedef float pf_f16v __attribute__((ext_vector_type(16)));
 
 // v_mfma_f32_32x32x16_f16 operand layout used below: A (32 x 16): lane l holds row l % 32, summation indices
@@ -294,14 +301,13 @@ typedef float pf_f16v __attribute__((ext_vector_type(16)));
 // l % 32, rows 8 (r / 4) + 4 (l / 32) + r % 4 for r = 0..15.  The summation index may be permuted freely as long as A
 // and B agree, which is used twice: the 16 head-dim elements of a step are [16 ks + 8 kh, +8) for lane half kh,
 // and the 16 positions of a P.V step are the ones the lane already holds in its S^T accumulator.
-// Eight waves in two groups of four: both groups hold the same 32 G-head query rows, group g takes the tiles of 32
-// positions with index = g mod 2 (its own staging buffers; the barriers are shared), and the two online-softmax states are
-// merged through LDS at the end.  A tile is one long dependent chain per wave (stage, barrier, 8 score MFMAs, softmax, 8
-// output MFMAs: about 1.4 us); splitting the positions halves the number of links of a row block's chain and gives each
-// SIMD a second wave to run under the first one's waits.  Tile parity is absolute, so a row's arithmetic does not depend
-// on how the prompt was chunked.
-template <int HD, int G>
-__global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __restrict__ Q, const __half* __restrict__ Kc,
+// NG groups of four waves (256 NG threads): every group holds the same 32 G-head query rows; with two groups, group g takes
+// the pairs of 32-position tiles (4 s + 2 g, 4 s + 2 g + 1) into its own staging buffers (the barriers are shared) and the two
+// online-softmax states are merged through LDS at the end, which halves the number of steps of a row block's chain and gives
+// each SIMD a second wave.  Tile indices are absolute, so with a given NG a row's arithmetic does not depend on how the prompt
+// was chunked.
+template <int HD, int G, int NG>
+__global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float* __restrict__ Q, const __half* __restrict__ Kc,
                                                                 const __half* __restrict__ Vc, float* __restrict__ O, int rows,
                                                                 int n_heads, int n_kv_heads, int64_t pos0, float scale) {
     constexpr int RPW = 32 / G;        // rows per wave (each with its G heads: 32 query vectors)
@@ -309,22 +315,27 @@ __global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __r
     constexpr int KS = HD / 16;        // MFMA steps over the head dimension
     constexpr int DT = HD / 32;        // 32-wide tiles of the output's head dimension
     constexpr int KP = HD * 2 + 16;    // LDS pitch of a K row (bytes)
-    constexpr int VP = 64 + 4;         // LDS pitch of a V^T row: 32 positions of fp16 + one word, an ODD number of words
+    constexpr int VP = HD * 2 + 32;    // LDS pitch of a V row: the four rows of a transposing read fall on different banks
     constexpr int PCS = 32 * HD / 8 / 256;  // 16-byte pieces of a 32-position tile per thread (1 or 2)
     static_assert(PCS == 1 || PCS == 2, "tile smaller than the workgroup");
-    // LDS: per group a K tile and a transposed V tile; the merge buffer (group 1's accumulators, running maximum and sum,
+    // LDS: per group two K tiles and two V tiles; the merge buffer (group 1's accumulators, running maximum and sum,
     // lane-contiguous) takes the same memory once the tiles are done, which keeps a workgroup under half the CU's LDS
-    constexpr int K_BYTES = 32 * KP, VT_BYTES = (HD * VP + 15) / 16 * 16, STAGE_BYTES = 2 * (K_BYTES + VT_BYTES);
-    constexpr int MERGE_BYTES = 4 * (16 * DT + 2) * 64 * 4;
+    constexpr int K_BYTES = 32 * KP, VT_BYTES = 32 * VP, STAGE_BYTES = 2 * NG * (K_BYTES + VT_BYTES);
+    constexpr int MERGE_BYTES = NG == 2 ? 4 * (16 * DT + 2) * 64 * 4 : 0;
     __shared__ __align__(16) uint8_t s_raw[STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES];
     float (*s_merge)[16 * DT + 2][64] = reinterpret_cast<float (*)[16 * DT + 2][64]>(s_raw);
-    const int grp = threadIdx.x >> 8;
-    uint8_t* const s_k = s_raw + grp * (K_BYTES + VT_BYTES);
-    uint8_t* const s_vt = s_k + K_BYTES;
+    const int grp = NG == 2 ? threadIdx.x >> 8 : 0;
+    uint8_t* const s_k = s_raw + grp * 2 * (K_BYTES + VT_BYTES);  // the group's two K tiles, then its two V tiles
+    uint8_t* const s_vt = s_k + 2 * K_BYTES;
     const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, kh = lane >> 5;
-    const int kvh = blockIdx.y;
-    const int m_base = (gridDim.x - 1 - blockIdx.x) * BM;  // longest row blocks are scheduled first
+    // Workgroups start in the order of their linear index, and a row block's work grows with its first row: the index runs
+    // over the kv heads fastest and from the last row block down, so the longest workgroups of ALL heads start first and the
+    // short ones fill the tail (with the heads outermost, a late head's longest blocks would start after the early heads'
+    // short ones and run alone at the end).  With 8 kv heads a head's workgroups also share one XCD and its L2.
+    const int wg = blockIdx.x + gridDim.x * blockIdx.y;
+    const int kvh = wg % (int)gridDim.y;
+    const int m_base = ((int)gridDim.x - 1 - wg / (int)gridDim.y) * BM;
     const int kv_dim = n_kv_heads * HD;
 
     const int row = m_base + wave * RPW + j / G, head = kvh * G + j % G;
@@ -352,113 +363,106 @@ __global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __r
     const int last_row = (m_base + BM < rows ? m_base + BM : rows) - 1;
     const int64_t t_end = pos0 + last_row;  // last position any query of this workgroup attends to
     const int ntiles = (int)(t_end / 32) + 1;
-    // staging: piece q = tid + 256 i of a tile is position q / (HD / 8), elements 8 (q % (HD / 8)) .. +8.
-    // Two tiles are kept in flight (register sets A and B, alternating): the rows come from HBM, and one tile's arithmetic
-    // is shorter than that round trip.  Every fetch is unconditional (tile indices past the end are clamped), so the
-    // number of loads in flight is static and waiting for set A does not wait for set B.
+    // The group's next pair of tiles is in flight in registers (sets A and B) while the current pair is worked on: the rows
+    // come from HBM or L2.  Every fetch is unconditional (tile indices past the end are clamped), so the number of loads in
+    // flight at each wait is static.
     uint4 kA0, kA1, vA0, vA1, kB0, kB1, vB0, vB1;  // scalars, not arrays: they must stay in registers across the loop
     kA1 = vA1 = kB1 = vB1 = make_uint4(0, 0, 0, 0);
-    // K piece i of a thread: position (tid + 256 i) / (HD / 8), elements 8 ((tid + 256 i) % (HD / 8)) .. +8 (a wave reads
-    // whole rows).  V pieces are laid out for the transposed LDS store, where the 64 lanes of a wave write one element
-    // each of rows 8 c + k at column p: a wave takes 16 positions x 4 element groups c, so that with the odd row pitch its
-    // lanes fall on all 32 banks (positions give 8 banks, the 4 groups are 8 banks apart); 4 positions x 16 groups, the K
-    // mapping, puts them on 4 (measured: bank conflicts were 59 % of the LDS cycles of the kernel).
-    auto k_piece = [&](int i, int& p, int& c) { const int q = tid + 256 * i; p = q / (HD / 8); c = q % (HD / 8); };
-    auto v_piece = [&](int i, int& p, int& c) { const int u = wave + 4 * i; p = 16 * (u & 1) + (lane & 15); c = 4 * (u >> 1) + (lane >> 4); };
-    auto piece_off = [&](int tile, int p, int c) {
-        int64_t t = (int64_t)tile * 32 + p;
-        t = t <= t_end ? t : t_end;  // rows past the end are masked below; never read past the appended rows
-        return t * kv_dim + (int64_t)kvh * HD + 8 * c;
-    };
+    // Piece i of a thread, for K and V alike: position (tid + 256 i) / (HD / 8), elements 8 ((tid + 256 i) % (HD / 8)) .. +8 (a
+    // wave reads whole rows).  Byte offsets into the caches fit 32 bits (checked at launch); a piece's offset for a tile is its
+    // offset in tile 0 plus the tile's, clamped to the same piece of the last visible position: rows past the end are masked
+    // below and nothing is read past the appended rows.
+    uint32_t pc_off[PCS], pc_max[PCS], pc_lds_k[PCS], pc_lds_v[PCS];
+#pragma unroll
+    for (int i = 0; i < PCS; ++i) {
+        const int q = tid + 256 * i, p = q / (HD / 8), c = q % (HD / 8);
+        const uint32_t col = (uint32_t)(kvh * HD + 8 * c);
+        pc_off[i] = ((uint32_t)p * (uint32_t)kv_dim + col) * 2u;
+        pc_max[i] = ((uint32_t)t_end * (uint32_t)kv_dim + col) * 2u;
+        pc_lds_k[i] = p * KP + 16 * c;
+        pc_lds_v[i] = p * VP + 16 * c;
+    }
+    const uint32_t tile_bytes = 32u * (uint32_t)kv_dim * 2u;
+    const char* const Kb = reinterpret_cast<const char*>(Kc);
+    const char* const Vb = reinterpret_cast<const char*>(Vc);
     auto fetch = [&](int tile, uint4& k0, uint4& v0, uint4& k1, uint4& v1) {
         tile = tile < ntiles ? tile : ntiles - 1;
-        int p, c;
-        k_piece(0, p, c);
-        k0 = *reinterpret_cast<const uint4*>(Kc + piece_off(tile, p, c));
-        v_piece(0, p, c);
-        v0 = *reinterpret_cast<const uint4*>(Vc + piece_off(tile, p, c));
+        const uint32_t tb = (uint32_t)tile * tile_bytes;
+        const uint32_t o0 = min(pc_off[0] + tb, pc_max[0]);
+        k0 = *reinterpret_cast<const uint4*>(Kb + o0);
+        v0 = *reinterpret_cast<const uint4*>(Vb + o0);
         if constexpr (PCS > 1) {
-            k_piece(1, p, c);
-            k1 = *reinterpret_cast<const uint4*>(Kc + piece_off(tile, p, c));
-            v_piece(1, p, c);
-            v1 = *reinterpret_cast<const uint4*>(Vc + piece_off(tile, p, c));
+            const uint32_t o1 = min(pc_off[1] + tb, pc_max[1]);
+            k1 = *reinterpret_cast<const uint4*>(Kb + o1);
+            v1 = *reinterpret_cast<const uint4*>(Vb + o1);
         }
     };
-    auto stage = [&](int i, const uint4& kr, const uint4& vr) {
-        int p, c;
-        k_piece(i, p, c);
-        *reinterpret_cast<uint4*>(s_k + p * KP + 16 * c) = kr;
-        v_piece(i, p, c);
-        uint8_t* vt = s_vt + (8 * c) * VP + 2 * p;  // transposed: V^T[d][position]
-        *reinterpret_cast<uint16_t*>(vt + 0 * VP) = (uint16_t)vr.x;
-        *reinterpret_cast<uint16_t*>(vt + 1 * VP) = (uint16_t)(vr.x >> 16);
-        *reinterpret_cast<uint16_t*>(vt + 2 * VP) = (uint16_t)vr.y;
-        *reinterpret_cast<uint16_t*>(vt + 3 * VP) = (uint16_t)(vr.y >> 16);
-        *reinterpret_cast<uint16_t*>(vt + 4 * VP) = (uint16_t)vr.z;
-        *reinterpret_cast<uint16_t*>(vt + 5 * VP) = (uint16_t)(vr.z >> 16);
-        *reinterpret_cast<uint16_t*>(vt + 6 * VP) = (uint16_t)vr.w;
-        *reinterpret_cast<uint16_t*>(vt + 7 * VP) = (uint16_t)(vr.w >> 16);
+    auto stage = [&](int buf, int i, const uint4& kr, const uint4& vr) {
+        *reinterpret_cast<uint4*>(s_k + buf * K_BYTES + pc_lds_k[i]) = kr;
+        *reinterpret_cast<uint4*>(s_vt + buf * VT_BYTES + pc_lds_v[i]) = vr;
     };
-    // one tile: stage it from its register set, refill the set with the tile two further on, then the arithmetic
-    auto do_tile = [&](int tile, uint4& k0, uint4& v0, uint4& k1, uint4& v1) {
-        __syncthreads();  // every wave has finished reading the previous tile
-        stage(0, k0, v0);
-        if constexpr (PCS > 1) stage(1, k1, v1);
+    // One step = two adjacent tiles of the group (64 positions): both are staged behind one pair of barriers, their score
+    // MFMA chains are independent (the matrix pipe runs one while the other's operands arrive), and they share one pass of the
+    // online softmax (one maximum, one correction, one rescale test).  The register sets are refilled with the group's next
+    // pair right after staging: in flight during the whole step.
+    auto do_step = [&](int t0) {
+        __syncthreads();  // every wave has finished reading the previous pair
+        stage(0, 0, kA0, vA0);
+        if constexpr (PCS > 1) stage(0, 1, kA1, vA1);
+        stage(1, 0, kB0, vB0);
+        if constexpr (PCS > 1) stage(1, 1, kB1, vB1);
         __syncthreads();
-        fetch(tile + 4, k0, v0, k1, v1);  // the group's tile after next: in flight during two tiles' arithmetic
+        fetch(t0 + 2 * NG, kA0, vA0, kA1, vA1);
+        fetch(t0 + 2 * NG + 1, kB0, vB0, kB1, vB1);
         issue_order_fence();
 
-        // K fragments are read four at a time, so the score MFMAs wait twice for a batch instead of each for its own read
-        // (all eight at once would need 16 more registers than the 256 a wave of this 512-thread workgroup has); the V^T
-        // fragments are requested behind the score MFMAs and arrive under the softmax arithmetic.
-        // S^T tile: rows = the tile's 32 positions, column = this lane's query vector
-        pf_f16v sc;
+        // S^T tiles: rows = a tile's 32 positions, column = this lane's query vector.  K fragments are read four at a time, so
+        // the MFMAs wait for a batch instead of each for its own read.
+        pf_f16v sc[2];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
+        for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int k0 = 0; k0 < KS; k0 += 4) {
-            pf_h8 ka[4];
+            for (int r = 0; r < 16; ++r) sc[u][r] = 0.0f;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) ka[u] = *reinterpret_cast<const pf_h8*>(s_k + j * KP + (16 * (k0 + u) + 8 * kh) * 2);
+        for (int k0 = 0; k0 < KS; k0 += 4)
 #pragma unroll
-            for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(ka[u]));  // no MFMA is moved up to behind its own read
+            for (int u = 0; u < 2; ++u) {
+                pf_h8 ka[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[u], qf[k0 + u], sc, 0, 0, 0);
-        }
-        pf_h4 vlo[2][DT], vhi[2][DT];  // into the registers the K fragments leave
+                for (int w = 0; w < 4; ++w) ka[w] = *reinterpret_cast<const pf_h8*>(s_k + u * K_BYTES + j * KP + (16 * (k0 + w) + 8 * kh) * 2);
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+                for (int w = 0; w < 4; ++w) asm volatile("" : "+v"(ka[w]));  // no MFMA is moved up to behind its own read
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const uint8_t* vrow = s_vt + (32 * dt + j) * VP + (16 * ks + 4 * kh) * 2;
-                vlo[ks][dt] = *reinterpret_cast<const pf_h4_a4*>(vrow);  // rows are 4-byte aligned
-                vhi[ks][dt] = *reinterpret_cast<const pf_h4_a4*>(vrow + 16);
+                for (int w = 0; w < 4; ++w) sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[w], qf[k0 + w], sc[u], 0, 0, 0);
             }
         // only the tiles on the diagonal hold positions some query of the workgroup must not see (workgroup-uniform)
-        if ((int64_t)tile * 32 + 31 > pos0 + m_base) {
-            const int lim = (int)(limit - (int64_t)tile * 32) - 4 * kh;  // position offsets of this lane: 8 (r / 4) + r % 4
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sc[r] = 8 * (r >> 2) + (r & 3) <= lim ? sc[r] : -INFINITY;
+        for (int u = 0; u < 2; ++u) {
+            const int tile = t0 + u;
+            if ((int64_t)tile * 32 + 31 > pos0 + m_base) {
+                issue_order_fence();  // keeps this a branch: as selects it would cost every tile 50 instructions
+                const int lim = (int)(limit - (int64_t)tile * 32) - 4 * kh;  // position offsets of this lane: 8 (r / 4) + r % 4
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sc[u][r] = 8 * (r >> 2) + (r & 3) <= lim ? sc[u][r] : -INFINITY;
+            }
         }
-        float mx = sc[0];
+        float mx = fmaxf(sc[0][0], sc[1][0]);
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // the column's other 16 positions
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(sc[0][r], sc[1][r]));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // the column's other positions
         const float m_new = fmaxf(m_run, mx);
         // group 1 may have seen no visible position of a query yet (-inf): exponentials then take 0 as the reference and are 0
         const float ms = m_new == -INFINITY ? 0.0f : m_new;
         const float corr = __builtin_amdgcn_exp2f(m_run - ms);
         float psum = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            sc[r] = __builtin_amdgcn_exp2f(sc[r] - ms);
-            psum += sc[r];
-        }
-        const pf_h8 pb0 = {(_Float16)sc[0], (_Float16)sc[1], (_Float16)sc[2], (_Float16)sc[3],
-                           (_Float16)sc[4], (_Float16)sc[5], (_Float16)sc[6], (_Float16)sc[7]};
-        const pf_h8 pb1 = {(_Float16)sc[8], (_Float16)sc[9], (_Float16)sc[10], (_Float16)sc[11],
-                           (_Float16)sc[12], (_Float16)sc[13], (_Float16)sc[14], (_Float16)sc[15]};
-        l_run = fmaf(l_run, corr, psum);  // this lane's 16 positions of each tile; the two halves are added at the end
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                sc[u][r] = __builtin_amdgcn_exp2f(sc[u][r] - ms);
+                psum += sc[u][r];
+            }
+        l_run = fmaf(l_run, corr, psum);  // this lane's positions; the two lane halves are added at the end
         // a running maximum that no lane of the wave has raised leaves every correction at exactly 1: the rescale is skipped
         if (__builtin_expect(__builtin_amdgcn_ballot_w64(m_new != m_run) != 0, 0)) {
 #pragma unroll
@@ -467,29 +471,43 @@ __global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __r
                 for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
         }
         m_run = m_new;
-        // O^T += V^T . P^T: step ks sums the positions of accumulator registers 8 ks .. 8 ks + 7
+        // O^T += V^T . P^T: step ks of a tile sums the positions of its accumulator registers 8 ks .. 8 ks + 7
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+        for (int u = 0; u < 2; ++u) {
+            const pf_h8 pb0 = {(_Float16)sc[u][0], (_Float16)sc[u][1], (_Float16)sc[u][2], (_Float16)sc[u][3],
+                               (_Float16)sc[u][4], (_Float16)sc[u][5], (_Float16)sc[u][6], (_Float16)sc[u][7]};
+            const pf_h8 pb1 = {(_Float16)sc[u][8], (_Float16)sc[u][9], (_Float16)sc[u][10], (_Float16)sc[u][11],
+                               (_Float16)sc[u][12], (_Float16)sc[u][13], (_Float16)sc[u][14], (_Float16)sc[u][15]};
+            pf_h4 vlo[2][DT], vhi[2][DT];
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const pf_h4 lo = vlo[ks][dt], hi = vhi[ks][dt];
-                const pf_h8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ks ? pb1 : pb0, acc[dt], 0, 0, 0);
-            }
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    // positions 16 ks + 4 kh .. +3 and the same + 8 of V column 32 dt + j (the lane's S^T rows)
+                    const uint8_t* vrow = s_vt + u * VT_BYTES + (16 * ks + 4 * kh + ((lane & 15) >> 2)) * VP +
+                                          (32 * dt + (j & 16) + 4 * (lane & 3)) * 2;
+                    vlo[ks][dt] = lds_read_tr16(vrow);
+                    vhi[ks][dt] = lds_read_tr16(vrow + 8 * VP);
+                }
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const pf_h4 lo = vlo[ks][dt], hi = vhi[ks][dt];
+                    const pf_h8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ks ? pb1 : pb0, acc[dt], 0, 0, 0);
+                }
+        }
     };
-    // Group g walks tiles g, g + 2, g + 4, ...; a tile index past the end is a tile of masked positions (its fetch is
-    // clamped, its probabilities are exact zeros), so both groups run the same number of steps and meet at every barrier.
-    fetch(grp, kA0, vA0, kA1, vA1);
-    fetch(grp + 2, kB0, vB0, kB1, vB1);
-    // steps in pairs, with nothing conditional between them: the count of loads in flight at each wait stays static
-    const int nsteps = (ntiles + 1) / 2;
-    int st = 0;
-    for (; st + 1 < nsteps; st += 2) {
-        do_tile(2 * st + grp, kA0, vA0, kA1, vA1);
-        do_tile(2 * st + 2 + grp, kB0, vB0, kB1, vB1);
-    }
-    if (st < nsteps) do_tile(2 * st + grp, kA0, vA0, kA1, vA1);  // workgroup-uniform
+    // Group g takes the tile pairs (4 s + 2 g, 4 s + 2 g + 1); a tile index past the end is a tile of masked positions (its
+    // fetch is clamped, its probabilities are exact zeros), so both groups run the same number of steps and meet at every
+    // barrier; nothing is conditional between the steps, so the count of loads in flight at each wait stays static.
+    fetch(2 * grp, kA0, vA0, kA1, vA1);
+    fetch(2 * grp + 1, kB0, vB0, kB1, vB1);
+    const int nsteps = (ntiles + 2 * NG - 1) / (2 * NG);
+    for (int st = 0; st < nsteps; ++st) do_step(2 * NG * st + 2 * grp);
     // ---- merge the two groups' states (same lane of waves w and w + 4 = same query vector, same output elements) ----
+    if constexpr (NG == 2) {
     __syncthreads();  // the merge buffer overlays the tiles: every wave has finished its last tile
     if (grp == 1) {
 #pragma unroll
@@ -511,6 +529,7 @@ __global__ __launch_bounds__(512) void prefill_attn_mfma_kernel(const float* __r
             for (int r = 0; r < 16; ++r) acc[dt][r] = fmaf(acc[dt][r], c0, s_merge[wave][16 * dt + r][lane] * c1);
         l_run = fmaf(l_run, c0, l1 * c1);
     }
+    }
     const float l = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = 1.0f / (l + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
     if (row < rows) {
@@ -529,7 +548,16 @@ static int prefill_attn_mfma_launch(int G, hipStream_t s, const float* Q, const 
                                     int n_heads, int n_kv_heads, int64_t pos0, float scale) {
     const int bm = 128 / G;
     const dim3 grid((rows + bm - 1) / bm, n_kv_heads);
-#define PTM_PA(GG) hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG>), grid, dim3(512), 0, s, Q, static_cast<const __half*>(Kc), static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale)
+    // up to 128 rows a row block has at most four tiles of its own chunk to share out: one group of four waves per workgroup
+    // (no merge, half the threads to start) is 2 - 3 us faster there; beyond, two groups split the tiles
+    const bool one = rows <= 128;
+#define PTM_PA(GG)                                                                                                          \
+    if (one)                                                                                                                \
+        hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG, 1>), grid, dim3(256), 0, s, Q, static_cast<const __half*>(Kc), \
+                           static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale);                      \
+    else                                                                                                                    \
+        hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG, 2>), grid, dim3(512), 0, s, Q, static_cast<const __half*>(Kc), \
+                           static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale)
     switch (G) {
         case 1: PTM_PA(1); break;
         case 2: PTM_PA(2); break;
@@ -651,7 +679,9 @@ int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void
         return kv_fp16 ? prefill_attn_launch<true, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
                        : prefill_attn_launch<false, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
     }
-    if (window == 0 && kv_fp16 && rows >= PTM_PREFILL_MFMA_MIN_ROWS && (G == 1 || G == 2 || G == 4 || G == 8))
+    // the MFMA kernel addresses the caches with 32-bit byte offsets
+    const bool offsets_fit = (pos0 + rows) * (int64_t)n_kv_heads * head_dim * 2 < ((int64_t)1 << 32);
+    if (window == 0 && kv_fp16 && offsets_fit && rows >= PTM_PREFILL_MFMA_MIN_ROWS && (G == 1 || G == 2 || G == 4 || G == 8))
         return head_dim == 128 ? prefill_attn_mfma_launch<128>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
                                : prefill_attn_mfma_launch<64>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
     if (kv_fp16)
