@@ -324,7 +324,7 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     constexpr int MERGE_BYTES = NG == 2 ? 4 * (16 * DT + 2) * 64 * 4 : 0;
     __shared__ __align__(16) uint8_t s_raw[STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES];
     float (*s_merge)[16 * DT + 2][64] = reinterpret_cast<float (*)[16 * DT + 2][64]>(s_raw);
-    const int grp = NG == 2 ? threadIdx.x >> 8 : 0;
+    const int grp = NG == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 8) : 0;  // wave-uniform: tile counters stay scalar
     uint8_t* const s_k = s_raw + grp * 2 * (K_BYTES + VT_BYTES);  // the group's two K tiles, then its two V tiles
     uint8_t* const s_vt = s_k + 2 * K_BYTES;
     const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
@@ -446,9 +446,11 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
                 for (int r = 0; r < 16; ++r) sc[u][r] = 8 * (r >> 2) + (r & 3) <= lim ? sc[u][r] : -INFINITY;
             }
         }
-        float mx = fmaxf(sc[0][0], sc[1][0]);
+        // v_max3_f32 by hand: fmaxf() first quiets each MFMA result with an instruction of its own (no NaN can occur here)
+        float mx = sc[0][0];
+        asm("v_max_f32 %0, %0, %1" : "+v"(mx) : "v"(sc[1][0]));
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(sc[0][r], sc[1][r]));
+        for (int r = 1; r < 16; ++r) asm("v_max3_f32 %0, %0, %1, %2" : "+v"(mx) : "v"(sc[0][r]), "v"(sc[1][r]));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // the column's other positions
         const float m_new = fmaxf(m_run, mx);
         // group 1 may have seen no visible position of a query yet (-inf): exponentials then take 0 as the reference and are 0
