@@ -49,6 +49,7 @@ int qgemm_f16_reduce_norm_prepare(const float* P, int splits, float* X, bool acc
                                   int add_one, void* ws_round, void* ws_plain, int M, int K, hipStream_t s);
 int qgemm_f16_splits(int N, int K, int M);
 size_t qgemm_f16_multi_split_bytes(int n, const int* N, const uint32_t* types, int K, int M);
+void qgemm_f16_multi_plan(int n, const int* N, const uint32_t* types, int K, int M, int* splits);
 int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const int64_t* strides, const int* N, float* const* Y,
                     int M, int K, void* ws_round, void* ws_plain, float* split_ws, size_t split_ws_bytes, hipStream_t s,
                     const float** deferred_P, int* deferred_splits);
@@ -311,9 +312,13 @@ static int prefill_alloc(ptm_decoder* d, int rows) {
         const ptm_layer& L = d->layers[li];
         const int N3[3] = {L.q.rows, L.k.rows, L.v.rows};
         const uint32_t t3[3] = {L.q.ggml_type, L.k.ggml_type, L.v.ggml_type};
+        const int N2[2] = {L.gate.rows, L.up.rows};  // so may gate and up
+        const uint32_t t2[2] = {L.gate.ggml_type, L.up.ggml_type};
         for (const int m : {128, 256, 1024, rows}) {
             const size_t b = qgemm_f16_multi_split_bytes(3, N3, t3, (int)H, m < rows ? m : rows);
             d->pf_split_bytes = b > d->pf_split_bytes ? b : d->pf_split_bytes;
+            const size_t b2 = qgemm_f16_multi_split_bytes(2, N2, t2, (int)H, m < rows ? m : rows);
+            d->pf_split_bytes = b2 > d->pf_split_bytes ? b2 : d->pf_split_bytes;
         }
     }
     const size_t o_split = take(d->pf_split_bytes);
@@ -392,8 +397,33 @@ static int prefill_chunk(ptm_decoder* d, const int* tokens_host, int M, int64_t 
         }
         PTM_TRY(norm_rows(pending, L.ffn_norm, uses(PTM_TYPE_Q4_K, {&L.gate, &L.up}), uses(PTM_TYPE_Q6_K, {&L.gate, &L.up})));
         pending = 0;
-        PTM_TRY(gemm(L.gate, d->pf_x, d->pf_gate, false, true));
-        PTM_TRY(gemm(L.up, d->pf_x, d->pf_up, false, true));
+        {
+            // Gate and up share one launch when that fills the chip better.  The eight-wave tile runs one workgroup per CU, so
+            // a launch costs ceil(tiles / 256) workgroup times: 2048 rows are 38 x 16 = 608 tiles per matrix, 3 + 3 rounds
+            // apart and 5 together; 512 rows, 152 tiles each, gain nothing (1 + 1 against 2).  Up to 256 rows (the two
+            // short row classes) always together: one launch less, and the launch is the cost there.  Beyond, only when both
+            // ways use the same K splits, so that the choice changes no result.
+            const uint32_t t2[2] = {L.gate.ggml_type, L.up.ggml_type};
+            const int N2[2] = {L.gate.rows, L.up.rows};
+            bool together = M <= 256;
+            if (!together) {
+                int sp2[2];
+                qgemm_f16_multi_plan(2, N2, t2, (int)H, M, sp2);
+                const int row_tiles = (M + 127) / 128;
+                const int tg = (N2[0] + 255) / 256 * row_tiles * sp2[0], tu = (N2[1] + 255) / 256 * row_tiles * sp2[1];
+                together = sp2[0] == qgemm_f16_splits(N2[0], (int)H, M) && sp2[1] == qgemm_f16_splits(N2[1], (int)H, M) &&
+                           (tg + tu + 255) / 256 < (tg + 255) / 256 + (tu + 255) / 256;
+            }
+            if (together) {
+                const void* W2[2] = {L.gate.data, L.up.data};
+                const int64_t s2[2] = {L.gate.row_stride_bytes, L.up.row_stride_bytes};
+                float* Y2[2] = {d->pf_gate, d->pf_up};
+                PTM_TRY(qgemm_f16_multi(2, t2, W2, s2, N2, Y2, M, H, d->pf_ws, d->pf_ws2, d->pf_split, d->pf_split_bytes, s, nullptr, nullptr));
+            } else {
+                PTM_TRY(gemm(L.gate, d->pf_x, d->pf_gate, false, true));
+                PTM_TRY(gemm(L.up, d->pf_x, d->pf_up, false, true));
+            }
+        }
         const bool act_ready = true;
         // SiLU.up (or, flagged through the add_one slot, GELU.up) fused into the conversion for the down projection
         PTM_TRY(qgemm_f16_prepare_fused(2, d->pf_gate, d->pf_up, 0.0f, c.ffn_gelu ? 1 : 0,
