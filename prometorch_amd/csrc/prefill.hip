@@ -315,7 +315,8 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     constexpr int KS = HD / 16;        // MFMA steps over the head dimension
     constexpr int DT = HD / 32;        // 32-wide tiles of the output's head dimension
     constexpr int KP = HD * 2 + 16;    // LDS pitch of a K row (bytes)
-    constexpr int VP = HD * 2 + 32;    // LDS pitch of a V row: the four rows of a transposing read fall on different banks
+    constexpr int VP = HD * 2 + 64;    // LDS pitch of a V row: 16 of the 64 banks on: the 32 lanes served together by a transposing
+                                       // read (4 rows x 2 blocks of 16 columns) cover all banks (measured: 191 ns per 64 KB against 238 with + 32)
     constexpr int PCS = 32 * HD / 8 / 256;  // 16-byte pieces of a 32-position tile per thread (1 or 2)
     static_assert(PCS == 1 || PCS == 2, "tile smaller than the workgroup");
     // LDS: per group two K tiles and two V tiles; the merge buffer (group 1's accumulators, running maximum and sum,
