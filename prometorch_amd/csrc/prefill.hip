@@ -172,6 +172,160 @@ __global__ __launch_bounds__(64) void qknorm_rope_kv_rows_kernel(float* __restri
     }
 }
 
+// Four values of a q / k / v row that may still be K-split partial sums: slab z holds them at P + z * total + idx
+__device__ __forceinline__ float4 qkv_part_load4(const float* __restrict__ P, int splits, int64_t total, int64_t idx,
+                                                 const float* __restrict__ bias, int col) {
+    float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int z0 = 0; z0 < splits; z0 += 4) {  // four slabs per batch, the slab index clamped: in flight together
+        float4 b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) b[u] = *reinterpret_cast<const float4*>(P + (int64_t)min(z0 + u, splits - 1) * total + idx);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (z0 + u == 0) a = b[u];
+            else if (z0 + u < splits) { a.x += b[u].x; a.y += b[u].y; a.z += b[u].z; a.w += b[u].w; }
+        }
+    }
+    if (bias) {
+        const float4 bb = *reinterpret_cast<const float4*>(bias + col);
+        a.x += bb.x; a.y += bb.y; a.z += bb.z; a.w += bb.w;
+    }
+    return a;
+}
+
+// The same work with head_dim / 8 lanes per head (head_dim 32, 64, 128 or 256) and 16-byte accesses: a lane owns four
+// rotation pairs (two runs of four elements), a wave 64 / (head_dim / 8) heads of one row.  grid (rows, q head blocks + kv
+// head blocks), one wave.  With one wave per (row, head) and 4-byte accesses the launch was bound by the number of
+// workgroups and requests: 82 k single-wave workgroups for 2048 rows of 40 heads.
+template <bool KV16, bool PART>
+__global__ __launch_bounds__(64) void qknorm_rope_kv_rows_quad_kernel(float* __restrict__ Q, float* __restrict__ K,
+                                                                      const float* __restrict__ V, const float* __restrict__ qw,
+                                                                      const float* __restrict__ kw, void* __restrict__ Kc,
+                                                                      void* __restrict__ Vc, const float* __restrict__ rope,
+                                                                      int n_heads, int n_kv_heads, int head_dim, int64_t pos0,
+                                                                      float eps, int add_one, int rope_interleaved,
+                                                                      const QkvParts parts) {
+    const int m = blockIdx.x, rows = gridDim.x;
+    const int lph = head_dim >> 3, hpw = 64 / lph;  // lanes per head, heads per wave
+    const int q_blocks = (n_heads + hpw - 1) / hpw;
+    const bool is_k = (int)blockIdx.y >= q_blocks;
+    const int hblk = is_k ? blockIdx.y - q_blocks : blockIdx.y;
+    const int lane = threadIdx.x, l = lane & (lph - 1);
+    const int nh = is_k ? n_kv_heads : n_heads;
+    const int h_raw = hblk * hpw + lane / lph;
+    const bool live = h_raw < nh;
+    const int h = live ? h_raw : nh - 1;  // idle lanes of the last block read the last head and store nothing
+    const int half = head_dim / 2, kv_dim = n_kv_heads * head_dim;
+    const int64_t pos = pos0 + m;
+    // the lane's two runs: NeoX pairs (4 l + e, half + 4 l + e); interleaved pairs (8 l + 2 e, 8 l + 2 e + 1) lie in
+    // elements 8 l .. 8 l + 7.  Either way they are the pairs 4 l .. 4 l + 3 of the rotation table.
+    const int e0 = rope_interleaved ? 8 * l : 4 * l, e1 = rope_interleaved ? 8 * l + 4 : half + 4 * l;
+    const int width = is_k ? kv_dim : n_heads * head_dim;
+    const int64_t row_off = (int64_t)m * width + (int64_t)h * head_dim;
+    float* vec = (is_k ? K : Q) + row_off;
+    const int w = is_k ? 1 : 0;
+    float4 a, b, va, vb;
+    va = vb = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if constexpr (PART) {
+        const int64_t total = (int64_t)rows * width;
+        a = qkv_part_load4(parts.P[w], parts.splits[w], total, row_off + e0, parts.bias[w], h * head_dim + e0);
+        b = qkv_part_load4(parts.P[w], parts.splits[w], total, row_off + e1, parts.bias[w], h * head_dim + e1);
+        if (is_k) {
+            va = qkv_part_load4(parts.P[2], parts.splits[2], total, row_off + e0, parts.bias[2], h * head_dim + e0);
+            vb = qkv_part_load4(parts.P[2], parts.splits[2], total, row_off + e1, parts.bias[2], h * head_dim + e1);
+        }
+    } else {
+        a = *reinterpret_cast<const float4*>(vec + e0);
+        b = *reinterpret_cast<const float4*>(vec + e1);
+        if (is_k) {
+            va = *reinterpret_cast<const float4*>(V + row_off + e0);
+            vb = *reinterpret_cast<const float4*>(V + row_off + e1);
+        }
+    }
+    const float* cs = rope + pos * head_dim;
+    const float4 c4 = *reinterpret_cast<const float4*>(cs + 4 * l), s4 = *reinterpret_cast<const float4*>(cs + half + 4 * l);
+    const float* nw = is_k ? kw : qw;
+    if (nw) {
+        float ss = fmaf(a.x, a.x, 0.0f);
+        ss = fmaf(a.y, a.y, ss); ss = fmaf(a.z, a.z, ss); ss = fmaf(a.w, a.w, ss);
+        ss = fmaf(b.x, b.x, ss); ss = fmaf(b.y, b.y, ss); ss = fmaf(b.z, b.z, ss); ss = fmaf(b.w, b.w, ss);
+        for (int o = lph >> 1; o >= 1; o >>= 1) ss += __shfl_xor(ss, o, 64);  // within the head's lanes
+        const float rs = 1.0f / sqrtf(ss / (float)head_dim + eps);
+        const float one = add_one ? 1.0f : 0.0f;
+        const float4 wa = *reinterpret_cast<const float4*>(nw + e0), wb = *reinterpret_cast<const float4*>(nw + e1);
+        a.x = a.x * rs * (wa.x + one); a.y = a.y * rs * (wa.y + one); a.z = a.z * rs * (wa.z + one); a.w = a.w * rs * (wa.w + one);
+        b.x = b.x * rs * (wb.x + one); b.y = b.y * rs * (wb.y + one); b.z = b.z * rs * (wb.z + one); b.w = b.w * rs * (wb.w + one);
+    }
+    // rotation of pair (x0, x1) by (c, s): (x0 c - x1 s, x0 s + x1 c)  (hot_loops.cpp:2035-2061)
+    auto rot = [](float& x0, float& x1, float c, float s) {
+        const float r0 = fmaf(x0, c, -(x1 * s)), r1 = fmaf(x0, s, x1 * c);
+        x0 = r0;
+        x1 = r1;
+    };
+    if (rope_interleaved) {
+        rot(a.x, a.y, c4.x, s4.x); rot(a.z, a.w, c4.y, s4.y); rot(b.x, b.y, c4.z, s4.z); rot(b.z, b.w, c4.w, s4.w);
+    } else {
+        rot(a.x, b.x, c4.x, s4.x); rot(a.y, b.y, c4.y, s4.y); rot(a.z, b.z, c4.z, s4.z); rot(a.w, b.w, c4.w, s4.w);
+    }
+    if (!live) return;
+    if (!PART || !is_k) {  // the rotated fp32 K rows have no reader in the prompt pass
+        *reinterpret_cast<float4*>(vec + e0) = a;
+        *reinterpret_cast<float4*>(vec + e1) = b;
+    }
+    if (is_k) {
+        const int64_t off = pos * kv_dim + (int64_t)h * head_dim;
+        if constexpr (KV16) {
+            auto pack = [](const float4& v) {
+                const __half2 lo = __floats2half2_rn(v.x, v.y), hi = __floats2half2_rn(v.z, v.w);
+                uint2 r;
+                __builtin_memcpy(&r.x, &lo, 4);
+                __builtin_memcpy(&r.y, &hi, 4);
+                return r;
+            };
+            __half* kc = static_cast<__half*>(Kc) + off;
+            __half* vc = static_cast<__half*>(Vc) + off;
+            *reinterpret_cast<uint2*>(kc + e0) = pack(a);
+            *reinterpret_cast<uint2*>(kc + e1) = pack(b);
+            *reinterpret_cast<uint2*>(vc + e0) = pack(va);
+            *reinterpret_cast<uint2*>(vc + e1) = pack(vb);
+        } else {
+            float* kc = static_cast<float*>(Kc) + off;
+            float* vc = static_cast<float*>(Vc) + off;
+            *reinterpret_cast<float4*>(kc + e0) = a;
+            *reinterpret_cast<float4*>(kc + e1) = b;
+            *reinterpret_cast<float4*>(vc + e0) = va;
+            *reinterpret_cast<float4*>(vc + e1) = vb;
+        }
+    }
+}
+
+// launches the 16-byte kernel when the shape and the pointers allow it, the one-wave-per-head kernel otherwise
+template <bool PART>
+static int qknorm_rope_kv_rows_launch(float* Q, float* K, const float* V, const float* q_norm_w, const float* k_norm_w,
+                                      void* K_cache, void* V_cache, const float* rope_table, int rows, int n_heads,
+                                      int n_kv_heads, int head_dim, int64_t pos0, float eps, int add_one, int kv_fp16,
+                                      int rope_interleaved, const QkvParts& parts, hipStream_t s) {
+    bool quad = head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256;
+    quad = quad && aligned16(Q) && aligned16(K) && aligned16(V) && aligned16(q_norm_w) && aligned16(k_norm_w) &&
+           aligned16(K_cache) && aligned16(V_cache) && aligned16(rope_table);
+    for (int i = 0; i < 3; ++i) quad = quad && aligned16(parts.P[i]) && aligned16(parts.bias[i]);
+#define PTM_QK(KERNEL, KV16, GRID)                                                                                         \
+    hipLaunchKernelGGL((KERNEL<KV16, PART>), GRID, dim3(64), 0, s, Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, rope_table, \
+                       n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, parts)
+    if (quad) {
+        const int hpw = 64 / (head_dim / 8);
+        const dim3 grid(rows, (n_heads + hpw - 1) / hpw + (n_kv_heads + hpw - 1) / hpw);
+        if (kv_fp16) PTM_QK(qknorm_rope_kv_rows_quad_kernel, true, grid);
+        else PTM_QK(qknorm_rope_kv_rows_quad_kernel, false, grid);
+    } else {
+        const dim3 grid(rows, n_heads + n_kv_heads);
+        if (kv_fp16) PTM_QK(qknorm_rope_kv_rows_kernel, true, grid);
+        else PTM_QK(qknorm_rope_kv_rows_kernel, false, grid);
+    }
+#undef PTM_QK
+    return launch_status();
+}
+
 template <bool KV16>
 __device__ __forceinline__ void pf_load8(const void* base, int64_t elem_off, float (&o)[8]) {
     if constexpr (KV16) {
@@ -611,14 +765,8 @@ int qknorm_rope_kv_rows_from_parts(const float* const* P, const int* splits, con
         parts.splits[i] = splits[i];
         parts.bias[i] = bias ? bias[i] : nullptr;
     }
-    const dim3 grid(rows, n_heads + n_kv_heads);
-    if (kv_fp16)
-        hipLaunchKernelGGL((qknorm_rope_kv_rows_kernel<true, true>), grid, dim3(64), 0, s, Q, Q, Q, q_norm_w, k_norm_w,
-                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, parts);
-    else
-        hipLaunchKernelGGL((qknorm_rope_kv_rows_kernel<false, true>), grid, dim3(64), 0, s, Q, Q, Q, q_norm_w, k_norm_w,
-                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, parts);
-    return launch_status();
+    return qknorm_rope_kv_rows_launch<true>(Q, Q, Q, q_norm_w, k_norm_w, K_cache, V_cache, rope_table, rows, n_heads, n_kv_heads,
+                                            head_dim, pos0, eps, add_one, kv_fp16, rope_interleaved, parts, s);
 }
 
 }  // namespace ptm
@@ -647,14 +795,8 @@ int ptm_qknorm_rope_kvwrite_rows(float* Q, float* K, const float* V, const float
         return PTM_E_SHAPE;
     if (pos0 < 0 || pos0 + rows > max_seq) return PTM_E_RANGE;  // never write outside the cache
     if (n_heads + n_kv_heads > 65535) return PTM_E_UNSUPPORTED;
-    const dim3 grid(rows, n_heads + n_kv_heads);
-    if (kv_fp16)
-        hipLaunchKernelGGL((qknorm_rope_kv_rows_kernel<true, false>), grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
-                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, QkvParts{});
-    else
-        hipLaunchKernelGGL((qknorm_rope_kv_rows_kernel<false, false>), grid, dim3(64), 0, as_stream(stream), Q, K, V, q_norm_w, k_norm_w,
-                           K_cache, V_cache, rope_table, n_heads, n_kv_heads, head_dim, pos0, eps, add_one, rope_interleaved ? 1 : 0, QkvParts{});
-    return launch_status();
+    return qknorm_rope_kv_rows_launch<false>(Q, K, V, q_norm_w, k_norm_w, K_cache, V_cache, rope_table, rows, n_heads, n_kv_heads,
+                                             head_dim, pos0, eps, add_one, kv_fp16, rope_interleaved, QkvParts{}, as_stream(stream));
 }
 
 int ptm_prefill_attention(const float* Q, const void* K_cache, const void* V_cache, float* O, int rows, int n_heads,
