@@ -65,7 +65,10 @@ def test_embedding_rows_rejects_bad_arguments(dev):
 
 
 @pytest.mark.parametrize("kv_fp16", [True, False])
-@pytest.mark.parametrize("nh,nkv,hd,pos0,rows", [(32, 8, 128, 2040, 9), (4, 2, 64, 0, 21), (8, 8, 128, 5, 3), (8, 4, 256, 5, 7)])
+@pytest.mark.parametrize("nh,nkv,hd,pos0,rows", [(32, 8, 128, 2040, 9), (4, 2, 64, 0, 21), (8, 8, 128, 5, 3), (8, 4, 256, 5, 7),
+                                                 (6, 2, 128, 3, 5),   # head counts that leave lanes of the last wave idle
+                                                 (3, 1, 64, 0, 4),
+                                                 (6, 2, 96, 3, 5)])   # a head width served by the one-wave-per-head kernel
 def test_qknorm_rope_kvwrite_rows_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, pos0, rows):
     max_seq = pos0 + rows + 3
     r = synth.rng_for(62, nh, hd, pos0)
