@@ -497,6 +497,46 @@ def test_qwen3_4b_shape_prefill_64_tokens(dev, po, seeds):
     dec.close()
 
 
+@pytest.mark.parametrize("n,chunk", [(1100, 0), (1100, 512), (1100, 300), (2048, 0)])
+def test_long_prompt_prefill_matches_token_by_token_decode(dev, seeds, n, chunk):
+    """The row classes real prompts run in (257..1024 rows, more than 1024; gate and up in one launch; two wave groups in
+    the attention): three full-width Qwen3-4B layers, the prompt prefilled in chunks of that size against the same decoder
+    fed one token at a time (the decode step is pinned against the oracle elsewhere).  Size-independent property:
+    prefill and stepping compute the same function.  A random-weight model amplifies the Q8 rounding noise of single
+    positions (see check_kv_rows), so the logits are compared at five prompt lengths and the bar is on their median, with
+    no length allowed to be far off."""
+    from prometorch_amd.decode import Decoder
+    cfg = dict(synth.QWEN3_4B)
+    cfg["n_layers"] = 3
+    seed = seeds["cfg4"]
+    layers = [synth.make_layer(seed, i, cfg) for i in range(3)]
+    head = synth.make_head(seed, cfg)
+    dec = Decoder(cfg, layers, head, max_seq=n + 16, kv_fp16=True, use_graph=True)
+    prompt = [int(t) for t in synth.rng_for(70, n).integers(0, cfg["vocab"], n)]
+    ends = list(range(n - 4, n + 1))
+    want, want_tok = {}, {}
+    for i, t in enumerate(prompt):
+        tok = dec.step(t)
+        if i + 1 in ends:
+            want[i + 1], want_tok[i + 1] = dec.logits().copy(), tok
+    want_k = [dec.k_cache[li][:n].float().cpu().numpy() for li in range(3)]
+    want_v = [dec.v_cache[li][:n].float().cpu().numpy() for li in range(3)]
+    rmss = []
+    for e in ends:
+        dec.set_past_len(0)
+        tok_p = dec.prefill(prompt[:e], chunk_rows=chunk)
+        err, rms, margin = logit_errors(dec.logits(), want[e])
+        rmss.append(rms)
+        if margin > 2 * err:
+            assert tok_p == want_tok[e], (e, margin, err)
+    print("prefill %d tokens chunk %d vs stepping: logit rms err/std at 5 lengths %s" % (n, chunk, ["%.1e" % r for r in rmss]), flush=True)
+    assert np.median(rmss) <= E2E_RMS_TOL and max(rmss) <= 0.25, rmss
+    for li in range(3):  # the cache as the last (full-length) prefill left it
+        check_kv_rows(dec.k_cache[li][:n].float().cpu().numpy(), want_k[li], li, "k")
+        check_kv_rows(dec.v_cache[li][:n].float().cpu().numpy(), want_v[li], li, "v")
+    dec.close()
+
+
 def test_qgemm_f16_random_shapes_vs_oracle(dev, po):
     """A fixed pseudo-random sweep of the fast prefill GEMM over row counts (both tile heights, ragged last tiles),
     widths and lengths (split and unsplit K), both weight types, against the oracle's row-by-row GEMVs."""
