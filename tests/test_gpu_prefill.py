@@ -497,7 +497,7 @@ def test_qwen3_4b_shape_prefill_64_tokens(dev, po, seeds):
     dec.close()
 
 
-@pytest.mark.parametrize("n,chunk", [(1100, 0), (1100, 512), (1100, 300), (2048, 0)])
+@pytest.mark.parametrize("n,chunk", [(1100, 0), (1100, 512), (1100, 1024), (1100, 300), (2048, 0)])
 def test_long_prompt_prefill_matches_token_by_token_decode(dev, seeds, n, chunk):
     """The row classes real prompts run in (257..1024 rows, more than 1024; gate and up in one launch; two wave groups in
     the attention): three full-width Qwen3-4B layers, the prompt prefilled in chunks of that size against the same decoder
