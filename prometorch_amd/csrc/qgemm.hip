@@ -656,10 +656,10 @@ struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh
 // of the current block, followed by the next block's weights, and written to the other LDS buffer during steps
 // 3..6, so the block ends with the next tile complete behind the only workgroup barrier of the block.  (After the
 // last block the same code re-fetches the last tile into the idle buffer: no conditionals in the steady-state loop.)
-// WAVES = 4: a wave owns 64 columns (two 32-column tiles) and all MT row tiles.  WAVES = 8 (MT = 4): waves w and w + 4
-// own one 32-column tile each of the same 64 columns, so a SIMD holds two waves and one's dequantisation and LDS reads
-// run under the other's MFMAs (the two pipes of a single wave barely overlap); no weight is dequantised twice, the X
-// tile in LDS is read by twice as many waves.
+// WAVES = 8 (what is launched, for every tile height): waves w and w + 4 own one 32-column strip each of the same 64
+// columns and all MT row tiles, so a SIMD holds two waves and one's dequantisation and LDS reads run under the other's
+// MFMAs (the two pipes of a single wave barely overlap); no weight is dequantised twice, the X tile in LDS is read by twice
+// as many waves.  WAVES = 4 (a wave owns both strips) is the layout this grew from: slower at every height.
 // (bx, by, bz) = (column tile, row tile, K split) of this workgroup; s_a = its dynamic LDS
 template <typename Tile, int MT, int WAVES>
 __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride, const _Float16* Xh,
@@ -672,7 +672,8 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
     constexpr int NT = 2 / (WAVES / 4);             // 32-column tiles per wave
     constexpr int RS = 2 * WAVES;                   // rows of the X tile that one fetch instruction of the workgroup covers
     constexpr int NPIECE = TM / RS;                 // 16-byte pieces of the X tile per thread
-    static_assert(WAVES == 4 || (WAVES == 8 && MT == 4), "wave layouts");
+    static_assert(WAVES == 4 || (WAVES == 8 && (MT == 4 || MT == 2 || MT == 1)), "wave layouts");
+    static_assert(NPIECE == 2 || NPIECE == 4 || NPIECE == 8 || NPIECE == 16, "pieces per thread");
     const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3;  // s_a: [2][TM * QF_PITCH]
     const int j = lane & 31, kh = lane >> 5;
     const int m0 = by * TM;
@@ -709,7 +710,8 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
     // workgroup, as the K splits of the narrow projections are, is mostly this prologue)
 #define QF_LD0(p) (*reinterpret_cast<const uint4*>(x_src + RS * (p) * x_row_bytes))
 #define QF_ST0(p, v) (*reinterpret_cast<uint4*>(x_dst + RS * (p) * QF_PITCH) = (v))
-    x0 = QF_LD0(0); x1 = QF_LD0(1); x2 = QF_LD0(2); x3 = QF_LD0(3);
+    x0 = QF_LD0(0); x1 = QF_LD0(1);
+    if constexpr (NPIECE >= 4) { x2 = QF_LD0(2); x3 = QF_LD0(3); }
     if constexpr (NPIECE >= 8) { x4 = QF_LD0(4); x5 = QF_LD0(5); x6 = QF_LD0(6); x7 = QF_LD0(7); }
     if constexpr (NPIECE >= 16) {
         x8 = QF_LD0(8); x9 = QF_LD0(9); x10 = QF_LD0(10); x11 = QF_LD0(11); x12 = QF_LD0(12);
@@ -720,7 +722,8 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
 #pragma unroll
     for (int t = 0; t < NT; ++t) cur[t].load(wrow[t], kh);
     issue_order_fence();
-    QF_ST0(0, x0); QF_ST0(1, x1); QF_ST0(2, x2); QF_ST0(3, x3);
+    QF_ST0(0, x0); QF_ST0(1, x1);
+    if constexpr (NPIECE >= 4) { QF_ST0(2, x2); QF_ST0(3, x3); }
     if constexpr (NPIECE >= 8) { QF_ST0(4, x4); QF_ST0(5, x5); QF_ST0(6, x6); QF_ST0(7, x7); }
     if constexpr (NPIECE >= 16) {
         QF_ST0(8, x8); QF_ST0(9, x9); QF_ST0(10, x10); QF_ST0(11, x11); QF_ST0(12, x12);
@@ -753,7 +756,8 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
                 // piece must not have the weight loads (HBM latency, one cache line per lane) in front of it.  The
                 // pieces are written to LDS in steps 3..6 with the weights still in flight; the weights are first
                 // needed at step 7.
-                x0 = QF_LD(0); x1 = QF_LD(1); x2 = QF_LD(2); x3 = QF_LD(3);
+                x0 = QF_LD(0); x1 = QF_LD(1);
+                if constexpr (NPIECE >= 4) { x2 = QF_LD(2); x3 = QF_LD(3); }
                 if constexpr (NPIECE >= 8) { x4 = QF_LD(4); x5 = QF_LD(5); x6 = QF_LD(6); x7 = QF_LD(7); }
                 if constexpr (NPIECE >= 16) {
                     x8 = QF_LD(8); x9 = QF_LD(9); x10 = QF_LD(10); x11 = QF_LD(11); x12 = QF_LD(12);
@@ -763,7 +767,10 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
 #pragma unroll
                 for (int t = 0; t < NT; ++t) nxt[t].load(wrow[t] + (int64_t)nb * Tile::kBlockBytes, kh);
             }
-            if (s == 3) { QF_ST(0, x0); QF_ST(1, x1); QF_ST(2, x2); QF_ST(3, x3); }
+            if (s == 3) {
+                QF_ST(0, x0); QF_ST(1, x1);
+                if constexpr (NPIECE >= 4) { QF_ST(2, x2); QF_ST(3, x3); }
+            }
             if constexpr (NPIECE >= 8) { if (s == 4) { QF_ST(4, x4); QF_ST(5, x5); QF_ST(6, x6); QF_ST(7, x7); } }
             if constexpr (NPIECE >= 16) {
                 if (s == 5) { QF_ST(8, x8); QF_ST(9, x9); QF_ST(10, x10); QF_ST(11, x11); }
@@ -1016,11 +1023,11 @@ void qgemm_f16_multi_plan(int n, const int* N, const uint32_t* types, int K, int
 }
 
 // Rows per workgroup in tiles of 32: 4 (128 rows: each dequantised weight serves twice as many products) unless that
-// leaves most of the chip idle; then 2 (64 rows, two workgroups per CU).  The Q6_K variant of the small tile does
-// not fit its registers, so it is used only where the big tile would be half empty anyway.  A row's sum does not
-// depend on the choice (same K order).
+// leaves most of the chip idle; then 2 (64 rows: twice the workgroups).  Prompts of up to 64 / 32 rows take the 64- / 32-row
+// tile: a quarter of the X tile traffic, LDS reads and MFMAs per block.  A row's sum does not depend on the choice (same K
+// order).  Threshold swept on the Qwen3-4B shapes: 128 workgroups, Q4_K only, is the best or tied at every prompt length.
 static int qgemm_f16_row_tiles(bool q4, int M, int N, int splits) {
-    if (M <= 32) return 1;  // short prompts: a quarter of the X tile traffic, LDS reads and MFMAs of the 128-row tile per block
+    if (M <= 32) return 1;
     if (M <= 64) return 2;
     const int wgs = ((N + QF_TN - 1) / QF_TN) * ((M + 127) / 128) * splits;
     return (q4 && wgs < 128) ? 2 : 4;  // 512 x 2560 x 9728 (152 workgroups): 60 us with 128 rows, 70 with 64; 512 x 4096 x 4096 (64): 80 / 68
@@ -1069,35 +1076,35 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
         else if (x_is_f32) hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, true>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
         else hipLaunchKernelGGL((qgemm_prepare_rows_f16_kernel<false, false>), dim3(mp), dim3(256), 0, s, X, Xh, rowscale, M, K);
     }
-    // rows per workgroup: 64 (two workgroups share a CU, so one's memory waits hide behind the other's arithmetic) or
-    // 128 (half the dequantisation work per product)
+    // rows per workgroup: 32, 64 or 128 (see qgemm_f16_row_tiles)
     const int MT = qgemm_f16_row_tiles(q4, M, N, splits);
     const int tm = 32 * MT;
     const size_t lds = 2 * (size_t)tm * QF_PITCH + 4 * (size_t)tm;  // 132 KB / 66 KB (two X tiles) + the row scales: above the default 64 KB cap of dynamic LDS
     static bool raised = false;
     if (!raised) {
         const int big = 2 * 128 * QF_PITCH + 4 * 128, small = 2 * 64 * QF_PITCH + 4 * 64;
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
         raised = true;
     }
     const dim3 grid((N + QF_TN - 1) / QF_TN, (M + tm - 1) / tm, splits);
     const uint8_t* Wb = static_cast<const uint8_t*>(W);
-    // 128-row tiles run with eight waves: 512 x 4096 x 14336 104 -> 92-94 us (Q4_K) against four waves,
-    // 321 -> 308 us for 512 x 14336 x 4096 (Q6_K)
-    const bool eight = MT == 4;
-    if (eight && q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
-    else if (eight) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
-    else if (q4 && MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
-    else if (q4 && MT == 1) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 1>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
-    else if (MT == 1) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 1>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
-    else if (q4) hipLaunchKernelGGL((qgemm_f16_kernel<Q4Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
-    else if (MT == 4) hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 4>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
-    else hipLaunchKernelGGL((qgemm_f16_kernel<Q6Tile, 2>), grid, dim3(256), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials);
+    // Every tile height runs with eight waves (two per SIMD, one 32-column strip each): against four waves owning two strips
+    // each, 512 x 4096 x 14336 104 -> 92 us (128 rows), 512 x 4096 x 4096 59.8 -> 45.3 us and 96 x 4096 x 2560 57.0 -> 42.7 us
+    // (64 rows), a 16-token prompt 4.09 -> 3.86 ms (32 rows); the 64-row Q6_K tile no longer spills.
+#define PTM_QF(TILE, MTV) hipLaunchKernelGGL((qgemm_f16_kernel<TILE, MTV, 8>), grid, dim3(512), lds, s, Wb, stride, Xh, rowscale, Y, M, K, N, acc, bps, partials)
+    if (q4) {
+        if (MT == 4) PTM_QF(Q4Tile, 4);
+        else if (MT == 2) PTM_QF(Q4Tile, 2);
+        else PTM_QF(Q4Tile, 1);
+    } else {
+        if (MT == 4) PTM_QF(Q6Tile, 4);
+        else if (MT == 2) PTM_QF(Q6Tile, 2);
+        else PTM_QF(Q6Tile, 1);
+    }
+#undef PTM_QF
     if (deferred_splits) *deferred_splits = partials ? splits : 0;
     if (partials && !deferred_splits) {
         const int64_t total = (int64_t)M * N;
@@ -1196,10 +1203,14 @@ int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const in
     if (!raised) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_multi_kernel<4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   2 * 128 * QF_PITCH + 4 * 128);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_multi_kernel<2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  2 * 64 * QF_PITCH + 4 * 64);
         raised = true;
     }
     if (M <= 32)  // short prompts: the 32-row tile (see qgemm_f16_row_tiles)
-        hipLaunchKernelGGL((qgemm_f16_multi_kernel<1, 4>), dim3(slots, 1), dim3(256), 2 * (size_t)32 * QF_PITCH + 4 * 32, s, a, M, K);
+        hipLaunchKernelGGL((qgemm_f16_multi_kernel<1, 8>), dim3(slots, 1), dim3(512), 2 * (size_t)32 * QF_PITCH + 4 * 32, s, a, M, K);
+    else if (M <= 64)
+        hipLaunchKernelGGL((qgemm_f16_multi_kernel<2, 8>), dim3(slots, 1), dim3(512), 2 * (size_t)64 * QF_PITCH + 4 * 64, s, a, M, K);
     else
         hipLaunchKernelGGL((qgemm_f16_multi_kernel<4, 8>), dim3(slots, (M + 127) / 128), dim3(512), 2 * (size_t)128 * QF_PITCH + 4 * 128, s, a, M, K);
     if (r.n > 0 && !deferred_P) hipLaunchKernelGGL(qgemm_split_reduce_multi_kernel, dim3(red_blocks), dim3(256), 0, s, r);
