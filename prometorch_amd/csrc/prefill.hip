@@ -824,8 +824,9 @@ int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void
         return kv_fp16 ? prefill_attn_launch<true, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
                        : prefill_attn_launch<false, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
     }
-    // the MFMA kernel addresses the caches with 32-bit byte offsets
-    const bool offsets_fit = (pos0 + rows) * (int64_t)n_kv_heads * head_dim * 2 < ((int64_t)1 << 32);
+    // the MFMA kernel addresses the caches with 32-bit byte offsets (computed for up to two tiles past the last position
+    // before they are clamped)
+    const bool offsets_fit = (pos0 + rows + 64) * (int64_t)n_kv_heads * head_dim * 2 < ((int64_t)1 << 32);
     if (window == 0 && kv_fp16 && offsets_fit && rows >= PTM_PREFILL_MFMA_MIN_ROWS && (G == 1 || G == 2 || G == 4 || G == 8))
         return head_dim == 128 ? prefill_attn_mfma_launch<128>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
                                : prefill_attn_mfma_launch<64>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
