@@ -652,9 +652,9 @@ struct Q6Tile {  // Q6_K: the lane's 16 bytes of ql for each (half, pair), of qh
     static constexpr bool kQ8Round = false;
 };
 
-// X tile of a super-block step in LDS.  The 16 pieces a thread owns of the NEXT block's tile are fetched at step 0
-// of the current block, followed by the next block's weights, and written to the other LDS buffer during steps
-// 3..6, so the block ends with the next tile complete behind the only workgroup barrier of the block.  (After the
+// X tile of a super-block step in LDS.  The pieces a thread owns of the NEXT block's tile are fetched during the first
+// steps of the current block, followed by the next block's weights, and written to the other LDS buffer during the
+// later steps, so the block ends with the next tile complete behind the only workgroup barrier of the block.  (After the
 // last block the same code re-fetches the last tile into the idle buffer: no conditionals in the steady-state loop.)
 // WAVES = 8 (what is launched, for every tile height): waves w and w + 4 own one 32-column strip each of the same 64
 // columns and all MT row tiles, so a SIMD holds two waves and one's dequantisation and LDS reads run under the other's
@@ -751,31 +751,47 @@ __device__ __forceinline__ void qgemm_f16_body(const uint8_t* W, int64_t stride,
         for (int s = 0; s < 8; ++s) {  // unrolled: the sub-block index selects registers
 #define QF_LD(p) (*reinterpret_cast<const uint4*>(x_from + RS * (p) * x_row_bytes))
 #define QF_ST(p, v) (*reinterpret_cast<uint4*>(x_nxt + RS * (p) * QF_PITCH) = (v))
-            if (s == 0) {
-                // All fetches of the block are issued here, tile pieces FIRST: loads return in order, so a wait for a
-                // piece must not have the weight loads (HBM latency, one cache line per lane) in front of it.  The
-                // pieces are written to LDS in steps 3..6 with the weights still in flight; the weights are first
-                // needed at step 7.
-                x0 = QF_LD(0); x1 = QF_LD(1);
-                if constexpr (NPIECE >= 4) { x2 = QF_LD(2); x3 = QF_LD(3); }
-                if constexpr (NPIECE >= 8) { x4 = QF_LD(4); x5 = QF_LD(5); x6 = QF_LD(6); x7 = QF_LD(7); }
-                if constexpr (NPIECE >= 16) {
+            // For the 128-row tile the fetches of the next block are spread over steps 0..3 and the LDS stores of the tile pieces
+            // over steps 4..7: issued in one burst at step 0 they held up the vector-memory path for everything behind them
+            // (512 x 4096 x 14336: 75.6 -> 72.1 us; a 2048-token prompt 26.3 -> 25.6 ms; prompts of up to 64 rows were 2 % slower
+            // with their few pieces spread, so the small tiles keep the burst).  Tile pieces go FIRST and the weights last (step 3):
+            // loads return in order, so a wait for a piece must not have the weight loads (HBM latency, one cache line per
+            // lane) in front of it; the weights are first needed at step 7.
+#define QF_W() _Pragma("unroll") for (int t = 0; t < NT; ++t) nxt[t].load(wrow[t] + (int64_t)nb * Tile::kBlockBytes, kh)
+            if constexpr (NPIECE == 8) {
+                if (s == 0) { x0 = QF_LD(0); x1 = QF_LD(1); }
+                if (s == 1) { x2 = QF_LD(2); x3 = QF_LD(3); }
+                if (s == 2) { x4 = QF_LD(4); x5 = QF_LD(5); }
+                if (s == 3) { x6 = QF_LD(6); x7 = QF_LD(7); issue_order_fence(); QF_W(); }
+                if (s == 4) { QF_ST(0, x0); QF_ST(1, x1); }
+                if (s == 5) { QF_ST(2, x2); QF_ST(3, x3); }
+                if (s == 6) { QF_ST(4, x4); QF_ST(5, x5); }
+                if (s == 7) { QF_ST(6, x6); QF_ST(7, x7); }
+            } else if constexpr (NPIECE <= 4) {  // the 64- and 32-row tiles: one burst and one step of stores measured faster there
+                if (s == 0) {
+                    x0 = QF_LD(0); x1 = QF_LD(1);
+                    if constexpr (NPIECE == 4) { x2 = QF_LD(2); x3 = QF_LD(3); }
+                    issue_order_fence();
+                    QF_W();
+                }
+                if (s == 3) {
+                    QF_ST(0, x0); QF_ST(1, x1);
+                    if constexpr (NPIECE == 4) { QF_ST(2, x2); QF_ST(3, x3); }
+                }
+            } else {  // 16 pieces (the four-wave 128-row layout): one burst at step 0, stores in steps 3..6
+                if (s == 0) {
+                    x0 = QF_LD(0); x1 = QF_LD(1); x2 = QF_LD(2); x3 = QF_LD(3); x4 = QF_LD(4); x5 = QF_LD(5); x6 = QF_LD(6); x7 = QF_LD(7);
                     x8 = QF_LD(8); x9 = QF_LD(9); x10 = QF_LD(10); x11 = QF_LD(11); x12 = QF_LD(12);
                     x13 = QF_LD(13); x14 = QF_LD(14); x15 = QF_LD(15);
+                    issue_order_fence();
+                    QF_W();
                 }
-                issue_order_fence();  // pieces before weights, as written
-#pragma unroll
-                for (int t = 0; t < NT; ++t) nxt[t].load(wrow[t] + (int64_t)nb * Tile::kBlockBytes, kh);
-            }
-            if (s == 3) {
-                QF_ST(0, x0); QF_ST(1, x1);
-                if constexpr (NPIECE >= 4) { QF_ST(2, x2); QF_ST(3, x3); }
-            }
-            if constexpr (NPIECE >= 8) { if (s == 4) { QF_ST(4, x4); QF_ST(5, x5); QF_ST(6, x6); QF_ST(7, x7); } }
-            if constexpr (NPIECE >= 16) {
+                if (s == 3) { QF_ST(0, x0); QF_ST(1, x1); QF_ST(2, x2); QF_ST(3, x3); }
+                if (s == 4) { QF_ST(4, x4); QF_ST(5, x5); QF_ST(6, x6); QF_ST(7, x7); }
                 if (s == 5) { QF_ST(8, x8); QF_ST(9, x9); QF_ST(10, x10); QF_ST(11, x11); }
                 if (s == 6) { QF_ST(12, x12); QF_ST(13, x13); QF_ST(14, x14); QF_ST(15, x15); }
             }
+#undef QF_W
 #undef QF_LD
 #undef QF_ST
             issue_order_fence();  // the fetches stay HERE, two steps ahead of their use (the compiler would sink them to it)
