@@ -472,6 +472,7 @@ __global__ __launch_bounds__(THREADS) void qgemm_prepare_fused_kernel(const floa
 // forms as qgemm_prepare_fused_kernel<1> produces them (same arithmetic, same reduction order: the row is staged in LDS
 // and walked with that kernel's two lane mappings).  One launch and one pass over the row instead of a reduction launch
 // and three sweeps of the conversion.
+template <int B>  // partial sums fetched per batch
 __global__ __launch_bounds__(256) void qgemm_reduce_norm_prepare_kernel(const float* __restrict__ P, int splits, float* __restrict__ X,
                                                                         int accumulate, const float* __restrict__ gamma, float eps,
                                                                         int add_one, _Float16* __restrict__ Xh_round,
@@ -492,15 +493,16 @@ __global__ __launch_bounds__(256) void qgemm_reduce_norm_prepare_kernel(const fl
     const int64_t total = (int64_t)M * K;
     float4* x4 = reinterpret_cast<float4*>(X + (int64_t)m * K);
     for (int i = tid; i < n4; i += 256) {
-        // eight partial sums per batch, fetched unconditionally (the index clamped) so that they are in flight together
+        // B partial sums per batch, fetched unconditionally (the index clamped) so that they are in flight together; B = 4
+        // where there are at most four slabs (half the clamped re-reads of the last one)
         const float4 o = accumulate ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int z0 = 0; z0 < splits; z0 += 8) {
-            float4 b[8];
+        for (int z0 = 0; z0 < splits; z0 += B) {
+            float4 b[B];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) b[u] = reinterpret_cast<const float4*>(P + min(z0 + u, splits - 1) * total + (int64_t)m * K)[i];
+            for (int u = 0; u < B; ++u) b[u] = reinterpret_cast<const float4*>(P + min(z0 + u, splits - 1) * total + (int64_t)m * K)[i];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < B; ++u) {
                 if (z0 + u == 0) a = b[u];
                 else if (z0 + u < splits) { a.x += b[u].x; a.y += b[u].y; a.z += b[u].z; a.w += b[u].w; }
             }
@@ -1143,8 +1145,12 @@ int qgemm_f16_reduce_norm_prepare(const float* P, int splits, float* X, bool acc
     _Float16* hp = static_cast<_Float16*>(ws_plain);
     float* rr = hr ? reinterpret_cast<float*>(hr + (int64_t)mp * K) : nullptr;
     float* rp = hp ? reinterpret_cast<float*>(hp + (int64_t)mp * K) : nullptr;
-    hipLaunchKernelGGL(qgemm_reduce_norm_prepare_kernel, dim3(mp), dim3(256), (size_t)K * 4, s, P, splits, X, accumulate ? 1 : 0,
-                       gamma, eps, add_one, hr, rr, hp, rp, M, K);
+    if (splits <= 4)
+        hipLaunchKernelGGL(qgemm_reduce_norm_prepare_kernel<4>, dim3(mp), dim3(256), (size_t)K * 4, s, P, splits, X, accumulate ? 1 : 0,
+                           gamma, eps, add_one, hr, rr, hp, rp, M, K);
+    else
+        hipLaunchKernelGGL(qgemm_reduce_norm_prepare_kernel<8>, dim3(mp), dim3(256), (size_t)K * 4, s, P, splits, X, accumulate ? 1 : 0,
+                           gamma, eps, add_one, hr, rr, hp, rp, M, K);
     return launch_status();
 }
 
