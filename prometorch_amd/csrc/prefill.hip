@@ -709,9 +709,11 @@ static int prefill_attn_mfma_launch(int G, hipStream_t s, const float* Q, const 
                                     int n_heads, int n_kv_heads, int64_t pos0, float scale) {
     const int bm = 128 / G;
     const dim3 grid((rows + bm - 1) / bm, n_kv_heads);
-    // up to 128 rows a row block has at most four tiles of its own chunk to share out: one group of four waves per workgroup
-    // (no merge, half the threads to start) is 2 - 3 us faster there; beyond, two groups split the tiles
-    const bool one = rows <= 128;
+    // Two groups halve the chain of a row block's tiles and cost a merge and twice the threads to start: with at most 16
+    // tiles per row block (the chunk ends within the first 512 positions) one group is faster (192 / 256 / 384 rows from
+    // position 0: 9.8 / 11.1 / 13.8 us against 12.5 / 12.6 / 14.9; 512 rows: 17.0 / 17.2), beyond it two are (768 rows: 21.8
+    // against 22.7; 256 rows at position 1024: 27.8 against 31.4)
+    const bool one = pos0 + rows <= 512;
 #define PTM_PA(GG)                                                                                                          \
     if (one)                                                                                                                \
         hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG, 1>), grid, dim3(256), 0, s, Q, static_cast<const __half*>(Kc), \
