@@ -98,7 +98,11 @@ int ptm_q6k_gemv_argmax(const void* W, const float* x, float* logits, int K, int
  * library (512 KiB per GPU, held until the process ends).  No counterpart in the reference.  N above
  * ptm_q6k_gemv_argmax_noalloc_max_rows() (262144) returns PTM_E_RANGE.  Calls no hipMalloc / hipFree.  All calls on one
  * GPU share that GPU's array: calls that overlap in time on one GPU (different streams) race; calls ordered on one
- * stream do not.  Same results as ptm_q6k_gemv_argmax. */
+ * stream do not.  Same results as ptm_q6k_gemv_argmax.
+ * The first call on a device looks the array's address up and raises the kernels' LDS cap; neither may happen while a
+ * stream is capturing.  A caller that captures calls ptm_q6k_gemv_argmax_noalloc_init() once per device beforehand, with
+ * that device current (it allocates nothing either); after it every call is capture-legal. */
+int ptm_q6k_gemv_argmax_noalloc_init(void);
 int ptm_q6k_gemv_argmax_noalloc_max_rows(void);
 int ptm_q6k_gemv_argmax_noalloc(const void* W, const float* x, float* logits, int K, int N, int64_t row_stride_bytes,
                                 int64_t* out_index, ptm_stream_t stream);
@@ -479,6 +483,10 @@ int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_ou
  * step yet), 1 replaying its captured hipGraph, 2 plain launches because capturing or instantiating the graph failed
  * once - not an error: the reference likewise falls back to eager launches (gguf_model.h:2660-2665, :3093-3104). */
 int ptm_decode_graph_state(const ptm_decoder* d, int sampled);
+/* Test seam for that fallback: the decoder's next capture attempt reports failure on the host before anything is recorded
+ * (no GPU error is provoked), so the steps that follow run as plain launches and ptm_decode_graph_state returns 2.  The
+ * reference has no such switch; its fallback (gguf_model.h:2660-2665) is reached only by a real capture failure. */
+int ptm_decode_debug_fail_next_capture(ptm_decoder* d);
 /* Device pointers to the last step's logits [vocab] and final-normed hidden [hidden]. */
 const float* ptm_decode_logits(ptm_decoder* d);
 const float* ptm_decode_hidden(ptm_decoder* d);

@@ -81,6 +81,7 @@ SIGNATURES = {
     "ptm_argmax_workspace_bytes": (i64, [i32]),
     "ptm_q6k_gemv_argmax": (i32, [vp, vp, vp, i32, i32, i64, vp, vp, vp]),
     "ptm_q6k_gemv_argmax_noalloc_max_rows": (i32, []),
+    "ptm_q6k_gemv_argmax_noalloc_init": (i32, []),
     "ptm_q6k_gemv_argmax_noalloc": (i32, [vp, vp, vp, i32, i32, i64, vp, vp]),
     "ptm_quant_gemv": (i32, [u32, vp, vp, vp, i32, i32, i64, i32, vp]),
     "ptm_q4k_fused_gate_up_gemv": (i32, [vp, vp, vp, vp, vp, i32, i32, i32, i64, vp]),
@@ -147,6 +148,7 @@ SIGNATURES = {
     "ptm_sample_token": (i32, [vp, i32, vp, C.POINTER(Sampling), vp, vp, vp, vp]),
     "ptm_mt19937_uniforms": (i32, [u32, i64, i64, C.POINTER(f32)]),
     "ptm_decode_graph_state": (i32, [vp, i32]),
+    "ptm_decode_debug_fail_next_capture": (i32, [vp]),
     "ptm_decode_logits": (vp, [vp]),
     "ptm_decode_hidden": (vp, [vp]),
     "ptm_decode_stream": (vp, [vp]),

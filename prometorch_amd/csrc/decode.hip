@@ -59,6 +59,7 @@ int qknorm_rope_kv_rows_from_parts(const float* const* P, const int* splits, con
                                    int max_seq, float eps, int add_one, int kv_fp16, int rope_interleaved, hipStream_t s);
 int qgemm_f16_prepare_fused(int pre, const float* X, const float* X2, float eps, int add_one, void* ws_round, void* ws_plain,
                             int M, int K, hipStream_t s);
+int sampler_launch_key(const ptm_sampling& host_params, int vocab);
 int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
                     const ptm_sampling* d_params, const float* d_uniforms, const int* d_step, void* workspace,
                     int64_t* out_token, int32_t* counts_rw, ArgmaxAdvance adv, bool ws_kept_clean, hipStream_t s);
@@ -99,6 +100,8 @@ struct ptm_decoder {
     hipGraphExec_t exec_s = nullptr;
     bool captured_s = false;
     bool eager_fallback = false, eager_fallback_s = false;  // capture or instantiation failed once: plain launches from then on
+    bool debug_fail_capture = false;  // test seam: the next capture attempt reports failure on the host, nothing is launched for it
+    int sampled_key = -1;             // launch sequence (sampler_launch_key) the sampled-step graph was captured with
     // sampling state: parameters (host + device copy), occurrence counts of generated tokens, uniform draws
     ptm_sampling sampling{0.0f, 1, 1.0f, 1.0f};
     bool sampling_set = false;
@@ -583,7 +586,9 @@ static int run_steps(ptm_decoder* d, int token, int n, bool sample = false) {
         // as the reference falls back to eager execution (gguf_model.h:2660-2665, :3093-3104).
         hipGraph_t g = nullptr;
         hipGraphExec_t ge = nullptr;
-        bool ok = hip_status(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal)) == PTM_OK;
+        bool ok = !d->debug_fail_capture;
+        d->debug_fail_capture = false;
+        if (ok) ok = hip_status(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal)) == PTM_OK;
         if (ok) {
             const int rc_enq = enqueue_step(d, sample);
             const int rc_end = hip_status(hipStreamEndCapture(s, &g));  // always ends the capture, also after a failed launch
@@ -594,6 +599,7 @@ static int run_steps(ptm_decoder* d, int token, int n, bool sample = false) {
             graph = g;
             exec = ge;
             captured = true;
+            if (sample) d->sampled_key = sampler_launch_key(d->sampling, d->cfg.vocab);
         } else {
             if (g) (void)hipGraphDestroy(g);
             (void)hipGetLastError();  // the failure has been handled: do not let it surface at the next launch check
@@ -626,6 +632,25 @@ int ptm_decode_sampling_begin(ptm_decoder* d, const ptm_sampling* params) {
     if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return rc;  // params may be a temporary of the caller
     d->sampling = *params;
     d->sampling_set = true;
+    // The sampler's launch sequence is chosen on the host from the parameters (candidate list or whole-vocabulary passes,
+    // with or without the top-k select and the nucleus walk): a captured sampled step only serves parameters of the same
+    // class.  A request of another class drops that graph; the next sampled step captures the new sequence.
+    if (d->captured_s && sampler_launch_key(*params, d->cfg.vocab) != d->sampled_key) {
+        (void)hipGraphExecDestroy(d->exec_s);
+        (void)hipGraphDestroy(d->graph_s);
+        d->exec_s = nullptr;
+        d->graph_s = nullptr;
+        d->captured_s = false;
+        d->sampled_key = -1;
+    }
+    return PTM_OK;
+}
+
+// Test seam for the capture fallback: the decoder's next capture attempt reports failure on the host before anything is
+// recorded, so the step goes on as plain launches exactly as after a real capture or instantiation failure.
+int ptm_decode_debug_fail_next_capture(ptm_decoder* d) {
+    if (!d) return PTM_E_NULL;
+    d->debug_fail_capture = true;
     return PTM_OK;
 }
 

@@ -222,8 +222,8 @@ static void q6k_raise_lds_cap_nb() {
 // Raise the dynamic-LDS cap of every variant once (rows longer than 15K values need more than the default
 // 64 KB); must happen outside stream capture, so the decoder calls it when it is created.
 void q6k_init_attributes() {
-    static bool done = false;
-    if (done) return;
+    static std::once_flag done;  // callers on two host threads: the second returns only after the caps are raised
+    std::call_once(done, [] {
     q6k_raise_lds_cap_nb<false, false, false, 1>();
     q6k_raise_lds_cap_nb<true, false, false, 1>();
     q6k_raise_lds_cap_nb<false, false, false, 3>();
@@ -231,7 +231,7 @@ void q6k_init_attributes() {
     q6k_raise_lds_cap_nb<false, true, false, 1>();
     q6k_raise_lds_cap_nb<false, true, true, 1>();
     q6k_raise_lds_cap_nb<false, false, true, 1>();
-    done = true;
+    });
 }
 
 template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
@@ -354,6 +354,15 @@ void* scratch_on_current_device(int* rc) {
 extern "C" {
 
 int ptm_q6k_gemv_argmax_noalloc_max_rows(void) { return PTM_NOALLOC_MAX_ROWS; }
+
+// One-time set-up for the current device, for callers that will call the entry point under stream capture: the symbol
+// lookup and the kernel attributes are not capture-legal, everything the entry point does afterwards is.
+int ptm_q6k_gemv_argmax_noalloc_init(void) {
+    int rc = PTM_OK;
+    if (!scratch_on_current_device(&rc)) return rc;
+    q6k_init_attributes();
+    return PTM_OK;
+}
 
 int ptm_q6k_gemv_argmax_noalloc(const void* W, const float* x, float* logits, int K, int N, int64_t stride,
                                 int64_t* out_index, ptm_stream_t stream) {

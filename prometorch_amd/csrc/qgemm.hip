@@ -18,6 +18,8 @@
 //   X is bf16 by contract, so products are exact; each 16-group sum is scaled by d*scale[n] in fp32.
 #include "ptm_common.h"
 
+#include <mutex>
+
 namespace ptm {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -1098,15 +1100,14 @@ int qgemm_f16_impl(uint32_t ggml_type, const void* W, const void* X, bool x_is_f
     const int MT = qgemm_f16_row_tiles(q4, M, N, splits);
     const int tm = 32 * MT;
     const size_t lds = 2 * (size_t)tm * QF_PITCH + 4 * (size_t)tm;  // 132 KB / 66 KB (two X tiles) + the row scales: above the default 64 KB cap of dynamic LDS
-    static bool raised = false;
-    if (!raised) {
+    static std::once_flag raised;  // two host threads may get here at once: the second waits until the caps are raised
+    std::call_once(raised, [] {
         const int big = 2 * 128 * QF_PITCH + 4 * 128, small = 2 * 64 * QF_PITCH + 4 * 64;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, big);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q4Tile, 2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_kernel<Q6Tile, 2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, small);
-        raised = true;
-    }
+    });
     const dim3 grid((N + QF_TN - 1) / QF_TN, (M + tm - 1) / tm, splits);
     const uint8_t* Wb = static_cast<const uint8_t*>(W);
     // Every tile height runs with eight waves (two per SIMD, one 32-column strip each): against four waves owning two strips
@@ -1221,14 +1222,13 @@ int qgemm_f16_multi(int n, const uint32_t* types, const void* const* W, const in
             part += (size_t)splits * M * N[i];
         }
     }
-    static bool raised = false;
-    if (!raised) {
+    static std::once_flag raised;
+    std::call_once(raised, [] {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_multi_kernel<4, 8>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   2 * 128 * QF_PITCH + 4 * 128);
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&qgemm_f16_multi_kernel<2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   2 * 64 * QF_PITCH + 4 * 64);
-        raised = true;
-    }
+    });
     if (M <= 32)  // short prompts: the 32-row tile (see qgemm_f16_row_tiles)
         hipLaunchKernelGGL((qgemm_f16_multi_kernel<1, 8>), dim3(slots, 1), dim3(512), 2 * (size_t)32 * QF_PITCH + 4 * 32, s, a, M, K);
     else if (M <= 64)

@@ -814,6 +814,14 @@ static int sampler_check(const ptm_sampling& p, int vocab) {
     return PTM_OK;
 }
 
+// Which launch sequence sampler_enqueue records for these parameters: 0 = candidate list (greedy included); otherwise the
+// whole-vocabulary passes, bit 1 = with the top-k select, bit 2 = with the nucleus walk.  A captured graph of one key must
+// not be replayed for parameters of another.
+int sampler_launch_key(const ptm_sampling& p, int vocab) {
+    if (!sampler_is_wide(p, vocab)) return 0;
+    return 1 | ((p.top_k > 0 && p.top_k < vocab) ? 2 : 0) | (p.top_p < 1.0f ? 4 : 0);
+}
+
 // host_params are validated here; when d_params is given the kernels read the device copy (which must hold the same values)
 int sampler_enqueue(const float* logits, int vocab, const int32_t* counts, const ptm_sampling& host_params,
                     const ptm_sampling* d_params, const float* d_uniforms, const int* d_step, void* workspace,

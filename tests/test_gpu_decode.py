@@ -252,6 +252,67 @@ def test_longrope_factors_decode_vs_reference_golden(dev, seeds, use_graph):
     dec.close()
 
 
+def test_capture_failure_falls_back_to_plain_launches(dev, po, seeds):
+    """The eager continuation after a failed graph capture (the reference's fallback, gguf_model.h:2660-2665, :3100-3104).  The
+    failure is forced on the host through ptm_decode_debug_fail_next_capture, before anything is recorded: no GPU error is
+    provoked.  State 2, tokens and logits as the oracle's, no second capture attempt after set_past_len; the sampled step
+    keeps its own state."""
+    from prometorch_amd.decode import Decoder
+    cfg = dict(synth.TINY)
+    layers = [synth.make_layer(seeds["tiny"], i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(seeds["tiny"], cfg)
+    kv = [synth.make_kv_prefill(seeds["tiny"], i, cfg, 19) for i in range(cfg["n_layers"])]
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=True)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=True)
+    ref = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=True)   # the same run on a captured graph
+    for i, (k, v) in enumerate(kv):
+        om.set_kv(i, k, v)
+        dec.set_kv(i, k, v)
+        ref.set_kv(i, k, v)
+    dec.set_past_len(19)
+    ref.set_past_len(19)
+    state = dec.L.ptm_decode_graph_state
+    assert state(dec.h, 0) == 0
+    assert dec.L.ptm_decode_debug_fail_next_capture(dec.h) == 0
+    to = tg = tr = 3
+    errs = []
+    for st in range(10):
+        to, tg, tr = om.step(to), dec.step(tg), ref.step(tr)
+        assert state(dec.h, 0) == 2, st                      # the very first step already attempted (and failed) the capture
+        errs.append(np.abs(dec.logits() - om.logits).max() / om.logits.std())
+        assert tg == to == tr, (st, errs[-1])
+        assert np.array_equal(dec.logits(), ref.logits()), st    # plain launches and the replayed graph run the same kernels
+    check_step_errors(errs)
+    assert state(ref.h, 0) == 1
+    # a rewind does not retry the capture (the seam is spent; a retry would succeed and report 1)
+    dec.set_past_len(19)
+    ref.set_past_len(19)
+    assert dec.greedy(3, 6) == ref.greedy(3, 6)
+    assert state(dec.h, 0) == 2
+    # the sampled step has a graph of its own: it still captures
+    assert state(dec.h, 1) == 0
+    dec.sampling_begin(0.8, 40, 0.9)
+    ref.sampling_begin(0.8, 40, 0.9)
+    dec.set_past_len(19)
+    ref.set_past_len(19)
+    us = [0.11, 0.52, 0.93, 0.34]
+    assert dec.sample(3, us) == ref.sample(3, us)
+    assert state(dec.h, 1) == 1 and state(dec.h, 0) == 2
+    # and falls back the same way when its capture fails
+    d2 = Decoder(cfg, layers, head, max_seq=64, kv_fp16=True, use_graph=True)
+    for i, (k, v) in enumerate(kv):
+        d2.set_kv(i, k, v)
+    d2.set_past_len(19)
+    d2.sampling_begin(0.8, 40, 0.9)
+    d2.L.ptm_decode_debug_fail_next_capture(d2.h)
+    ref.set_past_len(19)
+    ref.sampling_begin(0.8, 40, 0.9)
+    assert d2.sample(3, us) == ref.sample(3, us)
+    assert state(d2.h, 1) == 2 and state(d2.h, 0) == 0
+    for d in (dec, ref, d2):
+        d.close()
+
+
 def test_tiny_decode_with_a_strong_ffn_branch_vs_oracle(dev, po, seeds):
     """The default synthetic gains keep the feed-forward branch small beside attention (synth.NORM_SCALE); here its norm gain is
     ten times larger, so that gate / up / down move the logits by several of their standard deviations (checked against the

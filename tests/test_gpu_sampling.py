@@ -224,6 +224,55 @@ def test_decoder_sampled_generation_vs_oracle_loop(dev, po, seeds, use_graph, te
     dec.close()
 
 
+def test_one_decoder_serves_requests_of_every_parameter_class(dev, po, seeds):
+    """A serving loop calls sampling_begin per request on ONE decoder.  The sampler's launch sequence depends on the parameters
+    (candidate list; whole-vocabulary passes with / without the top-k select and the nucleus walk), and the sampled step is a
+    captured graph: a request of another class must not replay the previous class's graph.  Each request is checked against
+    the oracle's penalise -> sample -> feed-back loop (api_handlers.h:848-923, gguf_model.h:7658-7751)."""
+    from prometorch_amd.decode import Decoder
+    cfg = dict(synth.TINY, vocab=2048)   # room for a top-k beyond the candidate list (1024) that is still below the vocabulary
+    layers = [synth.make_layer(seeds["tiny"], i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(seeds["tiny"], cfg)
+    dec = Decoder(cfg, layers, head, max_seq=96, kv_fp16=True, use_graph=True)
+    prompt = [int(t) for t in synth.rng_for(85).integers(0, cfg["vocab"], 7)]
+    for t in prompt[:-1]:
+        dec.step(t)
+    n = 24
+    requests = [(0.8, 40, 0.9, 1.1),      # candidate list
+                (0.8, 0, 0.9, 1.0),       # top-k off, nucleus walk
+                (0.8, 1500, 1.0, 1.05),   # top-k beyond the list, no nucleus
+                (0.9, 1500, 0.85, 1.0),   # both
+                (1.1, 0, 1.0, 1.0),       # neither
+                (0.0, 40, 0.9, 1.2),      # greedy
+                (0.8, 40, 0.9, 1.1),      # the first class again
+                (0.7, 64, 0.95, 1.0)]     # same class, other values: served by the same graph through the device copy
+    compared = []
+    for req, (temperature, top_k, top_p, penalty) in enumerate(requests):
+        us = ops.mt19937_uniforms(42, 100 * req, n)
+        dec.set_past_len(len(prompt) - 1)
+        dec.sampling_begin(temperature, top_k, top_p, penalty)
+        got = dec.sample(prompt[-1], us[:9]) 
+        got += dec.sample(got[-1], us[9:])
+        assert dec.L.ptm_decode_graph_state(dec.h, 1) == 1, req
+        om = po.OracleModel(cfg, layers, head, 96, kv_fp16=True)
+        for t in prompt[:-1]:
+            om.step(t)
+        tol = gap_tol(cfg["vocab"], temperature, top_k) * 10
+        tok, generated = prompt[-1], []
+        for st in range(n):
+            om.step(tok)
+            lg = po.repetition_penalty(om.logits, generated, penalty) if generated else om.logits
+            tok, gap = po.sample_token(lg, temperature, top_k, top_p, us[st])
+            if gap <= max(tol, 1e-4):
+                break                                  # a draw on an interval edge: both answers are legitimate
+            assert got[st] == tok, (req, st, gap)
+            generated.append(tok)
+        compared.append(len(generated))
+    print("sampled steps compared per request:", compared, flush=True)
+    assert min(compared) >= 8 and sum(compared) >= 0.6 * n * len(requests), compared
+    dec.close()
+
+
 def test_decoder_sampling_errors(dev, seeds):
     from prometorch_amd.decode import Decoder
     cfg, layers, head = build_tiny(seeds)
