@@ -270,7 +270,7 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
                                                                  const float* __restrict__ pM, float* __restrict__ O,
                                                                  int n_heads, const int64_t* __restrict__ d_past,
                                                                  int64_t past_host, int max_seq,
-                                                                 uint8_t* __restrict__ q8_out) {
+                                                                 uint8_t* __restrict__ q8_out, int chunk_shift, int log2_units) {
     constexpr int NOUT = HD / 4, NSLOT = 256 / NOUT;
     __shared__ __align__(16) float4 s_stage[256];
     __shared__ float s_red[8];
@@ -280,8 +280,12 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
     // Every load of the common case goes out before the position is known: chunk slots past the last active one
     // are clamped into the allocation (ns_max chunks) and dropped by selects below, so the kernel makes one
     // memory round trip, not one for the position and a second for the data.
-    const int ns_max = (max_seq + FD_CHUNK - 1) / FD_CHUNK;
+    const int chunk = 1 << chunk_shift;  // positions per partial
+    const int ns_max = (max_seq + chunk - 1) >> chunk_shift;
     const int64_t past = d_past ? *d_past : past_host;
+    // partial maxima are natural-log scores, or base-2 ones (log2_units) from the matrix-core kernel
+    const float ek = log2_units ? 1.0f : 1.44269504088896340736f;
+    auto wexp = [ek](float x) { return __builtin_amdgcn_exp2f(x * ek); };
     float4 v[8];
     float mm[8];
 #pragma unroll
@@ -295,16 +299,16 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
     int64_t total = past + 1;
     if (total > max_seq) total = max_seq;
     if (total <= 0) return;
-    const int ns = (int)((total + FD_CHUNK - 1) / FD_CHUNK);
+    const int ns = (int)((total + chunk - 1) >> chunk_shift);
     float m = tid < ns ? pm_first : -INFINITY;
     for (int sI = tid + 256; sI < ns; sI += 256) m = fmaxf(m, pM[(int64_t)sI * n_heads + h]);
     m = max64(m);
     if ((tid & 63) == 0) s_red[tid >> 6] = m;
     __syncthreads();
     const float M = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    float den = tid < ns ? expf(pm_first - M) * pl_first : 0.0f;
+    float den = tid < ns ? wexp(pm_first - M) * pl_first : 0.0f;
     for (int sI = tid + 256; sI < ns; sI += 256)
-        den = fmaf(expf(pM[(int64_t)sI * n_heads + h] - M), pL[(int64_t)sI * n_heads + h], den);
+        den = fmaf(wexp(pM[(int64_t)sI * n_heads + h] - M), pL[(int64_t)sI * n_heads + h], den);
     den = sum64(den);
     if ((tid & 63) == 0) s_red[4 + (tid >> 6)] = den;
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -320,7 +324,7 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const bool on = (s0 + u * NSLOT) < ns;  // a select, not a zero weight: inactive slots may hold anything
-            const float w = expf(mm[u] - M);
+            const float w = wexp(mm[u] - M);
             sum.x = on ? fmaf(w, v[u].x, sum.x) : sum.x;
             sum.y = on ? fmaf(w, v[u].y, sum.y) : sum.y;
             sum.z = on ? fmaf(w, v[u].z, sum.z) : sum.z;
@@ -357,13 +361,15 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
 }
 
 static int fd_merge(int head_dim, int n_heads, hipStream_t s, const float* pO, const float* pL, const float* pM, float* O,
-                    const int64_t* d_past, int max_seq, uint8_t* q8_out = nullptr, int64_t past_host = 0) {
+                    const int64_t* d_past, int max_seq, uint8_t* q8_out = nullptr, int64_t past_host = 0,
+                    int chunk = FD_CHUNK, int log2_units = 0) {
+    const int chunk_shift = chunk == 128 ? 7 : 6;
     if (head_dim == 256)
-        hipLaunchKernelGGL(flash_decode_merge_kernel<256>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out);
+        hipLaunchKernelGGL(flash_decode_merge_kernel<256>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out, chunk_shift, log2_units);
     else if (head_dim == 128)
-        hipLaunchKernelGGL(flash_decode_merge_kernel<128>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out);
+        hipLaunchKernelGGL(flash_decode_merge_kernel<128>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out, chunk_shift, log2_units);
     else
-        hipLaunchKernelGGL(flash_decode_merge_kernel<64>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out);
+        hipLaunchKernelGGL(flash_decode_merge_kernel<64>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out, chunk_shift, log2_units);
     return launch_status();
 }
 
@@ -654,6 +660,329 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same front half on the matrix cores, for an fp16 cache.  The vector kernel above spends ~1400 instructions per
+// wave on 16 positions x G heads, three quarters of them conversions, cross-lane sums and address arithmetic around 264
+// FMAs, and the launch lasts as long as that chain whatever the context length (512 positions: 9.3 us for attention +
+// merge, 2240: 10.5 us).  Here a wave's positions are MFMA tiles:
+//   S^T[16 positions][16 head columns] = K tile . Q^T   v_mfma_f32_16x16x32_f16, A = the K rows exactly as they lie in the
+//       cache (lane l: row l % 16, elements 32 s + 8 (l / 16) .. +7 of step s: one 16-byte load, no conversion), B = the
+//       query heads as fp16 (columns past G repeat head 0 and are never stored);
+//   O[16 head rows][HD] = P . V                        A = the probabilities in the layout the first product left them in
+//       (lane l: head l % 16, positions 4 (l / 16) .. +3), B = V^T fragments from a wave-private LDS copy of the V rows through
+//       the transposing read ds_read_b64_tr_b16.
+// fp32 accuracy is kept by splitting the fp32 operands into two fp16 terms (q = q_hi + q_lo, p = p_hi + p_lo, 22 mantissa
+// bits; K and V are fp16 already, products are exact, accumulation is fp32), so the result stays within the vector kernel's
+// bar.  Scores are kept in base 2 (q is scaled by scale * log2 e before the split); the partial maxima are stored in those
+// units and the merge kernel is told so.  A wave takes TPW tiles of 16 positions, a workgroup a chunk of 64 TPW positions.
+// ---------------------------------------------------------------------------------------------
+typedef _Float16 fd_h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 fd_h4 __attribute__((ext_vector_type(4)));
+typedef short fd_s4 __attribute__((ext_vector_type(4)));
+typedef float fd_f4 __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i passes the address of four 16-bit values (row i / 4 of a 4-row
+// block, columns 4 (i % 4) .. +3 of a 16-column block) and receives column i of the four rows.
+__device__ __forceinline__ fd_h4 fd_lds_read_tr16(const uint8_t* p) {
+    typedef __attribute__((address_space(3))) fd_s4 lds_s4;
+    return __builtin_bit_cast(fd_h4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)p));
+}
+// max / sum over the four 16-lane rows of the wave (lanes with equal lane % 16), result in every lane
+__device__ __forceinline__ float fd_rows_max(float v) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float fd_rows_sum(float v) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+template <int HD, int G, int TPW>
+__global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const AttnArgs a) {
+    constexpr int HALF = HD / 2;
+    constexpr int KS = HD / 32;          // QK steps (32 head-dim elements each)
+    constexpr int DT = HD / 16;          // 16-wide tiles of the output's head dimension
+    constexpr int LPR = HD / 8;          // lanes per V row (16-byte pieces)
+    constexpr int RPL = 64 / LPR;        // V rows per load instruction of a wave
+    constexpr int VL = 16 / RPL;         // V loads per tile
+    constexpr int VP = HD * 2 + 64;      // LDS pitch of a V row: the four rows of a transposing read fall on different banks
+    constexpr int GP = G <= 4 ? 4 : 8;   // head slots of the wave partials
+    constexpr int CH = 64 * TPW;         // positions per workgroup
+    static_assert(G >= 1 && G <= 8 && (HD == 64 || HD == 128) && (TPW == 1 || TPW == 2), "shape");
+    __shared__ __align__(16) _Float16 s_qh[G][HD];
+    __shared__ __align__(16) _Float16 s_ql[G][HD];
+    __shared__ __align__(16) _Float16 s_nk[HD];
+    __shared__ __align__(16) uint8_t s_v[4][TPW][16 * VP];
+    __shared__ __align__(16) float s_o[4][HD][GP];
+    __shared__ float s_m[4][GP], s_l[4][GP];
+
+    const int64_t past = *a.d_past;
+    if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
+    const int64_t total = past + 1;
+    const int split = blockIdx.x, kvh = blockIdx.y;
+    const int64_t t0 = (int64_t)split * CH;
+    if (t0 >= total) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t t_begin = (a.window > 0 && total > a.window) ? total - a.window : 0;
+    if (t0 + CH <= t_begin) {
+        // a chunk wholly in front of the window: an empty partial (weight 2^(-inf - M) = 0 in the merge)
+        for (int e = tid; e < G * HD; e += FD_THREADS) {
+            const int g = e / HD, d = e % HD;
+            const int64_t oi = (int64_t)split * a.n_heads + kvh * G + g;
+            a.pO[oi * HD + d] = 0.0f;
+            if (d == 0) { a.pM[oi] = -INFINITY; a.pL[oi] = 0.0f; }
+        }
+        return;
+    }
+    const int j = lane & 15, rg = lane >> 4;
+    const int kv_dim = a.n_kv_heads * HD;
+    const bool on = lane < HALF;
+    const int lh = lane & (HALF - 1);
+    const bool has_norm = a.qw != nullptr;
+    const int64_t wt0 = t0 + (int64_t)wave * (16 * TPW);            // first position of this wave
+    const bool owner = past >= wt0 && past < wt0 + 16 * TPW;       // wave-uniform: this wave's tiles hold the new position
+
+    // ---- loads, all unconditional so that their count is static: first the few values of the prologue ... ----
+    const float* cs = a.rope + past * HD;
+    const float* qwp = has_norm ? a.qw : a.Q;  // a valid address either way; unused without norm weights
+    const float* kwp = has_norm ? a.kw : a.Q;
+    const int i0 = a.rope_interleaved ? 2 * lh : lh, i1 = a.rope_interleaved ? 2 * lh + 1 : lh + HALF;
+    constexpr int NQ = (G + 3) / 4;  // query heads a wave prepares: wave, wave + 4
+    float qx0[NQ], qx1[NQ];
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+        const int g = wave + 4 * n < G ? wave + 4 * n : 0;
+        const float* src = a.Q + (int64_t)(kvh * G + g) * HD;
+        qx0[n] = src[i0];
+        qx1[n] = src[i1];
+    }
+    const float qn0 = qwp[i0], qn1 = qwp[i1], kn0 = kwp[i0], kn1 = kwp[i1];
+    const float rc = cs[lh], rsn = cs[HALF + lh];
+    const float kx0 = a.K[(int64_t)kvh * HD + i0], kx1 = a.K[(int64_t)kvh * HD + i1];
+    const float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
+    issue_order_fence();
+    // ---- ... then the cached K/V rows of this wave's tiles (the new position is not cached: clamp below it) ----
+    uint4 kreg[TPW][KS], vreg[TPW][VL];
+    const int64_t last_cached = past > 0 ? past - 1 : 0;
+    const __half* Kh = static_cast<const __half*>(a.Kc) + (int64_t)kvh * HD;
+    const __half* Vh = static_cast<const __half*>(a.Vc) + (int64_t)kvh * HD;
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+        const int64_t tk = wt0 + 16 * u + j;
+        const int64_t tkc = tk < past ? tk : last_cached;
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            kreg[u][s] = *reinterpret_cast<const uint4*>(Kh + tkc * kv_dim + 32 * s + 8 * rg);
+    }
+#pragma unroll
+    for (int u = 0; u < TPW; ++u)
+#pragma unroll
+        for (int vl = 0; vl < VL; ++vl) {
+            const int64_t tv = wt0 + 16 * u + vl * RPL + lane / LPR;
+            const int64_t tvc = tv < past ? tv : last_cached;
+            vreg[u][vl] = *reinterpret_cast<const uint4*>(Vh + tvc * kv_dim + 8 * (lane % LPR));
+        }
+    issue_order_fence();
+
+    // ---- per-head RMSNorm + rotation of this wave's query heads, scaled into base-2 score units, as two fp16 terms ----
+    const float one = a.add_one ? 1.0f : 0.0f;
+    const float qs = a.scale * 1.44269504088896340736f;
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+        const int g = wave + 4 * n;
+        if (g >= G) continue;  // wave-uniform
+        float x0 = on ? qx0[n] : 0.0f, x1 = on ? qx1[n] : 0.0f;
+        if (has_norm) {
+            float ss = fmaf(x0, x0, 0.0f);
+            ss = fmaf(x1, x1, ss);
+            ss = sum64(ss);
+            const float rs = fast_rsqrt(ss * (1.0f / (float)HD) + a.eps);
+            x0 = x0 * rs * (qn0 + one);
+            x1 = x1 * rs * (qn1 + one);
+        }
+        if (on) {
+            const float r0 = fmaf(x0, rc, -(x1 * rsn)) * qs, r1 = fmaf(x0, rsn, x1 * rc) * qs;
+            const _Float16 h0 = (_Float16)r0, h1 = (_Float16)r1;
+            s_qh[g][i0] = h0;
+            s_qh[g][i1] = h1;
+            s_ql[g][i0] = (_Float16)(r0 - (float)h0);
+            s_ql[g][i1] = (_Float16)(r1 - (float)h1);
+        }
+    }
+    __half nv0 = __float2half_rn(0.0f), nv1 = nv0;
+    if (owner) {  // the new K row: normalised, rotated, rounded as the cache holds it; the new V row
+        float x0 = on ? kx0 : 0.0f, x1 = on ? kx1 : 0.0f;
+        if (has_norm) {
+            float ss = fmaf(x0, x0, 0.0f);
+            ss = fmaf(x1, x1, ss);
+            ss = sum64(ss);
+            const float rs = fast_rsqrt(ss * (1.0f / (float)HD) + a.eps);
+            x0 = x0 * rs * (kn0 + one);
+            x1 = x1 * rs * (kn1 + one);
+        }
+        const __half h0 = __float2half_rn(fmaf(x0, rc, -(x1 * rsn))), h1 = __float2half_rn(fmaf(x0, rsn, x1 * rc));
+        nv0 = __float2half_rn(vx0);
+        nv1 = __float2half_rn(vx1);
+        if (on) {
+            const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;
+            static_cast<__half*>(a.Kc)[rowoff + i0] = h0;
+            static_cast<__half*>(a.Kc)[rowoff + i1] = h1;
+            static_cast<__half*>(a.Vc)[rowoff + lh] = nv0;
+            static_cast<__half*>(a.Vc)[rowoff + lh + HALF] = nv1;
+            reinterpret_cast<__half*>(s_nk)[i0] = h0;
+            reinterpret_cast<__half*>(s_nk)[i1] = h1;
+        }
+    }
+    __syncthreads();  // the query heads come from the other waves (the new row stays within its wave)
+
+    // ---- B operands: head column j (columns past G repeat head 0), both terms ----
+    fd_h8 qh[KS], ql[KS];
+    {
+        const int jq = j < G ? j : 0;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            qh[s] = *reinterpret_cast<const fd_h8*>(&s_qh[jq][32 * s + 8 * rg]);
+            ql[s] = *reinterpret_cast<const fd_h8*>(&s_ql[jq][32 * s + 8 * rg]);
+        }
+    }
+    // ---- scores (base 2) of this wave's tiles: lane = (head j, positions 4 rg .. +3 of each tile) ----
+    fd_f4 sc[TPW];
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+        const int64_t tt0 = wt0 + 16 * u;
+        if (owner && past >= tt0 && past < tt0 + 16 && j == (int)(past - tt0)) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) kreg[u][s] = *reinterpret_cast<const uint4*>(&s_nk[32 * s + 8 * rg]);
+        }
+        fd_f4 c = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const fd_h8 kf = __builtin_bit_cast(fd_h8, kreg[u][s]);
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qh[s], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, ql[s], c, 0, 0, 0);
+        }
+        // only a tile that reaches the new position or the window's edge holds positions that do not count (wave-uniform)
+        if (tt0 + 16 > past || tt0 < t_begin) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t t = tt0 + 4 * rg + r;
+                c[r] = (t < total && t >= t_begin) ? c[r] : -INFINITY;
+            }
+        }
+        sc[u] = c;
+    }
+    // ---- this wave's V rows into its LDS tile, row-major; rows that do not count are zeroed (0 * garbage must not be NaN) ----
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+        const int64_t tt0 = wt0 + 16 * u;
+        const bool edge = tt0 + 16 > past || tt0 < t_begin;  // wave-uniform
+#pragma unroll
+        for (int vl = 0; vl < VL; ++vl) {
+            const int row = vl * RPL + lane / LPR;
+            uint4 v = vreg[u][vl];
+            if (edge) {
+                const int64_t t = tt0 + row;
+                if (!(t < past && t >= t_begin)) v = make_uint4(0u, 0u, 0u, 0u);
+            }
+            *reinterpret_cast<uint4*>(&s_v[wave][u][row * VP + 16 * (lane % LPR)]) = v;
+        }
+        if (owner && past >= tt0 && past < tt0 + 16 && on) {
+            __half* vrow = reinterpret_cast<__half*>(&s_v[wave][u][(int)(past - tt0) * VP]);
+            vrow[lh] = nv0;
+            vrow[lh + HALF] = nv1;
+        }
+    }
+    // the V^T fragments are requested before the softmax arithmetic, which covers the LDS round trip
+    fd_h4 vb[DT][TPW];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int u = 0; u < TPW; ++u)
+            vb[dt][u] = fd_lds_read_tr16(&s_v[wave][u][(4 * rg + (j >> 2)) * VP + (16 * dt + 4 * (j & 3)) * 2]);
+    // ---- wave-local softmax statistics ----
+    float m = fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3]));
+    if constexpr (TPW == 2) m = fmaxf(m, fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
+    m = fd_rows_max(m);
+    const float ms = m == -INFINITY ? 0.0f : m;  // a wave without valid positions contributes nothing
+    float l = 0.0f;
+    fd_h4 ph[TPW], pl[TPW];
+#pragma unroll
+    for (int u = 0; u < TPW; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float p = __builtin_amdgcn_exp2f(sc[u][r] - ms);  // -inf -> 0
+            l += p;
+            const _Float16 h = (_Float16)p;
+            ph[u][r] = h;
+            pl[u][r] = (_Float16)(p - (float)h);
+        }
+    l = fd_rows_sum(l);
+    // ---- O[head][dim] += P . V ----
+    fd_f4 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        fd_f4 c = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (TPW == 1) {
+            c = __builtin_amdgcn_mfma_f32_16x16x16f16(ph[0], vb[dt][0], c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_16x16x16f16(pl[0], vb[dt][0], c, 0, 0, 0);
+        } else {
+            // the 32 positions of both tiles in one product: summation index 8 rg + 4 u + r <-> position 16 u + 4 rg + r
+            const fd_h4 v0 = vb[dt][0], v1 = vb[dt][TPW - 1];
+            const fd_h8 b8 = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+            const fd_h8 ah = {ph[0][0], ph[0][1], ph[0][2], ph[0][3], ph[TPW - 1][0], ph[TPW - 1][1], ph[TPW - 1][2], ph[TPW - 1][3]};
+            const fd_h8 al = {pl[0][0], pl[0][1], pl[0][2], pl[0][3], pl[TPW - 1][0], pl[TPW - 1][1], pl[TPW - 1][2], pl[TPW - 1][3]};
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, b8, c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, b8, c, 0, 0, 0);
+        }
+        acc[dt] = c;
+    }
+    // lane (j, rg) holds O[head 4 rg + r][dim 16 dt + j]: head rows past G are the repeated columns' and are dropped
+    if (4 * rg < G) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            *reinterpret_cast<float4*>(&s_o[wave][16 * dt + j][4 * rg]) = make_float4(acc[dt][0], acc[dt][1], acc[dt][2], acc[dt][3]);
+    }
+    if (rg == 0 && j < G) { s_m[wave][j] = m; s_l[wave][j] = l; }
+    __syncthreads();
+    // ---- merge the four wave partials into the chunk's partial ----
+    for (int e = tid; e < G * HD; e += FD_THREADS) {
+        const int g = e / HD, d = e % HD;
+        const float m0 = s_m[0][g], m1 = s_m[1][g], m2 = s_m[2][g], m3 = s_m[3][g];
+        const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));  // finite: the chunk holds at least one valid position
+        const float w0 = __builtin_amdgcn_exp2f(m0 - M), w1 = __builtin_amdgcn_exp2f(m1 - M),
+                    w2 = __builtin_amdgcn_exp2f(m2 - M), w3 = __builtin_amdgcn_exp2f(m3 - M);
+        const float o = (w0 * s_o[0][d][g] + w1 * s_o[1][d][g]) + (w2 * s_o[2][d][g] + w3 * s_o[3][d][g]);
+        const int64_t oi = (int64_t)split * a.n_heads + kvh * G + g;
+        a.pO[oi * HD + d] = o;
+        if (d == 0) {
+            a.pM[oi] = M;
+            a.pL[oi] = (w0 * s_l[0][g] + w1 * s_l[1][g]) + (w2 * s_l[2][g] + w3 * s_l[3][g]);
+        }
+    }
+}
+
+template <int HD, int TPW>
+static int attn_mfma_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
+#define PTM_AM(GG) hipLaunchKernelGGL((attn_decode_mfma_kernel<HD, GG, TPW>), grid, dim3(FD_THREADS), 0, s, a)
+    switch (G) {
+        case 1: PTM_AM(1); break;
+        case 2: PTM_AM(2); break;
+        case 3: PTM_AM(3); break;
+        case 4: PTM_AM(4); break;
+        case 5: PTM_AM(5); break;
+        case 6: PTM_AM(6); break;
+        case 7: PTM_AM(7); break;
+        case 8: PTM_AM(8); break;
+        default: return PTM_E_UNSUPPORTED;
+    }
+#undef PTM_AM
+    return launch_status();
+}
+
 template <bool KV16, int HD>
 static int attn_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
 #define PTM_AT(GG) hipLaunchKernelGGL((attn_decode_fused_kernel<KV16, HD, GG>), grid, dim3(FD_THREADS), 0, s, a)
@@ -788,10 +1117,16 @@ int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, co
     const dim3 grid(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
     hipStream_t s = as_stream(stream);
     int rc;
-    if (kv_fp16) rc = head_dim == 128 ? attn_launch_g<true, 128>(G, grid, s, a) : attn_launch_g<true, 64>(G, grid, s, a);
-    else rc = head_dim == 128 ? attn_launch_g<false, 128>(G, grid, s, a) : attn_launch_g<false, 64>(G, grid, s, a);
-    if (rc != PTM_OK) return rc;
     if (o_q8 && (reinterpret_cast<uintptr_t>(o_q8) & 15u)) return PTM_E_ALIGN;
+    if (kv_fp16) {
+        // fp16 cache: the matrix-core kernel, chunks of 64 positions; partial maxima in base-2 units
+        rc = head_dim == 128 ? attn_mfma_launch_g<128, 1>(G, grid, s, a) : attn_mfma_launch_g<64, 1>(G, grid, s, a);
+        if (rc != PTM_OK) return rc;
+        return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
+                        static_cast<uint8_t*>(o_q8), 0, FD_CHUNK, 1);
+    }
+    rc = head_dim == 128 ? attn_launch_g<false, 128>(G, grid, s, a) : attn_launch_g<false, 64>(G, grid, s, a);
+    if (rc != PTM_OK) return rc;
     return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
                     static_cast<uint8_t*>(o_q8));
 }
