@@ -189,6 +189,30 @@ def make_layer(seed: int, layer: int, cfg: dict, norm_scale: dict | None = None,
     return out
 
 
+def center_q4k(W: np.ndarray) -> np.ndarray:
+    """The Q4_K super-blocks of W with their mins set equal to their scales and dmin = fp16(7.5 d): a block then holds
+    d * scale * (q - 7.5), values symmetric about zero.  (make_q4k's independent scales and mins give every weight a large
+    positive mean, d * 31.5 * 7.5 - dmin * 31.5; a network of such matrices is close to rank one - whatever token is fed, its
+    logits point along one of two directions.)"""
+    rows = W.shape[0]
+    blk = W.reshape(-1, 144).copy()
+    sc, _ = unpack_scales_k4(blk[:, 4:16])
+    blk[:, 4:16] = pack_scales_k4(sc, sc)
+    d = blk[:, 0:2].copy().view(np.float16).astype(np.float32)
+    blk[:, 2:4] = (np.float32(7.5) * d).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    return blk.reshape(rows, -1)
+
+
+def make_layer_centered(seed: int, layer: int, cfg: dict, norm_scale: dict | None = None) -> dict:
+    """make_layer with every Q4_K matrix centred (center_q4k): the same seeds, scales and quants."""
+    L = make_layer(seed, layer, cfg, norm_scale)
+    for name, _ in LAYER_MATS:
+        qt, W = L[name]
+        if qt == Q4_K:
+            L[name] = (qt, center_q4k(W))
+    return L
+
+
 def make_head(seed: int, cfg: dict) -> dict:
     """Tied Q6_K token-embedding / lm_head table and the output norm."""
     g = rng_for(seed, 3)

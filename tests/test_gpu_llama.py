@@ -35,6 +35,28 @@ def tiny_llama_with_cache(seeds, n=19):
 
 
 @pytest.mark.parametrize("use_graph", [False, True])
+def test_llama_teacher_forced_vs_reference_golden(dev, golden_llama, seeds, use_graph):
+    """16 distinct seeded ids fed step by step (the greedy run of this model repeats one id): argmax and logits of every step
+    against the compiled reference's run of the same feed."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = tiny_llama_with_cache(seeds)
+    dec = Decoder(cfg, layers, head, max_seq=64, kv_fp16=False, use_graph=use_graph)
+    for i, (k, v) in enumerate(kv):
+        dec.set_kv(i, k, v)
+    dec.set_past_len(19)
+    errs = []
+    for st, t in enumerate(int(t) for t in golden_llama["forced_feed"]):
+        tok = dec.step(t)
+        ref = golden_llama["forced_logits"][st]
+        errs.append(np.abs(dec.logits() - ref).max() / ref.std())
+        srt = np.sort(ref)
+        if (srt[-1] - srt[-2]) / ref.std() > 2 * max(errs[-1], 1e-4):
+            assert tok == int(golden_llama["forced_tokens"][st]), (st, errs[-1])
+    check_step_errors(errs)
+    dec.close()
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
 def test_llama_decode_fp32_kv_vs_reference_golden(dev, golden_llama, seeds, use_graph):
     from prometorch_amd.decode import Decoder
     cfg, layers, head, kv = tiny_llama_with_cache(seeds)

@@ -319,6 +319,26 @@ def test_gemma_style_decode_matches_the_reference(po, seeds):
         assert np.abs(l1[0] - g["logits"][0]).max() > 1e-2 * sigma, name
 
 
+@pytest.mark.parametrize("family", ["llama", "qwen2", "gemma"])
+def test_teacher_forced_family_runs_match_the_reference(po, seeds, family):
+    """The greedy runs of the tiny family models settle on one token (llama: 999 x 12); these runs feed 16 distinct seeded ids
+    instead, so every step reads another embedding row and appends other cache rows: oracle logits bit-identical to the
+    compiled reference's forward_decode_cpu (forced_* of golden_<family>.npz), argmax identical."""
+    import os
+    from prometorch_amd.testing import synth
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "golden_%s.npz" % family))
+    cfg, layers, head = getattr(synth, "tiny_" + family)(seeds["tiny"])
+    om = po.OracleModel(cfg, layers, head, 64, kv_fp16=False)
+    for i in range(cfg["n_layers"]):
+        om.set_kv(i, *synth.make_kv_prefill(seeds["tiny"], i, cfg, 19))
+    feed = [int(t) for t in g["forced_feed"]]
+    assert len(set(feed)) == 16
+    for st, t in enumerate(feed):
+        assert om.step(t) == int(g["forced_tokens"][st]), st
+        assert np.array_equal(om.logits.view(np.uint32), g["forced_logits"][st].view(np.uint32)), st
+    assert len(set(int(t) for t in g["forced_tokens"])) >= 9    # the outputs vary too
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_random_architectures_match_the_reference(po, seed):
     """synth.random_model draws every architectural switch at random (head width, heads per kv head, QK-norm, rotation
