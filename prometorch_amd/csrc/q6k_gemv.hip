@@ -15,6 +15,7 @@
 // Every pass issues a fixed number of block loads (template NB) behind the activation loads, so the compiler can
 // count the loads in flight and each block is consumed as soon as it has arrived.
 #include "q6k_body.h"
+#include "q6k_mfma_body.h"
 
 #include <mutex>
 
@@ -24,6 +25,13 @@ template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
 __global__ __launch_bounds__(Q6K_THREADS) void q6k_gemv_kernel(const Q6KArgs a) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
     q6k_gemv_body<ACC, ARGMAX, NORM, XCH, NB>(a, lds_raw, blockIdx.x);
+}
+
+// three waves per SIMD (at most 168 registers): with two the vector pipe idles while a wave waits for its staged block
+template <bool ACC, bool ARGMAX, bool NORM, int XL, int NB>
+__global__ __launch_bounds__(Q6K_THREADS) __attribute__((amdgpu_waves_per_eu(3, 3))) void q6k_mfma_gemv_kernel(const Q6KArgs a) {
+    extern __shared__ __align__(16) uint8_t lds_raw[];
+    q6k_mfma_gemv_body<ACC, ARGMAX, NORM, XL, NB>(a, lds_raw);
 }
 
 // Few rows, long rows (a down projection: 2560 x 9728, 4096 x 14336): with 4 rows per workgroup every workgroup
@@ -250,8 +258,27 @@ static int q6k_launch_xch(const Q6KArgs& a, int grid, size_t lds, hipStream_t s)
     }
 }
 
+// many rows: the matrix-core kernel (64 rows per workgroup, a 16-row tile per wave)
+template <bool ACC, bool ARGMAX, bool NORM>
+static int q6k_launch_mfma(const Q6KArgs& a, hipStream_t s) {
+    const int grid = q6k_mfma_workgroups(a.N);
+    const size_t lds = 4 * (size_t)a.K + 4 * 16 * Q6M_PITCH;   // x as two fp16 terms + a tile of 16 row-blocks per wave
+    const int nblk = a.K / 256;
+    const int nb = nblk >= 4 ? 4 : 2;   // blocks in flight per lane (even: a slot's block parity is fixed); they roll
+#define PTM_Q6M(XLV, NBV) hipLaunchKernelGGL((q6k_mfma_gemv_kernel<ACC, ARGMAX, NORM, XLV, NBV>), dim3(grid), dim3(Q6K_THREADS), lds, s, a)
+    if (a.K <= 4096) {
+        if (nb == 2) PTM_Q6M(4, 2);
+        else PTM_Q6M(4, 4);
+    } else {
+        PTM_Q6M(8, 4);
+    }
+#undef PTM_Q6M
+    return launch_status();
+}
+
 template <bool ACC, bool ARGMAX, bool NORM>
 static int q6k_launch(Q6KArgs& a, hipStream_t s) {
+    if (q6k_mfma_shape(a.N, a.K)) return q6k_launch_mfma<ACC, ARGMAX, NORM>(a, s);
     a.log2S = q6k_pick_log2S(a.N, a.K / 256);
     const int grid = q6k_workgroups(a.N, a.K);
     const size_t lds = (size_t)a.K * 4 + (size_t)a.K / 4;
@@ -289,7 +316,7 @@ int q6k_gemv_argmax_impl(const void* W, const float* x, const float* gamma, floa
     if (!out_index || !workspace) return PTM_E_NULL;
     if (gamma && !aligned16(gamma)) return PTM_E_ALIGN;
     if (xn_out && !aligned16(xn_out)) return PTM_E_ALIGN;
-    const int grid = q6k_workgroups(N, K);
+    const int grid = q6k_mfma_shape(N, K) ? q6k_mfma_workgroups(N) : q6k_workgroups(N, K);
     Q6KArgs a{static_cast<const uint8_t*>(W), x, logits, K, N, 0, stride, static_cast<float*>(workspace),
               reinterpret_cast<int*>(static_cast<float*>(workspace) + grid), gamma, eps, add_one, xn_out};
     const int rc2 = gamma ? q6k_launch<false, true, true>(a, s) : q6k_launch<false, true, false>(a, s);
