@@ -143,7 +143,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--cpu-tokens", type=int, default=12, help="tokens of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-tokens", type=int, default=16, help="tokens of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-child", type=int, default=0, help=argparse.SUPPRESS)  # the 1-thread CPU measurement, see cpu_child_main
+    ap.add_argument("--long-context", type=int, default=1, help="0: skip the decode measurements at 8192 / 32768 positions")
+    ap.add_argument("--mix-steps", type=int, default=64, help="decode steps of the alternating Q4_K / Q6_K type mix (0 = skip)")
     ap.add_argument("--gemma-steps", type=int, default=64,
                     help="decode steps of the Gemma-3-4B-shaped extra (0: skip it)")
     ap.add_argument("--llama-steps", type=int, default=64,
@@ -153,12 +156,24 @@ def main():
                     help="launch just this prompt-pass kernel a few times and print its time: the target of the counter "
                          "passes behind the figures quoted for it (rocprofv3 --pmc ... -- python3 bench.py --only ...)")
     args = ap.parse_args()
+    if args.cpu_child > 0:
+        os.dup2(json_fd, 1)
+        cpu_child_main(args.cpu_child)
+        return
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU (batch-1 decode); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
     if args.steps + args.warmup + N_PREFILL + 1 > MAX_SEQ:
         print("bench.py: steps + warmup must stay below %d" % (MAX_SEQ - N_PREFILL - 1), file=sys.stderr)
         sys.exit(2)
+
+    # the 1-thread CPU baseline runs beside everything below, in a child started before this process touches the GPU
+    child = None
+    if args.cpu_tokens > 0 and not args.only:
+        import subprocess
+        env = dict(os.environ, PT_NUM_THREADS="1", OMP_NUM_THREADS="1")
+        child = subprocess.Popen([sys.executable, os.path.abspath(__file__), "--cpu-child", str(args.cpu_tokens)],
+                                 stdout=subprocess.PIPE, env=env)
 
     import torch
     from prometorch_amd import _lib, ops
@@ -448,11 +463,100 @@ def main():
         del gdec, glayers, ghead
         torch.cuda.empty_cache()
 
+    # ---- what real Q4_K_M files look like: attn_v and ffn_down alternate between Q6_K and Q4_K from layer to layer
+    # (Q6_K in the first and the last eighth of the layers and in every third layer between, Q4_K elsewhere: the rule the
+    # reference's loader meets in such files, cpu_quant_gemv.h:1458-1460) -----------------------------------------------
+    mix = None
+    if args.mix_steps > 0:
+        nLm = cfg["n_layers"]
+
+        def more_bits(li):
+            return li < nLm // 8 or li >= 7 * nLm // 8 or (li - nLm // 8) % 3 == 2
+
+        mlayers = []
+        for li in range(nLm):
+            t = 14 if more_bits(li) else 12
+            mats = tuple((n, t if n in ("v", "down") else q) for n, q in synth.LAYER_MATS)
+            mlayers.append(layers[li] if t == 14 else synth.make_layer(SEED, li, cfg, mats=mats))
+        n_q6 = sum(1 for li in range(nLm) if more_bits(li))
+        mdec = Decoder(cfg, mlayers, head, max_seq=MAX_SEQ, kv_fp16=True, use_graph=True)
+        for i in range(nLm):
+            mdec.set_kv(i, *kvs[i])
+        mdec.set_past_len(N_PREFILL)
+        mtok = 1
+        for _ in range(args.warmup):
+            mtok = mdec.step(mtok)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.mix_steps):
+            mtok = mdec.step(mtok)
+        torch.cuda.synchronize()
+        mdt = time.perf_counter() - t1
+        # the Q4_K down projection 2560 x 9728 (accumulating), cycling the layers that hold one
+        q4_layers = [i for i in range(nLm) if not more_bits(i)]
+        xa4 = torch.randn(I, device="cuda")
+        yd4 = torch.zeros(H, device="cuda")
+        sd4 = I // 256 * 144
+        bd4 = H * sd4 + 4 * I + 4 * H
+        ML = mdec._layers
+        msd4 = event_time_ms(lambda i: ops.launch_q4km_persistent_gemv_accumulate(ML[q4_layers[i % len(q4_layers)]].down.data, xa4, yd4, I, H, sd4),
+                             360, torch)
+        mix = {"workload": "batch-1 greedy decode, Qwen3-4B shape with the attn_v / ffn_down types of a Q4_K_M file: Q6_K in %d layers, "
+                           "Q4_K in %d; fp16 KV prefilled %d, %d new tokens, host-synchronous" % (n_q6, nLm - n_q6, N_PREFILL, args.mix_steps),
+               "tok_s": args.mix_steps / mdt, "ms_per_token": mdt / args.mix_steps * 1e3,
+               "q4k_down_2560x9728": {"bytes": bd4, "us": msd4 * 1e3, "GBs": bd4 / msd4 / 1e6, "frac": bd4 / msd4 / 1e6 / HBM_PEAK_GBS}}
+        log("Q4_K_M file mix: %.1f tok/s; Q4_K down 2560x9728 %.2f us (%.2f of peak)" % (mix["tok_s"], msd4 * 1e3, mix["q4k_down_2560x9728"]["frac"]))
+        mdec.close()
+        del mdec, mlayers
+        torch.cuda.empty_cache()
+
+    # ---- decode deep into a long chat: the same model with 8192 and 32768 cached positions (fp16 cache, 4.8 GB at 32 k) ----
+    longctx = None
+    if args.long_context:
+        LMAX = 32768 + 256
+        ldec2 = Decoder(cfg, layers, head, max_seq=LMAX, kv_fp16=True, use_graph=True)
+        for i in range(cfg["n_layers"]):
+            ldec2.k_cache[i].normal_()
+            ldec2.v_cache[i].normal_()
+        nh, nkv, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+        S2 = ops.flash_decode_num_splits(LMAX)
+        q_ = torch.randn(nh * hd, device="cuda")
+        k_ = torch.randn(nkv * hd, device="cuda")
+        v_ = torch.randn(nkv * hd, device="cuda")
+        w_ = torch.ones(hd, device="cuda")
+        O_ = torch.empty(nh * hd, device="cuda")
+        pO_ = torch.empty(S2 * nh * hd, device="cuda")
+        pL_ = torch.empty(S2 * nh, device="cuda")
+        pM_ = torch.empty(S2 * nh, device="cuda")
+        rope_ = ops.rope_table(LMAX, hd, cfg["rope_base"]).cuda()
+        longctx = {"max_seq": LMAX}
+        for T in (2048, 8192, 32768):
+            ldec2.set_past_len(T)
+            ltok2 = 1
+            for _ in range(4):
+                ltok2 = ldec2.step(ltok2)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(32):
+                ltok2 = ldec2.step(ltok2)
+            torch.cuda.synchronize()
+            ldt2 = (time.perf_counter() - t1) / 32
+            past_ = torch.tensor([T + 20], dtype=torch.int64, device="cuda")
+            msa = event_time_ms(lambda i: ops.attn_decode_fused(q_, k_, v_, w_, w_, ldec2.k_cache[i % 36], ldec2.v_cache[i % 36], O_, pO_, pL_, pM_,
+                                                                rope_, nh, nkv, hd, past_, LMAX, hd ** -0.5, 1e-6), 72, torch)
+            kvb = 2 * (T + 20) * nkv * hd * 2
+            longctx["past_%d" % T] = {"tok_s": 1.0 / ldt2, "ms_per_token": ldt2 * 1e3, "attn_plus_merge_us": msa * 1e3,
+                                      "kv_bytes_per_layer": kvb, "attn_GBs": kvb / msa / 1e6}
+            log("past %d (cache of %d): %.1f tok/s, attention + merge %.1f us per layer (%.0f GB/s)" % (T, LMAX, 1.0 / ldt2, msa * 1e3, kvb / msa / 1e6))
+        ldec2.close()
+        del ldec2
+        torch.cuda.empty_cache()
+
     # ---- CPU baseline on this host: bounded sample of the same workload ---------------------------
     cpu = None
     if args.cpu_tokens > 0:
         try:
-            cpu = cpu_baseline(cfg, layers, head, kvs, args.cpu_tokens, toks, args.warmup)
+            cpu = cpu_baseline(cfg, layers, head, kvs, args.cpu_tokens, child)
         except Exception as e:  # the baseline is reported, never required
             log("cpu baseline failed: %r" % (e,))
     out = {
@@ -467,6 +571,8 @@ def main():
         "sampled_tok_s": sampled_tok_s, "sampled_chained_tok_s": sampled_chained_tok_s,
         "llama3_8b_shape": llama,
         "gemma3_4b_shape": gemma,
+        "q4km_file_type_mix": mix,
+        "long_context": longctx,
         "a100_published_tok_s": 82.6, "x_a100_published": tok_s / 82.6,
         "token_hbm_frac": per_token_bytes / (dt / args.steps) / 1e9 / HBM_PEAK_GBS,
     }
@@ -475,12 +581,13 @@ def main():
     os.close(json_fd)
 
 
-def cpu_baseline(cfg, layers, head, kvs, n_tokens, gpu_tokens, warmup):
-    """Time the reference CPU decode path on this host for n_tokens tokens of the same workload."""
+def cpu_measure(cfg, layers, head, kvs, n_tokens):
+    """The reference's CPU path (oracle/_ref when built, else this repository's C port) on this host with however many
+    threads its pool was created with: configs[0] / [1] / [2] as GB/s over the algorithmic bytes (median of 5 timed passes
+    after a warm-up pass, weights beyond the host caches), configs[3] as tokens per second over n_tokens greedy tokens."""
     from oracle import pyoracle as po
     from prometorch_amd.testing import synth
-    kind = "port"
-    model = None
+    kind, model, cores = "port", None, None
     if po.have_ref():
         try:
             emb = po.dequant(14, head["lm_head"]).reshape(cfg["vocab"], cfg["hidden"])
@@ -492,31 +599,95 @@ def cpu_baseline(cfg, layers, head, kvs, n_tokens, gpu_tokens, warmup):
     if model is None:
         model = po.OracleModel(cfg, layers, head, MAX_SEQ, kv_fp16=False)
         cores = po.lib().po_num_threads()
+    gemv = po.ref_gemv if kind == "reference" else po.gemv
+    H, I, V = cfg["hidden"], cfg["inter"], cfg["vocab"]
+    nL = len(layers)
+
+    def median5(fn):
+        fn(0)
+        ts = []
+        for rep in range(5):
+            t = time.perf_counter()
+            fn(rep + 1)
+            ts.append(time.perf_counter() - t)
+        return sorted(ts)[2]
+
+    out = {}
+    xh = synth.make_x(synth.rng_for(SEED, 11), H)
+    xi = synth.make_x(synth.rng_for(SEED, 12), I)
+    xq = synth.make_x(synth.rng_for(SEED, 13), cfg["n_heads"] * cfg["head_dim"])
+    # configs[0]: one Q4_K GEMV 9728 x 2560; a pass = 6 launches over 6 layers' gate matrices (84 MB), another 6 each pass
+    n0 = 6
+    b0 = layers[0]["gate"][1].size + 4 * H + 4 * I
+    t0 = median5(lambda rep: [gemv(12, layers[(n0 * rep + i) % nL]["gate"][1], xh) for i in range(n0)]) / n0
+    out["cfg0_q4k_gemv_9728x2560"] = {"us": t0 * 1e6, "GBs": b0 / t0 / 1e9}
+    # configs[1]: Q6_K lm_head 151936 x 2560 + argmax (319 MB per pass)
+    b1 = head["lm_head"].size + 4 * H + 4 * V
+    t1 = median5(lambda rep: int(np.argmax(gemv(14, head["lm_head"], xh))))
+    out["cfg1_q6k_lm_head_argmax"] = {"us": t1 * 1e6, "GBs": b1 / t1 / 1e9}
+    # configs[2]: the seven GEMVs of one decoder layer in the Q4_K_M mix (64 MB), another layer each pass
+    def layer_gemvs(rep):
+        L = layers[rep % nL]
+        for name, xx in (("q", xh), ("k", xh), ("v", xh), ("o", xq), ("gate", xh), ("up", xh), ("down", xi)):
+            gemv(L[name][0], L[name][1], xx)
+    b2 = sum(layers[0][n][1].size for n in ("q", "k", "v", "o", "gate", "up", "down"))
+    t2 = median5(layer_gemvs)
+    out["cfg2_layer_gemvs"] = {"us": t2 * 1e6, "GBs": b2 / t2 / 1e9}
+    # configs[3]: greedy tokens of the whole model after one warm-up token
     for i, (k, v) in enumerate(kvs):
         model.set_kv(i, k, v)
-    tok = model.step(1)  # warm-up token (page-in)
+    tok = model.step(1)
     t = time.perf_counter()
     for _ in range(n_tokens):
         tok = model.step(tok)
     dt = time.perf_counter() - t
-    log("cpu baseline (%s, %d threads): %.2f tok/s" % (kind, cores, n_tokens / dt))
     if hasattr(model, "close"):
         model.close()
-    # the same host on configs[0]: one Q4_K GEMV 9728x2560 through the reference's dispatcher (or the port's), cycling
-    # the 36 layers' gate matrices (504 MB, beyond the host caches)
-    gemv = po.ref_gemv if kind == "reference" else po.gemv
-    xg = synth.make_x(synth.rng_for(SEED, 11), cfg["hidden"])
-    gemv(12, layers[0]["gate"][1], xg)
-    t = time.perf_counter()
-    n_gemv = 3 * len(layers)
-    for i in range(n_gemv):
-        gemv(12, layers[i % len(layers)]["gate"][1], xg)
-    dtg = (time.perf_counter() - t) / n_gemv
-    wbytes = layers[0]["gate"][1].size + 4 * cfg["hidden"] + 4 * cfg["inter"]
-    log("cpu baseline GEMV 9728x2560: %.1f us, %.1f GB/s" % (dtg * 1e6, wbytes / dtg / 1e9))
-    return {"value": n_tokens / dt, "unit": "tok/s", "cores": int(cores), "kind": kind,
-            "sample": "%d greedy tokens of the same 36-layer model after 1 warm-up token, KV prefilled to %d (fp32 KV on the CPU)" % (n_tokens, N_PREFILL),
-            "cfg0_q4k_gemv_9728x2560": {"us": dtg * 1e6, "GBs": wbytes / dtg / 1e9, "launches": n_gemv}}
+    out["tok_s"] = n_tokens / dt
+    out["tokens"] = n_tokens
+    out["cores"] = int(cores)
+    out["kind"] = kind
+    log("cpu baseline (%s, %d threads): %.2f tok/s; cfg0 %.1f GB/s, cfg1 %.1f GB/s, cfg2 %.1f GB/s" %
+        (kind, cores, out["tok_s"], out["cfg0_q4k_gemv_9728x2560"]["GBs"], out["cfg1_q6k_lm_head_argmax"]["GBs"],
+         out["cfg2_layer_gemvs"]["GBs"]))
+    return out
+
+
+def cpu_child_main(n_tokens):
+    """`bench.py --cpu-child N`: the CPU measurement alone, in a process of its own that never touches the GPU.  The parent
+    starts it with PT_NUM_THREADS=1 (the reference sizes its thread pool once per process, c10/util/ThreadPool.h:96-109) before
+    it initialises the GPU itself, and reads the JSON line this prints."""
+    from prometorch_amd.testing import synth
+    cfg = dict(synth.QWEN3_4B)
+    layers = [synth.make_layer(SEED, i, cfg) for i in range(cfg["n_layers"])]
+    head = synth.make_head(SEED, cfg)
+    kvs = [synth.make_kv_prefill(SEED, i, cfg, N_PREFILL) for i in range(cfg["n_layers"])]
+    json_fd = os.dup(1)
+    os.dup2(2, 1)
+    res = cpu_measure(cfg, layers, head, kvs, n_tokens)
+    os.write(json_fd, (json.dumps(res) + "\n").encode())
+
+
+def cpu_baseline(cfg, layers, head, kvs, n_tokens, one_thread_child):
+    """cpu_baseline of the JSON line: the T-thread measurement made here, the 1-thread one collected from the child."""
+    full = cpu_measure(cfg, layers, head, kvs, n_tokens)
+    one = None
+    if one_thread_child is not None:
+        try:
+            stdout, _ = one_thread_child.communicate(timeout=600)
+            one = json.loads(stdout.decode().strip().splitlines()[-1])
+        except Exception as e:  # reported, never required
+            log("1-thread cpu baseline failed: %r" % (e,))
+    res = {"value": full["tok_s"], "unit": "tok/s", "cores": full["cores"], "kind": full["kind"],
+           "sample": "%d greedy tokens of the same 36-layer model after 1 warm-up token, KV prefilled to %d (fp32 KV on the CPU); "
+                     "configs[0..2]: median of 5 timed passes after a warm-up pass, GB/s over the algorithmic bytes" % (n_tokens, N_PREFILL),
+           "cfg0_q4k_gemv_9728x2560": full["cfg0_q4k_gemv_9728x2560"], "cfg1_q6k_lm_head_argmax": full["cfg1_q6k_lm_head_argmax"],
+           "cfg2_layer_gemvs": full["cfg2_layer_gemvs"]}
+    if one is not None:
+        res["one_thread"] = {"value": one["tok_s"], "unit": "tok/s", "cores": one["cores"], "tokens": one["tokens"],
+                             "cfg0_q4k_gemv_9728x2560": one["cfg0_q4k_gemv_9728x2560"],
+                             "cfg1_q6k_lm_head_argmax": one["cfg1_q6k_lm_head_argmax"], "cfg2_layer_gemvs": one["cfg2_layer_gemvs"]}
+    return res
 
 
 if __name__ == "__main__":

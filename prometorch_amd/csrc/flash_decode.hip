@@ -70,7 +70,10 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
         if (total <= 0 || total > max_seq) return;  // never touch memory outside the cache
     }
     if (total > max_seq) total = max_seq;
-    const int split = blockIdx.x, kvh = blockIdx.y;
+    // kv head fastest: workgroups are dispatched in index order, so the live chunks of ALL heads start before the chunks
+    // past the position (a cache far longer than the context: those workgroups only look at the position and leave)
+    const int wg_lin = blockIdx.x + gridDim.x * blockIdx.y;
+    const int kvh = wg_lin % (int)gridDim.y, split = wg_lin / (int)gridDim.y;
     const int64_t t0 = (int64_t)split * FD_CHUNK;
     if (t0 >= total) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -462,7 +465,10 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     const int64_t past = *a.d_past;
     if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
     const int64_t total = past + 1;
-    const int split = blockIdx.x, kvh = blockIdx.y;
+    // kv head fastest: workgroups are dispatched in index order, so the live chunks of ALL heads start before the chunks
+    // past the position (a cache far longer than the context: those workgroups only look at the position and leave)
+    const int wg_lin = blockIdx.x + gridDim.x * blockIdx.y;
+    const int kvh = wg_lin % (int)gridDim.y, split = wg_lin / (int)gridDim.y;
     const int64_t t0 = (int64_t)split * FD_CHUNK;
     if (t0 >= total) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -723,7 +729,10 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     const int64_t past = *a.d_past;
     if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
     const int64_t total = past + 1;
-    const int split = blockIdx.x, kvh = blockIdx.y;
+    // kv head fastest: workgroups are dispatched in index order, so the live chunks of ALL heads start before the chunks
+    // past the position (a cache far longer than the context: those workgroups only look at the position and leave)
+    const int wg_lin = blockIdx.x + gridDim.x * blockIdx.y;
+    const int kvh = wg_lin % (int)gridDim.y, split = wg_lin / (int)gridDim.y;
     const int64_t t0 = (int64_t)split * CH;
     if (t0 >= total) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
