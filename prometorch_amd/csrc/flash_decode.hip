@@ -15,6 +15,7 @@
 namespace ptm {
 
 enum { FD_CHUNK = 64, FD_THREADS = 256 };
+enum { FD_LONG_SPLITS = 64 };   // partials per head of the looping kernel for long caches (attn_decode_mfma_long_kernel)
 
 // e^x through the hardware base-2 exponential (v_exp_f32, 1 ulp): softmax weights need no more, and the libm
 // expf expands to a dozen instructions on a path whose cost is instruction count.  -inf gives 0.
@@ -38,6 +39,26 @@ __device__ __forceinline__ void load8(const void* base, int64_t elem_off, float 
         o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
         o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
     }
+}
+
+// Workgroup index -> (chunk, kv head).  Workgroups are dispatched in index order.  Chunks run fastest within a head (the
+// workgroups that start together then read rows far apart: with the head fastest, eight of them read adjacent 256-byte
+// pieces of the same rows and the launch took 0.6 us longer), but only in blocks of 64 chunks: all heads' chunks 0..63
+// come before any head's chunk 64, so that with a cache far longer than the context the live chunks of every head start
+// before the thousands of workgroups that only look at the position and leave.
+enum { FD_ORDER_BLOCK = 64 };
+__device__ __forceinline__ int fd_lin(int bx, int by, int gx) { return bx + gx * by; }
+__device__ __forceinline__ int fd_split_of(int bx, int by, int gx, int gy) {
+    const int lin = fd_lin(bx, by, gx), per = FD_ORDER_BLOCK * gy;
+    const int blk = lin / per, r = lin - blk * per;
+    const int width = min(FD_ORDER_BLOCK, gx - blk * FD_ORDER_BLOCK);   // chunks in this block (the last may be narrower)
+    return blk * FD_ORDER_BLOCK + r % width;
+}
+__device__ __forceinline__ int fd_head_of(int bx, int by, int gx, int gy) {
+    const int lin = fd_lin(bx, by, gx), per = FD_ORDER_BLOCK * gy;
+    const int blk = lin / per, r = lin - blk * per;
+    const int width = min(FD_ORDER_BLOCK, gx - blk * FD_ORDER_BLOCK);
+    return r / width;
 }
 
 // What a FUSED launch of the kernel below does first: per-head RMSNorm (optional) + rotation of the raw q heads and, in
@@ -70,10 +91,7 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
         if (total <= 0 || total > max_seq) return;  // never touch memory outside the cache
     }
     if (total > max_seq) total = max_seq;
-    // kv head fastest: workgroups are dispatched in index order, so the live chunks of ALL heads start before the chunks
-    // past the position (a cache far longer than the context: those workgroups only look at the position and leave)
-    const int wg_lin = blockIdx.x + gridDim.x * blockIdx.y;
-    const int kvh = wg_lin % (int)gridDim.y, split = wg_lin / (int)gridDim.y;
+    const int split = fd_split_of(blockIdx.x, blockIdx.y, gridDim.x, gridDim.y), kvh = fd_head_of(blockIdx.x, blockIdx.y, gridDim.x, gridDim.y);
     const int64_t t0 = (int64_t)split * FD_CHUNK;
     if (t0 >= total) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -283,8 +301,11 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
     // Every load of the common case goes out before the position is known: chunk slots past the last active one
     // are clamped into the allocation (ns_max chunks) and dropped by selects below, so the kernel makes one
     // memory round trip, not one for the position and a second for the data.
-    const int chunk = 1 << chunk_shift;  // positions per partial
-    const int ns_max = (max_seq + chunk - 1) >> chunk_shift;
+    // chunk_shift < 0: the partials of the looping kernel (at most FD_LONG_SPLITS of them, cpw chunks of 64 positions each)
+    const bool long_mode = chunk_shift < 0;
+    const int chunk = long_mode ? FD_CHUNK : 1 << chunk_shift;  // positions per chunk
+    const int cs_ = long_mode ? 6 : chunk_shift;
+    const int ns_max = long_mode ? min((max_seq + chunk - 1) >> cs_, (int)FD_LONG_SPLITS) : (max_seq + chunk - 1) >> cs_;
     const int64_t past = d_past ? *d_past : past_host;
     // partial maxima are natural-log scores, or base-2 ones (log2_units) from the matrix-core kernel
     const float ek = log2_units ? 1.0f : 1.44269504088896340736f;
@@ -302,7 +323,9 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
     int64_t total = past + 1;
     if (total > max_seq) total = max_seq;
     if (total <= 0) return;
-    const int ns = (int)((total + chunk - 1) >> chunk_shift);
+    const int n_chunks = (int)((total + chunk - 1) >> cs_);
+    const int cpw_ = long_mode ? (n_chunks + (int)FD_LONG_SPLITS - 1) / (int)FD_LONG_SPLITS : 1;
+    const int ns = long_mode ? (n_chunks + cpw_ - 1) / cpw_ : n_chunks;
     float m = tid < ns ? pm_first : -INFINITY;
     for (int sI = tid + 256; sI < ns; sI += 256) m = fmaxf(m, pM[(int64_t)sI * n_heads + h]);
     m = max64(m);
@@ -366,7 +389,7 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const float* __
 static int fd_merge(int head_dim, int n_heads, hipStream_t s, const float* pO, const float* pL, const float* pM, float* O,
                     const int64_t* d_past, int max_seq, uint8_t* q8_out = nullptr, int64_t past_host = 0,
                     int chunk = FD_CHUNK, int log2_units = 0) {
-    const int chunk_shift = chunk == 128 ? 7 : 6;
+    const int chunk_shift = chunk < 0 ? -1 : chunk == 128 ? 7 : 6;
     if (head_dim == 256)
         hipLaunchKernelGGL(flash_decode_merge_kernel<256>, dim3(n_heads), dim3(256), 0, s, pO, pL, pM, O, n_heads, d_past, past_host, max_seq, q8_out, chunk_shift, log2_units);
     else if (head_dim == 128)
@@ -465,10 +488,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_fused_kernel(const Att
     const int64_t past = *a.d_past;
     if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
     const int64_t total = past + 1;
-    // kv head fastest: workgroups are dispatched in index order, so the live chunks of ALL heads start before the chunks
-    // past the position (a cache far longer than the context: those workgroups only look at the position and leave)
-    const int wg_lin = blockIdx.x + gridDim.x * blockIdx.y;
-    const int kvh = wg_lin % (int)gridDim.y, split = wg_lin / (int)gridDim.y;
+    const int split = fd_split_of(blockIdx.x, blockIdx.y, gridDim.x, gridDim.y), kvh = fd_head_of(blockIdx.x, blockIdx.y, gridDim.x, gridDim.y);
     const int64_t t0 = (int64_t)split * FD_CHUNK;
     if (t0 >= total) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -729,10 +749,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     const int64_t past = *a.d_past;
     if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
     const int64_t total = past + 1;
-    // kv head fastest: workgroups are dispatched in index order, so the live chunks of ALL heads start before the chunks
-    // past the position (a cache far longer than the context: those workgroups only look at the position and leave)
-    const int wg_lin = blockIdx.x + gridDim.x * blockIdx.y;
-    const int kvh = wg_lin % (int)gridDim.y, split = wg_lin / (int)gridDim.y;
+    const int split = fd_split_of(blockIdx.x, blockIdx.y, gridDim.x, gridDim.y), kvh = fd_head_of(blockIdx.x, blockIdx.y, gridDim.x, gridDim.y);
     const int64_t t0 = (int64_t)split * CH;
     if (t0 >= total) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -974,6 +991,281 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Long caches (more than FD_LONG_SPLITS chunks of 64 positions fit): the same matrix-core kernel as a loop.  A launch always
+// has FD_LONG_SPLITS workgroups per kv head; workgroup s walks the chunks [s cpw, (s + 1) cpw), cpw = ceil(chunks in use /
+// FD_LONG_SPLITS), with a running maximum / sum / output per wave (online softmax) and leaves ONE partial.  Against one
+// workgroup per chunk this bounds the partials (64 per head instead of 512 at 32 k positions: the merge launch took 8.9 of
+// the 37 us there, and the partials 8 MB of traffic per layer) and the grid (a cache of 33 k positions launched 4128
+// workgroups of which 264 had work at 2 k: +1.4 us).  The next chunk's rows are in flight while the current one is worked on.
+// ---------------------------------------------------------------------------------------------
+__host__ __device__ inline int fd_long_cpw(int n_chunks) { return (n_chunks + FD_LONG_SPLITS - 1) / FD_LONG_SPLITS; }
+
+template <int HD, int G>
+__global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_long_kernel(const AttnArgs a) {
+    constexpr int HALF = HD / 2, KS = HD / 32, DT = HD / 16, LPR = HD / 8, RPL = 64 / LPR, VL = 16 / RPL, VP = HD * 2 + 64;
+    constexpr int GP = G <= 4 ? 4 : 8;
+    static_assert(G >= 1 && G <= 8 && (HD == 64 || HD == 128), "shape");
+    __shared__ __align__(16) _Float16 s_qh[G][HD];
+    __shared__ __align__(16) _Float16 s_ql[G][HD];
+    __shared__ __align__(16) _Float16 s_nk[HD];
+    __shared__ __align__(16) uint8_t s_v[4][16 * VP];
+    __shared__ __align__(16) float s_o[4][HD][GP];
+    __shared__ float s_m[4][GP], s_l[4][GP];
+
+    const int64_t past = *a.d_past;
+    if (past < 0 || past >= a.max_seq) return;          // never touch memory outside the cache
+    const int64_t total = past + 1;
+    const int split = blockIdx.x, kvh = blockIdx.y;
+    const int n_chunks = (int)((total + FD_CHUNK - 1) / FD_CHUNK);
+    const int cpw = fd_long_cpw(n_chunks);
+    const int c_first = split * cpw;
+    if (c_first >= n_chunks) return;
+    const int c_end = min(c_first + cpw, n_chunks);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t t_begin = (a.window > 0 && total > a.window) ? total - a.window : 0;
+    const int c_lo = max(c_first, (int)(t_begin / FD_CHUNK));   // chunks wholly in front of the window are skipped
+    if (c_lo >= c_end) {
+        for (int e = tid; e < G * HD; e += FD_THREADS) {
+            const int g = e / HD, d = e % HD;
+            const int64_t oi = (int64_t)split * a.n_heads + kvh * G + g;
+            a.pO[oi * HD + d] = 0.0f;
+            if (d == 0) { a.pM[oi] = -INFINITY; a.pL[oi] = 0.0f; }
+        }
+        return;
+    }
+    const int j = lane & 15, rg = lane >> 4;
+    const int kv_dim = a.n_kv_heads * HD;
+    const bool on = lane < HALF;
+    const int lh = lane & (HALF - 1);
+    const bool has_norm = a.qw != nullptr;
+    const int pc = (int)(past / FD_CHUNK);                                        // the chunk that holds the new position
+    const bool owner = pc >= c_lo && pc < c_end && (int)((past - (int64_t)pc * FD_CHUNK) / 16) == wave;  // wave-uniform
+
+    // ---- prologue loads (static count), then the first chunk's rows ----
+    const float* cs = a.rope + past * HD;
+    const float* qwp = has_norm ? a.qw : a.Q;
+    const float* kwp = has_norm ? a.kw : a.Q;
+    const int i0 = a.rope_interleaved ? 2 * lh : lh, i1 = a.rope_interleaved ? 2 * lh + 1 : lh + HALF;
+    constexpr int NQ = (G + 3) / 4;
+    float qx0[NQ], qx1[NQ];
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+        const int g = wave + 4 * n < G ? wave + 4 * n : 0;
+        const float* src = a.Q + (int64_t)(kvh * G + g) * HD;
+        qx0[n] = src[i0];
+        qx1[n] = src[i1];
+    }
+    const float qn0 = qwp[i0], qn1 = qwp[i1], kn0 = kwp[i0], kn1 = kwp[i1];
+    const float rc = cs[lh], rsn = cs[HALF + lh];
+    const float kx0 = a.K[(int64_t)kvh * HD + i0], kx1 = a.K[(int64_t)kvh * HD + i1];
+    const float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
+    issue_order_fence();
+    const int64_t last_cached = past > 0 ? past - 1 : 0;
+    const __half* Kh = static_cast<const __half*>(a.Kc) + (int64_t)kvh * HD;
+    const __half* Vh = static_cast<const __half*>(a.Vc) + (int64_t)kvh * HD;
+    auto fetch = [&](int c, uint4 (&kr)[KS], uint4 (&vr)[VL]) {   // this wave's 16 positions of chunk c; all loads unconditional
+        const int64_t wt0 = (int64_t)c * FD_CHUNK + 16 * wave;
+        const int64_t tk = wt0 + j;
+        const int64_t tkc = tk < past ? tk : last_cached;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) kr[s] = *reinterpret_cast<const uint4*>(Kh + tkc * kv_dim + 32 * s + 8 * rg);
+#pragma unroll
+        for (int vl = 0; vl < VL; ++vl) {
+            const int64_t tv = wt0 + vl * RPL + lane / LPR;
+            const int64_t tvc = tv < past ? tv : last_cached;
+            vr[vl] = *reinterpret_cast<const uint4*>(Vh + tvc * kv_dim + 8 * (lane % LPR));
+        }
+    };
+    uint4 kreg[KS], vreg[VL], knext[KS], vnext[VL];
+    fetch(c_lo, kreg, vreg);
+    issue_order_fence();
+
+    // ---- query heads (and, in the wave that owns it, the new K/V row) as in attn_decode_mfma_kernel ----
+    const float one = a.add_one ? 1.0f : 0.0f;
+    const float qs = a.scale * 1.44269504088896340736f;
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+        const int g = wave + 4 * n;
+        if (g >= G) continue;  // wave-uniform
+        float x0 = on ? qx0[n] : 0.0f, x1 = on ? qx1[n] : 0.0f;
+        if (has_norm) {
+            float ss = fmaf(x0, x0, 0.0f);
+            ss = fmaf(x1, x1, ss);
+            ss = sum64(ss);
+            const float rs = fast_rsqrt(ss * (1.0f / (float)HD) + a.eps);
+            x0 = x0 * rs * (qn0 + one);
+            x1 = x1 * rs * (qn1 + one);
+        }
+        if (on) {
+            const float r0 = fmaf(x0, rc, -(x1 * rsn)) * qs, r1 = fmaf(x0, rsn, x1 * rc) * qs;
+            const _Float16 h0 = (_Float16)r0, h1 = (_Float16)r1;
+            s_qh[g][i0] = h0;
+            s_qh[g][i1] = h1;
+            s_ql[g][i0] = (_Float16)(r0 - (float)h0);
+            s_ql[g][i1] = (_Float16)(r1 - (float)h1);
+        }
+    }
+    __half nv0 = __float2half_rn(0.0f), nv1 = nv0;
+    if (owner) {
+        float x0 = on ? kx0 : 0.0f, x1 = on ? kx1 : 0.0f;
+        if (has_norm) {
+            float ss = fmaf(x0, x0, 0.0f);
+            ss = fmaf(x1, x1, ss);
+            ss = sum64(ss);
+            const float rs = fast_rsqrt(ss * (1.0f / (float)HD) + a.eps);
+            x0 = x0 * rs * (kn0 + one);
+            x1 = x1 * rs * (kn1 + one);
+        }
+        const __half h0 = __float2half_rn(fmaf(x0, rc, -(x1 * rsn))), h1 = __float2half_rn(fmaf(x0, rsn, x1 * rc));
+        nv0 = __float2half_rn(vx0);
+        nv1 = __float2half_rn(vx1);
+        if (on) {
+            const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;
+            static_cast<__half*>(a.Kc)[rowoff + i0] = h0;
+            static_cast<__half*>(a.Kc)[rowoff + i1] = h1;
+            static_cast<__half*>(a.Vc)[rowoff + lh] = nv0;
+            static_cast<__half*>(a.Vc)[rowoff + lh + HALF] = nv1;
+            reinterpret_cast<__half*>(s_nk)[i0] = h0;
+            reinterpret_cast<__half*>(s_nk)[i1] = h1;
+        }
+    }
+    __syncthreads();
+    fd_h8 qh[KS], ql[KS];
+    {
+        const int jq = j < G ? j : 0;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            qh[s] = *reinterpret_cast<const fd_h8*>(&s_qh[jq][32 * s + 8 * rg]);
+            ql[s] = *reinterpret_cast<const fd_h8*>(&s_ql[jq][32 * s + 8 * rg]);
+        }
+    }
+
+    // ---- the chunks of this workgroup: running maximum m_run / sum l_run of head j (score layout), output acc (head rows) ----
+    float m_run = -INFINITY, l_run = 0.0f;
+    fd_f4 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = fd_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c = c_lo;; ++c) {
+        // the next chunk's rows travel while this one is worked on.  After the last chunk the loads still go out (a load under
+        // a branch would cost the compiler its count of the loads in flight) but every lane asks for the last cached row -
+        // a chunk index past the position clamps there - so they move a few bytes, and nobody waits for them
+        fetch(c + 1 < c_end ? c + 1 : pc + 1, knext, vnext);
+        issue_order_fence();
+        const int64_t tt0 = (int64_t)c * FD_CHUNK + 16 * wave;
+        const bool has_new = owner && c == pc;                     // wave-uniform: this tile holds the new position
+        const bool edge = tt0 + 16 > past || tt0 < t_begin;       // wave-uniform: some of its positions do not count
+        if (has_new && j == (int)(past - tt0)) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) kreg[s] = *reinterpret_cast<const uint4*>(&s_nk[32 * s + 8 * rg]);
+        }
+        fd_f4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const fd_h8 kf = __builtin_bit_cast(fd_h8, kreg[s]);
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qh[s], sc, 0, 0, 0);
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, ql[s], sc, 0, 0, 0);
+        }
+        if (edge) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t t = tt0 + 4 * rg + r;
+                sc[r] = (t < total && t >= t_begin) ? sc[r] : -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int vl = 0; vl < VL; ++vl) {
+            const int row = vl * RPL + lane / LPR;
+            uint4 v = vreg[vl];
+            if (edge) {
+                const int64_t t = tt0 + row;
+                if (!(t < past && t >= t_begin)) v = make_uint4(0u, 0u, 0u, 0u);
+            }
+            *reinterpret_cast<uint4*>(&s_v[wave][row * VP + 16 * (lane % LPR)]) = v;
+        }
+        if (has_new && on) {
+            __half* vrow = reinterpret_cast<__half*>(&s_v[wave][(int)(past - tt0) * VP]);
+            vrow[lh] = nv0;
+            vrow[lh + HALF] = nv1;
+        }
+        fd_h4 vb[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vb[dt] = fd_lds_read_tr16(&s_v[wave][(4 * rg + (j >> 2)) * VP + (16 * dt + 4 * (j & 3)) * 2]);
+        // online softmax: new maximum, correction of what has been summed so far
+        float m = fd_rows_max(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
+        const float m_new = fmaxf(m_run, m);
+        const float ms = m_new == -INFINITY ? 0.0f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m_run - ms);   // first chunk: 2^(-inf) = 0
+        float l = 0.0f;
+        fd_h4 ph, pl;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float p = __builtin_amdgcn_exp2f(sc[r] - ms);
+            l += p;
+            const _Float16 h = (_Float16)p;
+            ph[r] = h;
+            pl[r] = (_Float16)(p - (float)h);
+        }
+        l_run = fmaf(l_run, corr, fd_rows_sum(l));
+        m_run = m_new;
+        // the output rows of this lane are heads 4 rg + r: their corrections sit in lanes 4 rg + r of the lane's own row
+        float cr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, (lane & 48) | ((4 * rg + r) & 15), 64);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            fd_f4 cacc = {acc[dt][0] * cr[0], acc[dt][1] * cr[1], acc[dt][2] * cr[2], acc[dt][3] * cr[3]};
+            cacc = __builtin_amdgcn_mfma_f32_16x16x16f16(ph, vb[dt], cacc, 0, 0, 0);
+            cacc = __builtin_amdgcn_mfma_f32_16x16x16f16(pl, vb[dt], cacc, 0, 0, 0);
+            acc[dt] = cacc;
+        }
+        if (c + 1 >= c_end) break;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) kreg[s] = knext[s];
+#pragma unroll
+        for (int vl = 0; vl < VL; ++vl) vreg[vl] = vnext[vl];
+    }
+    if (4 * rg < G) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            *reinterpret_cast<float4*>(&s_o[wave][16 * dt + j][4 * rg]) = make_float4(acc[dt][0], acc[dt][1], acc[dt][2], acc[dt][3]);
+    }
+    if (rg == 0 && j < G) { s_m[wave][j] = m_run; s_l[wave][j] = l_run; }
+    __syncthreads();
+    for (int e = tid; e < G * HD; e += FD_THREADS) {
+        const int g = e / HD, d = e % HD;
+        const float m0 = s_m[0][g], m1 = s_m[1][g], m2 = s_m[2][g], m3 = s_m[3][g];
+        const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));  // finite: the chunks hold at least one valid position
+        const float w0 = __builtin_amdgcn_exp2f(m0 - M), w1 = __builtin_amdgcn_exp2f(m1 - M),
+                    w2 = __builtin_amdgcn_exp2f(m2 - M), w3 = __builtin_amdgcn_exp2f(m3 - M);
+        const float o = (w0 * s_o[0][d][g] + w1 * s_o[1][d][g]) + (w2 * s_o[2][d][g] + w3 * s_o[3][d][g]);
+        const int64_t oi = (int64_t)split * a.n_heads + kvh * G + g;
+        a.pO[oi * HD + d] = o;
+        if (d == 0) {
+            a.pM[oi] = M;
+            a.pL[oi] = (w0 * s_l[0][g] + w1 * s_l[1][g]) + (w2 * s_l[2][g] + w3 * s_l[3][g]);
+        }
+    }
+}
+
+template <int HD>
+static int attn_mfma_long_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
+#define PTM_AL(GG) hipLaunchKernelGGL((attn_decode_mfma_long_kernel<HD, GG>), grid, dim3(FD_THREADS), 0, s, a)
+    switch (G) {
+        case 1: PTM_AL(1); break;
+        case 2: PTM_AL(2); break;
+        case 3: PTM_AL(3); break;
+        case 4: PTM_AL(4); break;
+        case 5: PTM_AL(5); break;
+        case 6: PTM_AL(6); break;
+        case 7: PTM_AL(7); break;
+        case 8: PTM_AL(8); break;
+        default: return PTM_E_UNSUPPORTED;
+    }
+#undef PTM_AL
+    return launch_status();
+}
+
 template <int HD, int TPW>
 static int attn_mfma_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
 #define PTM_AM(GG) hipLaunchKernelGGL((attn_decode_mfma_kernel<HD, GG, TPW>), grid, dim3(FD_THREADS), 0, s, a)
@@ -1129,6 +1421,14 @@ int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, co
     if (o_q8 && (reinterpret_cast<uintptr_t>(o_q8) & 15u)) return PTM_E_ALIGN;
     if (kv_fp16) {
         // fp16 cache: the matrix-core kernel, chunks of 64 positions; partial maxima in base-2 units
+        if (ptm_flash_decode_num_splits(max_seq) > FD_LONG_SPLITS) {
+            // a cache of more than 4096 positions: the looping kernel, at most FD_LONG_SPLITS partials per head
+            const dim3 grid_long(FD_LONG_SPLITS, n_kv_heads);
+            rc = head_dim == 128 ? attn_mfma_long_launch_g<128>(G, grid_long, s, a) : attn_mfma_long_launch_g<64>(G, grid_long, s, a);
+            if (rc != PTM_OK) return rc;
+            return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
+                            static_cast<uint8_t*>(o_q8), 0, -1, 1);
+        }
         rc = head_dim == 128 ? attn_mfma_launch_g<128, 1>(G, grid, s, a) : attn_mfma_launch_g<64, 1>(G, grid, s, a);
         if (rc != PTM_OK) return rc;
         return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,

@@ -61,7 +61,10 @@ def test_gelu_mul_rms_norm_add_and_scale(dev, po):
 @pytest.mark.parametrize("kv_fp16", [True, False])
 @pytest.mark.parametrize("nh,nkv,hd,past,window", [(32, 8, 128, 2048, 1024), (4, 2, 64, 19, 8), (8, 4, 128, 130, 64),
                                                   (8, 8, 128, 5, 8), (16, 2, 64, 200, 1), (32, 8, 128, 511, 512),
-                                                  (8, 4, 256, 2048, 1024), (2, 1, 256, 19, 8), (8, 4, 256, 30, 0), (6, 2, 256, 62, 0)])
+                                                  (8, 4, 256, 2048, 1024), (2, 1, 256, 19, 8), (8, 4, 256, 30, 0), (6, 2, 256, 62, 0),
+                                                  # caches beyond 4096 positions: the looping kernel (several chunks per workgroup,
+                                                  # some or all of them in front of the window)
+                                                  (8, 2, 128, 9000, 1024), (4, 2, 64, 5000, 100), (8, 4, 128, 8200, 7000)])
 def test_attn_decode_fused_window_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past, window):
     """QK-norm + NeoX rotation + KV append + attention over the last `window` positions + merge, three tokens in a row:
     chunks wholly in front of the window are skipped, the chunk the window starts in is masked position by position."""

@@ -471,7 +471,12 @@ def test_elementwise_embedding_argmax(dev, po):
                                             (8, 8, 128, 0), (16, 2, 64, 63), (8, 1, 64, 64), (8, 8, 64, 130), (4, 2, 64, 29),
                                             (4, 2, 64, 31), (16, 2, 64, 61), (32, 8, 128, 14), (32, 8, 128, 62), (4, 4, 128, 5),
                                             (28, 4, 128, 2100), (40, 8, 128, 300), (12, 2, 128, 70), (24, 8, 64, 19),  # 7, 5, 6, 3 query heads per kv head
-                                            (32, 8, 128, 20000)])   # past the ~12 k positions where the reference's kernel stops
+                                            (32, 8, 128, 20000),    # past the ~12 k positions where the reference's kernel stops
+                                            # caches beyond 4096 positions take the looping kernel: one and several chunks per
+                                            # workgroup, a last workgroup with fewer chunks, the new position first / last in its
+                                            # chunk, other head shapes
+                                            (32, 8, 128, 4090), (8, 2, 128, 4159), (8, 2, 128, 4160), (28, 4, 128, 8191), (4, 2, 64, 8192),
+                                            (16, 2, 64, 12345), (40, 8, 128, 6000)])
 def test_attn_decode_fused_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past):
     """QK-norm + RoPE + KV append + attention + merge in one launch, three tokens in a row, against the oracle's pieces in the reference's order."""
     max_seq = ((past + 3 + 63) // 64 + 1) * 64
