@@ -30,6 +30,10 @@ PREFILL_TOL = 1e-2   # a single GEMM, max |y - y_cpu| / rms(y_cpu)
 STAGE_TOL = 5e-3     # one stage of a layer on identical inputs
 E2E_RMS_TOL = 1e-2   # whole model: rms of the logit difference / std of the oracle's logits
 E2E_MAX_TOL = 6e-2   # whole model: max of the same
+# 1100+ rows: the worst of five prompt lengths (the median is held to E2E_RMS_TOL).  Measured: four lengths at 1.5e-3 .. 2.8e-3,
+# the fifth (1100 tokens, a position where the int8 rounding noise tips a residual row) at 6.1e-2 .. 9.7e-2, against the oracle
+# as against this decoder's own token-by-token run; the bar is that plus half again
+LONG_RMS_WORST = 0.15
 
 
 def cu(a):
@@ -499,6 +503,48 @@ def test_qwen3_4b_shape_prefill_64_tokens(dev, po, seeds):
     dec.close()
 
 
+@pytest.mark.parametrize("n,chunk", [(1100, 512), (1100, 0)])
+def test_long_prompt_prefill_vs_oracle(dev, po, seeds, n, chunk):
+    """The row classes of real prompts (257..1024 rows and more than 1024; gate and up in one launch; two wave groups in the
+    attention; chunks that continue a filled cache) against the ORACLE, not only against this decoder's own stepping: three
+    full-width Qwen3-4B layers, an 1100-token prompt, the oracle fed token by token (1100 steps of 3 layers on the CPU).
+    Logits at five prompt lengths, greedy token where the margin allows, cache rows of every layer."""
+    from prometorch_amd.decode import Decoder
+    cfg = dict(synth.QWEN3_4B)
+    cfg["n_layers"] = 3
+    seed = seeds["cfg4"]
+    layers = [synth.make_layer(seed, i, cfg) for i in range(3)]
+    head = synth.make_head(seed, cfg)
+    om = po.OracleModel(cfg, layers, head, n + 16, kv_fp16=True)
+    dec = Decoder(cfg, layers, head, max_seq=n + 16, kv_fp16=True, use_graph=True)
+    prompt = [int(t) for t in synth.rng_for(70, n).integers(0, cfg["vocab"], n)]
+    ends = list(range(n - 4, n + 1))
+    want, want_tok = {}, {}
+    for i, t in enumerate(prompt):
+        tok_o = om.step(t)
+        if i + 1 in ends:
+            want[i + 1], want_tok[i + 1] = om.logits.copy(), tok_o
+    # A random-weight model amplifies the int8 rounding noise of single positions (the oracle does the same against itself
+    # under a 5e-4 input perturbation, test_q8_rounding_noise_floor_of_the_oracle), so the logits are compared at five prompt
+    # lengths: the bar of the whole-model comparison on their median, no length far off
+    rmss, errs = [], []
+    for e in ends:
+        dec.set_past_len(0)
+        tok_g = dec.prefill(prompt[:e], chunk_rows=chunk)
+        err, rms, margin = logit_errors(dec.logits(), want[e])
+        rmss.append(rms)
+        errs.append(err)
+        if margin > 2 * err:
+            assert tok_g == want_tok[e], (e, margin, err)
+    print("prefill %d tokens chunk %d vs oracle: logit rms err/std at 5 lengths %s, max %s" %
+          (n, chunk, ["%.1e" % r for r in rmss], ["%.1e" % r for r in errs]), flush=True)
+    assert np.median(rmss) <= E2E_RMS_TOL and max(rmss) <= LONG_RMS_WORST, rmss
+    for li in range(3):   # the cache as the last (full-length) prefill left it
+        check_kv_rows(dec.k_cache[li][:n].float().cpu().numpy(), om.k_cache[li][:n], li, "k")
+        check_kv_rows(dec.v_cache[li][:n].float().cpu().numpy(), om.v_cache[li][:n], li, "v")
+    dec.close()
+
+
 @pytest.mark.parametrize("n,chunk", [(1100, 0), (1100, 512), (1100, 1024), (1100, 300), (2048, 0)])
 def test_long_prompt_prefill_matches_token_by_token_decode(dev, seeds, n, chunk):
     """The row classes real prompts run in (257..1024 rows, more than 1024; gate and up in one launch; two wave groups in
@@ -532,7 +578,7 @@ def test_long_prompt_prefill_matches_token_by_token_decode(dev, seeds, n, chunk)
         if margin > 2 * err:
             assert tok_p == want_tok[e], (e, margin, err)
     print("prefill %d tokens chunk %d vs stepping: logit rms err/std at 5 lengths %s" % (n, chunk, ["%.1e" % r for r in rmss]), flush=True)
-    assert np.median(rmss) <= E2E_RMS_TOL and max(rmss) <= 0.25, rmss
+    assert np.median(rmss) <= E2E_RMS_TOL and max(rmss) <= LONG_RMS_WORST, rmss
     for li in range(3):  # the cache as the last (full-length) prefill left it
         check_kv_rows(dec.k_cache[li][:n].float().cpu().numpy(), want_k[li], li, "k")
         check_kv_rows(dec.v_cache[li][:n].float().cpu().numpy(), want_v[li], li, "v")
