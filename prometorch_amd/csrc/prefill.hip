@@ -460,11 +460,16 @@ typedef float pf_f16v __attribute__((ext_vector_type(16)));
 // online-softmax states are merged through LDS at the end, which halves the number of steps of a row block's chain and gives
 // each SIMD a second wave.  Tile indices are absolute, so with a given NG a row's arithmetic does not depend on how the prompt
 // was chunked.
+// G query heads per kv head: a row takes GP = the next power of two slots of a wave's 32 query vectors (G = 3: 4, G = 5..7: 8);
+// the slots past G repeat the last head and are not stored.  window > 0: a query at position p attends to (p - window, p]
+// only: the tile walk starts at the first tile any query of the workgroup can see, and the tiles that reach below some
+// query's window are masked like the diagonal ones.
 template <int HD, int G, int NG>
 __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float* __restrict__ Q, const __half* __restrict__ Kc,
                                                                 const __half* __restrict__ Vc, float* __restrict__ O, int rows,
-                                                                int n_heads, int n_kv_heads, int64_t pos0, float scale) {
-    constexpr int RPW = 32 / G;        // rows per wave (each with its G heads: 32 query vectors)
+                                                                int n_heads, int n_kv_heads, int64_t pos0, float scale, int window) {
+    constexpr int GP = G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8;   // head slots per row
+    constexpr int RPW = 32 / GP;       // rows per wave (each with its GP head slots: 32 query vectors)
     constexpr int BM = 4 * RPW;        // rows per workgroup
     constexpr int KS = HD / 16;        // MFMA steps over the head dimension
     constexpr int DT = HD / 32;        // 32-wide tiles of the output's head dimension
@@ -493,9 +498,12 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     const int m_base = ((int)gridDim.x - 1 - wg / (int)gridDim.y) * BM;
     const int kv_dim = n_kv_heads * HD;
 
-    const int row = m_base + wave * RPW + j / G, head = kvh * G + j % G;
+    const int slot = j % GP;
+    const bool dead = slot >= G;       // a padding slot: computed like its row's last head, never stored
+    const int row = m_base + wave * RPW + j / GP, head = kvh * G + (dead ? G - 1 : slot);
     const int row_c = row < rows ? row : rows - 1;
     const int64_t limit = pos0 + row_c;  // last position this query attends to
+    const int64_t lowest = window > 0 ? limit - window + 1 : 0;   // first one
     // scores are kept in base 2: q is scaled by scale * log2(e) before its rounding to fp16
     const float qs = scale * 1.44269504088896340736f;
     pf_h8 qf[KS];
@@ -518,6 +526,10 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     const int last_row = (m_base + BM < rows ? m_base + BM : rows) - 1;
     const int64_t t_end = pos0 + last_row;  // last position any query of this workgroup attends to
     const int ntiles = (int)(t_end / 32) + 1;
+    // with a window: the first position any query of the workgroup sees (its first row's), and the first position ALL of
+    // them see (its last row's): tiles below the former are skipped, tiles below the latter are masked
+    const int64_t t_first = window > 0 && pos0 + m_base - window + 1 > 0 ? pos0 + m_base - window + 1 : 0;
+    const int64_t t_all = window > 0 ? t_end - window + 1 : 0;
     // The group's next pair of tiles is in flight in registers (sets A and B) while the current pair is worked on: the rows
     // come from HBM or L2.  Every fetch is unconditional (tile indices past the end are clamped), so the number of loads in
     // flight at each wait is static.
@@ -604,6 +616,13 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
 #pragma unroll
                 for (int r = 0; r < 16; ++r) sc[u][r] = 8 * (r >> 2) + (r & 3) <= lim ? sc[u][r] : -INFINITY;
             }
+            if ((int64_t)tile * 32 < t_all) {   // the window's lower edge (workgroup-uniform; never taken without a window)
+                issue_order_fence();
+                const int64_t lo64 = lowest - (int64_t)tile * 32 - 4 * kh;
+                const int lo = lo64 > 64 ? 64 : (int)lo64;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sc[u][r] = 8 * (r >> 2) + (r & 3) >= lo ? sc[u][r] : -INFINITY;
+            }
         }
         // v_max3_f32 by hand: fmaxf() first quiets each MFMA result with an instruction of its own (no NaN can occur here)
         float mx = sc[0][0];
@@ -663,10 +682,11 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     // Group g takes the tile pairs (4 s + 2 g, 4 s + 2 g + 1); a tile index past the end is a tile of masked positions (its
     // fetch is clamped, its probabilities are exact zeros), so both groups run the same number of steps and meet at every
     // barrier; nothing is conditional between the steps, so the count of loads in flight at each wait stays static.
-    fetch(2 * grp, kA0, vA0, kA1, vA1);
-    fetch(2 * grp + 1, kB0, vB0, kB1, vB1);
+    const int st0 = (int)(t_first / 32) / (2 * NG);   // the step that holds the first visible tile
+    fetch(2 * NG * st0 + 2 * grp, kA0, vA0, kA1, vA1);
+    fetch(2 * NG * st0 + 2 * grp + 1, kB0, vB0, kB1, vB1);
     const int nsteps = (ntiles + 2 * NG - 1) / (2 * NG);
-    for (int st = 0; st < nsteps; ++st) do_step(2 * NG * st + 2 * grp);
+    for (int st = st0; st < nsteps; ++st) do_step(2 * NG * st + 2 * grp);
     // ---- merge the two groups' states (same lane of waves w and w + 4 = same query vector, same output elements) ----
     if constexpr (NG == 2) {
     __syncthreads();  // the merge buffer overlays the tiles: every wave has finished its last tile
@@ -682,7 +702,8 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     if (grp == 1) return;
     {
         const float m1 = s_merge[wave][16 * DT][lane], l1 = s_merge[wave][16 * DT + 1][lane];
-        const float mm = fmaxf(m_run, m1);  // finite: tile 0 belongs to group 0 and holds position 0
+        const float mm0 = fmaxf(m_run, m1);  // finite unless a window hides every tile of one group from this query
+        const float mm = mm0 == -INFINITY ? 0.0f : mm0;
         const float c0 = __builtin_amdgcn_exp2f(m_run - mm), c1 = __builtin_amdgcn_exp2f(m1 - mm);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -693,7 +714,7 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     }
     const float l = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = 1.0f / (l + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
-    if (row < rows) {
+    if (row < rows && !dead) {
         float* dst = O + ((int64_t)row * n_heads + head) * HD + 4 * kh;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -706,25 +727,32 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
 
 template <int HD>
 static int prefill_attn_mfma_launch(int G, hipStream_t s, const float* Q, const void* Kc, const void* Vc, float* O, int rows,
-                                    int n_heads, int n_kv_heads, int64_t pos0, float scale) {
-    const int bm = 128 / G;
+                                    int n_heads, int n_kv_heads, int64_t pos0, float scale, int window) {
+    const int gp = G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8;
+    const int bm = 128 / gp;
     const dim3 grid((rows + bm - 1) / bm, n_kv_heads);
     // Two groups halve the chain of a row block's tiles and cost a merge and twice the threads to start: with at most 16
     // tiles per row block (the chunk ends within the first 512 positions) one group is faster (192 / 256 / 384 rows from
     // position 0: 9.8 / 11.1 / 13.8 us against 12.5 / 12.6 / 14.9; 512 rows: 17.0 / 17.2), beyond it two are (768 rows: 21.8
     // against 22.7; 256 rows at position 1024: 27.8 against 31.4)
-    const bool one = pos0 + rows <= 512;
+    // (with a window a row block walks at most window + its own rows)
+    const int64_t span = window > 0 && window + bm < pos0 + rows ? window + bm : pos0 + rows;
+    const bool one = span <= 512;
 #define PTM_PA(GG)                                                                                                          \
     if (one)                                                                                                                \
         hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG, 1>), grid, dim3(256), 0, s, Q, static_cast<const __half*>(Kc), \
-                           static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale);                      \
+                           static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale, window);              \
     else                                                                                                                    \
         hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG, 2>), grid, dim3(512), 0, s, Q, static_cast<const __half*>(Kc), \
-                           static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale)
+                           static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale, window)
     switch (G) {
         case 1: PTM_PA(1); break;
         case 2: PTM_PA(2); break;
+        case 3: PTM_PA(3); break;
         case 4: PTM_PA(4); break;
+        case 5: PTM_PA(5); break;
+        case 6: PTM_PA(6); break;
+        case 7: PTM_PA(7); break;
         case 8: PTM_PA(8); break;
         default: return PTM_E_UNSUPPORTED;
     }
@@ -825,7 +853,6 @@ int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void
     const dim3 grid((rows + 3) / 4, n_kv_heads);
     hipStream_t s = as_stream(stream);
     if (window < 0) window = 0;
-    // the matrix-core kernel walks every tile from position 0; windowed layers take the fp32 kernel, which starts at the window
     if (head_dim == 256) {  // wide heads (gemma3): the fp32 kernel only
         return kv_fp16 ? prefill_attn_launch<true, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
                        : prefill_attn_launch<false, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
@@ -833,9 +860,9 @@ int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void
     // the MFMA kernel addresses the caches with 32-bit byte offsets (computed for up to two tiles past the last position
     // before they are clamped)
     const bool offsets_fit = (pos0 + rows + 64) * (int64_t)n_kv_heads * head_dim * 2 < ((int64_t)1 << 32);
-    if (window == 0 && kv_fp16 && offsets_fit && rows >= PTM_PREFILL_MFMA_MIN_ROWS && (G == 1 || G == 2 || G == 4 || G == 8))
-        return head_dim == 128 ? prefill_attn_mfma_launch<128>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale)
-                               : prefill_attn_mfma_launch<64>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale);
+    if (kv_fp16 && offsets_fit && rows >= PTM_PREFILL_MFMA_MIN_ROWS && G <= 8)
+        return head_dim == 128 ? prefill_attn_mfma_launch<128>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
+                               : prefill_attn_mfma_launch<64>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
     if (kv_fp16)
         return head_dim == 128 ? prefill_attn_launch<true, 128>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
                                : prefill_attn_launch<true, 64>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);

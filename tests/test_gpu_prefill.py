@@ -141,7 +141,11 @@ def test_qknorm_rope_kvwrite_rows_without_norm_weights(dev, po):
                                                  (32, 8, 128, 1000, 64), (32, 8, 128, 15000, 33), (8, 4, 256, 100, 20),
                                                  (2, 1, 256, 0, 5), (28, 4, 128, 50, 20), (40, 8, 128, 0, 17), (12, 2, 64, 7, 33),
                                                  # chunks that end beyond position 512: two wave groups per workgroup
-                                                 (8, 4, 64, 500, 70), (4, 4, 128, 480, 130), (16, 2, 128, 600, 40), (4, 4, 64, 0, 530)])
+                                                 (8, 4, 64, 500, 70), (4, 4, 128, 480, 130), (16, 2, 128, 600, 40), (4, 4, 64, 0, 530),
+                                                 # 3 / 5 / 6 / 7 query heads per kv head on the matrix cores (a row takes 4 or 8 head
+                                                 # slots, the spare ones are computed and dropped): both wave-group counts, ragged rows
+                                                 (24, 8, 64, 0, 100), (6, 2, 128, 700, 150), (20, 4, 128, 90, 257), (12, 2, 64, 520, 31),
+                                                 (28, 4, 128, 1000, 200), (14, 2, 64, 0, 16)])
 def test_prefill_attention_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, pos0, rows):
     """Row r attends to cache positions [0, pos0 + r]: later rows of the same batch must not leak in.  With an
     fp16 cache and 16 or more rows the matrix-core kernel runs (Q and the softmax weights rounded to fp16: bar
