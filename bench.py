@@ -458,7 +458,16 @@ def main():
                  "tok_s": args.gemma_steps / gdt, "ms_per_token": gdt / args.gemma_steps * 1e3,
                  "token_hbm_frac": g_bytes / (gdt / args.gemma_steps) / 1e9 / HBM_PEAK_GBS,
                  "a100_published_gemma3_4b_tok_s": 81.4}
-        log("gemma-3-4B shape: %.1f tok/s (%.3f ms/token), set up in %.1fs" % (gemma["tok_s"], gemma["ms_per_token"], t1 - t0))
+        gprompt = [int(t) for t in synth.rng_for(SEED + 2, 9).integers(0, gcfg["vocab"], 512)]
+        gdec.set_past_len(0)
+        gdec.prefill(gprompt)  # allocates the row scratch
+        t2 = time.perf_counter()
+        for _ in range(3):
+            gdec.set_past_len(0)
+            gdec.prefill(gprompt)
+        gemma["prefill_512_tokens_ms"] = (time.perf_counter() - t2) / 3 * 1e3
+        log("gemma-3-4B shape: %.1f tok/s (%.3f ms/token), 512-token prompt %.2f ms, set up in %.1fs"
+            % (gemma["tok_s"], gemma["ms_per_token"], gemma["prefill_512_tokens_ms"], t1 - t0))
         gdec.close()
         del gdec, glayers, ghead
         torch.cuda.empty_cache()

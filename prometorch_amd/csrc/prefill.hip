@@ -464,19 +464,25 @@ typedef float pf_f16v __attribute__((ext_vector_type(16)));
 // the slots past G repeat the last head and are not stored.  window > 0: a query at position p attends to (p - window, p]
 // only: the tile walk starts at the first tile any query of the workgroup can see, and the tiles that reach below some
 // query's window are masked like the diagonal ones.
-template <int HD, int G, int NG>
-__global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float* __restrict__ Q, const __half* __restrict__ Kc,
+// DS = 2 (head dimension 256, one group): waves w and w + 4 hold the same 32 query vectors and each computes all scores but
+// only one half of the output's head dimension, staging the tiles together.  A wave with the whole 256-wide output would
+// need 128 accumulator registers beside 64 of q fragments and 64 of tile pieces in flight: one wave per SIMD; with the
+// output split a SIMD holds two, and the repeated score MFMAs (half of a tile's work) cost less than the idle pipes would.
+template <int HD, int G, int NG, int DS = 1>
+__global__ __launch_bounds__(256 * NG * DS) void prefill_attn_mfma_kernel(const float* __restrict__ Q, const __half* __restrict__ Kc,
                                                                 const __half* __restrict__ Vc, float* __restrict__ O, int rows,
                                                                 int n_heads, int n_kv_heads, int64_t pos0, float scale, int window) {
     constexpr int GP = G <= 1 ? 1 : G <= 2 ? 2 : G <= 4 ? 4 : 8;   // head slots per row
     constexpr int RPW = 32 / GP;       // rows per wave (each with its GP head slots: 32 query vectors)
     constexpr int BM = 4 * RPW;        // rows per workgroup
     constexpr int KS = HD / 16;        // MFMA steps over the head dimension
-    constexpr int DT = HD / 32;        // 32-wide tiles of the output's head dimension
+    constexpr int DT = HD / 32 / DS;   // 32-wide tiles of the output's head dimension that this wave accumulates
+    static_assert(DS == 1 || (DS == 2 && NG == 1), "the output is split over the two wave sets of a single group");
     constexpr int KP = HD * 2 + 16;    // LDS pitch of a K row (bytes)
     constexpr int VP = HD * 2 + 64;    // LDS pitch of a V row: 16 of the 64 banks on: the 32 lanes served together by a transposing
                                        // read (4 rows x 2 blocks of 16 columns) cover all banks (measured: 191 ns per 64 KB against 238 with + 32)
-    constexpr int PCS = 32 * HD / 8 / 256;  // 16-byte pieces of a 32-position tile per thread (1 or 2)
+    constexpr int SN = 256 * DS;            // threads that stage a group's tiles
+    constexpr int PCS = 32 * HD / 8 / SN;   // 16-byte pieces of a 32-position tile per thread (1 or 2)
     static_assert(PCS == 1 || PCS == 2, "tile smaller than the workgroup");
     // LDS: per group two K tiles and two V tiles; the merge buffer (group 1's accumulators, running maximum and sum,
     // lane-contiguous) takes the same memory once the tiles are done, which keeps a workgroup under half the CU's LDS
@@ -489,6 +495,8 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     uint8_t* const s_vt = s_k + 2 * K_BYTES;
     const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 31, kh = lane >> 5;
+    const int dh = DS == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 8) : 0;  // which half of the output's head dimension
+    const int stid = DS == 2 ? (int)threadIdx.x : tid;                              // index among the staging threads
     // Workgroups start in the order of their linear index, and a row block's work grows with its first row: the index runs
     // over the kv heads fastest and from the last row block down, so the longest workgroups of ALL heads start first and the
     // short ones fill the tail (with the heads outermost, a late head's longest blocks would start after the early heads'
@@ -535,14 +543,14 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     // flight at each wait is static.
     uint4 kA0, kA1, vA0, vA1, kB0, kB1, vB0, vB1;  // scalars, not arrays: they must stay in registers across the loop
     kA1 = vA1 = kB1 = vB1 = make_uint4(0, 0, 0, 0);
-    // Piece i of a thread, for K and V alike: position (tid + 256 i) / (HD / 8), elements 8 ((tid + 256 i) % (HD / 8)) .. +8 (a
+    // Piece i of a thread, for K and V alike: position (stid + SN i) / (HD / 8), elements 8 ((stid + SN i) % (HD / 8)) .. +8 (a
     // wave reads whole rows).  Byte offsets into the caches fit 32 bits (checked at launch); a piece's offset for a tile is its
     // offset in tile 0 plus the tile's, clamped to the same piece of the last visible position: rows past the end are masked
     // below and nothing is read past the appended rows.
     uint32_t pc_off[PCS], pc_max[PCS], pc_lds_k[PCS], pc_lds_v[PCS];
 #pragma unroll
     for (int i = 0; i < PCS; ++i) {
-        const int q = tid + 256 * i, p = q / (HD / 8), c = q % (HD / 8);
+        const int q = stid + SN * i, p = q / (HD / 8), c = q % (HD / 8);
         const uint32_t col = (uint32_t)(kvh * HD + 8 * c);
         pc_off[i] = ((uint32_t)p * (uint32_t)kv_dim + col) * 2u;
         pc_max[i] = ((uint32_t)t_end * (uint32_t)kv_dim + col) * 2u;
@@ -665,7 +673,7 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
                 for (int dt = 0; dt < DT; ++dt) {
                     // positions 16 ks + 4 kh .. +3 and the same + 8 of V column 32 dt + j (the lane's S^T rows)
                     const uint8_t* vrow = s_vt + u * VT_BYTES + (16 * ks + 4 * kh + ((lane & 15) >> 2)) * VP +
-                                          (32 * dt + (j & 16) + 4 * (lane & 3)) * 2;
+                                          (32 * (dt + DT * dh) + (j & 16) + 4 * (lane & 3)) * 2;
                     vlo[ks][dt] = lds_read_tr16(vrow);
                     vhi[ks][dt] = lds_read_tr16(vrow + 8 * VP);
                 }
@@ -715,7 +723,7 @@ __global__ __launch_bounds__(256 * NG) void prefill_attn_mfma_kernel(const float
     const float l = l_run + __shfl_xor(l_run, 32, 64);
     const float inv = 1.0f / (l + 1e-10f);  // reference: inv_sum = 1/(sum_exp + 1e-10f), gguf_model.h:3589
     if (row < rows && !dead) {
-        float* dst = O + ((int64_t)row * n_heads + head) * HD + 4 * kh;
+        float* dst = O + ((int64_t)row * n_heads + head) * HD + 32 * DT * dh + 4 * kh;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -739,7 +747,10 @@ static int prefill_attn_mfma_launch(int G, hipStream_t s, const float* Q, const 
     const int64_t span = window > 0 && window + bm < pos0 + rows ? window + bm : pos0 + rows;
     const bool one = span <= 512;
 #define PTM_PA(GG)                                                                                                          \
-    if (one)                                                                                                                \
+    if constexpr (HD == 256)                                                                                                \
+        hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG, 1, 2>), grid, dim3(512), 0, s, Q, static_cast<const __half*>(Kc), \
+                           static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale, window);              \
+    else if (one)                                                                                                                \
         hipLaunchKernelGGL((prefill_attn_mfma_kernel<HD, GG, 1>), grid, dim3(256), 0, s, Q, static_cast<const __half*>(Kc), \
                            static_cast<const __half*>(Vc), O, rows, n_heads, n_kv_heads, pos0, scale, window);              \
     else                                                                                                                    \
@@ -853,13 +864,15 @@ int ptm_prefill_attention_window(const float* Q, const void* K_cache, const void
     const dim3 grid((rows + 3) / 4, n_kv_heads);
     hipStream_t s = as_stream(stream);
     if (window < 0) window = 0;
-    if (head_dim == 256) {  // wide heads (gemma3): the fp32 kernel only
-        return kv_fp16 ? prefill_attn_launch<true, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
-                       : prefill_attn_launch<false, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
-    }
     // the MFMA kernel addresses the caches with 32-bit byte offsets (computed for up to two tiles past the last position
     // before they are clamped)
     const bool offsets_fit = (pos0 + rows + 64) * (int64_t)n_kv_heads * head_dim * 2 < ((int64_t)1 << 32);
+    if (head_dim == 256) {  // wide heads (gemma3)
+        if (kv_fp16 && offsets_fit && rows >= PTM_PREFILL_MFMA_MIN_ROWS && G <= 8)
+            return prefill_attn_mfma_launch<256>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
+        return kv_fp16 ? prefill_attn_launch<true, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
+                       : prefill_attn_launch<false, 256>(G, grid, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);
+    }
     if (kv_fp16 && offsets_fit && rows >= PTM_PREFILL_MFMA_MIN_ROWS && G <= 8)
         return head_dim == 128 ? prefill_attn_mfma_launch<128>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window)
                                : prefill_attn_mfma_launch<64>(G, s, Q, K_cache, V_cache, O, rows, n_heads, n_kv_heads, pos0, scale, window);

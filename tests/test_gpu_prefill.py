@@ -145,7 +145,11 @@ def test_qknorm_rope_kvwrite_rows_without_norm_weights(dev, po):
                                                  # 3 / 5 / 6 / 7 query heads per kv head on the matrix cores (a row takes 4 or 8 head
                                                  # slots, the spare ones are computed and dropped): both wave-group counts, ragged rows
                                                  (24, 8, 64, 0, 100), (6, 2, 128, 700, 150), (20, 4, 128, 90, 257), (12, 2, 64, 520, 31),
-                                                 (28, 4, 128, 1000, 200), (14, 2, 64, 0, 16)])
+                                                 (28, 4, 128, 1000, 200), (14, 2, 64, 0, 16),
+                                                 # heads of 256 on the matrix cores (the output's head dimension split over two
+                                                 # sets of waves): 1 / 2 / 4 / 3 query heads per kv head, ragged rows, long walks
+                                                 (8, 4, 256, 0, 130), (4, 4, 256, 700, 67), (8, 2, 256, 33, 200), (6, 2, 256, 1200, 45),
+                                                 (16, 4, 256, 0, 512)])
 def test_prefill_attention_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, pos0, rows):
     """Row r attends to cache positions [0, pos0 + r]: later rows of the same batch must not leak in.  With an
     fp16 cache and 16 or more rows the matrix-core kernel runs (Q and the softmax weights rounded to fp16: bar
