@@ -70,7 +70,7 @@ int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const in
     Q6KArgs a6{static_cast<const uint8_t*>(W6), x, y6, K, N6, l6, stride6, nullptr, nullptr,
                gamma, eps, add_one, nullptr};
     const int n6 = (N6 + (32 >> l6) - 1) / (32 >> l6), n4w = q4k_workgroups(total, a4.log2S);
-    const size_t lds = (size_t)K * 4 + (size_t)K / 4;  // the Q6_K body's fp32 x + per-16 sums; Q4_K needs less
+    const size_t lds = q6k_x_lds_bytes(K);  // the Q6_K body's fp32 x + per-16 sums; Q4_K needs less
     static const int cand6[] = {2, 3, 5};
     const int nb6 = pick_blocks_per_pass((K / 256 + (1 << l6) - 1) >> l6, cand6, 3);
     const dim3 grid(n6 + n4w);

@@ -63,13 +63,21 @@ __device__ __forceinline__ void realign16(const uint4 w, uint32_t tail, uint32_t
     out[3] = __builtin_amdgcn_alignbyte(tail, w.w, mis);
 }
 
+// x in LDS: float4 slot i of the vector sits at slot i + i / 32 (one spare slot behind every 128 values).  A lane group
+// reads 16-byte pieces 128 values apart (the two halves of a super-block) and neighbouring groups read blocks 256
+// values apart: unpadded, the 16 lanes one ds_read_b128 pass serves would hit 4 of the 16 bank quads, four lanes each
+// (measured on the 2560 x 9728 down projection: 68 % of the LDS cycles were bank conflicts).
+__device__ __forceinline__ int q6k_xslot(int i4) { return i4 + (i4 >> 5); }
+inline __host__ __device__ int q6k_x_floats(int K) { return K + K / 32; }              // padded length of x in LDS
+inline size_t q6k_x_lds_bytes(int K) { return (size_t)q6k_x_floats(K) * 4 + (size_t)K / 4; }  // x and its per-16 sums
+
 // contribution of block b to lane j's chain
 __device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __restrict__ xf,
                                                 const float* __restrict__ xsum16, int b, int j) {
     const int half = j >> 2, jj = j & 3, which32 = jj >> 1, l16 = jj & 1;
     const int hshift = 2 * which32;
     const int xo = 128 * half + 32 * which32 + 16 * l16;  // x offset of the low-nibble 16; high-nibble +64
-    const float* xb = xf + b * 256 + xo;
+    const float* xb = xf + 4 * q6k_xslot((b * 256 + xo) >> 2);  // the 32 slots of a half block share one shift
     float s_lo = 0.0f, s_hi = 0.0f;
     uint32_t qlw[4], qhw[4];
     realign16(k.ql, k.ql_t, k.mis, qlw);
@@ -100,7 +108,7 @@ __device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __r
 template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
 __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw, int wg) {
     float* xf = reinterpret_cast<float*>(lds_raw);
-    float* xsum16 = xf + a.K;
+    float* xsum16 = xf + q6k_x_floats(a.K);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6, j = lane & 7, grp = lane >> 3;
     const int S = 1 << a.log2S;
@@ -118,7 +126,7 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
     // x (optionally RMS-normalised) goes to LDS with its per-16 sums: 4 consecutive float4 slots make one 16-group
     __shared__ float red[4];
     auto emit = [&](int i, float4 v) {
-        reinterpret_cast<float4*>(xf)[i] = v;
+        reinterpret_cast<float4*>(xf)[q6k_xslot(i)] = v;
         if constexpr (NORM) {
             if (wg == 0 && a.xn_out) reinterpret_cast<float4*>(a.xn_out)[i] = v;
         }

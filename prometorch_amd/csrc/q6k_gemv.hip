@@ -45,7 +45,7 @@ __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(
     extern __shared__ __align__(16) uint8_t lds_raw[];
     constexpr int S = 1 << LOG2S, ROWS_PER_WAVE = 8 >> LOG2S;
     float* xf = reinterpret_cast<float*>(lds_raw);
-    float* xsum16 = xf + a.K;
+    float* xsum16 = xf + q6k_x_floats(a.K);
     const int tid = threadIdx.x, nthr = blockDim.x;
     const int lane = tid & 63, wave = tid >> 6, j = lane & 7, grp = lane >> 3, sub = grp & (S - 1);
     const int r = (blockIdx.x * (nthr >> 6) + wave) * ROWS_PER_WAVE + (grp >> LOG2S);
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(
         if (i < n4) {
             const float4 v = make_float4(__uint_as_float(xv[u].x), __uint_as_float(xv[u].y), __uint_as_float(xv[u].z),
                                          __uint_as_float(xv[u].w));
-            reinterpret_cast<float4*>(xf)[i] = v;
+            reinterpret_cast<float4*>(xf)[q6k_xslot(i)] = v;
             float sm = (v.x + v.y) + (v.z + v.w);
             sm += dpp_f<0xB1>(sm);
             sm += dpp_f<0x4E>(sm);
@@ -137,7 +137,7 @@ template <bool ACC, int NB, int LOG2S>
 static int q6k_launch_tall_nb(const Q6KArgs& a, int waves, hipStream_t s) {
     const int rows_per_wg = waves * (8 >> LOG2S);
     const int grid = (a.N + rows_per_wg - 1) / rows_per_wg;
-    const size_t lds = (size_t)a.K * 4 + (size_t)a.K / 4;
+    const size_t lds = q6k_x_lds_bytes(a.K);
     const int xl = (a.K / 4 + 64 * waves - 1) / (64 * waves);
     if (xl <= 4) hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 4, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
     else hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
@@ -281,7 +281,7 @@ static int q6k_launch(Q6KArgs& a, hipStream_t s) {
     if (q6k_mfma_shape(a.N, a.K)) return q6k_launch_mfma<ACC, ARGMAX, NORM>(a, s);
     a.log2S = q6k_pick_log2S(a.N, a.K / 256);
     const int grid = q6k_workgroups(a.N, a.K);
-    const size_t lds = (size_t)a.K * 4 + (size_t)a.K / 4;
+    const size_t lds = q6k_x_lds_bytes(a.K);
     if constexpr (!ARGMAX && !NORM) {
         const Q6KTall tall = q6k_tall_shape(a.N, a.K);
         if (tall.waves > 0)
