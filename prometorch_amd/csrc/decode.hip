@@ -121,9 +121,15 @@ struct ptm_decoder {
     int* d_step = nullptr;
     int64_t* d_past = nullptr;
     int64_t* d_next = nullptr;
-    int64_t* d_tokens = nullptr;
+    int64_t* d_tokens = nullptr;  // the device's view of h_pinned: the step's last kernel stores the token id straight to the host
+    // Greedy steps resume where the device stands: when the caller feeds back the token the last greedy run produced (what a
+    // generate loop does), the device already holds it, the position and the step index, and no scalar-setting launch
+    // is needed.  out_base = index in h_pinned of the last run's first token.
+    bool dev_synced = false;
+    int64_t dev_token = -1;
+    int chain_base = 0, out_base = 0;
     bool untuned_types = false;   // some matrix is Q5_K / Q8_0 / Q5_0: no row-batched GEMM for it, prompts go token by token
-    int64_t* h_pinned = nullptr;  // [max_seq] pinned host staging for token ids
+    int64_t* h_pinned = nullptr;  // [max_seq] pinned host memory the token ids are written to by the device
     float* h_uniforms = nullptr;  // [max_seq] pinned host staging for the sampler's draws (an "async" copy from the
                                   // caller's pageable memory would be staged by the runtime synchronously)
     int64_t past_len = 0;
@@ -501,7 +507,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
                  o_hb = take(4 * (size_t)H), o_rope_swa = take(c.swa_window > 0 ? 4 * (size_t)c.max_seq * c.head_dim : 0),
                  o_xq8 = take((size_t)ptm_q8_bytes(qd > (H > c.inter ? H : c.inter) ? qd : (H > c.inter ? H : c.inter))),
                  o_ws = take((size_t)ptm_argmax_workspace_bytes(c.vocab)), o_tok = take(256), o_past = take(256),
-                 o_next = take(256), o_step = take(256), o_tokens = take(8 * (size_t)c.max_seq),
+                 o_next = take(256), o_step = take(256),
                  o_samp = take(256), o_counts = take(4 * (size_t)c.vocab), o_unif = take(4 * (size_t)c.max_seq),
                  o_sws = take((size_t)ptm_sampler_workspace_bytes());
     if ((rc = hip_status(hipMalloc(&d->slab, off))) != PTM_OK) { delete d; return rc; }
@@ -514,7 +520,6 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->hb = (float*)(base + o_hb); d->rope_swa = c.swa_window > 0 ? (float*)(base + o_rope_swa) : d->rope;
     d->amax_ws = base + o_ws; d->d_token = (int*)(base + o_tok); d->d_past = (int64_t*)(base + o_past);
     d->d_next = (int64_t*)(base + o_next); d->d_step = (int*)(base + o_step);
-    d->d_tokens = (int64_t*)(base + o_tokens);
     d->d_sampling = (ptm_sampling*)(base + o_samp); d->d_counts = (int32_t*)(base + o_counts);
     d->d_uniforms = (float*)(base + o_unif); d->sampler_ws = base + o_sws;
     if ((rc = hip_status(hipMemset(d->sampler_ws, 0, (size_t)ptm_sampler_workspace_bytes()))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
@@ -522,6 +527,9 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
 
     if ((rc = hip_status(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     if ((rc = hip_status(hipHostMalloc((void**)&d->h_pinned, 8 * (size_t)c.max_seq, hipHostMallocDefault))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
+    // token ids go from the step's last kernel straight to pinned host memory (an 8-byte store per token): no copy launch
+    // between the step and the host's read
+    if ((rc = hip_status(hipHostGetDevicePointer((void**)&d->d_tokens, d->h_pinned, 0))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     if ((rc = hip_status(hipHostMalloc((void**)&d->h_uniforms, 4 * (size_t)c.max_seq, hipHostMallocDefault))) != PTM_OK) { ptm_decode_destroy(d); return rc; }
     {
         std::vector<float> tab((size_t)c.max_seq * c.head_dim);
@@ -559,20 +567,28 @@ int ptm_decode_set_past_len(ptm_decoder* d, int64_t past_len) {
     if (!d) return PTM_E_NULL;
     if (past_len < 0 || past_len >= d->cfg.max_seq) return PTM_E_RANGE;
     d->past_len = past_len;
+    d->dev_synced = false;
     return PTM_OK;
 }
 
 // Run n chained steps starting from `token` (greedy, or sampled with the stored parameters and the uniforms already
-// on the device); token ids land in d_tokens[0..n) and h_pinned[0..n).
+// on the device); token ids land in h_pinned[out_base .. out_base + n).
 static int run_steps(ptm_decoder* d, int token, int n, bool sample = false) {
     if (d->status != PTM_OK) return PTM_E_STATE;
     if (n <= 0) return PTM_E_SHAPE;
     if (token < 0 || token >= d->cfg.vocab) return PTM_E_RANGE;
     if (d->past_len + n > d->cfg.max_seq) return PTM_E_RANGE;  // KV cache would overflow
     hipStream_t s = d->stream;
-    hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, s, d->d_token, token, d->d_past, d->past_len, d->d_step);
-    int rc = launch_status();
-    if (rc != PTM_OK) return rc;
+    int rc = PTM_OK;
+    // sampled steps index their uniform draws by the step counter: they always start from 0
+    const bool resume = !sample && d->dev_synced && (int64_t)token == d->dev_token && d->chain_base + n <= d->cfg.max_seq;
+    d->dev_synced = false;
+    if (!resume) {
+        hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, s, d->d_token, token, d->d_past, d->past_len, d->d_step);
+        if ((rc = launch_status()) != PTM_OK) return rc;
+        d->chain_base = 0;
+    }
+    d->out_base = d->chain_base;
     bool& captured = sample ? d->captured_s : d->captured;
     hipGraph_t& graph = sample ? d->graph_s : d->graph;
     hipGraphExec_t& exec = sample ? d->exec_s : d->exec;
@@ -611,9 +627,11 @@ static int run_steps(ptm_decoder* d, int token, int n, bool sample = false) {
         else rc = enqueue_step(d, sample);
         if (rc != PTM_OK) return d->status = rc;
     }
-    if ((rc = hip_status(hipMemcpyAsync(d->h_pinned, d->d_tokens, 8 * (size_t)n, hipMemcpyDeviceToHost, s))) != PTM_OK) return d->status = rc;
     if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return d->status = rc;
     d->past_len += n;
+    d->chain_base += n;
+    d->dev_token = d->h_pinned[d->out_base + n - 1];
+    d->dev_synced = !sample;
     return PTM_OK;
 }
 
@@ -662,7 +680,7 @@ int ptm_decode_sample(ptm_decoder* d, int token_id, int n, const float* uniforms
     int rc = hip_status(hipMemcpyAsync(d->d_uniforms, d->h_uniforms, 4 * (size_t)n, hipMemcpyHostToDevice, d->stream));
     if (rc != PTM_OK) return rc;
     if ((rc = run_steps(d, token_id, n, true)) != PTM_OK) return rc;
-    for (int i = 0; i < n; ++i) out_tokens[i] = d->h_pinned[i];
+    for (int i = 0; i < n; ++i) out_tokens[i] = d->h_pinned[d->out_base + i];
     return PTM_OK;
 }
 
@@ -731,9 +749,10 @@ int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_r
         // no row-batched GEMM for these types: the prompt is stepped, each step a full decode step whose token is dropped
         int rc = PTM_OK;
         for (int i = 0; i < n && rc == PTM_OK; ++i) rc = run_steps(d, tokens[i], 1);
-        if (rc == PTM_OK) *next_token = d->h_pinned[0];
+        if (rc == PTM_OK) *next_token = d->h_pinned[d->out_base];
         return rc;
     }
+    d->dev_synced = false;
     if (chunk_rows <= 0) chunk_rows = 2048;  // measured: 2048-row chunks run a 4096-token prompt 1.4x faster than 512-row ones
     if (chunk_rows > 2048) chunk_rows = 2048;  // bounds the row scratch (and the launch grids) whatever the prompt length
     if (chunk_rows > n) chunk_rows = n;
@@ -767,7 +786,6 @@ int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_r
         }
     }
     if (rc != PTM_OK) return d->status = rc;
-    if ((rc = hip_status(hipMemcpyAsync(d->h_pinned, d->d_tokens, 8, hipMemcpyDeviceToHost, s))) != PTM_OK) return d->status = rc;
     if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return d->status = rc;
     d->past_len += n;
     *next_token = d->h_pinned[0];
@@ -777,7 +795,7 @@ int ptm_decode_prefill(ptm_decoder* d, const int32_t* tokens, int n, int chunk_r
 int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token) {
     if (!d || !next_token) return PTM_E_NULL;
     const int rc = run_steps(d, token_id, 1);
-    if (rc == PTM_OK) *next_token = d->h_pinned[0];
+    if (rc == PTM_OK) *next_token = d->h_pinned[d->out_base];
     return rc;
 }
 
@@ -787,11 +805,11 @@ int ptm_decode_step_trace(ptm_decoder* d, int token_id, int64_t* next_token, flo
     if (token_id < 0 || token_id >= d->cfg.vocab) return PTM_E_RANGE;
     if (d->past_len + 1 > d->cfg.max_seq) return PTM_E_RANGE;
     hipStream_t s = d->stream;
+    d->dev_synced = false;
     hipLaunchKernelGGL(set_scalars_kernel, dim3(1), dim3(1), 0, s, d->d_token, token_id, d->d_past, d->past_len, d->d_step);
     int rc = launch_status();
     if (rc != PTM_OK) return rc;
     if ((rc = enqueue_step(d, false, trace_device)) != PTM_OK) return d->status = rc;
-    if ((rc = hip_status(hipMemcpyAsync(d->h_pinned, d->d_tokens, 8, hipMemcpyDeviceToHost, s))) != PTM_OK) return d->status = rc;
     if ((rc = hip_status(hipStreamSynchronize(s))) != PTM_OK) return d->status = rc;
     d->past_len += 1;
     *next_token = d->h_pinned[0];
@@ -801,7 +819,7 @@ int ptm_decode_step_trace(ptm_decoder* d, int token_id, int64_t* next_token, flo
 int ptm_decode_greedy(ptm_decoder* d, int first_token, int n, int64_t* tokens_out) {
     if (!d || !tokens_out) return PTM_E_NULL;
     const int rc = run_steps(d, first_token, n);
-    if (rc == PTM_OK) for (int i = 0; i < n; ++i) tokens_out[i] = d->h_pinned[i];
+    if (rc == PTM_OK) for (int i = 0; i < n; ++i) tokens_out[i] = d->h_pinned[d->out_base + i];
     return rc;
 }
 

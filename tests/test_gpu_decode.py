@@ -90,6 +90,75 @@ def test_tiny_decode_fp16_kv_vs_oracle_and_chained_greedy(dev, po, seeds, embedd
     dec2.close()
 
 
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_steps_that_resume_on_the_device_equal_steps_that_reset(dev, seeds, use_graph):
+    """A greedy step whose input is the token the previous greedy run produced starts from the device's own token, position
+    and step index (no scalar-setting launch); any other input, a chained run, a sampled run, a prompt or a position reset
+    in between must put the state back.  One decoder runs a mixed sequence of those; a second one has its position set
+    before every single step, which forces the reset path each time.  Tokens and logits must be identical."""
+    from prometorch_amd.decode import Decoder
+    cfg, layers, head, kv = build_tiny(seeds)
+    a = Decoder(cfg, layers, head, max_seq=96, kv_fp16=True, use_graph=use_graph)
+    b = Decoder(cfg, layers, head, max_seq=96, kv_fp16=True, use_graph=use_graph)
+    for i, (k, v) in enumerate(kv):
+        a.set_kv(i, k, v)
+        b.set_kv(i, k, v)
+    pos = 19
+    a.set_past_len(pos)
+
+    def b_step(tok):
+        nonlocal pos
+        b.set_past_len(pos)
+        out = b.step(tok)
+        pos += 1
+        return out
+
+    def same_logits():
+        assert np.array_equal(a.logits(), b.logits())
+
+    tok = 3
+    for _ in range(5):                       # resumed after the first
+        ta, tb = a.step(tok), b_step(tok)
+        assert ta == tb
+        same_logits()
+        tok = ta
+    forced = (tok + 7) % cfg["vocab"]        # not the token the device holds: reset
+    ta, tb = a.step(forced), b_step(forced)
+    assert ta == tb
+    same_logits()
+    tok = ta
+    chain = a.greedy(tok, 6)                 # a chained run resumes as well, and leaves the device in step with the host
+    for t in chain:
+        tok = b_step(tok)
+        assert tok == t
+    for _ in range(3):
+        ta, tb = a.step(tok), b_step(tok)
+        assert ta == tb
+        same_logits()
+        tok = ta
+    prompt = [5, 9, 2, 11, 7, 1, 30, 4, 8, 6, 12, 3, 17, 21, 2, 9, 40]   # a prompt in between: 17 rows
+    ta = a.prefill(prompt)
+    b.set_past_len(pos)
+    tb = b.prefill(prompt)
+    pos += len(prompt)
+    assert ta == tb
+    tok = ta
+    for _ in range(4):
+        ta, tb = a.step(tok), b_step(tok)
+        assert ta == tb
+        same_logits()
+        tok = ta
+    a.set_past_len(25)                       # rewind: the same token id as the device holds, but another position
+    pos = 25
+    for _ in range(3):
+        ta, tb = a.step(tok), b_step(tok)
+        assert ta == tb
+        same_logits()
+        tok = ta
+    a.close()
+    b.close()
+
+
 def test_decode_kv_overflow_and_bad_token_are_errors(dev, seeds):
     from prometorch_amd.decode import Decoder
     from prometorch_amd._lib import PtmError
