@@ -293,6 +293,11 @@ def main():
     lm = dec._cfg.lm_head.data
     ms1 = event_time_ms(lambda i: ops.q6k_gemv_argmax(lm, x, logits, H, V, stride6, idx, ws), 40, torch)
     gemv["cfg1_q6k_lm_head_argmax"] = {"bytes": b1, "us": ms1 * 1e3, "GBs": b1 / ms1 / 1e6, "frac": b1 / ms1 / 1e6 / HBM_PEAK_GBS}
+    # the GEMV launch by itself (logits only): the op above is this launch with per-workgroup argmax partials plus the
+    # one-workgroup launch that finishes the argmax
+    ms1g = event_time_ms(lambda i: ops.launch_q6k_gemv(lm, x, logits, H, V, stride6), 40, torch)
+    gemv["cfg1_q6k_lm_head_argmax"].update({"us_gemv_launch": ms1g * 1e3, "GBs_gemv_launch": b1 / ms1g / 1e6,
+                                            "frac_gemv_launch": b1 / ms1g / 1e6 / HBM_PEAK_GBS})
     # the Q4_K kernel on a launch large enough to amortise the launch floor (vocabulary-sized, 219 MB): shows what
     # the kernel sustains once the ~1.6 us launch + ramp no longer dominates, as it does for a 14 MB matrix
     Wbig = [torch.from_numpy(synth.make_q4k(synth.rng_for(SEED, 6 + i), V, H)).cuda() for i in range(3)]  # 657 MB > caches
