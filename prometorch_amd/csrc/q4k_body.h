@@ -209,7 +209,11 @@ __device__ __forceinline__ float silu_mul_ref(float g, float u) {
 // NB: super-blocks per lane group and pass; every pass issues exactly NB block loads, unconditionally (indices
 //     past the row's end are clamped, their terms dropped), so the count of loads in flight is static and a
 //     block is consumed as soon as it has arrived instead of after the whole prefetch.
-template <bool XQ8, bool NORM, bool ACC, int MODE, int NB>
+// ROLLT (very tall matrices: a workgroup walks several row tiles, each a single pass of NB blocks per lane group): the
+//     passes roll ACROSS tiles - a consumed block's registers are refilled with the same slot of the NEXT tile's row, so a
+//     wave never stands with nothing in flight between two tiles (behind the last tile the refills repeat that tile: their
+//     number stays static, the lines are in cache, nothing consumes them).
+template <bool XQ8, bool NORM, bool ACC, int MODE, int NB, bool ROLLT = false>
 __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int wg) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 7, grp = lane >> 3;
@@ -293,6 +297,53 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
     // ---- activation loads first, then the first tile's weight loads, then the activation prologue ----
     __shared__ float red[4];
     const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a, lds, red);
+    if constexpr (ROLLT) {
+        static_assert(MODE == 0, "tall single-projection launches only");
+        // one matrix (a.W[0], a.y[0]): a select over the argument struct's pointer arrays would push the struct to scratch
+        const uint8_t* const W0 = a.W[0];
+        float* const y0 = a.y[0];
+        const int64_t stride = a.stride;
+        const int total_rows = a.total_rows, log2S = a.log2S;
+        const int boff = sub * 144, bstep = 144 << log2S;
+        int tile = wg * tpw;
+        const int tile_end = min(tile + tpw, n_tiles);  // workgroup-uniform; the grid holds no workgroup without a tile
+        int r = (tile * 4 + wave) * rows_per_wave + (grp >> log2S);
+        const uint8_t* row = W0 + (int64_t)min(r, total_rows - 1) * stride;
+        uint4 hdr[NB], qv[NB];
+        issue_order_fence();
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const uint8_t* p = row + min(boff + u * bstep, (nblk - 1) * 144);
+            hdr[u] = *reinterpret_cast<const uint4*>(p);
+            qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+        }
+        issue_order_fence();
+        q4k_stage_finish<XQ8, NORM>(stg, a, lds, red);
+        for (; tile < tile_end; ++tile) {
+            const int r_next = tile + 1 < tile_end ? r + 4 * rows_per_wave : r;
+            const uint8_t* row_next = W0 + (int64_t)min(r_next, total_rows - 1) * stride;
+            float acc = 0.0f;
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                const int b = sub + (u << log2S);
+                const float t = q4k_block_term(hdr[u], qv[u], lds, a.K, min(b, nblk - 1), j);
+                acc += b < nblk ? t : 0.0f;
+                const uint8_t* p = row_next + min(boff + u * bstep, (nblk - 1) * 144);
+                hdr[u] = *reinterpret_cast<const uint4*>(p);
+                qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+            }
+            float p = sum8(acc);
+            if (S >= 2) p += dpp_f<0x128>(p);
+            if (S >= 4) p += __shfl_xor(p, 16, 64);
+            if (S >= 8) p += __shfl_xor(p, 32, 64);
+            if (r < total_rows && sub == 0 && j == 0) {
+                if constexpr (ACC) y0[r] += p;
+                else y0[r] = p;
+            }
+            r = r_next;
+        }
+        return;
+    }
     run_tile(wg * tpw, [&] { q4k_stage_finish<XQ8, NORM>(stg, a, lds, red); });
     // further tiles reuse the staged activations: the quantisation of x is paid once per workgroup
     for (int k = 1; k < tpw; ++k) {
@@ -326,6 +377,12 @@ inline int q4k_tiles_per_wg(int n_tiles) {
     int t = 1;
     while (t < 8 && (n_tiles + t - 1) / t > max_wgs) ++t;
     return t;
+}
+// The same for the kernel whose loads roll across a workgroup's tiles (q4k_gemv_tall_kernel): at most 768 workgroups, all
+// resident at once (151936 x 2560: 9496 tiles; 2048 / 1024 / 768 / 512 workgroups measured 42.2 / 41.7 / 41.5 / 41.0 us).
+inline int q4k_tiles_per_wg_rolling(int n_tiles) {
+    const int t = (n_tiles + 767) / 768;
+    return t > 16 ? 16 : t;
 }
 inline int q4k_blocks_per_pass(int nblk, int log2S) {
     static const int cand[] = {2, 3, 5, 10};

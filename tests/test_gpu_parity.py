@@ -159,9 +159,34 @@ def test_q4k_gemv_prequantized_matches_inkernel(dev, seeds):
     assert torch.equal(y1, y2)
 
 
+def test_q4k_gemv_tall_forms_agree(dev, po, seeds):
+    """The kernel for very tall Q4_K matrices (block loads rolling across a workgroup's row tiles) in its three forms - fp32
+    x, Q8 blocks handed in, accumulate - against the oracle and against each other."""
+    r = synth.rng_for(seeds["cfg1"], 7)
+    N, K = 40007, 2560
+    W = synth.make_q4k(r, N, K)
+    x = synth.make_x(r, K)
+    ref = po.gemv(12, W, x)
+    y = gpu_gemv(12, W, x)
+    assert rel_err(y, ref) <= GEMV_TOL
+    Wd, xd = cu(W), cu(x)
+    y2 = torch.empty(N, device="cuda")
+    q8 = torch.empty(ops.q8_bytes(K), dtype=torch.uint8, device="cuda")
+    ops.launch_quantize_q8(xd, q8, K)
+    ops.launch_q4km_q8_gemv(Wd, q8, y2, K, N, W.shape[1])
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y2.cpu().numpy()), bits(y))
+    y0 = synth.make_x(r, N)
+    ya = gpu_gemv(12, W, x, accumulate=True, y0=y0)
+    assert np.array_equal(bits(ya), bits(y0 + y))
+
+
 @pytest.mark.parametrize("qt,N,K", [(12, 33, 512), (12, 1, 256), (12, 77, 2560), (14, 7, 256), (14, 45, 1024),
                                     (12, 2560, 4096), (12, 2560, 9728), (14, 2560, 9728), (14, 1024, 2560),
-                                    (12, 31, 32768), (14, 5, 16384)])
+                                    (12, 31, 32768), (14, 5, 16384),
+                                    # very tall Q4_K matrices: a workgroup walks several row tiles and the block loads roll
+                                    # across them (two lane groups per row / one; 5, 2 and 3 blocks per group; ragged last tile)
+                                    (12, 40007, 2560), (12, 50001, 512), (12, 45013, 1280), (12, 41000, 768)])
 def test_gemv_shapes_vs_oracle(dev, po, qt, N, K):
     r = synth.rng_for(31, qt, N, K)
     W = synth.make_weight(r, qt, N, K)
