@@ -448,7 +448,9 @@ void ptm_decode_destroy(ptm_decoder* d);
 int ptm_decode_set_past_len(ptm_decoder* d, int64_t past_len);
 /* One greedy step: feeds token_id at position past_len, returns the argmax token through
  * *next_token (host), advances past_len.  Synchronous like forward_decode + GPU argmax
- * (gguf_model.h:3107, :4850-4859). */
+ * (gguf_model.h:3107, :4850-4859).  The token id reaches the host through pinned memory the step's last kernel
+ * writes (no copy launch); when token_id is the token the previous greedy call returned (a generate loop), the step
+ * starts from the token, position and step index the device already holds. */
 int ptm_decode_step(ptm_decoder* d, int token_id, int64_t* next_token);
 /* One greedy step run as plain launches that also copies out the residual stream after every layer's attention branch and
  * after its feed-forward branch: trace_device[n_layers][2][hidden] fp32 (device).  The hook the reference has as
