@@ -77,6 +77,7 @@ int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const in
     switch (q4k_blocks_per_pass(K / 256, a4.log2S)) {
         case 2: mixed_launch6<2>(nb6, grid, lds, s, a4, a6, n6); break;
         case 3: mixed_launch6<3>(nb6, grid, lds, s, a4, a6, n6); break;
+        case 4: mixed_launch6<4>(nb6, grid, lds, s, a4, a6, n6); break;
         case 5: mixed_launch6<5>(nb6, grid, lds, s, a4, a6, n6); break;
         default: mixed_launch6<10>(nb6, grid, lds, s, a4, a6, n6); break;
     }

@@ -385,8 +385,8 @@ inline int q4k_tiles_per_wg_rolling(int n_tiles) {
     return t > 16 ? 16 : t;
 }
 inline int q4k_blocks_per_pass(int nblk, int log2S) {
-    static const int cand[] = {2, 3, 5, 10};
-    return pick_blocks_per_pass((nblk + (1 << log2S) - 1) >> log2S, cand, 4);
+    static const int cand[] = {2, 3, 4, 5, 10};
+    return pick_blocks_per_pass((nblk + (1 << log2S) - 1) >> log2S, cand, 5);
 }
 
 }  // namespace ptm

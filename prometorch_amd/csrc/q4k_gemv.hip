@@ -62,6 +62,7 @@ static int q4k_launch(Q4KArgs& a, hipStream_t s) {
     switch (nb) {
         case 2: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 2>), grid, block, lds, s, a); break;
         case 3: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 3>), grid, block, lds, s, a); break;
+        case 4: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 4>), grid, block, lds, s, a); break;
         case 5: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 5>), grid, block, lds, s, a); break;
         default: hipLaunchKernelGGL((q4k_gemv_kernel<XQ8, NORM, ACC, MODE, 10>), grid, block, lds, s, a); break;
     }
