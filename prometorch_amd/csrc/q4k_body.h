@@ -298,17 +298,22 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
     __shared__ float red[4];
     const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a, lds, red);
     if constexpr (ROLLT) {
-        static_assert(MODE == 0, "tall single-projection launches only");
-        // one matrix (a.W[0], a.y[0]): a select over the argument struct's pointer arrays would push the struct to scratch
+        // MODE 0: one matrix (a.W[0], a.y[0]); MODE 1: virtual row 2 r = gate row r (a.W[0]), 2 r + 1 = up row r (a.W[1]).
+        // The pointers are taken out of the argument struct once: a select over its arrays per tile would push it to scratch.
         const uint8_t* const W0 = a.W[0];
+        const uint8_t* const W1 = MODE == 1 ? a.W[1] : a.W[0];
         float* const y0 = a.y[0];
-        const int64_t stride = a.stride;
+        auto row_ptr = [&](int rv) {   // virtual row (clamped) -> first byte of its weights
+            const int rc = min(rv, a.total_rows - 1);
+            if constexpr (MODE == 1) return ((rc & 1) ? W1 : W0) + (int64_t)(rc >> 1) * a.stride;
+            else return W0 + (int64_t)rc * a.stride;
+        };
         const int total_rows = a.total_rows, log2S = a.log2S;
         const int boff = sub * 144, bstep = 144 << log2S;
         int tile = wg * tpw;
         const int tile_end = min(tile + tpw, n_tiles);  // workgroup-uniform; the grid holds no workgroup without a tile
         int r = (tile * 4 + wave) * rows_per_wave + (grp >> log2S);
-        const uint8_t* row = W0 + (int64_t)min(r, total_rows - 1) * stride;
+        const uint8_t* row = row_ptr(r);
         uint4 hdr[NB], qv[NB];
         issue_order_fence();
 #pragma unroll
@@ -321,7 +326,7 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
         q4k_stage_finish<XQ8, NORM>(stg, a, lds, red);
         for (; tile < tile_end; ++tile) {
             const int r_next = tile + 1 < tile_end ? r + 4 * rows_per_wave : r;
-            const uint8_t* row_next = W0 + (int64_t)min(r_next, total_rows - 1) * stride;
+            const uint8_t* row_next = row_ptr(r_next);
             float acc = 0.0f;
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
@@ -336,9 +341,19 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
             if (S >= 2) p += dpp_f<0x128>(p);
             if (S >= 4) p += __shfl_xor(p, 16, 64);
             if (S >= 8) p += __shfl_xor(p, 32, 64);
-            if (r < total_rows && sub == 0 && j == 0) {
-                if constexpr (ACC) y0[r] += p;
-                else y0[r] = p;
+            if constexpr (MODE == 1) {
+                // gate and up of one row sit S groups apart
+                float other;
+                if (S == 1) other = dpp_f<0x128>(p);
+                else if (S == 2) other = __shfl_xor(p, 16, 64);
+                else other = __shfl_xor(p, 32, 64);
+                if (r < total_rows && (r & 1) == 0 && sub == 0 && j == 0)
+                    y0[r >> 1] = a.gelu ? gelu_mul_ref(p, other) : silu_mul_ref(p, other);
+            } else {
+                if (r < total_rows && sub == 0 && j == 0) {
+                    if constexpr (ACC) y0[r] += p;
+                    else y0[r] = p;
+                }
             }
             r = r_next;
         }

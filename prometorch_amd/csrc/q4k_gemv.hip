@@ -32,10 +32,10 @@ __global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_kernel(const Q4KArgs a) 
 }
 
 // a workgroup walks several row tiles, every tile one pass of NB blocks per lane group: the passes roll across the tiles
-template <bool XQ8, bool NORM, bool ACC, int NB>
+template <bool XQ8, bool NORM, bool ACC, int MODE, int NB>
 __global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_tall_kernel(const Q4KArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
-    q4k_gemv_body<XQ8, NORM, ACC, 0, NB, true>(a, lds, blockIdx.x);
+    q4k_gemv_body<XQ8, NORM, ACC, MODE, NB, true>(a, lds, blockIdx.x);
 }
 
 template <bool XQ8, bool NORM, bool ACC, int MODE>
@@ -46,15 +46,19 @@ static int q4k_launch(Q4KArgs& a, hipStream_t s) {
     const dim3 block(Q4K_THREADS);
     const size_t lds = (size_t)q8_bytes(a.K);
     const int nb = q4k_blocks_per_pass(a.K / 256, a.log2S);
-    if constexpr (MODE == 0) {
-        // one very tall matrix whose lane groups hold a row's blocks in a single pass: the loads roll across the tiles
+    {
+        // a very tall matrix (or gate / up pair) whose lane groups hold a row's blocks in a single pass: the loads roll
+        // across the tiles
         const int nb_max = (a.K / 256 + (1 << a.log2S) - 1) >> a.log2S;
-        if (a.n_mat == 1 && a.tiles_per_wg > 1 && nb_max <= nb && (nb == 5 || nb == 3 || nb == 2)) {
+        if ((MODE == 1 || a.n_mat == 1) && a.tiles_per_wg > 1 && nb_max <= nb && nb <= 5) {
             a.tiles_per_wg = q4k_tiles_per_wg_rolling(n_tiles);
             const dim3 grid((n_tiles + a.tiles_per_wg - 1) / a.tiles_per_wg);
-            if (nb == 5) hipLaunchKernelGGL((q4k_gemv_tall_kernel<XQ8, NORM, ACC, 5>), grid, block, lds, s, a);
-            else if (nb == 3) hipLaunchKernelGGL((q4k_gemv_tall_kernel<XQ8, NORM, ACC, 3>), grid, block, lds, s, a);
-            else hipLaunchKernelGGL((q4k_gemv_tall_kernel<XQ8, NORM, ACC, 2>), grid, block, lds, s, a);
+            switch (nb) {
+                case 2: hipLaunchKernelGGL((q4k_gemv_tall_kernel<XQ8, NORM, ACC, MODE, 2>), grid, block, lds, s, a); break;
+                case 3: hipLaunchKernelGGL((q4k_gemv_tall_kernel<XQ8, NORM, ACC, MODE, 3>), grid, block, lds, s, a); break;
+                case 4: hipLaunchKernelGGL((q4k_gemv_tall_kernel<XQ8, NORM, ACC, MODE, 4>), grid, block, lds, s, a); break;
+                default: hipLaunchKernelGGL((q4k_gemv_tall_kernel<XQ8, NORM, ACC, MODE, 5>), grid, block, lds, s, a); break;
+            }
             return launch_status();
         }
     }

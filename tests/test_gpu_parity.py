@@ -330,6 +330,31 @@ def test_fused_gemv_variants(dev, po, golden, seeds):
         assert rel_err(got.cpu().numpy(), ref) <= GEMV_TOL
 
 
+@pytest.mark.parametrize("N,K", [(14336, 4096), (11003, 2560), (30001, 1024)])
+def test_fused_gate_up_silu_tall_shapes_vs_oracle(dev, po, N, K):
+    """Gate / up pairs with more row tiles than a launch has workgroups (Llama-3-8B: 2 x 14336 x 4096): a workgroup walks
+    several tiles and the block loads roll across them; 4, 5 and 2 blocks per lane group, a ragged last tile."""
+    r = synth.rng_for(57, N, K)
+    Wg, Wu = synth.make_q4k(r, N, K), synth.make_q4k(r, N, K)
+    x = (synth.make_x(r, K) * 2.0).astype(np.float32)
+    gam = (1.0 + 0.1 * r.standard_normal(K)).astype(np.float32) * np.float32(0.05)
+    xn = po.rmsnorm(x, gam, 1e-6)
+    ref = po.silu_mul(po.gemv(12, Wg, xn), po.gemv(12, Wu, xn))
+    act = torch.empty(N, device="cuda")
+    ops.fused_rmsnorm_gate_up_silu(cu(x), cu(gam), cu(Wg), cu(Wu), act, K, N, Wg.shape[1], 1e-6, False)
+    torch.cuda.synchronize()
+    got = act.cpu().numpy()
+    assert np.all(np.isfinite(got))
+    # The launch normalises and quantises x itself: where its RMS scale differs from the oracle's in the last bit, an
+    # activation on a Q8 rounding boundary lands on the neighbouring int8 level and every output moves by up to ~1e-2 of the
+    # outputs' rms (the decode tests bound the same effect).  A wrong block, row or pairing would be an error of order 1
+    # everywhere: the bar is the usual one on the median element and the rounding-step one on the worst.
+    rms = np.sqrt((ref.astype(np.float64) ** 2).mean())
+    err = np.abs(got.astype(np.float64) - ref) / rms
+    print("gate/up", N, K, "median err %.2e max %.2e" % (np.median(err), err.max()))
+    assert np.median(err) <= GEMV_TOL and err.max() <= 2e-2
+
+
 # ---------------------------------------------------------------------------------------------
 # glue
 # ---------------------------------------------------------------------------------------------
