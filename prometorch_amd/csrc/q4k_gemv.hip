@@ -50,6 +50,8 @@ static int q4k_launch(Q4KArgs& a, hipStream_t s) {
         // a very tall matrix (or gate / up pair) whose lane groups hold a row's blocks in a single pass: the loads roll
         // across the tiles
         const int nb_max = (a.K / 256 + (1 << a.log2S) - 1) >> a.log2S;
+                // (only beyond 1280 tiles: the Qwen3-4B gate / up pair, 1216 tiles, as 608 workgroups of two rolling tiles measured
+        // 9.88 us against 9.45 with one tile per workgroup)
         if ((MODE == 1 || a.n_mat == 1) && a.tiles_per_wg > 1 && nb_max <= nb && nb <= 5) {
             a.tiles_per_wg = q4k_tiles_per_wg_rolling(n_tiles);
             const dim3 grid((n_tiles + a.tiles_per_wg - 1) / a.tiles_per_wg);
