@@ -38,6 +38,89 @@ __global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_tall_kernel(const Q4KArg
     q4k_gemv_body<XQ8, NORM, ACC, MODE, NB, true>(a, lds, blockIdx.x);
 }
 
+// Few rows, long rows (a Q4_K down projection: 2560 x 9728, as in the layers of a Q4_K_M file whose ffn_down is Q4_K): with
+// four rows per workgroup, 640 workgroups would each quantise the whole 9728-value activation vector for four rows' worth
+// of weights.  Here a workgroup is `waves` waves of one row each (the row's super-blocks strided over the wave's 8 lane
+// groups, up to three blocks of a group in flight, passes rolling), sized so that the launch is one workgroup per CU: x is quantised once per CU, a
+// half block of 16 values per thread.  Block-to-lane assignment and reduction order are those of q4k_gemv_body with 8 lane
+// groups per row, so the result is bit-identical to that kernel's.
+enum { Q4K_LONGROW_MAX_WAVES = 12 };
+template <bool ACC, int NB>
+__global__ __launch_bounds__(64 * Q4K_LONGROW_MAX_WAVES) void q4k_gemv_longrow_kernel(const uint8_t* __restrict__ W, int64_t stride,
+                                                                                   const float* __restrict__ x, float* y, int N, int K) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 7, sub = lane >> 3;
+    const int nblk = K / 256;
+    const int r = blockIdx.x * ((int)blockDim.x >> 6) + wave;
+    const bool live = r < N;
+    const uint8_t* row = W + (int64_t)(live ? r : N - 1) * stride;
+    // activation loads first (range-checked: zeros past the end), then the weights, then the Q8 arithmetic
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(x, K * 4);
+    float4 xv[4];
+    q4k_load16(rx, 16 * tid, xv);
+    issue_order_fence();
+    uint4 hdr[NB], qv[NB];
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        const uint8_t* p = row + (int64_t)min(sub + 8 * u, nblk - 1) * 144;
+        hdr[u] = *reinterpret_cast<const uint4*>(p);
+        qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+    }
+    issue_order_fence();
+    if (16 * tid < K) q4k_quantize16_store<false>(xv, xv, 1.0f, 0.0f, tid, lds, K);  // lanes t, t ^ 1 share a block: both inside or both outside
+    __syncthreads();
+    // passes roll as in q4k_gemv_body: a consumed block's registers are refilled from the next pass at once
+    const int nb_max = (nblk + 7) >> 3;
+    float acc = 0.0f;
+    int i0 = 0;
+    for (; i0 + NB < nb_max; i0 += NB) {
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int b = sub + 8 * (i0 + u);
+            const float t = q4k_block_term(hdr[u], qv[u], lds, K, min(b, nblk - 1), j);
+            acc += b < nblk ? t : 0.0f;
+            const uint8_t* p = row + (int64_t)min(sub + 8 * (i0 + NB + u), nblk - 1) * 144;
+            hdr[u] = *reinterpret_cast<const uint4*>(p);
+            qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        const int b = sub + 8 * (i0 + u);
+        const float t = q4k_block_term(hdr[u], qv[u], lds, K, min(b, nblk - 1), j);
+        acc += b < nblk ? t : 0.0f;
+    }
+    float p = sum8(acc);
+    p += dpp_f<0x128>(p);
+    p += __shfl_xor(p, 16, 64);
+    p += __shfl_xor(p, 32, 64);
+    if (live && lane == 0) {
+        if constexpr (ACC) y[r] += p;
+        else y[r] = p;
+    }
+}
+
+// waves per workgroup of that launch, or 0 when the shape is not one for it
+static int q4k_longrow_waves(int N, int K) {
+    if (K < 4096) return 0;                                        // long rows
+    const int waves = (N + 255) / 256;                            // one workgroup per CU
+    if (waves < 2 || waves > Q4K_LONGROW_MAX_WAVES) return 0;
+    if (K / 16 > 64 * waves) return 0;                            // a thread quantises one half block
+    return waves;
+}
+
+template <bool ACC>
+static int q4k_launch_longrow(const void* W, int64_t stride, const float* x, float* y, int N, int K, int waves, hipStream_t s) {
+    const dim3 grid((N + waves - 1) / waves), block(64 * waves);
+    const size_t lds = (size_t)q8_bytes(K);
+    const uint8_t* Wb = static_cast<const uint8_t*>(W);
+    // blocks in flight per lane group (2560 x 9728, five blocks per group: 1 / 2 / 3 / 5 in flight 7.52 / 6.96 / 6.85 / 6.97 us)
+    const int nb = (K / 256 + 7) / 8;
+    if (nb <= 2) hipLaunchKernelGGL((q4k_gemv_longrow_kernel<ACC, 2>), grid, block, lds, s, Wb, stride, x, y, N, K);
+    else hipLaunchKernelGGL((q4k_gemv_longrow_kernel<ACC, 3>), grid, block, lds, s, Wb, stride, x, y, N, K);
+    return launch_status();
+}
+
 template <bool XQ8, bool NORM, bool ACC, int MODE>
 static int q4k_launch(Q4KArgs& a, hipStream_t s) {
     a.log2S = q4k_pick_log2S(a.total_rows, a.K / 256, MODE == 1 ? 2 : 3);
@@ -112,6 +195,12 @@ int q4k_gemv_multi(int n_mat, const void* const* W, float* const* y, const int* 
         return accumulate ? q4k_launch<false, true, true, 0>(a, s) : q4k_launch<false, true, false, 0>(a, s);
     }
     if (x_is_q8) return accumulate ? q4k_launch<true, false, true, 0>(a, s) : q4k_launch<true, false, false, 0>(a, s);
+    if (n_mat == 1) {
+        const int waves = q4k_longrow_waves(N[0], K);
+        if (waves > 0)
+            return accumulate ? q4k_launch_longrow<true>(W[0], stride, static_cast<const float*>(x), y[0], N[0], K, waves, s)
+                              : q4k_launch_longrow<false>(W[0], stride, static_cast<const float*>(x), y[0], N[0], K, waves, s);
+    }
     return accumulate ? q4k_launch<false, false, true, 0>(a, s) : q4k_launch<false, false, false, 0>(a, s);
 }
 

@@ -181,12 +181,28 @@ def test_q4k_gemv_tall_forms_agree(dev, po, seeds):
     assert np.array_equal(bits(ya), bits(y0 + y))
 
 
+def test_q4k_gemv_long_rows_accumulate(dev, po, seeds):
+    """The few-long-rows Q4_K kernel (2560 x 9728) in its accumulating form: y0 + W.x, bit for bit the sum of y0 and the plain
+    form's result."""
+    r = synth.rng_for(seeds["cfg1"], 9)
+    W = synth.make_q4k(r, 2560, 9728)
+    x = synth.make_x(r, 9728)
+    y = gpu_gemv(12, W, x)
+    assert rel_err(y, po.gemv(12, W, x)) <= GEMV_TOL
+    y0 = synth.make_x(r, 2560)
+    ya = gpu_gemv(12, W, x, accumulate=True, y0=y0)
+    assert np.array_equal(bits(ya), bits(y0 + y))
+
+
 @pytest.mark.parametrize("qt,N,K", [(12, 33, 512), (12, 1, 256), (12, 77, 2560), (14, 7, 256), (14, 45, 1024),
                                     (12, 2560, 4096), (12, 2560, 9728), (14, 2560, 9728), (14, 1024, 2560),
                                     (12, 31, 32768), (14, 5, 16384),
                                     # very tall Q4_K matrices: a workgroup walks several row tiles and the block loads roll
                                     # across them (two lane groups per row / one; 5, 2 and 3 blocks per group; ragged last tile)
-                                    (12, 40007, 2560), (12, 50001, 512), (12, 45013, 1280), (12, 41000, 768)])
+                                    (12, 40007, 2560), (12, 50001, 512), (12, 45013, 1280), (12, 41000, 768),
+                                    # few long Q4_K rows (a Q4_K down projection): one row per wave, x quantised once per
+                                    # workgroup; ragged last workgroup, 2 / 5 blocks per lane group, 8 to 12 waves
+                                    (12, 2001, 9728), (12, 3000, 10240), (12, 2560, 6144)])
 def test_gemv_shapes_vs_oracle(dev, po, qt, N, K):
     r = synth.rng_for(31, qt, N, K)
     W = synth.make_weight(r, qt, N, K)
