@@ -39,7 +39,7 @@ __global__ __launch_bounds__(Q6K_THREADS) __attribute__((amdgpu_waves_per_eu(3, 
 // exceed the weights'.  Here a workgroup is `waves` waves of 8 >> LOG2S rows each (a row's super-blocks strided over
 // 1 << LOG2S lane groups), sized so that the launch is one workgroup per CU: x is staged once per CU.
 // XL = float4 loads of x per thread.
-enum { Q6K_TALL_MAX_WAVES = 12 };
+enum { Q6K_TALL_MAX_WAVES = 16 };
 template <bool ACC, int NB, int XL, int LOG2S>
 __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(const Q6KArgs a) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
@@ -114,12 +114,13 @@ __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(
 }
 
 // Shape of a tall launch: waves per workgroup and lane groups per row, or waves = 0 when the shape is not one for
-// it.  Rows that fill the chip once at one workgroup per CU: 8 lane groups per row while that needs at most 12 waves
-// (2560 x 9728: 10 waves), else 4 groups per row and two rows per wave
+// it.  Rows that fill the chip once at one workgroup per CU: 8 lane groups per row while that needs at most 16 waves
+// (2560 x 9728: 10 waves; 3584 x 18944, the down projection of a 7B model: 14 waves - on the four-row kernel, where 896
+// workgroups each staged 76 KB of x, that launch took 33 us), else 4 groups per row and two rows per wave
 // (4096 x 14336: 8 waves of 2 rows).
 struct Q6KTall { int waves, log2S; };
 inline Q6KTall q6k_tall_shape(int N, int K) {
-    if (K < 4096 || K > 14336) return {0, 0};
+    if (K < 4096 || K > 32768) return {0, 0};   // x and its sums in LDS: 4.4 bytes per value, at most 141 KB
     if (q6k_pick_log2S(N, K / 256) != 3) return {0, 0};   // only where the row tiles would be 4 rows anyway
     const int rows_per_wg = (N + 255) / 256;
     for (int l = 3; l >= 2; --l) {
@@ -133,11 +134,13 @@ inline Q6KTall q6k_tall_shape(int N, int K) {
     return {0, 0};
 }
 
+void q6k_init_attributes();
 template <bool ACC, int NB, int LOG2S>
 static int q6k_launch_tall_nb(const Q6KArgs& a, int waves, hipStream_t s) {
     const int rows_per_wg = waves * (8 >> LOG2S);
     const int grid = (a.N + rows_per_wg - 1) / rows_per_wg;
     const size_t lds = q6k_x_lds_bytes(a.K);
+    if (lds > 64 * 1024) q6k_init_attributes();
     const int xl = (a.K / 4 + 64 * waves - 1) / (64 * waves);
     if (xl <= 4) hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 4, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
     else hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
@@ -221,6 +224,14 @@ static void q6k_raise_lds_cap() {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_kernel<ACC, ARGMAX, NORM, XCH, NB>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
 }
+template <bool ACC, int LOG2S>
+static void q6k_raise_lds_cap_tall() {
+    const int cap = 144 * 1024;
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 1, 4, LOG2S>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 1, 8, LOG2S>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 2, 4, LOG2S>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 2, 8, LOG2S>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+}
 template <bool ACC, bool ARGMAX, bool NORM, int XCH>
 static void q6k_raise_lds_cap_nb() {
     q6k_raise_lds_cap<ACC, ARGMAX, NORM, XCH, 2>();
@@ -239,6 +250,10 @@ void q6k_init_attributes() {
     q6k_raise_lds_cap_nb<false, true, false, 1>();
     q6k_raise_lds_cap_nb<false, true, true, 1>();
     q6k_raise_lds_cap_nb<false, false, true, 1>();
+    q6k_raise_lds_cap_tall<false, 2>();
+    q6k_raise_lds_cap_tall<false, 3>();
+    q6k_raise_lds_cap_tall<true, 2>();
+    q6k_raise_lds_cap_tall<true, 3>();
     });
 }
 
