@@ -40,8 +40,12 @@ __global__ __launch_bounds__(Q6K_THREADS) __attribute__((amdgpu_waves_per_eu(3, 
 // 1 << LOG2S lane groups), sized so that the launch is one workgroup per CU: x is staged once per CU.
 // XL = float4 loads of x per thread.
 enum { Q6K_TALL_MAX_WAVES = 16 };
-template <bool ACC, int NB, int XL, int LOG2S>
-__global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(const Q6KArgs a) {
+// XMORE: rows of more than XL float4 per thread are staged in further rounds of loads (its own instantiation: the loop's
+// wait for everything in flight would cost the ordinary shapes 7 % on 4096 x 14336).
+// MAXW: the most waves a launch of the instantiation has (12, or 16 for the widest matrices: with the bound at 16 the 4096 x
+// 14336 launch, 8 waves, measured 14.7 us against 13.8).
+template <bool ACC, int NB, int XL, int LOG2S, bool XMORE = false, int MAXW = 12>
+__global__ __launch_bounds__(64 * MAXW) void q6k_gemv_tall_kernel(const Q6KArgs a) {
     extern __shared__ __align__(16) uint8_t lds_raw[];
     constexpr int S = 1 << LOG2S, ROWS_PER_WAVE = 8 >> LOG2S;
     float* xf = reinterpret_cast<float*>(lds_raw);
@@ -80,6 +84,27 @@ __global__ __launch_bounds__(64 * Q6K_TALL_MAX_WAVES) void q6k_gemv_tall_kernel(
             sm += dpp_f<0xB1>(sm);
             sm += dpp_f<0x4E>(sm);
             if ((tid & 3) == 0) xsum16[i >> 2] = sm;
+        }
+    }
+    // rows beyond XL float4 per thread (more than 16 K values with 8 waves): the rest in further rounds, fetched behind the
+    // weights (a loop with loads: the compiler waits for everything in flight there, which these rare shapes can afford)
+    if constexpr (XMORE)
+    for (int base = XL * nthr; base < n4; base += XL * nthr) {
+        u32x4 xw[XL];
+#pragma unroll
+        for (int u = 0; u < XL; ++u) xw[u] = __builtin_amdgcn_raw_buffer_load_b128(x4, (base + tid + nthr * u) * 16, 0, 0);
+#pragma unroll
+        for (int u = 0; u < XL; ++u) {
+            const int i = base + tid + nthr * u;
+            if (i < n4) {
+                const float4 v = make_float4(__uint_as_float(xw[u].x), __uint_as_float(xw[u].y), __uint_as_float(xw[u].z),
+                                             __uint_as_float(xw[u].w));
+                reinterpret_cast<float4*>(xf)[q6k_xslot(i)] = v;
+                float sm = (v.x + v.y) + (v.z + v.w);
+                sm += dpp_f<0xB1>(sm);
+                sm += dpp_f<0x4E>(sm);
+                if ((tid & 3) == 0) xsum16[i >> 2] = sm;
+            }
         }
     }
     __syncthreads();
@@ -123,13 +148,16 @@ inline Q6KTall q6k_tall_shape(int N, int K) {
     if (K < 4096 || K > 32768) return {0, 0};   // x and its sums in LDS: 4.4 bytes per value, at most 141 KB
     if (q6k_pick_log2S(N, K / 256) != 3) return {0, 0};   // only where the row tiles would be 4 rows anyway
     const int rows_per_wg = (N + 255) / 256;
-    for (int l = 3; l >= 2; --l) {
-        const int rpw = 8 >> l;
-        int waves = (rows_per_wg + rpw - 1) / rpw;
-        if (waves < 2) waves = 2;
-        if (waves > Q6K_TALL_MAX_WAVES) continue;
-        if (K / 4 > 8 * 64 * waves) continue;            // x in at most 8 loads per thread
-        return {waves, l};
+    // up to 12 waves first (4096 x 14336 as 8 waves of two rows: 13.8 us; as 16 waves of one row: 15 us), then up to 16
+    for (const int max_waves : {12, (int)Q6K_TALL_MAX_WAVES}) {
+        for (int l = 3; l >= 2; --l) {
+            const int rpw = 8 >> l;
+            int waves = (rows_per_wg + rpw - 1) / rpw;
+            if (waves < 2) waves = 2;
+            if (waves > max_waves) continue;
+            if (K / 4 > 16 * 64 * waves) continue;       // x in at most two rounds of 8 loads per thread
+            return {waves, l};
+        }
     }
     return {0, 0};
 }
@@ -141,9 +169,13 @@ static int q6k_launch_tall_nb(const Q6KArgs& a, int waves, hipStream_t s) {
     const int grid = (a.N + rows_per_wg - 1) / rows_per_wg;
     const size_t lds = q6k_x_lds_bytes(a.K);
     if (lds > 64 * 1024) q6k_init_attributes();
-    const int xl = (a.K / 4 + 64 * waves - 1) / (64 * waves);
-    if (xl <= 4) hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 4, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
-    else hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
+    const int xl = (a.K / 4 + 64 * waves - 1) / (64 * waves);   // beyond 8: a second round of 8
+    if (waves > 12) {
+        if (xl <= 8) hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8, LOG2S, false, 16>), dim3(grid), dim3(64 * waves), lds, s, a);
+        else hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8, LOG2S, true, 16>), dim3(grid), dim3(64 * waves), lds, s, a);
+    } else if (xl <= 4) hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 4, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
+    else if (xl <= 8) hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8, LOG2S>), dim3(grid), dim3(64 * waves), lds, s, a);
+    else hipLaunchKernelGGL((q6k_gemv_tall_kernel<ACC, NB, 8, LOG2S, true>), dim3(grid), dim3(64 * waves), lds, s, a);
     return launch_status();
 }
 template <bool ACC, int LOG2S>
@@ -231,6 +263,12 @@ static void q6k_raise_lds_cap_tall() {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 1, 8, LOG2S>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 2, 4, LOG2S>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 2, 8, LOG2S>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 1, 8, LOG2S, true>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 2, 8, LOG2S, true>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 1, 8, LOG2S, false, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 2, 8, LOG2S, false, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 1, 8, LOG2S, true, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&q6k_gemv_tall_kernel<ACC, 2, 8, LOG2S, true, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
 }
 template <bool ACC, bool ARGMAX, bool NORM, int XCH>
 static void q6k_raise_lds_cap_nb() {

@@ -596,7 +596,9 @@ def test_attn_decode_fused_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past):
 @pytest.mark.parametrize("N,K,accumulate", [(2500, 9728, True), (300, 4096, False), (77, 14336, True), (3000, 6912, False),
                                             (4096, 14336, True), (3300, 8192, False), (5119, 13824, False),  # two rows per wave
                                             # rows beyond 14336 values (more than 64 KB of LDS), 13 to 16 waves per workgroup
-                                            (3584, 18944, True), (3200, 16384, False), (4001, 20480, False), (5120, 17408, True)])
+                                            (3584, 18944, True), (3200, 16384, False), (4001, 20480, False), (5120, 17408, True),
+                                            # x in two rounds of loads per thread
+                                            (5120, 25600, True), (2100, 27648, False)])
 def test_q6k_long_rows_few_rows_vs_oracle(dev, po, N, K, accumulate):
     """Shapes served by the one-row-per-wave kernel (whole x staged once per workgroup): ragged row counts, both
     store modes, and a row stride wider than the row."""
