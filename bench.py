@@ -149,6 +149,7 @@ def main():
     ap.add_argument("--mix-steps", type=int, default=64, help="decode steps of the alternating Q4_K / Q6_K type mix (0 = skip)")
     ap.add_argument("--gemma-steps", type=int, default=64,
                     help="decode steps of the Gemma-3-4B-shaped extra (0: skip it)")
+    ap.add_argument("--qwen25-steps", type=int, default=64, help="decode steps of the Qwen2.5-7B-shaped model (0 = skip)")
     ap.add_argument("--llama-steps", type=int, default=64,
                     help="decode steps of the Llama-3-8B-shaped extra measurement (0 = skip)")
     ap.add_argument("--layers", type=int, default=36, help=argparse.SUPPRESS)  # debugging only; 36 is the workload
@@ -436,6 +437,40 @@ def main():
         del ldec, llayers, lhead
         torch.cuda.empty_cache()
 
+    # ---- the 7B size: Qwen2.5-7B-shaped Q4_K_M (7 query heads per kv head, q / k / v biases, no QK-norm; rows of 14 and 74
+    # super-blocks: the down projection 3584 x 18944 is the widest few-long-rows launch of the families here) -----------------
+    q25 = None
+    if args.qwen25_steps > 0:
+        t0 = time.perf_counter()
+        qcfg = dict(synth.QWEN25_7B)
+        _, qlayers, qhead = synth.qwen25_7b_like(SEED + 3, n_layers=qcfg["n_layers"], vocab=qcfg["vocab"])
+        qdec = Decoder(qcfg, qlayers, qhead, max_seq=MAX_SEQ, kv_fp16=True, use_graph=True)
+        for i in range(qcfg["n_layers"]):
+            qdec.set_kv(i, *synth.make_kv_prefill(SEED + 3, i, qcfg, N_PREFILL))
+        qdec.set_past_len(N_PREFILL)
+        qtok = 1
+        for _ in range(args.warmup):
+            qtok = qdec.step(qtok)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.qwen25_steps):
+            qtok = qdec.step(qtok)
+        torch.cuda.synchronize()
+        qdt = time.perf_counter() - t1
+        qH, qI, qV = qcfg["hidden"], qcfg["inter"], qcfg["vocab"]
+        qqd, qkvd = qcfg["n_heads"] * qcfg["head_dim"], qcfg["n_kv_heads"] * qcfg["head_dim"]
+        q_layer = (qqd * qH + qkvd * qH + qH * qqd + 2 * qI * qH) // 256 * 144 + (qkvd * qH + qH * qI) // 256 * 210
+        q_bytes = qcfg["n_layers"] * (q_layer + 2 * (N_PREFILL + args.warmup + args.qwen25_steps / 2) * qkvd * 2) + qV * (qH // 256 * 210)
+        q25 = {"workload": "batch-1 greedy decode, Qwen2.5-7B-shaped Q4_K_M (%d layers, %d hidden, %d x 128 heads on %d kv heads, "
+                           "%d intermediate, %d vocabulary, q / k / v biases), fp16 KV prefilled %d, %d new tokens, host-synchronous"
+                           % (qcfg["n_layers"], qH, qcfg["n_heads"], qcfg["n_kv_heads"], qI, qV, N_PREFILL, args.qwen25_steps),
+               "tok_s": args.qwen25_steps / qdt, "ms_per_token": qdt / args.qwen25_steps * 1e3,
+               "token_hbm_frac": q_bytes / (qdt / args.qwen25_steps) / 1e9 / HBM_PEAK_GBS}
+        log("qwen2.5-7B shape: %.1f tok/s (%.3f ms/token), set up in %.1fs" % (q25["tok_s"], q25["ms_per_token"], t1 - t0))
+        qdec.close()
+        del qdec, qlayers, qhead
+        torch.cuda.empty_cache()
+
     # ---- a third family: Gemma-3-4B-shaped Q4_K_M (256-wide heads, post-norms, GELU gate, sliding-window layers) ----
     gemma = None
     if args.gemma_steps > 0:
@@ -585,6 +620,7 @@ def main():
         "sampled_tok_s": sampled_tok_s, "sampled_chained_tok_s": sampled_chained_tok_s,
         "llama3_8b_shape": llama,
         "gemma3_4b_shape": gemma,
+        "qwen25_7b_shape": q25,
         "q4km_file_type_mix": mix,
         "long_context": longctx,
         "a100_published_tok_s": 82.6, "x_a100_published": tok_s / 82.6,
