@@ -18,12 +18,14 @@
 #include <vector>
 
 // flash_decode.hip: ptm_attn_decode_fused that also leaves the output as Q8 activation blocks (not part of the C ABI)
-extern "C" int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, const float* q_norm_w,
-                                         const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8,
-                                         float* partial_O, float* partial_lse, float* partial_max, const float* rope_table,
-                                         int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
-                                         float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
-                                         ptm_stream_t stream);
+extern "C" int ptm_attn_decode_fused_bias(const float* Q, const float* K, const float* V, const float* q_bias,
+                                          const float* k_bias, const float* v_bias, const float* q_norm_w,
+                                          const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8,
+                                          float* partial_O, float* partial_lse, float* partial_max, const float* rope_table,
+                                          int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                                          float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
+                                          ptm_stream_t stream);
+extern "C" int ptm_attn_decode_folds_bias(int head_dim, int kv_fp16);
 extern "C" int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, const float* q_norm_w,
                                         const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8,
                                         float* partial_O, float* partial_lse, float* partial_max, const float* rope_table,
@@ -222,15 +224,19 @@ static int enqueue_step(ptm_decoder* d, bool sample = false, float* trace = null
                 if (n4 > 0) PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->x, false, L.attn_norm, c.rms_eps, 0, H, s4, false, s));
             }
         }
-        if (L.q_bias) PTM_TRY(ptm_add_qkv_bias(d->q, d->k, d->v, L.q_bias, L.k_bias, L.v_bias, 1, c.n_heads * hd, c.n_kv_heads * hd, s));
+        // projection biases (qwen2): added by the attention launch where it can, else by a launch of their own
+        const bool fold_bias = L.q_bias && ptm_attn_decode_folds_bias(hd, c.kv_fp16);
+        if (L.q_bias && !fold_bias)
+            PTM_TRY(ptm_add_qkv_bias(d->q, d->k, d->v, L.q_bias, L.k_bias, L.v_bias, 1, c.n_heads * hd, c.n_kv_heads * hd, s));
         // QK-norm + RoPE + K/V append + split-KV attention in one launch, plus the small merge launch
         // a Q4_K output projection takes the attention output as the Q8 blocks the merge kernel leaves beside the fp32
         // vector: its prologue then copies 1.25 bytes per value instead of fetching and quantising 4
         const bool o_q8 = L.o.ggml_type == PTM_TYPE_Q4_K;
-        PTM_TRY(ptm_attn_decode_fused_win(d->q, d->k, d->v, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn,
-                                          o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM, local ? d->rope_swa : d->rope,
-                                          c.n_heads, c.n_kv_heads, hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd),
-                                          c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, local ? c.swa_window : 0, s));
+        PTM_TRY(ptm_attn_decode_fused_bias(d->q, d->k, d->v, fold_bias ? L.q_bias : nullptr, fold_bias ? L.k_bias : nullptr,
+                                           fold_bias ? L.v_bias : nullptr, L.q_norm, L.k_norm, L.k_cache, L.v_cache, d->attn,
+                                           o_q8 ? d->xq8 : nullptr, d->pO, d->pL, d->pM, local ? d->rope_swa : d->rope,
+                                           c.n_heads, c.n_kv_heads, hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd),
+                                           c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, local ? c.swa_window : 0, s));
         // x += Wo . attn, or with a post-norm: h = Wo . attn, x += RMSNorm(h) * w
         float* o_dst = L.post_attn_norm ? d->hb : d->x;
         const bool o_acc = !L.post_attn_norm;

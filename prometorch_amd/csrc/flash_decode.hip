@@ -422,6 +422,9 @@ struct AttnArgs {
     float scale, eps;
     int rope_interleaved;  // 0: NeoX pairs (d, d + HD/2); 1: pairs (2d, 2d + 1) as llama / mistral rotate (hot_loops.cpp:1962-2030)
     int window;            // > 0: only the last `window` positions are attended to (gemma3 local layers, gguf_model.h:3490-3500)
+    // biases of the q / k / v projections (qwen2, gguf_model.h:3419-3431), added to the raw vectors before norm and rotation
+    // by the kernels instantiated with BIAS; null otherwise
+    const float *qb, *kb, *vb;
 };
 
 // one wave: RMSNorm (optional) + NeoX rotation of a head held as pairs (t, t+HD/2); results to dst[HD]
@@ -727,7 +730,7 @@ __device__ __forceinline__ float fd_rows_sum(float v) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-template <int HD, int G, int TPW>
+template <int HD, int G, int TPW, bool BIAS = false>
 __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const AttnArgs a) {
     constexpr int HALF = HD / 2;
     constexpr int KS = HD / 32;          // QK steps (32 head-dim elements each)
@@ -778,18 +781,29 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     const float* kwp = has_norm ? a.kw : a.Q;
     const int i0 = a.rope_interleaved ? 2 * lh : lh, i1 = a.rope_interleaved ? 2 * lh + 1 : lh + HALF;
     constexpr int NQ = (G + 3) / 4;  // query heads a wave prepares: wave, wave + 4
-    float qx0[NQ], qx1[NQ];
+    float qx0[NQ], qx1[NQ], qb0[NQ], qb1[NQ];
 #pragma unroll
     for (int n = 0; n < NQ; ++n) {
         const int g = wave + 4 * n < G ? wave + 4 * n : 0;
         const float* src = a.Q + (int64_t)(kvh * G + g) * HD;
         qx0[n] = src[i0];
         qx1[n] = src[i1];
+        if constexpr (BIAS) {
+            qb0[n] = a.qb[(kvh * G + g) * HD + i0];
+            qb1[n] = a.qb[(kvh * G + g) * HD + i1];
+        }
     }
     const float qn0 = qwp[i0], qn1 = qwp[i1], kn0 = kwp[i0], kn1 = kwp[i1];
     const float rc = cs[lh], rsn = cs[HALF + lh];
-    const float kx0 = a.K[(int64_t)kvh * HD + i0], kx1 = a.K[(int64_t)kvh * HD + i1];
-    const float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
+    float kx0 = a.K[(int64_t)kvh * HD + i0], kx1 = a.K[(int64_t)kvh * HD + i1];
+    float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
+    float kb0 = 0.0f, kb1 = 0.0f, vb0 = 0.0f, vb1 = 0.0f;
+    if constexpr (BIAS) {
+        kb0 = a.kb[kvh * HD + i0];
+        kb1 = a.kb[kvh * HD + i1];
+        vb0 = a.vb[kvh * HD + lh];
+        vb1 = a.vb[kvh * HD + lh + HALF];
+    }
     issue_order_fence();
     // ---- ... then the cached K/V rows of this wave's tiles (the new position is not cached: clamp below it) ----
     uint4 kreg[TPW][KS], vreg[TPW][VL];
@@ -821,6 +835,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     for (int n = 0; n < NQ; ++n) {
         const int g = wave + 4 * n;
         if (g >= G) continue;  // wave-uniform
+        if constexpr (BIAS) { qx0[n] += qb0[n]; qx1[n] += qb1[n]; }
         float x0 = on ? qx0[n] : 0.0f, x1 = on ? qx1[n] : 0.0f;
         if (has_norm) {
             float ss = fmaf(x0, x0, 0.0f);
@@ -841,6 +856,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     }
     __half nv0 = __float2half_rn(0.0f), nv1 = nv0;
     if (owner) {  // the new K row: normalised, rotated, rounded as the cache holds it; the new V row
+        if constexpr (BIAS) { kx0 += kb0; kx1 += kb1; vx0 += vb0; vx1 += vb1; }
         float x0 = on ? kx0 : 0.0f, x1 = on ? kx1 : 0.0f;
         if (has_norm) {
             float ss = fmaf(x0, x0, 0.0f);
@@ -1001,7 +1017,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
 // ---------------------------------------------------------------------------------------------
 __host__ __device__ inline int fd_long_cpw(int n_chunks) { return (n_chunks + FD_LONG_SPLITS - 1) / FD_LONG_SPLITS; }
 
-template <int HD, int G>
+template <int HD, int G, bool BIAS = false>
 __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_long_kernel(const AttnArgs a) {
     constexpr int HALF = HD / 2, KS = HD / 32, DT = HD / 16, LPR = HD / 8, RPL = 64 / LPR, VL = 16 / RPL, VP = HD * 2 + 64;
     constexpr int GP = G <= 4 ? 4 : 8;
@@ -1048,18 +1064,29 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_long_kernel(const
     const float* kwp = has_norm ? a.kw : a.Q;
     const int i0 = a.rope_interleaved ? 2 * lh : lh, i1 = a.rope_interleaved ? 2 * lh + 1 : lh + HALF;
     constexpr int NQ = (G + 3) / 4;
-    float qx0[NQ], qx1[NQ];
+    float qx0[NQ], qx1[NQ], qb0[NQ], qb1[NQ];
 #pragma unroll
     for (int n = 0; n < NQ; ++n) {
         const int g = wave + 4 * n < G ? wave + 4 * n : 0;
         const float* src = a.Q + (int64_t)(kvh * G + g) * HD;
         qx0[n] = src[i0];
         qx1[n] = src[i1];
+        if constexpr (BIAS) {
+            qb0[n] = a.qb[(kvh * G + g) * HD + i0];
+            qb1[n] = a.qb[(kvh * G + g) * HD + i1];
+        }
     }
     const float qn0 = qwp[i0], qn1 = qwp[i1], kn0 = kwp[i0], kn1 = kwp[i1];
     const float rc = cs[lh], rsn = cs[HALF + lh];
-    const float kx0 = a.K[(int64_t)kvh * HD + i0], kx1 = a.K[(int64_t)kvh * HD + i1];
-    const float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
+    float kx0 = a.K[(int64_t)kvh * HD + i0], kx1 = a.K[(int64_t)kvh * HD + i1];
+    float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
+    float kb0 = 0.0f, kb1 = 0.0f, vb0 = 0.0f, vb1 = 0.0f;
+    if constexpr (BIAS) {
+        kb0 = a.kb[kvh * HD + i0];
+        kb1 = a.kb[kvh * HD + i1];
+        vb0 = a.vb[kvh * HD + lh];
+        vb1 = a.vb[kvh * HD + lh + HALF];
+    }
     issue_order_fence();
     const int64_t last_cached = past > 0 ? past - 1 : 0;
     const __half* Kh = static_cast<const __half*>(a.Kc) + (int64_t)kvh * HD;
@@ -1088,6 +1115,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_long_kernel(const
     for (int n = 0; n < NQ; ++n) {
         const int g = wave + 4 * n;
         if (g >= G) continue;  // wave-uniform
+        if constexpr (BIAS) { qx0[n] += qb0[n]; qx1[n] += qb1[n]; }
         float x0 = on ? qx0[n] : 0.0f, x1 = on ? qx1[n] : 0.0f;
         if (has_norm) {
             float ss = fmaf(x0, x0, 0.0f);
@@ -1108,6 +1136,7 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_long_kernel(const
     }
     __half nv0 = __float2half_rn(0.0f), nv1 = nv0;
     if (owner) {
+        if constexpr (BIAS) { kx0 += kb0; kx1 += kb1; vx0 += vb0; vx1 += vb1; }
         float x0 = on ? kx0 : 0.0f, x1 = on ? kx1 : 0.0f;
         if (has_norm) {
             float ss = fmaf(x0, x0, 0.0f);
@@ -1248,9 +1277,9 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_long_kernel(const
     }
 }
 
-template <int HD>
+template <int HD, bool BIAS>
 static int attn_mfma_long_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
-#define PTM_AL(GG) hipLaunchKernelGGL((attn_decode_mfma_long_kernel<HD, GG>), grid, dim3(FD_THREADS), 0, s, a)
+#define PTM_AL(GG) hipLaunchKernelGGL((attn_decode_mfma_long_kernel<HD, GG, BIAS>), grid, dim3(FD_THREADS), 0, s, a)
     switch (G) {
         case 1: PTM_AL(1); break;
         case 2: PTM_AL(2); break;
@@ -1266,9 +1295,9 @@ static int attn_mfma_long_launch_g(int G, dim3 grid, hipStream_t s, const AttnAr
     return launch_status();
 }
 
-template <int HD, int TPW>
+template <int HD, int TPW, bool BIAS>
 static int attn_mfma_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
-#define PTM_AM(GG) hipLaunchKernelGGL((attn_decode_mfma_kernel<HD, GG, TPW>), grid, dim3(FD_THREADS), 0, s, a)
+#define PTM_AM(GG) hipLaunchKernelGGL((attn_decode_mfma_kernel<HD, GG, TPW, BIAS>), grid, dim3(FD_THREADS), 0, s, a)
     switch (G) {
         case 1: PTM_AM(1); break;
         case 2: PTM_AM(2); break;
@@ -1386,12 +1415,21 @@ int ptm_flash_decode_pos(const float* Q, const void* K_cache, const void* V_cach
 // ptm_attn_decode_fused that can also leave the output as Q8 activation blocks (o_q8, may be NULL) for a Q4_K output
 // projection.  The decode runtime's entry; not declared in the public header.
 // window > 0: only the last `window` positions (the new one included) are attended to.
-int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, const float* q_norm_w,
-                              const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8, float* partial_O,
-                              float* partial_lse, float* partial_max, const float* rope_table,
-                              int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
-                              float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
-                              ptm_stream_t stream) {
+// 1 when ptm_attn_decode_fused_bias adds the projection biases itself for this cache type and head size
+int ptm_attn_decode_folds_bias(int head_dim, int kv_fp16) { return kv_fp16 && (head_dim == 64 || head_dim == 128); }
+
+// As ptm_attn_decode_fused_win with the biases of the q / k / v projections (all three or none) added to the raw vectors
+// before norm and rotation; only where ptm_attn_decode_folds_bias says so.
+int ptm_attn_decode_fused_bias(const float* Q, const float* K, const float* V, const float* q_bias, const float* k_bias,
+                               const float* v_bias, const float* q_norm_w,
+                               const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8, float* partial_O,
+                               float* partial_lse, float* partial_max, const float* rope_table,
+                               int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                               float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
+                               ptm_stream_t stream) {
+    const bool bias = q_bias != nullptr;
+    if (bias != (k_bias != nullptr) || bias != (v_bias != nullptr)) return PTM_E_NULL;
+    if (bias && !ptm_attn_decode_folds_bias(head_dim, kv_fp16)) return PTM_E_UNSUPPORTED;
     if (!Q || !K || !V || !K_cache || !V_cache || !O || !partial_O || !partial_lse || !partial_max ||
         !rope_table || !d_past_len)
         return PTM_E_NULL;
@@ -1413,7 +1451,8 @@ int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, co
                         static_cast<uint8_t*>(o_q8));
     }
     AttnArgs a{Q, K, V, q_norm_w, k_norm_w, rope_table, K_cache, V_cache, partial_O, partial_lse, partial_max,
-               d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps, rope_interleaved ? 1 : 0, window > 0 ? window : 0};
+               d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps, rope_interleaved ? 1 : 0, window > 0 ? window : 0,
+               q_bias, k_bias, v_bias};
     const int G = n_heads / n_kv_heads;
     const dim3 grid(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
     hipStream_t s = as_stream(stream);
@@ -1424,12 +1463,14 @@ int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, co
         if (ptm_flash_decode_num_splits(max_seq) > FD_LONG_SPLITS) {
             // a cache of more than 4096 positions: the looping kernel, at most FD_LONG_SPLITS partials per head
             const dim3 grid_long(FD_LONG_SPLITS, n_kv_heads);
-            rc = head_dim == 128 ? attn_mfma_long_launch_g<128>(G, grid_long, s, a) : attn_mfma_long_launch_g<64>(G, grid_long, s, a);
+            if (bias) rc = head_dim == 128 ? attn_mfma_long_launch_g<128, true>(G, grid_long, s, a) : attn_mfma_long_launch_g<64, true>(G, grid_long, s, a);
+            else rc = head_dim == 128 ? attn_mfma_long_launch_g<128, false>(G, grid_long, s, a) : attn_mfma_long_launch_g<64, false>(G, grid_long, s, a);
             if (rc != PTM_OK) return rc;
             return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
                             static_cast<uint8_t*>(o_q8), 0, -1, 1);
         }
-        rc = head_dim == 128 ? attn_mfma_launch_g<128, 1>(G, grid, s, a) : attn_mfma_launch_g<64, 1>(G, grid, s, a);
+        if (bias) rc = head_dim == 128 ? attn_mfma_launch_g<128, 1, true>(G, grid, s, a) : attn_mfma_launch_g<64, 1, true>(G, grid, s, a);
+        else rc = head_dim == 128 ? attn_mfma_launch_g<128, 1, false>(G, grid, s, a) : attn_mfma_launch_g<64, 1, false>(G, grid, s, a);
         if (rc != PTM_OK) return rc;
         return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
                         static_cast<uint8_t*>(o_q8), 0, FD_CHUNK, 1);
@@ -1438,6 +1479,17 @@ int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, co
     if (rc != PTM_OK) return rc;
     return fd_merge(head_dim, n_heads, s, partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
                     static_cast<uint8_t*>(o_q8));
+}
+
+int ptm_attn_decode_fused_win(const float* Q, const float* K, const float* V, const float* q_norm_w,
+                              const float* k_norm_w, void* K_cache, void* V_cache, float* O, void* o_q8, float* partial_O,
+                              float* partial_lse, float* partial_max, const float* rope_table,
+                              int n_heads, int n_kv_heads, int head_dim, const int64_t* d_past_len, int max_seq,
+                              float scale, float eps, int add_one, int kv_fp16, int rope_interleaved, int window,
+                              ptm_stream_t stream) {
+    return ptm_attn_decode_fused_bias(Q, K, V, nullptr, nullptr, nullptr, q_norm_w, k_norm_w, K_cache, V_cache, O, o_q8,
+                                      partial_O, partial_lse, partial_max, rope_table, n_heads, n_kv_heads, head_dim,
+                                      d_past_len, max_seq, scale, eps, add_one, kv_fp16, rope_interleaved, window, stream);
 }
 
 int ptm_attn_decode_fused_q8(const float* Q, const float* K, const float* V, const float* q_norm_w,

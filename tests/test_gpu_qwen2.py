@@ -45,6 +45,63 @@ def test_add_qkv_bias_is_one_fp32_add_per_element(dev, rows, qd, kvd):
         assert np.array_equal(bits(got.cpu().numpy()), bits(want))
 
 
+@pytest.mark.parametrize("nh,nkv,hd,past,max_seq,interleaved", [
+    (28, 4, 128, 2100, 2304, 0), (12, 2, 128, 300, 512, 0), (14, 2, 64, 63, 128, 0), (4, 4, 64, 0, 64, 1),
+    (28, 4, 128, 5000, 8192, 0), (16, 2, 64, 4097, 4224, 1)])
+def test_attention_launch_that_adds_the_biases_equals_the_separate_add(dev, nh, nkv, hd, past, max_seq, interleaved):
+    """With an fp16 cache and heads of 64 or 128 the decoder hands the bias vectors to the attention launch instead of
+    running the bias kernel first (caches of up to 4096 positions and beyond: both kernels): output, its Q8 blocks and the
+    appended cache rows are bit-identical to bias kernel + attention."""
+    import ctypes as C
+    from prometorch_amd import _lib
+    L = _lib.load()
+    vp = C.c_void_p
+    tail = [C.c_int, C.c_int, C.c_int, vp, C.c_int, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int]
+    plain, fold = L.ptm_attn_decode_fused_q8, L.ptm_attn_decode_fused_bias
+    plain.restype = fold.restype = C.c_int
+    plain.argtypes = [vp] * 13 + tail + [vp]
+    fold.argtypes = [vp] * 16 + tail + [C.c_int, vp]
+    assert L.ptm_attn_decode_folds_bias(hd, 1) == 1 and L.ptm_attn_decode_folds_bias(256, 1) == 0
+    assert L.ptm_attn_decode_folds_bias(hd, 0) == 0
+    r = synth.rng_for(93, nh, hd, past)
+    kvd, qd = nkv * hd, nh * hd
+    K0 = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16)
+    V0 = r.standard_normal((max_seq, kvd), dtype=np.float32).astype(np.float16)
+    S = ops.flash_decode_num_splits(max_seq)
+    table = ops.rope_table(max_seq, hd, 1e6).cuda()
+    d_past = torch.full((1,), past, dtype=torch.int64, device="cuda")
+    Q, K, V = synth.make_x(r, qd) * 3, synth.make_x(r, kvd) * 3, synth.make_x(r, kvd)
+    bq, bk, bv = synth.make_x(r, qd) * 2, synth.make_x(r, kvd) * 2, synth.make_x(r, kvd)
+    p = lambda t: t.data_ptr()
+    res = []
+    for folded in (False, True):
+        Kc, Vc = cu(K0), cu(V0)
+        pO, pL, pM = torch.empty(S * qd, device="cuda"), torch.empty(S * nh, device="cuda"), torch.empty(S * nh, device="cuda")
+        O = torch.empty(qd, device="cuda")
+        q8 = torch.zeros(ops.q8_bytes(qd), dtype=torch.uint8, device="cuda")
+        dQ, dK, dV, dbq, dbk, dbv = cu(Q), cu(K), cu(V), cu(bq), cu(bk), cu(bv)
+        if folded:
+            rc = fold(p(dQ), p(dK), p(dV), p(dbq), p(dbk), p(dbv), None, None, p(Kc), p(Vc), p(O), p(q8), p(pO), p(pL),
+                      p(pM), p(table), nh, nkv, hd, p(d_past), max_seq, 1.0 / np.sqrt(hd), 1e-6, 0, 1, interleaved, 0, None)
+        else:
+            ops.add_qkv_bias(dQ, dK, dV, dbq, dbk, dbv, 1, qd, kvd)
+            rc = plain(p(dQ), p(dK), p(dV), None, None, p(Kc), p(Vc), p(O), p(q8), p(pO), p(pL), p(pM), p(table), nh, nkv,
+                       hd, p(d_past), max_seq, 1.0 / np.sqrt(hd), 1e-6, 0, 1, interleaved, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        res.append((O.cpu().numpy(), q8.cpu().numpy(), Kc[past].cpu().numpy(), Vc[past].cpu().numpy()))
+    assert np.isfinite(res[0][0]).all() and np.abs(res[0][0]).max() > 0
+    for a, b in zip(*res):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    # where the launch cannot add them it says so and launches nothing
+    assert fold(16, 16, 16, 16, 16, 16, None, None, 16, 16, 16, None, 16, 16, 16, 16, 8, 4, 256, 16, 128, 1.0, 1e-6, 0, 1, 0, 0,
+                None) == -4
+    assert fold(16, 16, 16, 16, 16, 16, None, None, 16, 16, 16, None, 16, 16, 16, 16, 8, 4, 128, 16, 128, 1.0, 1e-6, 0, 0, 0, 0,
+                None) == -4
+    assert fold(16, 16, 16, 16, None, 16, None, None, 16, 16, 16, None, 16, 16, 16, 16, 8, 4, 128, 16, 128, 1.0, 1e-6, 0, 1, 0, 0,
+                None) == -1
+
+
 @pytest.mark.parametrize("use_graph", [False, True])
 def test_qwen2_teacher_forced_vs_reference_golden(dev, golden_qwen2, seeds, use_graph):
     """16 distinct seeded ids fed step by step (the greedy run of this model repeats one id): argmax and logits of every step
