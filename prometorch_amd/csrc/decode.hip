@@ -15,6 +15,7 @@
 
 #include <cstring>
 #include <new>
+#include <utility>
 #include <vector>
 
 // flash_decode.hip: ptm_attn_decode_fused that also leaves the output as Q8 activation blocks (not part of the C ABI)
@@ -70,7 +71,7 @@ __global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
 }
 int rmsnorm_mixed_gemv(int n4, const void* const* W4, float* const* y4, const int* N4, int64_t stride4,
                        const void* W6, float* y6, int N6, int64_t stride6, const float* x, const float* gamma,
-                       float eps, int add_one, int K, hipStream_t s);
+                       float eps, int add_one, int K, hipStream_t s, const float* pre_h, const float* pre_w, float* pre_out);
 
 __global__ void set_scalars_kernel(int* d_token, int token, int64_t* d_past, int64_t past, int* d_step) {
     *d_token = token;
@@ -116,6 +117,7 @@ struct ptm_decoder {
           *gate = nullptr, *up = nullptr, *logits = nullptr, *pO = nullptr, *pL = nullptr, *pM = nullptr,
           *rope = nullptr;
     float* hb = nullptr;        // [hidden] a branch's output in front of its post-norm
+    float* x2 = nullptr;        // [hidden] second residual buffer: a kernel that applies a deferred post-norm reads one, writes the other
     float* rope_swa = nullptr;  // rotation table of the sliding-window layers (their own base, no position scaling)
     uint8_t* xq8 = nullptr;
     void* amax_ws = nullptr;
@@ -193,6 +195,24 @@ static int enqueue_step(ptm_decoder* d, bool sample = false, float* trace = null
     else PTM_TRY(ptm_embedding_row_q6k(c.lm_head.data, d->x, d->d_token, H, c.lm_head.row_stride_bytes, s));
     if (c.scale_embeddings) PTM_TRY(ptm_scale(d->x, sqrtf((float)H), H, s));
 
+    // The residual stream is in xc.  The post-norm of a feed-forward branch (gemma: x += RMSNorm(h) * w) is not a launch of its
+    // own where the next layer's q / k / v launch can apply it in its prologue (the mixed Q4_K / Q6_K launch; vectors of up to
+    // 4096 values): that launch reads xc, h and w, and its first workgroup writes the updated residual to the other buffer,
+    // xo.  pend_h / pend_w: the post-norm waiting for the next layer.  A traced step applies every post-norm at once.
+    // (The same in front of the fused gate / up launch for the post-norm of the attention branch gains nothing: the two extra
+    // vectors in the prologue of its 1280 workgroups cost what the launch saves.)
+    float *xc = d->x, *xo = d->x2;
+    const float *pend_h = nullptr, *pend_w = nullptr;
+    auto qkv_is_mixed = [&](const ptm_layer& L) {
+        if (!tuned_type(L.q.ggml_type) || !tuned_type(L.k.ggml_type) || !tuned_type(L.v.ggml_type)) return false;
+        const int n6 = (L.q.ggml_type != PTM_TYPE_Q4_K) + (L.k.ggml_type != PTM_TYPE_Q4_K) + (L.v.ggml_type != PTM_TYPE_Q4_K);
+        return n6 == 1 && H <= 16384;
+    };
+    auto gate_up_is_fused = [&](const ptm_layer& L) {
+        return L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
+               L.gate.row_stride_bytes == L.up.row_stride_bytes && L.gate.rows == L.up.rows;
+    };
+    const bool may_defer = !trace && H <= 4096;
     for (int li = 0; li < c.n_layers; ++li) {
         const ptm_layer& L = d->layers[li];
         const bool local = layer_is_local(c, li);  // sliding-window layer: own rotation table, attention window
@@ -210,18 +230,22 @@ static int enqueue_step(ptm_decoder* d, bool sample = false, float* trace = null
             int64_t s4 = 0;  // the Q4_K projections of one launch share a row stride (checked at create)
             for (int i = 0; i < 3; ++i) if (w[i]->ggml_type == PTM_TYPE_Q4_K) { s4 = w[i]->row_stride_bytes; break; }
             if (!tuned_type(L.q.ggml_type) || !tuned_type(L.k.ggml_type) || !tuned_type(L.v.ggml_type)) {
-                PTM_TRY(ptm_rms_norm(d->x, L.attn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+                PTM_TRY(ptm_rms_norm(xc, L.attn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
                 for (int i = 0; i < 3; ++i) PTM_TRY(gemv_any(*w[i], d->xn, y[i], false, s));
             } else if (n6 == 1 && n4 >= 1 && H <= 16384) {
                 // the Q4_K_M mix (q, k in Q4_K; v in Q6_K): all three projections in one launch
                 PTM_TRY(rmsnorm_mixed_gemv(n4, W4, y4, N4, s4, w[i6]->data, y[i6], w[i6]->rows, w[i6]->row_stride_bytes,
-                                           d->x, L.attn_norm, c.rms_eps, 0, H, s));
+                                           xc, L.attn_norm, c.rms_eps, 0, H, s, pend_h, pend_w, pend_h ? xo : nullptr));
+                if (pend_h) {
+                    std::swap(xc, xo);
+                    pend_h = pend_w = nullptr;
+                }
             } else {
                 for (int i = 0; i < 3; ++i)
                     if (w[i]->ggml_type != PTM_TYPE_Q4_K)
-                        PTM_TRY(q6k_gemv_impl(w[i]->data, d->x, y[i], H, w[i]->rows, w[i]->row_stride_bytes, false,
+                        PTM_TRY(q6k_gemv_impl(w[i]->data, xc, y[i], H, w[i]->rows, w[i]->row_stride_bytes, false,
                                               L.attn_norm, c.rms_eps, 0, s));
-                if (n4 > 0) PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, d->x, false, L.attn_norm, c.rms_eps, 0, H, s4, false, s));
+                if (n4 > 0) PTM_TRY(q4k_gemv_multi(n4, W4, y4, N4, xc, false, L.attn_norm, c.rms_eps, 0, H, s4, false, s));
             }
         }
         // projection biases (qwen2): added by the attention launch where it can, else by a launch of their own
@@ -238,7 +262,7 @@ static int enqueue_step(ptm_decoder* d, bool sample = false, float* trace = null
                                            c.n_heads, c.n_kv_heads, hd, d->d_past, c.max_seq, 1.0f / sqrtf((float)hd),
                                            c.rms_eps, 0, c.kv_fp16, c.rope_interleaved, local ? c.swa_window : 0, s));
         // x += Wo . attn, or with a post-norm: h = Wo . attn, x += RMSNorm(h) * w
-        float* o_dst = L.post_attn_norm ? d->hb : d->x;
+        float* o_dst = L.post_attn_norm ? d->hb : xc;
         const bool o_acc = !L.post_attn_norm;
         if (o_q8) {
             const void* W = L.o.data;
@@ -247,14 +271,13 @@ static int enqueue_step(ptm_decoder* d, bool sample = false, float* trace = null
         } else {
             PTM_TRY(gemv_any(L.o, d->attn, o_dst, o_acc, s));
         }
-        if (L.post_attn_norm) PTM_TRY(ptm_rms_norm_add(d->hb, L.post_attn_norm, d->x, 1, H, c.rms_eps, 0, s));
-        if (trace) PTM_TRY(ptm_copy(d->x, trace + (size_t)(2 * li) * H, H, s));
-        if (L.gate.ggml_type == PTM_TYPE_Q4_K && L.up.ggml_type == PTM_TYPE_Q4_K &&
-            L.gate.row_stride_bytes == L.up.row_stride_bytes && L.gate.rows == L.up.rows) {
-            PTM_TRY(q4k_gate_up_silu(L.gate.data, L.up.data, d->x, false, L.ffn_norm, c.rms_eps, 0, d->act, H,
+        if (L.post_attn_norm) PTM_TRY(ptm_rms_norm_add(d->hb, L.post_attn_norm, xc, 1, H, c.rms_eps, 0, s));
+        if (trace) PTM_TRY(ptm_copy(xc, trace + (size_t)(2 * li) * H, H, s));
+        if (gate_up_is_fused(L)) {
+            PTM_TRY(q4k_gate_up_silu(L.gate.data, L.up.data, xc, false, L.ffn_norm, c.rms_eps, 0, d->act, H,
                                      L.gate.rows, L.gate.row_stride_bytes, s, c.ffn_gelu != 0));
         } else {
-            PTM_TRY(ptm_rms_norm(d->x, L.ffn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+            PTM_TRY(ptm_rms_norm(xc, L.ffn_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
             PTM_TRY(gemv_any(L.gate, d->xn, d->gate, false, s));
             PTM_TRY(gemv_any(L.up, d->xn, d->up, false, s));
             if (c.ffn_gelu) PTM_TRY(ptm_gelu_mul(d->gate, d->up, d->act, c.inter, s));
@@ -262,19 +285,24 @@ static int enqueue_step(ptm_decoder* d, bool sample = false, float* trace = null
         }
         if (L.post_ffn_norm) {
             PTM_TRY(gemv_any(L.down, d->act, d->hb, false, s));
-            PTM_TRY(ptm_rms_norm_add(d->hb, L.post_ffn_norm, d->x, 1, H, c.rms_eps, 0, s));
+            if (may_defer && li + 1 < c.n_layers && qkv_is_mixed(d->layers[li + 1])) {
+                pend_h = d->hb;  // applied by the next layer's q / k / v launch
+                pend_w = L.post_ffn_norm;
+            } else {
+                PTM_TRY(ptm_rms_norm_add(d->hb, L.post_ffn_norm, xc, 1, H, c.rms_eps, 0, s));
+            }
         } else {
-            PTM_TRY(gemv_any(L.down, d->act, d->x, true, s));  // x += Wdown . act
+            PTM_TRY(gemv_any(L.down, d->act, xc, true, s));  // x += Wdown . act
         }
-        if (trace) PTM_TRY(ptm_copy(d->x, trace + (size_t)(2 * li + 1) * H, H, s));
+        if (trace) PTM_TRY(ptm_copy(xc, trace + (size_t)(2 * li + 1) * H, H, s));
     }
     if (sample) {
         // logits (final RMSNorm in the lm_head prologue), then the sampler, whose last kernel does the step bookkeeping
         if (c.lm_head.ggml_type == PTM_TYPE_Q6_K) {
-            PTM_TRY(q6k_gemv_impl(c.lm_head.data, d->x, d->logits, H, c.vocab, c.lm_head.row_stride_bytes, false, c.out_norm,
+            PTM_TRY(q6k_gemv_impl(c.lm_head.data, xc, d->logits, H, c.vocab, c.lm_head.row_stride_bytes, false, c.out_norm,
                                   c.rms_eps, 0, s));
         } else {
-            PTM_TRY(ptm_rms_norm(d->x, c.out_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+            PTM_TRY(ptm_rms_norm(xc, c.out_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
             PTM_TRY(gemv_any(c.lm_head, d->xn, d->logits, false, s));
         }
         return sampler_enqueue(d->logits, c.vocab, d->d_counts, d->sampling, d->d_sampling, d->d_uniforms, d->d_step,
@@ -283,11 +311,11 @@ static int enqueue_step(ptm_decoder* d, bool sample = false, float* trace = null
     }
     if (c.lm_head.ggml_type == PTM_TYPE_Q6_K) {
         // final RMSNorm in the lm_head prologue, step bookkeeping in the argmax tail: two launches for the whole tail
-        return q6k_gemv_argmax_impl(c.lm_head.data, d->x, c.out_norm, c.rms_eps, 0, d->xn, d->logits, H, c.vocab,
+        return q6k_gemv_argmax_impl(c.lm_head.data, xc, c.out_norm, c.rms_eps, 0, d->xn, d->logits, H, c.vocab,
                                     c.lm_head.row_stride_bytes, d->d_next, d->amax_ws,
                                     ArgmaxAdvance{d->d_token, d->d_past, d->d_step, d->d_tokens, c.max_seq}, s);
     }
-    PTM_TRY(ptm_rms_norm(d->x, c.out_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
+    PTM_TRY(ptm_rms_norm(xc, c.out_norm, d->xn, 1, H, c.rms_eps, 0, nullptr, s));
     PTM_TRY(gemv_any(c.lm_head, d->xn, d->logits, false, s));
     PTM_TRY(ptm_argmax(d->logits, d->d_next, c.vocab, s));
     hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(1), 0, s, d->d_next, d->d_token, d->d_past, d->d_step,
@@ -510,7 +538,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
                  o_up = take(4 * (size_t)c.inter), o_logits = take(4 * (size_t)c.vocab),
                  o_pO = take(4 * (size_t)S * c.n_heads * c.head_dim), o_pL = take(4 * (size_t)S * c.n_heads),
                  o_pM = take(4 * (size_t)S * c.n_heads), o_rope = take(4 * (size_t)c.max_seq * c.head_dim),
-                 o_hb = take(4 * (size_t)H), o_rope_swa = take(c.swa_window > 0 ? 4 * (size_t)c.max_seq * c.head_dim : 0),
+                 o_hb = take(4 * (size_t)H), o_x2 = take(4 * (size_t)H), o_rope_swa = take(c.swa_window > 0 ? 4 * (size_t)c.max_seq * c.head_dim : 0),
                  o_xq8 = take((size_t)ptm_q8_bytes(qd > (H > c.inter ? H : c.inter) ? qd : (H > c.inter ? H : c.inter))),
                  o_ws = take((size_t)ptm_argmax_workspace_bytes(c.vocab)), o_tok = take(256), o_past = take(256),
                  o_next = take(256), o_step = take(256),
@@ -523,7 +551,7 @@ int ptm_decode_create(const ptm_decode_config* cfg, ptm_decoder** out) {
     d->act = (float*)(base + o_act); d->gate = (float*)(base + o_gate); d->up = (float*)(base + o_up);
     d->logits = (float*)(base + o_logits); d->pO = (float*)(base + o_pO); d->pL = (float*)(base + o_pL);
     d->pM = (float*)(base + o_pM); d->rope = (float*)(base + o_rope); d->xq8 = base + o_xq8;
-    d->hb = (float*)(base + o_hb); d->rope_swa = c.swa_window > 0 ? (float*)(base + o_rope_swa) : d->rope;
+    d->hb = (float*)(base + o_hb); d->x2 = (float*)(base + o_x2); d->rope_swa = c.swa_window > 0 ? (float*)(base + o_rope_swa) : d->rope;
     d->amax_ws = base + o_ws; d->d_token = (int*)(base + o_tok); d->d_past = (int64_t*)(base + o_past);
     d->d_next = (int64_t*)(base + o_next); d->d_step = (int*)(base + o_step);
     d->d_sampling = (ptm_sampling*)(base + o_samp); d->d_counts = (int32_t*)(base + o_counts);

@@ -283,6 +283,42 @@ __device__ __forceinline__ void stage_finish(const XStage<NCH>& st, int K, float
         if (1024 * c < n4) emit_chunk<NORM>(st.x[c], st.g[c], 1024 * c, n4, rs, add_one ? 1.0f : 0.0f, emit);
 }
 
+// The same staging with a deferred post-norm in front (K <= 4096, one chunk): the vector that is normalised is
+// x + RMSNorm(h) * w, formed by every workgroup from x, the branch output h and the post-norm weight w; pre_out (NULL in all
+// but one workgroup) receives that sum.  Slots past the end of the vectors load as zeros and stay zero.
+struct XStagePre { XChunk x, g, h, w; };
+
+__device__ __forceinline__ XStagePre stage_issue_pre(const float* x, const float* gamma, const float* h, const float* w, int K) {
+    XStagePre st;
+    st.h = load_chunk(make_rsrc(h, K * 4), 0);  // the branch output first: its sum of squares is the first thing needed
+    st.w = load_chunk(make_rsrc(w, K * 4), 0);
+    st.x = load_chunk(make_rsrc(x, K * 4), 0);
+    st.g = load_chunk(make_rsrc(gamma, K * 4), 0);
+    return st;
+}
+
+template <typename Emit>
+__device__ __forceinline__ void stage_finish_pre(const XStagePre& st, int K, float eps, int add_one, float* red4,
+                                                 float* pre_out, Emit emit) {
+    const int n4 = K / 4;
+    const float one = add_one ? 1.0f : 0.0f;
+    const float ssh = block_sum256(chunk_sumsq(st.h, 0.0f), red4);
+    const float rsh = 1.0f / sqrtf(ssh / (float)K + eps);
+    XChunk xe;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        xe.v[u].x = st.x.v[u].x + st.h.v[u].x * rsh * (st.w.v[u].x + one);
+        xe.v[u].y = st.x.v[u].y + st.h.v[u].y * rsh * (st.w.v[u].y + one);
+        xe.v[u].z = st.x.v[u].z + st.h.v[u].z * rsh * (st.w.v[u].z + one);
+        xe.v[u].w = st.x.v[u].w + st.h.v[u].w * rsh * (st.w.v[u].w + one);
+        const int i = (int)threadIdx.x + 256 * u;
+        if (pre_out && i < n4) reinterpret_cast<float4*>(pre_out)[i] = xe.v[u];
+    }
+    const float ss = block_sum256(chunk_sumsq(xe, 0.0f), red4);
+    const float rs = 1.0f / sqrtf(ss / (float)K + eps);
+    emit_chunk<true>(xe, st.g, 0, n4, rs, one, emit);
+}
+
 // Blocks per pass for a lane group that owns nb_max blocks: the candidate (from a small set, so that the
 // number of kernel instances stays small) that wastes the fewest padded block slots; ties go to the larger.
 inline int pick_blocks_per_pass(int nb_max, const int* cand, int n_cand) {

@@ -20,6 +20,13 @@ struct Q4KArgs {
     float eps;
     int add_one;
     int gelu;            // MODE 1: tanh-GELU(gate) * up (gemma) instead of SiLU(gate) * up
+    // PRE (with NORM, K <= 4096): the branch output of the previous projection still waits for its post-norm and residual
+    // add (gemma's post-attention / post-feed-forward norms, gguf_model.h:3656-3680, :3787-3807).  Every workgroup forms
+    // x + RMSNorm(pre_h) * pre_w itself before its own RMSNorm; workgroup 0 also stores that sum to pre_out, which must not
+    // be x (other workgroups still read x).
+    const float* pre_h;
+    const float* pre_w;
+    float* pre_out;
 };
 
 enum { Q4K_THREADS = 256, Q4K_U = 10 };
@@ -29,7 +36,7 @@ enum { Q4K_THREADS = 256, Q4K_U = 10 };
 // fp32 x: thread t owns the 16 consecutive values [16t, 16t+16), i.e. half a Q8 block (lanes t, t^1 share a
 // block), so the two exact divisions of the Q8 rule are paid once per 16 values.  Every workgroup quantises the
 // whole vector, so this prologue is kept short: its instructions are issued by every wave of the launch.
-struct Q4KStage { float4 x[4], g[4]; float rs; u32x4 q8[2]; };
+struct Q4KStage { float4 x[4], g[4], h[4], w[4]; float rs; u32x4 q8[2]; };
 
 __device__ __forceinline__ void q4k_load16(__amdgpu_buffer_rsrc_t r, int first, float4 (&v)[4]) {
 #pragma unroll
@@ -87,8 +94,9 @@ __device__ __forceinline__ void q4k_quantize16_store(const float4 (&xv)[4], cons
     }
 }
 
-template <bool XQ8, bool NORM>
+template <bool XQ8, bool NORM, bool PRE = false>
 __device__ __forceinline__ Q4KStage q4k_stage_issue(const Q4KArgs a, uint8_t* lds, float* red) {
+    static_assert(!PRE || (NORM && !XQ8), "the deferred post-norm comes with the RMSNorm prologue");
     Q4KStage st;
     const int tid = threadIdx.x;
     st.rs = 1.0f;
@@ -127,14 +135,18 @@ __device__ __forceinline__ Q4KStage q4k_stage_issue(const Q4KArgs a, uint8_t* ld
             }
         }
         issue_order_fence();
+        if constexpr (PRE) {  // the branch output first: its sum of squares is the first thing needed
+            q4k_load16(make_rsrc(a.pre_h, a.K * 4), 16 * tid, st.h);
+            q4k_load16(make_rsrc(a.pre_w, a.K * 4), 16 * tid, st.w);
+        }
         q4k_load16(rx, 16 * tid, st.x);
         if constexpr (NORM) q4k_load16(rg, 16 * tid, st.g);
     }
     return st;
 }
 
-template <bool XQ8, bool NORM>
-__device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KArgs a, uint8_t* lds, float* red) {
+template <bool XQ8, bool NORM, bool PRE = false>
+__device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KArgs a, uint8_t* lds, float* red, int wg = 0) {
     const int tid = threadIdx.x;
     if constexpr (XQ8) {
         uint4* dst = reinterpret_cast<uint4*>(lds);
@@ -144,6 +156,26 @@ __device__ __forceinline__ void q4k_stage_finish(const Q4KStage& st, const Q4KAr
             const int i = tid + Q4K_THREADS * u;
             if (i < n16) dst[i] = make_uint4(st.q8[u].x, st.q8[u].y, st.q8[u].z, st.q8[u].w);
         }
+    } else if constexpr (PRE) {
+        // x + RMSNorm(h) * w first (threads past the end hold zeros), then the kernel's own RMSNorm of that sum
+        const float one = a.add_one ? 1.0f : 0.0f;
+        const float ssh = block_sum256(q4k_sumsq16(st.h, 0.0f), red);
+        const float rsh = 1.0f / sqrtf(ssh / (float)a.K + a.eps);
+        float4 xv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            xv[u].x = st.x[u].x + st.h[u].x * rsh * (st.w[u].x + one);
+            xv[u].y = st.x[u].y + st.h[u].y * rsh * (st.w[u].y + one);
+            xv[u].z = st.x[u].z + st.h[u].z * rsh * (st.w[u].z + one);
+            xv[u].w = st.x[u].w + st.h[u].w * rsh * (st.w[u].w + one);
+        }
+        if (wg == 0 && a.pre_out && 16 * tid < a.K) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) reinterpret_cast<float4*>(a.pre_out)[4 * tid + u] = xv[u];
+        }
+        const float ss = block_sum256(q4k_sumsq16(xv, 0.0f), red);
+        const float rs = 1.0f / sqrtf(ss / (float)a.K + a.eps);
+        if (16 * tid < a.K) q4k_quantize16_store<true>(xv, st.g, rs, one, tid, lds, a.K);
     } else {
         float rs = st.rs;
         if constexpr (NORM) {
@@ -213,7 +245,7 @@ __device__ __forceinline__ float silu_mul_ref(float g, float u) {
 //     passes roll ACROSS tiles - a consumed block's registers are refilled with the same slot of the NEXT tile's row, so a
 //     wave never stands with nothing in flight between two tiles (behind the last tile the refills repeat that tile: their
 //     number stays static, the lines are in cache, nothing consumes them).
-template <bool XQ8, bool NORM, bool ACC, int MODE, int NB, bool ROLLT = false>
+template <bool XQ8, bool NORM, bool ACC, int MODE, int NB, bool ROLLT = false, bool PRE = false>
 __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int wg) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 7, grp = lane >> 3;
@@ -296,7 +328,8 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
 
     // ---- activation loads first, then the first tile's weight loads, then the activation prologue ----
     __shared__ float red[4];
-    const Q4KStage stg = q4k_stage_issue<XQ8, NORM>(a, lds, red);
+    static_assert(!(PRE && ROLLT), "the deferred post-norm is built into the one-tile-at-a-time form only");
+    const Q4KStage stg = q4k_stage_issue<XQ8, NORM, PRE>(a, lds, red);
     if constexpr (ROLLT) {
         // MODE 0: one matrix (a.W[0], a.y[0]); MODE 1: virtual row 2 r = gate row r (a.W[0]), 2 r + 1 = up row r (a.W[1]).
         // The pointers are taken out of the argument struct once: a select over its arrays per tile would push it to scratch.
@@ -359,7 +392,7 @@ __device__ __forceinline__ void q4k_gemv_body(const Q4KArgs a, uint8_t* lds, int
         }
         return;
     }
-    run_tile(wg * tpw, [&] { q4k_stage_finish<XQ8, NORM>(stg, a, lds, red); });
+    run_tile(wg * tpw, [&] { q4k_stage_finish<XQ8, NORM, PRE>(stg, a, lds, red, wg); });
     // further tiles reuse the staged activations: the quantisation of x is paid once per workgroup
     for (int k = 1; k < tpw; ++k) {
         const int tile = wg * tpw + k;

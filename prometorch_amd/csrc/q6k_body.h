@@ -18,6 +18,11 @@ struct Q6KArgs {
     float eps;
     int add_one;
     float* xn_out;       // NORM: if not NULL, workgroup 0 also stores the normalised x[K] here
+    // PRE (with NORM, K <= 4096): a deferred post-norm and residual add in front of the RMSNorm, x + RMSNorm(pre_h) * pre_w;
+    // workgroup 0 stores that sum to pre_out (not x: other workgroups still read x)
+    const float* pre_h;
+    const float* pre_w;
+    float* pre_out;
 };
 
 enum { Q6K_THREADS = 256, Q6K_U = 5 };
@@ -105,7 +110,7 @@ __device__ __forceinline__ float q6k_block_term(const Q6Blk& k, const float* __r
 // NB:  super-blocks per lane group and pass.  Every pass issues exactly NB block loads, unconditionally
 //      (block indices past the row's end are clamped and their terms dropped), so that the number of loads
 //      in flight is known at compile time and each block is consumed as soon as IT has arrived.
-template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB>
+template <bool ACC, bool ARGMAX, bool NORM, int XCH, int NB, bool PRE = false>
 __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw, int wg) {
     float* xf = reinterpret_cast<float*>(lds_raw);
     float* xsum16 = xf + q6k_x_floats(a.K);
@@ -136,13 +141,23 @@ __device__ __forceinline__ void q6k_gemv_body(const Q6KArgs a, uint8_t* lds_raw,
         if ((tid & 3) == 0) xsum16[i >> 2] = sm;
     };
     // activation loads first (loads complete in issue order), then the first pass of weight loads
-    const XStage<XCH> stg = stage_issue<NORM, XCH>(a.x, a.gamma, a.K, a.eps, a.add_one, red, emit);
+    static_assert(!PRE || (NORM && XCH == 1), "the deferred post-norm comes with the RMSNorm prologue of short vectors");
     Q6Blk blk[NB];
-    issue_order_fence();
+    if constexpr (PRE) {
+        const XStagePre stg = stage_issue_pre(a.x, a.gamma, a.pre_h, a.pre_w, a.K);
+        issue_order_fence();
 #pragma unroll
-    for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off, sc_off);
-    issue_order_fence();
-    stage_finish<NORM, XCH>(stg, a.K, a.eps, a.add_one, red, emit);
+        for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off, sc_off);
+        issue_order_fence();
+        stage_finish_pre(stg, a.K, a.eps, a.add_one, red, wg == 0 ? a.pre_out : nullptr, emit);
+    } else {
+        const XStage<XCH> stg = stage_issue<NORM, XCH>(a.x, a.gamma, a.K, a.eps, a.add_one, red, emit);
+        issue_order_fence();
+#pragma unroll
+        for (int u = 0; u < NB; ++u) blk[u] = q6k_load(row + (int64_t)min(sub + (u << a.log2S), nblk - 1) * 210, j, qh_off, sc_off);
+        issue_order_fence();
+        stage_finish<NORM, XCH>(stg, a.K, a.eps, a.add_one, red, emit);
+    }
     __syncthreads();
 
     // Passes roll: as soon as a block of pass p has been consumed its registers are refilled with the same slot of

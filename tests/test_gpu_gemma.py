@@ -214,6 +214,45 @@ def test_gemma_decode_fp16_kv_vs_oracle_and_chained_greedy(dev, po, seeds, past)
     dec2.close()
 
 
+@pytest.mark.parametrize("shape", ["tiny", "4b_layers"])
+def test_step_that_defers_the_post_ffn_norm_matches_the_traced_step(dev, seeds, shape):
+    """A plain step leaves the post-norm and residual add of a layer's feed-forward branch to the prologue of the next layer's
+    q / k / v launch; a traced step runs each as a launch of its own.  Same state, same token: the logits agree to the
+    bars of a decode step (the two sums of squares are taken in different orders, nothing else differs), and the traced
+    residual stream after the last layer is what the plain step's final norm saw (hidden = RMSNorm of it)."""
+    from prometorch_amd.decode import Decoder
+    if shape == "tiny":
+        cfg, layers, head = synth.tiny_gemma(seeds["tiny"])
+        past, max_seq = 19, 64
+    else:
+        cfg, layers, head = synth.gemma3_4b_like(seeds["cfg4"], n_layers=3, vocab=4096)
+        past, max_seq = 300, 512
+    decs = [Decoder(cfg, layers, head, max_seq=max_seq, kv_fp16=True, use_graph=g) for g in (False, True, False)]
+    for d in decs:
+        for i in range(cfg["n_layers"]):
+            d.set_kv(i, *synth.make_kv_prefill(seeds["tiny"], i, cfg, past))
+        d.set_past_len(past)
+    tok, errs = 5, []
+    for st in range(6):
+        t_eager, t_graph = decs[0].step(tok), decs[1].step(tok)
+        t_trace, trace = decs[2].step_trace(tok)
+        ref = decs[2].logits()
+        spread = ref.std()
+        assert np.array_equal(decs[0].logits(), decs[1].logits()), st      # eager and graph replay: the same launches
+        err = np.abs(decs[0].logits() - ref).max() / spread
+        errs.append(err)
+        x = trace[-1, 1].astype(np.float64)
+        want_hidden = x / np.sqrt((x * x).mean() + cfg["eps"]) * head["out_norm"].astype(np.float64)
+        assert np.abs(decs[0].hidden() - want_hidden).max() <= 2e-2 * np.abs(want_hidden).max(), st
+        srt = np.sort(ref)
+        if (srt[-1] - srt[-2]) / spread > 2 * max(err, 1e-4):
+            assert t_eager == t_trace == t_graph, st
+        tok = t_trace
+    check_step_errors(errs)
+    for d in decs:
+        d.close()
+
+
 @pytest.mark.parametrize("feature", ["scale_embeddings", "ffn_gelu", "swa_window", "rope_swa_base", "post_attn_norm", "post_ffn_norm"])
 def test_gemma_features_are_not_ignored(dev, seeds, golden_gemma, feature):
     from prometorch_amd.decode import Decoder
