@@ -148,7 +148,12 @@ inline Q6KTall q6k_tall_shape(int N, int K) {
     if (K < 4096 || K > 32768) return {0, 0};   // x and its sums in LDS: 4.4 bytes per value, at most 141 KB
     if (q6k_pick_log2S(N, K / 256) != 3) return {0, 0};   // only where the row tiles would be 4 rows anyway
     const int rows_per_wg = (N + 255) / 256;
-    // up to 12 waves first (4096 x 14336 as 8 waves of two rows: 13.8 us; as 16 waves of one row: 15 us), then up to 16
+    // 13 to 15 rows per workgroup, or 16 long ones: one row per wave beats 7 or 8 waves of two rows (3584 x 18944: 15.1 against
+    // 16.6 us, 3200 x 16384: 12.7 against 14.2, 4096 x 28672: 22.4 against 23.6; 4096 x 11008 ... 14336: within 2 % either way)
+    if (rows_per_wg >= 13 && rows_per_wg <= (int)Q6K_TALL_MAX_WAVES && (rows_per_wg < 16 || K >= 16384) &&
+        K / 4 <= 16 * 64 * rows_per_wg)
+        return {rows_per_wg, 3};
+    // else up to 12 waves first (4096 x 14336 as 8 waves of two rows: 13.2 us; as 16 waves of one row: 13.0 - 13.5), then up to 16
     for (const int max_waves : {12, (int)Q6K_TALL_MAX_WAVES}) {
         for (int l = 3; l >= 2; --l) {
             const int rpw = 8 >> l;
@@ -185,10 +190,12 @@ static int q6k_launch_tall(const Q6KArgs& a, int waves, hipStream_t s) {
     // the last workgroup served ends a full arithmetic phase behind the end of the stream.  With one block at a time the
     // requests of all workgroups interleave, every workgroup's arithmetic overlaps the stream, and the other waves of a
     // SIMD cover a wave's wait (2560 x 9728: 7.5 us against 10.4 with five blocks up front; 2, 3, 4 in flight: 9.6, 9.7, 11.4).
-    // Where a lane group walks many blocks (4096 x 14336: 14 per group, two rows per wave) a second block in flight pays for
-    // itself: 15.8 us against 19.4 with one, 16.5 with three, 17.5 with five.
+    // A second block in flight pays where a lane group walks many blocks AND the CU holds few of them at a time - two rows per
+    // wave (4096 x 14336, 8 waves: 13.2 us against 14.9 with one, 13.7 with three) or fewer than ten waves of one row
+    // (2048 x 16384: 9.2 against 10.0); with ten or more waves of one row it costs (3072 x 14336: 11.7 against 10.7;
+    // 3584 x 18944, 14 waves: 15.8 against 15.1).
     const int nb = (a.K / 256 + (1 << LOG2S) - 1) >> LOG2S;
-    if (nb > 6) return q6k_launch_tall_nb<ACC, 2, LOG2S>(a, waves, s);
+    if (nb > 6 && (LOG2S == 2 || waves < 10)) return q6k_launch_tall_nb<ACC, 2, LOG2S>(a, waves, s);
     return q6k_launch_tall_nb<ACC, 1, LOG2S>(a, waves, s);
 }
 
