@@ -41,23 +41,28 @@ __global__ __launch_bounds__(Q4K_THREADS) void q4k_gemv_tall_kernel(const Q4KArg
 // Few rows, long rows (a Q4_K down projection: 2560 x 9728, as in the layers of a Q4_K_M file whose ffn_down is Q4_K): with
 // four rows per workgroup, 640 workgroups would each quantise the whole 9728-value activation vector for four rows' worth
 // of weights.  Here a workgroup is `waves` waves of one row each (the row's super-blocks strided over the wave's 8 lane
-// groups, up to three blocks of a group in flight, passes rolling), sized so that the launch is one workgroup per CU: x is quantised once per CU, a
-// half block of 16 values per thread.  Block-to-lane assignment and reduction order are those of q4k_gemv_body with 8 lane
-// groups per row, so the result is bit-identical to that kernel's.
-enum { Q4K_LONGROW_MAX_WAVES = 12 };
-template <bool ACC, int NB>
-__global__ __launch_bounds__(64 * Q4K_LONGROW_MAX_WAVES) void q4k_gemv_longrow_kernel(const uint8_t* __restrict__ W, int64_t stride,
-                                                                                   const float* __restrict__ x, float* y, int N, int K) {
+// groups, two or three blocks of a group in flight, passes rolling), sized so that the launch is one workgroup per CU (two
+// for 17 to 32 rows per CU): x is quantised once per workgroup, one to three half blocks of 16 values per thread.
+// Block-to-lane assignment and reduction order are those of q4k_gemv_body with 8 lane groups per row, so the result is
+// bit-identical to that kernel's.  Against that kernel: 3584 x 18944 15.2 -> 11.3 us, 4096 x 14336 12.0 -> 9.8,
+// 5120 x 17408 15.9 -> 14.2, 8192 x 28672 31.1 -> 28.1.
+enum { Q4K_LONGROW_MAX_WAVES = 16 };
+// XL: half blocks of x a thread quantises (rows longer than 16 values per thread: up to three rounds); MAXW: the most waves
+// an instantiation is launched with
+template <bool ACC, int NB, int XL = 1, int MAXW = 12>
+__global__ __launch_bounds__(64 * MAXW) void q4k_gemv_longrow_kernel(const uint8_t* __restrict__ W, int64_t stride,
+                                                                  const float* __restrict__ x, float* y, int N, int K) {
     extern __shared__ __align__(16) uint8_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 7, sub = lane >> 3;
+    const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wave = tid >> 6, j = lane & 7, sub = lane >> 3;
     const int nblk = K / 256;
-    const int r = blockIdx.x * ((int)blockDim.x >> 6) + wave;
+    const int r = blockIdx.x * (nthr >> 6) + wave;
     const bool live = r < N;
     const uint8_t* row = W + (int64_t)(live ? r : N - 1) * stride;
     // activation loads first (range-checked: zeros past the end), then the weights, then the Q8 arithmetic
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(x, K * 4);
-    float4 xv[4];
-    q4k_load16(rx, 16 * tid, xv);
+    float4 xv[XL][4];
+#pragma unroll
+    for (int u = 0; u < XL; ++u) q4k_load16(rx, 16 * (tid + nthr * u), xv[u]);
     issue_order_fence();
     uint4 hdr[NB], qv[NB];
 #pragma unroll
@@ -67,7 +72,11 @@ __global__ __launch_bounds__(64 * Q4K_LONGROW_MAX_WAVES) void q4k_gemv_longrow_k
         qv[u] = *reinterpret_cast<const uint4*>(p + 16 + 16 * j);
     }
     issue_order_fence();
-    if (16 * tid < K) q4k_quantize16_store<false>(xv, xv, 1.0f, 0.0f, tid, lds, K);  // lanes t, t ^ 1 share a block: both inside or both outside
+#pragma unroll
+    for (int u = 0; u < XL; ++u) {  // lanes t, t ^ 1 share a block: both inside or both outside (nthr is a multiple of 64)
+        const int unit = tid + nthr * u;
+        if (16 * unit < K) q4k_quantize16_store<false>(xv[u], xv[u], 1.0f, 0.0f, unit, lds, K);
+    }
     __syncthreads();
     // passes roll as in q4k_gemv_body: a consumed block's registers are refilled from the next pass at once
     const int nb_max = (nblk + 7) >> 3;
@@ -100,25 +109,48 @@ __global__ __launch_bounds__(64 * Q4K_LONGROW_MAX_WAVES) void q4k_gemv_longrow_k
     }
 }
 
-// waves per workgroup of that launch, or 0 when the shape is not one for it
-static int q4k_longrow_waves(int N, int K) {
-    if (K < 4096) return 0;                                        // long rows
-    const int waves = (N + 255) / 256;                            // one workgroup per CU
-    if (waves < 2 || waves > Q4K_LONGROW_MAX_WAVES) return 0;
-    if (K / 16 > 64 * waves) return 0;                            // a thread quantises one half block
-    return waves;
+// waves per workgroup and half blocks of x per thread of that launch, or waves = 0 when the shape is not one for it.  Up to
+// 16 rows per CU make one workgroup per CU, up to 32 two (each quantises x for itself).
+struct Q4KLongrow { int waves, xl; };
+static Q4KLongrow q4k_longrow_shape(int N, int K) {
+    if (K < 4096) return {0, 0};                                  // long rows
+    const int rows_per_cu = (N + 255) / 256;
+    const int per_cu = (rows_per_cu + Q4K_LONGROW_MAX_WAVES - 1) / Q4K_LONGROW_MAX_WAVES;
+    if (per_cu > 2) return {0, 0};
+    const int waves = (rows_per_cu + per_cu - 1) / per_cu;
+    if (waves < 2) return {0, 0};
+    const int xl = (K / 16 + 64 * waves - 1) / (64 * waves);
+    if (xl > 3) return {0, 0};
+    return {waves, xl};
+}
+
+template <bool ACC, int NB>
+static int q4k_launch_longrow_nb(const void* W, int64_t stride, const float* x, float* y, int N, int K, Q4KLongrow sh, hipStream_t s) {
+    const dim3 grid((N + sh.waves - 1) / sh.waves), block(64 * sh.waves);
+    const size_t lds = (size_t)q8_bytes(K);
+    const uint8_t* Wb = static_cast<const uint8_t*>(W);
+#define PTM_LR(XL, MAXW) hipLaunchKernelGGL((q4k_gemv_longrow_kernel<ACC, NB, XL, MAXW>), grid, block, lds, s, Wb, stride, x, y, N, K)
+    if (sh.waves <= 12) {
+        if (sh.xl == 1) PTM_LR(1, 12);
+        else if (sh.xl == 2) PTM_LR(2, 12);
+        else PTM_LR(3, 12);
+    } else {
+        if (sh.xl == 1) PTM_LR(1, 16);
+        else if (sh.xl == 2) PTM_LR(2, 16);
+        else PTM_LR(3, 16);
+    }
+#undef PTM_LR
+    return launch_status();
 }
 
 template <bool ACC>
-static int q4k_launch_longrow(const void* W, int64_t stride, const float* x, float* y, int N, int K, int waves, hipStream_t s) {
-    const dim3 grid((N + waves - 1) / waves), block(64 * waves);
-    const size_t lds = (size_t)q8_bytes(K);
-    const uint8_t* Wb = static_cast<const uint8_t*>(W);
-    // blocks in flight per lane group (2560 x 9728, five blocks per group: 1 / 2 / 3 / 5 in flight 7.52 / 6.96 / 6.85 / 6.97 us)
+static int q4k_launch_longrow(const void* W, int64_t stride, const float* x, float* y, int N, int K, Q4KLongrow sh, hipStream_t s) {
+    // blocks in flight per lane group: two; three for workgroups of up to ten waves (2560 x 9728, 10 waves, five blocks per
+    // group: 1 / 2 / 3 / 5 in flight 7.5 / 7.0 / 6.9 / 7.0 us; 2048 x 11008, 8 waves: 2 / 3 in flight 6.6 / 6.2;
+    // 3072 x 8192, 12 waves: 5.9 / 6.5; 3584 x 18944, 14 waves: 1 / 2 / 3 in flight 12.8 / 11.3 / 12.2)
     const int nb = (K / 256 + 7) / 8;
-    if (nb <= 2) hipLaunchKernelGGL((q4k_gemv_longrow_kernel<ACC, 2>), grid, block, lds, s, Wb, stride, x, y, N, K);
-    else hipLaunchKernelGGL((q4k_gemv_longrow_kernel<ACC, 3>), grid, block, lds, s, Wb, stride, x, y, N, K);
-    return launch_status();
+    if (nb > 2 && sh.waves <= 10) return q4k_launch_longrow_nb<ACC, 3>(W, stride, x, y, N, K, sh, s);
+    return q4k_launch_longrow_nb<ACC, 2>(W, stride, x, y, N, K, sh, s);
 }
 
 template <bool XQ8, bool NORM, bool ACC, int MODE>
@@ -196,10 +228,10 @@ int q4k_gemv_multi(int n_mat, const void* const* W, float* const* y, const int* 
     }
     if (x_is_q8) return accumulate ? q4k_launch<true, false, true, 0>(a, s) : q4k_launch<true, false, false, 0>(a, s);
     if (n_mat == 1) {
-        const int waves = q4k_longrow_waves(N[0], K);
-        if (waves > 0)
-            return accumulate ? q4k_launch_longrow<true>(W[0], stride, static_cast<const float*>(x), y[0], N[0], K, waves, s)
-                              : q4k_launch_longrow<false>(W[0], stride, static_cast<const float*>(x), y[0], N[0], K, waves, s);
+        const Q4KLongrow sh = q4k_longrow_shape(N[0], K);
+        if (sh.waves > 0)
+            return accumulate ? q4k_launch_longrow<true>(W[0], stride, static_cast<const float*>(x), y[0], N[0], K, sh, s)
+                              : q4k_launch_longrow<false>(W[0], stride, static_cast<const float*>(x), y[0], N[0], K, sh, s);
     }
     return accumulate ? q4k_launch<false, false, true, 0>(a, s) : q4k_launch<false, false, false, 0>(a, s);
 }

@@ -190,12 +190,12 @@ static int q6k_launch_tall(const Q6KArgs& a, int waves, hipStream_t s) {
     // the last workgroup served ends a full arithmetic phase behind the end of the stream.  With one block at a time the
     // requests of all workgroups interleave, every workgroup's arithmetic overlaps the stream, and the other waves of a
     // SIMD cover a wave's wait (2560 x 9728: 7.5 us against 10.4 with five blocks up front; 2, 3, 4 in flight: 9.6, 9.7, 11.4).
-    // A second block in flight pays where a lane group walks many blocks AND the CU holds few of them at a time - two rows per
-    // wave (4096 x 14336, 8 waves: 13.2 us against 14.9 with one, 13.7 with three) or fewer than ten waves of one row
-    // (2048 x 16384: 9.2 against 10.0); with ten or more waves of one row it costs (3072 x 14336: 11.7 against 10.7;
-    // 3584 x 18944, 14 waves: 15.8 against 15.1).
+    // A second block in flight pays where the CU holds few blocks at a time - two rows per wave and many blocks per lane group
+    // (4096 x 14336, 8 waves: 13.2 us against 14.9 with one, 13.7 with three), or fewer than ten waves of one row
+    // (2048 x 16384: 9.2 against 10.0; 2048 x 11008: 7.6 against 8.1); with ten or more waves of one row it costs
+    // (3072 x 14336: 11.7 against 10.7; 3584 x 18944, 14 waves: 15.8 against 15.1; 2560 x 10240: 9.4 against 7.8).
     const int nb = (a.K / 256 + (1 << LOG2S) - 1) >> LOG2S;
-    if (nb > 6 && (LOG2S == 2 || waves < 10)) return q6k_launch_tall_nb<ACC, 2, LOG2S>(a, waves, s);
+    if ((LOG2S == 2 && nb > 6) || (LOG2S == 3 && waves < 10 && nb >= 4)) return q6k_launch_tall_nb<ACC, 2, LOG2S>(a, waves, s);
     return q6k_launch_tall_nb<ACC, 1, LOG2S>(a, waves, s);
 }
 

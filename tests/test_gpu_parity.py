@@ -181,6 +181,24 @@ def test_q4k_gemv_tall_forms_agree(dev, po, seeds):
     assert np.array_equal(bits(ya), bits(y0 + y))
 
 
+@pytest.mark.parametrize("N,K", [(2560, 9728), (3584, 18944), (4099, 14336), (5120, 25600), (2001, 11008)])
+def test_q4k_gemv_long_rows_equal_the_general_kernel(dev, N, K):
+    """fp32 x takes the few-long-rows kernel (x quantised once per workgroup), Q8 blocks handed in take the general one:
+    the same block-to-lane assignment and reduction order, so the same bits - with 8 to 16 waves, one to three half blocks
+    of x per thread, one and two workgroups per CU."""
+    r = synth.rng_for(37, N, K)
+    W = synth.make_q4k(r, N, K)
+    x = synth.make_x(r, K)
+    y = gpu_gemv(12, W, x)
+    Wd, xd = cu(W), cu(x)
+    y2 = torch.empty(N, device="cuda")
+    q8 = torch.empty(ops.q8_bytes(K), dtype=torch.uint8, device="cuda")
+    ops.launch_quantize_q8(xd, q8, K)
+    ops.launch_q4km_q8_gemv(Wd, q8, y2, K, N, W.shape[1])
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y2.cpu().numpy()), bits(y))
+
+
 def test_q4k_gemv_long_rows_accumulate(dev, po, seeds):
     """The few-long-rows Q4_K kernel (2560 x 9728) in its accumulating form: y0 + W.x, bit for bit the sum of y0 and the plain
     form's result."""
@@ -202,7 +220,10 @@ def test_q4k_gemv_long_rows_accumulate(dev, po, seeds):
                                     (12, 40007, 2560), (12, 50001, 512), (12, 45013, 1280), (12, 41000, 768),
                                     # few long Q4_K rows (a Q4_K down projection): one row per wave, x quantised once per
                                     # workgroup; ragged last workgroup, 2 / 5 blocks per lane group, 8 to 12 waves
-                                    (12, 2001, 9728), (12, 3000, 10240), (12, 2560, 6144)])
+                                    (12, 2001, 9728), (12, 3000, 10240), (12, 2560, 6144),
+                                    # the same with 13 to 16 waves, with two and three half blocks of x per thread, and with
+                                    # two workgroups per CU (17 to 32 rows per CU)
+                                    (12, 3584, 18944), (12, 4096, 4096), (12, 4099, 14336), (12, 5120, 25600), (12, 6007, 8192)])
 def test_gemv_shapes_vs_oracle(dev, po, qt, N, K):
     r = synth.rng_for(31, qt, N, K)
     W = synth.make_weight(r, qt, N, K)
