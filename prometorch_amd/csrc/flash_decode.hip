@@ -69,6 +69,32 @@ struct FdFuse {
     int add_one, rope_interleaved;
 };
 
+// Raw values of one item of the FUSED prologue (a query head or the new k row) as a lane holds them: rotation pairs
+// lane and lane + 64 (clamped into the head where the head has fewer pairs), their norm weights, the rotation row, and the
+// v row's values at the same places.
+struct FdItem { float x0[2], x1[2], n0[2], n1[2], c[2], s[2], v0[2], v1[2]; };
+template <int HD>
+__device__ __forceinline__ FdItem fd_item_load(const float* src, const float* nw, const float* cs, const float* vrow,
+                                               int interleaved, int lane) {
+    constexpr int HALF = HD / 2;
+    const float* nwp = nw ? nw : src;  // a valid address either way; unused without norm weights
+    FdItem e;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int t = min(lane + 64 * j, HALF - 1);
+        const int i0 = interleaved ? 2 * t : t, i1 = interleaved ? 2 * t + 1 : t + HALF;
+        e.x0[j] = src[i0];
+        e.x1[j] = src[i1];
+        e.n0[j] = nwp[i0];
+        e.n1[j] = nwp[i1];
+        e.c[j] = cs[t];
+        e.s[j] = cs[HALF + t];
+        e.v0[j] = vrow[t];
+        e.v1[j] = vrow[t + HALF];
+    }
+    return e;
+}
+
 // grid (max_splits, n_kv_heads); G = query heads per kv head; HD = head_dim.  FUSED: Q holds the raw projections and
 // the caches are appended to (the one-launch form for heads wider than the fused kernel further down covers).
 template <bool KV16, int HD, int G, bool FUSED = false>
@@ -111,6 +137,20 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     const int64_t col = (int64_t)kvh * HD + dl * 8;
     const int64_t past = total - 1;
 
+    // FUSED: what this wave's first item of the prologue needs (wave w prepares query heads w, w + 4, ..., then, in the
+    // workgroup that owns the new position, the new k row; a lane owns rotation pairs lane and lane + 64) is requested
+    // FIRST and unconditionally, from addresses that are valid for every wave: loads return in order, so behind the cache
+    // rows these few values would wait for all of them, and under a branch the compiler would wait for everything in flight.
+    static_assert(!FUSED || HD == 256, "the fused prologue is laid out for heads of 256 (two rotation pairs per lane)");
+    constexpr int HALF = HD / 2;
+    FdItem first{};
+    if constexpr (FUSED) {
+        const bool k_item = wave >= G;  // waves past the query heads fetch the k row (used by the owner's wave G only)
+        first = fd_item_load<HD>(k_item ? f.K + (int64_t)kvh * HD : Q + (int64_t)(kvh * G + wave) * HD, k_item ? f.kw : f.qw,
+                                 f.rope + past * HD, f.V + (int64_t)kvh * HD, f.rope_interleaved, lane);
+        issue_order_fence();
+    }
+
     // ---- all K and V rows of the chunk are requested up front: one HBM round trip (FUSED: the new position's row is
     // not in the cache yet, it comes from LDS below) ----
     float kreg[NPASS][8], vreg[NPASS][8];
@@ -125,69 +165,61 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
 
     float q[G][8];
     if constexpr (FUSED) {
-        constexpr int HALF = HD / 2;
+        issue_order_fence();
         const bool owner = past >= t0 && past < t0 + FD_CHUNK;
-        const float* cs = f.rope + past * HD;
         const float one = f.add_one ? 1.0f : 0.0f;
-        // wave w prepares heads w, w + 4, ...: the G query heads, then (owner only) the new k row; a lane owns rotation
-        // pairs lane and lane + 64
-        for (int it = wave; it < G + (owner ? 1 : 0); it += 4) {
+        // norm + rotation of one item from its loaded values; query heads go to s_q, the k row (with the v row) to the cache
+        // and to s_new
+        auto finish = [&](int it, FdItem& e) {
             const bool is_k = it == G;
-            const float* src = is_k ? f.K + (int64_t)kvh * HD : Q + (int64_t)(kvh * G + it) * HD;
-            const float* nw = is_k ? f.kw : f.qw;
-            float x0[2], x1[2];
-            int i0[2], i1[2];
-            bool on[2];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int t = lane + 64 * j;
-                on[j] = t < HALF;
-                i0[j] = f.rope_interleaved ? 2 * t : t;
-                i1[j] = f.rope_interleaved ? 2 * t + 1 : t + HALF;
-                x0[j] = on[j] ? src[i0[j]] : 0.0f;
-                x1[j] = on[j] ? src[i1[j]] : 0.0f;
-            }
-            if (nw) {
-                float ss = fmaf(x0[0], x0[0], 0.0f);
-                ss = fmaf(x1[0], x1[0], ss);
-                ss = fmaf(x0[1], x0[1], ss);
-                ss = fmaf(x1[1], x1[1], ss);
+            if ((is_k ? f.kw : f.qw) != nullptr) {
+                float ss = fmaf(e.x0[0], e.x0[0], 0.0f);
+                ss = fmaf(e.x1[0], e.x1[0], ss);
+                ss = fmaf(e.x0[1], e.x0[1], ss);
+                ss = fmaf(e.x1[1], e.x1[1], ss);
                 ss = sum64(ss);
                 const float rs = 1.0f / sqrtf(ss / (float)HD + f.eps);
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    if (on[j]) {
-                        x0[j] = x0[j] * rs * (nw[i0[j]] + one);
-                        x1[j] = x1[j] * rs * (nw[i1[j]] + one);
-                    }
+                for (int j = 0; j < 2; ++j) {
+                    e.x0[j] = e.x0[j] * rs * (e.n0[j] + one);
+                    e.x1[j] = e.x1[j] * rs * (e.n1[j] + one);
+                }
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                if (!on[j]) continue;
                 const int t = lane + 64 * j;
-                const float c = cs[t], sn = cs[HALF + t];
-                float r0 = fmaf(x0[j], c, -(x1[j] * sn)), r1 = fmaf(x0[j], sn, x1[j] * c);
+                if (t >= HALF) continue;
+                const int i0 = f.rope_interleaved ? 2 * t : t, i1 = f.rope_interleaved ? 2 * t + 1 : t + HALF;
+                float r0 = fmaf(e.x0[j], e.c[j], -(e.x1[j] * e.s[j])), r1 = fmaf(e.x0[j], e.s[j], e.x1[j] * e.c[j]);
                 if (!is_k) {
-                    s_q[it][i0[j]] = r0;
-                    s_q[it][i1[j]] = r1;
+                    s_q[it][i0] = r0;
+                    s_q[it][i1] = r1;
                 } else {
                     const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;
-                    float v0 = f.V[(int64_t)kvh * HD + t], v1 = f.V[(int64_t)kvh * HD + t + HALF];
+                    float v0 = e.v0[j], v1 = e.v1[j];
                     if constexpr (KV16) {
                         const __half h0 = __float2half_rn(r0), h1 = __float2half_rn(r1), g0 = __float2half_rn(v0), g1 = __float2half_rn(v1);
                         __half* kc = static_cast<__half*>(Kc) + rowoff;
                         __half* vc = static_cast<__half*>(Vc) + rowoff;
-                        kc[i0[j]] = h0; kc[i1[j]] = h1; vc[t] = g0; vc[t + HALF] = g1;
+                        kc[i0] = h0; kc[i1] = h1; vc[t] = g0; vc[t + HALF] = g1;
                         r0 = __half2float(h0); r1 = __half2float(h1); v0 = __half2float(g0); v1 = __half2float(g1);
                     } else {
                         float* kc = static_cast<float*>(Kc) + rowoff;
                         float* vc = static_cast<float*>(Vc) + rowoff;
-                        kc[i0[j]] = r0; kc[i1[j]] = r1; vc[t] = v0; vc[t + HALF] = v1;
+                        kc[i0] = r0; kc[i1] = r1; vc[t] = v0; vc[t + HALF] = v1;
                     }
-                    s_new[0][i0[j]] = r0; s_new[0][i1[j]] = r1;
+                    s_new[0][i0] = r0; s_new[0][i1] = r1;
                     s_new[1][t] = v0; s_new[1][t + HALF] = v1;
                 }
             }
+        };
+        const int n_items = G + (owner ? 1 : 0);
+        if (wave < n_items) finish(wave, first);
+        for (int it = wave + 4; it < n_items; it += 4) {  // more than three query heads per kv head: further items, fetched here
+            const bool is_k = it == G;
+            FdItem e = fd_item_load<HD>(is_k ? f.K + (int64_t)kvh * HD : Q + (int64_t)(kvh * G + it) * HD, is_k ? f.kw : f.qw,
+                                        f.rope + past * HD, f.V + (int64_t)kvh * HD, f.rope_interleaved, lane);
+            finish(it, e);
         }
         __syncthreads();
 #pragma unroll
