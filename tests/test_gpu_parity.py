@@ -181,11 +181,12 @@ def test_q4k_gemv_tall_forms_agree(dev, po, seeds):
     assert np.array_equal(bits(ya), bits(y0 + y))
 
 
-@pytest.mark.parametrize("N,K", [(2560, 9728), (3584, 18944), (4099, 14336), (5120, 25600), (2001, 11008)])
+@pytest.mark.parametrize("N,K", [(2560, 9728), (3584, 18944), (4099, 14336), (5120, 25600), (2001, 11008), (2560, 4096)])
 def test_q4k_gemv_long_rows_equal_the_general_kernel(dev, N, K):
-    """fp32 x takes the few-long-rows kernel (x quantised once per workgroup), Q8 blocks handed in take the general one:
-    the same block-to-lane assignment and reduction order, so the same bits - with 8 to 16 waves, one to three half blocks
-    of x per thread, one and two workgroups per CU."""
+    """One matrix of few long rows with fp32 x takes the one-row-per-wave kernel (x quantised once per workgroup); with Q8
+    blocks handed in, or as the first of three matrices of one launch, the same rows take the general kernel.  Same
+    block-to-lane assignment and reduction order, so the same bits - with 8 to 16 waves, one to three half blocks of x per
+    thread, one and two workgroups per CU."""
     r = synth.rng_for(37, N, K)
     W = synth.make_q4k(r, N, K)
     x = synth.make_x(r, K)
@@ -195,8 +196,16 @@ def test_q4k_gemv_long_rows_equal_the_general_kernel(dev, N, K):
     q8 = torch.empty(ops.q8_bytes(K), dtype=torch.uint8, device="cuda")
     ops.launch_quantize_q8(xd, q8, K)
     ops.launch_q4km_q8_gemv(Wd, q8, y2, K, N, W.shape[1])
+    yq, yk, yv = torch.empty(N, device="cuda"), torch.empty(1, device="cuda"), torch.empty(1, device="cuda")
+    ops.launch_q4km_fused_qkv_gemv(Wd, Wd[:1], Wd[:1], xd, yq, yk, yv, K, N, 1, 1, W.shape[1])
     torch.cuda.synchronize()
     assert np.array_equal(bits(y2.cpu().numpy()), bits(y))
+    assert np.array_equal(bits(yq.cpu().numpy()), bits(y))
+    y0 = synth.make_x(r, N)
+    y3 = cu(y0)
+    ops.launch_q4km_q8_gemv(Wd, q8, y3, K, N, W.shape[1], accumulate=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(y3.cpu().numpy()), bits(y0 + y))
 
 
 def test_q4k_gemv_long_rows_accumulate(dev, po, seeds):
