@@ -143,7 +143,8 @@ def test_reference_call_sites_compile_against_the_shim(tmp_path):
 
 
 def test_shim_context_setter_and_integration_snippet_compile(tmp_path):
-    """The snippet INTEGRATION.md shows (context set from the model's own fields inside a member function) compiles."""
+    """How a maintainer of the reference sets the shim's context: from the model's own fields, inside a member function, in front
+    of the launcher calls.  That snippet compiles."""
     if not (shutil.which("g++") and os.path.isdir("/opt/rocm/include")):
         pytest.skip("no g++ / ROCm headers")
     f = tmp_path / "ctx.cpp"
