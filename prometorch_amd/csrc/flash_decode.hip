@@ -248,6 +248,10 @@ __global__ __launch_bounds__(FD_THREADS) void flash_decode_partial_kernel(
     for (int pass = 0; pass < NPASS; ++pass) {
         const int tl = pass * PPB + wave * PPW + pl;
         const bool valid = t0 + tl < total && t0 + tl >= t_begin;
+        if (!valid) {  // a position that does not count holds a clamped row, possibly never written: 0 * garbage must not be NaN
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vreg[pass][i] = 0.0f;
+        }
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float d = 0.0f;
@@ -773,7 +777,8 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     constexpr int VP = HD * 2 + 64;      // LDS pitch of a V row: the four rows of a transposing read fall on different banks
     constexpr int GP = G <= 4 ? 4 : 8;   // head slots of the wave partials
     constexpr int CH = 64 * TPW;         // positions per workgroup
-    static_assert(G >= 1 && G <= 8 && (HD == 64 || HD == 128) && (TPW == 1 || TPW == 2), "shape");
+    constexpr int PP = (HALF + 63) / 64; // rotation pairs a lane holds in the prologue: pairs lane and (heads of 256) lane + 64
+    static_assert(G >= 1 && G <= 8 && (HD == 64 || HD == 128 || (HD == 256 && G <= 4)) && (TPW == 1 || TPW == 2), "shape");
     __shared__ __align__(16) _Float16 s_qh[G][HD];
     __shared__ __align__(16) _Float16 s_ql[G][HD];
     __shared__ __align__(16) _Float16 s_nk[HD];
@@ -801,8 +806,13 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     }
     const int j = lane & 15, rg = lane >> 4;
     const int kv_dim = a.n_kv_heads * HD;
-    const bool on = lane < HALF;
-    const int lh = lane & (HALF - 1);
+    bool on[PP];
+    int lh[PP];
+#pragma unroll
+    for (int p = 0; p < PP; ++p) {
+        on[p] = lane + 64 * p < HALF;
+        lh[p] = (lane + 64 * p) & (HALF - 1);
+    }
     const bool has_norm = a.qw != nullptr;
     const int64_t wt0 = t0 + (int64_t)wave * (16 * TPW);            // first position of this wave
     const bool owner = past >= wt0 && past < wt0 + 16 * TPW;       // wave-uniform: this wave's tiles hold the new position
@@ -811,30 +821,48 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     const float* cs = a.rope + past * HD;
     const float* qwp = has_norm ? a.qw : a.Q;  // a valid address either way; unused without norm weights
     const float* kwp = has_norm ? a.kw : a.Q;
-    const int i0 = a.rope_interleaved ? 2 * lh : lh, i1 = a.rope_interleaved ? 2 * lh + 1 : lh + HALF;
+    int i0[PP], i1[PP];
+#pragma unroll
+    for (int p = 0; p < PP; ++p) {
+        i0[p] = a.rope_interleaved ? 2 * lh[p] : lh[p];
+        i1[p] = a.rope_interleaved ? 2 * lh[p] + 1 : lh[p] + HALF;
+    }
     constexpr int NQ = (G + 3) / 4;  // query heads a wave prepares: wave, wave + 4
-    float qx0[NQ], qx1[NQ], qb0[NQ], qb1[NQ];
+    float qx0[NQ][PP], qx1[NQ][PP], qb0[NQ][PP], qb1[NQ][PP];
 #pragma unroll
     for (int n = 0; n < NQ; ++n) {
         const int g = wave + 4 * n < G ? wave + 4 * n : 0;
         const float* src = a.Q + (int64_t)(kvh * G + g) * HD;
-        qx0[n] = src[i0];
-        qx1[n] = src[i1];
-        if constexpr (BIAS) {
-            qb0[n] = a.qb[(kvh * G + g) * HD + i0];
-            qb1[n] = a.qb[(kvh * G + g) * HD + i1];
+#pragma unroll
+        for (int p = 0; p < PP; ++p) {
+            qx0[n][p] = src[i0[p]];
+            qx1[n][p] = src[i1[p]];
+            if constexpr (BIAS) {
+                qb0[n][p] = a.qb[(kvh * G + g) * HD + i0[p]];
+                qb1[n][p] = a.qb[(kvh * G + g) * HD + i1[p]];
+            }
         }
     }
-    const float qn0 = qwp[i0], qn1 = qwp[i1], kn0 = kwp[i0], kn1 = kwp[i1];
-    const float rc = cs[lh], rsn = cs[HALF + lh];
-    float kx0 = a.K[(int64_t)kvh * HD + i0], kx1 = a.K[(int64_t)kvh * HD + i1];
-    float vx0 = a.V[(int64_t)kvh * HD + lh], vx1 = a.V[(int64_t)kvh * HD + lh + HALF];
-    float kb0 = 0.0f, kb1 = 0.0f, vb0 = 0.0f, vb1 = 0.0f;
-    if constexpr (BIAS) {
-        kb0 = a.kb[kvh * HD + i0];
-        kb1 = a.kb[kvh * HD + i1];
-        vb0 = a.vb[kvh * HD + lh];
-        vb1 = a.vb[kvh * HD + lh + HALF];
+    float qn0[PP], qn1[PP], kn0[PP], kn1[PP], rc[PP], rsn[PP], kx0[PP], kx1[PP], vx0[PP], vx1[PP], kb0[PP], kb1[PP], vb0[PP], vb1[PP];
+#pragma unroll
+    for (int p = 0; p < PP; ++p) {
+        qn0[p] = qwp[i0[p]];
+        qn1[p] = qwp[i1[p]];
+        kn0[p] = kwp[i0[p]];
+        kn1[p] = kwp[i1[p]];
+        rc[p] = cs[lh[p]];
+        rsn[p] = cs[HALF + lh[p]];
+        kx0[p] = a.K[(int64_t)kvh * HD + i0[p]];
+        kx1[p] = a.K[(int64_t)kvh * HD + i1[p]];
+        vx0[p] = a.V[(int64_t)kvh * HD + lh[p]];
+        vx1[p] = a.V[(int64_t)kvh * HD + lh[p] + HALF];
+        kb0[p] = kb1[p] = vb0[p] = vb1[p] = 0.0f;
+        if constexpr (BIAS) {
+            kb0[p] = a.kb[kvh * HD + i0[p]];
+            kb1[p] = a.kb[kvh * HD + i1[p]];
+            vb0[p] = a.vb[kvh * HD + lh[p]];
+            vb1[p] = a.vb[kvh * HD + lh[p] + HALF];
+        }
     }
     issue_order_fence();
     // ---- ... then the cached K/V rows of this wave's tiles (the new position is not cached: clamp below it) ----
@@ -867,48 +895,74 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
     for (int n = 0; n < NQ; ++n) {
         const int g = wave + 4 * n;
         if (g >= G) continue;  // wave-uniform
-        if constexpr (BIAS) { qx0[n] += qb0[n]; qx1[n] += qb1[n]; }
-        float x0 = on ? qx0[n] : 0.0f, x1 = on ? qx1[n] : 0.0f;
+        float x0[PP], x1[PP];
+        float ss = 0.0f;
+#pragma unroll
+        for (int p = 0; p < PP; ++p) {
+            if constexpr (BIAS) { qx0[n][p] += qb0[n][p]; qx1[n][p] += qb1[n][p]; }
+            x0[p] = on[p] ? qx0[n][p] : 0.0f;
+            x1[p] = on[p] ? qx1[n][p] : 0.0f;
+            ss = fmaf(x0[p], x0[p], ss);
+            ss = fmaf(x1[p], x1[p], ss);
+        }
         if (has_norm) {
-            float ss = fmaf(x0, x0, 0.0f);
-            ss = fmaf(x1, x1, ss);
             ss = sum64(ss);
             const float rs = fast_rsqrt(ss * (1.0f / (float)HD) + a.eps);
-            x0 = x0 * rs * (qn0 + one);
-            x1 = x1 * rs * (qn1 + one);
+#pragma unroll
+            for (int p = 0; p < PP; ++p) {
+                x0[p] = x0[p] * rs * (qn0[p] + one);
+                x1[p] = x1[p] * rs * (qn1[p] + one);
+            }
         }
-        if (on) {
-            const float r0 = fmaf(x0, rc, -(x1 * rsn)) * qs, r1 = fmaf(x0, rsn, x1 * rc) * qs;
-            const _Float16 h0 = (_Float16)r0, h1 = (_Float16)r1;
-            s_qh[g][i0] = h0;
-            s_qh[g][i1] = h1;
-            s_ql[g][i0] = (_Float16)(r0 - (float)h0);
-            s_ql[g][i1] = (_Float16)(r1 - (float)h1);
+#pragma unroll
+        for (int p = 0; p < PP; ++p) {
+            if (on[p]) {
+                const float r0 = fmaf(x0[p], rc[p], -(x1[p] * rsn[p])) * qs, r1 = fmaf(x0[p], rsn[p], x1[p] * rc[p]) * qs;
+                const _Float16 h0 = (_Float16)r0, h1 = (_Float16)r1;
+                s_qh[g][i0[p]] = h0;
+                s_qh[g][i1[p]] = h1;
+                s_ql[g][i0[p]] = (_Float16)(r0 - (float)h0);
+                s_ql[g][i1[p]] = (_Float16)(r1 - (float)h1);
+            }
         }
     }
-    __half nv0 = __float2half_rn(0.0f), nv1 = nv0;
+    __half nv0[PP], nv1[PP];
+#pragma unroll
+    for (int p = 0; p < PP; ++p) nv0[p] = nv1[p] = __float2half_rn(0.0f);
     if (owner) {  // the new K row: normalised, rotated, rounded as the cache holds it; the new V row
-        if constexpr (BIAS) { kx0 += kb0; kx1 += kb1; vx0 += vb0; vx1 += vb1; }
-        float x0 = on ? kx0 : 0.0f, x1 = on ? kx1 : 0.0f;
+        float x0[PP], x1[PP];
+        float ss = 0.0f;
+#pragma unroll
+        for (int p = 0; p < PP; ++p) {
+            if constexpr (BIAS) { kx0[p] += kb0[p]; kx1[p] += kb1[p]; vx0[p] += vb0[p]; vx1[p] += vb1[p]; }
+            x0[p] = on[p] ? kx0[p] : 0.0f;
+            x1[p] = on[p] ? kx1[p] : 0.0f;
+            ss = fmaf(x0[p], x0[p], ss);
+            ss = fmaf(x1[p], x1[p], ss);
+        }
         if (has_norm) {
-            float ss = fmaf(x0, x0, 0.0f);
-            ss = fmaf(x1, x1, ss);
             ss = sum64(ss);
             const float rs = fast_rsqrt(ss * (1.0f / (float)HD) + a.eps);
-            x0 = x0 * rs * (kn0 + one);
-            x1 = x1 * rs * (kn1 + one);
+#pragma unroll
+            for (int p = 0; p < PP; ++p) {
+                x0[p] = x0[p] * rs * (kn0[p] + one);
+                x1[p] = x1[p] * rs * (kn1[p] + one);
+            }
         }
-        const __half h0 = __float2half_rn(fmaf(x0, rc, -(x1 * rsn))), h1 = __float2half_rn(fmaf(x0, rsn, x1 * rc));
-        nv0 = __float2half_rn(vx0);
-        nv1 = __float2half_rn(vx1);
-        if (on) {
-            const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;
-            static_cast<__half*>(a.Kc)[rowoff + i0] = h0;
-            static_cast<__half*>(a.Kc)[rowoff + i1] = h1;
-            static_cast<__half*>(a.Vc)[rowoff + lh] = nv0;
-            static_cast<__half*>(a.Vc)[rowoff + lh + HALF] = nv1;
-            reinterpret_cast<__half*>(s_nk)[i0] = h0;
-            reinterpret_cast<__half*>(s_nk)[i1] = h1;
+        const int64_t rowoff = past * kv_dim + (int64_t)kvh * HD;
+#pragma unroll
+        for (int p = 0; p < PP; ++p) {
+            const __half h0 = __float2half_rn(fmaf(x0[p], rc[p], -(x1[p] * rsn[p]))), h1 = __float2half_rn(fmaf(x0[p], rsn[p], x1[p] * rc[p]));
+            nv0[p] = __float2half_rn(vx0[p]);
+            nv1[p] = __float2half_rn(vx1[p]);
+            if (on[p]) {
+                static_cast<__half*>(a.Kc)[rowoff + i0[p]] = h0;
+                static_cast<__half*>(a.Kc)[rowoff + i1[p]] = h1;
+                static_cast<__half*>(a.Vc)[rowoff + lh[p]] = nv0[p];
+                static_cast<__half*>(a.Vc)[rowoff + lh[p] + HALF] = nv1[p];
+                reinterpret_cast<__half*>(s_nk)[i0[p]] = h0;
+                reinterpret_cast<__half*>(s_nk)[i1[p]] = h1;
+            }
         }
     }
     __syncthreads();  // the query heads come from the other waves (the new row stays within its wave)
@@ -964,10 +1018,15 @@ __global__ __launch_bounds__(FD_THREADS) void attn_decode_mfma_kernel(const Attn
             }
             *reinterpret_cast<uint4*>(&s_v[wave][u][row * VP + 16 * (lane % LPR)]) = v;
         }
-        if (owner && past >= tt0 && past < tt0 + 16 && on) {
+        if (owner && past >= tt0 && past < tt0 + 16) {
             __half* vrow = reinterpret_cast<__half*>(&s_v[wave][u][(int)(past - tt0) * VP]);
-            vrow[lh] = nv0;
-            vrow[lh + HALF] = nv1;
+#pragma unroll
+            for (int p = 0; p < PP; ++p) {
+                if (on[p]) {
+                    vrow[lh[p]] = nv0[p];
+                    vrow[lh[p] + HALF] = nv1[p];
+                }
+            }
         }
     }
     // the V^T fragments are requested before the softmax arithmetic, which covers the LDS round trip
@@ -1330,16 +1389,26 @@ static int attn_mfma_long_launch_g(int G, dim3 grid, hipStream_t s, const AttnAr
 template <int HD, int TPW, bool BIAS>
 static int attn_mfma_launch_g(int G, dim3 grid, hipStream_t s, const AttnArgs& a) {
 #define PTM_AM(GG) hipLaunchKernelGGL((attn_decode_mfma_kernel<HD, GG, TPW, BIAS>), grid, dim3(FD_THREADS), 0, s, a)
-    switch (G) {
-        case 1: PTM_AM(1); break;
-        case 2: PTM_AM(2); break;
-        case 3: PTM_AM(3); break;
-        case 4: PTM_AM(4); break;
-        case 5: PTM_AM(5); break;
-        case 6: PTM_AM(6); break;
-        case 7: PTM_AM(7); break;
-        case 8: PTM_AM(8); break;
-        default: return PTM_E_UNSUPPORTED;
+    if constexpr (HD == 256) {  // up to four query heads per kv head (the wave partials of more would not fit the static LDS)
+        switch (G) {
+            case 1: PTM_AM(1); break;
+            case 2: PTM_AM(2); break;
+            case 3: PTM_AM(3); break;
+            case 4: PTM_AM(4); break;
+            default: return PTM_E_UNSUPPORTED;
+        }
+    } else {
+        switch (G) {
+            case 1: PTM_AM(1); break;
+            case 2: PTM_AM(2); break;
+            case 3: PTM_AM(3); break;
+            case 4: PTM_AM(4); break;
+            case 5: PTM_AM(5); break;
+            case 6: PTM_AM(6); break;
+            case 7: PTM_AM(7); break;
+            case 8: PTM_AM(8); break;
+            default: return PTM_E_UNSUPPORTED;
+        }
     }
 #undef PTM_AM
     return launch_status();
@@ -1469,8 +1538,21 @@ int ptm_attn_decode_fused_bias(const float* Q, const float* K, const float* V, c
     if (n_heads <= 0 || n_kv_heads <= 0 || max_seq <= 0 || (n_heads % n_kv_heads) != 0) return PTM_E_SHAPE;
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return PTM_E_UNSUPPORTED;
     if (!aligned16(K_cache) || !aligned16(V_cache) || !aligned16(partial_O) || !aligned16(O)) return PTM_E_ALIGN;
+    if (head_dim == 256 && kv_fp16 && !bias && n_heads / n_kv_heads <= 4 && ptm_flash_decode_num_splits(max_seq) <= FD_LONG_SPLITS) {
+        // heads of 256 (gemma3), fp16 cache of up to 4096 positions: the matrix-core kernel, two rotation pairs per lane
+        if (o_q8 && (reinterpret_cast<uintptr_t>(o_q8) & 15u)) return PTM_E_ALIGN;
+        AttnArgs a256{Q, K, V, q_norm_w, k_norm_w, rope_table, K_cache, V_cache, partial_O, partial_lse, partial_max,
+                      d_past_len, n_heads, n_kv_heads, max_seq, add_one, scale, eps, rope_interleaved ? 1 : 0,
+                      window > 0 ? window : 0, nullptr, nullptr, nullptr};
+        const dim3 grid256(ptm_flash_decode_num_splits(max_seq), n_kv_heads);
+        const int rc256 = attn_mfma_launch_g<256, 1, false>(n_heads / n_kv_heads, grid256, as_stream(stream), a256);
+        if (rc256 != PTM_OK) return rc256;
+        return fd_merge(head_dim, n_heads, as_stream(stream), partial_O, partial_lse, partial_max, O, d_past_len, max_seq,
+                        static_cast<uint8_t*>(o_q8), 0, FD_CHUNK, 1);
+    }
     if (head_dim == 256) {
-        // heads this wide (gemma3): the plain split-KV kernel with the norm / rotation / append prologue in front
+        // heads this wide with an fp32 cache, more query heads per kv head or a longer cache: the plain split-KV kernel with
+        // the norm / rotation / append prologue in front
         if (o_q8 && (reinterpret_cast<uintptr_t>(o_q8) & 15u)) return PTM_E_ALIGN;
         const FdFuse f{K, V, q_norm_w, k_norm_w, rope_table, eps, add_one, rope_interleaved ? 1 : 0};
         const dim3 grid256(ptm_flash_decode_num_splits(max_seq), n_kv_heads);

@@ -149,7 +149,9 @@ def test_rows_rotation_interleaved_vs_reference_golden(dev, po, seeds, golden_ll
 
 
 @pytest.mark.parametrize("kv_fp16", [True, False])
-@pytest.mark.parametrize("nh,nkv,hd,past", [(32, 8, 128, 2048), (4, 2, 64, 19), (8, 8, 128, 0), (16, 2, 64, 63), (32, 8, 128, 14)])
+@pytest.mark.parametrize("nh,nkv,hd,past", [(32, 8, 128, 2048), (4, 2, 64, 19), (8, 8, 128, 0), (16, 2, 64, 63), (32, 8, 128, 14),
+                                            # heads of 256: two rotation pairs per lane in the matrix-core kernel
+                                            (4, 2, 256, 63), (4, 1, 256, 200), (3, 3, 256, 0)])
 def test_attn_decode_fused_llama_style_vs_oracle(dev, po, kv_fp16, nh, nkv, hd, past):
     """No norm weights + interleaved rotation + KV append + attention + merge, three tokens in a row."""
     max_seq = ((past + 3 + 63) // 64 + 1) * 64
