@@ -64,7 +64,7 @@ def test_gelu_mul_rms_norm_add_and_scale(dev, po):
                                                   (8, 4, 256, 2048, 1024), (2, 1, 256, 19, 8), (8, 4, 256, 30, 0), (6, 2, 256, 62, 0),
                                                   # heads of 256 with 1 and 4 query heads per kv head (matrix-core kernel, chunk
                                                   # edge crossed), with 5 (the vector kernel) and beyond 4096 positions (the same)
-                                                  (4, 4, 256, 127, 0), (4, 1, 256, 63, 40), (5, 1, 256, 70, 0), (2, 1, 256, 5000, 300),
+                                                  (4, 4, 256, 127, 0), (4, 1, 256, 63, 40), (5, 1, 256, 70, 0), (2, 1, 256, 5000, 300), (4, 1, 256, 8190, 0),
                                                   # caches beyond 4096 positions: the looping kernel (several chunks per workgroup,
                                                   # some or all of them in front of the window)
                                                   (8, 2, 128, 9000, 1024), (4, 2, 64, 5000, 100), (8, 4, 128, 8200, 7000)])
