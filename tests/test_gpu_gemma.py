@@ -217,7 +217,7 @@ def test_gemma_decode_fp16_kv_vs_oracle_and_chained_greedy(dev, po, seeds, past)
     dec2.close()
 
 
-@pytest.mark.parametrize("shape", ["tiny", "4b_layers"])
+@pytest.mark.parametrize("shape", ["tiny", "4b_layers", "hidden_4096", "hidden_4352"])
 def test_step_that_defers_the_post_ffn_norm_matches_the_traced_step(dev, seeds, shape):
     """A plain step leaves the post-norm and residual add of a layer's feed-forward branch to the prologue of the next layer's
     q / k / v launch; a traced step runs each as a launch of its own.  Same state, same token: the logits agree to the
@@ -226,6 +226,18 @@ def test_step_that_defers_the_post_ffn_norm_matches_the_traced_step(dev, seeds, 
     from prometorch_amd.decode import Decoder
     if shape == "tiny":
         cfg, layers, head = synth.tiny_gemma(seeds["tiny"])
+        past, max_seq = 19, 64
+    elif shape.startswith("hidden_"):
+        # 4096 values: the longest vector the q / k / v prologue applies the post-norm to; 4352: one block beyond, every
+        # post-norm a launch of its own (the two step forms then run the same launches)
+        cfg = dict(synth.TINY, hidden=int(shape[7:]), n_layers=3, scale_embeddings=True, ffn_gelu=True, swa_window=8,
+                   swa_pattern=3, rope_swa_base=1.0e4, rope_scale=8.0)
+        layers = [synth.make_layer(seeds["tiny"], i, cfg) for i in range(cfg["n_layers"])]
+        for i, L in enumerate(layers):
+            g = synth.rng_for(seeds["tiny"], 6, i)
+            for name in ("post_attn_norm", "post_ffn_norm"):
+                L[name] = (np.float32(0.5) * (np.float32(1.0) + np.float32(0.1) * g.standard_normal(cfg["hidden"], dtype=np.float32))).astype(np.float32)
+        head = synth.make_head(seeds["tiny"], cfg)
         past, max_seq = 19, 64
     else:
         cfg, layers, head = synth.gemma3_4b_like(seeds["cfg4"], n_layers=3, vocab=4096)
